@@ -1,0 +1,334 @@
+// ONNX Conv (2-D, NCHW / OIHW, cross-correlation), forward and backward.
+//   * 1x1 / stride 1 / no pad / group 1 is a batched GEMM per image, Y[b] = W . X[b], and is
+//     handed to the MFMA GEMM with the channel bias and activation in its epilogue;
+//   * depthwise (group == C == M) stages the input rows a strip of outputs needs in LDS with
+//     coalesced loads and computes the stencil from LDS (HBM-bound: every input byte is read
+//     once per strip);
+//   * everything else runs a direct kernel, one thread per output, accumulating c, hy, hx
+//     sequentially in fp32 — the summation order of the reference's pure expansion.
+#include "common.h"
+
+namespace dml {
+namespace {
+
+struct ConvGeom {
+    int n, c, h, w, m, kh, kw, sh, sw, ph, pw, dh, dw, group, oh, ow, cg, mg, act;
+};
+
+// ---------------------------------------------------------------- direct forward
+template <typename T>
+__global__ __launch_bounds__(256) void conv_direct_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                          const T* __restrict__ bias, T* __restrict__ y, ConvGeom g,
+                                                          int64_t total) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+        const int ox = (int)(i % g.ow);
+        const int oy = (int)((i / g.ow) % g.oh);
+        const int m = (int)((i / ((int64_t)g.ow * g.oh)) % g.m);
+        const int b = (int)(i / ((int64_t)g.ow * g.oh * g.m));
+        const int grp = m / g.mg;
+        float acc = bias ? to_f32(bias[m]) : 0.f;
+        for (int c = 0; c < g.cg; ++c) {
+            const T* xp = x + ((int64_t)b * g.c + grp * g.cg + c) * g.h * g.w;
+            const T* wp = w + ((int64_t)m * g.cg + c) * g.kh * g.kw;
+            for (int hy = 0; hy < g.kh; ++hy) {
+                const int iy = oy * g.sh - g.ph + hy * g.dh;
+                if (iy < 0 || iy >= g.h) continue;
+                for (int hx = 0; hx < g.kw; ++hx) {
+                    const int ix = ox * g.sw - g.pw + hx * g.dw;
+                    if (ix < 0 || ix >= g.w) continue;
+                    acc += to_f32(wp[hy * g.kw + hx]) * to_f32(xp[(int64_t)iy * g.w + ix]);
+                }
+            }
+        }
+        y[i] = from_f32<T>(apply_act(g.act, acc));
+    }
+}
+
+// ---------------------------------------------------------------- depthwise forward
+// One workgroup per (image, channel, strip of ROWS output rows). LDS holds the input rows of the
+// strip, zero-padded left/right, so the stencil needs no bounds checks along x.
+template <typename T, int KH, int KW>
+__global__ __launch_bounds__(256) void conv_depthwise_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                             const T* __restrict__ bias, T* __restrict__ y, ConvGeom g,
+                                                             int rows_per_strip, int strips) {
+    extern __shared__ float tile[];  // [in_rows][wp]
+    const int strip = blockIdx.x % strips;
+    const int64_t plane = blockIdx.x / strips;  // b * C + c
+    const int c = (int)(plane % g.c);
+    const int oy0 = strip * rows_per_strip;
+    const int oy1 = min(oy0 + rows_per_strip, g.oh);
+    const int wp = g.w + 2 * g.pw;
+    const int iy0 = oy0 * g.sh - g.ph;
+    const int in_rows = (oy1 - oy0 - 1) * g.sh + (KH - 1) * g.dh + 1;
+    const T* xp = x + plane * g.h * g.w;
+    for (int i = threadIdx.x; i < in_rows * wp; i += 256) {
+        const int r = i / wp, col = i % wp - g.pw;
+        const int iy = iy0 + r;
+        float v = 0.f;
+        if (iy >= 0 && iy < g.h && col >= 0 && col < g.w) v = to_f32(xp[(int64_t)iy * g.w + col]);
+        tile[i] = v;
+    }
+    float wr[KH * KW];
+#pragma unroll
+    for (int i = 0; i < KH * KW; ++i) wr[i] = to_f32(w[(int64_t)c * KH * KW + i]);
+    const float bv = bias ? to_f32(bias[c]) : 0.f;
+    __syncthreads();
+    T* yp = y + plane * g.oh * g.ow;
+    const int outs = (oy1 - oy0) * g.ow;
+    for (int i = threadIdx.x; i < outs; i += 256) {
+        const int oy = i / g.ow, ox = i % g.ow;
+        const float* tp = tile + (oy * g.sh) * wp + ox * g.sw;
+        float acc = bv;
+#pragma unroll
+        for (int hy = 0; hy < KH; ++hy)
+#pragma unroll
+            for (int hx = 0; hx < KW; ++hx) acc += wr[hy * KW + hx] * tp[hy * g.dh * wp + hx * g.dw];
+        yp[(int64_t)(oy0 + oy) * g.ow + ox] = from_f32<T>(apply_act(g.act, acc));
+    }
+}
+
+// ---------------------------------------------------------------- direct backward
+// dX[b,c,iy,ix] = sum_{m in group, hy, hx : iy = oy*sh - ph + hy*dh, ...} W[m,c',hy,hx] * dY[b,m,oy,ox]
+__global__ __launch_bounds__(256) void conv_bwd_data_kernel(const float* __restrict__ dy, const float* __restrict__ w,
+                                                            float* __restrict__ dx, ConvGeom g, int64_t total) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+        const int ix = (int)(i % g.w);
+        const int iy = (int)((i / g.w) % g.h);
+        const int c = (int)((i / ((int64_t)g.w * g.h)) % g.c);
+        const int b = (int)(i / ((int64_t)g.w * g.h * g.c));
+        const int grp = c / g.cg, cc = c % g.cg;
+        float acc = 0.f;
+        for (int mm = 0; mm < g.mg; ++mm) {
+            const int m = grp * g.mg + mm;
+            const float* gp = dy + ((int64_t)b * g.m + m) * g.oh * g.ow;
+            const float* wp = w + ((int64_t)m * g.cg + cc) * g.kh * g.kw;
+            for (int hy = 0; hy < g.kh; ++hy) {
+                const int ty = iy + g.ph - hy * g.dh;
+                if (ty < 0 || ty % g.sh) continue;
+                const int oy = ty / g.sh;
+                if (oy >= g.oh) continue;
+                for (int hx = 0; hx < g.kw; ++hx) {
+                    const int tx = ix + g.pw - hx * g.dw;
+                    if (tx < 0 || tx % g.sw) continue;
+                    const int ox = tx / g.sw;
+                    if (ox >= g.ow) continue;
+                    acc += wp[hy * g.kw + hx] * gp[(int64_t)oy * g.ow + ox];
+                }
+            }
+        }
+        dx[i] = acc;
+    }
+}
+
+// dW[m,c',hy,hx] = sum_{b,oy,ox} dY[b,m,oy,ox] * X[b, grp*cg+c', oy*sh-ph+hy*dh, ox*sw-pw+hx*dw];
+// one workgroup per weight element.
+__global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                              float* __restrict__ dw, ConvGeom g) {
+    __shared__ float scratch[4];
+    int64_t i = blockIdx.x;
+    const int hx = (int)(i % g.kw); i /= g.kw;
+    const int hy = (int)(i % g.kh); i /= g.kh;
+    const int cc = (int)(i % g.cg); i /= g.cg;
+    const int m = (int)i;
+    const int c = (m / g.mg) * g.cg + cc;
+    const int64_t per_img = (int64_t)g.oh * g.ow;
+    float acc = 0.f;
+    for (int64_t j = threadIdx.x; j < per_img * g.n; j += 256) {
+        const int b = (int)(j / per_img);
+        const int r = (int)(j % per_img);
+        const int oy = r / g.ow, ox = r % g.ow;
+        const int iy = oy * g.sh - g.ph + hy * g.dh, ix = ox * g.sw - g.pw + hx * g.dw;
+        if (iy < 0 || iy >= g.h || ix < 0 || ix >= g.w) continue;
+        acc += dy[((int64_t)b * g.m + m) * per_img + r] * x[(((int64_t)b * g.c + c) * g.h + iy) * g.w + ix];
+    }
+    acc = block_reduce<OpSum, 4>(acc, scratch);
+    if (threadIdx.x == 0) dw[blockIdx.x] = acc;
+}
+
+// ---------------------------------------------------------------- host side
+int make_geom(const dmlhip_conv2d_desc* d, ConvGeom* g, const char* what) {
+    DML_REQUIRE(d, DMLHIP_ERR_NULL, "%s: NULL descriptor", what);
+    DML_REQUIRE(d->n >= 0 && d->c >= 0 && d->h >= 0 && d->w >= 0 && d->m >= 0, DMLHIP_ERR_SHAPE,
+                "%s: negative tensor extent", what);
+    DML_REQUIRE(d->kh >= 1 && d->kw >= 1 && d->stride_h >= 1 && d->stride_w >= 1 && d->dil_h >= 1 && d->dil_w >= 1 &&
+                    d->pad_h >= 0 && d->pad_w >= 0 && d->group >= 1,
+                DMLHIP_ERR_SHAPE, "%s: kernel/stride/dilation/group must be >= 1 and pads >= 0", what);
+    DML_REQUIRE(d->c % d->group == 0 && d->m % d->group == 0, DMLHIP_ERR_SHAPE,
+                "%s: channels (%lld in, %lld out) not divisible by group %lld", what, (long long)d->c, (long long)d->m,
+                (long long)d->group);
+    const int64_t lim = 1 << 30;
+    DML_REQUIRE(d->n < lim && d->c < lim && d->h < lim && d->w < lim && d->m < lim && d->kh < lim && d->kw < lim &&
+                    d->stride_h < lim && d->stride_w < lim && d->pad_h < lim && d->pad_w < lim && d->dil_h < lim &&
+                    d->dil_w < lim,
+                DMLHIP_ERR_SHAPE, "%s: extent exceeds 2^30", what);
+    DML_REQUIRE(valid_act(d->act), DMLHIP_ERR_ENUM, "%s: bad act", what);
+    const int64_t eh = (d->kh - 1) * d->dil_h + 1, ew = (d->kw - 1) * d->dil_w + 1;
+    const int64_t oh = d->h + 2 * d->pad_h >= eh ? (d->h + 2 * d->pad_h - eh) / d->stride_h + 1 : 0;
+    const int64_t ow = d->w + 2 * d->pad_w >= ew ? (d->w + 2 * d->pad_w - ew) / d->stride_w + 1 : 0;
+    DML_REQUIRE((double)d->n * d->m * oh * ow < 9e18 / 16 && (double)d->n * d->c * d->h * d->w < 9e18 / 16,
+                DMLHIP_ERR_SHAPE, "%s: tensor size overflows", what);
+    g->n = (int)d->n; g->c = (int)d->c; g->h = (int)d->h; g->w = (int)d->w; g->m = (int)d->m;
+    g->kh = (int)d->kh; g->kw = (int)d->kw; g->sh = (int)d->stride_h; g->sw = (int)d->stride_w;
+    g->ph = (int)d->pad_h; g->pw = (int)d->pad_w; g->dh = (int)d->dil_h; g->dw = (int)d->dil_w;
+    g->group = (int)d->group; g->oh = (int)oh; g->ow = (int)ow;
+    g->cg = g->c / g->group; g->mg = g->m / g->group; g->act = d->act;
+    return 0;
+}
+
+inline unsigned grid_for(int64_t total) {
+    int64_t gsz = ceil_div(total, 256);
+    if (gsz > 256 * 64) gsz = 256 * 64;
+    return (unsigned)(gsz < 1 ? 1 : gsz);
+}
+
+template <typename T>
+int conv_forward(const dmlhip_conv2d_desc* d, const void* x, const void* w, const void* bias, void* y, void* stream) {
+    ConvGeom g;
+    if (int e = make_geom(d, &g, "conv2d")) return e;
+    const int64_t total = (int64_t)g.n * g.m * g.oh * g.ow;
+    if (total == 0) return 0;
+    DML_REQUIRE(y && w && (x || g.c == 0), DMLHIP_ERR_NULL, "conv2d: NULL tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+
+    // 1x1, stride 1, no pad, group 1: Y[b] (M x HW) = W (M x C) . X[b] (C x HW)
+    if (g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1 && g.c > 0) {
+        dmlhip_gemm_desc gd = {};
+        const int64_t hw = (int64_t)g.h * g.w;
+        gd.m = g.m; gd.n = hw; gd.k = g.c;
+        gd.batch[0] = 1; gd.batch[1] = 1; gd.batch[2] = g.n;
+        gd.a_stride_m = g.c; gd.a_stride_k = 1;
+        gd.b_stride_k = hw; gd.b_stride_n = 1; gd.b_stride_batch[2] = (int64_t)g.c * hw;
+        gd.c_stride_m = hw; gd.c_stride_batch[2] = (int64_t)g.m * hw;
+        gd.alpha = 1.f; gd.beta = 0.f;
+        gd.out_dtype = sizeof(T) == 2 ? DMLHIP_F16 : DMLHIP_F32;
+        gd.bias_dtype = gd.out_dtype;
+        gd.act = g.act;
+        gd.bias_along_m = 1;
+        return sizeof(T) == 2 ? dmlhip_gemm_f16(&gd, w, x, y, bias, nullptr, nullptr, stream)
+                              : dmlhip_gemm_f32(&gd, w, x, y, bias, nullptr, nullptr, stream);
+    }
+    // depthwise with a small square-ish stencil
+    if (g.group == g.c && g.m == g.c && ((g.kh == 3 && g.kw == 3) || (g.kh == 5 && g.kw == 5))) {
+        const int wp = g.w + 2 * g.pw;
+        // rows per strip: keep the LDS tile under 32 KiB so several workgroups share a CU
+        int rows = g.oh;
+        while (rows > 1 && (size_t)((rows - 1) * g.sh + (g.kh - 1) * g.dh + 1) * wp * sizeof(float) > 32 * 1024)
+            rows = (rows + 1) / 2;
+        const size_t lds = (size_t)((rows - 1) * g.sh + (g.kh - 1) * g.dh + 1) * wp * sizeof(float);
+        if (lds <= 64 * 1024) {
+            const int strips = (g.oh + rows - 1) / rows;
+            const int64_t blocks = (int64_t)g.n * g.c * strips;
+            DML_REQUIRE(blocks <= 2147483647LL, DMLHIP_ERR_SHAPE, "conv2d: too many depthwise strips");
+            if (g.kh == 3)
+                hipLaunchKernelGGL((conv_depthwise_kernel<T, 3, 3>), (unsigned)blocks, 256, lds, st, (const T*)x,
+                                   (const T*)w, (const T*)bias, (T*)y, g, rows, strips);
+            else
+                hipLaunchKernelGGL((conv_depthwise_kernel<T, 5, 5>), (unsigned)blocks, 256, lds, st, (const T*)x,
+                                   (const T*)w, (const T*)bias, (T*)y, g, rows, strips);
+            return launch_status("conv2d(depthwise)");
+        }
+    }
+    hipLaunchKernelGGL((conv_direct_kernel<T>), grid_for(total), 256, 0, st, (const T*)x, (const T*)w, (const T*)bias,
+                       (T*)y, g, total);
+    return launch_status("conv2d(direct)");
+}
+
+}  // namespace
+}  // namespace dml
+
+using namespace dml;
+
+extern "C" {
+
+int dmlhip_conv2d_out_shape(const dmlhip_conv2d_desc* d, int64_t* oh, int64_t* ow) {
+    ConvGeom g;
+    if (int e = make_geom(d, &g, "conv2d_out_shape")) return e;
+    DML_REQUIRE(oh && ow, DMLHIP_ERR_NULL, "conv2d_out_shape: NULL output pointer");
+    *oh = g.oh;
+    *ow = g.ow;
+    return 0;
+}
+
+int dmlhip_conv2d_f32(const dmlhip_conv2d_desc* d, const void* x, const void* w, const void* bias, void* y,
+                      void* stream) {
+    return conv_forward<float>(d, x, w, bias, y, stream);
+}
+
+int dmlhip_conv2d_f16(const dmlhip_conv2d_desc* d, const void* x, const void* w, const void* bias, void* y,
+                      void* stream) {
+    return conv_forward<_Float16>(d, x, w, bias, y, stream);
+}
+
+int dmlhip_conv2d_backward_data_f32(const dmlhip_conv2d_desc* d, const void* dy, const void* w, void* dx,
+                                    void* stream) {
+    ConvGeom g;
+    if (int e = make_geom(d, &g, "conv2d_backward_data")) return e;
+    const int64_t total = (int64_t)g.n * g.c * g.h * g.w;
+    if (total == 0) return 0;
+    DML_REQUIRE(dx && w && (dy || (int64_t)g.oh * g.ow * g.m == 0), DMLHIP_ERR_NULL,
+                "conv2d_backward_data: NULL tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1 && g.m > 0) {
+        // dX[b] (C x HW) = W^T (C x M) . dY[b] (M x HW)
+        dmlhip_gemm_desc gd = {};
+        const int64_t hw = (int64_t)g.h * g.w;
+        gd.m = g.c; gd.n = hw; gd.k = g.m;
+        gd.batch[0] = 1; gd.batch[1] = 1; gd.batch[2] = g.n;
+        gd.a_stride_m = 1; gd.a_stride_k = g.c;
+        gd.b_stride_k = hw; gd.b_stride_n = 1; gd.b_stride_batch[2] = (int64_t)g.m * hw;
+        gd.c_stride_m = hw; gd.c_stride_batch[2] = (int64_t)g.c * hw;
+        gd.alpha = 1.f; gd.out_dtype = DMLHIP_F32; gd.bias_dtype = DMLHIP_F32;
+        return dmlhip_gemm_f32(&gd, w, dy, dx, nullptr, nullptr, nullptr, stream);
+    }
+    hipLaunchKernelGGL(conv_bwd_data_kernel, grid_for(total), 256, 0, st, (const float*)dy, (const float*)w, (float*)dx,
+                       g, total);
+    return launch_status("conv2d_backward_data");
+}
+
+size_t dmlhip_conv2d_backward_weight_workspace_bytes(const dmlhip_conv2d_desc* d) {
+    ConvGeom g;
+    if (make_geom(d, &g, "conv2d_backward_weight")) return 0;
+    if (g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1 && g.n > 1)
+        return (size_t)g.n * g.m * g.c * sizeof(float) + dmlhip_reduce_workspace_bytes(1, g.n, (int64_t)g.m * g.c);
+    return 0;
+}
+
+int dmlhip_conv2d_backward_weight_f32(const dmlhip_conv2d_desc* d, const void* x, const void* dy, void* dw,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+    ConvGeom g;
+    if (int e = make_geom(d, &g, "conv2d_backward_weight")) return e;
+    const int64_t total = (int64_t)g.m * g.cg * g.kh * g.kw;
+    if (total == 0) return 0;
+    DML_REQUIRE(dw, DMLHIP_ERR_NULL, "conv2d_backward_weight: NULL output");
+    const int64_t red = (int64_t)g.n * g.oh * g.ow;
+    DML_REQUIRE(red == 0 || (x && dy), DMLHIP_ERR_NULL, "conv2d_backward_weight: NULL tensor pointer");
+    DML_REQUIRE(total <= 2147483647LL, DMLHIP_ERR_SHAPE, "conv2d_backward_weight: too many weights");
+    hipStream_t st = (hipStream_t)stream;
+    if (g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1 && red > 0) {
+        // per image: P[b] (M x C) = dY[b] (M x HW) . X[b]^T (HW x C); then dW = sum_b P[b]
+        const size_t need = dmlhip_conv2d_backward_weight_workspace_bytes(d);
+        DML_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), DMLHIP_ERR_WORKSPACE,
+                    "conv2d_backward_weight: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        dmlhip_gemm_desc gd = {};
+        const int64_t hw = (int64_t)g.h * g.w;
+        gd.m = g.m; gd.n = g.c; gd.k = hw;
+        gd.batch[0] = 1; gd.batch[1] = 1; gd.batch[2] = g.n;
+        gd.a_stride_m = hw; gd.a_stride_k = 1; gd.a_stride_batch[2] = (int64_t)g.m * hw;
+        gd.b_stride_k = 1; gd.b_stride_n = hw; gd.b_stride_batch[2] = (int64_t)g.c * hw;
+        gd.c_stride_m = g.c; gd.c_stride_batch[2] = (int64_t)g.m * g.c;
+        gd.alpha = 1.f; gd.out_dtype = DMLHIP_F32; gd.bias_dtype = DMLHIP_F32;
+        if (g.n == 1) return dmlhip_gemm_f32(&gd, dy, x, dw, nullptr, nullptr, nullptr, stream);
+        float* part = (float*)workspace;
+        if (int e = dmlhip_gemm_f32(&gd, dy, x, part, nullptr, nullptr, nullptr, stream)) return e;
+        const size_t part_bytes = (size_t)g.n * g.m * g.c * sizeof(float);
+        return dmlhip_reduce_f32(DMLHIP_RSUM, part, dw, DMLHIP_F32, 1, g.n, (int64_t)g.m * g.c,
+                                 (char*)workspace + part_bytes, workspace_bytes - part_bytes, stream);
+    }
+    hipLaunchKernelGGL(conv_bwd_weight_kernel, (unsigned)total, 256, 0, st, (const float*)x, (const float*)dy,
+                       (float*)dw, g);
+    return launch_status("conv2d_backward_weight");
+}
+
+}  // extern "C"

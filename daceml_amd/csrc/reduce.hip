@@ -1,0 +1,223 @@
+// Reductions over one (collapsed) axis of a dense tensor viewed as [outer, r, inner]:
+// ReduceSum / ReduceMax / ReduceMin / ReduceMean and GlobalAveragePool. fp32 accumulation.
+//   inner == 1 : each row of r elements is reduced by a wavefront (short rows) or a workgroup.
+//   inner  > 1 : column reduction; lanes run along `inner` (coalesced, 128-bit when aligned),
+//                four wavefronts stride over r, and r is split across workgroups when
+//                outer*inner alone cannot fill the chip; partial results go through a caller
+//                workspace and a second, tiny pass, so the result is deterministic.
+#include "common.h"
+
+namespace dml {
+namespace {
+
+constexpr int kRedBlock = 256;
+constexpr int kRedWaves = kRedBlock / kWave;
+
+template <int OP> struct RedOp;
+template <> struct RedOp<DMLHIP_RSUM> { using op = OpSum; __device__ __host__ static float init() { return 0.f; } };
+template <> struct RedOp<DMLHIP_RMEAN> { using op = OpSum; __device__ __host__ static float init() { return 0.f; } };
+template <> struct RedOp<DMLHIP_RMAX> { using op = OpMax; __device__ __host__ static float init() { return -INFINITY; } };
+template <> struct RedOp<DMLHIP_RMIN> { using op = OpMin; __device__ __host__ static float init() { return INFINITY; } };
+
+// ---------------------------------------------------------------- inner == 1
+template <typename TIn, typename TOut, int OP, bool WAVE>
+__global__ __launch_bounds__(kRedBlock) void row_reduce_kernel(const TIn* __restrict__ x, TOut* __restrict__ y,
+                                                               int64_t rows, int64_t r, float scale) {
+    using Op = typename RedOp<OP>::op;
+    __shared__ float scratch[kRedWaves];
+    const int64_t row = WAVE ? (int64_t)blockIdx.x * kRedWaves + threadIdx.x / kWave : (int64_t)blockIdx.x;
+    const int tid = WAVE ? (threadIdx.x & (kWave - 1)) : threadIdx.x;
+    const int nth = WAVE ? kWave : kRedBlock;
+    float a0 = RedOp<OP>::init(), a1 = a0, a2 = a0, a3 = a0;
+    if (row < rows) {
+        const TIn* xr = x + row * r;
+        int64_t c = tid;
+        for (; c + 3 * nth < r; c += 4 * nth) {
+            a0 = Op::f(a0, to_f32(xr[c]));
+            a1 = Op::f(a1, to_f32(xr[c + nth]));
+            a2 = Op::f(a2, to_f32(xr[c + 2 * nth]));
+            a3 = Op::f(a3, to_f32(xr[c + 3 * nth]));
+        }
+        for (; c < r; c += nth) a0 = Op::f(a0, to_f32(xr[c]));
+    }
+    float a = Op::f(Op::f(a0, a1), Op::f(a2, a3));
+    if constexpr (WAVE) {
+        a = wave_reduce<Op>(a);
+    } else {
+        a = block_reduce<Op, kRedWaves>(a, scratch);
+    }
+    if (row < rows && tid == 0) y[row] = from_f32<TOut>(a * scale);
+}
+
+// ---------------------------------------------------------------- inner > 1
+// grid: x = column tiles, y = outer, z = splits of r. V = elements per lane along inner.
+template <typename TIn, typename TOut, int OP, int V>
+__global__ __launch_bounds__(kRedBlock) void col_reduce_kernel(const TIn* __restrict__ x, TOut* __restrict__ y,
+                                                               int64_t outer, int64_t r, int64_t inner,
+                                                               int64_t r_per_split, float scale) {
+    using Op = typename RedOp<OP>::op;
+    typedef TIn vec_t __attribute__((ext_vector_type(V)));
+    __shared__ float lds[kRedWaves][kWave * V];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t col = ((int64_t)blockIdx.x * kWave + lane) * V;
+    const int64_t o = blockIdx.y;
+    const int64_t r0 = (int64_t)blockIdx.z * r_per_split;
+    const int64_t r1 = r0 + r_per_split < r ? r0 + r_per_split : r;
+    float acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = RedOp<OP>::init();
+    if (col < inner) {
+        const TIn* base = x + o * r * inner + col;
+        for (int64_t i = r0 + wave; i < r1; i += kRedWaves) {
+            if constexpr (V > 1) {
+                vec_t v = *reinterpret_cast<const vec_t*>(base + i * inner);
+#pragma unroll
+                for (int e = 0; e < V; ++e) acc[e] = Op::f(acc[e], to_f32(v[e]));
+            } else {
+                acc[0] = Op::f(acc[0], to_f32(base[i * inner]));
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) lds[wave][lane * V + e] = acc[e];
+    __syncthreads();
+    if (wave == 0 && col < inner) {
+        TOut* out = y + ((int64_t)blockIdx.z * outer + o) * inner + col;
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            float a = lds[0][lane * V + e];
+#pragma unroll
+            for (int w = 1; w < kRedWaves; ++w) a = Op::f(a, lds[w][lane * V + e]);
+            out[e] = from_f32<TOut>(a * scale);
+        }
+    }
+}
+
+struct ColPlan {
+    int v;           // elements per lane
+    int64_t tiles;   // column tiles
+    int64_t splits;  // splits of r
+    int64_t r_per_split;
+};
+
+template <typename TIn>
+ColPlan plan_cols(const void* x, int64_t outer, int64_t r, int64_t inner) {
+    ColPlan p;
+    constexpr int VN = VecOf<TIn>::n;
+    p.v = (inner % VN == 0 && aligned16(x)) ? VN : 1;
+    p.tiles = ceil_div(inner, (int64_t)kWave * p.v);
+    const int64_t blocks = p.tiles * outer;
+    int64_t splits = 1;
+    if (blocks < 1024) {
+        splits = ceil_div(1024, blocks);
+        const int64_t max_splits = ceil_div(r, 4 * kRedWaves);  // at least 16 rows per workgroup
+        if (splits > max_splits) splits = max_splits;
+        if (splits < 1) splits = 1;
+        if (splits > 65535) splits = 65535;
+    }
+    p.r_per_split = r > 0 ? ceil_div(r, splits) : 1;
+    p.splits = r > 0 ? ceil_div(r, p.r_per_split) : 1;
+    return p;
+}
+
+template <typename TIn, typename TOut, int OP>
+int col_launch(const TIn* x, TOut* y, int64_t outer, int64_t r, int64_t inner, int v, int64_t tiles, int64_t splits,
+               int64_t r_per_split, float scale, hipStream_t st) {
+    dim3 grid((unsigned)tiles, (unsigned)outer, (unsigned)splits);
+    constexpr int VN = VecOf<TIn>::n;
+    if (v == VN)
+        hipLaunchKernelGGL((col_reduce_kernel<TIn, TOut, OP, VN>), grid, kRedBlock, 0, st, x, y, outer, r, inner,
+                           r_per_split, scale);
+    else
+        hipLaunchKernelGGL((col_reduce_kernel<TIn, TOut, OP, 1>), grid, kRedBlock, 0, st, x, y, outer, r, inner,
+                           r_per_split, scale);
+    return launch_status("reduce(columns)");
+}
+
+template <typename TIn, typename TOut, int OP>
+int reduce_typed(const TIn* x, TOut* y, int64_t outer, int64_t r, int64_t inner, void* ws, size_t ws_bytes,
+                 hipStream_t st) {
+    const float scale = OP == DMLHIP_RMEAN ? 1.0f / (float)r : 1.0f;
+    if (inner == 1) {
+        if (r <= 2048) {
+            hipLaunchKernelGGL((row_reduce_kernel<TIn, TOut, OP, true>), (unsigned)ceil_div(outer, kRedWaves), kRedBlock,
+                               0, st, x, y, outer, r, scale);
+        } else {
+            hipLaunchKernelGGL((row_reduce_kernel<TIn, TOut, OP, false>), (unsigned)outer, kRedBlock, 0, st, x, y,
+                               outer, r, scale);
+        }
+        return launch_status("reduce(rows)");
+    }
+    const ColPlan p = plan_cols<TIn>(x, outer, r, inner);
+    if (p.splits == 1) return col_launch<TIn, TOut, OP>(x, y, outer, r, inner, p.v, p.tiles, 1, r, scale, st);
+    const size_t need = (size_t)p.splits * outer * inner * sizeof(float);
+    DML_REQUIRE(ws && ws_bytes >= need, DMLHIP_ERR_WORKSPACE, "reduce: workspace of %zu bytes needed, %zu given", need,
+                ws_bytes);
+    float* part = (float*)ws;
+    if (int e = col_launch<TIn, float, OP>(x, part, outer, r, inner, p.v, p.tiles, p.splits, p.r_per_split, 1.0f, st))
+        return e;
+    // second pass: [1, splits, outer*inner] fp32 -> TOut, same op (sum for mean), then the scale
+    const int64_t inner2 = outer * inner;
+    const int v2 = (inner2 % 4 == 0) ? 4 : 1;
+    const int64_t tiles2 = ceil_div(inner2, (int64_t)kWave * v2);
+    return col_launch<float, TOut, OP>(part, y, 1, p.splits, inner2, v2, tiles2, 1, p.splits, scale, st);
+}
+
+template <typename TIn>
+int reduce_impl(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r, int64_t inner, void* ws,
+                size_t ws_bytes, void* stream) {
+    DML_REQUIRE(op >= DMLHIP_RSUM && op <= DMLHIP_RMEAN, DMLHIP_ERR_ENUM, "reduce: unknown op %d", op);
+    DML_REQUIRE(out_dtype == DMLHIP_F16 || out_dtype == DMLHIP_F32, DMLHIP_ERR_ENUM, "reduce: unknown out_dtype");
+    DML_REQUIRE(outer >= 0 && r >= 0 && inner >= 0, DMLHIP_ERR_SHAPE, "reduce: negative extent");
+    DML_REQUIRE(outer <= 2147483647 && (inner == 1 || outer <= 65535), DMLHIP_ERR_SHAPE,
+                "reduce: outer extent %lld too large", (long long)outer);
+    DML_REQUIRE(r == 0 || inner == 0 || outer <= (INT64_MAX / 16) / r / inner, DMLHIP_ERR_SHAPE,
+                "reduce: size overflows");
+    if (outer == 0 || inner == 0) return 0;
+    DML_REQUIRE(r > 0 || op == DMLHIP_RSUM, DMLHIP_ERR_SHAPE, "reduce: empty axis only defined for sum");
+    DML_REQUIRE(x || r == 0, DMLHIP_ERR_NULL, "reduce: NULL input");
+    DML_REQUIRE(y, DMLHIP_ERR_NULL, "reduce: NULL output");
+    hipStream_t st = (hipStream_t)stream;
+    const TIn* xp = (const TIn*)x;
+#define DML_RED(OP)                                                                                          \
+    case OP:                                                                                                 \
+        return out_dtype == DMLHIP_F32                                                                       \
+                   ? reduce_typed<TIn, float, OP>(xp, (float*)y, outer, r, inner, ws, ws_bytes, st)          \
+                   : reduce_typed<TIn, _Float16, OP>(xp, (_Float16*)y, outer, r, inner, ws, ws_bytes, st)
+    switch (op) {
+        DML_RED(DMLHIP_RSUM);
+        DML_RED(DMLHIP_RMAX);
+        DML_RED(DMLHIP_RMIN);
+        default: DML_RED(DMLHIP_RMEAN);
+    }
+#undef DML_RED
+}
+
+}  // namespace
+}  // namespace dml
+
+using namespace dml;
+
+extern "C" {
+
+size_t dmlhip_reduce_workspace_bytes(int64_t outer, int64_t r, int64_t inner) {
+    if (outer <= 0 || r <= 0 || inner <= 1) return 0;
+    // alignment-independent upper bound: the plan with the most splits
+    const int64_t tiles_min = ceil_div(inner, (int64_t)kWave * 8);
+    int64_t splits = ceil_div(1024, tiles_min * outer);
+    const int64_t max_splits = ceil_div(r, 4 * kRedWaves);
+    if (splits > max_splits) splits = max_splits;
+    if (splits <= 1) return 0;
+    return (size_t)(splits + 1) * outer * inner * sizeof(float);
+}
+
+int dmlhip_reduce_f16(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r, int64_t inner,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+    return reduce_impl<_Float16>(op, x, y, out_dtype, outer, r, inner, workspace, workspace_bytes, stream);
+}
+int dmlhip_reduce_f32(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r, int64_t inner,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+    return reduce_impl<float>(op, x, y, out_dtype, outer, r, inner, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,605 @@
+// Row-wise, HBM-bound nodes: Softmax and the fused LayerNormalization chain, forward and
+// backward. One wavefront owns one row: the row is read once with 128-bit loads, kept in
+// registers, reduced with DPP lane permutes, and written once. Rows that do not fit the
+// register budget or are not 16-byte aligned take a workgroup-per-row fallback.
+#include "common.h"
+
+namespace dml {
+namespace {
+
+constexpr int kRowBlock = 256;                 // threads per workgroup
+constexpr int kRowsPerBlock = kRowBlock / kWave;
+
+template <typename T> struct ExpFn;
+// fp16 I/O: the result is rounded to 11 bits, so the hardware exp2 is exact enough.
+template <> struct ExpFn<_Float16> {
+    __device__ __forceinline__ static float f(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+};
+template <> struct ExpFn<float> {
+    __device__ __forceinline__ static float f(float x) { return expf(x); }
+};
+
+// ------------------------------------------------------------------ softmax, wave per row
+template <typename T, int VPL>
+__global__ __launch_bounds__(kRowBlock) void softmax_wave_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                 int64_t rows, int cols) {
+    using V = typename VecOf<T>::type;
+    constexpr int VN = VecOf<T>::n;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const V* xr = reinterpret_cast<const V*>(x + row * cols);
+    V* yr = reinterpret_cast<V*>(y + row * cols);
+    const int nvec = cols / VN;
+
+    float v[VPL][VN];
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        if (vi < nvec) {
+            V t = __builtin_nontemporal_load(xr + vi);
+#pragma unroll
+            for (int e = 0; e < VN; ++e) {
+                v[j][e] = to_f32(t[e]);
+                m = fmaxf(m, v[j][e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VN; ++e) v[j][e] = -INFINITY;
+        }
+    }
+    m = wave_reduce<OpMax>(m);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+#pragma unroll
+        for (int e = 0; e < VN; ++e) {
+            v[j][e] = ExpFn<T>::f(v[j][e] - m);
+            s += v[j][e];
+        }
+    s = wave_reduce<OpSum>(s);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        if (vi < nvec) {
+            V t;
+#pragma unroll
+            for (int e = 0; e < VN; ++e) t[e] = from_f32<T>(v[j][e] / s);
+            __builtin_nontemporal_store(t, yr + vi);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ softmax, block per row
+template <typename T>
+__global__ __launch_bounds__(kRowBlock) void softmax_block_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                  int64_t cols) {
+    __shared__ float scratch[kRowsPerBlock];
+    const T* xr = x + (int64_t)blockIdx.x * cols;
+    T* yr = y + (int64_t)blockIdx.x * cols;
+    float m = -INFINITY;
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock) m = fmaxf(m, to_f32(xr[c]));
+    m = block_reduce<OpMax, kRowsPerBlock>(m, scratch);
+    float s = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock) s += ExpFn<T>::f(to_f32(xr[c]) - m);
+    s = block_reduce<OpSum, kRowsPerBlock>(s, scratch);
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock)
+        yr[c] = from_f32<T>(ExpFn<T>::f(to_f32(xr[c]) - m) / s);
+}
+
+// ------------------------------------------------------------------ softmax backward
+template <typename T, int VPL>
+__global__ __launch_bounds__(kRowBlock) void softmax_bwd_wave_kernel(const T* __restrict__ y,
+                                                                     const T* __restrict__ dy,
+                                                                     T* __restrict__ dx, int64_t rows,
+                                                                     int cols) {
+    using V = typename VecOf<T>::type;
+    constexpr int VN = VecOf<T>::n;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const V* yr = reinterpret_cast<const V*>(y + row * cols);
+    const V* gr = reinterpret_cast<const V*>(dy + row * cols);
+    V* dr = reinterpret_cast<V*>(dx + row * cols);
+    const int nvec = cols / VN;
+    float yv[VPL][VN], pv[VPL][VN];
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        if (vi < nvec) {
+            V a = __builtin_nontemporal_load(yr + vi);
+            V b = __builtin_nontemporal_load(gr + vi);
+#pragma unroll
+            for (int e = 0; e < VN; ++e) {
+                yv[j][e] = to_f32(a[e]);
+                pv[j][e] = yv[j][e] * to_f32(b[e]);
+                s += pv[j][e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VN; ++e) { yv[j][e] = 0.f; pv[j][e] = 0.f; }
+        }
+    }
+    s = wave_reduce<OpSum>(s);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        if (vi < nvec) {
+            V t;
+#pragma unroll
+            for (int e = 0; e < VN; ++e) t[e] = from_f32<T>(pv[j][e] - yv[j][e] * s);
+            __builtin_nontemporal_store(t, dr + vi);
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kRowBlock) void softmax_bwd_block_kernel(const T* __restrict__ y,
+                                                                      const T* __restrict__ dy,
+                                                                      T* __restrict__ dx, int64_t cols) {
+    __shared__ float scratch[kRowsPerBlock];
+    const int64_t off = (int64_t)blockIdx.x * cols;
+    float s = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock) s += to_f32(y[off + c]) * to_f32(dy[off + c]);
+    s = block_reduce<OpSum, kRowsPerBlock>(s, scratch);
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock) {
+        const float yy = to_f32(y[off + c]);
+        dx[off + c] = from_f32<T>(yy * to_f32(dy[off + c]) - yy * s);
+    }
+}
+
+// ------------------------------------------------------------------ layernorm forward, wave per row
+template <typename T, int VPL>
+__global__ __launch_bounds__(kRowBlock) void layernorm_wave_kernel(
+    const T* __restrict__ x, const T* __restrict__ res, const T* __restrict__ gamma,
+    const T* __restrict__ beta, T* __restrict__ y, T* __restrict__ sum_out, float* __restrict__ mean,
+    float* __restrict__ rstd, int64_t rows, int cols, float eps) {
+    using V = typename VecOf<T>::type;
+    constexpr int VN = VecOf<T>::n;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const int nvec = cols / VN;
+    const V* xr = reinterpret_cast<const V*>(x + row * cols);
+    const V* rr = res ? reinterpret_cast<const V*>(res + row * cols) : nullptr;
+    float v[VPL][VN];
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        if (vi < nvec) {
+            V t = xr[vi];
+            if (rr) {
+                V r = rr[vi];
+                // the fused ONNXAdd rounds to the tensor dtype, as the separate node would
+#pragma unroll
+                for (int e = 0; e < VN; ++e) t[e] = from_f32<T>(to_f32(t[e]) + to_f32(r[e]));
+                if (sum_out) reinterpret_cast<V*>(sum_out + row * cols)[vi] = t;
+            } else if (sum_out) {
+                reinterpret_cast<V*>(sum_out + row * cols)[vi] = t;
+            }
+#pragma unroll
+            for (int e = 0; e < VN; ++e) {
+                v[j][e] = to_f32(t[e]);
+                s += v[j][e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VN; ++e) v[j][e] = 0.f;
+        }
+    }
+    const float mu = wave_reduce<OpSum>(s) / (float)cols;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        if (vi < nvec) {
+#pragma unroll
+            for (int e = 0; e < VN; ++e) {
+                v[j][e] -= mu;
+                q += v[j][e] * v[j][e];
+            }
+        }
+    }
+    const float var = wave_reduce<OpSum>(q) / (float)cols;
+    const float inv = 1.0f / sqrtf(var + eps);
+    if (lane == 0) {
+        if (mean) mean[row] = mu;
+        if (rstd) rstd[row] = inv;
+    }
+    const V* gv = reinterpret_cast<const V*>(gamma);
+    const V* bv = reinterpret_cast<const V*>(beta);
+    V* yr = reinterpret_cast<V*>(y + row * cols);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        if (vi < nvec) {
+            V g = gv[vi], b = bv[vi], t;
+#pragma unroll
+            for (int e = 0; e < VN; ++e) t[e] = from_f32<T>(v[j][e] * inv * to_f32(g[e]) + to_f32(b[e]));
+            yr[vi] = t;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kRowBlock) void layernorm_block_kernel(
+    const T* __restrict__ x, const T* __restrict__ res, const T* __restrict__ gamma,
+    const T* __restrict__ beta, T* __restrict__ y, T* __restrict__ sum_out, float* __restrict__ mean,
+    float* __restrict__ rstd, int64_t cols, float eps) {
+    __shared__ float scratch[kRowsPerBlock];
+    const int64_t off = (int64_t)blockIdx.x * cols;
+    auto load = [&](int64_t c) -> float {
+        if (res) return to_f32(from_f32<T>(to_f32(x[off + c]) + to_f32(res[off + c])));
+        return to_f32(x[off + c]);
+    };
+    float s = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock) {
+        const float t = load(c);
+        if (sum_out) sum_out[off + c] = from_f32<T>(t);
+        s += t;
+    }
+    const float mu = block_reduce<OpSum, kRowsPerBlock>(s, scratch) / (float)cols;
+    float q = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock) {
+        const float d = load(c) - mu;
+        q += d * d;
+    }
+    const float var = block_reduce<OpSum, kRowsPerBlock>(q, scratch) / (float)cols;
+    const float inv = 1.0f / sqrtf(var + eps);
+    if (threadIdx.x == 0) {
+        if (mean) mean[blockIdx.x] = mu;
+        if (rstd) rstd[blockIdx.x] = inv;
+    }
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock)
+        y[off + c] = from_f32<T>((load(c) - mu) * inv * to_f32(gamma[c]) + to_f32(beta[c]));
+}
+
+// ------------------------------------------------------------------ layernorm backward
+// Stage 1: a workgroup walks a slab of rows, one wavefront per row at a time. Each lane keeps
+// the running column sums of dy*xhat (dgamma) and dy (dbeta) for the columns it owns; after the
+// slab the four wavefronts are combined through LDS and one partial row per workgroup goes to the
+// workspace. Stage 2 sums the partial rows. dx is written in stage 1.
+template <typename T, int VPL>
+__global__ __launch_bounds__(kRowBlock) void layernorm_bwd_wave_kernel(
+    const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ mean,
+    const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx,
+    float* __restrict__ part, int64_t rows, int cols) {
+    using V = typename VecOf<T>::type;
+    constexpr int VN = VecOf<T>::n;
+    extern __shared__ float lds[];  // [2][kRowsPerBlock][cols]
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int nvec = cols / VN;
+    float g[VPL][VN], accg[VPL][VN], accb[VPL][VN];
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        V t = {};
+        if (vi < nvec) t = reinterpret_cast<const V*>(gamma)[vi];
+#pragma unroll
+        for (int e = 0; e < VN; ++e) { g[j][e] = to_f32(t[e]); accg[j][e] = 0.f; accb[j][e] = 0.f; }
+    }
+    for (int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + wave; row < rows;
+         row += (int64_t)gridDim.x * kRowsPerBlock) {
+        const float mu = mean[row], inv = rstd[row];
+        const V* xr = reinterpret_cast<const V*>(x + row * cols);
+        const V* gr = reinterpret_cast<const V*>(dy + row * cols);
+        float xh[VPL][VN], gd[VPL][VN];
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const int vi = lane + j * kWave;
+            if (vi < nvec) {
+                V a = xr[vi], b = gr[vi];
+#pragma unroll
+                for (int e = 0; e < VN; ++e) {
+                    const float d = to_f32(b[e]);
+                    xh[j][e] = (to_f32(a[e]) - mu) * inv;
+                    accg[j][e] += d * xh[j][e];
+                    accb[j][e] += d;
+                    gd[j][e] = d * g[j][e];
+                    s1 += gd[j][e];
+                    s2 += gd[j][e] * xh[j][e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VN; ++e) { xh[j][e] = 0.f; gd[j][e] = 0.f; }
+            }
+        }
+        s1 = wave_reduce<OpSum>(s1) / (float)cols;
+        s2 = wave_reduce<OpSum>(s2) / (float)cols;
+        V* dr = reinterpret_cast<V*>(dx + row * cols);
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const int vi = lane + j * kWave;
+            if (vi < nvec) {
+                V t;
+#pragma unroll
+                for (int e = 0; e < VN; ++e) t[e] = from_f32<T>((gd[j][e] - s1 - xh[j][e] * s2) * inv);
+                dr[vi] = t;
+            }
+        }
+    }
+    float* lg = lds + (size_t)wave * cols;
+    float* lb = lds + (size_t)(kRowsPerBlock + wave) * cols;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        if (vi < nvec) {
+#pragma unroll
+            for (int e = 0; e < VN; ++e) { lg[vi * VN + e] = accg[j][e]; lb[vi * VN + e] = accb[j][e]; }
+        }
+    }
+    __syncthreads();
+    float* pg = part + (size_t)blockIdx.x * 2 * cols;
+    for (int c = threadIdx.x; c < cols; c += kRowBlock) {
+        float a = 0.f, b = 0.f;
+#pragma unroll
+        for (int w = 0; w < kRowsPerBlock; ++w) {
+            a += lds[(size_t)w * cols + c];
+            b += lds[(size_t)(kRowsPerBlock + w) * cols + c];
+        }
+        pg[c] = a;
+        pg[cols + c] = b;
+    }
+}
+
+__global__ void layernorm_bwd_finish_kernel(const float* __restrict__ part, float* __restrict__ dgamma,
+                                            float* __restrict__ dbeta, int nparts, int cols) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    float a = 0.f, b = 0.f;
+    for (int p = 0; p < nparts; ++p) {
+        a += part[(size_t)p * 2 * cols + c];
+        b += part[(size_t)p * 2 * cols + cols + c];
+    }
+    dgamma[c] = a;
+    dbeta[c] = b;
+}
+
+// fallback: dx, workgroup per row
+template <typename T>
+__global__ __launch_bounds__(kRowBlock) void layernorm_bwd_dx_block_kernel(
+    const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ mean,
+    const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx, int64_t cols) {
+    __shared__ float scratch[kRowsPerBlock];
+    const int64_t off = (int64_t)blockIdx.x * cols;
+    const float mu = mean[blockIdx.x], inv = rstd[blockIdx.x];
+    float s1 = 0.f, s2 = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock) {
+        const float gd = to_f32(dy[off + c]) * to_f32(gamma[c]);
+        const float xh = (to_f32(x[off + c]) - mu) * inv;
+        s1 += gd;
+        s2 += gd * xh;
+    }
+    s1 = block_reduce<OpSum, kRowsPerBlock>(s1, scratch) / (float)cols;
+    s2 = block_reduce<OpSum, kRowsPerBlock>(s2, scratch) / (float)cols;
+    for (int64_t c = threadIdx.x; c < cols; c += kRowBlock) {
+        const float gd = to_f32(dy[off + c]) * to_f32(gamma[c]);
+        const float xh = (to_f32(x[off + c]) - mu) * inv;
+        dx[off + c] = from_f32<T>((gd - s1 - xh * s2) * inv);
+    }
+}
+
+// fallback: dgamma/dbeta partials, thread per column over a slab of rows
+template <typename T>
+__global__ void layernorm_bwd_cols_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                          const float* __restrict__ mean, const float* __restrict__ rstd,
+                                          float* __restrict__ part, int64_t rows, int64_t cols) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    float a = 0.f, b = 0.f;
+    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        const float d = to_f32(dy[r * cols + c]);
+        a += d * (to_f32(x[r * cols + c]) - mean[r]) * rstd[r];
+        b += d;
+    }
+    part[(size_t)blockIdx.y * 2 * cols + c] = a;
+    part[(size_t)blockIdx.y * 2 * cols + cols + c] = b;
+}
+
+// ------------------------------------------------------------------ host dispatch
+int check_rows(const char* what, int64_t rows, int64_t cols) {
+    DML_REQUIRE(rows >= 0 && cols >= 0, DMLHIP_ERR_SHAPE, "%s: negative extent (rows=%lld, cols=%lld)", what,
+                (long long)rows, (long long)cols);
+    DML_REQUIRE(rows <= (int64_t)2147483647 * kRowsPerBlock, DMLHIP_ERR_SHAPE, "%s: too many rows (%lld)", what,
+                (long long)rows);
+    DML_REQUIRE(cols == 0 || rows <= (INT64_MAX / 16) / cols, DMLHIP_ERR_SHAPE, "%s: rows*cols overflows", what);
+    return 0;
+}
+
+template <typename T>
+bool wave_path_ok(int64_t cols, int max_vpl) {
+    constexpr int VN = VecOf<T>::n;
+    return cols % VN == 0 && cols <= (int64_t)kWave * VN * max_vpl;
+}
+
+template <typename T>
+int softmax_impl(const void* x, void* y, int64_t rows, int64_t cols, void* stream) {
+    if (int e = check_rows("softmax", rows, cols)) return e;
+    if (rows == 0 || cols == 0) return 0;
+    DML_REQUIRE(x && y, DMLHIP_ERR_NULL, "softmax: NULL tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const T* xp = (const T*)x;
+    T* yp = (T*)y;
+    constexpr int VN = VecOf<T>::n;
+    const unsigned grid = (unsigned)ceil_div(rows, kRowsPerBlock);
+    if (wave_path_ok<T>(cols, 4) && aligned16(x) && aligned16(y)) {
+        const int vpl = (int)ceil_div(cols, kWave * VN);
+        switch (vpl) {
+            case 1: hipLaunchKernelGGL((softmax_wave_kernel<T, 1>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
+            case 2: hipLaunchKernelGGL((softmax_wave_kernel<T, 2>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
+            case 3: hipLaunchKernelGGL((softmax_wave_kernel<T, 3>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
+            default: hipLaunchKernelGGL((softmax_wave_kernel<T, 4>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
+        }
+    } else {
+        DML_REQUIRE(rows <= 2147483647, DMLHIP_ERR_SHAPE, "softmax: too many rows for the generic path");
+        hipLaunchKernelGGL((softmax_block_kernel<T>), (unsigned)rows, kRowBlock, 0, st, xp, yp, cols);
+    }
+    return launch_status("softmax");
+}
+
+template <typename T>
+int softmax_bwd_impl(const void* y, const void* dy, void* dx, int64_t rows, int64_t cols, void* stream) {
+    if (int e = check_rows("softmax_backward", rows, cols)) return e;
+    if (rows == 0 || cols == 0) return 0;
+    DML_REQUIRE(y && dy && dx, DMLHIP_ERR_NULL, "softmax_backward: NULL tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const T* yp = (const T*)y;
+    const T* gp = (const T*)dy;
+    T* dp = (T*)dx;
+    constexpr int VN = VecOf<T>::n;
+    const unsigned grid = (unsigned)ceil_div(rows, kRowsPerBlock);
+    if (wave_path_ok<T>(cols, 4) && aligned16(y) && aligned16(dy) && aligned16(dx)) {
+        const int vpl = (int)ceil_div(cols, kWave * VN);
+        switch (vpl) {
+            case 1: hipLaunchKernelGGL((softmax_bwd_wave_kernel<T, 1>), grid, kRowBlock, 0, st, yp, gp, dp, rows, (int)cols); break;
+            case 2: hipLaunchKernelGGL((softmax_bwd_wave_kernel<T, 2>), grid, kRowBlock, 0, st, yp, gp, dp, rows, (int)cols); break;
+            case 3: hipLaunchKernelGGL((softmax_bwd_wave_kernel<T, 3>), grid, kRowBlock, 0, st, yp, gp, dp, rows, (int)cols); break;
+            default: hipLaunchKernelGGL((softmax_bwd_wave_kernel<T, 4>), grid, kRowBlock, 0, st, yp, gp, dp, rows, (int)cols); break;
+        }
+    } else {
+        DML_REQUIRE(rows <= 2147483647, DMLHIP_ERR_SHAPE, "softmax_backward: too many rows for the generic path");
+        hipLaunchKernelGGL((softmax_bwd_block_kernel<T>), (unsigned)rows, kRowBlock, 0, st, yp, gp, dp, cols);
+    }
+    return launch_status("softmax_backward");
+}
+
+template <typename T>
+int layernorm_impl(const void* x, const void* residual, const void* gamma, const void* beta, void* y,
+                   void* sum_out, float* mean, float* rstd, int64_t rows, int64_t cols, float eps, void* stream) {
+    if (int e = check_rows("layernorm", rows, cols)) return e;
+    DML_REQUIRE(eps >= 0.f, DMLHIP_ERR_SHAPE, "layernorm: negative epsilon");
+    if (rows == 0 || cols == 0) return 0;
+    DML_REQUIRE(x && gamma && beta && y, DMLHIP_ERR_NULL, "layernorm: NULL tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const T *xp = (const T*)x, *rp = (const T*)residual, *gp = (const T*)gamma, *bp = (const T*)beta;
+    T *yp = (T*)y, *sp = (T*)sum_out;
+    constexpr int VN = VecOf<T>::n;
+    const bool al = aligned16(x) && aligned16(y) && aligned16(gamma) && aligned16(beta) &&
+                    (!residual || aligned16(residual)) && (!sum_out || aligned16(sum_out));
+    if (wave_path_ok<T>(cols, 4) && al) {
+        const unsigned grid = (unsigned)ceil_div(rows, kRowsPerBlock);
+        const int vpl = (int)ceil_div(cols, kWave * VN);
+#define DML_LN_LAUNCH(V) hipLaunchKernelGGL((layernorm_wave_kernel<T, V>), grid, kRowBlock, 0, st, xp, rp, gp, bp, yp, sp, mean, rstd, rows, (int)cols, eps)
+        switch (vpl) {
+            case 1: DML_LN_LAUNCH(1); break;
+            case 2: DML_LN_LAUNCH(2); break;
+            case 3: DML_LN_LAUNCH(3); break;
+            default: DML_LN_LAUNCH(4); break;
+        }
+#undef DML_LN_LAUNCH
+    } else {
+        DML_REQUIRE(rows <= 2147483647, DMLHIP_ERR_SHAPE, "layernorm: too many rows for the generic path");
+        hipLaunchKernelGGL((layernorm_block_kernel<T>), (unsigned)rows, kRowBlock, 0, st, xp, rp, gp, bp, yp, sp, mean,
+                           rstd, cols, eps);
+    }
+    return launch_status("layernorm");
+}
+
+int ln_bwd_parts(int64_t rows) {
+    int64_t p = ceil_div(rows, kRowsPerBlock * 4);
+    if (p < 1) p = 1;
+    if (p > 512) p = 512;
+    return (int)p;
+}
+
+template <typename T>
+int layernorm_bwd_impl(const void* dy, const void* x, const float* mean, const float* rstd, const void* gamma,
+                       void* dx, float* dgamma, float* dbeta, int64_t rows, int64_t cols, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+    if (int e = check_rows("layernorm_backward", rows, cols)) return e;
+    if (cols == 0) return 0;
+    DML_REQUIRE(dgamma && dbeta, DMLHIP_ERR_NULL, "layernorm_backward: NULL gradient pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (rows == 0) {
+        hipLaunchKernelGGL(layernorm_bwd_finish_kernel, (unsigned)ceil_div(cols, 256), 256, 0, st, (const float*)nullptr,
+                           dgamma, dbeta, 0, (int)cols);
+        return launch_status("layernorm_backward");
+    }
+    DML_REQUIRE(dy && x && mean && rstd && gamma && dx, DMLHIP_ERR_NULL, "layernorm_backward: NULL tensor pointer");
+    DML_REQUIRE(cols <= 2147483647, DMLHIP_ERR_SHAPE, "layernorm_backward: cols too large");
+    const size_t need = dmlhip_layernorm_backward_workspace_bytes(rows, cols);
+    DML_REQUIRE(workspace && workspace_bytes >= need, DMLHIP_ERR_WORKSPACE,
+                "layernorm_backward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    const T *gp = (const T*)dy, *xp = (const T*)x, *gm = (const T*)gamma;
+    T* dp = (T*)dx;
+    float* part = (float*)workspace;
+    const int parts = ln_bwd_parts(rows);
+    constexpr int VN = VecOf<T>::n;
+    const bool al = aligned16(dy) && aligned16(x) && aligned16(gamma) && aligned16(dx);
+    const size_t lds = (size_t)2 * kRowsPerBlock * cols * sizeof(float);
+    if (wave_path_ok<T>(cols, 4) && al && lds <= 64 * 1024) {
+        const int vpl = (int)ceil_div(cols, kWave * VN);
+#define DML_LNB_LAUNCH(V) hipLaunchKernelGGL((layernorm_bwd_wave_kernel<T, V>), (unsigned)parts, kRowBlock, lds, st, gp, xp, mean, rstd, gm, dp, part, rows, (int)cols)
+        switch (vpl) {
+            case 1: DML_LNB_LAUNCH(1); break;
+            case 2: DML_LNB_LAUNCH(2); break;
+            case 3: DML_LNB_LAUNCH(3); break;
+            default: DML_LNB_LAUNCH(4); break;
+        }
+#undef DML_LNB_LAUNCH
+    } else {
+        DML_REQUIRE(rows <= 2147483647, DMLHIP_ERR_SHAPE, "layernorm_backward: too many rows for the generic path");
+        hipLaunchKernelGGL((layernorm_bwd_dx_block_kernel<T>), (unsigned)rows, kRowBlock, 0, st, gp, xp, mean, rstd, gm,
+                           dp, cols);
+        if (int e = launch_status("layernorm_backward(dx)")) return e;
+        dim3 grid((unsigned)ceil_div(cols, 256), (unsigned)parts);
+        hipLaunchKernelGGL((layernorm_bwd_cols_kernel<T>), grid, 256, 0, st, gp, xp, mean, rstd, part, rows, cols);
+    }
+    if (int e = launch_status("layernorm_backward(stage 1)")) return e;
+    hipLaunchKernelGGL(layernorm_bwd_finish_kernel, (unsigned)ceil_div(cols, 256), 256, 0, st, (const float*)part,
+                       dgamma, dbeta, parts, (int)cols);
+    return launch_status("layernorm_backward(stage 2)");
+}
+
+}  // namespace
+}  // namespace dml
+
+using namespace dml;
+
+extern "C" {
+
+int dmlhip_softmax_f16(const void* x, void* y, int64_t rows, int64_t cols, void* stream) {
+    return softmax_impl<_Float16>(x, y, rows, cols, stream);
+}
+int dmlhip_softmax_f32(const void* x, void* y, int64_t rows, int64_t cols, void* stream) {
+    return softmax_impl<float>(x, y, rows, cols, stream);
+}
+int dmlhip_softmax_backward_f16(const void* y, const void* dy, void* dx, int64_t rows, int64_t cols, void* stream) {
+    return softmax_bwd_impl<_Float16>(y, dy, dx, rows, cols, stream);
+}
+int dmlhip_softmax_backward_f32(const void* y, const void* dy, void* dx, int64_t rows, int64_t cols, void* stream) {
+    return softmax_bwd_impl<float>(y, dy, dx, rows, cols, stream);
+}
+int dmlhip_layernorm_f16(const void* x, const void* residual, const void* gamma, const void* beta, void* y,
+                         void* sum_out, float* mean, float* rstd, int64_t rows, int64_t cols, float eps,
+                         void* stream) {
+    return layernorm_impl<_Float16>(x, residual, gamma, beta, y, sum_out, mean, rstd, rows, cols, eps, stream);
+}
+int dmlhip_layernorm_f32(const void* x, const void* residual, const void* gamma, const void* beta, void* y,
+                         void* sum_out, float* mean, float* rstd, int64_t rows, int64_t cols, float eps,
+                         void* stream) {
+    return layernorm_impl<float>(x, residual, gamma, beta, y, sum_out, mean, rstd, rows, cols, eps, stream);
+}
+size_t dmlhip_layernorm_backward_workspace_bytes(int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    return (size_t)ln_bwd_parts(rows) * 2 * (size_t)cols * sizeof(float);
+}
+int dmlhip_layernorm_backward_f16(const void* dy, const void* x, const float* mean, const float* rstd,
+                                  const void* gamma, void* dx, float* dgamma, float* dbeta, int64_t rows,
+                                  int64_t cols, void* workspace, size_t workspace_bytes, void* stream) {
+    return layernorm_bwd_impl<_Float16>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, rows, cols, workspace,
+                                        workspace_bytes, stream);
+}
+int dmlhip_layernorm_backward_f32(const void* dy, const void* x, const float* mean, const float* rstd,
+                                  const void* gamma, void* dx, float* dgamma, float* dbeta, int64_t rows,
+                                  int64_t cols, void* workspace, size_t workspace_bytes, void* stream) {
+    return layernorm_bwd_impl<float>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, rows, cols, workspace,
+                                     workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,419 @@
+"""Tensor-level launchers: torch tensors in, one dmlhip_* call each.
+
+PyTorch is used here only for device memory and the current HIP stream. Every function checks
+device / dtype / layout, allocates the outputs (``torch.empty``, as the reference dispatcher does,
+daceml/torch/dispatchers/ctypes_module.py:53-69), and calls the C ABI. There is no fallback: a
+missing library or a non-zero status raises.
+"""
+import ctypes
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib as L
+
+_SUFFIX = {torch.float16: "f16", torch.float32: "f32"}
+_CODE = {torch.float16: L.F16, torch.float32: L.F32}
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _fn(name: str, dtype: torch.dtype):
+    try:
+        return getattr(L.load(), "dmlhip_%s_%s" % (name, _SUFFIX[dtype]))
+    except KeyError:
+        raise TypeError("dtype %s not supported by the HIP kernels (float16 / float32 only)" % dtype)
+
+
+def _check(*tensors, dtype=None):
+    first = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("HIP kernels need device tensors; got a %s tensor" % t.device)
+        if first is None:
+            first = t
+        elif t.device != first.device:
+            raise ValueError("tensors live on different devices")
+        if dtype is not None and t.dtype != dtype:
+            raise TypeError("expected dtype %s, got %s" % (dtype, t.dtype))
+
+
+def _dense(t: torch.Tensor) -> torch.Tensor:
+    # inputs are forced contiguous, as in ctypes_module.py:58
+    return t if t.is_contiguous() else t.contiguous()
+
+
+_workspaces = {}
+
+
+def workspace(nbytes: int, device) -> torch.Tensor:
+    """Per-device scratch buffer, grown on demand and reused (kernels on one stream are ordered)."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+# ----------------------------------------------------------------------------- row-wise
+def softmax(x: torch.Tensor, axis: int = -1, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """opset-12 Softmax: coalesce to [prod(shape[:axis]), prod(shape[axis:])]."""
+    _check(x, out)
+    x = _dense(x)
+    axis = axis % x.dim() if x.dim() else 0
+    cols = 1
+    for s in x.shape[axis:]:
+        cols *= s
+    rows = x.numel() // cols if cols else 0
+    y = torch.empty_like(x) if out is None else out
+    L.check(_fn("softmax", x.dtype)(_ptr(x), _ptr(y), rows, cols, _stream()))
+    return y
+
+
+def softmax_backward(y: torch.Tensor, dy: torch.Tensor, axis: int = -1) -> torch.Tensor:
+    _check(y, dy, dtype=y.dtype)
+    y, dy = _dense(y), _dense(dy)
+    axis = axis % y.dim()
+    if axis != y.dim() - 1:
+        raise NotImplementedError("softmax backward reduces over the single axis `axis`; only the last axis is fused")
+    cols = y.shape[-1]
+    rows = y.numel() // cols if cols else 0
+    dx = torch.empty_like(y)
+    L.check(_fn("softmax_backward", y.dtype)(_ptr(y), _ptr(dy), _ptr(dx), rows, cols, _stream()))
+    return dx
+
+
+def layernorm(x, gamma, beta, eps=1e-5, residual=None, want_sum=False, want_stats=False):
+    """Returns (y, sum_or_None, mean_or_None, rstd_or_None); normalises over the last axis."""
+    _check(x, gamma, beta, residual, dtype=x.dtype)
+    x, gamma, beta = _dense(x), _dense(gamma), _dense(beta)
+    if residual is not None:
+        residual = _dense(residual)
+        if residual.shape != x.shape:
+            raise ValueError("residual must have the shape of x")
+    cols = x.shape[-1]
+    if gamma.numel() != cols or beta.numel() != cols:
+        raise ValueError("gamma/beta must have %d elements" % cols)
+    rows = x.numel() // cols if cols else 0
+    y = torch.empty_like(x)
+    s = torch.empty_like(x) if want_sum else None
+    mean = torch.empty(rows, dtype=torch.float32, device=x.device) if want_stats else None
+    rstd = torch.empty(rows, dtype=torch.float32, device=x.device) if want_stats else None
+    L.check(_fn("layernorm", x.dtype)(_ptr(x), _ptr(residual), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(s), _ptr(mean),
+                                      _ptr(rstd), rows, cols, float(eps), _stream()))
+    return y, s, mean, rstd
+
+
+def layernorm_backward(dy, x, mean, rstd, gamma):
+    """Returns (dx, dgamma_fp32, dbeta_fp32)."""
+    _check(dy, x, gamma, dtype=x.dtype)
+    _check(mean, rstd, dtype=torch.float32)
+    dy, x, gamma = _dense(dy), _dense(x), _dense(gamma)
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    dx = torch.empty_like(x)
+    dgamma = torch.empty(cols, dtype=torch.float32, device=x.device)
+    dbeta = torch.empty(cols, dtype=torch.float32, device=x.device)
+    need = L.load().dmlhip_layernorm_backward_workspace_bytes(rows, cols)
+    ws = workspace(need, x.device)
+    L.check(_fn("layernorm_backward", x.dtype)(_ptr(dy), _ptr(x), _ptr(mean), _ptr(rstd), _ptr(gamma), _ptr(dx),
+                                               _ptr(dgamma), _ptr(dbeta), rows, cols, _ptr(ws), ws.numel(), _stream()))
+    return dx, dgamma, dbeta
+
+
+# ----------------------------------------------------------------------------- elementwise
+def _bcast_strides(t: torch.Tensor, shape: Sequence[int]):
+    nd = len(shape)
+    pad = nd - t.dim()
+    if pad < 0:
+        raise ValueError("operand has more dims than the output")
+    strides = []
+    for i in range(nd):
+        if i < pad:
+            strides.append(0)
+            continue
+        ext, st = t.shape[i - pad], t.stride(i - pad)
+        if ext == shape[i]:
+            strides.append(st if ext != 1 else 0)
+        elif ext == 1:
+            strides.append(0)
+        else:
+            raise ValueError("shapes %s and %s do not broadcast" % (tuple(t.shape), tuple(shape)))
+    return strides
+
+
+def binary(op: int, a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _check(a, b, out, dtype=a.dtype)
+    a, b = _dense(a), _dense(b)
+    shape = torch.broadcast_shapes(a.shape, b.shape)
+    if len(shape) > L.MAX_DIMS:
+        raise NotImplementedError("more than %d dims" % L.MAX_DIMS)
+    c = torch.empty(shape, dtype=a.dtype, device=a.device) if out is None else out
+    sa, sb = _bcast_strides(a, shape), _bcast_strides(b, shape)
+    L.check(_fn("binary", a.dtype)(op, _ptr(a), _ptr(b), _ptr(c), len(shape), L.i64_array(shape), L.i64_array(sa),
+                                   L.i64_array(sb), _stream()))
+    return c
+
+
+def unary(op: int, x: torch.Tensor, param: float = 0.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _check(x, out)
+    x = _dense(x)
+    y = torch.empty_like(x) if out is None else out
+    L.check(_fn("unary", x.dtype)(op, _ptr(x), _ptr(y), x.numel(), float(param), _stream()))
+    return y
+
+
+def unary_backward(op: int, x: torch.Tensor, dy: torch.Tensor, param: float = 0.0) -> torch.Tensor:
+    _check(x, dy, dtype=x.dtype)
+    x, dy = _dense(x), _dense(dy)
+    dx = torch.empty_like(x)
+    L.check(_fn("unary_backward", x.dtype)(op, _ptr(x), _ptr(dy), _ptr(dx), x.numel(), float(param), _stream()))
+    return dx
+
+
+def sum_variadic(inputs: Sequence[torch.Tensor]) -> torch.Tensor:
+    if not inputs:
+        raise ValueError("Sum needs at least one input")
+    _check(*inputs, dtype=inputs[0].dtype)
+    shape = inputs[0].shape
+    for t in inputs:
+        if t.shape != shape:
+            raise ValueError("Sum: all inputs must have the output's shape (no broadcasting)")
+    tensors = [_dense(t) for t in inputs]
+    out = torch.empty_like(tensors[0])
+    fn = _fn("sum", out.dtype)
+    first = True
+    i = 0
+    while i < len(tensors):  # eight inputs per launch; later launches fold the running sum in
+        chunk = tensors[i:i + (8 if first else 7)]
+        ptrs = ([] if first else [out]) + chunk
+        arr = (ctypes.c_void_p * len(ptrs))(*[t.data_ptr() for t in ptrs])
+        L.check(fn(arr, len(ptrs), _ptr(out), out.numel(), _stream()))
+        i += len(chunk)
+        first = False
+    return out
+
+
+def bias_gelu(x: torch.Tensor, bias: Optional[torch.Tensor], want_pre: bool = False):
+    _check(x, bias, dtype=x.dtype)
+    x = _dense(x)
+    cols = x.shape[-1]
+    if bias is not None:
+        bias = _dense(bias)
+        if bias.numel() != cols:
+            raise ValueError("bias must have %d elements" % cols)
+    rows = x.numel() // cols if cols else 0
+    y = torch.empty_like(x)
+    pre = torch.empty_like(x) if want_pre else None
+    L.check(_fn("bias_gelu", x.dtype)(_ptr(x), _ptr(bias), _ptr(y), _ptr(pre), rows, cols, _stream()))
+    return y, pre
+
+
+def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    _check(x)
+    x = _dense(x)
+    y = torch.empty(x.shape, dtype=dtype, device=x.device)
+    L.check(L.load().dmlhip_cast(_CODE[x.dtype], _CODE[dtype], _ptr(x), _ptr(y), x.numel(), _stream()))
+    return y
+
+
+# ----------------------------------------------------------------------------- reductions / transpose
+def reduce(op: int, x: torch.Tensor, axes: Optional[Sequence[int]], keepdims: bool = True,
+           out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Reduce over `axes` (must be adjacent after normalisation; None = all)."""
+    _check(x)
+    x = _dense(x)
+    nd = x.dim()
+    axes = sorted(set(range(nd) if axes is None else [a % nd for a in axes]))
+    if not axes:
+        raise ValueError("empty axes")
+    if axes != list(range(axes[0], axes[-1] + 1)):
+        raise NotImplementedError("reduced axes must be adjacent")
+    outer = 1
+    for s in x.shape[:axes[0]]:
+        outer *= s
+    r = 1
+    for a in axes:
+        r *= x.shape[a]
+    inner = 1
+    for s in x.shape[axes[-1] + 1:]:
+        inner *= s
+    out_dtype = out_dtype or x.dtype
+    kept = [1 if i in axes else s for i, s in enumerate(x.shape)]
+    dropped = [s for i, s in enumerate(x.shape) if i not in axes]
+    y = torch.empty(kept if keepdims else dropped, dtype=out_dtype, device=x.device)
+    lib = L.load()
+    need = lib.dmlhip_reduce_workspace_bytes(outer, r, inner)
+    ws = workspace(need, x.device) if need else None
+    if inner > 1 and outer > 65535:
+        raise NotImplementedError("column reduction with more than 65535 outer slices")
+    L.check(_fn("reduce", x.dtype)(op, _ptr(x), _ptr(y), _CODE[out_dtype], outer, r, inner, _ptr(ws),
+                                   ws.numel() if ws is not None else 0, _stream()))
+    return y
+
+
+def transpose(x: torch.Tensor, perm: Optional[Sequence[int]] = None) -> torch.Tensor:
+    _check(x)
+    x = _dense(x)
+    nd = x.dim()
+    perm = list(reversed(range(nd))) if perm is None else [p % nd for p in perm]
+    if nd > L.MAX_DIMS:
+        raise NotImplementedError("more than %d dims" % L.MAX_DIMS)
+    y = torch.empty([x.shape[p] for p in perm], dtype=x.dtype, device=x.device)
+    L.check(_fn("transpose", x.dtype)(_ptr(x), _ptr(y), nd, L.i64_array(x.shape), L.i64_array(perm), _stream()))
+    return y
+
+
+# ----------------------------------------------------------------------------- contraction
+def gemm(desc: "L.GemmDesc", a, b, c, bias=None, residual=None, pre_out=None):
+    """Raw strided-batched GEMM; `desc` fully describes operand layout."""
+    _check(a, b, c, bias, residual, pre_out)
+    if a.dtype != b.dtype:
+        raise TypeError("operand dtypes differ")
+    L.check(_fn("gemm", a.dtype)(ctypes.byref(desc), _ptr(a), _ptr(b), _ptr(c), _ptr(bias), _ptr(residual),
+                                 _ptr(pre_out), _stream()))
+    return c
+
+
+def _fill_desc(plan, alpha, beta, out_dtype, bias, act) -> "L.GemmDesc":
+    d = L.GemmDesc()
+    d.m, d.n, d.k = plan.m, plan.n, plan.k
+    for i in range(3):
+        d.batch[i] = plan.batch[i]
+        d.a_stride_batch[i] = plan.a_stride_batch[i]
+        d.b_stride_batch[i] = plan.b_stride_batch[i]
+        d.c_stride_batch[i] = plan.c_stride_batch[i]
+    d.a_stride_m, d.a_stride_k = plan.a_stride_m, plan.a_stride_k
+    d.b_stride_k, d.b_stride_n = plan.b_stride_k, plan.b_stride_n
+    d.c_stride_m = plan.c_stride_m
+    d.alpha, d.beta = float(alpha), float(beta)
+    d.out_dtype = _CODE[out_dtype]
+    d.bias_dtype = _CODE[bias.dtype] if bias is not None else L.F16
+    d.act = act
+    return d
+
+
+def einsum(equation: str, a: torch.Tensor, b: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+           out_dtype: Optional[torch.dtype] = None, alpha: float = 1.0, beta: float = 0.0,
+           bias: Optional[torch.Tensor] = None, act: int = L.ACT_NONE, residual: Optional[torch.Tensor] = None,
+           pre_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Two-operand einsum as one strided batched GEMM launch.
+
+    Operands are used with the strides they have (views are not copied). `bias` is indexed by the
+    innermost output index. When one launch cannot express the equation the operands are first
+    re-laid-out with the transpose kernel (still no host fallback).
+    """
+    from . import contraction as C
+    _check(a, b, out, bias, residual, pre_out)
+    if a.dtype != b.dtype:
+        raise TypeError("einsum operands must share a dtype")
+    out_dtype = out_dtype or a.dtype
+    if a.dtype == torch.float32 and out_dtype != torch.float32:
+        raise TypeError("fp32 contractions produce fp32")
+    try:
+        plan = C.plan_contraction(equation, a.shape, a.stride(), b.shape, b.stride())
+    except C.NotApplicable:
+        if bias is not None or residual is not None or pre_out is not None or out is not None or beta != 0.0:
+            raise
+        return _einsum_via_relayout(equation, a, b, out_dtype, alpha, act)
+    if out is None:
+        out = torch.empty(plan.out_shape, dtype=out_dtype, device=a.device)
+    else:
+        if tuple(out.shape) != tuple(plan.out_shape) or not out.is_contiguous() or out.dtype != out_dtype:
+            raise ValueError("`out` must be a dense %s tensor of shape %s" % (out_dtype, plan.out_shape))
+    for t in (residual, pre_out):
+        if t is not None and (tuple(t.shape) != tuple(plan.out_shape) or not t.is_contiguous()
+                              or t.dtype != out_dtype):
+            raise ValueError("residual / pre_out must match the output's shape, dtype and layout")
+    if bias is not None and (bias.dim() != 1 or bias.numel() != plan.n or not bias.is_contiguous()):
+        raise ValueError("bias must be a dense vector over the innermost output index")
+    x, y = (b, a) if plan.swapped else (a, b)
+    desc = _fill_desc(plan, alpha, beta, out_dtype, bias, act)
+    return gemm(desc, x, y, out, bias, residual, pre_out)
+
+
+def _einsum_via_relayout(equation, a, b, out_dtype, alpha, act):
+    from . import contraction as C
+    (ta, tb), out = C.parse(equation)
+    batch = [l for l in out if l in ta and l in tb]
+    m_let = [l for l in out if l in ta and l not in tb]
+    n_let = [l for l in out if l in tb and l not in ta]
+    k_let = [l for l in ta if l in tb and l not in out]
+    na = "".join(batch + m_let + k_let)
+    nb = "".join(batch + k_let + n_let)
+    no = "".join(batch + m_let + n_let)
+    if sorted(na) != sorted(ta) or sorted(nb) != sorted(tb):
+        raise C.NotApplicable("index summed inside a single operand: %s" % equation)
+    a2 = transpose(a, [ta.index(l) for l in na])
+    b2 = transpose(b, [tb.index(l) for l in nb])
+    res = einsum("%s,%s->%s" % (na, nb, no), a2, b2, out_dtype=out_dtype, alpha=alpha, act=act)
+    if no != out:
+        res = transpose(res, [no.index(l) for l in out])
+    return res
+
+
+# ----------------------------------------------------------------------------- convolution
+def _conv_desc(x_shape, w_shape, strides, pads, dilations, group, act) -> "L.Conv2dDesc":
+    if len(x_shape) != 4 or len(w_shape) != 4:
+        raise NotImplementedError("only 2-D convolutions (NCHW / OIHW)")
+    pads = list(pads)
+    if len(pads) == 4:
+        if pads[0] != pads[2] or pads[1] != pads[3]:
+            raise NotImplementedError("asymmetric pads")
+        pads = pads[:2]
+    d = L.Conv2dDesc()
+    d.n, d.c, d.h, d.w = [int(v) for v in x_shape]
+    d.m, d.kh, d.kw = int(w_shape[0]), int(w_shape[2]), int(w_shape[3])
+    d.stride_h, d.stride_w = [int(v) for v in strides]
+    d.pad_h, d.pad_w = [int(v) for v in pads]
+    d.dil_h, d.dil_w = [int(v) for v in dilations]
+    d.group = int(group)
+    d.act = act
+    if int(w_shape[1]) * d.group != d.c:
+        raise ValueError("weight has %d input channels per group, expected %d" % (w_shape[1], d.c // max(d.group, 1)))
+    return d
+
+
+def conv_out_shape(desc: "L.Conv2dDesc"):
+    oh, ow = ctypes.c_int64(), ctypes.c_int64()
+    L.check(L.load().dmlhip_conv2d_out_shape(ctypes.byref(desc), ctypes.byref(oh), ctypes.byref(ow)))
+    return oh.value, ow.value
+
+
+def conv2d(x, w, bias=None, strides=(1, 1), pads=(0, 0), dilations=(1, 1), group=1, act: int = L.ACT_NONE):
+    _check(x, w, bias, dtype=x.dtype)
+    x, w = _dense(x), _dense(w)
+    bias = None if bias is None else _dense(bias)
+    d = _conv_desc(x.shape, w.shape, strides, pads, dilations, group, act)
+    oh, ow = conv_out_shape(d)
+    y = torch.empty((d.n, d.m, oh, ow), dtype=x.dtype, device=x.device)
+    L.check(_fn("conv2d", x.dtype)(ctypes.byref(d), _ptr(x), _ptr(w), _ptr(bias), _ptr(y), _stream()))
+    return y
+
+
+def conv2d_backward(x, w, dy, strides=(1, 1), pads=(0, 0), dilations=(1, 1), group=1, need_dx=True, need_dw=True):
+    """Returns (dx or None, dw or None); fp32 only."""
+    _check(x, w, dy, dtype=torch.float32)
+    x, w, dy = _dense(x), _dense(w), _dense(dy)
+    d = _conv_desc(x.shape, w.shape, strides, pads, dilations, group, L.ACT_NONE)
+    lib = L.load()
+    dx = dw = None
+    if need_dx:
+        dx = torch.empty_like(x)
+        L.check(lib.dmlhip_conv2d_backward_data_f32(ctypes.byref(d), _ptr(dy), _ptr(w), _ptr(dx), _stream()))
+    if need_dw:
+        dw = torch.empty_like(w)
+        need = lib.dmlhip_conv2d_backward_weight_workspace_bytes(ctypes.byref(d))
+        ws = workspace(need, x.device) if need else None
+        L.check(lib.dmlhip_conv2d_backward_weight_f32(ctypes.byref(d), _ptr(x), _ptr(dy), _ptr(dw), _ptr(ws),
+                                                      ws.numel() if ws is not None else 0, _stream()))
+    return dx, dw

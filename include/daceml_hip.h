@@ -1,0 +1,231 @@
+/*
+ * daceml_hip.h — C ABI of libdaceml_hip.so: hand-written gfx950 (MI355X) kernels for the
+ * ONNX library-node hot path of DaCeML.
+ *
+ * The reference (spcl/daceml) has no compiled sources; what these entry points replace are
+ * the *call sites* through which its expansions reach native code:
+ *   - the SDFG that a "pure" expansion returns and DaCe compiles
+ *     (daceml/onnx/op_implementations/pure_implementations.py, img_op_implementations.py),
+ *   - the cuDNN calls emitted as C++ tasklets
+ *     (daceml/onnx/op_implementations/cudnn_implementations.py:360-410),
+ *   - cuBLAS reached through DaCe's BLAS library nodes
+ *     (daceml/util/utils.py:226-229).
+ * Each declaration cites the reference expansion whose semantics it implements.
+ *
+ * Calling convention
+ *   - tensors are dense row-major device pointers unless strides are passed explicitly;
+ *   - every call is asynchronous on `stream` (a hipStream_t passed as void*; NULL = the
+ *     null stream), never synchronises, never allocates or frees, and never keeps a pointer;
+ *   - scratch memory is caller-provided and sized by the matching *_workspace_bytes query;
+ *   - return value: 0 = launched; < 0 = argument error detected on the host before any device
+ *     work (safe to call on a machine without a GPU); > 0 = hipError_t of a failed launch.
+ *     dmlhip_last_error_string() describes the last failure on the calling thread.
+ *   - "_f16" entry points read/write IEEE half and always compute and accumulate in fp32
+ *     (the effect of daceml/transformation/mixed_precision.py:5-35); "_f32" entry points
+ *     are fp32 end to end with no fast-math (daceml/__init__.py:13-19).
+ */
+#ifndef DACEML_HIP_H
+#define DACEML_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DMLHIP_VERSION 100 /* major*10000 + minor*100 + patch */
+#define DMLHIP_MAX_DIMS 6
+
+enum {
+    DMLHIP_OK = 0,
+    DMLHIP_ERR_NULL = -1,        /* a required pointer is NULL */
+    DMLHIP_ERR_SHAPE = -2,       /* negative / inconsistent / overflowing extents */
+    DMLHIP_ERR_UNSUPPORTED = -3, /* valid ONNX, but outside what the kernels cover */
+    DMLHIP_ERR_ALIGN = -4,       /* pointer or stride alignment requirement violated */
+    DMLHIP_ERR_WORKSPACE = -5,   /* workspace NULL or smaller than the query says */
+    DMLHIP_ERR_ENUM = -6         /* unknown op / dtype / epilogue code */
+};
+
+/* element types used for "out_dtype"/"bias_dtype" style arguments */
+enum { DMLHIP_F16 = 0, DMLHIP_F32 = 1 };
+
+int dmlhip_version(void);
+const char* dmlhip_last_error_string(void);
+
+/* ------------------------------------------------------------------ Softmax
+ * Softmax "pure": pure_implementations.py:309-319. The caller coalesces
+ * [shape[:axis], shape[axis:]] into rows x cols (opset-12 semantics); y = exp(x-max)/sum. */
+int dmlhip_softmax_f16(const void* x, void* y, int64_t rows, int64_t cols, void* stream);
+int dmlhip_softmax_f32(const void* x, void* y, int64_t rows, int64_t cols, void* stream);
+
+/* DefaultSoftmaxBackward: autodiff/implementations/onnx_ops.py:237-275.
+ * dx = y*dy - y*sum_row(y*dy), in one pass. */
+int dmlhip_softmax_backward_f16(const void* y, const void* dy, void* dx, int64_t rows,
+                                int64_t cols, void* stream);
+int dmlhip_softmax_backward_f32(const void* y, const void* dy, void* dx, int64_t rows,
+                                int64_t cols, void* stream);
+
+/* ------------------------------------------------------------------ LayerNormalization
+ * The opset-12 export has no LayerNormalization node; the reference runs the chain
+ * ReduceMean, Sub, Pow, ReduceMean, Add, Sqrt, Div, Mul, Add
+ * (pure_implementations.py:101-103,81-83,39-41,76-78,34-36,91-93). This is that chain fused:
+ * mu = mean(s), var = mean((s-mu)^2) (biased, two-pass), y = (s-mu)/sqrt(var+eps)*gamma+beta,
+ * with s = x (+ residual when residual != NULL: the preceding ONNXAdd fused in).
+ * Optional outputs (NULL to skip): sum_out = s (same dtype as x), mean / rstd = per-row
+ * fp32 statistics for the backward node. */
+int dmlhip_layernorm_f16(const void* x, const void* residual, const void* gamma,
+                         const void* beta, void* y, void* sum_out, float* mean, float* rstd,
+                         int64_t rows, int64_t cols, float eps, void* stream);
+int dmlhip_layernorm_f32(const void* x, const void* residual, const void* gamma,
+                         const void* beta, void* y, void* sum_out, float* mean, float* rstd,
+                         int64_t rows, int64_t cols, float eps, void* stream);
+
+/* Backward of the chain above (what the SymPy tasklet reversal of
+ * autodiff/backward_pass_generator.py:1284-1421 plus ReverseReduce, dace_nodes.py:13-105,
+ * compute as many small maps). dx has x's dtype; dgamma/dbeta are fp32 master gradients
+ * (overwritten, not accumulated). Needs a workspace. */
+size_t dmlhip_layernorm_backward_workspace_bytes(int64_t rows, int64_t cols);
+int dmlhip_layernorm_backward_f16(const void* dy, const void* x, const float* mean,
+                                  const float* rstd, const void* gamma, void* dx,
+                                  float* dgamma, float* dbeta, int64_t rows, int64_t cols,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+int dmlhip_layernorm_backward_f32(const void* dy, const void* x, const float* mean,
+                                  const float* rstd, const void* gamma, void* dx,
+                                  float* dgamma, float* dbeta, int64_t rows, int64_t cols,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ elementwise
+ * Add/Sub/Mul/Div/Pow "pure": pure_implementations.py:39-41,76-93 (NumPy broadcasting).
+ * `shape` is the broadcast output shape (ndim <= DMLHIP_MAX_DIMS); a_strides / b_strides are
+ * element strides per output dim, 0 where the operand is broadcast. c is dense. */
+enum { DMLHIP_ADD = 0, DMLHIP_SUB = 1, DMLHIP_MUL = 2, DMLHIP_DIV = 3, DMLHIP_POW = 4 };
+int dmlhip_binary_f16(int op, const void* a, const void* b, void* c, int ndim,
+                      const int64_t* shape, const int64_t* a_strides,
+                      const int64_t* b_strides, void* stream);
+int dmlhip_binary_f32(int op, const void* a, const void* b, void* c, int ndim,
+                      const int64_t* shape, const int64_t* a_strides,
+                      const int64_t* b_strides, void* stream);
+
+/* Unary maps: Erf (pure_implementations.py:106-108), Sqrt (:34-36), Exp/Log (:24-31),
+ * Tanh (:289-291), Relu (:556-560), Sigmoid (:741-743), Reciprocal (:283-286).
+ * GELU = the exported chain Div,Erf,Add,Mul,Mul fused: 0.5*x*(1+erf(x/sqrt(2))).
+ * SWISH = Mul(x, Sigmoid(x)) fused. SCALE: y = x*param (Mul/Div by a scalar constant). */
+enum {
+    DMLHIP_ERF = 0, DMLHIP_SQRT = 1, DMLHIP_EXP = 2, DMLHIP_LOG = 3, DMLHIP_TANH = 4,
+    DMLHIP_RELU = 5, DMLHIP_SIGMOID = 6, DMLHIP_RECIPROCAL = 7, DMLHIP_GELU = 8,
+    DMLHIP_SWISH = 9, DMLHIP_SCALE = 10, DMLHIP_IDENTITY = 11
+};
+int dmlhip_unary_f16(int op, const void* x, void* y, int64_t n, float param, void* stream);
+int dmlhip_unary_f32(int op, const void* x, void* y, int64_t n, float param, void* stream);
+
+/* Backward of the unary maps above that have one (GELU, SWISH, SIGMOID, RELU, TANH, ERF, SCALE):
+ * dx = dy * f'(x), x being the forward *input*. */
+int dmlhip_unary_backward_f16(int op, const void* x, const void* dy, void* dx, int64_t n,
+                              float param, void* stream);
+int dmlhip_unary_backward_f32(int op, const void* x, const void* dy, void* dx, int64_t n,
+                              float param, void* stream);
+
+/* PureSum: pure_implementations.py:584-646 — variadic same-shape sum, 1..8 inputs. */
+int dmlhip_sum_f16(const void* const* inputs, int n_inputs, void* out, int64_t n, void* stream);
+int dmlhip_sum_f32(const void* const* inputs, int n_inputs, void* out, int64_t n, void* stream);
+
+/* Add(bias[cols]) followed by the GELU chain, fused; bias may be NULL.
+ * pre_out (nullable) receives x+bias, which the backward needs. */
+int dmlhip_bias_gelu_f16(const void* x, const void* bias, void* y, void* pre_out, int64_t rows,
+                         int64_t cols, void* stream);
+int dmlhip_bias_gelu_f32(const void* x, const void* bias, void* y, void* pre_out, int64_t rows,
+                         int64_t cols, void* stream);
+
+/* Cast "pure": pure_implementations.py:329-377, between DMLHIP_F16 and DMLHIP_F32. */
+int dmlhip_cast(int src_dtype, int dst_dtype, const void* x, void* y, int64_t n, void* stream);
+
+/* ------------------------------------------------------------------ reductions
+ * ReduceSum/Max/Min/Mean "pure": pure_implementations.py:101-103,294-306;
+ * GlobalAveragePool "pure": img_op_implementations.py:415-417 (= MEAN with inner 1).
+ * Input viewed as [outer, r, inner] (the reduced axes must be adjacent; the caller collapses
+ * them); output [outer, inner] of out_dtype. Accumulates in fp32. */
+enum { DMLHIP_RSUM = 0, DMLHIP_RMAX = 1, DMLHIP_RMIN = 2, DMLHIP_RMEAN = 3 };
+size_t dmlhip_reduce_workspace_bytes(int64_t outer, int64_t r, int64_t inner);
+int dmlhip_reduce_f16(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r,
+                      int64_t inner, void* workspace, size_t workspace_bytes, void* stream);
+int dmlhip_reduce_f32(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r,
+                      int64_t inner, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ Transpose
+ * Transpose "pure"/"einsum": pure_implementations.py:322-326,746-778.
+ * y = transpose(x, perm); `shape` is x's shape, ndim <= DMLHIP_MAX_DIMS. */
+int dmlhip_transpose_f16(const void* x, void* y, int ndim, const int64_t* shape,
+                         const int64_t* perm, void* stream);
+int dmlhip_transpose_f32(const void* x, void* y, int ndim, const int64_t* shape,
+                         const int64_t* perm, void* stream);
+
+/* ------------------------------------------------------------------ contractions
+ * PureEinsum / PureMatMul / PureGemm: pure_implementations.py:111-252,380-553, which the
+ * reference lowers to cuBLAS (strided-batched) GEMM through DaCe. One strided, batched GEMM:
+ *
+ *   C[b0,b1,b2][m,n] = epilogue( alpha * sum_k A[b...][m,k] * B[b...][k,n] ) (+ beta*C)
+ *
+ * with arbitrary element strides for m/k/n in A and B (so the Transpose nodes around a
+ * contraction fold into operand layout, the effect of transformation/einsum_fusion.py:102-151)
+ * and unit stride for n in C. Products accumulate in fp32 on MFMA.
+ * epilogue: v = alpha*acc; if bias: v += bias[n] (or bias[m]); if pre_out: pre_out[m,n] = v;
+ *           v = act(v); if residual: v += residual[m,n]; if beta: v += beta*C;
+ */
+enum {
+    DMLHIP_ACT_NONE = 0, DMLHIP_ACT_GELU = 1, DMLHIP_ACT_SWISH = 2, DMLHIP_ACT_SIGMOID = 3,
+    DMLHIP_ACT_RELU = 4
+};
+typedef struct dmlhip_gemm_desc {
+    int64_t m, n, k;
+    int64_t batch[3];       /* batch extents; use 1 for unused dims */
+    int64_t a_stride_m, a_stride_k, a_stride_batch[3];
+    int64_t b_stride_k, b_stride_n, b_stride_batch[3];
+    int64_t c_stride_m, c_stride_batch[3]; /* stride of n in C is 1 */
+    float alpha, beta;
+    int out_dtype;          /* DMLHIP_F16 or DMLHIP_F32: type of C, pre_out and residual */
+    int bias_dtype;         /* type of bias[n] */
+    int act;                /* DMLHIP_ACT_* */
+    int bias_along_m;       /* 0: bias[n] (Linear / Gemm C vector); 1: bias[m] (conv channel bias) */
+} dmlhip_gemm_desc;
+/* inputs fp16 */
+int dmlhip_gemm_f16(const dmlhip_gemm_desc* desc, const void* a, const void* b, void* c,
+                    const void* bias, const void* residual, void* pre_out, void* stream);
+/* inputs fp32, true fp32 MFMA (no reduced-precision path); out_dtype must be DMLHIP_F32 */
+int dmlhip_gemm_f32(const dmlhip_gemm_desc* desc, const void* a, const void* b, void* c,
+                    const void* bias, const void* residual, void* pre_out, void* stream);
+
+/* ------------------------------------------------------------------ Conv
+ * ONNX Conv, 2-D, NCHW / OIHW, cross-correlation:
+ *   Y[b,m,oy,ox] = B[m] + sum_{c,hy,hx} W[m,c,hy,hx] * X[b, g*C/G+c, oy*sy-pt+hy*dy, ox*sx-pl+hx*dx]
+ * PureConv2D (img_op_implementations.py:164-330) covers stride 1 / no pad / group 1; the
+ * general attribute handling follows CudnnConvolution (cudnn_implementations.py:148-275,
+ * symmetric pads, groups incl. depthwise) and the output-size rule of
+ * shape_inference/symbolic_shape_infer.py:466-526. bias may be NULL.
+ * act: a DMLHIP_ACT_* code applied to the result (e.g. SWISH = the Sigmoid+Mul pair that
+ * follows the conv in the exported graph, fused). */
+typedef struct dmlhip_conv2d_desc {
+    int64_t n, c, h, w;       /* X */
+    int64_t m, kh, kw;        /* W is [m, c/group, kh, kw] */
+    int64_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, group;
+    int act;
+} dmlhip_conv2d_desc;
+int dmlhip_conv2d_out_shape(const dmlhip_conv2d_desc* d, int64_t* oh, int64_t* ow);
+int dmlhip_conv2d_f32(const dmlhip_conv2d_desc* d, const void* x, const void* w,
+                      const void* bias, void* y, void* stream);
+int dmlhip_conv2d_f16(const dmlhip_conv2d_desc* d, const void* x, const void* w,
+                      const void* bias, void* y, void* stream);
+/* cudnnConvolutionBackwardData / BackwardFilter (autodiff/implementations/onnx_ops.py:663-703)
+ * and the ATen depthwise backward (onnx_ops.py:1201-1231). dw is overwritten. The bias
+ * gradient is dmlhip_reduce over [n, m, oh*ow] done by the caller (two reduce calls). */
+int dmlhip_conv2d_backward_data_f32(const dmlhip_conv2d_desc* d, const void* dy, const void* w,
+                                    void* dx, void* stream);
+size_t dmlhip_conv2d_backward_weight_workspace_bytes(const dmlhip_conv2d_desc* d);
+int dmlhip_conv2d_backward_weight_f32(const dmlhip_conv2d_desc* d, const void* x,
+                                      const void* dy, void* dw, void* workspace,
+                                      size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DACEML_HIP_H */

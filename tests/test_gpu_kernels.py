@@ -1,0 +1,425 @@
+"""GPU parity: every dmlhip_* kernel against the NumPy oracle on the same seeded inputs.
+
+fp32 paths: rtol 1e-5 / atol 1e-6. fp16 paths (fp32 accumulation): rtol 2e-2 / atol 1e-2 against the
+oracle evaluated in fp64 on the fp16-rounded inputs. All calls go through the C ABI (ctypes).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ops as O
+from tests.util import assert_close, dev, host, rng
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float16, torch.float32]
+
+
+def _np(dtype):
+    return np.float16 if dtype == torch.float16 else np.float32
+
+
+def _inputs(seed, shape, dtype, scale=1.0):
+    """Seeded N(0, scale) data rounded to `dtype`, plus its fp64 image for the oracle."""
+    x = (rng(seed).standard_normal(shape) * scale).astype(_np(dtype))
+    return x, x.astype(np.float64)
+
+
+# ----------------------------------------------------------------------------- softmax
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape,axis", [((4, 16, 64, 512), -1), ((3, 7, 100), -1), ((5, 1000), 1), ((2, 3, 4, 8), 1),
+                                        ((6, 33), 0), ((2, 5000), -1), ((64, 1536), -1), ((7, 2048), -1), ((3, 1), -1)])
+def test_softmax(dtype, shape, axis):
+    from daceml_amd import kernels as K
+    x, x64 = _inputs(1, shape, dtype, 3.0)
+    y = K.softmax(dev(x), axis=axis)
+    assert y.dtype == dtype and tuple(y.shape) == shape
+    assert_close(host(y), O.softmax(x64, axis=axis), dtype, "softmax %s axis=%d" % (shape, axis))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_softmax_edge_cases(dtype):
+    from daceml_amd import kernels as K
+    # constant rows -> 1/n; large magnitudes must not overflow (max subtraction)
+    x = np.full((4, 512), 7.0, dtype=_np(dtype))
+    x[1] = -30000.0 if dtype == torch.float16 else -1e30
+    x[2, 5] = 60000.0 if dtype == torch.float16 else 1e30
+    y = host(K.softmax(dev(x)))
+    assert np.isfinite(y).all()
+    assert_close(y[0], np.full(512, 1 / 512), dtype, "constant row")
+    assert_close(y[1], np.full(512, 1 / 512), dtype, "very negative constant row")
+    assert y[2, 5] == pytest.approx(1.0) and y[2].sum() == pytest.approx(1.0, abs=1e-3)
+    # empty tensors are a no-op, not an error
+    e = torch.empty((0, 16), dtype=dtype, device="cuda")
+    assert K.softmax(e).shape == (0, 16)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(2, 4, 64, 512), (5, 100), (3, 4096), (3, 5000)])
+def test_softmax_backward(dtype, shape):
+    from daceml_amd import kernels as K
+    x, x64 = _inputs(2, shape, dtype)
+    y64 = O.softmax(x64, axis=-1)
+    y = y64.astype(_np(dtype))
+    dy, dy64 = _inputs(3, shape, dtype)
+    dx = K.softmax_backward(dev(y), dev(dy), axis=-1)
+    want = O.softmax_backward(y.astype(np.float64), dy64, axis=len(shape) - 1)
+    assert_close(host(dx), want, dtype, "softmax_backward %s" % (shape, ))
+
+
+# ----------------------------------------------------------------------------- layernorm
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(8, 64, 1024), (3, 5, 768), (7, 100), (4, 4096), (2, 3, 36)])
+@pytest.mark.parametrize("residual", [False, True])
+def test_layernorm(dtype, shape, residual):
+    from daceml_amd import kernels as K
+    h = shape[-1]
+    x, x64 = _inputs(4, shape, dtype)
+    g = (rng(5).uniform(0.5, 1.5, h)).astype(_np(dtype))
+    b = (rng(6).standard_normal(h) * 0.1).astype(_np(dtype))
+    r = None
+    s64 = x64
+    if residual:
+        r, r64 = _inputs(7, shape, dtype)
+        s64 = (x64 + r64).astype(_np(dtype)).astype(np.float64)  # the Add node rounds to the tensor dtype
+    y, s, mean, rstd = K.layernorm(dev(x), dev(g), dev(b), 1e-5, residual=None if r is None else dev(r),
+                                   want_sum=True, want_stats=True)
+    want, mu, var = O.layernorm_chain(s64, g.astype(np.float64), b.astype(np.float64), 1e-5)
+    assert_close(host(y), want, dtype, "layernorm %s" % (shape, ))
+    assert_close(host(s), s64, dtype, "layernorm sum_out")
+    assert_close(host(mean), mu.reshape(-1), torch.float32, "mean", rtol=1e-4, atol=1e-5)
+    assert_close(host(rstd), 1 / np.sqrt(var.reshape(-1) + 1e-5), torch.float32, "rstd", rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_layernorm_invariants(dtype):
+    from daceml_amd import kernels as K
+    h = 1024
+    x, _ = _inputs(8, (16, h), dtype)
+    one = np.ones(h, _np(dtype))
+    zero = np.zeros(h, _np(dtype))
+    y = host(K.layernorm(dev(x), dev(one), dev(zero))[0]).astype(np.float64)
+    assert np.abs(y.mean(-1)).max() < 2e-3 and np.abs(y.var(-1) - 1).max() < 5e-3
+    # a constant row normalises to beta
+    c = np.full((2, h), 3.0, _np(dtype))
+    b = (rng(9).standard_normal(h) * 0.1).astype(_np(dtype))
+    y = host(K.layernorm(dev(c), dev(one), dev(b))[0])
+    assert_close(y, np.broadcast_to(b.astype(np.float64), (2, h)), dtype, "constant row -> beta")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4, 128, 1024), (37, 768), (5, 100), (3, 4096)])
+def test_layernorm_backward(dtype, shape):
+    from daceml_amd import kernels as K
+    h = shape[-1]
+    x, x64 = _inputs(10, shape, dtype)
+    dy, dy64 = _inputs(11, shape, dtype)
+    g = (rng(12).uniform(0.5, 1.5, h)).astype(_np(dtype))
+    _, _, mean, rstd = K.layernorm(dev(x), dev(g), dev(g), 1e-5, want_stats=True)
+    dx, dg, db = K.layernorm_backward(dev(dy), dev(x), mean, rstd, dev(g))
+    wdx, wdg, wdb = O.layernorm_backward(dy64, x64, g.astype(np.float64), 1e-5)
+    assert dg.dtype == torch.float32 and db.dtype == torch.float32
+    assert_close(host(dx), wdx, dtype, "ln dx", rtol=None if dtype == torch.float16 else 1e-4, atol=None if dtype == torch.float16 else 1e-5)
+    rows = x.size // h
+    # column sums over `rows` terms: fp32 accumulation error grows with sqrt(rows)
+    assert_close(host(dg), wdg, torch.float32, "ln dgamma", rtol=1e-4, atol=1e-5 * np.sqrt(rows))
+    assert_close(host(db), wdb, torch.float32, "ln dbeta", rtol=1e-4, atol=1e-5 * np.sqrt(rows))
+
+
+# ----------------------------------------------------------------------------- elementwise
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+@pytest.mark.parametrize("sa,sb", [((4, 8, 64), (4, 8, 64)), ((4, 8, 64), (64, )), ((64, ), (4, 8, 64)),
+                                   ((4, 8, 64), (1, )), ((1, ), (5, 7)), ((4, 1, 6), (1, 5, 6)), ((3, 5), (3, 1)),
+                                   ((2, 3, 4, 5, 6), (3, 1, 5, 1)), ((1000, 33), (33, )), ((7, ), (7, ))])
+def test_binary(dtype, op, sa, sb):
+    from daceml_amd import _lib as L, kernels as K
+    a, a64 = _inputs(13, sa, dtype)
+    b, b64 = _inputs(14, sb, dtype)
+    if op == "div":
+        b = (np.abs(b) + 0.5).astype(_np(dtype))
+        b64 = b.astype(np.float64)
+    code = {"add": L.ADD, "sub": L.SUB, "mul": L.MUL, "div": L.DIV}[op]
+    want = getattr(O, op)(a64, b64)
+    got = K.binary(code, dev(a), dev(b))
+    assert tuple(got.shape) == want.shape
+    assert_close(host(got), want, dtype, "%s %s %s" % (op, sa, sb))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_pow(dtype):
+    from daceml_amd import _lib as L, kernels as K
+    a, a64 = _inputs(15, (33, 65), dtype)
+    two = np.array(2.0, _np(dtype))
+    assert_close(host(K.binary(L.POW, dev(a), dev(two))), O.pow_(a64, 2.0), dtype, "pow 2")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["erf", "sqrt", "exp", "log", "tanh", "relu", "sigmoid", "reciprocal", "gelu", "swish"])
+def test_unary(dtype, name):
+    from daceml_amd import _lib as L, kernels as K
+    x, x64 = _inputs(16, (37, 129), dtype)
+    if name in ("sqrt", "log", "reciprocal"):
+        x = (np.abs(x) + 0.25).astype(_np(dtype))
+        x64 = x.astype(np.float64)
+    fn = {"gelu": O.gelu_chain, "swish": O.swish}.get(name) or getattr(O, name)
+    code = getattr(L, name.upper())
+    assert_close(host(K.unary(code, dev(x))), fn(x64), dtype, name)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["gelu", "swish", "sigmoid", "relu", "tanh"])
+def test_unary_backward(dtype, name):
+    from daceml_amd import _lib as L, kernels as K
+    x, x64 = _inputs(17, (41, 64), dtype)
+    dy, dy64 = _inputs(18, (41, 64), dtype)
+    t = torch.tensor(x64, requires_grad=True)
+    f = {"gelu": lambda v: torch.nn.functional.gelu(v), "swish": lambda v: v * torch.sigmoid(v),
+         "sigmoid": torch.sigmoid, "relu": torch.relu, "tanh": torch.tanh}[name]
+    f(t).backward(torch.tensor(dy64))
+    got = K.unary_backward(getattr(L, name.upper()), dev(x), dev(dy))
+    assert_close(host(got), t.grad.numpy(), dtype, name + " backward")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_in", [1, 2, 3, 8, 11])
+def test_sum(dtype, n_in):
+    from daceml_amd import kernels as K
+    xs = [_inputs(20 + i, (5, 7, 33), dtype) for i in range(n_in)]
+    got = K.sum_variadic([dev(x) for x, _ in xs])
+    assert_close(host(got), O.sum_variadic(*[x64 for _, x64 in xs]), dtype, "sum of %d" % n_in)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4, 64, 4096), (7, 100), (3, 5)])
+def test_bias_gelu(dtype, shape):
+    from daceml_amd import kernels as K
+    x, x64 = _inputs(30, shape, dtype)
+    b, b64 = _inputs(31, shape[-1:], dtype, 0.1)
+    y, pre = K.bias_gelu(dev(x), dev(b), want_pre=True)
+    u64 = (x64 + b64).astype(_np(dtype)).astype(np.float64)
+    assert_close(host(pre), u64, dtype, "bias add")
+    assert_close(host(y), O.gelu_chain(u64), dtype, "bias+gelu")
+
+
+def test_cast():
+    from daceml_amd import kernels as K
+    x = rng(32).standard_normal((5, 33)).astype(np.float32)
+    h = K.cast(dev(x), torch.float16)
+    assert h.dtype == torch.float16
+    np.testing.assert_array_equal(h.cpu().numpy(), x.astype(np.float16))
+    np.testing.assert_array_equal(K.cast(h, torch.float32).cpu().numpy(), x.astype(np.float16).astype(np.float32))
+
+
+# ----------------------------------------------------------------------------- reductions / transpose
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["sum", "mean", "max", "min"])
+@pytest.mark.parametrize("shape,axes", [((8, 64, 100), [-1]), ((6, 5000), [1]), ((4096, 256), [0]), ((3, 40, 7), [1]),
+                                        ((4, 6, 8, 10), [2, 3]), ((2, 1024, 64), [0, 1]), ((5, 7), None), ((3, 1, 9), [1])])
+@pytest.mark.parametrize("keepdims", [1, 0])
+def test_reduce(dtype, name, shape, axes, keepdims):
+    from daceml_amd import _lib as L, kernels as K
+    x, x64 = _inputs(40, shape, dtype)
+    code = {"sum": L.RSUM, "mean": L.RMEAN, "max": L.RMAX, "min": L.RMIN}[name]
+    want = getattr(O, "reduce_" + name)(x64, axes, keepdims)
+    got = K.reduce(code, dev(x), axes, bool(keepdims), out_dtype=torch.float32)
+    assert tuple(got.shape) == want.shape
+    n = x.size // max(want.size, 1)
+    assert_close(host(got), want, torch.float32, "reduce_%s %s %s" % (name, shape, axes), rtol=1e-5,
+                 atol=1e-6 * max(1.0, np.sqrt(n)) if name == "sum" else 1e-6)
+    got_t = K.reduce(code, dev(x), axes, bool(keepdims))
+    assert got_t.dtype == dtype
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape,perm", [((8, 64, 16, 32), (0, 2, 1, 3)), ((37, 65), None), ((3, 5, 7), (2, 0, 1)),
+                                        ((2, 3, 4, 5, 6), (4, 3, 2, 1, 0)), ((4, 1, 9), (1, 2, 0)), ((6, ), None),
+                                        ((2, 16, 64, 40), (0, 1, 3, 2)), ((5, 6, 7, 8), (0, 1, 2, 3)),
+                                        ((2, 3, 4, 5, 6, 7), (5, 0, 3, 1, 4, 2))])
+def test_transpose(dtype, shape, perm):
+    from daceml_amd import kernels as K
+    x, _ = _inputs(50, shape, dtype)
+    got = K.transpose(dev(x), perm)
+    want = O.transpose(x, perm)
+    assert tuple(got.shape) == want.shape
+    np.testing.assert_array_equal(got.cpu().numpy(), want)  # a copy: bit-exact
+
+
+# ----------------------------------------------------------------------------- fp16 contractions
+def _set_cfg(cfg):
+    from daceml_amd import _lib as L
+    L.load().dmlhip_debug_force_gemm_config(cfg)
+
+
+GEMM_CASES = [
+    # equation, shapes (before any view), scale
+    ("aik,kj->aij", (2, 96, 200), (200, 136)),       # ragged everywhere
+    ("aik,jk->aij", (2, 256, 128), (384, 128)),      # weight stored [out, in]
+    ("baik,bakj->baij", (2, 3, 130, 64), (2, 3, 64, 72)),
+    ("aij,kj->aik", (2, 128, 256), (192, 256)),      # backward w.r.t. activations
+    ("aij,aik->kj", (2, 136, 256), (2, 136, 200)),   # backward w.r.t. weights: both operands row-contiguous
+    ("bsnd,btnd->bnst", (2, 70, 4, 64), (2, 90, 4, 64)),
+    ("bnst,btnd->bsnd", (2, 4, 72, 96), (2, 96, 4, 64)),
+    ("ik,kj->ij", (300, 1000), (1000, 260)),
+    ("ik,kj->ji", (40, 24), (24, 56)),
+    ("ik,k->i", (33, 40), (40, )),
+    ("ik,kj->ij", (5, 7), (7, 3)),                   # unaligned: generic loader
+]
+
+
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2])
+@pytest.mark.parametrize("eq,sa,sb", GEMM_CASES)
+def test_einsum_f16(cfg, eq, sa, sb):
+    from daceml_amd import kernels as K
+    a, a64 = _inputs(60, sa, torch.float16)
+    b, b64 = _inputs(61, sb, torch.float16)
+    _set_cfg(cfg)
+    try:
+        got = K.einsum(eq, dev(a), dev(b))
+    finally:
+        _set_cfg(-1)
+    want = O.einsum(eq, a64, b64)
+    assert tuple(got.shape) == want.shape
+    assert_close(host(got), want, torch.float16, "einsum %s cfg=%d" % (eq, cfg))
+    # fp32 output of the same product: only accumulation-order error remains
+    got32 = K.einsum(eq, dev(a), dev(b), out_dtype=torch.float32)
+    k = a.size * b.size // max(want.size, 1)
+    assert_close(host(got32), want, torch.float32, "einsum %s fp32 out" % eq, rtol=1e-4, atol=2e-4)
+    del k
+
+
+def test_einsum_f16_views_fold_transposes():
+    """A permuted view feeds the GEMM without a copy (Transpose folded into operand strides)."""
+    from daceml_amd import kernels as K
+    q, q64 = _inputs(62, (2, 80, 4, 64), torch.float16)  # [b, s, n, d]
+    k, k64 = _inputs(63, (2, 80, 4, 64), torch.float16)
+    qh = dev(q).permute(0, 2, 1, 3)   # [b, n, s, d] view
+    kt = dev(k).permute(0, 2, 3, 1)   # [b, n, d, t] view
+    got = K.einsum("baik,bakj->baij", qh, kt, alpha=0.125)
+    want = 0.125 * np.einsum("bsnd,btnd->bnst", q64, k64)
+    assert_close(host(got), want, torch.float16, "scores from views")
+
+
+def test_gemm_f16_epilogue():
+    from daceml_amd import _lib as L, kernels as K
+    a, a64 = _inputs(64, (2, 100, 128), torch.float16)
+    w, w64 = _inputs(65, (264, 128), torch.float16, 0.1)
+    bias, bias64 = _inputs(66, (264, ), torch.float16, 0.5)
+    res, res64 = _inputs(67, (2, 100, 264), torch.float16)
+    pre = torch.empty((2, 100, 264), dtype=torch.float16, device="cuda")
+    got = K.einsum("aik,jk->aij", dev(a), dev(w), bias=dev(bias), act=L.ACT_GELU, residual=dev(res), pre_out=pre)
+    u = (np.einsum("aik,jk->aij", a64, w64) + bias64)
+    assert_close(host(pre), u, torch.float16, "pre-activation")
+    u16 = host(pre).astype(np.float64)
+    assert_close(host(got), O.gelu_chain(u16) + res64, torch.float16, "bias+gelu+residual epilogue")
+    # beta accumulation into an fp32 output (master-gradient accumulation)
+    acc0 = rng(68).standard_normal((264, 128)).astype(np.float32)
+    acc = dev(acc0)
+    dy, dy64 = _inputs(69, (2, 100, 264), torch.float16)
+    K.einsum("aij,aik->jk", dev(dy), dev(a), out=acc, out_dtype=torch.float32, beta=1.0)
+    assert_close(host(acc), acc0 + np.einsum("aij,aik->jk", dy64, a64), torch.float32, "beta accumulate", rtol=1e-4,
+                 atol=1e-3)
+
+
+def test_gemm_f16_config_shapes():
+    """BERT-large attention-score contraction at its real per-head shape, two batch entries."""
+    from daceml_amd import kernels as K
+    q, q64 = _inputs(70, (1, 2, 512, 64), torch.float16)
+    k, k64 = _inputs(71, (1, 2, 64, 512), torch.float16)
+    got = K.einsum("baik,bakj->baij", dev(q), dev(k))
+    assert_close(host(got), np.einsum("baik,bakj->baij", q64, k64), torch.float16, "scores 512x512x64")
+    x, x64 = _inputs(72, (1, 512, 1024), torch.float16)
+    w, w64 = _inputs(73, (1024, 4096), torch.float16, 0.02)
+    got = K.einsum("aik,kj->aij", dev(x), dev(w))
+    assert_close(host(got), np.einsum("aik,kj->aij", x64, w64), torch.float16, "ffn1 512x4096x1024")
+
+
+# ----------------------------------------------------------------------------- fp32 contractions
+@pytest.mark.parametrize("eq,sa,sb", GEMM_CASES)
+def test_einsum_f32(eq, sa, sb):
+    from daceml_amd import kernels as K
+    # inputs scaled so that products stay O(1/k): the 1e-5 / 1e-6 bound is about rounding, not range
+    a = (rng(80).standard_normal(sa) * 0.25).astype(np.float32)
+    b = (rng(81).standard_normal(sb) * 0.25).astype(np.float32)
+    got = K.einsum(eq, dev(a), dev(b))
+    want = O.einsum(eq, a.astype(np.float64), b.astype(np.float64))
+    kdim = a.size * b.size // max(want.size, 1)
+    del kdim
+    assert_close(host(got), want, torch.float32, "einsum f32 %s" % eq, rtol=1e-5, atol=2e-6)
+
+
+def test_gemm_f32_epilogue():
+    from daceml_amd import _lib as L, kernels as K
+    a = (rng(82).standard_normal((70, 96)) * 0.3).astype(np.float32)
+    w = (rng(83).standard_normal((96, 200)) * 0.3).astype(np.float32)
+    bias = rng(84).standard_normal(200).astype(np.float32)
+    res = rng(85).standard_normal((70, 200)).astype(np.float32)
+    got = K.einsum("ik,kj->ij", dev(a), dev(w), bias=dev(bias), act=L.ACT_GELU, residual=dev(res), alpha=0.5)
+    u = 0.5 * (a.astype(np.float64) @ w.astype(np.float64)) + bias
+    assert_close(host(got), O.gelu_chain(u) + res, torch.float32, "f32 epilogue", rtol=1e-5, atol=2e-6)
+
+
+# ----------------------------------------------------------------------------- convolution
+CONV_CASES = [
+    # x shape, w shape, strides, pads, dilations, group, bias
+    ((5, 3, 10, 10), (16, 3, 3, 3), (2, 2), (0, 0), (1, 1), 1, False),      # README / plot_conv example (config 1)
+    ((8, 3, 32, 32), (6, 3, 5, 5), (1, 1), (0, 0), (1, 1), 1, True),        # test_conv_expansion shapes
+    ((2, 8, 14, 14), (12, 8, 1, 1), (1, 1), (0, 0), (1, 1), 1, True),       # 1x1 -> GEMM
+    ((3, 32, 28, 28), (192, 32, 1, 1), (1, 1), (0, 0), (1, 1), 1, True),    # MBConv expand, small spatial
+    ((2, 12, 30, 30), (12, 1, 3, 3), (2, 2), (1, 1), (1, 1), 12, True),     # depthwise s2 p1
+    ((2, 6, 17, 19), (6, 1, 5, 5), (1, 1), (2, 2), (1, 1), 6, False),       # depthwise 5x5 odd sizes
+    ((2, 8, 9, 9), (4, 4, 3, 3), (1, 1), (1, 1), (1, 1), 2, True),          # grouped
+    ((1, 2, 12, 12), (3, 2, 3, 3), (1, 1), (2, 2), (2, 2), 1, False),       # dilated
+    ((2, 4, 8, 8), (6, 4, 1, 1), (2, 2), (0, 0), (1, 1), 1, True),          # 1x1 strided -> direct
+]
+
+
+@pytest.mark.parametrize("xs,ws,st,pd,dl,grp,has_bias", CONV_CASES)
+def test_conv2d_f32(xs, ws, st, pd, dl, grp, has_bias):
+    from daceml_amd import kernels as K
+    x = rng(90).uniform(0, 1, xs).astype(np.float32)
+    w = (rng(91).uniform(0, 1, ws) / np.sqrt(np.prod(ws[1:]))).astype(np.float32)
+    b = rng(92).standard_normal(ws[0]).astype(np.float32) if has_bias else None
+    got = K.conv2d(dev(x), dev(w), None if b is None else dev(b), st, pd, dl, grp)
+    want = O.conv2d(x.astype(np.float64), w.astype(np.float64), None if b is None else b.astype(np.float64), st,
+                    (pd[0], pd[1], pd[0], pd[1]), dl, grp)
+    assert tuple(got.shape) == want.shape
+    assert_close(host(got), want, torch.float32, "conv %s %s" % (xs, ws))
+
+
+def test_conv2d_f32_swish_epilogue():
+    from daceml_amd import _lib as L, kernels as K
+    for xs, ws, st, pd, grp in [((2, 16, 12, 12), (24, 16, 1, 1), (1, 1), (0, 0), 1),
+                                ((2, 24, 12, 12), (24, 1, 3, 3), (2, 2), (1, 1), 24)]:
+        x = rng(93).standard_normal(xs).astype(np.float32)
+        w = (rng(94).standard_normal(ws) * np.sqrt(2.0 / np.prod(ws[1:]))).astype(np.float32)
+        b = (rng(95).standard_normal(ws[0]) * 0.1).astype(np.float32)
+        got = K.conv2d(dev(x), dev(w), dev(b), st, pd, (1, 1), grp, act=L.ACT_SWISH)
+        want = O.swish(O.conv2d(x.astype(np.float64), w.astype(np.float64), b.astype(np.float64), st,
+                                (pd[0], pd[1], pd[0], pd[1]), (1, 1), grp))
+        assert_close(host(got), want, torch.float32, "conv+swish %s" % (ws, ))
+
+
+@pytest.mark.parametrize("xs,ws,st,pd,dl,grp,has_bias", CONV_CASES)
+def test_conv2d_backward_f32(xs, ws, st, pd, dl, grp, has_bias):
+    from daceml_amd import kernels as K
+    x = rng(96).uniform(-1, 1, xs).astype(np.float32)
+    w = (rng(97).uniform(-1, 1, ws) / np.sqrt(np.prod(ws[1:]))).astype(np.float32)
+    y = O.conv2d(x, w, None, st, (pd[0], pd[1], pd[0], pd[1]), dl, grp)
+    dy = (rng(98).standard_normal(y.shape) / np.sqrt(y[0, 0].size)).astype(np.float32)
+    dx, dw = K.conv2d_backward(dev(x), dev(w), dev(dy), st, pd, dl, grp)
+    wdx, wdw, _ = O.conv2d_backward(x.astype(np.float64), w.astype(np.float64), dy.astype(np.float64), st,
+                                    (pd[0], pd[1], pd[0], pd[1]), dl, grp)
+    assert_close(host(dx), wdx, torch.float32, "conv dx %s" % (ws, ), rtol=1e-5, atol=2e-6)
+    assert_close(host(dw), wdw, torch.float32, "conv dw %s" % (ws, ), rtol=1e-5, atol=2e-6)
+
+
+def test_conv2d_f16_1x1_and_depthwise():
+    from daceml_amd import kernels as K
+    for xs, ws, st, pd, grp in [((2, 32, 16, 16), (48, 32, 1, 1), (1, 1), (0, 0), 1),
+                                ((2, 16, 15, 15), (16, 1, 3, 3), (2, 2), (1, 1), 16)]:
+        x, x64 = _inputs(99, xs, torch.float16)
+        w, w64 = _inputs(100, ws, torch.float16, 0.2)
+        got = K.conv2d(dev(x), dev(w), None, st, pd, (1, 1), grp)
+        want = O.conv2d(x64, w64, None, st, (pd[0], pd[1], pd[0], pd[1]), (1, 1), grp)
+        assert_close(host(got), want, torch.float16, "conv f16 %s" % (ws, ))
