@@ -1,0 +1,168 @@
+"""Headline benchmark: one BERT-large encoder layer (fp16, B=8, S=512, hidden 1024, 16 heads, FFN 4096),
+forward + autodiff backward through the "hip" library-node implementations, on one MI355X.
+
+Prints ONE JSON line (see the keys below). `value` is ms per forward+backward step with all inputs
+resident in HBM. `roofline` describes the dominant kernel (the fp16 MFMA GEMM): algorithmic FLOPs of
+all contraction launches of a step divided by their summed HIP-event durations. `hbm_nodes` does the
+same against the HBM roofline for the memory-bound nodes. `cpu_baseline` is the NumPy restatement of the
+reference's pure expansions (oracle/) timed on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+METRIC = "BERT-large encoder layer fp16 fwd+bwd ms/iter at 1 GPU; % MFMA & HBM roofline"
+B, S, H, HEADS, FFN = 8, 512, 1024, 16, 4096
+
+
+def build_program(device):
+    import torch
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.runtime import CompiledSDFG
+    from daceml_amd.transformation import fusion
+    from oracle import bert_layer as OB  # parameter names / init only
+
+    sdfg = graphs.bert_encoder_layer(B, S, H, HEADS, FFN, torch.float16, eps=1e-12)
+    fusion.auto_optimize(sdfg, training=True)
+    add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + OB.PARAM_NAMES,
+                      grad_dtypes={n: torch.float32 for n in OB.PARAM_NAMES})
+    return CompiledSDFG(sdfg, device=device), OB
+
+
+def synthetic_inputs(OB, device):
+    """Seeded synthetic data of the config's shape: x, dy ~ N(0,1); weights N(0, 0.02), biases 0, LN 1/0."""
+    import numpy as np
+    import torch
+    p = OB.init_params(H, FFN, 1234 + 4, np.float32)
+    rng = np.random.default_rng(1234 + 5)
+    x = rng.standard_normal((B, S, H)).astype(np.float16)
+    dy = rng.standard_normal((B, S, H)).astype(np.float16)
+    args = {"x": torch.from_numpy(x).to(device), "gradient_y": torch.from_numpy(dy).to(device),
+            "y": torch.empty((B, S, H), dtype=torch.float16, device=device),
+            "gradient_x": torch.empty((B, S, H), dtype=torch.float16, device=device)}
+    for n in OB.PARAM_NAMES:
+        args[n] = torch.from_numpy(p[n].astype(np.float16)).to(device)
+        args["gradient_" + n] = torch.empty(p[n].shape, dtype=torch.float32, device=device)
+    return args, x, dy, p
+
+
+def kernel_breakdown(prog, reps=10):
+    """HIP-event duration of every launch (events on the stream the kernels run on), averaged."""
+    acc = None
+    for _ in range(reps):
+        rows = prog.launch_timed()
+        if acc is None:
+            acc = [[l, 0.0] for l, _ in rows]
+        for i, (_, ms) in enumerate(rows):
+            acc[i][1] += ms
+    return [(l, ms / reps) for l, ms in acc]
+
+
+def cpu_baseline(OB, x, dy, p, budget_s=25.0):
+    """The oracle's forward+backward (fp32 NumPy, BLAS contractions) on the full workload, repeated within
+    a time budget."""
+    import numpy as np
+    x32 = x.astype(np.float32)
+    dy32 = dy.astype(np.float32)
+    p32 = {k: v.astype(np.float32) for k, v in p.items()}
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while True:
+        t0 = time.perf_counter()
+        _, saved = OB.forward(x32, p32, HEADS, eps=1e-12, keep=True)
+        OB.backward(x32, p32, HEADS, dy32, saved, eps=1e-12)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() + times[-1] > t_end or len(times) >= 5:
+            break
+    try:
+        from threadpoolctl import threadpool_info
+        cores = max([i.get("num_threads", 1) for i in threadpool_info()] or [1])
+    except Exception:
+        cores = os.cpu_count() or 1
+    return {"value": round(min(times) * 1e3, 2), "unit": "ms/iter", "cores": int(cores), "kind": "port",
+            "sample": "full workload (B=8, S=512), %d fwd+bwd repetitions of the NumPy restatement of the pure "
+                      "expansions in fp32, best of them" % len(times)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--verbose", action="store_true", help="per-launch table on stderr")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures the single-GPU path only: this build uses one GPU (no collectives, no sharding); "
+                 "run with --gpus 1")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+
+    prog, OB = build_program(device)
+    args, x, dy, p = synthetic_inputs(OB, device)
+    prog(**args)  # binds pointers, first run
+    for _ in range(a.warmup):
+        prog.launch()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        prog.launch()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / a.steps * 1e3
+
+    rows = kernel_breakdown(prog)
+    if a.verbose:
+        for l, t in rows:
+            rate = ("%7.1f TFLOP/s" % (l.flops / (t * 1e-3) / 1e12)) if l.flops else \
+                   ("%7.1f GB/s" % (l.bytes_moved / (t * 1e-3) / 1e9)) if l.bytes_moved else ""
+            sys.stderr.write("%-9s %-28s %-44s %8.1f us %s\n" % (l.state[-9:], l.kind, l.label[:44], t * 1e3, rate))
+    gemm_ms = sum(t for l, t in rows if l.kind == "gemm")
+    gemm_flops = sum(l.flops for l, _ in rows if l.kind == "gemm")
+    n_gemm = sum(1 for l, _ in rows if l.kind == "gemm")
+    tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
+    hbm = {}
+    for l, t in rows:
+        if l.kind == "gemm" or l.bytes_moved == 0:
+            continue
+        e = hbm.setdefault(l.kind, {"ms": 0.0, "bytes": 0, "launches": 0})
+        e["ms"] += t
+        e["bytes"] += l.bytes_moved
+        e["launches"] += 1
+    for e in hbm.values():
+        e["GB/s"] = round(e["bytes"] / (e["ms"] * 1e-3) / 1e9, 1)
+        e["frac"] = round(e["GB/s"] / PEAK_HBM_GBS, 4)
+        e["ms"] = round(e["ms"], 4)
+    out = {
+        "metric": METRIC, "value": round(ms, 4), "unit": "ms/iter", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (fp32 accumulate, fp32 master gradients)", "data": "synthetic",
+        "config": {"workload": "BERT-large encoder layer forward + autodiff backward, B=8 S=512 hidden=1024 heads=16 "
+                               "ffn=4096, fp16 (BASELINE.json configs[4])",
+                   "launches_per_step": len(prog.launches)},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_FP16_TFLOPS, 4), "traffic": None,
+                     "kernel": "gemm_f16_kernel (all %d contraction launches of a step)" % n_gemm,
+                     "flops_per_step": gemm_flops, "ms_per_step": round(gemm_ms, 4)},
+        "hbm_nodes": hbm,
+        "sum_of_kernel_ms": round(sum(t for _, t in rows), 4),
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(OB, x, dy, p)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

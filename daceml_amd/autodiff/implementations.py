@@ -1,0 +1,309 @@
+"""Backward implementations that keep the backward pass on hand-written kernels.
+
+Without these, the reference's generator would expand each forward node with a "pure" implementation
+and differentiate the resulting tasklets symbolically (backward_pass_generator.py:425-494), which
+bypasses any native forward implementation. Counterparts: ``DefaultEinsumBackward`` and
+``DefaultSoftmaxBackward`` (daceml/autodiff/implementations/onnx_ops.py:54-138,237-275), the cuDNN /
+ATen Conv backward (:494-733,1140-1265).
+"""
+from typing import List, Optional, Tuple
+
+import torch
+
+from .. import contraction as C
+from .. import onnx as donnx
+from ..sdfg import Node, contiguous_strides
+from .base_abc import (AutoDiffException, BackwardContext, BackwardGroup, BackwardImplementation, BackwardResult,
+                       autoregister_params)
+
+NAME = "hip"
+
+
+# ----------------------------------------------------------------------------- helpers
+def _in_arr(ctx: BackwardContext, node, conn) -> Optional[str]:
+    for e in ctx.forward_state.in_edges_by_connector(node, conn):
+        return e.data.data
+    return None
+
+
+def _out_arr(ctx: BackwardContext, node, conn) -> Optional[str]:
+    for e in ctx.forward_state.out_edges_by_connector(node, conn):
+        return e.data.data
+    return None
+
+
+def connect_input_from_forward(forward_node, backward_node, ctx: BackwardContext, conn: str, as_conn: str = None):
+    """Feed the array on input `conn` of the forward node to the reverse node (autodiff/utils.py)."""
+    arr = _in_arr(ctx, forward_node, conn)
+    _read(ctx, arr, backward_node, as_conn or conn)
+
+
+def connect_output_from_forward(forward_node, backward_node, ctx: BackwardContext, conn: str, as_conn: str = None):
+    """Feed a forward *output* to the reverse node — torch's save_for_backward (autodiff/utils.py:224-261)."""
+    arr = _out_arr(ctx, forward_node, conn)
+    _read(ctx, arr, backward_node, as_conn or conn)
+
+
+def _read(ctx, arr, node, conn):
+    st = ctx.backward_state
+    if conn not in node.in_connectors:
+        node.add_in_connector(conn)
+    st.add_edge(st.add_read(arr), None, node, conn, ctx.backward_sdfg.make_array_memlet(arr))
+
+
+def _write(ctx, node, conn, arr):
+    st = ctx.backward_state
+    if conn not in node.out_connectors:
+        node.add_out_connector(conn)
+    st.add_edge(node, conn, st.add_write(arr), None, ctx.backward_sdfg.make_array_memlet(arr))
+
+
+def _ensure_forward_output(ctx: BackwardContext, node, conn: str, shape, dtype) -> str:
+    """Make the forward node produce optional output `conn` (statistics, pre-activation) if it does not."""
+    arr = _out_arr(ctx, node, conn)
+    if arr is not None:
+        return arr
+    name, _ = ctx.forward_sdfg.add_transient("%s_%s" % (node.label, conn), shape, dtype)
+    node.add_out_connector(conn)
+    st = ctx.forward_state
+    st.add_edge(node, conn, st.add_write(name), None, ctx.forward_sdfg.make_array_memlet(name))
+    return name
+
+
+def _new(ctx, op: str, label: str, **attrs):
+    node = donnx.get_onnx_node(op)(label, **attrs)
+    ctx.backward_state.add_node(node)
+    return node
+
+
+# ----------------------------------------------------------------------------- contractions
+def _einsum_backward(forward_node, ctx: BackwardContext, given, required, eq: str, alpha: float, act: str,
+                     bias_conn: Optional[str], residual_conn: Optional[str]):
+    sdfg = ctx.forward_sdfg
+    out = _out_arr(ctx, forward_node, "Output")
+    od = sdfg.arrays[out]
+    group = BackwardGroup(forward_node.label + "_backward")
+    req, passthrough = {}, {}
+    grad_src: Optional[Tuple[Node, str]] = None   # producer of d(pre-activation) when an activation is undone
+    dpre_arr = None
+    if act != "none":
+        if act != "gelu":
+            raise AutoDiffException("no backward for activation %r" % act)
+        pre = _ensure_forward_output(ctx, forward_node, "PreActivation", od.shape, od.dtype)
+        gg = _new(ctx, "GeluGrad", forward_node.label + "_act_grad")
+        _read(ctx, pre, gg, "X")
+        group.map_input("Output_grad", gg, "dY")
+        dpre_arr, _ = sdfg.add_transient("gradient_" + pre, od.shape, od.dtype)
+        _write(ctx, gg, "dX", dpre_arr)
+
+    def feed_dout(node, conn):
+        if dpre_arr is not None:
+            _read(ctx, dpre_arr, node, conn)
+        else:
+            node.add_in_connector(conn)
+            group.map_input("Output_grad", node, conn)
+
+    for conn in required:
+        if conn in ("Inputs__0", "Inputs__1"):
+            idx = int(conn[-1])
+            others, rev_eq = C.reverse_equation(eq, idx)
+            es = _new(ctx, "FusedEinsum", "%s_grad_%d" % (forward_node.label, idx), equation=rev_eq, alpha=alpha)
+            feed_dout(es, "Inputs__0")
+            connect_input_from_forward(forward_node, es, ctx, "Inputs__%d" % others[0], "Inputs__1")
+            group.map_output(conn + "_grad", es, "Output")
+            req[conn] = conn + "_grad"
+        elif conn == bias_conn:
+            nd = len(od.shape)
+            rs = _new(ctx, "ReduceSum", forward_node.label + "_bias_grad", axes=list(range(nd - 1)), keepdims=0)
+            feed_dout(rs, "data")
+            group.map_output(conn + "_grad", rs, "reduced")
+            req[conn] = conn + "_grad"
+        elif conn == residual_conn:
+            if act != "none":
+                raise AutoDiffException("residual after an activation is not produced by the fusion pass")
+            passthrough[conn] = "Output"
+        else:
+            raise AutoDiffException("unexpected input connector %r" % conn)
+    return group, BackwardResult(required_grad_names=req, given_grad_names={"Output": "Output_grad"},
+                                 passthrough=passthrough)
+
+
+@autoregister_params(op="Einsum", name=NAME)
+class HipEinsumBackward(BackwardImplementation):
+    """DefaultEinsumBackward (onnx_ops.py:54-138): one new contraction per required input, with the
+    equation of reverse_einsum_wrt_input (:25-51); they run on the same MFMA GEMM."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, _ = C.parse(node.equation)
+            return len(ins) == 2
+        except C.NotApplicable:
+            return False
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        return _einsum_backward(forward_node, context, given_gradients, required_gradients,
+                                forward_node.equation.replace(" ", ""), 1.0, "none", None, None)
+
+
+@autoregister_params(op="FusedEinsum", name=NAME)
+class HipFusedEinsumBackward(BackwardImplementation):
+    """Backward of a contraction with folded scale / bias / GELU / residual: GeluGrad on the stored
+    pre-activation, a column ReduceSum for the bias, two contractions for the operands; the residual's
+    gradient is the incoming gradient itself."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        return node.activation in ("none", "gelu") and not node.accumulate
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        st = context.forward_state
+        conns = [e.dst_conn for e in st.in_edges(forward_node)]
+        return _einsum_backward(forward_node, context, given_gradients, required_gradients,
+                                forward_node.equation.replace(" ", ""), forward_node.alpha, forward_node.activation,
+                                "Bias" if "Bias" in conns else None, "Residual" if "Residual" in conns else None)
+
+
+# ----------------------------------------------------------------------------- softmax / layernorm
+@autoregister_params(op="Softmax", name=NAME)
+class HipSoftmaxBackward(BackwardImplementation):
+    """DefaultSoftmaxBackward (onnx_ops.py:237-275) as one SoftmaxGrad node; needs the forward output."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        for e in state.in_edges_by_connector(node, "input"):
+            nd = len(sdfg.arrays[e.data.data].shape)
+            return node.axis % nd == nd - 1
+        return False
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        sg = _new(context, "SoftmaxGrad", forward_node.label + "_backward", axis=-1)
+        connect_output_from_forward(forward_node, sg, context, "output", "Y")
+        return sg, BackwardResult(required_grad_names={"input": "dX"}, given_grad_names={"output": "dY"})
+
+
+def _ln_backward(forward_node, ctx, x_arr, scale_conn, bias_conn, x_conns, mean_conn, rstd_conn, required):
+    sdfg = ctx.forward_sdfg
+    xd = sdfg.arrays[x_arr]
+    rows = xd.total_size // xd.shape[-1]
+    mean = _ensure_forward_output(ctx, forward_node, mean_conn, (rows, ), torch.float32)
+    rstd = _ensure_forward_output(ctx, forward_node, rstd_conn, (rows, ), torch.float32)
+    g = _new(ctx, "LayerNormalizationGrad", forward_node.label + "_backward", axis=-1)
+    _read(ctx, x_arr, g, "X")
+    connect_input_from_forward(forward_node, g, ctx, scale_conn, "scale")
+    _read(ctx, mean, g, "mean")
+    _read(ctx, rstd, g, "inv_std_var")
+    return g, mean, rstd
+
+
+@autoregister_params(op="LayerNormalization", name=NAME)
+class HipLayerNormalizationBackward(BackwardImplementation):
+    """Backward of the fused LayerNorm chain: one LayerNormalizationGrad node (plus the forward node's
+    Mean / InvStdDev outputs, added here if the forward graph did not ask for them)."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        return True
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        x = _in_arr(context, forward_node, "X")
+        g, _, _ = _ln_backward(forward_node, context, x, "Scale", "B", ["X"], "Mean", "InvStdDev", required_gradients)
+        sdfg = context.forward_sdfg
+        h = sdfg.arrays[x].shape[-1]
+        req = {"X": "X_grad", "Scale": "scale_grad", "B": "bias_grad"}
+        # the kernel always produces all three; unused ones land in scratch transients
+        for conn, gconn in req.items():
+            if conn not in required_gradients:
+                shape = sdfg.arrays[x].shape if conn == "X" else (h, )
+                dt = sdfg.arrays[x].dtype if conn == "X" else torch.float32
+                name, _ = sdfg.add_transient("%s_unused_%s" % (forward_node.label, gconn), shape, dt)
+                _write(context, g, gconn, name)
+        return g, BackwardResult(required_grad_names={c: req[c] for c in required_gradients if c in req},
+                                 given_grad_names={"Y": "Y_grad"})
+
+
+# ----------------------------------------------------------------------------- elementwise
+def _make_unary_backward(op: str, grad_op: str, in_conn: str, out_conn: str):
+    class _B(BackwardImplementation):
+        @staticmethod
+        def backward(forward_node, context, given_gradients, required_gradients):
+            g = _new(context, grad_op, forward_node.label + "_backward")
+            connect_input_from_forward(forward_node, g, context, in_conn, "X")
+            return g, BackwardResult(required_grad_names={in_conn: "dX"}, given_grad_names={out_conn: "dY"})
+
+    _B.__name__ = "Hip%sBackward" % op
+    _B.__doc__ = "dX = dY * f'(X) as one %s node." % grad_op
+    return autoregister_params(op=op, name=NAME)(_B)
+
+
+HipGeluBackward = _make_unary_backward("Gelu", "GeluGrad", "X", "Y")
+HipSwishBackward = _make_unary_backward("Swish", "SwishGrad", "X", "Y")
+HipSigmoidBackward = _make_unary_backward("Sigmoid", "SigmoidGrad", "X", "Y")
+HipReluBackward = _make_unary_backward("Relu", "ReluGrad", "X", "Y")
+HipTanhBackward = _make_unary_backward("Tanh", "TanhGrad", "input", "output")
+
+
+@autoregister_params(op="Add", name=NAME)
+class HipAddBackward(BackwardImplementation):
+    """Add: the gradient passes through to an operand of the output's shape; a broadcast operand gets
+    the gradient reduced over the broadcast (leading) dims — ReverseReduce in reverse
+    (autodiff/implementations/dace_nodes.py:13-105)."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            out = next(iter(state.out_edges_by_connector(node, "C"))).data.data
+            oshape = sdfg.arrays[out].shape
+            for conn in ("A", "B"):
+                arr = next(iter(state.in_edges_by_connector(node, conn))).data.data
+                shp = sdfg.arrays[arr].shape
+                if shp == oshape:
+                    continue
+                k = len(shp)
+                if not (k <= len(oshape) and tuple(oshape[len(oshape) - k:]) == tuple(shp)):
+                    return False
+            return True
+        except StopIteration:
+            return False
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        sdfg = context.forward_sdfg
+        oshape = sdfg.arrays[_out_arr(context, forward_node, "C")].shape
+        group = BackwardGroup(forward_node.label + "_backward")
+        req, passthrough = {}, {}
+        for conn in required_gradients:
+            shp = sdfg.arrays[_in_arr(context, forward_node, conn)].shape
+            if shp == oshape:
+                passthrough[conn] = "C"
+            else:
+                rs = _new(context, "ReduceSum", "%s_%s_grad" % (forward_node.label, conn),
+                          axes=list(range(len(oshape) - len(shp))), keepdims=0)
+                rs.add_in_connector("data")
+                group.map_input("C_grad", rs, "data")
+                group.map_output(conn + "_grad", rs, "reduced")
+                req[conn] = conn + "_grad"
+        return group, BackwardResult(required_grad_names=req, given_grad_names={"C": "C_grad"},
+                                     passthrough=passthrough)
+
+
+# ----------------------------------------------------------------------------- convolution
+@autoregister_params(op="Conv", name=NAME)
+class HipConvBackward(BackwardImplementation):
+    """One ConvGrad node for dX, dW, dB — the three cuDNN backward calls of onnx_ops.py:663-703. fp32; a Conv
+    with a folded activation is not differentiated (un-fuse it first)."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        return getattr(node, "_activation", "none") == "none"
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        attrs = {k: getattr(forward_node, k) for k in ("auto_pad", "dilations", "group", "kernel_shape", "pads",
+                                                       "strides")}
+        g = _new(context, "ConvGrad", forward_node.label + "_backward", **attrs)
+        connect_input_from_forward(forward_node, g, context, "X")
+        connect_input_from_forward(forward_node, g, context, "W")
+        names = {"X": "dX", "W": "dW", "B": "dB"}
+        for c in required_gradients:
+            g.add_out_connector(names[c])
+        return g, BackwardResult(required_grad_names={c: names[c] for c in required_gradients},
+                                 given_grad_names={"Y": "dY"})

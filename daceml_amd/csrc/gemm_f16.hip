@@ -17,6 +17,8 @@
 // into RU chunks of eight K values, so no separate transpose kernel or HBM round trip is needed.
 #include "common.h"
 
+#include <type_traits>
+
 namespace dml {
 namespace {
 
@@ -26,85 +28,122 @@ constexpr int kRowBytes = BK * 2;
 constexpr int kXcds = 8;
 
 struct GemmArgs {
-    const _Float16* a;
-    const _Float16* b;
-    void* c;
-    const void* bias;
-    const void* residual;
-    void* pre;
     int m, n, k;
     int64_t sam, sak, sbn, sbk, scm;
     int batch1, batch2;  // extents of the two inner batch dims (outer one is implied)
     int64_t sab[3], sbb[3], scb[3];
     float alpha, beta;
-    int out_f32, bias_f32, act, bias_m;
+    int out_f32, bias_f32, act, bias_m, c_vec;
     int tiles_m, tiles_n;
     long long total_blocks;
 };
 
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 
 // ---------------------------------------------------------------- global -> registers
-// K-contiguous operand: thread t loads chunks q = t + i*256 of the [R][64] tile.
+// The loaders are branch-free in the steady state. Rows past the end of the operand are clamped to
+// the last valid row (they only feed rows/columns of C that are never stored); K past the end is
+// zero-filled, and only the last K step takes that path. Offsets are 32-bit element offsets from
+// the operand's batch base (the host falls back to the generic loader when they would not fit).
+
+// K-contiguous operand (k % 8 == 0): thread t loads chunks q = t + i*256 of the [R][64] tile.
+// Loads never branch: a chunk past the end of K is fetched from the last valid chunk instead and
+// replaced by zeros when it is written to LDS.
 template <int R>
 struct LoaderKC {
     static constexpr int N = R * 8 / kThreads;
     u32x4 v[N];
-    __device__ __forceinline__ void load(const _Float16* base, int64_t s_row, int row0, int rows, int k0, int k) {
+    int off[N];
+    int c8;       // first k of this thread's chunk inside a K step
+    int k_valid;  // k of the tile held in v[] minus its k0 (chunks with c8 >= k_valid are zero)
+    __device__ __forceinline__ void init(int64_t s_row, int64_t, int row0, int rows) {
+        c8 = (threadIdx.x & 7) * 8;
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             const int q = threadIdx.x + i * kThreads;
-            const int r = q >> 3, c = q & 7;
-            const int gr = row0 + r, gk = k0 + c * 8;
-            const _Float16* p = base + (int64_t)gr * s_row + gk;
-            if (gr < rows && gk + 8 <= k) {
-                v[i] = *reinterpret_cast<const u32x4*>(p);
-            } else {
-                half8 h = {};
-                if (gr < rows) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (gk + e < k) h[e] = p[e];
-                }
-                v[i] = __builtin_bit_cast(u32x4, h);
-            }
+            const int r = min(row0 + (q >> 3), rows - 1);
+            off[i] = (int)(r * s_row);
         }
     }
+    __device__ __forceinline__ void load(const _Float16* base, int64_t, int k0, int k) {
+        k_valid = k - k0;
+        const int kc = min(k0 + c8, k - 8);
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = *reinterpret_cast<const u32x4*>(base + off[i] + kc);
+    }
     __device__ __forceinline__ void store(char* tile) const {
+        const bool ok = c8 < k_valid;
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             const int q = threadIdx.x + i * kThreads;
             const int r = q >> 3, c = q & 7;
-            *reinterpret_cast<u32x4*>(tile + r * kRowBytes + ((c ^ swz(r)) << 4)) = v[i];
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4*>(tile + r * kRowBytes + ((c ^ swz(r)) << 4)) = ok ? v[i] : z;
         }
     }
 };
 
-// Row-contiguous operand (element (row, k) at k*s_k + row): thread t owns K block kb = t/32
-// (eight K values) of the RU rows starting at (t%32)*RU.
+// K-contiguous operand with k % 64 == 0, loaded straight into LDS (global_load_lds, 16 bytes per
+// lane): no staging registers and no LDS store instructions. One wave instruction fills 1 KiB =
+// eight tile rows; lane l lands at (row l/8, chunk slot l%8) of that group, so it fetches the
+// global chunk that the swizzle maps to this slot.
+template <int R>
+struct LoaderKCDirect {
+    static constexpr int N = R / 32;  // instructions per wavefront per tile
+    int off[N];
+    int wave;
+    __device__ __forceinline__ void init(int64_t s_row, int64_t, int row0, int rows) {
+        const int lane = threadIdx.x & (kWave - 1);
+        wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int r = (i * 4 + wave) * 8 + (lane >> 3);
+            const int c = (lane & 7) ^ swz(r);
+            off[i] = (int)(min(row0 + r, rows - 1) * s_row) + c * 8;
+        }
+    }
+    __device__ __forceinline__ void issue(const _Float16* base, int k0, char* tile) const {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(base + off[i] + k0),
+                (__attribute__((address_space(3))) void*)(tile + (i * 4 + wave) * 1024), 16, 0, 0);
+        }
+    }
+    __device__ __forceinline__ void load(const _Float16*, int64_t, int, int) {}
+    __device__ __forceinline__ void store(char*) const {}
+};
+
+// Row-contiguous operand (element (row, k) at k*s_k + row; rows % RU == 0): thread t owns K block
+// kb = t/32 (eight K values) of the RU rows starting at (t%32)*RU and transposes them in registers.
+// K rows past the end are fetched from row k-1 and zeroed on the way to LDS.
 template <int R>
 struct LoaderRC {
     static constexpr int RU = R / 32;  // 4 for R=128, 8 for R=256
     typedef _Float16 rowvec __attribute__((ext_vector_type(RU)));
     rowvec v[8];
-    __device__ __forceinline__ void load(const _Float16* base, int64_t s_k, int row0, int rows, int k0, int k) {
-        const int kb = threadIdx.x >> 5, rg = threadIdx.x & 31;
-        const int gr = row0 + rg * RU;
+    int off;
+    int k_valid;
+    __device__ __forceinline__ void init(int64_t, int64_t, int row0, int rows) {
+        const int rg = threadIdx.x & 31;
+        off = min(row0 + rg * RU, rows - RU);
+    }
+    __device__ __forceinline__ void load(const _Float16* base, int64_t s_k, int k0, int k) {
+        const int kb8 = (threadIdx.x >> 5) * 8;
+        k_valid = k - k0 - kb8;
+        const _Float16* p = base + off;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const int gk = k0 + kb * 8 + j;
-            const _Float16* p = base + (int64_t)gk * s_k + gr;
-            if (gk < k && gr + RU <= rows) {
-                v[j] = *reinterpret_cast<const rowvec*>(p);
-            } else {
-                rowvec h = {};
-                if (gk < k) {
-#pragma unroll
-                    for (int e = 0; e < RU; ++e)
-                        if (gr + e < rows) h[e] = p[e];
-                }
-                v[j] = h;
-            }
+            const int gk = min(k0 + kb8 + j, k - 1);
+            v[j] = *reinterpret_cast<const rowvec*>(p + (int64_t)gk * s_k);
         }
     }
     __device__ __forceinline__ void store(char* tile) const {
@@ -113,30 +152,34 @@ struct LoaderRC {
         for (int e = 0; e < RU; ++e) {
             half8 o;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) o[j] = v[j][e];
+            for (int j = 0; j < 8; ++j) o[j] = j < k_valid ? v[j][e] : (_Float16)0;
             const int r = rg * RU + e;
             *reinterpret_cast<half8*>(tile + r * kRowBytes + ((kb ^ swz(r)) << 4)) = o;
         }
     }
 };
 
-// Any strides, any alignment: element loads. Correct everywhere, fast nowhere.
+// Any strides, any alignment: guarded element loads. Correct everywhere, fast nowhere.
 template <int R>
 struct LoaderGeneric {
     static constexpr int N = R * 8 / kThreads;
     half8 v[N];
-    __device__ __forceinline__ void load(const _Float16* base, int64_t s_row, int64_t s_k, int row0, int rows, int k0,
-                                         int k) {
-#pragma unroll
+    int64_t s_row_, s_k_;
+    int row0_, rows_;
+    __device__ __forceinline__ void init(int64_t s_row, int64_t s_k, int row0, int rows) {
+        s_row_ = s_row; s_k_ = s_k; row0_ = row0; rows_ = rows;
+    }
+    __device__ __forceinline__ void load(const _Float16* base, int64_t, int k0, int k) {
+#pragma unroll 1
         for (int i = 0; i < N; ++i) {
             const int q = threadIdx.x + i * kThreads;
             const int r = q >> 3, c = q & 7;
-            const int gr = row0 + r, gk = k0 + c * 8;
+            const int gr = row0_ + r, gk = k0 + c * 8;
             half8 h = {};
-            if (gr < rows) {
+            if (gr < rows_) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    if (gk + e < k) h[e] = base[(int64_t)gr * s_row + (int64_t)(gk + e) * s_k];
+                    if (gk + e < k) h[e] = base[(int64_t)gr * s_row_ + (int64_t)(gk + e) * s_k_];
             }
             v[i] = h;
         }
@@ -155,19 +198,116 @@ template <int R, int MODE> struct LoaderSel;
 template <int R> struct LoaderSel<R, 0> { using type = LoaderKC<R>; };
 template <int R> struct LoaderSel<R, 1> { using type = LoaderRC<R>; };
 template <int R> struct LoaderSel<R, 2> { using type = LoaderGeneric<R>; };
+template <int R> struct LoaderSel<R, 3> { using type = LoaderKCDirect<R>; };
 
-template <int MODE, typename L>
-__device__ __forceinline__ void do_load(L& l, const _Float16* base, int64_t s_row, int64_t s_k, int row0, int rows,
-                                        int k0, int k) {
-    if constexpr (MODE == 0) l.load(base, s_row, row0, rows, k0, k);
-    else if constexpr (MODE == 1) l.load(base, s_k, row0, rows, k0, k);
-    else l.load(base, s_row, s_k, row0, rows, k0, k);
+// ---------------------------------------------------------------- epilogue helper
+// One wavefront writes a 32 x WN strip held in LDS (fp32, row pitch WN+4) to C: lane -> (row,
+// eight consecutive columns). v = alpha*acc + bias; pre_out = v; v = act(v) + residual + beta*C.
+// ACT = false compiles the activation switch out (most contractions have none).
+template <typename OutT> struct OutVec;
+template <> struct OutVec<_Float16> { typedef half8 type; };
+template <> struct OutVec<float> { typedef float type __attribute__((ext_vector_type(8))); };
+
+template <typename OutT, int WN, bool ACT>
+__device__ __forceinline__ void store_strip(const GemmArgs& g, void* c_ptr, void* pre_ptr, const void* res_ptr,
+                                            const void* bias_ptr, const float* strip, int mb, int nb, int64_t coff,
+                                            int lane) {
+    typedef typename OutVec<OutT>::type ovec;
+    constexpr int PITCH = WN + 4;
+    constexpr int CPR = WN / 8;
+    constexpr int ITER = 32 * CPR / kWave;
+    OutT* C = reinterpret_cast<OutT*>(c_ptr);
+    OutT* P = reinterpret_cast<OutT*>(pre_ptr);
+    const OutT* R = reinterpret_cast<const OutT*>(res_ptr);
+    // without an activation the body is small: unroll so that LDS reads and global stores of
+    // several rows overlap; with one, keep a single copy of the activation code
+#pragma unroll(ACT ? 1 : 4)
+    for (int it = 0; it < ITER; ++it) {
+        const int idx = it * kWave + lane;
+        const int r = idx / CPR, c8 = (idx % CPR) * 8;
+        const int m = mb + r, n = nb + c8;
+        if (m >= g.m || n >= g.n) continue;
+        const floatx4 lo = *reinterpret_cast<const floatx4*>(strip + r * PITCH + c8);
+        const floatx4 hi = *reinterpret_cast<const floatx4*>(strip + r * PITCH + c8 + 4);
+        float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        const int64_t off = coff + (int64_t)m * g.scm + n;
+        const bool full = g.c_vec && n + 8 <= g.n;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= g.alpha;
+        if (bias_ptr) {
+            if (g.bias_m) {
+                const float b = g.bias_f32 ? reinterpret_cast<const float*>(bias_ptr)[m]
+                                           : (float)reinterpret_cast<const _Float16*>(bias_ptr)[m];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += b;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int ne = min(n + e, g.n - 1);
+                    v[e] += g.bias_f32 ? reinterpret_cast<const float*>(bias_ptr)[ne]
+                                       : (float)reinterpret_cast<const _Float16*>(bias_ptr)[ne];
+                }
+            }
+        }
+        if (full) {
+            if (P) {
+                ovec pv;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    pv[e] = (OutT)v[e];
+                    v[e] = (float)pv[e];  // the un-fused graph reads the stored pre-activation back
+                }
+                *reinterpret_cast<ovec*>(P + off) = pv;
+            }
+            if constexpr (ACT) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = apply_act(g.act, v[e]);
+            }
+            if (R) {
+                const ovec rv = *reinterpret_cast<const ovec*>(R + off);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += (float)rv[e];
+            }
+            if (g.beta != 0.f) {
+                const ovec cv = *reinterpret_cast<const ovec*>(C + off);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += g.beta * (float)cv[e];
+            }
+            ovec ov;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ov[e] = (OutT)v[e];
+            *reinterpret_cast<ovec*>(C + off) = ov;
+        } else {
+            // ragged or unaligned tail: element by element (rare; kept out of line by the branch)
+            const int cnt = min(8, g.n - n);
+            float x = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (e < cnt) {
+                    x = v[e];
+                    if (P) {
+                        const OutT h = (OutT)x;
+                        P[off + e] = h;
+                        x = (float)h;
+                    }
+                    if constexpr (ACT) x = apply_act(g.act, x);
+                    if (R) x += (float)R[off + e];
+                    if (g.beta != 0.f) x += g.beta * (float)C[off + e];
+                    C[off + e] = (OutT)x;
+                }
+            }
+        }
+    }
 }
 
 // ---------------------------------------------------------------- the kernel
-// AMODE / BMODE: 0 = K-contiguous, 1 = row-contiguous, 2 = generic strides.
-template <int BM, int BN, int WM, int WN, int AMODE, int BMODE>
-__global__ __launch_bounds__(kThreads) void gemm_f16_kernel(GemmArgs g) {
+// AMODE / BMODE: 0 = K-contiguous via registers, 1 = row-contiguous, 2 = generic strides,
+// 3 = K-contiguous straight to LDS (k % 64 == 0).
+template <int BM, int BN, int WM, int WN, int AMODE, int BMODE, bool ACT>
+__global__ __launch_bounds__(kThreads) void gemm_f16_kernel(const _Float16* __restrict__ a_ptr,
+                                                            const _Float16* __restrict__ b_ptr, void* c_ptr,
+                                                            const void* bias_ptr, const void* res_ptr, void* pre_ptr,
+                                                            const GemmArgs g) {
     static_assert((BM / WM) * (BN / WN) == kThreads / kWave, "four wavefronts per workgroup");
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes;
@@ -189,8 +329,8 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(GemmArgs g) {
     const int z2 = (int)(batch % g.batch2);
     const int z1 = (int)((batch / g.batch2) % g.batch1);
     const int z0 = (int)(batch / ((long long)g.batch2 * g.batch1));
-    const _Float16* A = g.a + z0 * g.sab[0] + z1 * g.sab[1] + z2 * g.sab[2];
-    const _Float16* B = g.b + z0 * g.sbb[0] + z1 * g.sbb[1] + z2 * g.sbb[2];
+    const _Float16* A = a_ptr + z0 * g.sab[0] + z1 * g.sab[1] + z2 * g.sab[2];
+    const _Float16* B = b_ptr + z0 * g.sbb[0] + z1 * g.sbb[1] + z2 * g.sbb[2];
     const int64_t coff = z0 * g.scb[0] + z1 * g.scb[1] + z2 * g.scb[2];
     const int m0 = tm * BM, n0 = tn * BN;
 
@@ -210,99 +350,106 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(GemmArgs g) {
     typename LoaderSel<BN, BMODE>::type lb;
 
     const int nk = (g.k + BK - 1) / BK;
-    do_load<AMODE>(la, A, g.sam, g.sak, m0, g.m, 0, g.k);
-    do_load<BMODE>(lb, B, g.sbn, g.sbk, n0, g.n, 0, g.k);
-    la.store(lds);
-    lb.store(lds + A_BYTES);
+    la.init(g.sam, g.sak, m0, g.m);
+    lb.init(g.sbn, g.sbk, n0, g.n);
+    if (nk > 0) {
+        if constexpr (AMODE == 3) la.issue(A, 0, lds);
+        if constexpr (BMODE == 3) lb.issue(B, 0, lds + A_BYTES);
+        la.load(A, g.sak, 0, g.k);
+        lb.load(B, g.sbk, 0, g.k);
+        la.store(lds);
+        lb.store(lds + A_BYTES);
+    }
     __syncthreads();
 
+    // Fragment reads are software-pipelined one K sub-step (16) ahead of the MFMAs that consume
+    // them, and the barrier that publishes the next tile sits before the last sub-step, so the LDS
+    // latency of the first fragments of tile t+1 hides behind the last MFMAs of tile t.
     const int frow = lane & 31, fk = lane >> 5;
+    const int a_row = wm * WM + frow, b_row = wn * WN + frow;
+    half8 af[2][TM], bf[2][TN];
+    auto read_frags = [&](const char* buf, int kk, half8(&fa)[TM], half8(&fb)[TN]) {
+        const int c = kk * 2 + fk;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int r = a_row + i * 32;
+            fa[i] = *reinterpret_cast<const half8*>(buf + r * kRowBytes + ((c ^ swz(r)) << 4));
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int r = b_row + j * 32;
+            fb[j] = *reinterpret_cast<const half8*>(buf + A_BYTES + r * kRowBytes + ((c ^ swz(r)) << 4));
+        }
+    };
+    if (nk > 0) read_frags(lds, 0, af[0], bf[0]);
     for (int kt = 0; kt < nk; ++kt) {
         char* cur = lds + (kt & 1) * (A_BYTES + B_BYTES);
         char* nxt = lds + ((kt + 1) & 1) * (A_BYTES + B_BYTES);
         const bool more = kt + 1 < nk;
+#ifndef LAB_NO_GLOBAL
         if (more) {
-            do_load<AMODE>(la, A, g.sam, g.sak, m0, g.m, (kt + 1) * BK, g.k);
-            do_load<BMODE>(lb, B, g.sbn, g.sbk, n0, g.n, (kt + 1) * BK, g.k);
+            if constexpr (AMODE == 3) la.issue(A, (kt + 1) * BK, nxt);
+            if constexpr (BMODE == 3) lb.issue(B, (kt + 1) * BK, nxt + A_BYTES);
+            la.load(A, g.sak, (kt + 1) * BK, g.k);
+            lb.load(B, g.sbk, (kt + 1) * BK, g.k);
         }
-        const char* at = cur + (wm * WM + frow) * kRowBytes;
-        const char* bt = cur + A_BYTES + (wn * WN + frow) * kRowBytes;
+#endif
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
-            half8 af[TM], bf[TN];
-            const int c = kk * 2 + fk;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int r = wm * WM + i * 32 + frow;
-                af[i] = *reinterpret_cast<const half8*>(at + i * 32 * kRowBytes + ((c ^ swz(r)) << 4));
+            if (kk + 1 < BK / 16) {
+                read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+            } else {
+#ifndef LAB_NO_STORE
+                if (more) {
+                    la.store(nxt);
+                    lb.store(nxt + A_BYTES);
+                }
+#endif
+                __syncthreads();
+                if (more) read_frags(nxt, 0, af[0], bf[0]);
             }
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int r = wn * WN + j * 32 + frow;
-                bf[j] = *reinterpret_cast<const half8*>(bt + j * 32 * kRowBytes + ((c ^ swz(r)) << 4));
-            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[kk & 1][i], bf[kk & 1][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (more) {
-            la.store(nxt);
-            lb.store(nxt + A_BYTES);
-        }
-        __syncthreads();
     }
+    __syncthreads();
 
-    // ---- epilogue. acc[i][j][e] is C[m, n] with n = l%32 and m = (e/4)*8 + (l/32)*4 + e%4
-    // inside the 32x32 block.
+    // ---- epilogue. acc[i][j][e] is C[m, n] with n = l%32 and m = (e/4)*8 + (l/32)*4 + e%4 inside
+    // the 32x32 block. Each wavefront stages one 32 x WN strip at a time in its own LDS region and
+    // reads it back row-wise, so that global accesses are 128-bit and contiguous along n.
+    constexpr int PITCH = WN + 4;
+    float* strip = reinterpret_cast<float*>(lds) + wave * 32 * PITCH;
     const int ncol = lane & 31, mgrp = lane >> 5;
+    static_for<0, TM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        static_for<0, TN>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int n = n0 + wn * WN + j * 32 + ncol;
-        if (n >= g.n) continue;
-        float bias_n = 0.f;
-        if (g.bias && !g.bias_m) bias_n = g.bias_f32 ? reinterpret_cast<const float*>(g.bias)[n]
-                                                     : (float)reinterpret_cast<const _Float16*>(g.bias)[n];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm * WM + i * 32 + (e >> 2) * 8 + mgrp * 4 + (e & 3);
-                if (m >= g.m) continue;
-                const int64_t off = coff + (int64_t)m * g.scm + n;
-                float bias = bias_n;
-                if (g.bias && g.bias_m) bias = g.bias_f32 ? reinterpret_cast<const float*>(g.bias)[m]
-                                                          : (float)reinterpret_cast<const _Float16*>(g.bias)[m];
-                float v = g.alpha * acc[i][j][e] + bias;
-                if (g.out_f32) {
-                    if (g.pre) reinterpret_cast<float*>(g.pre)[off] = v;
-                    v = apply_act(g.act, v);
-                    if (g.residual) v += reinterpret_cast<const float*>(g.residual)[off];
-                    if (g.beta != 0.f) v += g.beta * reinterpret_cast<float*>(g.c)[off];
-                    reinterpret_cast<float*>(g.c)[off] = v;
-                } else {
-                    if (g.pre) {
-                        // the un-fused graph stores the pre-activation in fp16 and reads it back
-                        const _Float16 h = (_Float16)v;
-                        reinterpret_cast<_Float16*>(g.pre)[off] = h;
-                        v = (float)h;
-                    }
-                    v = apply_act(g.act, v);
-                    if (g.residual) v += (float)reinterpret_cast<const _Float16*>(g.residual)[off];
-                    if (g.beta != 0.f) v += g.beta * (float)reinterpret_cast<_Float16*>(g.c)[off];
-                    reinterpret_cast<_Float16*>(g.c)[off] = (_Float16)v;
-                }
-            }
-        }
-    }
+            for (int e = 0; e < 16; ++e)
+                strip[((e >> 2) * 8 + mgrp * 4 + (e & 3)) * PITCH + j * 32 + ncol] = acc[i][j][e];
+        });
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int mb = m0 + wm * WM + i * 32, nb = n0 + wn * WN;
+        if (g.out_f32) store_strip<float, WN, ACT>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, strip, mb, nb, coff, lane);
+        else store_strip<_Float16, WN, ACT>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, strip, mb, nb, coff, lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    });
 }
 
 // ---------------------------------------------------------------- host side
 enum { CFG_128x128 = 0, CFG_256x128 = 1, CFG_256x256 = 2 };
 
 template <int BM, int BN, int WM, int WN>
-int launch_cfg(GemmArgs& g, int amode, int bmode, long long batch, hipStream_t st) {
+int launch_cfg(GemmArgs& g, const _Float16* pa, const _Float16* pb, void* pc, const void* pbias, const void* pres,
+               void* ppre, int amode, int bmode, long long batch, hipStream_t st) {
     g.tiles_m = (g.m + BM - 1) / BM;
     g.tiles_n = (g.n + BN - 1) / BN;
     const long long total = (long long)g.tiles_m * g.tiles_n * batch;
@@ -311,7 +458,8 @@ int launch_cfg(GemmArgs& g, int amode, int bmode, long long batch, hipStream_t s
     const size_t lds = (size_t)2 * (BM + BN) * kRowBytes;
 #define DML_GEMM_CASE(AM, BMD)                                                                                \
     if (amode == AM && bmode == BMD) {                                                                        \
-        auto kern = gemm_f16_kernel<BM, BN, WM, WN, AM, BMD>;                                                 \
+        auto kern = g.act != DMLHIP_ACT_NONE ? gemm_f16_kernel<BM, BN, WM, WN, AM, BMD, true>                  \
+                                             : gemm_f16_kernel<BM, BN, WM, WN, AM, BMD, false>;                \
         if (lds > 64 * 1024) {                                                                                \
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
                                                (int)lds);                                                     \
@@ -320,13 +468,16 @@ int launch_cfg(GemmArgs& g, int amode, int bmode, long long batch, hipStream_t s
                 return (int)e;                                                                                \
             }                                                                                                 \
         }                                                                                                     \
-        hipLaunchKernelGGL(kern, (unsigned)total, kThreads, lds, st, g);                                      \
+        hipLaunchKernelGGL(kern, (unsigned)total, kThreads, lds, st, pa, pb, pc, pbias, pres, ppre, g);                                      \
         return launch_status("gemm_f16");                                                                     \
     }
     DML_GEMM_CASE(0, 0)
     DML_GEMM_CASE(0, 1)
     DML_GEMM_CASE(1, 0)
     DML_GEMM_CASE(1, 1)
+    DML_GEMM_CASE(3, 3)
+    DML_GEMM_CASE(3, 1)
+    DML_GEMM_CASE(1, 3)
     if constexpr (BM == 128 && BN == 128) {
         DML_GEMM_CASE(2, 2)
     }
@@ -335,18 +486,22 @@ int launch_cfg(GemmArgs& g, int amode, int bmode, long long batch, hipStream_t s
     return DMLHIP_ERR_UNSUPPORTED;
 }
 
-// 0 = K-contiguous with 16-byte-aligned rows, 1 = row-contiguous likewise, 2 = anything else
-int operand_mode(const void* p, int64_t s_row, int64_t s_k, const int64_t* sb, const int64_t* batch) {
+// 0 = K-contiguous, 1 = row-contiguous (both with 16-byte-aligned vectors, extents that are
+// multiples of the vector length and 32-bit element offsets), 2 = anything else.
+int operand_mode(const void* p, int64_t rows, int64_t k, int64_t s_row, int64_t s_k, const int64_t* sb,
+                 const int64_t* batch) {
     bool bs_ok = true;
     for (int i = 0; i < 3; ++i)
         if (batch[i] > 1 && sb[i] % 8 != 0) bs_ok = false;
     if (!aligned16(p) || !bs_ok) return 2;
-    if (s_k == 1 && s_row % 8 == 0) return 0;
-    if (s_row == 1 && s_k % 8 == 0) return 1;
+    if ((double)(rows - 1) * s_row + (double)(k + 64) * s_k > 2.0e9) return 2;
+    if (s_k == 1 && s_row % 8 == 0 && k % 8 == 0) return 0;
+    if (s_row == 1 && s_k % 8 == 0 && rows % 8 == 0) return 1;
     return 2;
 }
 
 int g_force_cfg = -1;  // test hook: pin the tile configuration
+int g_direct_lds = 1;  // test hook: 0 forces the register-staged loaders
 
 }  // namespace
 }  // namespace dml
@@ -357,6 +512,7 @@ extern "C" {
 
 // Not part of the public header: lets the tests exercise every tile configuration.
 void dmlhip_debug_force_gemm_config(int cfg) { g_force_cfg = cfg; }
+void dmlhip_debug_gemm_direct_lds(int on) { g_direct_lds = on; }
 
 int dmlhip_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, void* c, const void* bias,
                     const void* residual, void* pre_out, void* stream) {
@@ -384,12 +540,6 @@ int dmlhip_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, voi
     DML_REQUIRE(d->k == 0 || (a && b), DMLHIP_ERR_NULL, "gemm_f16: NULL operand");
 
     GemmArgs g;
-    g.a = (const _Float16*)a;
-    g.b = (const _Float16*)b;
-    g.c = c;
-    g.bias = bias;
-    g.residual = residual;
-    g.pre = pre_out;
     g.m = (int)d->m; g.n = (int)d->n; g.k = (int)d->k;
     g.sam = d->a_stride_m; g.sak = d->a_stride_k; g.sbn = d->b_stride_n; g.sbk = d->b_stride_k;
     g.scm = d->c_stride_m;
@@ -400,10 +550,30 @@ int dmlhip_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, voi
     g.alpha = d->alpha; g.beta = d->beta;
     g.out_f32 = d->out_dtype == DMLHIP_F32; g.bias_f32 = d->bias_dtype == DMLHIP_F32; g.act = d->act;
     g.bias_m = d->bias_along_m != 0;
+    {
+        // 128-bit accesses to C / pre_out / residual need 8-element granularity everywhere
+        const int gran = 8;
+        bool ok = aligned16(c) && (!residual || aligned16(residual)) && (!pre_out || aligned16(pre_out)) &&
+                  d->c_stride_m % gran == 0;
+        if (g.out_f32)
+            ok = ok && (reinterpret_cast<uintptr_t>(c) % 32 == 0) &&
+                 (!residual || reinterpret_cast<uintptr_t>(residual) % 32 == 0) &&
+                 (!pre_out || reinterpret_cast<uintptr_t>(pre_out) % 32 == 0);
+        for (int i = 0; i < 3; ++i)
+            if (d->batch[i] > 1 && d->c_stride_batch[i] % gran != 0) ok = false;
+        g.c_vec = ok;
+    }
 
-    int amode = d->k == 0 ? 0 : operand_mode(a, d->a_stride_m, d->a_stride_k, d->a_stride_batch, d->batch);
-    int bmode = d->k == 0 ? 0 : operand_mode(b, d->b_stride_n, d->b_stride_k, d->b_stride_batch, d->batch);
+    int amode = d->k == 0 ? 0 : operand_mode(a, d->m, d->k, d->a_stride_m, d->a_stride_k, d->a_stride_batch, d->batch);
+    int bmode = d->k == 0 ? 0 : operand_mode(b, d->n, d->k, d->b_stride_n, d->b_stride_k, d->b_stride_batch, d->batch);
     if (amode == 2 || bmode == 2) amode = bmode = 2;
+    // K-contiguous operands go straight to LDS when K is a whole number of steps; a K-contiguous
+    // operand paired with a register-path K-contiguous one keeps the register path for both.
+    if (d->k % BK == 0 && d->k > 0 && g_direct_lds) {
+        if (amode == 0 && bmode == 0) amode = bmode = 3;
+        else if (amode == 0 && bmode == 1) amode = 3;
+        else if (amode == 1 && bmode == 0) bmode = 3;
+    }
     hipStream_t st = (hipStream_t)stream;
 
     int cfg = g_force_cfg;
@@ -416,9 +586,12 @@ int dmlhip_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, voi
     }
     if (amode == 2) cfg = CFG_128x128;
     switch (cfg) {
-        case CFG_256x256: return launch_cfg<256, 256, 128, 128>(g, amode, bmode, batch, st);
-        case CFG_256x128: return launch_cfg<256, 128, 128, 64>(g, amode, bmode, batch, st);
-        default: return launch_cfg<128, 128, 64, 64>(g, amode, bmode, batch, st);
+        case CFG_256x256: return launch_cfg<256, 256, 128, 128>(g, (const _Float16*)a, (const _Float16*)b, c, bias, residual, pre_out, amode, bmode,
+                                                   batch, st);
+        case CFG_256x128: return launch_cfg<256, 128, 128, 64>(g, (const _Float16*)a, (const _Float16*)b, c, bias, residual, pre_out, amode, bmode,
+                                                   batch, st);
+        default: return launch_cfg<128, 128, 64, 64>(g, (const _Float16*)a, (const _Float16*)b, c, bias, residual, pre_out, amode, bmode,
+                                                   batch, st);
     }
 }
 

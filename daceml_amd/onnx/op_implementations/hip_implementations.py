@@ -1,0 +1,896 @@
+"""The "hip" implementations of the ONNX library nodes: each ``forward`` returns a ``HipTasklet`` that
+calls one (or a few) hand-written gfx950 kernels through the ``dmlhip_*`` C ABI.
+
+Counterparts in the reference: the "pure" expansions of
+daceml/onnx/op_implementations/pure_implementations.py and img_op_implementations.py (whose results
+these must reproduce) and the cuDNN expansion of cudnn_implementations.py (whose role — a native
+library behind an expansion — these play). ``forward_can_be_applied`` never raises: anything outside
+what the kernels cover returns False.
+"""
+import math
+from typing import List, Optional, Sequence
+
+import torch
+
+from ... import _lib as L
+from ... import contraction as C
+from ...hip_tasklet import (F32, I32, I64, HipCall, HipTasklet, I64Array, Null, Ptr, PtrArray, Stream, Struct,
+                            USize, ViewTasklet, Workspace, WorkspaceBytes)
+from ...sdfg import (FLOAT_DTYPES, SDFG, Array, SDFGState, in_desc_with_name, out_desc_with_name)
+from ..forward_implementation_abc import ONNXForward
+from ..nodes import ONNXOp
+from .utils import op_implementation
+
+IMPL = "hip"
+_SFX = {torch.float16: "f16", torch.float32: "f32"}
+_CODE = {torch.float16: L.F16, torch.float32: L.F32}
+_ACT = {"none": L.ACT_NONE, "gelu": L.ACT_GELU, "swish": L.ACT_SWISH, "sigmoid": L.ACT_SIGMOID, "relu": L.ACT_RELU}
+
+
+# ----------------------------------------------------------------------------- helpers
+def _connected(node: ONNXOp, state: SDFGState, is_input: bool) -> List[str]:
+    edges = state.in_edges(node) if is_input else state.out_edges(node)
+    return [e.dst_conn if is_input else e.src_conn for e in edges]
+
+
+def _has_in(node, state, name) -> bool:
+    return name in _connected(node, state, True)
+
+
+def _has_out(node, state, name) -> bool:
+    return name in _connected(node, state, False)
+
+
+def _descs(node, state, sdfg):
+    ins = {e.dst_conn: sdfg.arrays[e.data.data] for e in state.in_edges(node)}
+    outs = {e.src_conn: sdfg.arrays[e.data.data] for e in state.out_edges(node)}
+    return ins, outs
+
+
+def _float_ok(*descs: Array) -> bool:
+    if not descs:
+        return False
+    dt = descs[0].dtype
+    return dt in FLOAT_DTYPES and all(d.dtype == dt for d in descs)
+
+
+def _dense(*descs: Array) -> bool:
+    return all(d.is_contiguous() for d in descs)
+
+
+def _prod(xs: Sequence[int]) -> int:
+    n = 1
+    for x in xs:
+        n *= int(x)
+    return n
+
+
+def _tasklet(node, state, calls, workspace_bytes=0, flops=0, bytes_moved=0, kind=""):
+    return HipTasklet(node.label + "_hip", _connected(node, state, True), _connected(node, state, False), calls,
+                      workspace_bytes, flops, bytes_moved, kind or node.schema.name)
+
+
+def _opt(node, state, name, is_input=True):
+    present = _has_in(node, state, name) if is_input else _has_out(node, state, name)
+    return Ptr(name) if present else Null()
+
+
+def _nbytes(*descs: Array) -> int:
+    return sum(d.total_size * (2 if d.dtype == torch.float16 else 4) for d in descs)
+
+
+# ----------------------------------------------------------------------------- contractions
+def _gemm_struct(plan: C.GemmPlan, alpha, beta, out_dtype, bias_dtype, act) -> L.GemmDesc:
+    d = L.GemmDesc()
+    d.m, d.n, d.k = plan.m, plan.n, plan.k
+    for i in range(3):
+        d.batch[i] = plan.batch[i]
+        d.a_stride_batch[i] = plan.a_stride_batch[i]
+        d.b_stride_batch[i] = plan.b_stride_batch[i]
+        d.c_stride_batch[i] = plan.c_stride_batch[i]
+    d.a_stride_m, d.a_stride_k = plan.a_stride_m, plan.a_stride_k
+    d.b_stride_k, d.b_stride_n = plan.b_stride_k, plan.b_stride_n
+    d.c_stride_m = plan.c_stride_m
+    d.alpha, d.beta = float(alpha), float(beta)
+    d.out_dtype = _CODE[out_dtype]
+    d.bias_dtype = _CODE[bias_dtype]
+    d.act = act
+    d.bias_along_m = 0
+    return d
+
+
+def _einsum_plan(equation: str, a: Array, b: Array) -> Optional[C.GemmPlan]:
+    try:
+        return C.plan_contraction(equation, a.shape, a.strides, b.shape, b.strides)
+    except (C.NotApplicable, ValueError):
+        return None
+
+
+def _einsum_can_apply(equation: str, inputs: List[Array], out: Array, allow_f32_out=False) -> bool:
+    if "..." in equation or not inputs or not _float_ok(*inputs):
+        return False
+    if out.dtype != inputs[0].dtype and not (allow_f32_out and out.dtype == torch.float32):
+        return False
+    if not out.is_contiguous():
+        return False
+    try:
+        if len(inputs) == 1:
+            perm = C.transpose_perm(equation)
+            return perm is not None and inputs[0].is_contiguous() and len(perm) <= L.MAX_DIMS
+        if len(inputs) != 2:
+            return False
+        plan = _einsum_plan(equation, inputs[0], inputs[1])
+        return plan is not None and tuple(plan.out_shape) == tuple(out.shape)
+    except (C.NotApplicable, ValueError):
+        return False
+
+
+def _einsum_tasklet(node, state, equation, a_conn, b_conn, out_conn, a: Array, b: Array, out: Array, alpha=1.0,
+                    beta=0.0, act=L.ACT_NONE, bias: Optional[str] = None, bias_desc: Optional[Array] = None,
+                    residual: Optional[str] = None, pre_out: Optional[str] = None):
+    plan = C.plan_contraction(equation, a.shape, a.strides, b.shape, b.strides)
+    desc = _gemm_struct(plan, alpha, beta, out.dtype, bias_desc.dtype if bias_desc is not None else out.dtype, act)
+    x, y = (b_conn, a_conn) if plan.swapped else (a_conn, b_conn)
+    sym = "dmlhip_gemm_" + _SFX[a.dtype]
+    call = HipCall(sym, [Struct(desc, "dmlhip_gemm_desc"), Ptr(x), Ptr(y), Ptr(out_conn),
+                         Ptr(bias) if bias else Null(), Ptr(residual) if residual else Null(),
+                         Ptr(pre_out) if pre_out else Null(), Stream()])
+    extra = [d for d in (bias_desc, ) if d is not None]
+    return _tasklet(node, state, [call], flops=plan.flops, bytes_moved=_nbytes(a, b, out, *extra), kind="gemm")
+
+
+@op_implementation(op="Einsum", name=IMPL)
+class HipEinsum(ONNXForward):
+    """PureEinsum (pure_implementations.py:219-252): two-operand contractions become one MFMA GEMM
+    launch; one-operand permutations become the transpose kernel (EinsumTranspose, :746-778)."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins = [sdfg.arrays[e.data.data] for e in node.iter_inputs_in_onnx_order(state)]
+            out = out_desc_with_name(node, state, sdfg, "Output")
+            return _einsum_can_apply(node.equation.replace(" ", ""), ins, out)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        eq = node.equation.replace(" ", "")
+        edges = node.iter_inputs_in_onnx_order(state)
+        ins = [sdfg.arrays[e.data.data] for e in edges]
+        out = out_desc_with_name(node, state, sdfg, "Output")
+        if len(ins) == 1:
+            perm = C.transpose_perm(eq)
+            call = HipCall("dmlhip_transpose_" + _SFX[out.dtype],
+                           [Ptr("Inputs__0"), Ptr("Output"), I32(len(perm)), I64Array(tuple(ins[0].shape)),
+                            I64Array(tuple(perm)), Stream()])
+            return _tasklet(node, state, [call], bytes_moved=_nbytes(ins[0], out), kind="transpose")
+        return _einsum_tasklet(node, state, eq, "Inputs__0", "Inputs__1", "Output", ins[0], ins[1], out)
+
+
+@op_implementation(op="FusedEinsum", name=IMPL)
+class HipFusedEinsum(ONNXForward):
+    """A contraction with the scale / bias Add / activation / residual Add that followed it in the
+    exported graph folded into the GEMM epilogue, and Transposes of its operands folded into operand
+    strides (the job of transformation/einsum_fusion.py:102-151 in the reference)."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            if "Inputs__0" not in ins or "Inputs__1" not in ins or "Inputs__2" in ins:
+                return False
+            out = outs["Output"]
+            if node.activation not in _ACT:
+                return False
+            if not _einsum_can_apply(node.equation.replace(" ", ""), [ins["Inputs__0"], ins["Inputs__1"]], out,
+                                     allow_f32_out=True):
+                return False
+            plan = _einsum_plan(node.equation.replace(" ", ""), ins["Inputs__0"], ins["Inputs__1"])
+            if "Bias" in ins:
+                b = ins["Bias"]
+                if not (b.dtype in FLOAT_DTYPES and b.is_contiguous() and b.total_size == plan.n
+                        and b.shape[-1] == plan.n):
+                    return False
+            for name, d in (("Residual", ins.get("Residual")), ("PreActivation", outs.get("PreActivation"))):
+                if d is not None and not (d.is_contiguous() and tuple(d.shape) == tuple(out.shape)
+                                          and d.dtype == out.dtype):
+                    return False
+            return True
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        return _einsum_tasklet(node, state, node.equation.replace(" ", ""), "Inputs__0", "Inputs__1", "Output",
+                               ins["Inputs__0"], ins["Inputs__1"], outs["Output"], alpha=node.alpha,
+                               beta=1.0 if node.accumulate else 0.0, act=_ACT[node.activation],
+                               bias="Bias" if "Bias" in ins else None, bias_desc=ins.get("Bias"),
+                               residual="Residual" if "Residual" in ins else None,
+                               pre_out="PreActivation" if "PreActivation" in outs else None)
+
+
+@op_implementation(op="MatMul", name=IMPL)
+class HipMatMul(ONNXForward):
+    """PureMatMul (pure_implementations.py:111-216): same einsum lowering, then one GEMM launch."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            a = in_desc_with_name(node, state, sdfg, "A")
+            b = in_desc_with_name(node, state, sdfg, "B")
+            y = out_desc_with_name(node, state, sdfg, "Y")
+            if len(a.shape) < 2 or len(b.shape) < 2:  # 1-D operands refused (:114-121)
+                return False
+            return _einsum_can_apply(C.matmul_equation(len(a.shape), len(b.shape)), [a, b], y)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        a = in_desc_with_name(node, state, sdfg, "A")
+        b = in_desc_with_name(node, state, sdfg, "B")
+        y = out_desc_with_name(node, state, sdfg, "Y")
+        return _einsum_tasklet(node, state, C.matmul_equation(len(a.shape), len(b.shape)), "A", "B", "Y", a, b, y)
+
+
+@op_implementation(op="Gemm", name=IMPL)
+class HipGemm(ONNXForward):
+    """PureGemm (pure_implementations.py:380-553): alpha*op(A)op(B) + beta*C with C a vector over the
+    last result index (how nn.Linear exports); alpha and the bias go into the GEMM epilogue."""
+    @staticmethod
+    def _eq(node):
+        a, b = "ik", "kj"
+        if node.transA == 1:
+            a = a[::-1]
+        if node.transB == 1:
+            b = b[::-1]
+        return "%s,%s->ij" % (a, b)
+
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            a, b, y = ins["A"], ins["B"], outs["Y"]
+            if len(a.shape) != 2 or len(b.shape) != 2:
+                return False
+            if not _einsum_can_apply(HipGemm._eq(node), [a, b], y):
+                return False
+            if "C" in ins and node.beta != 0:
+                c = ins["C"]
+                if node.beta != 1 or not c.is_contiguous() or c.dtype != y.dtype:
+                    return False
+                if not (c.total_size == y.shape[-1] and c.shape[-1] == y.shape[-1]):
+                    return False
+            return True
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        use_c = "C" in ins and node.beta != 0
+        return _einsum_tasklet(node, state, HipGemm._eq(node), "A", "B", "Y", ins["A"], ins["B"], outs["Y"],
+                               alpha=node.alpha, bias="C" if use_c else None, bias_desc=ins["C"] if use_c else None)
+
+
+# ----------------------------------------------------------------------------- softmax / layernorm
+@op_implementation(op="Softmax", name=IMPL)
+class HipSoftmax(ONNXForward):
+    """Softmax (pure_implementations.py:309-319), opset-12 semantics: everything from ``axis`` on is one
+    row. One pass over HBM instead of the four maps and three temporaries of the pure expansion."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            x = in_desc_with_name(node, state, sdfg, "input")
+            y = out_desc_with_name(node, state, sdfg, "output")
+            nd = len(x.shape)
+            return (_float_ok(x, y) and _dense(x, y) and x.shape == y.shape and nd >= 1
+                    and -nd <= node.axis < nd)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "input")
+        axis = node.axis % len(x.shape)
+        cols = _prod(x.shape[axis:])
+        rows = _prod(x.shape[:axis])
+        call = HipCall("dmlhip_softmax_" + _SFX[x.dtype], [Ptr("input"), Ptr("output"), I64(rows), I64(cols), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="softmax")
+
+
+@op_implementation(op="SoftmaxGrad", name=IMPL)
+class HipSoftmaxGrad(ONNXForward):
+    """The node DefaultSoftmaxBackward builds from ONNXMul / ONNXReduceSum / a subtraction map
+    (autodiff/implementations/onnx_ops.py:237-275), as one kernel: dx = y*dy - y*sum(y*dy)."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            y, dy, dx = ins["Y"], ins["dY"], outs["dX"]
+            nd = len(y.shape)
+            return (_float_ok(y, dy, dx) and _dense(y, dy, dx) and y.shape == dy.shape == dx.shape
+                    and node.axis % nd == nd - 1)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        y = in_desc_with_name(node, state, sdfg, "Y")
+        cols = y.shape[-1]
+        rows = _prod(y.shape[:-1])
+        call = HipCall("dmlhip_softmax_backward_" + _SFX[y.dtype],
+                       [Ptr("Y"), Ptr("dY"), Ptr("dX"), I64(rows), I64(cols), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=3 * _nbytes(y), kind="softmax_backward")
+
+
+def _ln_common(x: Array, gamma: Array, beta: Optional[Array], axis: int) -> bool:
+    nd = len(x.shape)
+    if nd < 1 or axis % nd != nd - 1:
+        return False
+    h = x.shape[-1]
+    ok = gamma.total_size == h and gamma.is_contiguous() and gamma.dtype == x.dtype
+    if beta is not None:
+        ok = ok and beta.total_size == h and beta.is_contiguous() and beta.dtype == x.dtype
+    return ok
+
+
+def _stat_ok(d: Optional[Array], rows: int) -> bool:
+    return d is None or (d.dtype == torch.float32 and d.is_contiguous() and d.total_size == rows)
+
+
+@op_implementation(op="LayerNormalization", name=IMPL)
+class HipLayerNormalization(ONNXForward):
+    """The exporter's nine-node chain ReduceMean, Sub, Pow, ReduceMean, Add, Sqrt, Div, Mul, Add
+    (pure_implementations.py:101-103,81-83,39-41,76-78,34-36,91-93), fused by the fusion pass into
+    this node and run as one kernel (biased two-pass variance, division by sqrt(var+eps))."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, y = ins["X"], outs["Y"]
+            if "B" not in ins or not (_float_ok(x, y) and _dense(x, y) and x.shape == y.shape):
+                return False
+            rows = _prod(x.shape[:-1])
+            return (_ln_common(x, ins["Scale"], ins["B"], node.axis) and _stat_ok(outs.get("Mean"), rows)
+                    and _stat_ok(outs.get("InvStdDev"), rows) and node.epsilon >= 0)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "X")
+        rows, cols = _prod(x.shape[:-1]), x.shape[-1]
+        call = HipCall("dmlhip_layernorm_" + _SFX[x.dtype],
+                       [Ptr("X"), Null(), Ptr("Scale"), Ptr("B"), Ptr("Y"), Null(), _opt(node, state, "Mean", False),
+                        _opt(node, state, "InvStdDev", False), I64(rows), I64(cols), F32(node.epsilon), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="layernorm")
+
+
+@op_implementation(op="SkipLayerNormalization", name=IMPL)
+class HipSkipLayerNormalization(ONNXForward):
+    """Residual ONNXAdd (pure_implementations.py:76-78) followed by the LayerNorm chain, in one kernel;
+    the sum is rounded to the tensor dtype as the separate Add node would."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, s, y = ins["input"], ins["skip"], outs["output"]
+            if "beta" not in ins or not (_float_ok(x, s, y) and _dense(x, s, y) and x.shape == y.shape == s.shape):
+                return False
+            rows = _prod(x.shape[:-1])
+            so = outs.get("input_skip_bias_sum")
+            if so is not None and not (so.is_contiguous() and so.shape == x.shape and so.dtype == x.dtype):
+                return False
+            return (_ln_common(x, ins["gamma"], ins["beta"], -1) and _stat_ok(outs.get("mean"), rows)
+                    and _stat_ok(outs.get("inv_std_var"), rows) and node.epsilon >= 0)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "input")
+        rows, cols = _prod(x.shape[:-1]), x.shape[-1]
+        has_sum = _has_out(node, state, "input_skip_bias_sum")
+        call = HipCall("dmlhip_layernorm_" + _SFX[x.dtype],
+                       [Ptr("input"), Ptr("skip"), Ptr("gamma"), Ptr("beta"), Ptr("output"),
+                        _opt(node, state, "input_skip_bias_sum", False), _opt(node, state, "mean", False),
+                        _opt(node, state, "inv_std_var", False), I64(rows), I64(cols), F32(node.epsilon), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=(4 if has_sum else 3) * _nbytes(x), kind="add_layernorm")
+
+
+@op_implementation(op="LayerNormalizationGrad", name=IMPL)
+class HipLayerNormalizationGrad(ONNXForward):
+    """Backward of the LayerNorm chain: what the SymPy tasklet reversal plus ReverseReduce
+    (autodiff/backward_pass_generator.py:1284-1421, autodiff/implementations/dace_nodes.py:13-105)
+    evaluate as a sequence of maps. dX in the tensor dtype, scale/bias gradients in fp32."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, dy, dx = ins["X"], ins["Y_grad"], outs["X_grad"]
+            rows, h = _prod(x.shape[:-1]), x.shape[-1]
+            if not (_float_ok(x, dy, dx) and _dense(x, dy, dx) and x.shape == dy.shape == dx.shape):
+                return False
+            for name in ("scale_grad", "bias_grad"):
+                d = outs[name]
+                if not (d.dtype == torch.float32 and d.is_contiguous() and d.total_size == h):
+                    return False
+            return (_ln_common(x, ins["scale"], None, node.axis) and _stat_ok(ins["mean"], rows)
+                    and _stat_ok(ins["inv_std_var"], rows))
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "X")
+        rows, cols = _prod(x.shape[:-1]), x.shape[-1]
+        ws = L.load().dmlhip_layernorm_backward_workspace_bytes(rows, cols)
+        call = HipCall("dmlhip_layernorm_backward_" + _SFX[x.dtype],
+                       [Ptr("Y_grad"), Ptr("X"), Ptr("mean"), Ptr("inv_std_var"), Ptr("scale"), Ptr("X_grad"),
+                        Ptr("scale_grad"), Ptr("bias_grad"), I64(rows), I64(cols), Workspace(), WorkspaceBytes(),
+                        Stream()])
+        return _tasklet(node, state, [call], workspace_bytes=ws, bytes_moved=3 * _nbytes(x), kind="layernorm_backward")
+
+
+# ----------------------------------------------------------------------------- elementwise
+def _bcast_strides(desc: Array, shape: Sequence[int]) -> Optional[List[int]]:
+    nd = len(shape)
+    pad = nd - len(desc.shape)
+    if pad < 0:
+        return None
+    out = []
+    for i in range(nd):
+        if i < pad:
+            out.append(0)
+            continue
+        ext, st = desc.shape[i - pad], desc.strides[i - pad]
+        if ext == shape[i]:
+            out.append(st if ext != 1 else 0)
+        elif ext == 1:
+            out.append(0)
+        else:
+            return None
+    return out
+
+
+def _broadcast_shape(a: Sequence[int], b: Sequence[int]) -> Optional[tuple]:
+    nd = max(len(a), len(b))
+    a = (1, ) * (nd - len(a)) + tuple(a)
+    b = (1, ) * (nd - len(b)) + tuple(b)
+    out = []
+    for x, y in zip(a, b):
+        if x != y and x != 1 and y != 1:
+            return None
+        out.append(max(x, y) if min(x, y) != 0 else 0)
+    return tuple(out)
+
+
+def _make_binary(op_name: str, code: int, a_conn="A", b_conn="B", c_conn="C"):
+    class _Binary(ONNXForward):
+        @staticmethod
+        def forward_can_be_applied(node, state, sdfg) -> bool:
+            try:
+                a = in_desc_with_name(node, state, sdfg, a_conn)
+                b = in_desc_with_name(node, state, sdfg, b_conn)
+                c = out_desc_with_name(node, state, sdfg, c_conn)
+                shape = _broadcast_shape(a.shape, b.shape)
+                return (_float_ok(a, b, c) and shape is not None and shape == tuple(c.shape) and c.is_contiguous()
+                        and len(shape) <= L.MAX_DIMS and a.view_of is None and b.view_of is None)
+            except Exception:
+                return False
+
+        @staticmethod
+        def forward(node, state, sdfg):
+            a = in_desc_with_name(node, state, sdfg, a_conn)
+            b = in_desc_with_name(node, state, sdfg, b_conn)
+            c = out_desc_with_name(node, state, sdfg, c_conn)
+            shape = tuple(c.shape)
+            call = HipCall("dmlhip_binary_" + _SFX[c.dtype],
+                           [I32(code), Ptr(a_conn), Ptr(b_conn), Ptr(c_conn), I32(len(shape)), I64Array(shape),
+                            I64Array(tuple(_bcast_strides(a, shape))), I64Array(tuple(_bcast_strides(b, shape))),
+                            Stream()])
+            return _tasklet(node, state, [call], bytes_moved=_nbytes(a, b, c), kind="elementwise")
+
+    _Binary.__name__ = "Hip" + op_name
+    _Binary.__doc__ = ("%s with NumPy broadcasting (pure_implementations.py:39-41,76-93): one vectorised kernel."
+                       % op_name)
+    return op_implementation(op=op_name, name=IMPL)(_Binary)
+
+
+HipAdd = _make_binary("Add", L.ADD)
+HipSub = _make_binary("Sub", L.SUB)
+HipMul = _make_binary("Mul", L.MUL)
+HipDiv = _make_binary("Div", L.DIV)
+HipPow = _make_binary("Pow", L.POW, "X", "Y", "Z")
+
+
+def _make_unary(op_name: str, code: int, in_conn: str, out_conn: str, doc: str):
+    class _Unary(ONNXForward):
+        @staticmethod
+        def forward_can_be_applied(node, state, sdfg) -> bool:
+            try:
+                x = in_desc_with_name(node, state, sdfg, in_conn)
+                y = out_desc_with_name(node, state, sdfg, out_conn)
+                return _float_ok(x, y) and _dense(x, y) and x.total_size == y.total_size
+            except Exception:
+                return False
+
+        @staticmethod
+        def forward(node, state, sdfg):
+            x = in_desc_with_name(node, state, sdfg, in_conn)
+            call = HipCall("dmlhip_unary_" + _SFX[x.dtype],
+                           [I32(code), Ptr(in_conn), Ptr(out_conn), I64(x.total_size), F32(0.0), Stream()])
+            return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="elementwise")
+
+    _Unary.__name__ = "Hip" + op_name
+    _Unary.__doc__ = doc
+    return op_implementation(op=op_name, name=IMPL)(_Unary)
+
+
+HipSqrt = _make_unary("Sqrt", L.SQRT, "X", "Y", "Sqrt (pure_implementations.py:34-36).")
+HipRelu = _make_unary("Relu", L.RELU, "X", "Y", "Relu (pure_implementations.py:556-560).")
+HipSigmoid = _make_unary("Sigmoid", L.SIGMOID, "X", "Y", "Sigmoid (pure_implementations.py:741-743).")
+HipReciprocal = _make_unary("Reciprocal", L.RECIPROCAL, "X", "Y", "Reciprocal (pure_implementations.py:283-286).")
+HipErf = _make_unary("Erf", L.ERF, "input", "output", "Erf (pure_implementations.py:106-108).")
+HipExp = _make_unary("Exp", L.EXP, "input", "output", "Exp (pure_implementations.py:29-31).")
+HipLog = _make_unary("Log", L.LOG, "input", "output", "Log (pure_implementations.py:24-26).")
+HipTanh = _make_unary("Tanh", L.TANH, "input", "output", "Tanh (pure_implementations.py:289-291).")
+HipIdentity = _make_unary("Identity", L.IDENTITY, "input", "output", "Identity (pure_implementations.py:255-257).")
+HipGelu = _make_unary("Gelu", L.GELU, "X", "Y",
+                      "The exporter's Div, Erf, Add, Mul, Mul chain (pure_implementations.py:91-93,106-108,76-78,"
+                      "86-88) fused: exact-erf GELU.")
+HipSwish = _make_unary("Swish", L.SWISH, "X", "Y", "Mul(x, Sigmoid(x)) (pure_implementations.py:86-88,741-743) fused.")
+
+
+def _make_unary_grad(op_name: str, code: int, doc: str):
+    class _UnaryGrad(ONNXForward):
+        @staticmethod
+        def forward_can_be_applied(node, state, sdfg) -> bool:
+            try:
+                ins, outs = _descs(node, state, sdfg)
+                x, dy, dx = ins["X"], ins["dY"], outs["dX"]
+                return _float_ok(x, dy, dx) and _dense(x, dy, dx) and x.shape == dy.shape == dx.shape
+            except Exception:
+                return False
+
+        @staticmethod
+        def forward(node, state, sdfg):
+            x = in_desc_with_name(node, state, sdfg, "X")
+            call = HipCall("dmlhip_unary_backward_" + _SFX[x.dtype],
+                           [I32(code), Ptr("X"), Ptr("dY"), Ptr("dX"), I64(x.total_size), F32(0.0), Stream()])
+            return _tasklet(node, state, [call], bytes_moved=3 * _nbytes(x), kind="elementwise_backward")
+
+    _UnaryGrad.__name__ = "Hip" + op_name
+    _UnaryGrad.__doc__ = doc
+    return op_implementation(op=op_name, name=IMPL)(_UnaryGrad)
+
+
+_GRAD_DOC = ("dX = dY * f'(X): the tasklet the SymPy reversal of backward_pass_generator.py:1284-1421 derives for "
+             "this map, as one kernel.")
+HipGeluGrad = _make_unary_grad("GeluGrad", L.GELU, _GRAD_DOC)
+HipSwishGrad = _make_unary_grad("SwishGrad", L.SWISH, _GRAD_DOC)
+HipSigmoidGrad = _make_unary_grad("SigmoidGrad", L.SIGMOID, _GRAD_DOC)
+HipReluGrad = _make_unary_grad("ReluGrad", L.RELU, _GRAD_DOC)
+HipTanhGrad = _make_unary_grad("TanhGrad", L.TANH, _GRAD_DOC)
+
+
+@op_implementation(op="BiasGelu", name=IMPL)
+class HipBiasGelu(ONNXForward):
+    """Bias ONNXAdd followed by the GELU chain, one kernel."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            a, b, c = ins["A"], ins["B"], outs["C"]
+            return (_float_ok(a, b, c) and _dense(a, b, c) and a.shape == c.shape and len(a.shape) >= 1
+                    and b.total_size == a.shape[-1] and b.shape[-1] == a.shape[-1])
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        a = in_desc_with_name(node, state, sdfg, "A")
+        rows, cols = _prod(a.shape[:-1]), a.shape[-1]
+        call = HipCall("dmlhip_bias_gelu_" + _SFX[a.dtype],
+                       [Ptr("A"), Ptr("B"), Ptr("C"), Null(), I64(rows), I64(cols), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(a), kind="elementwise")
+
+
+@op_implementation(op="Sum", name=IMPL)
+class HipSum(ONNXForward):
+    """PureSum (pure_implementations.py:584-646): all inputs have the output's shape."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins = [sdfg.arrays[e.data.data] for e in node.iter_inputs_in_onnx_order(state)]
+            out = out_desc_with_name(node, state, sdfg, "sum")
+            return (_float_ok(out, *ins) and _dense(out, *ins) and all(d.shape == out.shape for d in ins)
+                    and len(ins) >= 1)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        conns = [e.dst_conn for e in node.iter_inputs_in_onnx_order(state)]
+        out = out_desc_with_name(node, state, sdfg, "sum")
+        calls, first, i = [], True, 0
+        while i < len(conns):
+            chunk = conns[i:i + (8 if first else 7)]
+            ptrs = ([] if first else ["sum"]) + chunk
+            calls.append(HipCall("dmlhip_sum_" + _SFX[out.dtype],
+                                 [PtrArray(tuple(ptrs)), I32(len(ptrs)), Ptr("sum"), I64(out.total_size), Stream()]))
+            i += len(chunk)
+            first = False
+        return _tasklet(node, state, calls, bytes_moved=(len(conns) + 1) * _nbytes(out), kind="elementwise")
+
+
+@op_implementation(op="Cast", name=IMPL)
+class HipCast(ONNXForward):
+    """Cast between fp16 and fp32 (pure_implementations.py:329-377)."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            x = in_desc_with_name(node, state, sdfg, "input")
+            y = out_desc_with_name(node, state, sdfg, "output")
+            return (x.dtype in FLOAT_DTYPES and y.dtype in FLOAT_DTYPES and _dense(x, y) and x.shape == y.shape)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "input")
+        y = out_desc_with_name(node, state, sdfg, "output")
+        call = HipCall("dmlhip_cast", [I32(_CODE[x.dtype]), I32(_CODE[y.dtype]), Ptr("input"), Ptr("output"),
+                                       I64(x.total_size), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=_nbytes(x, y), kind="elementwise")
+
+
+# ----------------------------------------------------------------------------- reductions
+def _reduce_geometry(shape, axes):
+    nd = len(shape)
+    axes = sorted(set(range(nd) if axes is None else [a % nd for a in axes]))
+    if not axes or axes != list(range(axes[0], axes[-1] + 1)):
+        return None
+    return _prod(shape[:axes[0]]), _prod(shape[axes[0]:axes[-1] + 1]), _prod(shape[axes[-1] + 1:]), axes
+
+
+def _make_reduce(op_name: str, code: int, doc: str):
+    class _Reduce(ONNXForward):
+        @staticmethod
+        def forward_can_be_applied(node, state, sdfg) -> bool:
+            try:
+                x = in_desc_with_name(node, state, sdfg, "data")
+                y = out_desc_with_name(node, state, sdfg, "reduced")
+                geo = _reduce_geometry(x.shape, node.axes)
+                if geo is None or not (x.dtype in FLOAT_DTYPES and y.dtype in FLOAT_DTYPES and _dense(x, y)):
+                    return False
+                outer, r, inner, _ = geo
+                if inner > 1 and outer > 65535:
+                    return False
+                if r == 0 and code != L.RSUM:
+                    return False
+                return y.total_size == outer * inner
+            except Exception:
+                return False
+
+        @staticmethod
+        def forward(node, state, sdfg):
+            x = in_desc_with_name(node, state, sdfg, "data")
+            y = out_desc_with_name(node, state, sdfg, "reduced")
+            outer, r, inner, _ = _reduce_geometry(x.shape, node.axes)
+            ws = L.load().dmlhip_reduce_workspace_bytes(outer, r, inner)
+            call = HipCall("dmlhip_reduce_" + _SFX[x.dtype],
+                           [I32(code), Ptr("data"), Ptr("reduced"), I32(_CODE[y.dtype]), I64(outer), I64(r), I64(inner),
+                            Workspace(), WorkspaceBytes(), Stream()])
+            return _tasklet(node, state, [call], workspace_bytes=ws, bytes_moved=_nbytes(x, y), kind="reduce")
+
+    _Reduce.__name__ = "Hip" + op_name
+    _Reduce.__doc__ = doc
+    return op_implementation(op=op_name, name=IMPL)(_Reduce)
+
+
+HipReduceSum = _make_reduce("ReduceSum", L.RSUM, "ReduceSum (pure_implementations.py:294-296); adjacent axes.")
+HipReduceMax = _make_reduce("ReduceMax", L.RMAX, "ReduceMax (pure_implementations.py:299-301); adjacent axes.")
+HipReduceMin = _make_reduce("ReduceMin", L.RMIN, "ReduceMin (pure_implementations.py:304-306); adjacent axes.")
+HipReduceMean = _make_reduce("ReduceMean", L.RMEAN, "ReduceMean (pure_implementations.py:101-103); adjacent axes.")
+
+
+@op_implementation(op="GlobalAveragePool", name=IMPL)
+class HipGlobalAveragePool(ONNXForward):
+    """GlobalAveragePool "pure" (img_op_implementations.py:415-417): mean over H and W."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            x = in_desc_with_name(node, state, sdfg, "X")
+            y = out_desc_with_name(node, state, sdfg, "Y")
+            return (_float_ok(x, y) and _dense(x, y) and len(x.shape) == 4
+                    and y.total_size == x.shape[0] * x.shape[1] and x.shape[2] * x.shape[3] > 0)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "X")
+        call = HipCall("dmlhip_reduce_" + _SFX[x.dtype],
+                       [I32(L.RMEAN), Ptr("X"), Ptr("Y"), I32(_CODE[x.dtype]), I64(x.shape[0] * x.shape[1]),
+                        I64(x.shape[2] * x.shape[3]), I64(1), Null(), USize(0), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=_nbytes(x), kind="reduce")
+
+
+# ----------------------------------------------------------------------------- data movement
+@op_implementation(op="Transpose", name=IMPL)
+class HipTranspose(ONNXForward):
+    """Transpose (pure_implementations.py:322-326,746-778)."""
+    @staticmethod
+    def _perm(node, nd):
+        return list(reversed(range(nd))) if node.perm is None else [p % nd for p in node.perm]
+
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            x = in_desc_with_name(node, state, sdfg, "data")
+            y = out_desc_with_name(node, state, sdfg, "transposed")
+            nd = len(x.shape)
+            perm = HipTranspose._perm(node, nd)
+            return (_float_ok(x, y) and _dense(x, y) and nd <= L.MAX_DIMS and sorted(perm) == list(range(nd))
+                    and tuple(x.shape[p] for p in perm) == tuple(y.shape))
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "data")
+        perm = HipTranspose._perm(node, len(x.shape))
+        call = HipCall("dmlhip_transpose_" + _SFX[x.dtype],
+                       [Ptr("data"), Ptr("transposed"), I32(len(perm)), I64Array(tuple(x.shape)), I64Array(tuple(perm)),
+                        Stream()])
+        return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="transpose")
+
+
+@op_implementation(op="Reshape", name=IMPL)
+class HipReshape(ONNXForward):
+    """Reshape (pure_implementations.py:571-573): a dense copy into the output descriptor."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            x = in_desc_with_name(node, state, sdfg, "data")
+            y = out_desc_with_name(node, state, sdfg, "reshaped")
+            return _float_ok(x, y) and _dense(x, y) and x.total_size == y.total_size
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "data")
+        call = HipCall("dmlhip_unary_" + _SFX[x.dtype],
+                       [I32(L.IDENTITY), Ptr("data"), Ptr("reshaped"), I64(x.total_size), F32(0.0), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="elementwise")
+
+
+# ----------------------------------------------------------------------------- convolution
+def _conv_struct(node, x: Array, w: Array, act=L.ACT_NONE) -> Optional[L.Conv2dDesc]:
+    """Attribute handling of CudnnConvolution (cudnn_implementations.py:148-275): 2-D, symmetric pads,
+    auto_pad NOTSET, any stride / dilation / group."""
+    if len(x.shape) != 4 or len(w.shape) != 4 or node.auto_pad != "NOTSET":
+        return None
+    strides = list(node.strides) if node.strides is not None else [1, 1]
+    dil = list(node.dilations) if node.dilations is not None else [1, 1]
+    pads = list(node.pads) if node.pads is not None else [0, 0, 0, 0]
+    if len(strides) != 2 or len(dil) != 2 or len(pads) != 4:
+        return None
+    if pads[0] != pads[2] or pads[1] != pads[3]:
+        return None
+    if node.kernel_shape is not None and list(node.kernel_shape) != list(w.shape[2:]):
+        return None
+    group = int(node.group)
+    if group < 1 or x.shape[1] != w.shape[1] * group or w.shape[0] % group:
+        return None
+    d = L.Conv2dDesc()
+    d.n, d.c, d.h, d.w = x.shape
+    d.m, d.kh, d.kw = w.shape[0], w.shape[2], w.shape[3]
+    d.stride_h, d.stride_w = strides
+    d.pad_h, d.pad_w = pads[0], pads[1]
+    d.dil_h, d.dil_w = dil
+    d.group = group
+    d.act = act
+    return d
+
+
+def _conv_out_hw(d: L.Conv2dDesc):
+    eh = (d.kh - 1) * d.dil_h + 1
+    ew = (d.kw - 1) * d.dil_w + 1
+    oh = (d.h + 2 * d.pad_h - eh) // d.stride_h + 1 if d.h + 2 * d.pad_h >= eh else 0
+    ow = (d.w + 2 * d.pad_w - ew) // d.stride_w + 1 if d.w + 2 * d.pad_w >= ew else 0
+    return oh, ow
+
+
+@op_implementation(op="Conv", name=IMPL)
+class HipConv(ONNXForward):
+    """ONNX Conv. PureConv2D (img_op_implementations.py:164-330) covers stride 1 / no pad / group 1 only
+    and the reference otherwise needs cuDNN or ONNX Runtime; this covers strides, symmetric pads,
+    dilations and groups: 1x1 as an MFMA GEMM, depthwise from LDS-staged rows, the rest directly.
+    A private ``_activation`` attribute set by the fusion pass folds a following Swish / Sigmoid in."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, w, y = ins["X"], ins["W"], outs["Y"]
+            if not (_float_ok(x, w, y) and _dense(x, w, y)):
+                return False
+            if "B" in ins and not (ins["B"].dtype == x.dtype and ins["B"].is_contiguous()
+                                   and ins["B"].total_size == w.shape[0]):
+                return False
+            d = _conv_struct(node, x, w)
+            if d is None:
+                return False
+            oh, ow = _conv_out_hw(d)
+            return tuple(y.shape) == (x.shape[0], w.shape[0], oh, ow)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        x, w, y = ins["X"], ins["W"], outs["Y"]
+        d = _conv_struct(node, x, w, _ACT[getattr(node, "_activation", "none")])
+        call = HipCall("dmlhip_conv2d_" + _SFX[x.dtype],
+                       [Struct(d, "dmlhip_conv2d_desc"), Ptr("X"), Ptr("W"), _opt(node, state, "B"), Ptr("Y"), Stream()])
+        flops = 2 * y.total_size * (w.shape[1] * w.shape[2] * w.shape[3])
+        return _tasklet(node, state, [call], flops=flops, bytes_moved=_nbytes(x, w, y), kind="conv")
+
+
+@op_implementation(op="ConvGrad", name=IMPL)
+class HipConvGrad(ONNXForward):
+    """cudnnConvolutionBackwardData / BackwardFilter / BackwardBias
+    (autodiff/implementations/onnx_ops.py:663-703) and the ATen depthwise backward (:1201-1231); fp32."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, w, dy = ins["X"], ins["W"], ins["dY"]
+            if x.dtype != torch.float32 or not (_float_ok(x, w, dy) and _dense(x, w, dy)):
+                return False
+            d = _conv_struct(node, x, w)
+            if d is None:
+                return False
+            oh, ow = _conv_out_hw(d)
+            if tuple(dy.shape) != (x.shape[0], w.shape[0], oh, ow):
+                return False
+            for name, ref in (("dX", x), ("dW", w)):
+                if name in outs and not (outs[name].shape == ref.shape and outs[name].is_contiguous()
+                                         and outs[name].dtype == torch.float32):
+                    return False
+            if "dB" in outs and not (outs["dB"].total_size == w.shape[0] and outs["dB"].dtype == torch.float32):
+                return False
+            return x.shape[0] <= 65535
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        x, w, dy = ins["X"], ins["W"], ins["dY"]
+        d = _conv_struct(node, x, w)
+        lib = L.load()
+        calls, ws = [], 0
+        if "dX" in outs:
+            calls.append(HipCall("dmlhip_conv2d_backward_data_f32",
+                                 [Struct(d, "dmlhip_conv2d_desc"), Ptr("dY"), Ptr("W"), Ptr("dX"), Stream()]))
+        if "dW" in outs:
+            import ctypes
+            ws = max(ws, lib.dmlhip_conv2d_backward_weight_workspace_bytes(ctypes.byref(d)))
+            calls.append(HipCall("dmlhip_conv2d_backward_weight_f32",
+                                 [Struct(d, "dmlhip_conv2d_desc"), Ptr("X"), Ptr("dY"), Ptr("dW"), Workspace(),
+                                  WorkspaceBytes(), Stream()]))
+        if "dB" in outs:
+            # dB[m] = sum_{b, y, x} dY[b, m, y, x]: reduce the spatial dims into the head of the
+            # workspace, then the batch dim from there
+            n, m = dy.shape[0], dy.shape[1]
+            hw = dy.shape[2] * dy.shape[3]
+            part = (n * m * 4 + 255) // 256 * 256
+            ws = max(ws, part + lib.dmlhip_reduce_workspace_bytes(1, n, m))
+            calls.append(HipCall("dmlhip_reduce_f32", [I32(L.RSUM), Ptr("dY"), Workspace(), I32(L.F32), I64(n * m),
+                                                       I64(hw), I64(1), Null(), USize(0), Stream()]))
+            calls.append(HipCall("dmlhip_reduce_f32", [I32(L.RSUM), Workspace(), Ptr("dB"), I32(L.F32), I64(1), I64(n),
+                                                       I64(m), Workspace(part), WorkspaceBytes(part), Stream()]))
+        return _tasklet(node, state, calls, workspace_bytes=ws, bytes_moved=_nbytes(x, w, dy), kind="conv_backward")

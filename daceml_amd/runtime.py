@@ -1,0 +1,241 @@
+"""Expansion and execution of SDFGs made of ONNX library nodes.
+
+``expand_onnx_nodes`` is daceml.util.utils.expand_onnx_nodes (daceml/util/utils.py:156-203): every
+``ONNXOp`` is replaced by the result of its selected implementation. ``CompiledSDFG`` is the stand-in
+for DaCe's compiled SDFG plus DaCeML's ctypes dispatcher (daceml/torch/dispatchers/ctypes_module.py):
+transients are owned by the SDFG and allocated once, caller arrays are passed per call, every kernel
+is enqueued on the caller's current stream without synchronising (the ``nosync`` states of
+ctypes_module.py:210-211).
+
+Binding is done once: each launch becomes ``(ctypes function, tuple of ctypes arguments)``. Pointers of
+caller-owned arrays live in shared mutable ``c_void_p`` objects that are updated on every call, so the
+steady state is one ctypes call per kernel and no Python-side planning.
+"""
+import ctypes
+import logging
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from . import _lib as L
+from . import hip_tasklet as T
+from .onnx.nodes import ONNXOp
+from .sdfg import SDFG, AccessNode, Array, SDFGState
+
+log = logging.getLogger(__name__)
+
+_ITEM = {torch.float16: 2, torch.float32: 4, torch.float64: 8, torch.int64: 8, torch.int32: 4, torch.bool: 1}
+
+
+def expand_onnx_nodes(sdfg: SDFG, predicate=None) -> int:
+    """Expand all ONNX library nodes (recursively: an expansion may return nodes that are themselves
+    ONNX library nodes). Returns the number of expansions."""
+    count = 0
+    for state in sdfg.states():
+        changed = True
+        while changed:
+            changed = False
+            for node in state.nodes():
+                if isinstance(node, ONNXOp) and (predicate is None or predicate(node)):
+                    result = node.expand(sdfg, state)
+                    _replace_node(state, node, result)
+                    count += 1
+                    changed = True
+    return count
+
+
+def _replace_node(state: SDFGState, node, new):
+    for e in state.in_edges(node):
+        if e.dst_conn not in new.in_connectors:
+            raise ValueError("expansion of %r lacks input connector %r" % (node, e.dst_conn))
+    for e in state.out_edges(node):
+        if e.src_conn not in new.out_connectors:
+            raise ValueError("expansion of %r lacks output connector %r" % (node, e.src_conn))
+    state.add_node(new)
+    for e in state.edges():
+        if e.dst is node:
+            e.dst = new
+        if e.src is node:
+            e.src = new
+    state._nodes.remove(node)
+
+
+class _Launch:
+    __slots__ = ("fn", "args", "label", "symbol", "flops", "bytes_moved", "kind", "state")
+
+    def __init__(self, fn, args, label, symbol, flops, bytes_moved, kind, state):
+        self.fn, self.args, self.label, self.symbol = fn, args, label, symbol
+        self.flops, self.bytes_moved, self.kind, self.state = flops, bytes_moved, kind, state
+
+
+class CompiledSDFG:
+    """An expanded SDFG bound to device buffers; call it with the non-transient arrays by name."""
+    def __init__(self, sdfg: SDFG, device: Optional[torch.device] = None, expand: bool = True):
+        self.sdfg = sdfg
+        self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
+        if self.device.type != "cuda":
+            raise ValueError("the HIP implementations run on a GPU device; got %s" % self.device)
+        self.lib = L.load()
+        if expand:
+            expand_onnx_nodes(sdfg)
+        self._keep = []                       # ctypes objects that must outlive the launches
+        self._ptr: Dict[str, ctypes.c_void_p] = {}
+        self._derived = []                    # (c_void_p, base name, byte offset)
+        self._ptr_arrays = []                 # (ctypes array, [(slot, name)])
+        self._stream = ctypes.c_void_p(0)
+        self.buffers: Dict[str, torch.Tensor] = {}
+        self._allocate()
+        self._launches: List[_Launch] = []
+        ws = 0
+        for state in sdfg.states():
+            for node in state.topological_sort():
+                if isinstance(node, ONNXOp):
+                    raise RuntimeError("unexpanded library node %r" % node)
+                ws = max(ws, getattr(node, "workspace_bytes", 0))
+        self._ws_bytes = max(int(ws), 256)
+        self._workspace = torch.empty(self._ws_bytes, dtype=torch.uint8, device=self.device)
+        for state in sdfg.states():
+            for node in state.topological_sort():
+                self._bind_node(state, node)
+        self._refresh()
+
+    # -- memory ------------------------------------------------------------
+    def _allocate(self):
+        for name, desc in self.sdfg.arrays.items():
+            self._ptr[name] = ctypes.c_void_p(0)
+        for name, desc in self.sdfg.arrays.items():
+            if desc.view_of is not None:
+                self._derived.append((self._ptr[name], desc.view_of, desc.view_offset * _ITEM[desc.dtype]))
+            elif name in self.sdfg.constants:
+                t = self.sdfg.constants[name].to(device=self.device, dtype=desc.dtype).contiguous()
+                if tuple(t.shape) != desc.shape:
+                    raise ValueError("constant %r has shape %s, descriptor says %s" % (name, tuple(t.shape), desc.shape))
+                self.buffers[name] = t
+            elif desc.transient:
+                self.buffers[name] = torch.empty(desc.shape, dtype=desc.dtype, device=self.device)
+        for name, t in self.buffers.items():
+            self._ptr[name].value = t.data_ptr()
+
+    def _refresh(self):
+        for obj, base, off in self._derived:
+            obj.value = (self._ptr[base].value or 0) + off
+        for arr, slots in self._ptr_arrays:
+            for i, name in slots:
+                arr[i] = self._ptr[name].value
+
+    # -- binding -----------------------------------------------------------
+    def _bind_node(self, state: SDFGState, node):
+        calls = getattr(node, "calls", None)
+        if calls is None:
+            if isinstance(node, AccessNode):
+                return
+            raise RuntimeError("node %r has no HIP calls; only HipTasklet / ViewTasklet nodes can run" % node)
+        conn_to_array = {}
+        for e in state.in_edges(node):
+            conn_to_array[e.dst_conn] = e.data.data
+        for e in state.out_edges(node):
+            conn_to_array[e.src_conn] = e.data.data
+        for call in calls:
+            fn = getattr(self.lib, call.symbol)
+            args = []
+            for a in call.args:
+                if isinstance(a, T.Ptr):
+                    name = conn_to_array[a.conn]
+                    if a.offset:
+                        obj = ctypes.c_void_p(0)
+                        self._derived.append((obj, name, a.offset * _ITEM[self.sdfg.arrays[name].dtype]))
+                        args.append(obj)
+                    else:
+                        args.append(self._ptr[name])
+                elif isinstance(a, T.Null):
+                    args.append(ctypes.c_void_p(0))
+                elif isinstance(a, T.I64):
+                    args.append(ctypes.c_int64(a.value))
+                elif isinstance(a, T.I32):
+                    args.append(ctypes.c_int(a.value))
+                elif isinstance(a, T.F32):
+                    args.append(ctypes.c_float(a.value))
+                elif isinstance(a, T.USize):
+                    args.append(ctypes.c_size_t(a.value))
+                elif isinstance(a, T.I64Array):
+                    arr = (ctypes.c_int64 * max(len(a.values), 1))(*a.values)
+                    self._keep.append(arr)
+                    args.append(arr)
+                elif isinstance(a, T.PtrArray):
+                    arr = (ctypes.c_void_p * len(a.conns))()
+                    self._ptr_arrays.append((arr, [(i, conn_to_array[c]) for i, c in enumerate(a.conns)]))
+                    args.append(arr)
+                elif isinstance(a, T.Struct):
+                    self._keep.append(a.value)
+                    args.append(ctypes.byref(a.value))
+                elif isinstance(a, T.Workspace):
+                    args.append(ctypes.c_void_p(self._workspace.data_ptr() + a.offset))
+                elif isinstance(a, T.WorkspaceBytes):
+                    args.append(ctypes.c_size_t(self._ws_bytes - a.offset))
+                elif isinstance(a, T.Stream):
+                    args.append(self._stream)
+                else:
+                    raise TypeError("unknown HIP call argument %r" % (a, ))
+            # work is attributed to the node's first call only (later calls are follow-up passes)
+            first = call is calls[0]
+            self._launches.append(_Launch(fn, tuple(args), node.label, call.symbol, node.flops if first else 0,
+                                          node.bytes_moved if first else 0, node.kind, state.label))
+
+    # -- execution -----------------------------------------------------------
+    def _bind_arguments(self, kwargs: Dict[str, torch.Tensor]):
+        for name, desc in self.sdfg.arrays.items():
+            if desc.transient or name in self.sdfg.constants or desc.view_of is not None:
+                continue
+            if name not in kwargs:
+                raise TypeError("missing argument %r (arrays to pass: %s)" % (name, sorted(self.arglist())))
+            t = kwargs[name]
+            if not isinstance(t, torch.Tensor) or t.device != self.device:
+                raise ValueError("argument %r must be a tensor on %s" % (name, self.device))
+            if t.dtype != desc.dtype or tuple(t.shape) != desc.shape:
+                raise ValueError("argument %r: expected %s %s, got %s %s" % (name, desc.dtype, desc.shape, t.dtype,
+                                                                             tuple(t.shape)))
+            if tuple(t.stride()) != desc.strides and t.numel() > 1:
+                raise ValueError("argument %r must have strides %s (pass a contiguous tensor)" % (name, desc.strides))
+            self._ptr[name].value = t.data_ptr()
+        extra = set(kwargs) - set(self.sdfg.arrays)
+        if extra:
+            raise TypeError("unknown argument(s) %s" % sorted(extra))
+        self._refresh()
+
+    def arglist(self) -> Dict[str, Array]:
+        return {k: v for k, v in self.sdfg.arrays.items()
+                if not v.transient and k not in self.sdfg.constants and v.view_of is None}
+
+    def __call__(self, **kwargs):
+        self._bind_arguments(kwargs)
+        self.launch()
+
+    def launch(self, states: Optional[Sequence[str]] = None):
+        """Enqueue every kernel (of the named states) on the current stream, with the pointers of the
+        last binding."""
+        self._stream.value = torch.cuda.current_stream(self.device).cuda_stream
+        for l in self._launches:
+            if states is not None and l.state not in states:
+                continue
+            status = l.fn(*l.args)
+            if status != 0:
+                raise L.HipKernelError(status, "%s (%s): %s" % (l.label, l.symbol, L.last_error()))
+
+    def launch_timed(self):
+        """Like launch(), with a HIP event pair around every kernel; returns [(launch, ms)]."""
+        self._stream.value = torch.cuda.current_stream(self.device).cuda_stream
+        events = []
+        for l in self._launches:
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            status = l.fn(*l.args)
+            e.record()
+            if status != 0:
+                raise L.HipKernelError(status, "%s (%s): %s" % (l.label, l.symbol, L.last_error()))
+            events.append((l, s, e))
+        torch.cuda.synchronize(self.device)
+        return [(l, s.elapsed_time(e)) for l, s, e in events]
+
+    @property
+    def launches(self) -> Sequence[_Launch]:
+        return tuple(self._launches)

@@ -1,0 +1,557 @@
+"""Graph rewrites that turn the exporter's decomposed opset-12 graph into the nodes the HIP kernels
+implement in one launch.
+
+Modelled on the reference's pattern-replacement machinery: ``ReplacementTransformation``
+(daceml/transformation/replacement.py:67-181) for the chain -> node rewrites,
+``HorizontalEinsumFusion`` (daceml/transformation/einsum_fusion.py:102-151) for folding Transposes
+into contractions, ``PadConvFusion`` (daceml/transformation/pad_conv_fusion.py:80-97) for folding a
+neighbour into a Conv. Every rewrite keeps the graph's results equal to the composition of the pure
+expansions it replaces (that composition is the oracle of the fused kernels).
+
+    fuse_gelu                Div, Erf, Add, Mul, Mul                      -> Gelu
+    fuse_layernorm           ReduceMean, Sub, Pow, ReduceMean, Add, Sqrt,
+                             Div, Mul, Add                                -> LayerNormalization
+    fuse_swish               Sigmoid, Mul                                 -> Swish
+    lower_matmul             MatMul                                       -> Einsum (PureMatMul's lowering)
+    fold_views               Transpose / Reshape around an Einsum         -> operand letters / dense views
+    fuse_epilogues           Einsum, [Div|Mul const], [Add bias], [Gelu],
+                             [Add residual]                               -> FusedEinsum
+    fuse_skip_layernorm      Add, LayerNormalization                      -> SkipLayerNormalization
+    fuse_conv_activation     Conv, Swish | Sigmoid | Relu                 -> Conv(_activation)
+"""
+import math
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from .. import contraction as C
+from .. import onnx as donnx
+from ..onnx.nodes import ONNXOp
+from ..sdfg import SDFG, AccessNode, Array, Edge, SDFGState, contiguous_strides
+
+
+# ----------------------------------------------------------------------------- graph helpers
+def _producer(state: SDFGState, array: str) -> Optional[Tuple[ONNXOp, str]]:
+    for e in state.edges():
+        if e.data.data == array and isinstance(e.dst, AccessNode) and not isinstance(e.src, AccessNode):
+            return e.src, e.src_conn
+    return None
+
+
+def _consumers(state: SDFGState, array: str) -> List[Tuple[ONNXOp, str]]:
+    return [(e.dst, e.dst_conn) for e in state.edges()
+            if e.data.data == array and isinstance(e.src, AccessNode) and not isinstance(e.dst, AccessNode)]
+
+
+def _in_array(state: SDFGState, node, conn: str) -> Optional[str]:
+    for e in state.in_edges_by_connector(node, conn):
+        return e.data.data
+    return None
+
+
+def _out_array(state: SDFGState, node, conn: str) -> Optional[str]:
+    for e in state.out_edges_by_connector(node, conn):
+        return e.data.data
+    return None
+
+
+def _is_op(node, name: str) -> bool:
+    return isinstance(node, ONNXOp) and node.schema.name == name
+
+
+def _internal(sdfg: SDFG, state: SDFGState, array: str, n_consumers: int = 1) -> bool:
+    """A transient that only the matched pattern reads."""
+    d = sdfg.arrays[array]
+    return d.transient and d.view_of is None and len(_consumers(state, array)) == n_consumers
+
+
+def _scalar_const(sdfg: SDFG, array: Optional[str]) -> Optional[float]:
+    if array is None or array not in sdfg.constants or sdfg.arrays[array].total_size != 1:
+        return None
+    if array in sdfg.constants_exact:
+        return sdfg.constants_exact[array]
+    return float(sdfg.constants[array].reshape(-1)[0])
+
+
+def _remove_node(state: SDFGState, node):
+    """Remove a library node together with access nodes that are left without edges."""
+    neighbours = [e.src for e in state.in_edges(node)] + [e.dst for e in state.out_edges(node)]
+    state.remove_node(node)
+    for n in neighbours:
+        if isinstance(n, AccessNode) and not state.in_edges(n) and not state.out_edges(n) and n in state.nodes():
+            state.remove_node(n)
+
+
+def _drop_unused_arrays(sdfg: SDFG):
+    used = set()
+    for st in sdfg.states():
+        for e in st.edges():
+            used.add(e.data.data)
+    # keep bases of views that are in use
+    for name in list(used):
+        d = sdfg.arrays.get(name)
+        while d is not None and d.view_of is not None:
+            used.add(d.view_of)
+            d = sdfg.arrays.get(d.view_of)
+    for name in list(sdfg.arrays):
+        if name not in used and sdfg.arrays[name].transient:
+            del sdfg.arrays[name]
+            sdfg.constants.pop(name, None)
+    for name in list(sdfg.constants):
+        if name not in used:
+            sdfg.constants.pop(name)
+            sdfg.constants_exact.pop(name, None)
+            sdfg.arrays.pop(name, None)
+
+
+def _add_node(sdfg: SDFG, state: SDFGState, op: str, label: str, inputs: Dict[str, str], outputs: Dict[str, str],
+              **attrs) -> ONNXOp:
+    node = donnx.get_onnx_node(op)(label, **attrs)
+    state.add_node(node)
+    for conn, arr in inputs.items():
+        if conn not in node.in_connectors:
+            node.add_in_connector(conn)
+        state.add_edge(state.add_read(arr), None, node, conn, sdfg.make_array_memlet(arr))
+    for conn, arr in outputs.items():
+        if conn not in node.out_connectors:
+            node.add_out_connector(conn)
+        state.add_edge(node, conn, state.add_write(arr), None, sdfg.make_array_memlet(arr))
+    return node
+
+
+def _binary_operands(state, node) -> Tuple[str, str]:
+    return _in_array(state, node, "A"), _in_array(state, node, "B")
+
+
+# ----------------------------------------------------------------------------- GELU
+def fuse_gelu(sdfg: SDFG) -> int:
+    """x -> Div(sqrt 2) -> Erf -> Add(1) -> Mul(x, .) -> Mul(0.5)  ==>  Gelu(x)."""
+    count = 0
+    for state in sdfg.states():
+        for erf in [n for n in state.nodes() if _is_op(n, "Erf")]:
+            d_arr = _in_array(state, erf, "input")
+            prod = _producer(state, d_arr)
+            if prod is None or not _is_op(prod[0], "Div") or not _internal(sdfg, state, d_arr):
+                continue
+            div = prod[0]
+            x, c = _binary_operands(state, div)
+            cv = _scalar_const(sdfg, c)
+            if cv is None or abs(cv - math.sqrt(2.0)) > 1e-3:
+                continue
+            e_arr = _out_array(state, erf, "output")
+            cons = _consumers(state, e_arr)
+            if len(cons) != 1 or not _is_op(cons[0][0], "Add") or not _internal(sdfg, state, e_arr):
+                continue
+            add = cons[0][0]
+            other = [a for a in _binary_operands(state, add) if a != e_arr]
+            if len(other) != 1 or _scalar_const(sdfg, other[0]) != 1.0:
+                continue
+            a_arr = _out_array(state, add, "C")
+            cons = _consumers(state, a_arr)
+            if len(cons) != 1 or not _is_op(cons[0][0], "Mul") or not _internal(sdfg, state, a_arr):
+                continue
+            mulx = cons[0][0]
+            if set(_binary_operands(state, mulx)) != {x, a_arr}:
+                continue
+            m_arr = _out_array(state, mulx, "C")
+            cons = _consumers(state, m_arr)
+            if len(cons) != 1 or not _is_op(cons[0][0], "Mul") or not _internal(sdfg, state, m_arr):
+                continue
+            mulh = cons[0][0]
+            other = [a for a in _binary_operands(state, mulh) if a != m_arr]
+            if len(other) != 1 or _scalar_const(sdfg, other[0]) != 0.5:
+                continue
+            out = _out_array(state, mulh, "C")
+            for n in (div, erf, add, mulx, mulh):
+                _remove_node(state, n)
+            _add_node(sdfg, state, "Gelu", erf.label.replace("_erf", "") + "_fused", {"X": x}, {"Y": out})
+            count += 1
+    _drop_unused_arrays(sdfg)
+    return count
+
+
+# ----------------------------------------------------------------------------- LayerNorm
+def fuse_layernorm(sdfg: SDFG) -> int:
+    count = 0
+    for state in sdfg.states():
+        for sqrt in [n for n in state.nodes() if _is_op(n, "Sqrt")]:
+            m = _match_layernorm(sdfg, state, sqrt)
+            if m is None:
+                continue
+            x, gamma, beta, eps, out, nodes = m
+            for n in nodes:
+                _remove_node(state, n)
+            _add_node(sdfg, state, "LayerNormalization", sqrt.label.replace("_sqrt", "") + "_fused",
+                      {"X": x, "Scale": gamma, "B": beta}, {"Y": out}, axis=-1, epsilon=eps)
+            count += 1
+    _drop_unused_arrays(sdfg)
+    return count
+
+
+def _match_layernorm(sdfg, state, sqrt):
+    def single(arr, op):
+        p = _producer(state, arr)
+        return p[0] if p is not None and _is_op(p[0], op) else None
+
+    ve = _in_array(state, sqrt, "X")
+    addeps = single(ve, "Add")
+    if addeps is None or not _internal(sdfg, state, ve):
+        return None
+    ops = _binary_operands(state, addeps)
+    eps_arr = [a for a in ops if _scalar_const(sdfg, a) is not None]
+    var_arr = [a for a in ops if a not in eps_arr]
+    if len(eps_arr) != 1 or len(var_arr) != 1 or not _internal(sdfg, state, var_arr[0]):
+        return None
+    eps = _scalar_const(sdfg, eps_arr[0])
+    var = single(var_arr[0], "ReduceMean")
+    if var is None:
+        return None
+    sq_arr = _in_array(state, var, "data")
+    powr = single(sq_arr, "Pow")
+    if powr is None or not _internal(sdfg, state, sq_arr) or _scalar_const(sdfg, _in_array(state, powr, "Y")) != 2.0:
+        return None
+    cen_arr = _in_array(state, powr, "X")
+    sub = single(cen_arr, "Sub")
+    if sub is None or not _internal(sdfg, state, cen_arr, 2):
+        return None
+    x, mean_arr = _binary_operands(state, sub)
+    mean = single(mean_arr, "ReduceMean")
+    if mean is None or _in_array(state, mean, "data") != x or not _internal(sdfg, state, mean_arr):
+        return None
+    nd = len(sdfg.arrays[x].shape)
+    for r in (mean, var):
+        axes = [a % nd for a in (r.axes or [])]
+        if axes != [nd - 1] or not r.keepdims:
+            return None
+    std_arr = _out_array(state, sqrt, "Y")
+    cons = _consumers(state, std_arr)
+    if len(cons) != 1 or not _is_op(cons[0][0], "Div") or not _internal(sdfg, state, std_arr):
+        return None
+    div = cons[0][0]
+    if _binary_operands(state, div) != (cen_arr, std_arr):
+        return None
+    nrm = _out_array(state, div, "C")
+    cons = _consumers(state, nrm)
+    if len(cons) != 1 or not _is_op(cons[0][0], "Mul") or not _internal(sdfg, state, nrm):
+        return None
+    mul = cons[0][0]
+    gamma = [a for a in _binary_operands(state, mul) if a != nrm]
+    sc = _out_array(state, mul, "C")
+    cons = _consumers(state, sc)
+    if len(gamma) != 1 or len(cons) != 1 or not _is_op(cons[0][0], "Add") or not _internal(sdfg, state, sc):
+        return None
+    add = cons[0][0]
+    beta = [a for a in _binary_operands(state, add) if a != sc]
+    h = sdfg.arrays[x].shape[-1]
+    if len(beta) != 1 or sdfg.arrays[gamma[0]].total_size != h or sdfg.arrays[beta[0]].total_size != h:
+        return None
+    out = _out_array(state, add, "C")
+    return x, gamma[0], beta[0], eps, out, [mean, sub, powr, var, addeps, sqrt, div, mul, add]
+
+
+# ----------------------------------------------------------------------------- Swish
+def fuse_swish(sdfg: SDFG) -> int:
+    count = 0
+    for state in sdfg.states():
+        for sig in [n for n in state.nodes() if _is_op(n, "Sigmoid")]:
+            x = _in_array(state, sig, "X")
+            s = _out_array(state, sig, "Y")
+            cons = _consumers(state, s)
+            if len(cons) != 1 or not _is_op(cons[0][0], "Mul") or not _internal(sdfg, state, s):
+                continue
+            mul = cons[0][0]
+            if set(_binary_operands(state, mul)) != {x, s} or sdfg.arrays[x].shape != sdfg.arrays[s].shape:
+                continue
+            out = _out_array(state, mul, "C")
+            _remove_node(state, sig)
+            _remove_node(state, mul)
+            _add_node(sdfg, state, "Swish", sig.label.replace("_sigmoid", "") + "_fused", {"X": x}, {"Y": out})
+            count += 1
+    _drop_unused_arrays(sdfg)
+    return count
+
+
+def fuse_conv_activation(sdfg: SDFG) -> int:
+    """Conv followed only by Swish / Sigmoid / Relu: the activation moves into the conv kernel."""
+    names = {"Swish": "swish", "Sigmoid": "sigmoid", "Relu": "relu"}
+    count = 0
+    for state in sdfg.states():
+        for conv in [n for n in state.nodes() if _is_op(n, "Conv")]:
+            if getattr(conv, "_activation", "none") != "none":
+                continue
+            y = _out_array(state, conv, "Y")
+            cons = _consumers(state, y)
+            if len(cons) != 1 or not isinstance(cons[0][0], ONNXOp) or cons[0][0].schema.name not in names:
+                continue
+            if not _internal(sdfg, state, y):
+                continue
+            act = cons[0][0]
+            out = _out_array(state, act, "Y")
+            for e in state.out_edges(conv):
+                state.remove_edge(e)
+            _remove_node(state, act)
+            for n in [n for n in state.nodes() if isinstance(n, AccessNode) and n.data == y]:
+                if not state.in_edges(n) and not state.out_edges(n):
+                    state.remove_node(n)
+            state.add_edge(conv, "Y", state.add_write(out), None, sdfg.make_array_memlet(out))
+            conv._activation = names[act.schema.name]
+            count += 1
+    _drop_unused_arrays(sdfg)
+    return count
+
+
+# ----------------------------------------------------------------------------- contractions
+def lower_matmul(sdfg: SDFG) -> int:
+    """MatMul -> Einsum with the equation PureMatMul builds (pure_implementations.py:132-191)."""
+    count = 0
+    for state in sdfg.states():
+        for mm in [n for n in state.nodes() if _is_op(n, "MatMul")]:
+            a, b = _in_array(state, mm, "A"), _in_array(state, mm, "B")
+            y = _out_array(state, mm, "Y")
+            ra, rb = len(sdfg.arrays[a].shape), len(sdfg.arrays[b].shape)
+            if ra < 2 or rb < 2:
+                continue
+            eq = C.matmul_equation(ra, rb)
+            _remove_node(state, mm)
+            _add_node(sdfg, state, "Einsum", mm.label, {"Inputs__0": a, "Inputs__1": b}, {"Output": y}, equation=eq)
+            count += 1
+    return count
+
+
+def _einsum_terms(node) -> Tuple[List[str], str]:
+    ins, out = C.parse(node.equation)
+    return ins, out
+
+
+def _plannable(sdfg, eq: str, a: str, b: str) -> bool:
+    da, db = sdfg.arrays[a], sdfg.arrays[b]
+    try:
+        C.plan_contraction(eq, da.shape, da.strides, db.shape, db.strides)
+        return True
+    except (C.NotApplicable, ValueError):
+        return False
+
+
+def _reshape_to_view(sdfg: SDFG, state: SDFGState, reshape) -> bool:
+    """A Reshape of a dense array moves nothing: its output becomes a dense view of its input."""
+    src = _in_array(state, reshape, "data")
+    dst = _out_array(state, reshape, "reshaped")
+    ds, dd = sdfg.arrays[src], sdfg.arrays[dst]
+    if not ds.is_contiguous() or not dd.transient or ds.total_size != dd.total_size or ds.dtype != dd.dtype:
+        return False
+    base, off = src, 0
+    while sdfg.arrays[base].view_of is not None:
+        off += sdfg.arrays[base].view_offset
+        base = sdfg.arrays[base].view_of
+    dd.view_of, dd.view_offset = base, off
+    dd.strides = contiguous_strides(dd.shape)
+    _remove_node(state, reshape)
+    # consumers of the view must still be ordered after the producer of the base: keep that
+    # dependency visible by remembering the alias
+    sdfg.arrays[dst]._alias_source = src
+    return True
+
+
+def fold_views(sdfg: SDFG) -> int:
+    """Fold Transposes next to two-operand Einsums into the equation's letters, and Reshapes of dense
+    arrays into views, so that head split / merge and weight transposes cost no kernel and no HBM pass."""
+    count = 0
+    for state in sdfg.states():
+        changed = True
+        while changed:
+            changed = False
+            for es in [n for n in state.nodes() if _is_op(n, "Einsum") or _is_op(n, "FusedEinsum")]:
+                terms, out_t = _einsum_terms(es)
+                if len(terms) != 2:
+                    continue
+                arrays = [_in_array(state, es, "Inputs__0"), _in_array(state, es, "Inputs__1")]
+                # ---- operands
+                for i in (0, 1):
+                    prod = _producer(state, arrays[i])
+                    if prod is None:
+                        continue
+                    pnode = prod[0]
+                    if _is_op(pnode, "Transpose") and sdfg.arrays[arrays[i]].transient:
+                        src = _in_array(state, pnode, "data")
+                        nd = len(sdfg.arrays[src].shape)
+                        perm = list(reversed(range(nd))) if pnode.perm is None else [p % nd for p in pnode.perm]
+                        letters = [None] * nd
+                        for pos, p in enumerate(perm):
+                            letters[p] = terms[i][pos]
+                        new_terms = list(terms)
+                        new_terms[i] = "".join(letters)
+                        new_arrays = list(arrays)
+                        new_arrays[i] = src
+                        eq = "%s,%s->%s" % (new_terms[0], new_terms[1], out_t)
+                        if not _plannable(sdfg, eq, new_arrays[0], new_arrays[1]):
+                            continue
+                        edge = next(iter(state.in_edges_by_connector(es, "Inputs__%d" % i)))
+                        old_access = edge.src
+                        state.remove_edge(edge)
+                        state.add_edge(state.add_read(src), None, es, "Inputs__%d" % i, sdfg.make_array_memlet(src))
+                        if not state.in_edges(old_access) and not state.out_edges(old_access):
+                            state.remove_node(old_access)
+                        es.equation = eq
+                        if not _consumers(state, arrays[i]):
+                            _remove_node(state, pnode)
+                        count += 1
+                        changed = True
+                        break
+                    if _is_op(pnode, "Reshape") and _reshape_to_view(sdfg, state, pnode):
+                        count += 1
+                        changed = True
+                        break
+                if changed:
+                    break
+                # ---- result
+                y = _out_array(state, es, "Output")
+                cons = _consumers(state, y)
+                if len(cons) == 1 and _is_op(cons[0][0], "Transpose") and _internal(sdfg, state, y) \
+                        and _is_op(es, "Einsum"):
+                    tr = cons[0][0]
+                    nd = len(out_t)
+                    perm = list(reversed(range(nd))) if tr.perm is None else [p % nd for p in tr.perm]
+                    new_out = "".join(out_t[p] for p in perm)
+                    eq = "%s,%s->%s" % (terms[0], terms[1], new_out)
+                    if _plannable(sdfg, eq, arrays[0], arrays[1]):
+                        dst = _out_array(state, tr, "transposed")
+                        for e in state.out_edges(es):
+                            state.remove_edge(e)
+                        _remove_node(state, tr)
+                        for n in [n for n in state.nodes() if isinstance(n, AccessNode) and n.data == y]:
+                            if not state.in_edges(n) and not state.out_edges(n):
+                                state.remove_node(n)
+                        state.add_edge(es, "Output", state.add_write(dst), None, sdfg.make_array_memlet(dst))
+                        es.equation = eq
+                        count += 1
+                        changed = True
+                        break
+                if len(cons) == 1 and _is_op(cons[0][0], "Reshape") and _reshape_to_view(sdfg, state, cons[0][0]):
+                    count += 1
+                    changed = True
+                    break
+    _drop_unused_arrays(sdfg)
+    return count
+
+
+def fuse_epilogues(sdfg: SDFG, keep_preactivation: bool = False) -> int:
+    """Einsum -> [Div | Mul by a scalar constant] -> [Add bias over the last index] -> [Gelu] ->
+    [Add residual of the same shape]  ==>  one FusedEinsum. With ``keep_preactivation`` the value
+    before the activation stays available as the PreActivation output (training needs it)."""
+    count = 0
+    for state in sdfg.states():
+        for es in [n for n in state.nodes() if _is_op(n, "Einsum")]:
+            terms, out_t = _einsum_terms(es)
+            if len(terms) != 2:
+                continue
+            a, b = _in_array(state, es, "Inputs__0"), _in_array(state, es, "Inputs__1")
+            if not _plannable(sdfg, es.equation, a, b):
+                continue
+            cur = _out_array(state, es, "Output")
+            shape = sdfg.arrays[cur].shape
+            absorbed, alpha, bias, act, residual, pre = [], 1.0, None, "none", None, None
+
+            def sole_consumer(arr):
+                cons = _consumers(state, arr)
+                if len(cons) == 1 and _internal(sdfg, state, arr) and isinstance(cons[0][0], ONNXOp):
+                    return cons[0][0]
+                return None
+
+            nxt = sole_consumer(cur)
+            # scale
+            if nxt is not None and nxt.schema.name in ("Div", "Mul"):
+                x, c = _binary_operands(state, nxt)
+                if x != cur and nxt.schema.name == "Mul":
+                    x, c = c, x
+                cv = _scalar_const(sdfg, c)
+                if x == cur and cv is not None and cv != 0:
+                    alpha = 1.0 / cv if nxt.schema.name == "Div" else cv
+                    absorbed.append(nxt)
+                    cur = _out_array(state, nxt, "C")
+                    nxt = sole_consumer(cur)
+            # bias
+            if nxt is not None and nxt.schema.name == "Add":
+                other = [o for o in _binary_operands(state, nxt) if o != cur]
+                if len(other) == 1:
+                    od = sdfg.arrays[other[0]]
+                    if (od.total_size == shape[-1] and od.shape[-1] == shape[-1] and od.is_contiguous()
+                            and _producer(state, other[0]) is None):
+                        bias = other[0]
+                        absorbed.append(nxt)
+                        cur = _out_array(state, nxt, "C")
+                        nxt = sole_consumer(cur)
+            # activation
+            if nxt is not None and nxt.schema.name == "Gelu":
+                act = "gelu"
+                pre = cur
+                absorbed.append(nxt)
+                cur = _out_array(state, nxt, "Y")
+                nxt = sole_consumer(cur)
+            # residual
+            if nxt is not None and nxt.schema.name == "Add":
+                other = [o for o in _binary_operands(state, nxt) if o != cur]
+                if len(other) == 1 and sdfg.arrays[other[0]].shape == shape and sdfg.arrays[other[0]].is_contiguous() \
+                        and sdfg.arrays[other[0]].dtype == sdfg.arrays[cur].dtype:
+                    residual = other[0]
+                    absorbed.append(nxt)
+                    cur = _out_array(state, nxt, "C")
+            if not absorbed:
+                continue
+            for n in absorbed:
+                _remove_node(state, n)
+            _remove_node(state, es)
+            inputs = {"Inputs__0": a, "Inputs__1": b}
+            if bias:
+                inputs["Bias"] = bias
+            if residual:
+                inputs["Residual"] = residual
+            outputs = {"Output": cur}
+            if pre is not None and keep_preactivation:
+                outputs["PreActivation"] = pre
+            _add_node(sdfg, state, "FusedEinsum", es.label + "_fused", inputs, outputs, equation=es.equation,
+                      alpha=alpha, activation=act)
+            count += 1
+    _drop_unused_arrays(sdfg)
+    return count
+
+
+def fuse_skip_layernorm(sdfg: SDFG) -> int:
+    """Add(x, skip) -> LayerNormalization  ==>  SkipLayerNormalization (for residual Adds that did not
+    end up in a GEMM epilogue)."""
+    count = 0
+    for state in sdfg.states():
+        for ln in [n for n in state.nodes() if _is_op(n, "LayerNormalization")]:
+            x = _in_array(state, ln, "X")
+            prod = _producer(state, x)
+            if prod is None or not _is_op(prod[0], "Add") or not _internal(sdfg, state, x):
+                continue
+            add = prod[0]
+            p, q = _binary_operands(state, add)
+            if sdfg.arrays[p].shape != sdfg.arrays[q].shape or sdfg.arrays[p].shape != sdfg.arrays[x].shape:
+                continue
+            if _out_array(state, ln, "Mean") or _out_array(state, ln, "InvStdDev"):
+                continue
+            gamma, beta = _in_array(state, ln, "Scale"), _in_array(state, ln, "B")
+            out = _out_array(state, ln, "Y")
+            _remove_node(state, add)
+            _remove_node(state, ln)
+            _add_node(sdfg, state, "SkipLayerNormalization", ln.label.replace("_fused", "") + "_skip",
+                      {"input": p, "skip": q, "gamma": gamma, "beta": beta}, {"output": out}, epsilon=ln.epsilon)
+            count += 1
+    _drop_unused_arrays(sdfg)
+    return count
+
+
+def auto_optimize(sdfg: SDFG, training: bool = False) -> Dict[str, int]:
+    """The pass pipeline, in dependency order (cf. daceml.util.utils.auto_optimize,
+    daceml/util/utils.py:205-235). Returns how often each rewrite fired."""
+    stats = {}
+    stats["gelu"] = fuse_gelu(sdfg)
+    stats["layernorm"] = fuse_layernorm(sdfg)
+    stats["swish"] = fuse_swish(sdfg)
+    stats["conv_activation"] = fuse_conv_activation(sdfg)
+    stats["matmul_to_einsum"] = lower_matmul(sdfg)
+    stats["views"] = fold_views(sdfg)
+    stats["epilogues"] = fuse_epilogues(sdfg, keep_preactivation=training)
+    stats["skip_layernorm"] = fuse_skip_layernorm(sdfg)
+    return stats

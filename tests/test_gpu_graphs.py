@@ -1,0 +1,151 @@
+"""GPU parity of whole graphs run through the library-node registry, the fusion pass, the autodiff
+registry and the runtime: BERT encoder layer forward / backward and the MBConv block, against the NumPy
+oracle on the same seeded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bert_layer as OB
+from oracle import ops as O
+from tests.util import assert_close, dev, host, rng
+
+pytestmark = pytest.mark.gpu
+
+
+def _bert_inputs(b, s, h, ffn, dtype, seed=1234, bias_std=0.02):
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    p = OB.init_params(h, ffn, seed, np.float32, bias_std=bias_std)
+    r = rng(seed + 1)
+    p["ln1_g"] = r.uniform(0.5, 1.5, h).astype(np.float32)
+    p["ln2_g"] = r.uniform(0.5, 1.5, h).astype(np.float32)
+    p["ln1_b"] = (r.standard_normal(h) * 0.1).astype(np.float32)
+    p["ln2_b"] = (r.standard_normal(h) * 0.1).astype(np.float32)
+    x = r.standard_normal((b, s, h)).astype(np.float32)
+    p = {k: v.astype(npdt) for k, v in p.items()}
+    return x.astype(npdt), p
+
+
+def _compile(sdfg):
+    from daceml_amd.runtime import CompiledSDFG
+    return CompiledSDFG(sdfg)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("fused", [True, False])
+def test_bert_layer_forward(dtype, fused):
+    from daceml_amd import graphs
+    from daceml_amd.transformation import fusion
+    b, s, h, heads, ffn = 2, 128, 256, 4, 1024
+    x, p = _bert_inputs(b, s, h, ffn, dtype)
+    sdfg = graphs.bert_encoder_layer(b, s, h, heads, ffn, dtype, eps=1e-5)
+    if fused:
+        stats = fusion.auto_optimize(sdfg)
+        assert stats["layernorm"] == 2 and stats["gelu"] == 1 and stats["epilogues"] == 7
+        names = [n.schema.name for n in sdfg.states()[0].library_nodes()]
+        assert sorted(set(names)) == ["Einsum", "FusedEinsum", "LayerNormalization", "Softmax"]
+    prog = _compile(sdfg)
+    y = torch.empty((b, s, h), dtype=dtype, device="cuda")
+    prog(x=dev(x), y=y, **{k: dev(v) for k, v in p.items()})
+    want = OB.forward(x.astype(np.float64), {k: v.astype(np.float64) for k, v in p.items()}, heads, eps=1e-5)
+    if dtype == torch.float16:
+        assert_close(host(y), want, dtype, "bert layer forward fused=%s" % fused)
+    else:
+        # a chain of ~12 fp32 nodes with K up to 1024: rounding accumulates beyond one node's 1e-5 / 1e-6
+        assert_close(host(y), want, dtype, "bert layer forward fused=%s" % fused, rtol=1e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_bert_layer_backward(dtype):
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.transformation import fusion
+    b, s, h, heads, ffn = 2, 128, 256, 4, 1024
+    x, p = _bert_inputs(b, s, h, ffn, dtype)
+    dy = rng(77).standard_normal((b, s, h)).astype(x.dtype)
+    sdfg = graphs.bert_encoder_layer(b, s, h, heads, ffn, dtype, eps=1e-5)
+    fusion.auto_optimize(sdfg, training=True)
+    grads = add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + OB.PARAM_NAMES,
+                              grad_dtypes={n: torch.float32 for n in OB.PARAM_NAMES})
+    # the backward state contains only nodes with hand-written kernels
+    bnames = {n.schema.name for n in sdfg.states()[1].library_nodes()}
+    assert bnames == {"FusedEinsum", "SoftmaxGrad", "LayerNormalizationGrad", "GeluGrad", "ReduceSum", "Sum"}
+    prog = _compile(sdfg)
+    args = {"x": dev(x), "y": torch.empty((b, s, h), dtype=dtype, device="cuda"), "gradient_y": dev(dy)}
+    args.update({k: dev(v) for k, v in p.items()})
+    out = {"gradient_x": torch.empty((b, s, h), dtype=dtype, device="cuda")}
+    for n in OB.PARAM_NAMES:
+        out["gradient_" + n] = torch.empty(p[n].shape, dtype=torch.float32, device="cuda")
+    prog(**args, **out)
+    x64 = x.astype(np.float64)
+    p64 = {k: v.astype(np.float64) for k, v in p.items()}
+    _, saved = OB.forward(x64, p64, heads, eps=1e-5, keep=True)
+    want = OB.backward(x64, p64, heads, dy.astype(np.float64), saved, eps=1e-5)
+    assert grads["x"] == "gradient_x"
+    if dtype == torch.float16:
+        assert_close(host(out["gradient_x"]), want["x"], dtype, "dx")
+        for n in OB.PARAM_NAMES:
+            # fp32 master gradients of fp16 activations: relative to the gradient's scale
+            scale = float(np.abs(want[n]).max())
+            # (the key bias has an exactly zero gradient — softmax is shift invariant — so the bound
+            # needs an absolute floor at the fp16 noise level of the sums that cancel)
+            assert_close(host(out["gradient_" + n]), want[n], dtype, "d" + n, rtol=2e-2, atol=2e-2 * scale + 1e-3)
+    else:
+        assert_close(host(out["gradient_x"]), want["x"], dtype, "dx", rtol=1e-4, atol=2e-5)
+        for n in OB.PARAM_NAMES:
+            scale = float(np.abs(want[n]).max())
+            assert_close(host(out["gradient_" + n]), want[n], dtype, "d" + n, rtol=1e-4, atol=1e-5 * max(scale, 1.0))
+
+
+def test_mbconv_block_forward():
+    from daceml_amd import graphs
+    from daceml_amd.transformation import fusion
+    b, cin, hw, cout = 3, 16, 28, 24
+    r = rng(4)
+    sdfg = graphs.mbconv_block(b, cin, hw, expand=6, cout=cout, se_reduce=4, stride=2, dtype=torch.float32)
+    x = r.standard_normal((b, cin, hw, hw)).astype(np.float32)
+    params = {}
+    for name, desc in sdfg.arglist().items():
+        if name in ("x", "y"):
+            continue
+        if name.endswith("_w"):
+            fan_in = int(np.prod(desc.shape[1:]))
+            params[name] = (r.standard_normal(desc.shape) * np.sqrt(2.0 / fan_in)).astype(np.float32)
+        else:
+            params[name] = (r.standard_normal(desc.shape) * 0.1).astype(np.float32)
+    stats = fusion.auto_optimize(sdfg)
+    assert stats["swish"] == 3 and stats["conv_activation"] == 4
+    prog = _compile(sdfg)
+    oh = (hw + 2 - 3) // 2 + 1
+    y = torch.empty((b, cout, oh, oh), dtype=torch.float32, device="cuda")
+    prog(x=dev(x), y=y, **{k: dev(v) for k, v in params.items()})
+    # oracle: the unfused node sequence
+    f = {k: v.astype(np.float64) for k, v in params.items()}
+    t = O.swish(O.conv2d(x.astype(np.float64), f["expand_w"], f["expand_b"]))
+    t = O.swish(O.conv2d(t, f["dw_w"], f["dw_b"], strides=(2, 2), pads=(1, 1, 1, 1), group=cin * 6))
+    se = O.global_average_pool(t)
+    se = O.swish(O.conv2d(se, f["se1_w"], f["se1_b"]))
+    se = O.sigmoid(O.conv2d(se, f["se2_w"], f["se2_b"]))
+    want = O.conv2d(O.mul(t, se), f["proj_w"], f["proj_b"])
+    # the reference's own tolerance for this block is 1e-3 (tests/torch/test_efficientnet_block.py:50-54);
+    # five chained fp32 nodes hold 1e-5 relative with a slightly wider absolute floor
+    assert_close(host(y), want, torch.float32, "mbconv forward", rtol=1e-5, atol=5e-6)
+
+
+def test_selection_levels_and_refusal():
+    """node.implementation > class default > package default; an inapplicable node raises, it does not
+    fall back silently."""
+    import daceml_amd.onnx as donnx
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.sdfg import SDFG
+    sdfg = SDFG("t")
+    st = sdfg.add_state()
+    sdfg.add_array("a", (4, 8), torch.float16)
+    sdfg.add_array("b", (4, 8), torch.float16)
+    node = donnx.ONNXSoftmax("sm", axis=-1)
+    st.add_edge(st.add_read("a"), None, node, "input", sdfg.make_array_memlet("a"))
+    st.add_edge(node, "output", st.add_write("b"), None, sdfg.make_array_memlet("b"))
+    node.implementation = "does-not-exist"
+    with pytest.raises(donnx.NotApplicable):
+        expand_onnx_nodes(sdfg)
+    node.implementation = None
+    assert expand_onnx_nodes(sdfg) == 1
