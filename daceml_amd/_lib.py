@@ -77,6 +77,8 @@ SIGNATURES = {
     "dmlhip_transpose_f16": (c_int, [_P, _P, c_int, _I64P, _I64P, _P]),
     "dmlhip_transpose_f32": (c_int, [_P, _P, c_int, _I64P, _I64P, _P]),
     "dmlhip_gemm_f16": (c_int, [POINTER(GemmDesc), _P, _P, _P, _P, _P, _P, _P]),
+    "dmlhip_gemm_f16_workspace_bytes": (c_size_t, [POINTER(GemmDesc)]),
+    "dmlhip_gemm_f16_ws": (c_int, [POINTER(GemmDesc), _P, _P, _P, _P, _P, _P, _P, c_size_t, _P]),
     "dmlhip_gemm_f32": (c_int, [POINTER(GemmDesc), _P, _P, _P, _P, _P, _P, _P]),
     "dmlhip_conv2d_out_shape": (c_int, [POINTER(Conv2dDesc), _I64P, _I64P]),
     "dmlhip_conv2d_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, _P]),

@@ -92,6 +92,40 @@ __device__ __forceinline__ float block_reduce(float v, float* scratch) {
     return r;
 }
 
+// Second stage of the two-stage column reductions: out[c] = scale * Op over p < parts of
+// part[p*row_stride + c]. 64 columns per workgroup, 16 wavefronts striding over the partial rows with
+// several independent loads in flight each (the partial matrix is small, so this stage is latency
+// bound and wants many short chains rather than few long ones).
+template <typename Op, typename TOut>
+__global__ __launch_bounds__(1024) void reduce_partials_kernel(const float* __restrict__ part, TOut* __restrict__ out,
+                                                               int parts, int64_t row_stride, int64_t cols, float init,
+                                                               float scale) {
+    __shared__ float lds[16][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t c = (int64_t)blockIdx.x * kWave + lane;
+    float a0 = init, a1 = init, a2 = init, a3 = init;
+    if (c < cols) {
+        const float* base = part + c;
+        int p = wave;
+        for (; p + 48 < parts; p += 64) {
+            const float v0 = base[(int64_t)p * row_stride];
+            const float v1 = base[(int64_t)(p + 16) * row_stride];
+            const float v2 = base[(int64_t)(p + 32) * row_stride];
+            const float v3 = base[(int64_t)(p + 48) * row_stride];
+            a0 = Op::f(a0, v0); a1 = Op::f(a1, v1); a2 = Op::f(a2, v2); a3 = Op::f(a3, v3);
+        }
+        for (; p < parts; p += 16) a0 = Op::f(a0, base[(int64_t)p * row_stride]);
+    }
+    lds[wave][lane] = Op::f(Op::f(a0, a1), Op::f(a2, a3));
+    __syncthreads();
+    if (wave == 0 && c < cols) {
+        float a = lds[0][lane];
+#pragma unroll
+        for (int w = 1; w < 16; ++w) a = Op::f(a, lds[w][lane]);
+        out[c] = from_f32<TOut>(a * scale);
+    }
+}
+
 // ---------------------------------------------------------------- math
 // exact-GELU pieces; no fast-math anywhere on fp32 paths.
 __device__ __forceinline__ float gelu_f(float x) {
@@ -103,6 +137,26 @@ __device__ __forceinline__ float gelu_grad_f(float x) {
     return cdf + x * pdf;
 }
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// GELU for fp16 tensors: erf by Abramowitz-Stegun 7.1.26 (absolute error < 1.5e-7, far below the
+// half-precision rounding of the result) on the hardware exp2 / reciprocal. Not used on fp32 paths.
+__device__ __forceinline__ float gelu_half_f(float x) {
+    const float z = fabsf(x) * 0.70710678118654752440f;
+    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
+    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+    const float e = 1.0f - poly * __builtin_amdgcn_exp2f(-z * z * 1.44269504088896340736f);
+    return 0.5f * x * (1.0f + copysignf(e, x));
+}
+
+__device__ __forceinline__ float apply_act_half(int act, float v) {
+    switch (act) {
+        case DMLHIP_ACT_GELU: return gelu_half_f(v);
+        case DMLHIP_ACT_SWISH: return v * sigmoid_f(v);
+        case DMLHIP_ACT_SIGMOID: return sigmoid_f(v);
+        case DMLHIP_ACT_RELU: return fmaxf(v, 0.f);
+        default: return v;
+    }
+}
 
 __device__ __forceinline__ float apply_act(int act, float v) {
     switch (act) {

@@ -221,7 +221,7 @@ __device__ __forceinline__ void store_strip(const GemmArgs& g, void* c_ptr, void
     const OutT* R = reinterpret_cast<const OutT*>(res_ptr);
     // without an activation the body is small: unroll so that LDS reads and global stores of
     // several rows overlap; with one, keep a single copy of the activation code
-#pragma unroll(ACT ? 1 : 4)
+#pragma unroll(ACT ? 2 : 4)
     for (int it = 0; it < ITER; ++it) {
         const int idx = it * kWave + lane;
         const int r = idx / CPR, c8 = (idx % CPR) * 8;
@@ -261,7 +261,7 @@ __device__ __forceinline__ void store_strip(const GemmArgs& g, void* c_ptr, void
             }
             if constexpr (ACT) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] = apply_act(g.act, v[e]);
+                for (int e = 0; e < 8; ++e) v[e] = apply_act_half(g.act, v[e]);
             }
             if (R) {
                 const ovec rv = *reinterpret_cast<const ovec*>(R + off);
@@ -290,7 +290,7 @@ __device__ __forceinline__ void store_strip(const GemmArgs& g, void* c_ptr, void
                         P[off + e] = h;
                         x = (float)h;
                     }
-                    if constexpr (ACT) x = apply_act(g.act, x);
+                    if constexpr (ACT) x = apply_act_half(g.act, x);
                     if (R) x += (float)R[off + e];
                     if (g.beta != 0.f) x += g.beta * (float)C[off + e];
                     C[off + e] = (OutT)x;
@@ -514,8 +514,8 @@ extern "C" {
 void dmlhip_debug_force_gemm_config(int cfg) { g_force_cfg = cfg; }
 void dmlhip_debug_gemm_direct_lds(int on) { g_direct_lds = on; }
 
-int dmlhip_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, void* c, const void* bias,
-                    const void* residual, void* pre_out, void* stream) {
+static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, void* c, const void* bias,
+                        const void* residual, void* pre_out, void* stream) {
     DML_REQUIRE(d, DMLHIP_ERR_NULL, "gemm_f16: NULL descriptor");
     DML_REQUIRE(d->m >= 0 && d->n >= 0 && d->k >= 0, DMLHIP_ERR_SHAPE, "gemm_f16: negative extent");
     DML_REQUIRE(d->m <= 2147483647 / 2 && d->n <= 2147483647 / 2 && d->k <= 2147483647 / 2, DMLHIP_ERR_SHAPE,
@@ -593,6 +593,59 @@ int dmlhip_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, voi
         default: return launch_cfg<128, 128, 64, 64>(g, (const _Float16*)a, (const _Float16*)b, c, bias, residual, pre_out, amode, bmode,
                                                    batch, st);
     }
+}
+
+// Number of K splits worth taking for this problem (1 = none).
+static int split_k_factor(const dmlhip_gemm_desc* d) {
+    if (!d || d->m <= 0 || d->n <= 0 || d->k < 1024 || d->batch[0] != 1) return 1;
+    long long batch = d->batch[1] * d->batch[2];
+    const long long tiles = ceil_div(d->m, 128) * ceil_div(d->n, 128) * batch;
+    if (tiles > 128) return 1;
+    int s = 1;
+    while (tiles * s * 2 <= 256 && d->k / (s * 2) >= 256 && d->k % (s * 2 * 64) == 0) s *= 2;
+    return s;
+}
+
+size_t dmlhip_gemm_f16_workspace_bytes(const dmlhip_gemm_desc* d) {
+    const int s = split_k_factor(d);
+    if (s <= 1) return 0;
+    return (size_t)s * d->batch[1] * d->batch[2] * d->m * d->n * sizeof(float);
+}
+
+int dmlhip_gemm_f16_ws(const dmlhip_gemm_desc* d, const void* a, const void* b, void* c, const void* bias,
+                       const void* residual, void* pre_out, void* workspace, size_t workspace_bytes, void* stream) {
+    const int s = split_k_factor(d);
+    const bool plain = d && !bias && !residual && !pre_out && d->beta == 0.f && d->act == DMLHIP_ACT_NONE;
+    if (s <= 1 || !plain || !workspace || workspace_bytes < dmlhip_gemm_f16_workspace_bytes(d) || !a || !b || !c ||
+        d->c_stride_m != d->n || (d->batch[1] * d->batch[2] > 1))
+        return run_gemm_f16(d, a, b, c, bias, residual, pre_out, stream);
+    // stage 1: batch slot 0 enumerates the K slices; partial C tiles are dense fp32 [s][m][n]
+    dmlhip_gemm_desc p = *d;
+    p.k = d->k / s;
+    p.batch[0] = s;
+    p.a_stride_batch[0] = p.k * d->a_stride_k;
+    p.b_stride_batch[0] = p.k * d->b_stride_k;
+    p.c_stride_batch[0] = d->m * d->n;
+    p.c_stride_m = d->n;
+    p.alpha = 1.f;
+    p.out_dtype = DMLHIP_F32;
+    if (int e = run_gemm_f16(&p, a, b, workspace, nullptr, nullptr, nullptr, stream)) return e;
+    // stage 2: sum the slices, scale by alpha, convert
+    const int64_t cols = d->m * d->n;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned grid = (unsigned)ceil_div(cols, kWave);
+    if (d->out_dtype == DMLHIP_F32)
+        hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, (const float*)workspace, (float*)c,
+                           s, cols, cols, 0.f, d->alpha);
+    else
+        hipLaunchKernelGGL((reduce_partials_kernel<OpSum, _Float16>), grid, 1024, 0, st, (const float*)workspace,
+                           (_Float16*)c, s, cols, cols, 0.f, d->alpha);
+    return launch_status("gemm_f16(split-K sum)");
+}
+
+int dmlhip_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, void* c, const void* bias,
+                    const void* residual, void* pre_out, void* stream) {
+    return run_gemm_f16(d, a, b, c, bias, residual, pre_out, stream);
 }
 
 }  // extern "C"

@@ -156,11 +156,12 @@ int reduce_typed(const TIn* x, TOut* y, int64_t outer, int64_t r, int64_t inner,
     float* part = (float*)ws;
     if (int e = col_launch<TIn, float, OP>(x, part, outer, r, inner, p.v, p.tiles, p.splits, p.r_per_split, 1.0f, st))
         return e;
-    // second pass: [1, splits, outer*inner] fp32 -> TOut, same op (sum for mean), then the scale
+    // second pass over the fp32 partials [splits, outer*inner] -> TOut, same op, then the scale
     const int64_t inner2 = outer * inner;
-    const int v2 = (inner2 % 4 == 0) ? 4 : 1;
-    const int64_t tiles2 = ceil_div(inner2, (int64_t)kWave * v2);
-    return col_launch<float, TOut, OP>(part, y, 1, p.splits, inner2, v2, tiles2, 1, p.splits, scale, st);
+    using Op = typename RedOp<OP>::op;
+    hipLaunchKernelGGL((reduce_partials_kernel<Op, TOut>), (unsigned)ceil_div(inner2, kWave), 1024, 0, st,
+                       (const float*)part, y, (int)p.splits, inner2, inner2, RedOp<OP>::init(), scale);
+    return launch_status("reduce(partials)");
 }
 
 template <typename TIn>

@@ -347,17 +347,12 @@ __global__ __launch_bounds__(kRowBlock) void layernorm_bwd_wave_kernel(
     }
 }
 
-__global__ void layernorm_bwd_finish_kernel(const float* __restrict__ part, float* __restrict__ dgamma,
-                                            float* __restrict__ dbeta, int nparts, int cols) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= cols) return;
-    float a = 0.f, b = 0.f;
-    for (int p = 0; p < nparts; ++p) {
-        a += part[(size_t)p * 2 * cols + c];
-        b += part[(size_t)p * 2 * cols + cols + c];
-    }
-    dgamma[c] = a;
-    dbeta[c] = b;
+void launch_ln_bwd_finish(const float* part, float* dgamma, float* dbeta, int nparts, int64_t cols, hipStream_t st) {
+    const unsigned grid = (unsigned)ceil_div(cols, kWave);
+    hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, part, dgamma, nparts, 2 * cols, cols,
+                       0.f, 1.f);
+    hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, part ? part + cols : part, dbeta,
+                       nparts, 2 * cols, cols, 0.f, 1.f);
 }
 
 // fallback: dx, workgroup per row
@@ -516,8 +511,7 @@ int layernorm_bwd_impl(const void* dy, const void* x, const float* mean, const f
     DML_REQUIRE(dgamma && dbeta, DMLHIP_ERR_NULL, "layernorm_backward: NULL gradient pointer");
     hipStream_t st = (hipStream_t)stream;
     if (rows == 0) {
-        hipLaunchKernelGGL(layernorm_bwd_finish_kernel, (unsigned)ceil_div(cols, 256), 256, 0, st, (const float*)nullptr,
-                           dgamma, dbeta, 0, (int)cols);
+        launch_ln_bwd_finish(nullptr, dgamma, dbeta, 0, cols, st);
         return launch_status("layernorm_backward");
     }
     DML_REQUIRE(dy && x && mean && rstd && gamma && dx, DMLHIP_ERR_NULL, "layernorm_backward: NULL tensor pointer");
@@ -551,8 +545,7 @@ int layernorm_bwd_impl(const void* dy, const void* x, const float* mean, const f
         hipLaunchKernelGGL((layernorm_bwd_cols_kernel<T>), grid, 256, 0, st, gp, xp, mean, rstd, part, rows, cols);
     }
     if (int e = launch_status("layernorm_backward(stage 1)")) return e;
-    hipLaunchKernelGGL(layernorm_bwd_finish_kernel, (unsigned)ceil_div(cols, 256), 256, 0, st, (const float*)part,
-                       dgamma, dbeta, parts, (int)cols);
+    launch_ln_bwd_finish(part, dgamma, dbeta, parts, cols, st);
     return launch_status("layernorm_backward(stage 2)");
 }
 

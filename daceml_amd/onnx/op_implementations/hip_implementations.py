@@ -131,12 +131,18 @@ def _einsum_tasklet(node, state, equation, a_conn, b_conn, out_conn, a: Array, b
     plan = C.plan_contraction(equation, a.shape, a.strides, b.shape, b.strides)
     desc = _gemm_struct(plan, alpha, beta, out.dtype, bias_desc.dtype if bias_desc is not None else out.dtype, act)
     x, y = (b_conn, a_conn) if plan.swapped else (a_conn, b_conn)
-    sym = "dmlhip_gemm_" + _SFX[a.dtype]
-    call = HipCall(sym, [Struct(desc, "dmlhip_gemm_desc"), Ptr(x), Ptr(y), Ptr(out_conn),
-                         Ptr(bias) if bias else Null(), Ptr(residual) if residual else Null(),
-                         Ptr(pre_out) if pre_out else Null(), Stream()])
+    ptrs = [Struct(desc, "dmlhip_gemm_desc"), Ptr(x), Ptr(y), Ptr(out_conn), Ptr(bias) if bias else Null(),
+            Ptr(residual) if residual else Null(), Ptr(pre_out) if pre_out else Null()]
+    ws = 0
+    if a.dtype == torch.float16:
+        import ctypes
+        ws = L.load().dmlhip_gemm_f16_workspace_bytes(ctypes.byref(desc))
+        call = HipCall("dmlhip_gemm_f16_ws", ptrs + [Workspace(), WorkspaceBytes(), Stream()])
+    else:
+        call = HipCall("dmlhip_gemm_f32", ptrs + [Stream()])
     extra = [d for d in (bias_desc, ) if d is not None]
-    return _tasklet(node, state, [call], flops=plan.flops, bytes_moved=_nbytes(a, b, out, *extra), kind="gemm")
+    return _tasklet(node, state, [call], workspace_bytes=ws, flops=plan.flops, bytes_moved=_nbytes(a, b, out, *extra),
+                    kind="gemm")
 
 
 @op_implementation(op="Einsum", name=IMPL)

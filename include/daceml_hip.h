@@ -191,6 +191,15 @@ typedef struct dmlhip_gemm_desc {
 /* inputs fp16 */
 int dmlhip_gemm_f16(const dmlhip_gemm_desc* desc, const void* a, const void* b, void* c,
                     const void* bias, const void* residual, void* pre_out, void* stream);
+/* Same, with a scratch buffer: when C has too few tiles to fill the chip and K is long (the
+ * weight-gradient contractions), K is split across workgroups, fp32 partial tiles go to the
+ * workspace and a second pass sums them (deterministic, no atomics). Only plain products
+ * (no bias / activation / residual / pre_out / beta) are split; everything else runs as above.
+ * A NULL or short workspace simply disables the split. */
+size_t dmlhip_gemm_f16_workspace_bytes(const dmlhip_gemm_desc* desc);
+int dmlhip_gemm_f16_ws(const dmlhip_gemm_desc* desc, const void* a, const void* b, void* c,
+                       const void* bias, const void* residual, void* pre_out, void* workspace,
+                       size_t workspace_bytes, void* stream);
 /* inputs fp32, true fp32 MFMA (no reduced-precision path); out_dtype must be DMLHIP_F32 */
 int dmlhip_gemm_f32(const dmlhip_gemm_desc* desc, const void* a, const void* b, void* c,
                     const void* bias, const void* residual, void* pre_out, void* stream);

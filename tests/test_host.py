@@ -1,0 +1,361 @@
+"""CPU-only tests of the host side: the C ABI loads and exports what include/daceml_hip.h declares,
+argument errors are reported before any device work, the einsum planner, the library-node registry
+(three selection levels, late registration, validation), the fusion pass and the autodiff registry."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ----------------------------------------------------------------------------- C ABI
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "daceml_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dmlhip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from daceml_amd import _lib as L
+    names = _declared_symbols()
+    assert len(names) >= 35
+    for n in names:
+        assert hasattr(lib, n), "libdaceml_hip.so does not export %s" % n
+        assert n in L.SIGNATURES, "%s has no ctypes signature" % n
+    assert sorted(L.SIGNATURES) == names
+    assert lib.dmlhip_version() == 100
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from daceml_amd import _lib as L
+    monkeypatch.setattr(L, "_lib", None)
+    monkeypatch.setattr(L, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(L.HipLibraryMissing):
+        L.load()
+
+
+def test_argument_errors_need_no_gpu(lib):
+    """Negative return codes come from host-side validation, before any launch."""
+    from daceml_amd import _lib as L
+    p = ctypes.c_void_p(16)  # never dereferenced
+    assert lib.dmlhip_softmax_f16(p, p, -1, 4, None) == L.ERR_SHAPE
+    assert "negative" in L.last_error()
+    assert lib.dmlhip_softmax_f16(None, p, 4, 4, None) == L.ERR_NULL
+    assert lib.dmlhip_softmax_f32(None, None, 0, 16, None) == 0          # empty: no-op, not an error
+    assert lib.dmlhip_layernorm_f16(p, None, p, p, p, None, None, None, 4, 8, -1.0, None) == L.ERR_SHAPE
+    assert lib.dmlhip_layernorm_backward_f16(p, p, p, p, p, p, p, p, 8, 64, None, 0, None) == L.ERR_WORKSPACE
+    assert lib.dmlhip_layernorm_backward_workspace_bytes(4096, 1024) > 0
+    shape = L.i64_array([4, 4])
+    assert lib.dmlhip_binary_f16(99, p, p, p, 2, shape, shape, shape, None) == L.ERR_ENUM
+    assert lib.dmlhip_binary_f16(L.ADD, p, p, p, 9, shape, shape, shape, None) == L.ERR_SHAPE
+    assert lib.dmlhip_unary_f32(L.GELU, ctypes.c_void_p(2), p, 8, 0.0, None) == L.ERR_ALIGN
+    assert lib.dmlhip_cast(L.F16, 7, p, p, 4, None) == L.ERR_ENUM
+    perm = L.i64_array([0, 0])
+    assert lib.dmlhip_transpose_f16(p, p, 2, shape, perm, None) == L.ERR_SHAPE
+    assert lib.dmlhip_reduce_f16(L.RMEAN, p, p, L.F32, 4, 0, 1, None, 0, None) == L.ERR_SHAPE   # mean of nothing
+    d = L.GemmDesc()
+    d.m, d.n, d.k = 4, 4, -1
+    assert lib.dmlhip_gemm_f16(ctypes.byref(d), p, p, p, None, None, None, None) == L.ERR_SHAPE
+    d.k = 4
+    d.batch[0] = d.batch[1] = d.batch[2] = 1
+    d.c_stride_m = 2  # rows of C would overlap
+    assert lib.dmlhip_gemm_f16(ctypes.byref(d), p, p, p, None, None, None, None) == L.ERR_SHAPE
+    d.c_stride_m = 4
+    d.out_dtype = 5
+    assert lib.dmlhip_gemm_f16(ctypes.byref(d), p, p, p, None, None, None, None) == L.ERR_ENUM
+    d.out_dtype = L.F16
+    assert lib.dmlhip_gemm_f32(ctypes.byref(d), p, p, p, None, None, None, None) == L.ERR_ENUM  # f32 in -> f32 out
+    assert lib.dmlhip_gemm_f16(None, p, p, p, None, None, None, None) == L.ERR_NULL
+    c = L.Conv2dDesc()
+    c.n, c.c, c.h, c.w, c.m, c.kh, c.kw = 1, 4, 8, 8, 6, 3, 3
+    c.stride_h = c.stride_w = c.dil_h = c.dil_w = 1
+    c.group = 3   # 4 channels not divisible by 3
+    assert lib.dmlhip_conv2d_f32(ctypes.byref(c), p, p, None, p, None) == L.ERR_SHAPE
+    c.group = 1
+    oh, ow = ctypes.c_int64(), ctypes.c_int64()
+    assert lib.dmlhip_conv2d_out_shape(ctypes.byref(c), ctypes.byref(oh), ctypes.byref(ow)) == 0
+    assert (oh.value, ow.value) == (6, 6)
+    c.stride_h = c.stride_w = 2   # config 1 of the baseline: 10x10, k3, s2 -> 4x4
+    c.h = c.w = 10
+    lib.dmlhip_conv2d_out_shape(ctypes.byref(c), ctypes.byref(oh), ctypes.byref(ow))
+    assert (oh.value, ow.value) == (4, 4)
+
+
+def test_kernels_refuse_host_tensors():
+    from daceml_amd import kernels as K
+    with pytest.raises(ValueError):
+        K.softmax(torch.zeros(2, 4, dtype=torch.float16))
+    with pytest.raises(TypeError):
+        K._fn("softmax", torch.float64)
+
+
+# ----------------------------------------------------------------------------- einsum planner
+def _plan(eq, sa, sb, stra=None, strb=None):
+    from daceml_amd import contraction as C
+    return C.plan_contraction(eq, sa, stra or C.contiguous_strides(sa), sb, strb or C.contiguous_strides(sb))
+
+
+def test_planner_bert_contractions():
+    from daceml_amd import contraction as C
+    p = _plan("aik,kj->aij", (8, 512, 1024), (1024, 1024))
+    assert (p.m, p.n, p.k, p.batch) == (4096, 1024, 1024, [1, 1, 1]) and p.a_stride_k == 1 and p.b_stride_n == 1
+    p = _plan("aik,jk->aij", (8, 512, 1024), (4096, 1024))          # weight stored [out, in]
+    assert (p.b_stride_k, p.b_stride_n) == (1, 1024)
+    p = _plan("baik,bakj->baij", (8, 16, 512, 64), (8, 16, 64, 512))
+    assert (p.m, p.n, p.k, p.batch) == (512, 512, 64, [1, 1, 128])
+    p = _plan("biak,bjak->baij", (8, 512, 16, 64), (8, 512, 16, 64))  # head split folded into strides
+    assert p.batch == [1, 8, 16] and p.a_stride_m == 1024 and p.a_stride_batch[1:] == [512 * 1024, 64]
+    p = _plan("baik,bkaj->biaj", (8, 16, 512, 512), (8, 512, 16, 64))  # head merge folded into C's strides
+    assert p.n == 64 and p.c_stride_m == 1024 and p.c_stride_batch[1:] == [512 * 1024, 64]
+    p = _plan("aij,aik->jk", (8, 512, 4096), (8, 512, 1024))        # weight gradient: K = (a, i) merged
+    assert (p.m, p.n, p.k) == (4096, 1024, 4096) and p.a_stride_m == 1 and not p.swapped
+    p = _plan("ik,kj->ji", (4, 5), (5, 6))
+    assert p.swapped and (p.m, p.n) == (6, 4)
+    assert p.flops == 2 * 4 * 5 * 6
+    assert C.reverse_equation("ik,kj->ij", 0) == ([1], "ij,kj->ik")
+    assert C.reverse_equation("ik,kj->ij", 1) == ([0], "ij,ik->kj")
+    assert C.matmul_equation(3, 2) == "aik,kj->aij" and C.matmul_equation(4, 4) == "baik,bakj->baij"
+    assert C.transpose_perm("zyxw->zxyw") == [0, 2, 1, 3] and C.transpose_perm("ij->i") is None
+
+
+@pytest.mark.parametrize("eq,sa,sb", [("ii,ij->j", (3, 3), (3, 4)), ("ij,jk->ik...", (2, 2), (2, 2)),
+                                      ("ijl,jk->ik", (2, 3, 4), (3, 5)), ("bik,bkj->ijb", (2, 3, 4), (2, 4, 5))])
+def test_planner_refuses(eq, sa, sb):
+    from daceml_amd import contraction as C
+    with pytest.raises(C.NotApplicable):
+        _plan(eq, sa, sb)
+
+
+def test_planner_matches_numpy_semantics_by_emulation():
+    """Execute plans with plain index arithmetic on the host: pins the stride bookkeeping."""
+    from daceml_amd import contraction as C
+    rng = np.random.default_rng(0)
+    for eq, sa, sb in [("biak,bjak->baij", (2, 5, 3, 4), (2, 6, 3, 4)), ("aij,aik->jk", (2, 3, 4), (2, 3, 5)),
+                       ("ik,kj->ji", (3, 4), (4, 5)), ("baik,bkaj->biaj", (2, 3, 4, 5), (2, 5, 3, 6))]:
+        a, b = rng.standard_normal(sa), rng.standard_normal(sb)
+        p = _plan(eq, sa, sb)
+        x, y = (b, a) if p.swapped else (a, b)
+        xf, yf = x.reshape(-1), y.reshape(-1)
+        out = np.zeros(int(np.prod(p.out_shape)))
+        for z0 in range(p.batch[0]):
+            for z1 in range(p.batch[1]):
+                for z2 in range(p.batch[2]):
+                    z = (z0, z1, z2)
+                    ao = sum(z[i] * p.a_stride_batch[i] for i in range(3))
+                    bo = sum(z[i] * p.b_stride_batch[i] for i in range(3))
+                    co = sum(z[i] * p.c_stride_batch[i] for i in range(3))
+                    for m in range(p.m):
+                        for n in range(p.n):
+                            acc = 0.0
+                            for k in range(p.k):
+                                acc += xf[ao + m * p.a_stride_m + k * p.a_stride_k] * \
+                                       yf[bo + k * p.b_stride_k + n * p.b_stride_n]
+                            out[co + m * p.c_stride_m + n] = acc
+        np.testing.assert_allclose(out.reshape(p.out_shape), np.einsum(eq, a, b), rtol=1e-12)
+
+
+# ----------------------------------------------------------------------------- registry
+def _softmax_sdfg(dtype=torch.float16, shape=(4, 8)):
+    import daceml_amd.onnx as donnx
+    from daceml_amd.sdfg import SDFG
+    sdfg = SDFG("t")
+    st = sdfg.add_state()
+    sdfg.add_array("a", shape, dtype)
+    sdfg.add_array("b", shape, dtype)
+    node = donnx.ONNXSoftmax("sm", axis=-1)
+    st.add_edge(st.add_read("a"), None, node, "input", sdfg.make_array_memlet("a"))
+    st.add_edge(node, "output", st.add_write("b"), None, sdfg.make_array_memlet("b"))
+    return sdfg, st, node
+
+
+def test_registry_mirrors_reference_api():
+    import daceml_amd.onnx as donnx
+    from daceml_amd.onnx import ONNXForward, op_implementation
+    for op in ["MatMul", "Einsum", "Gemm", "Softmax", "Add", "Sub", "Mul", "Div", "Sum", "Erf", "ReduceMean",
+               "ReduceSum", "Transpose", "Conv", "GlobalAveragePool", "Sigmoid", "LayerNormalization", "Gelu",
+               "BiasGelu"]:
+        impls = dict(ONNXForward.registered_implementations(op))
+        assert "hip" in impls, op
+        assert "hip" in donnx.get_onnx_node(op).implementations
+    assert donnx.has_onnx_node("Conv") and not donnx.has_onnx_node("NoSuchOp")
+    with pytest.raises(ValueError):
+        donnx.get_onnx_node("NoSuchOp")
+    with pytest.raises(ValueError):
+        donnx.ONNXEinsum("e")                     # required attribute missing
+    with pytest.raises(TypeError):
+        donnx.ONNXSoftmax("s", nonsense=1)
+
+    # an implementation registered late is visible on the node class too
+    calls = []
+
+    @op_implementation(op="Softmax", name="probe")
+    class Probe(ONNXForward):
+        @staticmethod
+        def forward_can_be_applied(node, state, sdfg):
+            return sdfg.arrays["a"].dtype == torch.float16
+
+        @staticmethod
+        def forward(node, state, sdfg):
+            calls.append(node.label)
+            return donnx.ONNXSoftmax.implementations["hip"].forward(node, state, sdfg)
+
+    try:
+        assert "probe" in donnx.ONNXSoftmax.implementations
+        # package default < class default < node.implementation
+        sdfg, st, node = _softmax_sdfg()
+        assert node.selected_implementation() == "hip"
+        old = donnx.default_implementation
+        donnx.default_implementation = "probe"
+        assert node.selected_implementation() == "probe"
+        donnx.ONNXSoftmax.default_implementation = "hip"
+        assert node.selected_implementation() == "hip"
+        node.implementation = "probe"
+        assert node.selected_implementation() == "probe"
+        node.expand(sdfg, st)
+        assert calls == ["sm"]
+        # inapplicable -> explicit refusal, no silent fallback
+        sdfg32, st32, node32 = _softmax_sdfg(torch.float32)
+        node32.implementation = "probe"
+        with pytest.raises(donnx.NotApplicable):
+            node32.expand(sdfg32, st32)
+    finally:
+        donnx.default_implementation = old
+        donnx.ONNXSoftmax.default_implementation = None
+        donnx.ONNXSoftmax.implementations.pop("probe", None)
+        ONNXForward.unregister(Probe)
+
+
+def test_validate_checks_connectors():
+    import daceml_amd.onnx as donnx
+    from daceml_amd.sdfg import SDFG
+    sdfg, st, node = _softmax_sdfg()
+    node.validate(sdfg, st)
+    # missing required output
+    sdfg2 = SDFG("v")
+    st2 = sdfg2.add_state()
+    sdfg2.add_array("a", (2, 2), torch.float32)
+    n2 = donnx.ONNXSoftmax("s")
+    st2.add_edge(st2.add_read("a"), None, n2, "input", sdfg2.make_array_memlet("a"))
+    with pytest.raises(ValueError, match="output"):
+        n2.validate(sdfg2, st2)
+    # variadic numbering must be 0..n-1
+    sdfg2.add_array("o", (2, 2), torch.float32)
+    s = donnx.ONNXSum("sum")
+    s.add_in_connector("data_0__1")
+    st2.add_edge(st2.add_read("a"), None, s, "data_0__1", sdfg2.make_array_memlet("a"))
+    st2.add_edge(s, "sum", st2.add_write("o"), None, sdfg2.make_array_memlet("o"))
+    with pytest.raises(ValueError, match="numbered"):
+        s.validate(sdfg2, st2)
+    with pytest.raises(ValueError):
+        donnx.parse_variadic_param("x__01")
+    assert donnx.parse_variadic_param("Inputs__3") == ("Inputs", 3)
+    # integer tensors are not supported element types
+    sdfg3 = SDFG("i")
+    st3 = sdfg3.add_state()
+    sdfg3.add_array("a", (2, ), torch.uint8)
+    sdfg3.add_array("b", (2, ), torch.uint8)
+    r = donnx.ONNXRelu("r")
+    st3.add_edge(st3.add_read("a"), None, r, "X", sdfg3.make_array_memlet("a"))
+    st3.add_edge(r, "Y", st3.add_write("b"), None, sdfg3.make_array_memlet("b"))
+    with pytest.raises(TypeError):
+        r.validate(sdfg3, st3)
+
+
+def test_forward_can_be_applied_never_raises_and_refuses():
+    import daceml_amd.onnx as donnx
+    from daceml_amd.sdfg import SDFG
+    hip = donnx.ONNXConv.implementations["hip"]
+    sdfg = SDFG("c")
+    st = sdfg.add_state()
+    sdfg.add_array("x", (1, 3, 8, 8), torch.float32)
+    sdfg.add_array("w", (4, 3, 3, 3), torch.float32)
+    sdfg.add_array("y", (1, 4, 6, 6), torch.float32)
+    conv = donnx.ONNXConv("conv", pads=[1, 0, 0, 0])            # asymmetric pads: refused
+    for arr, conn in (("x", "X"), ("w", "W")):
+        st.add_edge(st.add_read(arr), None, conv, conn, sdfg.make_array_memlet(arr))
+    st.add_edge(conv, "Y", st.add_write("y"), None, sdfg.make_array_memlet("y"))
+    assert hip.forward_can_be_applied(conv, st, sdfg) is False
+    conv.pads = None
+    assert hip.forward_can_be_applied(conv, st, sdfg) is True
+    conv.auto_pad = "SAME_UPPER"
+    assert hip.forward_can_be_applied(conv, st, sdfg) is False
+    # a node with no edges at all: False, not an exception
+    assert donnx.ONNXSoftmax.implementations["hip"].forward_can_be_applied(donnx.ONNXSoftmax("s"), st, sdfg) is False
+    # Einsum with an ellipsis (refused by PureEinsum as well)
+    es = donnx.ONNXEinsum("e", equation="...ij,jk->...ik")
+    assert donnx.ONNXEinsum.implementations["hip"].forward_can_be_applied(es, st, sdfg) is False
+
+
+# ----------------------------------------------------------------------------- fusion / autodiff
+def test_fusion_pipeline_on_bert_layer():
+    from daceml_amd import graphs
+    from daceml_amd.transformation import fusion
+    sdfg = graphs.bert_encoder_layer(2, 64, 128, 4, 512, torch.float16)
+    st = sdfg.states()[0]
+    before = [n.schema.name for n in st.library_nodes()]
+    assert before.count("MatMul") == 8 and before.count("Erf") == 1 and before.count("ReduceMean") == 4
+    stats = fusion.auto_optimize(sdfg, training=True)
+    assert stats == {"gelu": 1, "layernorm": 2, "swish": 0, "conv_activation": 0, "matmul_to_einsum": 8,
+                     "views": 15, "epilogues": 7, "skip_layernorm": 0}
+    after = {n.label: n for n in st.library_nodes()}
+    assert sorted(n.schema.name for n in after.values()) == ["Einsum"] + ["FusedEinsum"] * 7 + \
+        ["LayerNormalization"] * 2 + ["Softmax"]
+    assert after["scores_fused"].equation == "biak,bjak->baij"          # head split folded into letters
+    assert abs(after["scores_fused"].alpha - 1 / np.sqrt(32)) < 1e-12   # Div(sqrt d) -> alpha
+    assert after["context"].equation == "baik,bkaj->biaj"               # head merge folded into the output
+    assert after["ffn1_matmul_fused"].activation == "gelu"
+    conns = {e.dst_conn for e in st.in_edges(after["o_matmul_fused"])}
+    assert conns == {"Inputs__0", "Inputs__1", "Bias", "Residual"}
+    assert after["ln1_fused"].epsilon == 1e-12                          # not the fp16-rounded 0.0
+    assert all(e.dst_conn != "Inputs__1" or sdfg.arrays[e.data.data].shape == (128, 128)
+               for e in st.in_edges(after["q_matmul_fused"]))           # weight used as stored, no Transpose
+
+
+def test_fusion_leaves_non_matching_chains_alone():
+    from daceml_amd import graphs
+    from daceml_amd.transformation import fusion
+    g = graphs.GraphBuilder("t", torch.float32)
+    x = g.input("x", (4, 8))
+    y = g.gelu(x, "g")
+    # a second consumer of an internal value makes the chain non-fusable
+    erf_out = [a for a in g.sdfg.arrays if "erf" in a][0]
+    z = g.node("Relu", {"X": erf_out}, {"Y": (4, 8)})["Y"]
+    g.output(y, "y")
+    g.output(z, "z")
+    assert fusion.fuse_gelu(g.sdfg) == 0
+
+
+def test_backward_pass_structure():
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import (BackwardImplementation, add_backward_pass, find_backward_implementation)
+    from daceml_amd.transformation import fusion
+    from oracle.bert_layer import PARAM_NAMES
+    sdfg = graphs.bert_encoder_layer(2, 64, 128, 4, 512, torch.float16)
+    fusion.auto_optimize(sdfg, training=True)
+    st = sdfg.states()[0]
+    grads = add_backward_pass(sdfg, st, ["y"], ["x"] + PARAM_NAMES, grad_dtypes={n: torch.float32 for n in PARAM_NAMES})
+    assert grads["x"] == "gradient_x" and all(grads[n] == "gradient_" + n for n in PARAM_NAMES)
+    assert sdfg.arrays["gradient_q_w"].dtype == torch.float32 and not sdfg.arrays["gradient_q_w"].transient
+    assert sdfg.arrays["gradient_x"].dtype == torch.float16
+    bst = sdfg.states()[1]
+    names = [n.schema.name for n in bst.library_nodes()]
+    assert names.count("FusedEinsum") == 16 and names.count("LayerNormalizationGrad") == 2
+    assert names.count("SoftmaxGrad") == 1 and names.count("GeluGrad") == 1 and names.count("Sum") == 2
+    assert names.count("ReduceSum") == 6
+    # equations follow reverse_einsum_wrt_input
+    eqs = {n.label: n.equation for n in bst.library_nodes() if n.schema.name == "FusedEinsum"}
+    assert eqs["q_matmul_fused_grad_0"] == "aij,jk->aik" and eqs["q_matmul_fused_grad_1"] == "aij,aik->jk"
+    # the forward LayerNorm nodes were given statistics outputs for the backward to read
+    ln = [n for n in st.library_nodes() if n.schema.name == "LayerNormalization"][0]
+    assert {e.src_conn for e in st.out_edges(ln)} == {"Y", "Mean", "InvStdDev"}
+    # registry lookup honours node.backward_implementation
+    sm = [n for n in st.library_nodes() if n.schema.name == "Softmax"][0]
+    impl = find_backward_implementation(sdfg, st, sm)
+    assert impl is not None and issubclass(impl, BackwardImplementation)
+    # everything in both states expands with the hip implementations
+    from daceml_amd.runtime import expand_onnx_nodes
+    assert expand_onnx_nodes(sdfg) == len(names) + 11

@@ -1,0 +1,317 @@
+"""Pins the CPU oracle (oracle/) before anything is compared with it.
+
+The reference holds no golden vectors for the ops on this path: its own tests compare with NumPy /
+PyTorch on unseeded inputs (tests/pure_expansions/test_expansions.py:29-63,187-237,387-405,
+tests/pure_expansions/test_conv_expansion.py:9-66, tests/autodiff/torch/test_pytorch.py:96-150). So each
+oracle function is pinned the same way, against an *independent* routine (torch / scipy library
+functions, torch.autograd, explicit loops), plus closed forms and invariants chosen so that a dropped
+term, a wrong sign / axis or a transposed operand fails.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import bert_layer as OB
+from oracle import ops as O
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ----------------------------------------------------------------------------- softmax
+@pytest.mark.parametrize("shape,axis", [((4, 7), 1), ((2, 3, 5, 6), -1), ((2, 3, 5, 6), 3), ((3, 4, 5), 2)])
+def test_softmax_last_axis_matches_torch(shape, axis):
+    x = rng(0).standard_normal(shape)
+    np.testing.assert_allclose(O.softmax(x, axis), F.softmax(torch.tensor(x), dim=-1).numpy(), rtol=1e-12, atol=1e-14)
+
+
+def test_softmax_opset12_axis_coalescing():
+    """axis=1 on a 4-D tensor normalises over axes 1,2,3 *together* (opset < 13), unlike torch's dim=1."""
+    x = rng(1).standard_normal((2, 3, 4, 5))
+    y = O.softmax(x, 1)
+    want = F.softmax(torch.tensor(x).reshape(2, -1), dim=1).reshape(2, 3, 4, 5).numpy()
+    np.testing.assert_allclose(y, want, rtol=1e-12, atol=1e-14)
+    assert not np.allclose(y, F.softmax(torch.tensor(x), dim=1).numpy())
+    np.testing.assert_allclose(y.reshape(2, -1).sum(1), 1.0, rtol=1e-12)
+    # axis 0: everything is one row, keepdims False in the reference
+    y0 = O.softmax(x, 0)
+    assert y0.shape == x.shape and abs(y0.sum() - 1.0) < 1e-12
+
+
+def test_softmax_invariants():
+    x = rng(2).standard_normal((5, 33))
+    y = O.softmax(x, -1)
+    np.testing.assert_allclose(O.softmax(x + 100.0, -1), y, rtol=1e-10)       # shift invariance
+    np.testing.assert_allclose(O.softmax(np.full((2, 8), 3.0), -1), 1 / 8)    # constant row
+    big = np.array([[1e4, 0.0, -1e4]])
+    np.testing.assert_allclose(O.softmax(big, -1), [[1.0, 0.0, 0.0]], atol=1e-300)  # no overflow
+
+
+def test_softmax_backward_matches_autograd():
+    x = torch.tensor(rng(3).standard_normal((3, 4, 9)), requires_grad=True)
+    dy = torch.tensor(rng(4).standard_normal((3, 4, 9)))
+    y = F.softmax(x, dim=-1)
+    y.backward(dy)
+    np.testing.assert_allclose(O.softmax_backward(y.detach().numpy(), dy.numpy(), 2), x.grad.numpy(), rtol=1e-10,
+                               atol=1e-12)
+    # rows of the gradient sum to zero (softmax outputs are constrained to the simplex)
+    assert np.abs(O.softmax_backward(y.detach().numpy(), dy.numpy(), 2).sum(-1)).max() < 1e-12
+
+
+# ----------------------------------------------------------------------------- layernorm / gelu
+def test_layernorm_chain_matches_torch_and_two_pass_loop():
+    x = rng(5).standard_normal((3, 5, 16))
+    g = rng(6).uniform(0.5, 1.5, 16)
+    b = rng(7).standard_normal(16) * 0.1
+    y, mean, var = O.layernorm_chain(x, g, b, 1e-5)
+    want = F.layer_norm(torch.tensor(x), (16, ), torch.tensor(g), torch.tensor(b), 1e-5).numpy()
+    np.testing.assert_allclose(y, want, rtol=1e-11, atol=1e-12)
+    for i in range(3):
+        for j in range(5):
+            row = x[i, j]
+            mu = sum(row) / 16
+            v = sum((t - mu)**2 for t in row) / 16          # biased, two-pass
+            assert abs(mean[i, j, 0] - mu) < 1e-14 and abs(var[i, j, 0] - v) < 1e-14
+            np.testing.assert_allclose(y[i, j], (row - mu) / math.sqrt(v + 1e-5) * g + b, rtol=1e-12)
+
+
+def test_layernorm_invariants():
+    x = rng(8).standard_normal((4, 64))
+    y, _, _ = O.layernorm_chain(x, np.ones(64), np.zeros(64), 0.0)
+    np.testing.assert_allclose(y.mean(-1), 0.0, atol=1e-14)
+    np.testing.assert_allclose(y.var(-1), 1.0, rtol=1e-12)
+    b = rng(9).standard_normal(64)
+    yc, _, _ = O.layernorm_chain(np.full((2, 64), 3.0), np.ones(64), b, 1e-5)
+    np.testing.assert_allclose(yc, np.broadcast_to(b, (2, 64)), atol=1e-12)   # constant row -> beta
+
+
+def test_layernorm_backward_matches_autograd():
+    x = torch.tensor(rng(10).standard_normal((2, 7, 24)), requires_grad=True)
+    g = torch.tensor(rng(11).uniform(0.5, 1.5, 24), requires_grad=True)
+    b = torch.tensor(rng(12).standard_normal(24), requires_grad=True)
+    dy = torch.tensor(rng(13).standard_normal((2, 7, 24)))
+    F.layer_norm(x, (24, ), g, b, 1e-5).backward(dy)
+    dx, dg, db = O.layernorm_backward(dy.numpy(), x.detach().numpy(), g.detach().numpy(), 1e-5)
+    np.testing.assert_allclose(dx, x.grad.numpy(), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(dg, g.grad.numpy(), rtol=1e-10)
+    np.testing.assert_allclose(db, b.grad.numpy(), rtol=1e-10)
+
+
+def test_gelu_is_exact_erf_form_not_tanh():
+    x = rng(14).standard_normal(1000) * 3
+    np.testing.assert_allclose(O.gelu_chain(x), F.gelu(torch.tensor(x), approximate="none").numpy(), rtol=1e-12,
+                               atol=1e-14)
+    assert np.abs(O.gelu_chain(x) - F.gelu(torch.tensor(x), approximate="tanh").numpy()).max() > 1e-4
+    assert O.gelu_chain(np.array([0.0]))[0] == 0.0
+    np.testing.assert_allclose(O.gelu_chain(np.array([10.0, -10.0])), [10.0, 0.0], atol=1e-12)
+    t = torch.tensor(x, requires_grad=True)
+    dy = rng(15).standard_normal(1000)
+    F.gelu(t).backward(torch.tensor(dy))
+    np.testing.assert_allclose(O.gelu_backward(dy, x), t.grad.numpy(), rtol=1e-10, atol=1e-12)
+
+
+def test_sigmoid_swish():
+    x = rng(16).standard_normal(100) * 4
+    np.testing.assert_allclose(O.sigmoid(x), torch.sigmoid(torch.tensor(x)).numpy(), rtol=1e-12)
+    np.testing.assert_allclose(O.swish(x), F.silu(torch.tensor(x)).numpy(), rtol=1e-12)
+    t = torch.tensor(x, requires_grad=True)
+    F.silu(t).backward(torch.ones(100, dtype=torch.float64))
+    np.testing.assert_allclose(O.swish_backward(np.ones(100), x), t.grad.numpy(), rtol=1e-10)
+
+
+# ----------------------------------------------------------------------------- elementwise / reductions
+def test_binary_broadcasting_and_sum():
+    a = rng(17).standard_normal((2, 3, 4))
+    b = rng(18).standard_normal((3, 1))
+    for name, fn in (("add", np.add), ("sub", np.subtract), ("mul", np.multiply), ("div", np.divide)):
+        np.testing.assert_array_equal(getattr(O, name)(a, b), fn(a, b))
+    assert not np.allclose(O.sub(a, b), O.sub(b, a))  # operand order matters
+    np.testing.assert_array_equal(O.sum_variadic(a, a, a), 3 * a)
+    with pytest.raises(ValueError):
+        O.sum_variadic(a, b)  # PureSum does not broadcast
+
+
+@pytest.mark.parametrize("name,ref", [("sum", torch.sum), ("mean", torch.mean), ("max", torch.amax),
+                                      ("min", torch.amin)])
+@pytest.mark.parametrize("axes,keepdims", [([1], 1), ([-1], 0), ([0, 1], 1), ([1, 2], 0)])
+def test_reductions_match_torch(name, ref, axes, keepdims):
+    x = rng(19).standard_normal((3, 4, 5))
+    got = getattr(O, "reduce_" + name)(x, axes, keepdims)
+    want = ref(torch.tensor(x), dim=axes, keepdim=bool(keepdims)).numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-13)
+    # the reference's literal known answer: ReduceSum over [1,2,3,4] = 10 (tests/test_onnx_return_scalars.py:43-46)
+    assert O.reduce_sum(np.array([1.0, 2.0, 3.0, 4.0]), [0], 0) == 10.0
+
+
+def test_global_average_pool():
+    x = rng(20).standard_normal((2, 3, 4, 5))
+    np.testing.assert_allclose(O.global_average_pool(x), F.adaptive_avg_pool2d(torch.tensor(x), 1).numpy(), rtol=1e-13)
+
+
+# ----------------------------------------------------------------------------- contractions
+def test_matmul_equation_table():
+    """Strings PureMatMul builds (pure_implementations.py:132-191); the two BERT cases are the ones the
+    survey of the reference derives by hand."""
+    assert O.matmul_equation((8, 512, 1024), (1024, 1024)) == "aik,kj->aij"
+    assert O.matmul_equation((8, 16, 512, 64), (8, 16, 64, 512)) == "baik,bakj->baij"
+    assert O.matmul_equation((4, 5), (5, 6)) == "ik,kj->ij"
+    assert O.matmul_equation((5, 6), (3, 6, 7)) == "ik,akj->aij"
+    assert O.matmul_equation((2, 3, 4, 5), (5, 6)) == "baik,kj->baij"
+    assert O.matmul_equation((7, ), (7, 3)) == "k,kj->j"
+    assert O.matmul_equation((3, 7), (7, )) == "ik,k->i"
+
+
+@pytest.mark.parametrize("sa,sb", [((4, 5), (5, 6)), ((2, 4, 5), (5, 6)), ((2, 3, 4, 5), (2, 3, 5, 6)),
+                                   ((4, 5), (3, 5, 6))])
+def test_matmul_matches_numpy_at(sa, sb):
+    a, b = rng(21).standard_normal(sa), rng(22).standard_normal(sb)
+    np.testing.assert_allclose(O.matmul(a, b), a @ b, rtol=1e-12)      # the check of test_expansions.py:29-63
+
+
+def test_einsum_and_its_backward():
+    a, b = rng(23).standard_normal((3, 4, 5)), rng(24).standard_normal((5, 6))
+    np.testing.assert_allclose(O.einsum("bij, jk -> bik", a, b), torch.einsum("bij,jk->bik", torch.tensor(a),
+                                                                              torch.tensor(b)).numpy(), rtol=1e-12)
+    with pytest.raises(NotImplementedError):
+        O.einsum("...ij,jk->...ik", a, b)
+    # reverse_einsum_wrt_input: the two strings spelled out in the analysis of onnx_ops.py:42-51
+    assert O.reverse_einsum_wrt_input("ik,kj->ij", 0) == ([1], "ij,kj->ik")
+    assert O.reverse_einsum_wrt_input("ik,kj->ij", 1) == ([0], "ij,ik->kj")
+    ta, tb = torch.tensor(a, requires_grad=True), torch.tensor(b, requires_grad=True)
+    dy = rng(25).standard_normal((3, 4, 6))
+    torch.einsum("bij,jk->bik", ta, tb).backward(torch.tensor(dy))
+    np.testing.assert_allclose(O.einsum_backward("bij,jk->bik", [a, b], dy, 0), ta.grad.numpy(), rtol=1e-12)
+    np.testing.assert_allclose(O.einsum_backward("bij,jk->bik", [a, b], dy, 1), tb.grad.numpy(), rtol=1e-12)
+
+
+def test_gemm_attributes():
+    a, b, c = rng(26).standard_normal((4, 5)), rng(27).standard_normal((6, 5)), rng(28).standard_normal(6)
+    np.testing.assert_allclose(O.gemm(a, b, c, alpha=0.5, beta=2.0, transB=1), 0.5 * a @ b.T + 2.0 * c, rtol=1e-12)
+    np.testing.assert_allclose(O.gemm(a.T.copy(), b.T.copy(), None, transA=1), a @ b.T, rtol=1e-12)
+    np.testing.assert_allclose(O.gemm(a, b, c, transB=1), F.linear(torch.tensor(a), torch.tensor(b),
+                                                                    torch.tensor(c)).numpy(), rtol=1e-12)
+
+
+def test_transpose_default_perm_reverses():
+    x = rng(29).standard_normal((2, 3, 4))
+    assert O.transpose(x).shape == (4, 3, 2)
+    np.testing.assert_array_equal(O.transpose(x, [1, 0, 2]), np.swapaxes(x, 0, 1))
+
+
+# ----------------------------------------------------------------------------- conv
+CONV_CASES = [
+    ((5, 3, 10, 10), (16, 3, 3, 3), (2, 2), (0, 0), (1, 1), 1),   # README / examples/plot_conv.py:16-46
+    ((2, 3, 8, 8), (4, 3, 3, 3), (1, 1), (0, 0), (1, 1), 1),      # what PureConv2D itself covers
+    ((2, 6, 9, 9), (6, 1, 3, 3), (2, 2), (1, 1), (1, 1), 6),      # depthwise
+    ((1, 4, 7, 7), (6, 2, 3, 3), (1, 1), (1, 1), (1, 1), 2),      # grouped
+    ((1, 2, 9, 9), (3, 2, 3, 3), (1, 1), (2, 2), (2, 2), 1),      # dilated
+    ((2, 5, 6, 6), (7, 5, 1, 1), (1, 1), (0, 0), (1, 1), 1),      # pointwise
+]
+
+
+@pytest.mark.parametrize("xs,ws,st,pd,dl,grp", CONV_CASES)
+def test_conv_matches_torch_and_loops(xs, ws, st, pd, dl, grp):
+    x, w, b = rng(30).uniform(0, 1, xs), rng(31).uniform(0, 1, ws), rng(32).standard_normal(ws[0])
+    pads = (pd[0], pd[1], pd[0], pd[1])
+    want = F.conv2d(torch.tensor(x), torch.tensor(w), torch.tensor(b), st, pd, dl, grp).numpy()
+    np.testing.assert_allclose(O.conv2d(x, w, b, st, pads, dl, grp), want, rtol=1e-12, atol=1e-13)
+    if x.size * w.size < 2e6:
+        np.testing.assert_allclose(O.conv2d_loops(x, w, b, st, pads, dl, grp), want, rtol=1e-12, atol=1e-13)
+    assert want.shape[2] == O.conv_out_size(xs[2], ws[2], st[0], 2 * pd[0], dl[0])
+
+
+def test_conv_config1_shape_and_center_tap():
+    assert O.conv2d(np.zeros((5, 3, 10, 10)), np.zeros((16, 3, 3, 3)), None, (2, 2)).shape == (5, 16, 4, 4)
+    # a kernel that is 1 at (hy, hx) = (0, 2) picks X[..., oy, ox + 2]: cross-correlation, not convolution
+    x = rng(33).standard_normal((1, 1, 5, 5))
+    w = np.zeros((1, 1, 3, 3))
+    w[0, 0, 0, 2] = 1.0
+    np.testing.assert_array_equal(O.conv2d(x, w)[0, 0], x[0, 0, 0:3, 2:5])
+
+
+@pytest.mark.parametrize("xs,ws,st,pd,dl,grp", CONV_CASES)
+def test_conv_backward_matches_autograd(xs, ws, st, pd, dl, grp):
+    x = torch.tensor(rng(34).standard_normal(xs), requires_grad=True)
+    w = torch.tensor(rng(35).standard_normal(ws), requires_grad=True)
+    b = torch.tensor(rng(36).standard_normal(ws[0]), requires_grad=True)
+    y = F.conv2d(x, w, b, st, pd, dl, grp)
+    dy = rng(37).standard_normal(tuple(y.shape))
+    y.backward(torch.tensor(dy))
+    dx, dw, db = O.conv2d_backward(x.detach().numpy(), w.detach().numpy(), dy, st, (pd[0], pd[1], pd[0], pd[1]), dl, grp,
+                                   has_bias=True)
+    np.testing.assert_allclose(dx, x.grad.numpy(), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(dw, w.grad.numpy(), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(db, b.grad.numpy(), rtol=1e-11, atol=1e-12)
+
+
+# ----------------------------------------------------------------------------- whole layer
+def _torch_bert_layer(x, p, heads, eps):
+    """An independent restatement with torch library calls (F.linear, F.softmax, F.layer_norm, F.gelu)."""
+    t = {k: torch.tensor(v, requires_grad=True) for k, v in p.items()}
+    xt = torch.tensor(x, requires_grad=True)
+    bsz, seq, hid = x.shape
+    d = hid // heads
+
+    def split(v):
+        return v.view(bsz, seq, heads, d).permute(0, 2, 1, 3)
+
+    q, k, v = (split(F.linear(xt, t[n + "_w"], t[n + "_b"])) for n in "qkv")
+    probs = F.softmax(q @ k.transpose(-1, -2) / math.sqrt(d), dim=-1)
+    ctx = (probs @ v).permute(0, 2, 1, 3).reshape(bsz, seq, hid)
+    h1 = F.layer_norm(F.linear(ctx, t["o_w"], t["o_b"]) + xt, (hid, ), t["ln1_g"], t["ln1_b"], eps)
+    act = F.gelu(F.linear(h1, t["ffn1_w"], t["ffn1_b"]))
+    y = F.layer_norm(F.linear(act, t["ffn2_w"], t["ffn2_b"]) + h1, (hid, ), t["ln2_g"], t["ln2_b"], eps)
+    return xt, t, y
+
+
+def test_bert_layer_forward_backward_matches_torch():
+    b, s, h, heads, ffn = 2, 12, 32, 4, 64
+    p = OB.init_params(h, ffn, 3, np.float64, bias_std=0.05)
+    r = rng(38)
+    p["ln1_g"], p["ln2_g"] = r.uniform(0.5, 1.5, h), r.uniform(0.5, 1.5, h)
+    p["ln1_b"], p["ln2_b"] = r.standard_normal(h) * 0.1, r.standard_normal(h) * 0.1
+    x, dy = r.standard_normal((b, s, h)), r.standard_normal((b, s, h))
+    y, saved = OB.forward(x, p, heads, eps=1e-5, keep=True)
+    grads = OB.backward(x, p, heads, dy, saved, eps=1e-5)
+    xt, t, yt = _torch_bert_layer(x, p, heads, 1e-5)
+    np.testing.assert_allclose(y, yt.detach().numpy(), rtol=1e-10, atol=1e-12)
+    yt.backward(torch.tensor(dy))
+    np.testing.assert_allclose(grads["x"], xt.grad.numpy(), rtol=1e-8, atol=1e-11)
+    for n in OB.PARAM_NAMES:
+        np.testing.assert_allclose(grads[n], t[n].grad.numpy(), rtol=1e-8, atol=1e-10, err_msg=n)
+
+
+def test_bert_layer_matches_huggingface_bertlayer():
+    """The module the reference's own integration test runs (tests/torch/test_bert_encoder.py:13-19),
+    built from a local config (nothing is downloaded)."""
+    transformers = pytest.importorskip("transformers")
+    try:
+        from transformers.models.bert.modeling_bert import BertConfig, BertLayer
+    except Exception as e:  # pragma: no cover
+        pytest.skip("BertLayer not importable: %s" % e)
+    b, s, h, heads, ffn = 2, 10, 32, 4, 64
+    cfg = BertConfig(hidden_size=h, num_attention_heads=heads, intermediate_size=ffn, hidden_dropout_prob=0.0,
+                     attention_probs_dropout_prob=0.0)
+    try:
+        cfg._attn_implementation = "eager"
+    except Exception:
+        pass
+    torch.manual_seed(0)
+    layer = BertLayer(cfg).double().eval()
+    sd = layer.state_dict()
+    p = {}
+    for long, short in (("attention.self.query", "q"), ("attention.self.key", "k"), ("attention.self.value", "v"),
+                        ("attention.output.dense", "o"), ("intermediate.dense", "ffn1"), ("output.dense", "ffn2")):
+        p[short + "_w"] = sd[long + ".weight"].numpy()
+        p[short + "_b"] = sd[long + ".bias"].numpy()
+    p["ln1_g"], p["ln1_b"] = sd["attention.output.LayerNorm.weight"].numpy(), sd["attention.output.LayerNorm.bias"].numpy()
+    p["ln2_g"], p["ln2_b"] = sd["output.LayerNorm.weight"].numpy(), sd["output.LayerNorm.bias"].numpy()
+    x = rng(39).standard_normal((b, s, h))
+    with torch.no_grad():
+        out = layer(torch.tensor(x))
+    out = out[0] if isinstance(out, (tuple, list)) else out
+    np.testing.assert_allclose(OB.forward(x, p, heads, eps=cfg.layer_norm_eps), out.numpy(), rtol=1e-9, atol=1e-11)
