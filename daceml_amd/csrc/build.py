@@ -21,6 +21,7 @@ SOURCES = [
     "reduce.hip",
     "transpose.hip",
     "gemm_f16.hip",
+    "gemm_f16_pipe.hip",
     "gemm_f32.hip",
     "conv.hip",
 ]

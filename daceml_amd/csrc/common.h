@@ -126,6 +126,23 @@ __global__ __launch_bounds__(1024) void reduce_partials_kernel(const float* __re
     }
 }
 
+// Same reduction for few, wide partial rows (split-K sums): every thread owns four consecutive columns
+// and walks the `parts` rows with 128-bit loads. Requires cols % 4 == 0 and 16-byte aligned rows.
+template <typename TOut>
+__global__ __launch_bounds__(256) void sum_partials_vec4_kernel(const float* __restrict__ part, TOut* __restrict__ out,
+                                                                int parts, int64_t row_stride, int64_t cols, float scale) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i * 4 < cols; i += stride) {
+        floatx4 acc = *reinterpret_cast<const floatx4*>(part + i * 4);
+        for (int p = 1; p < parts; ++p) {
+            const floatx4 v = *reinterpret_cast<const floatx4*>(part + (int64_t)p * row_stride + i * 4);
+            acc += v;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[i * 4 + e] = from_f32<TOut>(acc[e] * scale);
+    }
+}
+
 // ---------------------------------------------------------------- math
 // exact-GELU pieces; no fast-math anywhere on fp32 paths.
 __device__ __forceinline__ float gelu_f(float x) {

@@ -15,38 +15,11 @@
 // or row-contiguous (stride_m/n == 1, i.e. the transposed storage). The latter is transposed in
 // registers on the way to LDS: a thread loads eight K-rows of RU adjacent rows and re-packs them
 // into RU chunks of eight K values, so no separate transpose kernel or HBM round trip is needed.
-#include "common.h"
-
-#include <type_traits>
+#include "gemm_f16_common.h"
 
 namespace dml {
+using namespace gemm16;
 namespace {
-
-constexpr int kThreads = 256;
-constexpr int BK = 64;         // K elements per step
-constexpr int kRowBytes = BK * 2;
-constexpr int kXcds = 8;
-
-struct GemmArgs {
-    int m, n, k;
-    int64_t sam, sak, sbn, sbk, scm;
-    int batch1, batch2;  // extents of the two inner batch dims (outer one is implied)
-    int64_t sab[3], sbb[3], scb[3];
-    float alpha, beta;
-    int out_f32, bias_f32, act, bias_m, c_vec;
-    int tiles_m, tiles_n;
-    long long total_blocks;
-};
-
-template <int I, int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
-__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 
 // ---------------------------------------------------------------- global -> registers
 // The loaders are branch-free in the steady state. Rows past the end of the operand are clamped to
@@ -199,106 +172,6 @@ template <int R> struct LoaderSel<R, 0> { using type = LoaderKC<R>; };
 template <int R> struct LoaderSel<R, 1> { using type = LoaderRC<R>; };
 template <int R> struct LoaderSel<R, 2> { using type = LoaderGeneric<R>; };
 template <int R> struct LoaderSel<R, 3> { using type = LoaderKCDirect<R>; };
-
-// ---------------------------------------------------------------- epilogue helper
-// One wavefront writes a 32 x WN strip held in LDS (fp32, row pitch WN+4) to C: lane -> (row,
-// eight consecutive columns). v = alpha*acc + bias; pre_out = v; v = act(v) + residual + beta*C.
-// ACT = false compiles the activation switch out (most contractions have none).
-template <typename OutT> struct OutVec;
-template <> struct OutVec<_Float16> { typedef half8 type; };
-template <> struct OutVec<float> { typedef float type __attribute__((ext_vector_type(8))); };
-
-template <typename OutT, int WN, bool ACT>
-__device__ __forceinline__ void store_strip(const GemmArgs& g, void* c_ptr, void* pre_ptr, const void* res_ptr,
-                                            const void* bias_ptr, const float* strip, int mb, int nb, int64_t coff,
-                                            int lane) {
-    typedef typename OutVec<OutT>::type ovec;
-    constexpr int PITCH = WN + 4;
-    constexpr int CPR = WN / 8;
-    constexpr int ITER = 32 * CPR / kWave;
-    OutT* C = reinterpret_cast<OutT*>(c_ptr);
-    OutT* P = reinterpret_cast<OutT*>(pre_ptr);
-    const OutT* R = reinterpret_cast<const OutT*>(res_ptr);
-    // without an activation the body is small: unroll so that LDS reads and global stores of
-    // several rows overlap; with one, keep a single copy of the activation code
-#pragma unroll(ACT ? 2 : 4)
-    for (int it = 0; it < ITER; ++it) {
-        const int idx = it * kWave + lane;
-        const int r = idx / CPR, c8 = (idx % CPR) * 8;
-        const int m = mb + r, n = nb + c8;
-        if (m >= g.m || n >= g.n) continue;
-        const floatx4 lo = *reinterpret_cast<const floatx4*>(strip + r * PITCH + c8);
-        const floatx4 hi = *reinterpret_cast<const floatx4*>(strip + r * PITCH + c8 + 4);
-        float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        const int64_t off = coff + (int64_t)m * g.scm + n;
-        const bool full = g.c_vec && n + 8 <= g.n;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] *= g.alpha;
-        if (bias_ptr) {
-            if (g.bias_m) {
-                const float b = g.bias_f32 ? reinterpret_cast<const float*>(bias_ptr)[m]
-                                           : (float)reinterpret_cast<const _Float16*>(bias_ptr)[m];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] += b;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int ne = min(n + e, g.n - 1);
-                    v[e] += g.bias_f32 ? reinterpret_cast<const float*>(bias_ptr)[ne]
-                                       : (float)reinterpret_cast<const _Float16*>(bias_ptr)[ne];
-                }
-            }
-        }
-        if (full) {
-            if (P) {
-                ovec pv;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    pv[e] = (OutT)v[e];
-                    v[e] = (float)pv[e];  // the un-fused graph reads the stored pre-activation back
-                }
-                *reinterpret_cast<ovec*>(P + off) = pv;
-            }
-            if constexpr (ACT) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] = apply_act_half(g.act, v[e]);
-            }
-            if (R) {
-                const ovec rv = *reinterpret_cast<const ovec*>(R + off);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] += (float)rv[e];
-            }
-            if (g.beta != 0.f) {
-                const ovec cv = *reinterpret_cast<const ovec*>(C + off);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] += g.beta * (float)cv[e];
-            }
-            ovec ov;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) ov[e] = (OutT)v[e];
-            *reinterpret_cast<ovec*>(C + off) = ov;
-        } else {
-            // ragged or unaligned tail: element by element (rare; kept out of line by the branch)
-            const int cnt = min(8, g.n - n);
-            float x = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                if (e < cnt) {
-                    x = v[e];
-                    if (P) {
-                        const OutT h = (OutT)x;
-                        P[off + e] = h;
-                        x = (float)h;
-                    }
-                    if constexpr (ACT) x = apply_act_half(g.act, x);
-                    if (R) x += (float)R[off + e];
-                    if (g.beta != 0.f) x += g.beta * (float)C[off + e];
-                    C[off + e] = (OutT)x;
-                }
-            }
-        }
-    }
-}
 
 // ---------------------------------------------------------------- the kernel
 // AMODE / BMODE: 0 = K-contiguous via registers, 1 = row-contiguous, 2 = generic strides,
@@ -475,9 +348,6 @@ int launch_cfg(GemmArgs& g, const _Float16* pa, const _Float16* pb, void* pc, co
     DML_GEMM_CASE(0, 1)
     DML_GEMM_CASE(1, 0)
     DML_GEMM_CASE(1, 1)
-    DML_GEMM_CASE(3, 3)
-    DML_GEMM_CASE(3, 1)
-    DML_GEMM_CASE(1, 3)
     if constexpr (BM == 128 && BN == 128) {
         DML_GEMM_CASE(2, 2)
     }
@@ -567,17 +437,22 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
     int amode = d->k == 0 ? 0 : operand_mode(a, d->m, d->k, d->a_stride_m, d->a_stride_k, d->a_stride_batch, d->batch);
     int bmode = d->k == 0 ? 0 : operand_mode(b, d->n, d->k, d->b_stride_n, d->b_stride_k, d->b_stride_batch, d->batch);
     if (amode == 2 || bmode == 2) amode = bmode = 2;
-    // K-contiguous operands go straight to LDS when K is a whole number of steps; a K-contiguous
-    // operand paired with a register-path K-contiguous one keeps the register path for both.
-    if (d->k % BK == 0 && d->k > 0 && g_direct_lds) {
-        if (amode == 0 && bmode == 0) amode = bmode = 3;
-        else if (amode == 0 && bmode == 1) amode = 3;
-        else if (amode == 1 && bmode == 0) bmode = 3;
-    }
     hipStream_t st = (hipStream_t)stream;
 
     int cfg = g_force_cfg;
-    if (cfg < 0) {
+    // Both operands vector-loadable and K a whole number of steps: the fully pipelined kernel.
+    if (amode != 2 && d->k % BK == 0 && d->k > 0 && g_direct_lds) {
+        if (cfg < 0) {
+            auto blocks = [&](int bm, int bn) { return (long long)ceil_div(d->m, bm) * ceil_div(d->n, bn) * batch; };
+            // measured on MI355X: with more than one 128x128 tile per CU, two resident workgroups with
+            // two LDS stages each beat one workgroup with a deeper ring (and the 256-wide tiles)
+            if (blocks(128, 128) > 256) cfg = 3;
+            else cfg = 0;
+        }
+        return launch_pipelined(g, (const _Float16*)a, (const _Float16*)b, c, bias, residual, pre_out, amode == 1 ? 4 : 3,
+                                bmode == 1 ? 4 : 3, cfg, batch, st);
+    }
+    if (cfg < 0 || cfg > 2) {
         // Largest tile that still yields at least one workgroup per CU.
         auto blocks = [&](int bm, int bn) { return (long long)ceil_div(d->m, bm) * ceil_div(d->n, bn) * batch; };
         if (blocks(256, 256) >= 256) cfg = CFG_256x256;
@@ -633,6 +508,17 @@ int dmlhip_gemm_f16_ws(const dmlhip_gemm_desc* d, const void* a, const void* b, 
     // stage 2: sum the slices, scale by alpha, convert
     const int64_t cols = d->m * d->n;
     hipStream_t st = (hipStream_t)stream;
+    if (cols % 4 == 0) {
+        int64_t blocks = ceil_div(cols / 4, 256);
+        if (blocks > 256 * 16) blocks = 256 * 16;
+        if (d->out_dtype == DMLHIP_F32)
+            hipLaunchKernelGGL((sum_partials_vec4_kernel<float>), (unsigned)blocks, 256, 0, st, (const float*)workspace,
+                               (float*)c, s, cols, cols, d->alpha);
+        else
+            hipLaunchKernelGGL((sum_partials_vec4_kernel<_Float16>), (unsigned)blocks, 256, 0, st,
+                               (const float*)workspace, (_Float16*)c, s, cols, cols, d->alpha);
+        return launch_status("gemm_f16(split-K sum)");
+    }
     const unsigned grid = (unsigned)ceil_div(cols, kWave);
     if (d->out_dtype == DMLHIP_F32)
         hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, (const float*)workspace, (float*)c,

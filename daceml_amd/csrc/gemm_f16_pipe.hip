@@ -1,0 +1,326 @@
+// Fully pipelined fp16 MFMA GEMM: both operands stream from global memory straight into a ring of
+// NSTAGE LDS tiles (global_load_lds, 16 bytes per lane, no staging registers, no LDS store
+// instructions), with loads for tile t+NSTAGE-1 in flight while tile t is multiplied. Waiting is
+// explicit: s_waitcnt vmcnt(n) lets the newest NSTAGE-2 tiles stay outstanding across the barrier
+// that publishes tile t+1.
+//
+// Operand kinds
+//   KC  K-contiguous (stride_k == 1): LDS tile [rows][64 k], 128-byte rows, 16-byte chunk c of row r at
+//       slot c ^ ((r ^ r>>3) & 7); fragments are ds_read_b128.
+//   RC  row-contiguous (stride_row == 1, the transposed storage): LDS tile [64 k][rows], chunk (8 rows)
+//       c of K row k at slot c ^ ((k & 3) << 2); fragments are two ds_read_b64_tr_b16 — the LDS
+//       transpose read of gfx950 hands every lane four consecutive k of its row, which is exactly the
+//       MFMA operand layout, so no transpose is done in registers or in a separate pass.
+// Requirements (checked by the host): K % 64 == 0, 16-byte aligned bases and strides, rows % 8 == 0
+// for RC operands, 32-bit element offsets.
+#include "gemm_f16_common.h"
+
+namespace dml {
+namespace gemm16 {
+namespace {
+
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void lds_dma16(const _Float16* gptr, char* lds_dst) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gptr,
+                                     (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
+}
+
+// ---------------------------------------------------------------- LDS reads
+// Fragment reads are issued as inline assembly so that the compiler neither guesses at aliasing
+// between them and the in-flight global->LDS transfers (it would wait for *all* transfers before a
+// transpose read) nor places the waits: the kernel waits explicitly (lgkmcnt / vmcnt counters).
+template <int OFFSET>
+__device__ __forceinline__ half8 lds_read_b128(uint32_t addr) {
+    half8 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+
+template <int OFFSET>
+__device__ __forceinline__ half4v lds_read_tr16_b64(uint32_t addr) {
+    half4v v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+
+template <int N>
+__device__ __forceinline__ void wait_lgkm() {
+    static_assert(N >= 0 && N <= 15, "lgkmcnt is a 4-bit counter");
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int VM>
+__device__ __forceinline__ void wait_vm_lgkm0() {
+    static_assert(VM >= 0 && VM <= 63, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(VM) : "memory");
+}
+
+// ---------------------------------------------------------------- operand streams
+// A stream owns one operand: where each lane's 16-byte DMA pieces come from, and where each lane
+// reads its MFMA fragments. `T` = number of 32-row MFMA blocks this wavefront multiplies.
+template <int R, int KIND, int T> struct Stream;
+
+template <int R, int T>
+struct Stream<R, 0, T> {  // K-contiguous: tile [R][64 k], chunk c of row r at slot c ^ (r & 7)
+    static constexpr int N = R / 32;   // DMA instructions per wavefront per tile
+    static constexpr int READS = T;    // LDS read instructions per K sub-step
+    int off[N];
+    uint32_t faddr[4];                 // fragment address of block 0 for each K sub-step (stage 0)
+    __device__ __forceinline__ void init(int64_t s_row, int64_t, int row0, int rows, int wave, int lane, int wrow0,
+                                         uint32_t tile0) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int r = (i * 4 + wave) * 8 + (lane >> 3);
+            const int c = (lane & 7) ^ (r & 7);
+            off[i] = (int)(min(row0 + r, rows - 1) * s_row) + c * 8;
+        }
+        const int r = wrow0 + (lane & 31);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+            faddr[kk] = tile0 + r * kRowBytes + ((((kk * 2 + (lane >> 5))) ^ (r & 7)) << 4);
+    }
+    __device__ __forceinline__ void issue(const _Float16* base, int64_t, int k0, char* tile, int wave) const {
+#pragma unroll
+        for (int i = 0; i < N; ++i) lds_dma16(base + off[i] + k0, tile + (i * 4 + wave) * 1024);
+    }
+    template <int KK>
+    __device__ __forceinline__ void frags(uint32_t stage_off, half8 (&f)[T]) const {
+        const uint32_t a = faddr[KK] + stage_off;
+        static_for<0, T>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            f[i] = lds_read_b128<i * 32 * kRowBytes>(a);
+        });
+    }
+};
+
+template <int R, int T>
+struct Stream<R, 1, T> {  // row-contiguous: tile [64 k][R], chunk c (8 rows) of K row k at slot c ^ ((k & 3) << 2)
+    static constexpr int N = R / 32;
+    static constexpr int P = R * 2;    // bytes per K row of the tile
+    static constexpr int READS = 2 * T;
+    int off[N];
+    uint32_t faddr[T];                 // per 32-row block: address of this lane's first transpose read (stage 0)
+    __device__ __forceinline__ void init(int64_t, int64_t s_k, int row0, int rows, int wave, int lane, int wrow0,
+                                         uint32_t tile0) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int o = (i * 4 + wave) * 1024 + lane * 16;
+            const int kl = o / P, pos = (o % P) >> 4;
+            const int cidx = pos ^ ((kl & 3) << 2);
+            off[i] = (int)(kl * s_k) + min(row0 + cidx * 8, rows - 8);
+        }
+        // transpose read: the 16 lanes of group G = l/16 jointly read K rows kq..kq+3 of 16 tile rows; lane
+        // s = l%16 points at K row s/4, rows 4*(s%4)..+3 of them, and receives four consecutive K of row s.
+        // G%2 picks the 16-row half of the 32-row block, G/2 the K half of the 16-k sub-step.
+        const int s = lane & 15, grp = lane >> 4;
+        const int kq = (grp >> 1) * 8 + (s >> 2);
+#pragma unroll
+        for (int i = 0; i < T; ++i) {
+            const int row = wrow0 + i * 32 + (grp & 1) * 16 + 4 * (s & 3);
+            faddr[i] = tile0 + kq * P + (((row >> 3) ^ ((kq & 3) << 2)) << 4) + (row & 7) * 2;
+        }
+    }
+    __device__ __forceinline__ void issue(const _Float16* base, int64_t s_k, int k0, char* tile, int wave) const {
+        const _Float16* p = base + (int64_t)k0 * s_k;
+#pragma unroll
+        for (int i = 0; i < N; ++i) lds_dma16(p + off[i], tile + (i * 4 + wave) * 1024);
+    }
+    template <int KK>
+    __device__ __forceinline__ void frags(uint32_t stage_off, half8 (&f)[T]) const {
+        static_for<0, T>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            const uint32_t a = faddr[i] + stage_off;
+            const half4v lo = lds_read_tr16_b64<KK * 16 * P>(a);
+            const half4v hi = lds_read_tr16_b64<KK * 16 * P + 4 * P>(a);
+            f[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        });
+    }
+};
+
+// ---------------------------------------------------------------- kernel
+template <int BM, int BN, int WM, int WN, int AKIND, int BKIND, int NSTAGE, bool ACT>
+__global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16* __restrict__ a_ptr,
+                                                                 const _Float16* __restrict__ b_ptr, void* c_ptr,
+                                                                 const void* bias_ptr, const void* res_ptr,
+                                                                 void* pre_ptr, const GemmArgs g) {
+    static_assert((BM / WM) * (BN / WN) == kThreads / kWave, "four wavefronts per workgroup");
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes, STAGE = A_BYTES + B_BYTES;
+    constexpr int LPT = BM / 32 + BN / 32;  // DMA instructions per wavefront per tile
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+
+    long long bid = blockIdx.x;
+    {
+        const long long total = g.total_blocks;
+        const long long xcd = bid % kXcds, idx = bid / kXcds;
+        const long long base = total / kXcds, rem = total % kXcds;
+        bid = xcd * base + (xcd < rem ? xcd : rem) + idx;
+    }
+    const int tiles = g.tiles_m * g.tiles_n;
+    const long long batch = bid / tiles;
+    const int tile = (int)(bid % tiles);
+    const int tm = tile / g.tiles_n, tn = tile % g.tiles_n;
+    const int z2 = (int)(batch % g.batch2);
+    const int z1 = (int)((batch / g.batch2) % g.batch1);
+    const int z0 = (int)(batch / ((long long)g.batch2 * g.batch1));
+    const _Float16* A = a_ptr + z0 * g.sab[0] + z1 * g.sab[1] + z2 * g.sab[2];
+    const _Float16* B = b_ptr + z0 * g.sbb[0] + z1 * g.sbb[1] + z2 * g.sbb[2];
+    const int64_t coff = z0 * g.scb[0] + z1 * g.scb[1] + z2 * g.scb[2];
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int wm = wave / (BN / WN), wn = wave % (BN / WN);
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+    Stream<BM, AKIND, TM> sa;
+    Stream<BN, BKIND, TN> sb;
+    sa.init(g.sam, g.sak, m0, g.m, wave, lane, wm * WM, lds0);
+    sb.init(g.sbn, g.sbk, n0, g.n, wave, lane, wn * WN, lds0 + A_BYTES);
+    constexpr int READS = Stream<BM, AKIND, TM>::READS + Stream<BN, BKIND, TN>::READS;
+    constexpr int READS_W = READS > 15 ? 15 : READS;  // lgkmcnt saturates at 15: waiting for one more is harmless
+
+    const int nk = g.k / BK;
+    // prologue: tiles 0 .. NSTAGE-2 in flight
+#pragma unroll
+    for (int s = 0; s < NSTAGE - 1; ++s) {
+        if (s < nk) {
+            sa.issue(A, g.sak, s * BK, lds + s * STAGE, wave);
+            sb.issue(B, g.sbk, s * BK, lds + s * STAGE + A_BYTES, wave);
+        }
+    }
+    if (nk >= NSTAGE - 1) wait_vm_lgkm0<(NSTAGE - 2) * LPT>();
+    else wait_vm_lgkm0<0>();
+    __builtin_amdgcn_s_barrier();
+
+    half8 af[2][TM], bf[2][TN];
+    if (nk > 0) {
+        sa.template frags<0>(0u, af[0]);
+        sb.template frags<0>(0u, bf[0]);
+    }
+
+    int cur_stage = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        const uint32_t cur_off = (uint32_t)cur_stage * STAGE;
+        const int nxt_stage = cur_stage + 1 == NSTAGE ? 0 : cur_stage + 1;
+        // the stage that held tile kt-1 is free (every wavefront passed the barrier of step kt-1 after
+        // its last read of it had completed): refill it with tile kt+NSTAGE-1
+        const int fill = kt + NSTAGE - 1;
+        if (fill < nk) {
+            const int fs = cur_stage == 0 ? NSTAGE - 1 : cur_stage - 1;
+            sa.issue(A, g.sak, fill * BK, lds + fs * STAGE, wave);
+            sb.issue(B, g.sbk, fill * BK, lds + fs * STAGE + A_BYTES, wave);
+        }
+        const bool more = kt + 1 < nk;
+        static_for<0, BK / 16>([&](auto kc) {
+            constexpr int kk = decltype(kc)::value;
+            constexpr int nb = (kk + 1) & 1;
+            if constexpr (kk + 1 < BK / 16) {
+                // fragments of the next sub-step, then wait for everything older than them
+                sa.template frags<kk + 1>(cur_off, af[nb]);
+                sb.template frags<kk + 1>(cur_off, bf[nb]);
+                wait_lgkm<READS_W>();
+            } else {
+                // last sub-step: its fragments are the only reads outstanding. Tile kt+1 must have
+                // landed for every wavefront before anybody reads it.
+                if (fill < nk) wait_vm_lgkm0<(NSTAGE - 2) * LPT>();
+                else wait_vm_lgkm0<0>();
+                __builtin_amdgcn_s_barrier();
+                if (more) {
+                    sa.template frags<0>((uint32_t)nxt_stage * STAGE, af[0]);
+                    sb.template frags<0>((uint32_t)nxt_stage * STAGE, bf[0]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[kk & 1][i], bf[kk & 1][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        cur_stage = nxt_stage;
+    }
+    wait_vm_lgkm0<0>();
+    __syncthreads();
+
+    // ---- epilogue (see store_strip): 32 x WN strips through this wavefront's LDS region
+    constexpr int PITCH = WN + 4;
+    float* strip = reinterpret_cast<float*>(lds) + wave * 32 * PITCH;
+    const int ncol = lane & 31, mgrp = lane >> 5;
+    static_for<0, TM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        static_for<0, TN>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                strip[((e >> 2) * 8 + mgrp * 4 + (e & 3)) * PITCH + j * 32 + ncol] = acc[i][j][e];
+        });
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int mb = m0 + wm * WM + i * 32, nb = n0 + wn * WN;
+        if (g.out_f32) store_strip<float, WN, ACT>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, strip, mb, nb, coff, lane);
+        else store_strip<_Float16, WN, ACT>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, strip, mb, nb, coff, lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    });
+}
+
+template <int BM, int BN, int WM, int WN, int NSTAGE>
+int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, const void* bias, const void* res, void* pre,
+                int akind, int bkind, long long batch, hipStream_t st) {
+    g.tiles_m = (g.m + BM - 1) / BM;
+    g.tiles_n = (g.n + BN - 1) / BN;
+    const long long total = (long long)g.tiles_m * g.tiles_n * batch;
+    DML_REQUIRE(total <= 2147483647LL, DMLHIP_ERR_SHAPE, "gemm_f16: %lld workgroups exceed the grid limit", total);
+    g.total_blocks = total;
+    size_t lds = (size_t)NSTAGE * (BM + BN) * kRowBytes;
+    const size_t epi = (size_t)4 * 32 * (WN + 4) * sizeof(float);
+    if (lds < epi) lds = epi;
+#define DML_PIPE_CASE(AK, BKD, ACTV)                                                                          \
+    if (akind == AK && bkind == BKD && (g.act != DMLHIP_ACT_NONE) == ACTV) {                                  \
+        auto kern = gemm_f16_pipe_kernel<BM, BN, WM, WN, AK, BKD, NSTAGE, ACTV>;                              \
+        if (lds > 64 * 1024) {                                                                                \
+            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                               (int)lds);                                                     \
+            if (e != hipSuccess) {                                                                            \
+                set_error("gemm_f16: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));        \
+                return (int)e;                                                                                \
+            }                                                                                                 \
+        }                                                                                                     \
+        hipLaunchKernelGGL(kern, (unsigned)total, kThreads, lds, st, a, b, c, bias, res, pre, g);             \
+        return launch_status("gemm_f16(pipelined)");                                                          \
+    }
+    DML_PIPE_CASE(0, 0, false) DML_PIPE_CASE(0, 1, false) DML_PIPE_CASE(1, 0, false) DML_PIPE_CASE(1, 1, false)
+    DML_PIPE_CASE(0, 0, true) DML_PIPE_CASE(0, 1, true) DML_PIPE_CASE(1, 0, true) DML_PIPE_CASE(1, 1, true)
+#undef DML_PIPE_CASE
+    set_error("gemm_f16: no pipelined kernel for operand kinds %d/%d", akind, bkind);
+    return DMLHIP_ERR_UNSUPPORTED;
+}
+
+}  // namespace
+
+int launch_pipelined(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, const void* bias, const void* residual,
+                     void* pre, int amode, int bmode, int cfg, long long batch, hipStream_t st) {
+    const int ak = amode == 4 ? 1 : 0, bk = bmode == 4 ? 1 : 0;
+    switch (cfg) {
+        case 2: return launch_tile<256, 256, 128, 128, 2>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+        case 1: return launch_tile<256, 128, 128, 64, 3>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+        case 3: return launch_tile<128, 128, 64, 64, 2>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+        default: return launch_tile<128, 128, 64, 64, 4>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+    }
+}
+
+}  // namespace gemm16
+}  // namespace dml

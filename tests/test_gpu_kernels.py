@@ -267,7 +267,7 @@ GEMM_CASES = [
 ]
 
 
-@pytest.mark.parametrize("cfg", [-1, 0, 1, 2])
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3])
 @pytest.mark.parametrize("eq,sa,sb", GEMM_CASES)
 def test_einsum_f16(cfg, eq, sa, sb):
     from daceml_amd import kernels as K
