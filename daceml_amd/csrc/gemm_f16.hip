@@ -286,32 +286,29 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(const _Float16* __re
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[kk & 1][i], bf[kk & 1][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][j], af[kk & 1][i], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
     __syncthreads();
 
-    // ---- epilogue. acc[i][j][e] is C[m, n] with n = l%32 and m = (e/4)*8 + (l/32)*4 + e%4 inside
-    // the 32x32 block. Each wavefront stages one 32 x WN strip at a time in its own LDS region and
-    // reads it back row-wise, so that global accesses are 128-bit and contiguous along n.
+    // ---- epilogue. With the swapped MFMA operands acc[i][j][e] is C[m, n] with m = l%32 and
+    // n = (e/4)*8 + (l/32)*4 + e%4 inside the 32x32 block. Each wavefront stages one 32 x WN strip at a
+    // time in its own LDS region and reads it back row-wise, so that global accesses are 128-bit and
+    // contiguous along n.
     constexpr int PITCH = WN + 4;
     float* strip = reinterpret_cast<float*>(lds) + wave * 32 * PITCH;
-    const int ncol = lane & 31, mgrp = lane >> 5;
+    float bias_n[8];
+    load_bias_n<WN>(g, bias_ptr, n0 + wn * WN, lane, bias_n);
     static_for<0, TM>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        static_for<0, TN>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-#pragma unroll
-            for (int e = 0; e < 16; ++e)
-                strip[((e >> 2) * 8 + mgrp * 4 + (e & 3)) * PITCH + j * 32 + ncol] = acc[i][j][e];
-        });
+        stage_strip<TN, PITCH>(strip, acc[i], lane);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         const int mb = m0 + wm * WM + i * 32, nb = n0 + wn * WN;
-        if (g.out_f32) store_strip<float, WN, ACT>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, strip, mb, nb, coff, lane);
-        else store_strip<_Float16, WN, ACT>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, strip, mb, nb, coff, lane);
+        if (g.out_f32) store_strip<float, WN, ACT ? EPI_GENERAL_ACT : EPI_GENERAL>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, bias_n, strip, mb, nb, coff, lane);
+        else store_strip<_Float16, WN, ACT ? EPI_GENERAL_ACT : EPI_GENERAL>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, bias_n, strip, mb, nb, coff, lane);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     });
@@ -441,7 +438,8 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
 
     int cfg = g_force_cfg;
     // Both operands vector-loadable and K a whole number of steps: the fully pipelined kernel.
-    if (amode != 2 && d->k % BK == 0 && d->k > 0 && g_direct_lds) {
+    if (amode != 2 && d->k % BK == 0 && d->k > 0 && g_direct_lds &&
+        epilogue_kind(g, bias, residual, pre_out) != EPI_GENERAL_ACT) {
         if (cfg < 0) {
             auto blocks = [&](int bm, int bn) { return (long long)ceil_div(d->m, bm) * ceil_div(d->n, bn) * batch; };
             // measured on MI355X: with more than one 128x128 tile per CU, two resident workgroups with

@@ -34,8 +34,27 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+__device__ __forceinline__ int swz16(int row) { return (row & 7) ^ ((row >> 3) & 1); }  // period 16 rows
 
-// ---------------------------------------------------------------- epilogue helper
+// ---------------------------------------------------------------- epilogue helpers
+// The kernels issue the MFMA with the operands swapped (B fragment first): a lane then holds, for the
+// output row m = lane % 32 of a 32x32 block, the columns n = 8*(e/4) + 4*(lane/32) + e%4 — four
+// consecutive columns per group of four accumulator registers, which go to the LDS strip as one
+// 128-bit write. PITCH = WN + 4 floats keeps both these writes and the row-wise reads of store_strip
+// free of bank conflicts.
+template <int TN, int PITCH>
+__device__ __forceinline__ void stage_strip(float* strip, const floatx16 (&acc)[TN], int lane) {
+    float* row = strip + (lane & 31) * PITCH + (lane >> 5) * 4;
+    static_for<0, TN>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            floatx4 v = {acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]};
+            *reinterpret_cast<floatx4*>(row + j * 32 + q * 8) = v;
+        }
+    });
+}
+
 // One wavefront writes a 32 x WN strip held in LDS (fp32, row pitch WN+4) to C: lane -> (row,
 // eight consecutive columns). v = alpha*acc + bias; pre_out = v; v = act(v) + residual + beta*C.
 // ACT = false compiles the activation switch out (most contractions have none).
@@ -43,114 +62,158 @@ template <typename OutT> struct OutVec;
 template <> struct OutVec<_Float16> { typedef half8 type; };
 template <> struct OutVec<float> { typedef float type __attribute__((ext_vector_type(8))); };
 
-template <typename OutT, int WN, bool ACT>
+// Epilogue variants (template parameter EPI), chosen on the host so that the common cases carry no
+// loads inside the store loop: on this target loads and stores share one completion counter and
+// complete out of order with respect to each other, so any wait for a load also waits for every
+// store issued before it (a full write round trip per iteration).
+//   EPI_PLAIN    v = alpha*acc + bias[n]                       -> C
+//   EPI_ACT      same, pre_out = v, v = act(v)                 -> C (and pre-activation)   no loads
+//   EPI_GENERAL  + bias along m, residual, beta*C               (loads per strip, issued before the stores)
+//   EPI_GENERAL_ACT  EPI_GENERAL with the activation switch compiled in
+constexpr int EPI_PLAIN = 0, EPI_ACT = 1, EPI_GENERAL = 2, EPI_GENERAL_ACT = 3;
+
+inline int epilogue_kind(const GemmArgs& g, const void* bias, const void* residual, const void* pre) {
+    const bool loads = residual || g.beta != 0.f || (bias && g.bias_m);
+    const bool act = g.act != DMLHIP_ACT_NONE;
+    if (loads) return act ? EPI_GENERAL_ACT : EPI_GENERAL;
+    return (act || pre) ? EPI_ACT : EPI_PLAIN;
+}
+
+// The eight column-bias values of a lane (its columns are the same for every strip of the wavefront's tile, so
+// this runs once, before the first store).
+template <int WN>
+__device__ __forceinline__ void load_bias_n(const GemmArgs& g, const void* bias_ptr, int nb, int lane, float (&bias_n)[8]) {
+    constexpr int CPR = WN / 8;
+    const int n = nb + (lane % CPR) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) bias_n[e] = 0.f;
+    if (!bias_ptr || g.bias_m || n >= g.n) return;
+    if (n + 8 <= g.n && ((reinterpret_cast<uintptr_t>(bias_ptr) + (size_t)n * (g.bias_f32 ? 4 : 2)) & 15) == 0) {
+        if (g.bias_f32) {
+            const floatx4 b0 = *reinterpret_cast<const floatx4*>(reinterpret_cast<const float*>(bias_ptr) + n);
+            const floatx4 b1 = *reinterpret_cast<const floatx4*>(reinterpret_cast<const float*>(bias_ptr) + n + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { bias_n[e] = b0[e]; bias_n[e + 4] = b1[e]; }
+        } else {
+            const half8 b = *reinterpret_cast<const half8*>(reinterpret_cast<const _Float16*>(bias_ptr) + n);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) bias_n[e] = (float)b[e];
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int ne = min(n + e, g.n - 1);
+            bias_n[e] = g.bias_f32 ? reinterpret_cast<const float*>(bias_ptr)[ne]
+                                   : (float)reinterpret_cast<const _Float16*>(bias_ptr)[ne];
+        }
+    }
+}
+
+template <typename OutT, int WN, int EPI>
 __device__ __forceinline__ void store_strip(const GemmArgs& g, void* c_ptr, void* pre_ptr, const void* res_ptr,
-                                            const void* bias_ptr, const float* strip, int mb, int nb, int64_t coff,
-                                            int lane) {
+                                            const void* bias_ptr, const float (&bias_n)[8], const float* strip, int mb,
+                                            int nb, int64_t coff, int lane) {
     typedef typename OutVec<OutT>::type ovec;
     constexpr int PITCH = WN + 4;
     constexpr int CPR = WN / 8;
     constexpr int ITER = 32 * CPR / kWave;
+    constexpr int RSTEP = kWave / CPR;  // rows between two iterations of a lane
+    constexpr bool ACT = EPI == EPI_ACT || EPI == EPI_GENERAL_ACT;
+    constexpr bool GENERAL = EPI == EPI_GENERAL || EPI == EPI_GENERAL_ACT;
     OutT* C = reinterpret_cast<OutT*>(c_ptr);
     OutT* P = reinterpret_cast<OutT*>(pre_ptr);
     const OutT* R = reinterpret_cast<const OutT*>(res_ptr);
-    // A lane keeps its eight columns for the whole strip (64 % CPR == 0): the column bias is loaded once,
-    // as one 128-bit access when it is aligned.
-    float bias_n[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (bias_ptr && !g.bias_m) {
-        const int n = nb + (lane % CPR) * 8;
-        if (n + 8 <= g.n && ((reinterpret_cast<uintptr_t>(bias_ptr) + (size_t)n * (g.bias_f32 ? 4 : 2)) & 15) == 0) {
-            if (g.bias_f32) {
-                const floatx4 b0 = *reinterpret_cast<const floatx4*>(reinterpret_cast<const float*>(bias_ptr) + n);
-                const floatx4 b1 = *reinterpret_cast<const floatx4*>(reinterpret_cast<const float*>(bias_ptr) + n + 4);
+    // A lane keeps its eight columns for the whole strip (64 % CPR == 0).
+    const int r0 = lane / CPR, c8 = (lane % CPR) * 8;
+    const int n = nb + c8;
+    if (n >= g.n) return;
+    const bool full = g.c_vec && n + 8 <= g.n;
+    const int64_t off0 = coff + (int64_t)(mb + r0) * g.scm + n;
+    const int64_t rstep = (int64_t)RSTEP * g.scm;
+
+    if (full) {
+        // operands that have to be loaded (general variants only): all of the strip's loads first
+        ovec rv[GENERAL ? ITER : 1], cv[GENERAL ? ITER : 1];
+        float bm[GENERAL ? ITER : 1];
+        if constexpr (GENERAL) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { bias_n[e] = b0[e]; bias_n[e + 4] = b1[e]; }
-            } else {
-                const half8 b = *reinterpret_cast<const half8*>(reinterpret_cast<const _Float16*>(bias_ptr) + n);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) bias_n[e] = (float)b[e];
-            }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int ne = min(n + e, g.n - 1);
-                if (n < g.n) bias_n[e] = g.bias_f32 ? reinterpret_cast<const float*>(bias_ptr)[ne]
-                                                     : (float)reinterpret_cast<const _Float16*>(bias_ptr)[ne];
-            }
-        }
-    }
-    // without an activation the body is small: unroll so that LDS reads and global stores of
-    // several rows overlap; with one, keep few copies of the activation code
-#pragma unroll(ACT ? 2 : 4)
-    for (int it = 0; it < ITER; ++it) {
-        const int idx = it * kWave + lane;
-        const int r = idx / CPR, c8 = (idx % CPR) * 8;
-        const int m = mb + r, n = nb + c8;
-        if (m >= g.m || n >= g.n) continue;
-        const floatx4 lo = *reinterpret_cast<const floatx4*>(strip + r * PITCH + c8);
-        const floatx4 hi = *reinterpret_cast<const floatx4*>(strip + r * PITCH + c8 + 4);
-        float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        const int64_t off = coff + (int64_t)m * g.scm + n;
-        const bool full = g.c_vec && n + 8 <= g.n;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] *= g.alpha;
-        if (bias_ptr) {
-            if (g.bias_m) {
-                const float b = g.bias_f32 ? reinterpret_cast<const float*>(bias_ptr)[m]
-                                           : (float)reinterpret_cast<const _Float16*>(bias_ptr)[m];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] += b;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] += bias_n[e];
+            for (int it = 0; it < ITER; ++it) {
+                const int m = min(mb + r0 + it * RSTEP, g.m - 1);
+                const int64_t off = coff + (int64_t)m * g.scm + n;
+                if (R) rv[it] = *reinterpret_cast<const ovec*>(R + off);
+                if (g.beta != 0.f) cv[it] = *reinterpret_cast<const ovec*>(C + off);
+                bm[it] = 0.f;
+                if (bias_ptr && g.bias_m)
+                    bm[it] = g.bias_f32 ? reinterpret_cast<const float*>(bias_ptr)[m]
+                                        : (float)reinterpret_cast<const _Float16*>(bias_ptr)[m];
             }
         }
-        if (full) {
-            if (P) {
-                ovec pv;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    pv[e] = (OutT)v[e];
-                    v[e] = (float)pv[e];  // the un-fused graph reads the stored pre-activation back
+        for (int it = 0; it < ITER; ++it) {
+            const int r = r0 + it * RSTEP;
+            if (mb + r >= g.m) break;
+            const floatx4 lo = *reinterpret_cast<const floatx4*>(strip + r * PITCH + c8);
+            const floatx4 hi = *reinterpret_cast<const floatx4*>(strip + r * PITCH + c8 + 4);
+            float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            const int64_t off = off0 + it * rstep;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = v[e] * g.alpha + bias_n[e];
+            if constexpr (GENERAL) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += bm[it];
+            }
+            if constexpr (EPI != EPI_PLAIN) {
+                if (P) {
+                    ovec pv;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        pv[e] = (OutT)v[e];
+                        v[e] = (float)pv[e];  // the un-fused graph reads the stored pre-activation back
+                    }
+                    *reinterpret_cast<ovec*>(P + off) = pv;
                 }
-                *reinterpret_cast<ovec*>(P + off) = pv;
             }
             if constexpr (ACT) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] = apply_act_half(g.act, v[e]);
             }
-            if (R) {
-                const ovec rv = *reinterpret_cast<const ovec*>(R + off);
+            if constexpr (GENERAL) {
+                if (R) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] += (float)rv[e];
-            }
-            if (g.beta != 0.f) {
-                const ovec cv = *reinterpret_cast<const ovec*>(C + off);
+                    for (int e = 0; e < 8; ++e) v[e] += (float)rv[it][e];
+                }
+                if (g.beta != 0.f) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] += g.beta * (float)cv[e];
+                    for (int e = 0; e < 8; ++e) v[e] += g.beta * (float)cv[it][e];
+                }
             }
             ovec ov;
 #pragma unroll
             for (int e = 0; e < 8; ++e) ov[e] = (OutT)v[e];
             *reinterpret_cast<ovec*>(C + off) = ov;
-        } else {
-            // ragged or unaligned tail: element by element (rare; kept out of line by the branch)
-            const int cnt = min(8, g.n - n);
-            float x = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                if (e < cnt) {
-                    x = v[e];
-                    if (P) {
-                        const OutT h = (OutT)x;
-                        P[off + e] = h;
-                        x = (float)h;
-                    }
-                    if constexpr (ACT) x = apply_act_half(g.act, x);
-                    if (R) x += (float)R[off + e];
-                    if (g.beta != 0.f) x += g.beta * (float)C[off + e];
-                    C[off + e] = (OutT)x;
+        }
+    } else {
+        // ragged or unaligned columns: element by element (rare)
+        const int cnt = min(8, g.n - n);
+        for (int it = 0; it < ITER; ++it) {
+            const int r = r0 + it * RSTEP, m = mb + r;
+            if (m >= g.m) break;
+            const int64_t off = off0 + it * rstep;
+            float bmv = 0.f;
+            if (bias_ptr && g.bias_m)
+                bmv = g.bias_f32 ? reinterpret_cast<const float*>(bias_ptr)[m]
+                                 : (float)reinterpret_cast<const _Float16*>(bias_ptr)[m];
+            for (int e = 0; e < cnt; ++e) {
+                float x = strip[r * PITCH + c8 + e] * g.alpha + bias_n[e] + bmv;
+                if (P) {
+                    const OutT h = (OutT)x;
+                    P[off + e] = h;
+                    x = (float)h;
                 }
+                if (g.act != DMLHIP_ACT_NONE) x = apply_act_half(g.act, x);
+                if (R) x += (float)R[off + e];
+                if (g.beta != 0.f) x += g.beta * (float)C[off + e];
+                C[off + e] = (OutT)x;
             }
         }
     }

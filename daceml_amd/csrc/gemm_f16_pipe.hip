@@ -6,7 +6,9 @@
 //
 // Operand kinds
 //   KC  K-contiguous (stride_k == 1): LDS tile [rows][64 k], 128-byte rows, 16-byte chunk c of row r at
-//       slot c ^ ((r ^ r>>3) & 7); fragments are ds_read_b128.
+//       slot c ^ (r & 7) ^ (r>>3 & 1) (rows r and r+8 share a bank window, the second term separates them;
+//       the pattern repeats every 16 rows, so fragment blocks 32 rows apart differ by a constant offset);
+//       fragments are ds_read_b128.
 //   RC  row-contiguous (stride_row == 1, the transposed storage): LDS tile [64 k][rows], chunk (8 rows)
 //       c of K row k at slot c ^ ((k & 3) << 2); fragments are two ds_read_b64_tr_b16 — the LDS
 //       transpose read of gfx950 hands every lane four consecutive k of its row, which is exactly the
@@ -63,7 +65,7 @@ __device__ __forceinline__ void wait_vm_lgkm0() {
 template <int R, int KIND, int T> struct Stream;
 
 template <int R, int T>
-struct Stream<R, 0, T> {  // K-contiguous: tile [R][64 k], chunk c of row r at slot c ^ (r & 7)
+struct Stream<R, 0, T> {  // K-contiguous: tile [R][64 k], chunk c of row r at slot c ^ swz16(r)
     static constexpr int N = R / 32;   // DMA instructions per wavefront per tile
     static constexpr int READS = T;    // LDS read instructions per K sub-step
     int off[N];
@@ -73,13 +75,13 @@ struct Stream<R, 0, T> {  // K-contiguous: tile [R][64 k], chunk c of row r at s
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             const int r = (i * 4 + wave) * 8 + (lane >> 3);
-            const int c = (lane & 7) ^ (r & 7);
+            const int c = (lane & 7) ^ swz16(r);
             off[i] = (int)(min(row0 + r, rows - 1) * s_row) + c * 8;
         }
         const int r = wrow0 + (lane & 31);
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
-            faddr[kk] = tile0 + r * kRowBytes + ((((kk * 2 + (lane >> 5))) ^ (r & 7)) << 4);
+            faddr[kk] = tile0 + r * kRowBytes + ((((kk * 2 + (lane >> 5))) ^ swz16(r)) << 4);
     }
     __device__ __forceinline__ void issue(const _Float16* base, int64_t, int k0, char* tile, int wave) const {
 #pragma unroll
@@ -139,8 +141,20 @@ struct Stream<R, 1, T> {  // row-contiguous: tile [64 k][R], chunk c (8 rows) of
     }
 };
 
+#ifdef DML_GEMM_TRACE
+// Lab-only timeline: lane `slot` of one VGPR receives the low half of the shader clock; written out at the end.
+__device__ unsigned* dml_gemm_trace_buf;
+#define DML_TR(slot)                                                                                               \
+    do {                                                                                                           \
+        const int s_ = (slot);                                                                                     \
+        if (s_ < 64) { const int t_ = (int)__builtin_readcyclecounter(); trace_v = ((int)(threadIdx.x & 63) == s_) ? t_ : trace_v; } \
+    } while (0)
+#else
+#define DML_TR(slot)
+#endif
+
 // ---------------------------------------------------------------- kernel
-template <int BM, int BN, int WM, int WN, int AKIND, int BKIND, int NSTAGE, bool ACT>
+template <int BM, int BN, int WM, int WN, int AKIND, int BKIND, int NSTAGE, int EPI>
 __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16* __restrict__ a_ptr,
                                                                  const _Float16* __restrict__ b_ptr, void* c_ptr,
                                                                  const void* bias_ptr, const void* res_ptr,
@@ -151,6 +165,10 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     constexpr int LPT = BM / 32 + BN / 32;  // DMA instructions per wavefront per tile
     extern __shared__ __attribute__((aligned(16))) char lds[];
 
+#ifdef DML_GEMM_TRACE
+    int trace_v = 0;
+#endif
+    DML_TR(0);
     long long bid = blockIdx.x;
     {
         const long long total = g.total_blocks;
@@ -199,9 +217,12 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
             sb.issue(B, g.sbk, s * BK, lds + s * STAGE + A_BYTES, wave);
         }
     }
+    DML_TR(1);
     if (nk >= NSTAGE - 1) wait_vm_lgkm0<(NSTAGE - 2) * LPT>();
     else wait_vm_lgkm0<0>();
+    DML_TR(2);
     __builtin_amdgcn_s_barrier();
+    DML_TR(3);
 
     half8 af[2][TM], bf[2][TN];
     if (nk > 0) {
@@ -226,16 +247,20 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
             constexpr int kk = decltype(kc)::value;
             constexpr int nb = (kk + 1) & 1;
             if constexpr (kk + 1 < BK / 16) {
-                // fragments of the next sub-step, then wait for everything older than them
+                // fragments of the next sub-step, then wait for everything older than them (measured: fetching
+                // a whole K step of fragments ahead instead does not shorten the step)
                 sa.template frags<kk + 1>(cur_off, af[nb]);
                 sb.template frags<kk + 1>(cur_off, bf[nb]);
                 wait_lgkm<READS_W>();
             } else {
                 // last sub-step: its fragments are the only reads outstanding. Tile kt+1 must have
                 // landed for every wavefront before anybody reads it.
+                DML_TR(4 + 3 * kt);
                 if (fill < nk) wait_vm_lgkm0<(NSTAGE - 2) * LPT>();
                 else wait_vm_lgkm0<0>();
+                DML_TR(5 + 3 * kt);
                 __builtin_amdgcn_s_barrier();
+                DML_TR(6 + 3 * kt);
                 if (more) {
                     sa.template frags<0>((uint32_t)nxt_stage * STAGE, af[0]);
                     sb.template frags<0>((uint32_t)nxt_stage * STAGE, bf[0]);
@@ -246,35 +271,33 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[kk & 1][i], bf[kk & 1][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][j], af[kk & 1][i], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         });
         cur_stage = nxt_stage;
     }
     wait_vm_lgkm0<0>();
     __syncthreads();
+    DML_TR(62);
 
     // ---- epilogue (see store_strip): 32 x WN strips through this wavefront's LDS region
     constexpr int PITCH = WN + 4;
     float* strip = reinterpret_cast<float*>(lds) + wave * 32 * PITCH;
-    const int ncol = lane & 31, mgrp = lane >> 5;
+    float bias_n[8];
+    load_bias_n<WN>(g, bias_ptr, n0 + wn * WN, lane, bias_n);
     static_for<0, TM>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        static_for<0, TN>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-#pragma unroll
-            for (int e = 0; e < 16; ++e)
-                strip[((e >> 2) * 8 + mgrp * 4 + (e & 3)) * PITCH + j * 32 + ncol] = acc[i][j][e];
-        });
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        stage_strip<TN, PITCH>(strip, acc[i], lane);
+        __builtin_amdgcn_wave_barrier();  // LDS serves a wavefront's accesses in program order
         const int mb = m0 + wm * WM + i * 32, nb = n0 + wn * WN;
-        if (g.out_f32) store_strip<float, WN, ACT>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, strip, mb, nb, coff, lane);
-        else store_strip<_Float16, WN, ACT>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, strip, mb, nb, coff, lane);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        if (g.out_f32) store_strip<float, WN, EPI>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, bias_n, strip, mb, nb, coff, lane);
+        else store_strip<_Float16, WN, EPI>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, bias_n, strip, mb, nb, coff, lane);
         __builtin_amdgcn_wave_barrier();
     });
+#ifdef DML_GEMM_TRACE
+    DML_TR(63);
+    if (dml_gemm_trace_buf) dml_gemm_trace_buf[((size_t)blockIdx.x * 4 + wave) * 64 + lane] = (unsigned)trace_v;
+#endif
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE>
@@ -288,8 +311,13 @@ int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, cons
     size_t lds = (size_t)NSTAGE * (BM + BN) * kRowBytes;
     const size_t epi = (size_t)4 * 32 * (WN + 4) * sizeof(float);
     if (lds < epi) lds = epi;
+    const int ek = epilogue_kind(g, bias, res, pre);
+    if (ek == EPI_GENERAL_ACT) {
+        set_error("gemm_f16: the pipelined kernel has no activation + residual/beta/row-bias epilogue");
+        return DMLHIP_ERR_UNSUPPORTED;
+    }
 #define DML_PIPE_CASE(AK, BKD, ACTV)                                                                          \
-    if (akind == AK && bkind == BKD && (g.act != DMLHIP_ACT_NONE) == ACTV) {                                  \
+    if (akind == AK && bkind == BKD && ek == ACTV) {                                                          \
         auto kern = gemm_f16_pipe_kernel<BM, BN, WM, WN, AK, BKD, NSTAGE, ACTV>;                              \
         if (lds > 64 * 1024) {                                                                                \
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
@@ -302,8 +330,10 @@ int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, cons
         hipLaunchKernelGGL(kern, (unsigned)total, kThreads, lds, st, a, b, c, bias, res, pre, g);             \
         return launch_status("gemm_f16(pipelined)");                                                          \
     }
-    DML_PIPE_CASE(0, 0, false) DML_PIPE_CASE(0, 1, false) DML_PIPE_CASE(1, 0, false) DML_PIPE_CASE(1, 1, false)
-    DML_PIPE_CASE(0, 0, true) DML_PIPE_CASE(0, 1, true) DML_PIPE_CASE(1, 0, true) DML_PIPE_CASE(1, 1, true)
+    DML_PIPE_CASE(0, 0, EPI_PLAIN) DML_PIPE_CASE(0, 1, EPI_PLAIN) DML_PIPE_CASE(1, 0, EPI_PLAIN) DML_PIPE_CASE(1, 1, EPI_PLAIN)
+    DML_PIPE_CASE(0, 0, EPI_ACT) DML_PIPE_CASE(0, 1, EPI_ACT) DML_PIPE_CASE(1, 0, EPI_ACT) DML_PIPE_CASE(1, 1, EPI_ACT)
+    DML_PIPE_CASE(0, 0, EPI_GENERAL) DML_PIPE_CASE(0, 1, EPI_GENERAL) DML_PIPE_CASE(1, 0, EPI_GENERAL)
+    DML_PIPE_CASE(1, 1, EPI_GENERAL)
 #undef DML_PIPE_CASE
     set_error("gemm_f16: no pipelined kernel for operand kinds %d/%d", akind, bkind);
     return DMLHIP_ERR_UNSUPPORTED;
