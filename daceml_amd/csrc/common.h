@@ -95,11 +95,12 @@ __device__ __forceinline__ float block_reduce(float v, float* scratch) {
 // Second stage of the two-stage column reductions: out[c] = scale * Op over p < parts of
 // part[p*row_stride + c]. 64 columns per workgroup, 16 wavefronts striding over the partial rows with
 // several independent loads in flight each (the partial matrix is small, so this stage is latency
-// bound and wants many short chains rather than few long ones).
+// bound and wants many short chains rather than few long ones). With `out1` set, columns >= cols0 go to
+// out1[c - cols0]: two results that share one partial matrix finish in one launch.
 template <typename Op, typename TOut>
 __global__ __launch_bounds__(1024) void reduce_partials_kernel(const float* __restrict__ part, TOut* __restrict__ out,
                                                                int parts, int64_t row_stride, int64_t cols, float init,
-                                                               float scale) {
+                                                               float scale, TOut* __restrict__ out1, int64_t cols0) {
     __shared__ float lds[16][kWave];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int64_t c = (int64_t)blockIdx.x * kWave + lane;
@@ -122,7 +123,8 @@ __global__ __launch_bounds__(1024) void reduce_partials_kernel(const float* __re
         float a = lds[0][lane];
 #pragma unroll
         for (int w = 1; w < 16; ++w) a = Op::f(a, lds[w][lane]);
-        out[c] = from_f32<TOut>(a * scale);
+        if (out1 && c >= cols0) out1[c - cols0] = from_f32<TOut>(a * scale);
+        else out[c] = from_f32<TOut>(a * scale);
     }
 }
 

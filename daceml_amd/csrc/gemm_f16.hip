@@ -520,10 +520,10 @@ int dmlhip_gemm_f16_ws(const dmlhip_gemm_desc* d, const void* a, const void* b, 
     const unsigned grid = (unsigned)ceil_div(cols, kWave);
     if (d->out_dtype == DMLHIP_F32)
         hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, (const float*)workspace, (float*)c,
-                           s, cols, cols, 0.f, d->alpha);
+                           s, cols, cols, 0.f, d->alpha, (float*)nullptr, (int64_t)0);
     else
         hipLaunchKernelGGL((reduce_partials_kernel<OpSum, _Float16>), grid, 1024, 0, st, (const float*)workspace,
-                           (_Float16*)c, s, cols, cols, 0.f, d->alpha);
+                           (_Float16*)c, s, cols, cols, 0.f, d->alpha, (_Float16*)nullptr, (int64_t)0);
     return launch_status("gemm_f16(split-K sum)");
 }
 

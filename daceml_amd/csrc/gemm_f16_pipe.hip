@@ -16,48 +16,11 @@
 // Requirements (checked by the host): K % 64 == 0, 16-byte aligned bases and strides, rows % 8 == 0
 // for RC operands, 32-bit element offsets.
 #include "gemm_f16_common.h"
+#include "lds_ops.h"
 
 namespace dml {
 namespace gemm16 {
 namespace {
-
-typedef _Float16 half4v __attribute__((ext_vector_type(4)));
-typedef short short4v __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ void lds_dma16(const _Float16* gptr, char* lds_dst) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gptr,
-                                     (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
-}
-
-// ---------------------------------------------------------------- LDS reads
-// Fragment reads are issued as inline assembly so that the compiler neither guesses at aliasing
-// between them and the in-flight global->LDS transfers (it would wait for *all* transfers before a
-// transpose read) nor places the waits: the kernel waits explicitly (lgkmcnt / vmcnt counters).
-template <int OFFSET>
-__device__ __forceinline__ half8 lds_read_b128(uint32_t addr) {
-    half8 v;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
-    return v;
-}
-
-template <int OFFSET>
-__device__ __forceinline__ half4v lds_read_tr16_b64(uint32_t addr) {
-    half4v v;
-    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
-    return v;
-}
-
-template <int N>
-__device__ __forceinline__ void wait_lgkm() {
-    static_assert(N >= 0 && N <= 15, "lgkmcnt is a 4-bit counter");
-    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
-}
-
-template <int VM>
-__device__ __forceinline__ void wait_vm_lgkm0() {
-    static_assert(VM >= 0 && VM <= 63, "vmcnt is a 6-bit counter");
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(VM) : "memory");
-}
 
 // ---------------------------------------------------------------- operand streams
 // A stream owns one operand: where each lane's 16-byte DMA pieces come from, and where each lane

@@ -1,0 +1,55 @@
+// LDS primitives shared by the kernels that stream operand tiles from global memory straight into
+// LDS (global_load_lds) and read MFMA fragments back with explicit waits.
+//
+// Fragment reads are inline assembly so that the compiler neither guesses at aliasing between them
+// and the in-flight global->LDS transfers (it would wait for *all* transfers before a transpose
+// read) nor places the waits: the kernels wait explicitly on the lgkmcnt / vmcnt counters.
+#pragma once
+
+#include "common.h"
+
+namespace dml {
+
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+
+// 16 bytes per lane, global -> LDS without staging registers. The LDS destination of lane l is
+// lds_dst + 16*l; lds_dst must be wavefront-uniform.
+__device__ __forceinline__ void lds_dma16(const _Float16* gptr, char* lds_dst) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gptr,
+                                     (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
+}
+
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
+}
+
+template <int OFFSET>
+__device__ __forceinline__ half8 lds_read_b128(uint32_t addr) {
+    half8 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+
+// LDS transpose read: within each group of 16 lanes, lane s points at four consecutive 16-bit
+// elements of row s/4 (columns 4*(s%4)..+3 of the group's 16 columns); lane j receives column j of
+// the four rows. A lane thus gets four consecutive K values of "its" column, the MFMA operand layout.
+template <int OFFSET>
+__device__ __forceinline__ half4v lds_read_tr16_b64(uint32_t addr) {
+    half4v v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+
+template <int N>
+__device__ __forceinline__ void wait_lgkm() {
+    static_assert(N >= 0 && N <= 15, "lgkmcnt is a 4-bit counter");
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int VM>
+__device__ __forceinline__ void wait_vm_lgkm0() {
+    static_assert(VM >= 0 && VM <= 63, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(VM) : "memory");
+}
+
+}  // namespace dml

@@ -160,7 +160,8 @@ int reduce_typed(const TIn* x, TOut* y, int64_t outer, int64_t r, int64_t inner,
     const int64_t inner2 = outer * inner;
     using Op = typename RedOp<OP>::op;
     hipLaunchKernelGGL((reduce_partials_kernel<Op, TOut>), (unsigned)ceil_div(inner2, kWave), 1024, 0, st,
-                       (const float*)part, y, (int)p.splits, inner2, inner2, RedOp<OP>::init(), scale);
+                       (const float*)part, y, (int)p.splits, inner2, inner2, RedOp<OP>::init(), scale, (TOut*)nullptr,
+                       (int64_t)0);
     return launch_status("reduce(partials)");
 }
 

@@ -348,11 +348,10 @@ __global__ __launch_bounds__(kRowBlock) void layernorm_bwd_wave_kernel(
 }
 
 void launch_ln_bwd_finish(const float* part, float* dgamma, float* dbeta, int nparts, int64_t cols, hipStream_t st) {
-    const unsigned grid = (unsigned)ceil_div(cols, kWave);
-    hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, part, dgamma, nparts, 2 * cols, cols,
-                       0.f, 1.f);
-    hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, part ? part + cols : part, dbeta,
-                       nparts, 2 * cols, cols, 0.f, 1.f);
+    // partial rows are [dgamma | dbeta]: one launch finishes both
+    const unsigned grid = (unsigned)ceil_div(2 * cols, kWave);
+    hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, part, dgamma, nparts, 2 * cols, 2 * cols,
+                       0.f, 1.f, dbeta, cols);
 }
 
 // fallback: dx, workgroup per row

@@ -215,7 +215,8 @@ def test_cast():
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["sum", "mean", "max", "min"])
 @pytest.mark.parametrize("shape,axes", [((8, 64, 100), [-1]), ((6, 5000), [1]), ((4096, 256), [0]), ((3, 40, 7), [1]),
-                                        ((4, 6, 8, 10), [2, 3]), ((2, 1024, 64), [0, 1]), ((5, 7), None), ((3, 1, 9), [1])])
+                                        ((4, 6, 8, 10), [2, 3]), ((2, 1024, 64), [0, 1]), ((5, 7), None), ((3, 1, 9), [1]),
+                                        ((4100, 1024), [0]), ((2, 2500, 512), [1])])
 @pytest.mark.parametrize("keepdims", [1, 0])
 def test_reduce(dtype, name, shape, axes, keepdims):
     from daceml_amd import _lib as L, kernels as K
