@@ -44,6 +44,15 @@ class Conv2dDesc(Structure):
     ]
 
 
+class AttentionDesc(Structure):
+    """struct dmlhip_attention_desc"""
+    _fields_ = [
+        ("batch", c_int64 * 2), ("seq_q", c_int64), ("seq_k", c_int64), ("head_dim", c_int64),
+        ("q_stride", c_int64 * 3), ("k_stride", c_int64 * 3), ("v_stride", c_int64 * 3), ("o_stride", c_int64 * 3),
+        ("scale", c_float),
+    ]
+
+
 _P = c_void_p
 _I64P = POINTER(c_int64)
 
@@ -86,6 +95,10 @@ SIGNATURES = {
     "dmlhip_conv2d_backward_data_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P]),
     "dmlhip_conv2d_backward_weight_workspace_bytes": (c_size_t, [POINTER(Conv2dDesc)]),
     "dmlhip_conv2d_backward_weight_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, c_size_t, _P]),
+    "dmlhip_attention_f16": (c_int, [POINTER(AttentionDesc), _P, _P, _P, _P, _P, _P]),
+    "dmlhip_attention_backward_workspace_bytes": (c_size_t, [POINTER(AttentionDesc)]),
+    "dmlhip_attention_backward_f16": (c_int, [POINTER(AttentionDesc), POINTER(AttentionDesc), _P, _P, _P, _P, _P, _P, _P,
+                                              _P, _P, _P, c_size_t, _P]),
 }
 
 # exported for the test-suite only (not declared in the public header)

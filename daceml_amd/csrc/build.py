@@ -24,6 +24,7 @@ SOURCES = [
     "gemm_f16_pipe.hip",
     "gemm_f32.hip",
     "conv.hip",
+    "attention.hip",
 ]
 
 # -packed-fp32-ops: keep the compiler from forming packed-fp32 VALU instructions.

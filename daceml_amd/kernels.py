@@ -417,3 +417,50 @@ def conv2d_backward(x, w, dy, strides=(1, 1), pads=(0, 0), dilations=(1, 1), gro
         L.check(lib.dmlhip_conv2d_backward_weight_f32(ctypes.byref(d), _ptr(x), _ptr(dy), _ptr(dw), _ptr(ws),
                                                       ws.numel() if ws is not None else 0, _stream()))
     return dx, dw
+
+
+# ----------------------------------------------------------------------------- fused attention
+def _attn_strides(t: torch.Tensor):
+    if t.dim() != 4 or t.stride(3) != 1:
+        raise ValueError("attention tensors are [batch0, batch1, seq, head_dim] views with a contiguous head_dim")
+    return tuple(int(t.stride(i)) for i in range(3))
+
+
+def _attn_desc(q, k, v, o, scale):
+    d = L.AttentionDesc()
+    d.batch[0], d.batch[1] = q.shape[0], q.shape[1]
+    d.seq_q, d.seq_k, d.head_dim = q.shape[2], k.shape[2], q.shape[3]
+    for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("o_stride", o)):
+        for i, sv in enumerate(_attn_strides(t)):
+            getattr(d, name)[i] = sv
+    d.scale = float(scale)
+    return d
+
+
+def attention(q, k, v, scale, out=None, need_lse=True):
+    """softmax(scale * q k^T) v for [b0, b1, seq, 64] fp16 views (any batch / sequence strides). Returns (out, lse)."""
+    _check(q, k, v, dtype=torch.float16)
+    if k.shape[:2] != q.shape[:2] or v.shape[:3] != k.shape[:3] or k.shape[3] != q.shape[3] or v.shape[3] != q.shape[3]:
+        raise ValueError("attention: incompatible shapes %s %s %s" % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty(q.shape[:3], dtype=torch.float32, device=q.device) if need_lse else None
+    d = _attn_desc(q, k, v, out, scale)
+    L.check(L.load().dmlhip_attention_f16(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _stream()))
+    return out, lse
+
+
+def attention_backward(q, k, v, out, lse, dout, scale):
+    """Gradients (dq, dk, dv) of :func:`attention`; dense outputs."""
+    _check(q, k, v, out, dout, dtype=torch.float16)
+    dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), \
+        torch.empty_like(k, memory_format=torch.contiguous_format), torch.empty_like(v, memory_format=torch.contiguous_format)
+    d = _attn_desc(q, k, v, out, scale)
+    g = _attn_desc(dq, dk, dv, dout, scale)
+    lib = L.load()
+    need = lib.dmlhip_attention_backward_workspace_bytes(ctypes.byref(d))
+    ws = workspace(need, q.device)
+    L.check(lib.dmlhip_attention_backward_f16(ctypes.byref(d), ctypes.byref(g), _ptr(q), _ptr(k), _ptr(v), _ptr(out),
+                                              _ptr(lse), _ptr(dout), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(),
+                                              _stream()))
+    return dq, dk, dv

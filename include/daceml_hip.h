@@ -234,6 +234,34 @@ int dmlhip_conv2d_backward_weight_f32(const dmlhip_conv2d_desc* d, const void* x
                                       const void* dy, void* dw, void* workspace,
                                       size_t workspace_bytes, void* stream);
 
+/* ---- fused attention ----------------------------------------------------------------------
+ * O = softmax(scale * Q K^T, over keys) V for fp16 tensors, computed without writing the
+ * [seq_q, seq_k] scores to memory. Replaces the node chain the reference expands separately:
+ * Einsum / MatMul(Q, K) (pure_implementations.py:111-252), the scalar Mul / Div (:76-93),
+ * Softmax(axis=-1) (:309-319) and Einsum(P, V); the backward entry point replaces the nodes
+ * DefaultEinsumBackward and DefaultSoftmaxBackward emit for that chain
+ * (autodiff/implementations/onnx_ops.py:25-138, 237-275). No mask, no dropout.
+ * Tensors are [batch0, batch1, seq, head_dim] views: element strides for batch0, batch1 and
+ * seq are given per tensor (multiples of 8), head_dim is contiguous and must be 64.
+ * lse (optional in forward, required by backward): fp32 [batch0, batch1, seq_q] dense,
+ * lse = log(sum_k exp(scale * q.k)) per query row. */
+typedef struct dmlhip_attention_desc {
+    int64_t batch[2];
+    int64_t seq_q, seq_k, head_dim;
+    int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3];
+    float scale;
+} dmlhip_attention_desc;
+int dmlhip_attention_f16(const dmlhip_attention_desc* d, const void* q, const void* k,
+                         const void* v, void* o, void* lse, void* stream);
+/* grad: strides of dq / dk / dv / do in the q / k / v / o slots (extents and scale are taken
+ * from d). workspace: dmlhip_attention_backward_workspace_bytes(d) bytes (row dots do.o). */
+size_t dmlhip_attention_backward_workspace_bytes(const dmlhip_attention_desc* d);
+int dmlhip_attention_backward_f16(const dmlhip_attention_desc* d,
+                                  const dmlhip_attention_desc* grad, const void* q,
+                                  const void* k, const void* v, const void* o, const void* lse,
+                                  const void* d_o, void* dq, void* dk, void* dv,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

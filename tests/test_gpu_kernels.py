@@ -428,3 +428,53 @@ def test_conv2d_f16_1x1_and_depthwise():
         got = K.conv2d(dev(x), dev(w), None, st, pd, (1, 1), grp)
         want = O.conv2d(x64, w64, None, st, (pd[0], pd[1], pd[0], pd[1]), (1, 1), grp)
         assert_close(host(got), want, torch.float16, "conv f16 %s" % (ws, ))
+
+
+# ----------------------------------------------------------------------------- fused attention
+ATTN_CASES = [
+    # (batch0, batch1, seq_q, seq_k, layout)   layout "bhsd" = dense, "bshd" = head-split view of [b, s, h*d]
+    (2, 3, 128, 128, "bhsd"), (1, 2, 512, 512, "bshd"), (2, 2, 100, 77, "bhsd"), (1, 1, 1, 1, "bhsd"),
+    (1, 3, 33, 200, "bshd"), (2, 1, 257, 64, "bhsd"), (1, 2, 64, 321, "bshd"),
+]
+
+
+def _attn_tensor(seed, b0, b1, s, layout, scale=1.0):
+    x = (rng(seed).standard_normal((b0, b1, s, 64)) * scale).astype(np.float16)
+    if layout == "bhsd":
+        return dev(x), x.astype(np.float64)
+    base = dev(np.ascontiguousarray(x.transpose(0, 2, 1, 3)))  # [b0, s, b1, 64]
+    return base.permute(0, 2, 1, 3), x.astype(np.float64)
+
+
+@pytest.mark.parametrize("b0,b1,sq,sk,layout", ATTN_CASES)
+def test_attention_forward(b0, b1, sq, sk, layout):
+    from daceml_amd import kernels as K
+    q, q64 = _attn_tensor(70, b0, b1, sq, layout)
+    k, k64 = _attn_tensor(71, b0, b1, sk, layout)
+    v, v64 = _attn_tensor(72, b0, b1, sk, layout)
+    scale = 0.125
+    out, lse = K.attention(q, k, v, scale)
+    want, want_lse = O.attention(q64, k64, v64, scale)
+    assert_close(host(out), want, torch.float16, "attention %s" % ((b0, b1, sq, sk, layout), ))
+    assert_close(host(lse), want_lse, torch.float32, "attention lse", rtol=1e-3, atol=1e-3)
+    # rows of softmax sum to one: with v = 1 the output is exactly representable
+    ones = torch.ones_like(v)
+    out1, _ = K.attention(q, k, ones, scale)
+    np.testing.assert_allclose(host(out1), 1.0, rtol=0, atol=2e-3)
+
+
+@pytest.mark.parametrize("b0,b1,sq,sk,layout", ATTN_CASES)
+def test_attention_backward(b0, b1, sq, sk, layout):
+    from daceml_amd import kernels as K
+    q, q64 = _attn_tensor(73, b0, b1, sq, layout)
+    k, k64 = _attn_tensor(74, b0, b1, sk, layout)
+    v, v64 = _attn_tensor(75, b0, b1, sk, layout)
+    do, do64 = _attn_tensor(76, b0, b1, sq, layout)
+    scale = 0.125
+    out, lse = K.attention(q, k, v, scale)
+    dq, dk, dv = K.attention_backward(q, k, v, out, lse, do, scale)
+    wq, wk, wv = O.attention_backward(q64, k64, v64, scale, do64)
+    for name, got, want in (("dq", dq, wq), ("dk", dk, wk), ("dv", dv, wv)):
+        s = max(1.0, float(np.abs(want).max()))
+        assert_close(host(got), want, torch.float16, "attention backward %s %s" % (name, (b0, b1, sq, sk, layout)),
+                     atol=1e-2 * s)

@@ -188,6 +188,35 @@ def test_einsum_and_its_backward():
     np.testing.assert_allclose(O.einsum_backward("bij,jk->bik", [a, b], dy, 1), tb.grad.numpy(), rtol=1e-12)
 
 
+def test_attention_matches_torch_sdpa_and_autograd():
+    """The fused-attention oracle is the composition of pinned parts; pin the composition too: against
+    torch's scaled_dot_product_attention and its autograd in fp64, a brute-force loop, and invariants."""
+    q = rng(90).standard_normal((2, 3, 7, 8))
+    k = rng(91).standard_normal((2, 3, 5, 8))
+    v = rng(92).standard_normal((2, 3, 5, 8))
+    do = rng(93).standard_normal((2, 3, 7, 8))
+    scale = 0.37
+    out, lse = O.attention(q, k, v, scale)
+    tq, tk, tv = (torch.tensor(t, requires_grad=True) for t in (q, k, v))
+    ref = F.scaled_dot_product_attention(tq, tk, tv, scale=scale)
+    np.testing.assert_allclose(out, ref.detach().numpy(), rtol=1e-12, atol=1e-12)
+    ref.backward(torch.tensor(do))
+    dq, dk, dv = O.attention_backward(q, k, v, scale, do)
+    for got, want in ((dq, tq.grad), (dk, tk.grad), (dv, tv.grad)):
+        np.testing.assert_allclose(got, want.numpy(), rtol=1e-11, atol=1e-12)
+    # brute force for one (batch, head, query)
+    s = np.array([scale * sum(q[1, 2, 4, d] * k[1, 2, j, d] for d in range(8)) for j in range(5)])
+    p = np.exp(s) / np.exp(s).sum()
+    np.testing.assert_allclose(out[1, 2, 4], sum(p[j] * v[1, 2, j] for j in range(5)), rtol=1e-12)
+    np.testing.assert_allclose(lse[1, 2, 4], math.log(np.exp(s).sum()), rtol=1e-12)
+    # invariants: v = const -> out = const; a single key -> out = v; dq + (dk transported) sum rule: sum_j dS = 0
+    np.testing.assert_allclose(O.attention(q, k, np.ones_like(v), scale)[0], 1.0, rtol=1e-13)
+    np.testing.assert_allclose(O.attention(q, k[:, :, :1], v[:, :, :1], scale)[0], np.broadcast_to(v[:, :, :1], q.shape))
+    # scale = 0: uniform probabilities, dq = 0
+    dq0, _, _ = O.attention_backward(q, k, v, 0.0, do)
+    np.testing.assert_array_equal(dq0, 0.0)
+
+
 def test_gemm_attributes():
     a, b, c = rng(26).standard_normal((4, 5)), rng(27).standard_normal((6, 5)), rng(28).standard_normal(6)
     np.testing.assert_allclose(O.gemm(a, b, c, alpha=0.5, beta=2.0, transB=1), 0.5 * a @ b.T + 2.0 * c, rtol=1e-12)
