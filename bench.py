@@ -133,9 +133,13 @@ def main():
     gemm_flops = sum(l.flops for l, _ in rows if l.kind == "gemm")
     n_gemm = sum(1 for l, _ in rows if l.kind == "gemm")
     tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
+    attn = {}
+    for l, t in rows:
+        if l.kind in ("attention", "attention_backward"):
+            attn[l.kind] = {"ms": round(t, 4), "flops": l.flops, "TFLOP/s": round(l.flops / (t * 1e-3) / 1e12, 1)}
     hbm = {}
     for l, t in rows:
-        if l.kind == "gemm" or l.bytes_moved == 0:
+        if l.kind in ("gemm", "attention", "attention_backward") or l.bytes_moved == 0:
             continue
         e = hbm.setdefault(l.kind, {"ms": 0.0, "bytes": 0, "launches": 0})
         e["ms"] += t
@@ -156,6 +160,7 @@ def main():
                      "frac": round(tflops / PEAK_FP16_TFLOPS, 4), "traffic": None,
                      "kernel": "gemm_f16_kernel (all %d contraction launches of a step)" % n_gemm,
                      "flops_per_step": gemm_flops, "ms_per_step": round(gemm_ms, 4)},
+        "attention_nodes": attn,
         "hbm_nodes": hbm,
         "sum_of_kernel_ms": round(sum(t for _, t in rows), 4),
     }

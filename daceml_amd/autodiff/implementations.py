@@ -182,6 +182,39 @@ class HipSoftmaxBackward(BackwardImplementation):
         return sg, BackwardResult(required_grad_names={"input": "dX"}, given_grad_names={"output": "dY"})
 
 
+@autoregister_params(op="FusedAttention", name=NAME)
+class HipFusedAttentionBackward(BackwardImplementation):
+    """One FusedAttentionGrad node; the forward node is made to emit its log-sum-exp rows, which replace the
+    probability matrix that DefaultSoftmaxBackward (onnx_ops.py:237-275) would forward."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        return True
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        sdfg = context.forward_sdfg
+        q = sdfg.arrays[_in_arr(context, forward_node, "Q")]
+        pm = forward_node.q_perm
+        lse_shape = tuple(1 if pm[i] < 0 else q.shape[pm[i]] for i in range(3))
+        lse = _ensure_forward_output(context, forward_node, "LogSumExp", lse_shape, torch.float32)
+        g = _new(context, "FusedAttentionGrad", forward_node.label + "_backward", scale=forward_node.scale,
+                 q_perm=forward_node.q_perm, k_perm=forward_node.k_perm, v_perm=forward_node.v_perm,
+                 o_perm=forward_node.o_perm)
+        for conn in ("Q", "K", "V"):
+            connect_input_from_forward(forward_node, g, context, conn)
+        connect_output_from_forward(forward_node, g, context, "Output", "O")
+        _read(context, lse, g, "LogSumExp")
+        req = {}
+        for conn in ("Q", "K", "V"):
+            if conn in required_gradients:
+                req[conn] = "d" + conn
+            else:  # the kernels always produce all three
+                d = sdfg.arrays[_in_arr(context, forward_node, conn)]
+                scratch, _ = sdfg.add_transient("%s_unused_d%s" % (forward_node.label, conn), d.shape, d.dtype)
+                _write(context, g, "d" + conn, scratch)
+        return g, BackwardResult(required_grad_names=req, given_grad_names={"Output": "dO"})
+
+
 def _ln_backward(forward_node, ctx, x_arr, scale_conn, bias_conn, x_conns, mean_conn, rstd_conn, required):
     sdfg = ctx.forward_sdfg
     xd = sdfg.arrays[x_arr]

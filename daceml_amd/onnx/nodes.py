@@ -124,6 +124,12 @@ SCHEMAS = [
     # produced by the fusion pass, never by an importer
     _schema("FusedEinsum", "Inputs* Bias? Residual?", "Output PreActivation?", since=1, equation=REQUIRED,
             alpha=1.0, activation="none", accumulate=0),
+    # Einsum(Q,K) [* scale] -> Softmax(last axis) -> Einsum(P,V) as one node (the scores never reach memory).
+    # *_perm: which dimension of that tensor is (batch0, batch1, sequence, head); -1 for an absent batch dim.
+    _schema("FusedAttention", "Q K V", "Output LogSumExp?", since=1, scale=1.0, q_perm=REQUIRED, k_perm=REQUIRED,
+            v_perm=REQUIRED, o_perm=REQUIRED),
+    _schema("FusedAttentionGrad", "Q K V O LogSumExp dO", "dQ dK dV", since=1, scale=1.0, q_perm=REQUIRED,
+            k_perm=REQUIRED, v_perm=REQUIRED, o_perm=REQUIRED),
     # backward nodes emitted by the "hip" BackwardImplementations (names follow the ONNX Runtime
     # training contrib ops)
     _schema("SoftmaxGrad", "dY Y", "dX", since=1, axis=-1),

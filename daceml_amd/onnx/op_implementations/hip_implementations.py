@@ -900,3 +900,110 @@ class HipConvGrad(ONNXForward):
             calls.append(HipCall("dmlhip_reduce_f32", [I32(L.RSUM), Workspace(), Ptr("dB"), I32(L.F32), I64(1), I64(n),
                                                        I64(m), Workspace(part), WorkspaceBytes(part), Stream()]))
         return _tasklet(node, state, calls, workspace_bytes=ws, bytes_moved=_nbytes(x, w, dy), kind="conv_backward")
+
+
+# ----------------------------------------------------------------------------- fused attention
+def _attn_struct(perm_descs, q: Array, k: Array, scale: float, q_perm, k_perm) -> L.AttentionDesc:
+    """perm_descs: four (descriptor, perm) pairs in the q / k / v / o slots of dmlhip_attention_desc."""
+    d = L.AttentionDesc()
+    for i in (0, 1):
+        d.batch[i] = 1 if q_perm[i] < 0 else int(q.shape[q_perm[i]])
+    d.seq_q, d.seq_k, d.head_dim = int(q.shape[q_perm[2]]), int(k.shape[k_perm[2]]), int(q.shape[q_perm[3]])
+    for name, (desc, perm) in zip(("q_stride", "k_stride", "v_stride", "o_stride"), perm_descs):
+        for i in range(3):
+            getattr(d, name)[i] = 0 if perm[i] < 0 else int(desc.strides[perm[i]])
+    d.scale = float(scale)
+    return d
+
+
+def _attn_ok(node, descs_perms) -> bool:
+    """Shapes of the four tensors agree with each other and with what the kernel covers."""
+    (q, qp), (k, kp), (v, vp), (o, op_) = descs_perms
+    for d, pm in descs_perms:
+        if d.dtype != torch.float16 or len(pm) != 4 or d.shape[pm[3]] != 64 or d.strides[pm[3]] != 1:
+            return False
+        if any(pm[i] >= 0 and d.strides[pm[i]] % 8 for i in range(3)):
+            return False
+        if sorted(i for i in pm if i >= 0) != list(range(len(d.shape))):
+            return False
+
+    def ext(d, pm, i):
+        return 1 if pm[i] < 0 else d.shape[pm[i]]
+
+    for i in (0, 1):
+        if len({ext(q, qp, i), ext(k, kp, i), ext(v, vp, i), ext(o, op_, i)}) != 1:
+            return False
+    return ext(k, kp, 2) == ext(v, vp, 2) and ext(q, qp, 2) == ext(o, op_, 2) and ext(k, kp, 2) > 0
+
+
+@op_implementation(op="FusedAttention", name=IMPL)
+class HipFusedAttention(ONNXForward):
+    """softmax(scale * Q K^T) V in one kernel: the composition of PureEinsum (pure_implementations.py:219-252),
+    the scalar Mul (:86-88), Softmax over the last axis (:309-319) and a second PureEinsum, without the score
+    matrix in memory. Optional output LogSumExp (fp32, [batch0, batch1, seq_q]) is what the backward node needs
+    instead of the probabilities."""
+    @staticmethod
+    def _pairs(node, ins, outs):
+        return [(ins["Q"], node.q_perm), (ins["K"], node.k_perm), (ins["V"], node.v_perm), (outs["Output"], node.o_perm)]
+
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            if not _attn_ok(node, HipFusedAttention._pairs(node, ins, outs)):
+                return False
+            lse = outs.get("LogSumExp")
+            return lse is None or (lse.dtype == torch.float32 and lse.is_contiguous())
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        pairs = HipFusedAttention._pairs(node, ins, outs)
+        d = _attn_struct(pairs, ins["Q"], ins["K"], node.scale, node.q_perm, node.k_perm)
+        call = HipCall("dmlhip_attention_f16", [Struct(d, "dmlhip_attention_desc"), Ptr("Q"), Ptr("K"), Ptr("V"),
+                                                Ptr("Output"), _opt(node, state, "LogSumExp", False), Stream()])
+        bh = d.batch[0] * d.batch[1]
+        return _tasklet(node, state, [call], flops=4 * bh * d.seq_q * d.seq_k * 64,
+                        bytes_moved=_nbytes(ins["Q"], ins["K"], ins["V"], outs["Output"]), kind="attention")
+
+
+@op_implementation(op="FusedAttentionGrad", name=IMPL)
+class HipFusedAttentionGrad(ONNXForward):
+    """Backward of FusedAttention: what DefaultEinsumBackward and DefaultSoftmaxBackward
+    (autodiff/implementations/onnx_ops.py:25-138, 237-275) compute for the chain, recomputing the
+    probabilities from Q, K and the stored log-sum-exp."""
+    @staticmethod
+    def _pairs(node, ins, outs):
+        fwd = [(ins["Q"], node.q_perm), (ins["K"], node.k_perm), (ins["V"], node.v_perm), (ins["O"], node.o_perm)]
+        grad = [(outs["dQ"], node.q_perm), (outs["dK"], node.k_perm), (outs["dV"], node.v_perm), (ins["dO"], node.o_perm)]
+        return fwd, grad
+
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            fwd, grad = HipFusedAttentionGrad._pairs(node, ins, outs)
+            lse = ins["LogSumExp"]
+            return _attn_ok(node, fwd) and _attn_ok(node, grad) and lse.dtype == torch.float32 and lse.is_contiguous()
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        import ctypes
+        ins, outs = _descs(node, state, sdfg)
+        fwd, grad = HipFusedAttentionGrad._pairs(node, ins, outs)
+        d = _attn_struct(fwd, ins["Q"], ins["K"], node.scale, node.q_perm, node.k_perm)
+        g = _attn_struct(grad, ins["Q"], ins["K"], node.scale, node.q_perm, node.k_perm)
+        ws = L.load().dmlhip_attention_backward_workspace_bytes(ctypes.byref(d))
+        call = HipCall("dmlhip_attention_backward_f16",
+                       [Struct(d, "dmlhip_attention_desc"), Struct(g, "dmlhip_attention_desc"), Ptr("Q"), Ptr("K"),
+                        Ptr("V"), Ptr("O"), Ptr("LogSumExp"), Ptr("dO"), Ptr("dQ"), Ptr("dK"), Ptr("dV"), Workspace(),
+                        WorkspaceBytes(), Stream()])
+        bh = d.batch[0] * d.batch[1]
+        return _tasklet(node, state, [call], workspace_bytes=ws, flops=8 * bh * d.seq_q * d.seq_k * 64,  # four contractions; the recomputed scores are not counted
+                       
+                        bytes_moved=_nbytes(ins["Q"], ins["K"], ins["V"], ins["O"], ins["dO"], outs["dQ"], outs["dK"],
+                                            outs["dV"]), kind="attention_backward")

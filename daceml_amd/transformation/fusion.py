@@ -17,6 +17,7 @@ expansions it replaces (that composition is the oracle of the fused kernels).
     fuse_epilogues           Einsum, [Div|Mul const], [Add bias], [Gelu],
                              [Add residual]                               -> FusedEinsum
     fuse_skip_layernorm      Add, LayerNormalization                      -> SkipLayerNormalization
+    fuse_attention           Einsum(Q,K)[*scale], Softmax, Einsum(P,V)    -> FusedAttention
     fuse_conv_activation     Conv, Swish | Sigmoid | Relu                 -> Conv(_activation)
 """
 import math
@@ -542,7 +543,102 @@ def fuse_skip_layernorm(sdfg: SDFG) -> int:
     return count
 
 
-def auto_optimize(sdfg: SDFG, training: bool = False) -> Dict[str, int]:
+def _attention_roles(eq_scores: str, eq_context: str):
+    """Letters of the two contractions -> dimension roles. Returns (q_is_first, q_perm, k_perm, v_perm, o_perm) or
+    None when the pair is not softmax(Q K^T) V over the last axis of the scores."""
+    try:
+        (t0, t1), ts = C.parse(eq_scores)
+        (c0, c1), to = C.parse(eq_context)
+    except (C.NotApplicable, ValueError):
+        return None
+    if len(set(ts)) != len(ts) or len(ts) < 2 or len(c0) != len(ts):
+        return None
+    key, query = ts[-1], ts[-2]
+    batch = ts[:-2]
+    if len(batch) > 2:
+        return None
+    # which scores operand holds the queries
+    if query in t0 and key in t1 and query not in t1 and key not in t0:
+        tq, tk, q_first = t0, t1, True
+    elif query in t1 and key in t0 and query not in t0 and key not in t1:
+        tq, tk, q_first = t1, t0, False
+    else:
+        return None
+    contracted = [l for l in tq if l not in ts]
+    if len(contracted) != 1 or contracted[0] not in tk or any(l not in tq or l not in tk for l in batch):
+        return None
+    if sorted(tq) != sorted(list(batch) + [query, contracted[0]]) or sorted(tk) != sorted(list(batch) + [key, contracted[0]]):
+        return None
+    hd = contracted[0]
+    # context: operand 0 is the probabilities, dimension for dimension the scores
+    rename = dict(zip(ts, c0))
+    ckey, cquery, cbatch = rename[key], rename[query], [rename[l] for l in batch]
+    if len(set(c0)) != len(c0) or ckey in to or ckey not in c1 or cquery in c1 or cquery not in to:
+        return None
+    head = [l for l in c1 if l != ckey and l not in cbatch]
+    if len(head) != 1 or sorted(c1) != sorted(cbatch + [ckey, head[0]]) or sorted(to) != sorted(cbatch + [cquery, head[0]]):
+        return None
+
+    def perm(term, b, seq, h):
+        pad = [-1] * (2 - len(b))
+        return tuple(pad + [term.index(l) for l in b] + [term.index(seq), term.index(h)])
+
+    return (q_first, perm(tq, batch, query, hd), perm(tk, batch, key, hd), perm(c1, cbatch, ckey, head[0]),
+            perm(to, cbatch, cquery, head[0]))
+
+
+def fuse_attention(sdfg: SDFG) -> int:
+    """Einsum(Q, K) with an optional folded scale -> Softmax over the keys -> Einsum(P, V) becomes one
+    FusedAttention node when neither the scores nor the probabilities are read by anything else."""
+    count = 0
+    for state in sdfg.states():
+        for sm in [n for n in state.nodes() if _is_op(n, "Softmax")]:
+            x, y = _in_array(state, sm, "input"), _out_array(state, sm, "output")
+            nd = len(sdfg.arrays[x].shape)
+            if sm.axis % nd != nd - 1 or not _internal(sdfg, state, x) or not _internal(sdfg, state, y):
+                continue
+            prod = _producer(state, x)
+            cons = _consumers(state, y)
+            if prod is None or len(cons) != 1 or cons[0][1] != "Inputs__0":
+                continue
+            es, ctx = prod[0], cons[0][0]
+            if not (_is_op(es, "Einsum") or _is_op(es, "FusedEinsum")) or not _is_op(ctx, "Einsum"):
+                continue
+            scale = 1.0
+            if _is_op(es, "FusedEinsum"):
+                conns = {e.dst_conn for e in state.in_edges(es)} | {e.src_conn for e in state.out_edges(es)}
+                if conns - {"Inputs__0", "Inputs__1", "Output"} or es.activation != "none" or es.accumulate:
+                    continue
+                scale = float(es.alpha)
+            roles = _attention_roles(es.equation.replace(" ", ""), ctx.equation.replace(" ", ""))
+            if roles is None:
+                continue
+            q_first, q_perm, k_perm, v_perm, o_perm = roles
+            qa = _in_array(state, es, "Inputs__0" if q_first else "Inputs__1")
+            ka = _in_array(state, es, "Inputs__1" if q_first else "Inputs__0")
+            va = _in_array(state, ctx, "Inputs__1")
+            oa = _out_array(state, ctx, "Output")
+            ok = True
+            for arr, pm in ((qa, q_perm), (ka, k_perm), (va, v_perm), (oa, o_perm)):
+                d = sdfg.arrays[arr]
+                if d.dtype != torch.float16 or d.shape[pm[3]] != 64 or d.strides[pm[3]] != 1 \
+                        or any(d.strides[i] % 8 for i in pm[:3] if i >= 0):
+                    ok = False
+            if not ok:
+                continue
+            label = ctx.label + "_attention"
+            _remove_node(state, es)
+            _remove_node(state, sm)
+            _remove_node(state, ctx)
+            _add_node(sdfg, state, "FusedAttention", label, {"Q": qa, "K": ka, "V": va}, {"Output": oa}, scale=scale,
+                      q_perm=q_perm, k_perm=k_perm, v_perm=v_perm, o_perm=o_perm)
+            count += 1
+    if count:
+        _drop_unused_arrays(sdfg)
+    return count
+
+
+def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True) -> Dict[str, int]:
     """The pass pipeline, in dependency order (cf. daceml.util.utils.auto_optimize,
     daceml/util/utils.py:205-235). Returns how often each rewrite fired."""
     stats = {}
@@ -554,4 +650,5 @@ def auto_optimize(sdfg: SDFG, training: bool = False) -> Dict[str, int]:
     stats["views"] = fold_views(sdfg)
     stats["epilogues"] = fuse_epilogues(sdfg, keep_preactivation=training)
     stats["skip_layernorm"] = fuse_skip_layernorm(sdfg)
+    stats["attention"] = fuse_attention(sdfg) if attention else 0
     return stats

@@ -31,7 +31,7 @@ def _compile(sdfg):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["attention", True, False])
 def test_bert_layer_forward(dtype, fused):
     from daceml_amd import graphs
     from daceml_amd.transformation import fusion
@@ -39,10 +39,15 @@ def test_bert_layer_forward(dtype, fused):
     x, p = _bert_inputs(b, s, h, ffn, dtype)
     sdfg = graphs.bert_encoder_layer(b, s, h, heads, ffn, dtype, eps=1e-5)
     if fused:
-        stats = fusion.auto_optimize(sdfg)
+        stats = fusion.auto_optimize(sdfg, attention=fused == "attention")
         assert stats["layernorm"] == 2 and stats["gelu"] == 1 and stats["epilogues"] == 7
         names = [n.schema.name for n in sdfg.states()[0].library_nodes()]
-        assert sorted(set(names)) == ["Einsum", "FusedEinsum", "LayerNormalization", "Softmax"]
+        if fused == "attention" and dtype == torch.float16:  # the fused kernel is fp16 only
+            assert stats["attention"] == 1
+            assert sorted(set(names)) == ["FusedAttention", "FusedEinsum", "LayerNormalization"]
+        else:
+            assert stats["attention"] == 0
+            assert sorted(set(names)) == ["Einsum", "FusedEinsum", "LayerNormalization", "Softmax"]
     prog = _compile(sdfg)
     y = torch.empty((b, s, h), dtype=dtype, device="cuda")
     prog(x=dev(x), y=y, **{k: dev(v) for k, v in p.items()})
@@ -54,8 +59,8 @@ def test_bert_layer_forward(dtype, fused):
         assert_close(host(y), want, dtype, "bert layer forward fused=%s" % fused, rtol=1e-4, atol=2e-5)
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-def test_bert_layer_backward(dtype):
+@pytest.mark.parametrize("dtype,attention", [(torch.float16, True), (torch.float16, False), (torch.float32, False)])
+def test_bert_layer_backward(dtype, attention):
     from daceml_amd import graphs
     from daceml_amd.autodiff import add_backward_pass
     from daceml_amd.transformation import fusion
@@ -63,12 +68,15 @@ def test_bert_layer_backward(dtype):
     x, p = _bert_inputs(b, s, h, ffn, dtype)
     dy = rng(77).standard_normal((b, s, h)).astype(x.dtype)
     sdfg = graphs.bert_encoder_layer(b, s, h, heads, ffn, dtype, eps=1e-5)
-    fusion.auto_optimize(sdfg, training=True)
+    fusion.auto_optimize(sdfg, training=True, attention=attention)
     grads = add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + OB.PARAM_NAMES,
                               grad_dtypes={n: torch.float32 for n in OB.PARAM_NAMES})
     # the backward state contains only nodes with hand-written kernels
     bnames = {n.schema.name for n in sdfg.states()[1].library_nodes()}
-    assert bnames == {"FusedEinsum", "SoftmaxGrad", "LayerNormalizationGrad", "GeluGrad", "ReduceSum", "Sum"}
+    if attention:
+        assert bnames == {"FusedEinsum", "FusedAttentionGrad", "LayerNormalizationGrad", "GeluGrad", "ReduceSum", "Sum"}
+    else:
+        assert bnames == {"FusedEinsum", "SoftmaxGrad", "LayerNormalizationGrad", "GeluGrad", "ReduceSum", "Sum"}
     prog = _compile(sdfg)
     args = {"x": dev(x), "y": torch.empty((b, s, h), dtype=dtype, device="cuda"), "gradient_y": dev(dy)}
     args.update({k: dev(v) for k, v in p.items()})

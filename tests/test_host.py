@@ -300,7 +300,7 @@ def test_fusion_pipeline_on_bert_layer():
     assert before.count("MatMul") == 8 and before.count("Erf") == 1 and before.count("ReduceMean") == 4
     stats = fusion.auto_optimize(sdfg, training=True)
     assert stats == {"gelu": 1, "layernorm": 2, "swish": 0, "conv_activation": 0, "matmul_to_einsum": 8,
-                     "views": 15, "epilogues": 7, "skip_layernorm": 0}
+                     "views": 15, "epilogues": 7, "skip_layernorm": 0, "attention": 0}  # head dim 32: not fused
     after = {n.label: n for n in st.library_nodes()}
     assert sorted(n.schema.name for n in after.values()) == ["Einsum"] + ["FusedEinsum"] * 7 + \
         ["LayerNormalization"] * 2 + ["Softmax"]
@@ -313,6 +313,46 @@ def test_fusion_pipeline_on_bert_layer():
     assert after["ln1_fused"].epsilon == 1e-12                          # not the fp16-rounded 0.0
     assert all(e.dst_conn != "Inputs__1" or sdfg.arrays[e.data.data].shape == (128, 128)
                for e in st.in_edges(after["q_matmul_fused"]))           # weight used as stored, no Transpose
+
+
+def test_attention_fusion_roles_and_graph():
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.transformation import fusion
+    roles = fusion._attention_roles
+    # BERT's head-split letters: tensors are [batch, seq, head, d]
+    assert roles("biak,bjak->baij", "baik,bkaj->biaj") == (True, (0, 2, 1, 3), (0, 2, 1, 3), (0, 2, 1, 3), (0, 2, 1, 3))
+    # dense [b, h, s, d]; keys given first; one batch dim; none
+    assert roles("abik,abjk->abij", "abij,abjd->abid") == (True, (0, 1, 2, 3), (0, 1, 2, 3), (0, 1, 2, 3), (0, 1, 2, 3))
+    assert roles("abjk,abik->abij", "abij,abjd->abid")[0] is False
+    assert roles("bik,bjk->bij", "bij,bjd->bid") == (True, (-1, 0, 1, 2), (-1, 0, 1, 2), (-1, 0, 1, 2), (-1, 0, 1, 2))
+    assert roles("ik,jk->ij", "ij,jd->id")[1] == (-1, -1, 0, 1)
+    # not attention: softmax axis is not the contracted one of the second product; outer product; 3 batch dims
+    assert roles("abik,abjk->abij", "abij,abid->abjd") is None
+    assert roles("abik,abjk->abji", "abij,abjd->abid") is None or roles("abik,abjk->abji", "abij,abjd->abid")[0] is False
+    assert roles("abcik,abcjk->abcij", "abcij,abcjd->abcid") is None
+    assert roles("abik,abjl->abij", "abij,abjd->abid") is None
+
+    sdfg = graphs.bert_encoder_layer(2, 64, 256, 4, 512, torch.float16)   # head dim 64
+    stats = fusion.auto_optimize(sdfg, training=True)
+    assert stats["attention"] == 1
+    st = sdfg.states()[0]
+    names = sorted(n.schema.name for n in st.library_nodes())
+    assert names == ["FusedAttention"] + ["FusedEinsum"] * 6 + ["LayerNormalization"] * 2
+    att = [n for n in st.library_nodes() if n.schema.name == "FusedAttention"][0]
+    assert att.scale == 0.125 and att.q_perm == (0, 2, 1, 3)
+    assert not any("scores" in a or "softmax" in a for a in sdfg.arrays)   # the score matrix is gone
+    from oracle import bert_layer as OB
+    add_backward_pass(sdfg, st, ["y"], ["x"] + OB.PARAM_NAMES)
+    back = [n for n in sdfg.states()[1].library_nodes() if n.schema.name == "FusedAttentionGrad"]
+    assert len(back) == 1
+    ins = {e.dst_conn for e in sdfg.states()[1].in_edges(back[0])}
+    assert ins == {"Q", "K", "V", "O", "LogSumExp", "dO"}
+    # the forward node now also emits the log-sum-exp rows
+    assert "LogSumExp" in {e.src_conn for e in st.out_edges(att)}
+    # fp32 graphs keep the unfused chain (the kernel is fp16 only)
+    s32 = graphs.bert_encoder_layer(2, 64, 256, 4, 512, torch.float32)
+    assert fusion.auto_optimize(s32)["attention"] == 0
 
 
 def test_fusion_leaves_non_matching_chains_alone():
