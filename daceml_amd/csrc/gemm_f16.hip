@@ -442,8 +442,9 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
         epilogue_kind(g, bias, residual, pre_out) != EPI_GENERAL_ACT) {
         if (cfg < 0) {
             auto blocks = [&](int bm, int bn) { return (long long)ceil_div(d->m, bm) * ceil_div(d->n, bn) * batch; };
-            // measured on MI355X: with more than one 128x128 tile per CU, two resident workgroups with
-            // two LDS stages each beat one workgroup with a deeper ring (and the 256-wide tiles)
+            // measured on MI355X inside the BERT layer: with more than one 128x128 tile per CU, two resident
+            // workgroups with two LDS stages each beat one workgroup with a deeper ring and the 256-wide
+            // tiles (whose epilogue, one workgroup per CU, overlaps with nothing)
             if (blocks(128, 128) > 256) cfg = 3;
             else cfg = 0;
         }

@@ -50,6 +50,10 @@ struct Stream<R, 0, T> {  // K-contiguous: tile [R][64 k], chunk c of row r at s
 #pragma unroll
         for (int i = 0; i < N; ++i) lds_dma16(base + off[i] + k0, tile + (i * 4 + wave) * 1024);
     }
+    template <int I>
+    __device__ __forceinline__ void issue_one(const _Float16* base, int64_t, int k0, char* tile, int wave) const {
+        lds_dma16(base + off[I] + k0, tile + (I * 4 + wave) * 1024);
+    }
     template <int KK>
     __device__ __forceinline__ void frags(uint32_t stage_off, half8 (&f)[T]) const {
         const uint32_t a = faddr[KK] + stage_off;
@@ -91,6 +95,10 @@ struct Stream<R, 1, T> {  // row-contiguous: tile [64 k][R], chunk c (8 rows) of
         const _Float16* p = base + (int64_t)k0 * s_k;
 #pragma unroll
         for (int i = 0; i < N; ++i) lds_dma16(p + off[i], tile + (i * 4 + wave) * 1024);
+    }
+    template <int I>
+    __device__ __forceinline__ void issue_one(const _Float16* base, int64_t s_k, int k0, char* tile, int wave) const {
+        lds_dma16(base + (int64_t)k0 * s_k + off[I], tile + (I * 4 + wave) * 1024);
     }
     template <int KK>
     __device__ __forceinline__ void frags(uint32_t stage_off, half8 (&f)[T]) const {
@@ -199,11 +207,19 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
         const int nxt_stage = cur_stage + 1 == NSTAGE ? 0 : cur_stage + 1;
         // the stage that held tile kt-1 is free (every wavefront passed the barrier of step kt-1 after
         // its last read of it had completed): refill it with tile kt+NSTAGE-1
+        // With three or more stages the transfers are issued in three portions, each right after the MFMAs of
+        // sub-steps 0..2 have been queued: the matrix pipe keeps running while this wavefront computes
+        // addresses and issues them. With two stages the tile is needed at the end of this very step, so it
+        // is requested at once.
+        constexpr bool SPREAD = NSTAGE >= 3;
         const int fill = kt + NSTAGE - 1;
-        if (fill < nk) {
-            const int fs = cur_stage == 0 ? NSTAGE - 1 : cur_stage - 1;
-            sa.issue(A, g.sak, fill * BK, lds + fs * STAGE, wave);
-            sb.issue(B, g.sbk, fill * BK, lds + fs * STAGE + A_BYTES, wave);
+        const int fs = cur_stage == 0 ? NSTAGE - 1 : cur_stage - 1;
+        char* fill_tile = lds + fs * STAGE;
+        if constexpr (!SPREAD) {
+            if (fill < nk) {
+                sa.issue(A, g.sak, fill * BK, fill_tile, wave);
+                sb.issue(B, g.sbk, fill * BK, fill_tile + A_BYTES, wave);
+            }
         }
         const bool more = kt + 1 < nk;
         static_for<0, BK / 16>([&](auto kc) {
@@ -236,6 +252,17 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][j], af[kk & 1][i], acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr (SPREAD && kk < 3) {
+                if (fill < nk) {
+                    constexpr int NA = BM / 32;
+                    static_for<kk * LPT / 3, (kk + 1) * LPT / 3>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        if constexpr (j < NA) sa.template issue_one<j>(A, g.sak, fill * BK, fill_tile, wave);
+                        else sb.template issue_one<j - NA>(B, g.sbk, fill * BK, fill_tile + A_BYTES, wave);
+                    });
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         });
         cur_stage = nxt_stage;
     }
