@@ -20,6 +20,12 @@ if ROOT not in sys.path:
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# Bytes that cross the L2 <-> fabric boundary for the 18 GEMM launches of one step: rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE (one run each, of `bench.py --steps 3 --warmup 2 --no-cpu-baseline --calibrate-copy`), each
+# scaled by what the same counter reads for the 128 MiB copy kernel of --calibrate-copy (FETCH_SIZE x 2.000,
+# WRITE_SIZE x 1.000). Measured, not computed here: it goes stale when the GEMM tiling changes.
+GEMM_TRAFFIC_BYTES_PER_STEP = {"fetched": 1187.8e6, "written": 285.2e6}
+
 METRIC = "BERT-large encoder layer fp16 fwd+bwd ms/iter at 1 GPU; % MFMA & HBM roofline"
 B, S, H, HEADS, FFN = 8, 512, 1024, 16, 4096
 
@@ -101,6 +107,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--verbose", action="store_true", help="per-launch table on stderr")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="after the timed region, launch a plain 128 MiB -> 128 MiB copy kernel three times: under "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its counters give the scale of those counters")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures the single-GPU path only: this build uses one GPU (no collectives, no sharding); "
@@ -123,6 +132,14 @@ def main():
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / a.steps * 1e3
 
+    if a.calibrate_copy:
+        from daceml_amd import _lib as L, kernels as K
+        src = torch.zeros(64 << 20, dtype=torch.float16, device=device)   # 128 MiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            K.unary(L.IDENTITY, src, out=dst)
+        torch.cuda.synchronize()
+
     rows = kernel_breakdown(prog)
     if a.verbose:
         for l, t in rows:
@@ -132,6 +149,7 @@ def main():
     gemm_ms = sum(t for l, t in rows if l.kind == "gemm")
     gemm_flops = sum(l.flops for l, _ in rows if l.kind == "gemm")
     n_gemm = sum(1 for l, _ in rows if l.kind == "gemm")
+    gemm_bytes = sum(l.bytes_moved for l, _ in rows if l.kind == "gemm")
     tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
     attn = {}
     for l, t in rows:
@@ -157,8 +175,11 @@ def main():
                                "ffn=4096, fp16 (BASELINE.json configs[4])",
                    "launches_per_step": len(prog.launches)},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / PEAK_FP16_TFLOPS, 4), "traffic": None,
-                     "kernel": "gemm_f16_kernel (all %d contraction launches of a step)" % n_gemm,
+                     "frac": round(tflops / PEAK_FP16_TFLOPS, 4),
+                     "traffic": GEMM_TRAFFIC_BYTES_PER_STEP["fetched"] + GEMM_TRAFFIC_BYTES_PER_STEP["written"],
+                     "traffic_note": "bytes per step over the same launches (rocprofv3 FETCH_SIZE + WRITE_SIZE, "
+                                     "calibrated on a copy kernel); algorithmic bytes of those launches: %d" % gemm_bytes,
+                     "kernel": "gemm_f16_pipe_kernel (all %d contraction launches of a step)" % n_gemm,
                      "flops_per_step": gemm_flops, "ms_per_step": round(gemm_ms, 4)},
         "attention_nodes": attn,
         "hbm_nodes": hbm,
