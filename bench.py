@@ -42,6 +42,7 @@ def build_program(device):
     fusion.auto_optimize(sdfg, training=True)
     add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + OB.PARAM_NAMES,
                       grad_dtypes={n: torch.float32 for n in OB.PARAM_NAMES})
+    fusion.optimize_backward(sdfg)
     return CompiledSDFG(sdfg, device=device), OB
 
 

@@ -14,6 +14,7 @@ OK = 0
 ERR_NULL, ERR_SHAPE, ERR_UNSUPPORTED, ERR_ALIGN, ERR_WORKSPACE, ERR_ENUM = -1, -2, -3, -4, -5, -6
 F16, F32 = 0, 1
 ADD, SUB, MUL, DIV, POW = range(5)
+MULTI_MAX = 8  # DMLHIP_MULTI_MAX
 (ERF, SQRT, EXP, LOG, TANH, RELU, SIGMOID, RECIPROCAL, GELU, SWISH, SCALE, IDENTITY) = range(12)
 RSUM, RMAX, RMIN, RMEAN = range(4)
 ACT_NONE, ACT_GELU, ACT_SWISH, ACT_SIGMOID, ACT_RELU = range(5)
@@ -95,6 +96,11 @@ SIGNATURES = {
     "dmlhip_conv2d_backward_data_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P]),
     "dmlhip_conv2d_backward_weight_workspace_bytes": (c_size_t, [POINTER(Conv2dDesc)]),
     "dmlhip_conv2d_backward_weight_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, c_size_t, _P]),
+    "dmlhip_reduce_sum_multi_workspace_bytes": (c_size_t, [c_int, _I64P, _I64P]),
+    "dmlhip_reduce_sum_multi_f16": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), c_int, _I64P, _I64P, _P, c_size_t,
+                                            _P]),
+    "dmlhip_reduce_sum_multi_f32": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), c_int, _I64P, _I64P, _P, c_size_t,
+                                            _P]),
     "dmlhip_attention_f16": (c_int, [POINTER(AttentionDesc), _P, _P, _P, _P, _P, _P]),
     "dmlhip_attention_backward_workspace_bytes": (c_size_t, [POINTER(AttentionDesc)]),
     "dmlhip_attention_backward_f16": (c_int, [POINTER(AttentionDesc), POINTER(AttentionDesc), _P, _P, _P, _P, _P, _P, _P,

@@ -150,7 +150,14 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     const int tiles = g.tiles_m * g.tiles_n;
     const long long batch = bid / tiles;
     const int tile = (int)(bid % tiles);
-    const int tm = tile / g.tiles_n, tn = tile % g.tiles_n;
+    // Tiles are walked in groups of kGroupM tile rows, column by column inside a group: the workgroups that
+    // are resident together (and the contiguous run of tiles an XCD gets) then cover a squarish patch of C and
+    // share few rows of A and few columns of B, which is what fits an XCD's 4 MB L2.
+    constexpr int kGroupM = 8;
+    const int per_group = kGroupM * g.tiles_n;
+    const int group = tile / per_group, in_group = tile % per_group;
+    const int rows_here = min(g.tiles_m - group * kGroupM, kGroupM);
+    const int tm = group * kGroupM + in_group % rows_here, tn = in_group / rows_here;
     const int z2 = (int)(batch % g.batch2);
     const int z1 = (int)((batch / g.batch2) % g.batch1);
     const int z0 = (int)(batch / ((long long)g.batch2 * g.batch1));

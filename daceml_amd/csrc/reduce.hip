@@ -165,6 +165,145 @@ int reduce_typed(const TIn* x, TOut* y, int64_t outer, int64_t r, int64_t inner,
     return launch_status("reduce(partials)");
 }
 
+// ---------------------------------------------------------------- several column sums in one launch pair
+// y_t[c] = sum_r x_t[r, c] for up to DMLHIP_MULTI_MAX independent row-major matrices (the bias gradients of a
+// backward pass: each alone is a latency-bound pair of tiny launches). grid: x = column tiles of the widest
+// matrix, y = row splits, z = matrix; fp32 partials [split][cols] per matrix, then one finishing launch.
+struct MultiRedArgs {
+    const void* x[DMLHIP_MULTI_MAX];
+    void* y[DMLHIP_MULTI_MAX];
+    long long rows[DMLHIP_MULTI_MAX], cols[DMLHIP_MULTI_MAX], part_off[DMLHIP_MULTI_MAX], rows_per_split[DMLHIP_MULTI_MAX];
+    int splits[DMLHIP_MULTI_MAX];
+    int count;
+};
+
+template <typename TIn>
+__global__ __launch_bounds__(kRedBlock) void multi_col_sum_kernel(const MultiRedArgs a, float* __restrict__ part) {
+    constexpr int V = VecOf<TIn>::n;
+    typedef typename VecOf<TIn>::type vec_t;
+    __shared__ float lds[kRedWaves][kWave * V];
+    const int t = blockIdx.z;
+    const long long cols = a.cols[t];
+    if ((int)blockIdx.y >= a.splits[t] || (long long)blockIdx.x * kWave * V >= cols) return;  // whole workgroup leaves
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const long long col = ((long long)blockIdx.x * kWave + lane) * V;
+    const long long r0 = (long long)blockIdx.y * a.rows_per_split[t];
+    const long long r1 = r0 + a.rows_per_split[t] < a.rows[t] ? r0 + a.rows_per_split[t] : a.rows[t];
+    float acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = 0.f;
+    if (col < cols) {
+        const TIn* base = reinterpret_cast<const TIn*>(a.x[t]) + col;
+        long long i = r0 + wave;
+        for (; i + 3 * kRedWaves < r1; i += 4 * kRedWaves) {
+            const vec_t v0 = *reinterpret_cast<const vec_t*>(base + i * cols);
+            const vec_t v1 = *reinterpret_cast<const vec_t*>(base + (i + kRedWaves) * cols);
+            const vec_t v2 = *reinterpret_cast<const vec_t*>(base + (i + 2 * kRedWaves) * cols);
+            const vec_t v3 = *reinterpret_cast<const vec_t*>(base + (i + 3 * kRedWaves) * cols);
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc[e] += (to_f32(v0[e]) + to_f32(v1[e])) + (to_f32(v2[e]) + to_f32(v3[e]));
+        }
+        for (; i < r1; i += kRedWaves) {
+            const vec_t v = *reinterpret_cast<const vec_t*>(base + i * cols);
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc[e] += to_f32(v[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) lds[wave][lane * V + e] = acc[e];
+    __syncthreads();
+    if (wave == 0 && col < cols) {
+        float* out = part + a.part_off[t] + (long long)blockIdx.y * cols + col;
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            float s = lds[0][lane * V + e];
+#pragma unroll
+            for (int w = 1; w < kRedWaves; ++w) s += lds[w][lane * V + e];
+            out[e] = s;
+        }
+    }
+}
+
+template <typename TOut>
+__global__ __launch_bounds__(1024) void multi_partials_kernel(const MultiRedArgs a, const float* __restrict__ part) {
+    __shared__ float lds[16][kWave];
+    const int t = blockIdx.y;
+    const long long cols = a.cols[t];
+    if ((long long)blockIdx.x * kWave >= cols) return;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const long long c = (long long)blockIdx.x * kWave + lane;
+    float s = 0.f;
+    if (c < cols) {
+        const float* base = part + a.part_off[t] + c;
+        for (int p = wave; p < a.splits[t]; p += 16) s += base[(long long)p * cols];
+    }
+    lds[wave][lane] = s;
+    __syncthreads();
+    if (wave == 0 && c < cols) {
+        float v = lds[0][lane];
+#pragma unroll
+        for (int w = 1; w < 16; ++w) v += lds[w][lane];
+        reinterpret_cast<TOut*>(a.y[t])[c] = from_f32<TOut>(v);
+    }
+}
+
+int multi_plan(int count, const int64_t* rows, const int64_t* cols, MultiRedArgs& a, long long& part_floats, int& max_splits,
+               long long& max_cols) {
+    DML_REQUIRE(count >= 1 && count <= DMLHIP_MULTI_MAX, DMLHIP_ERR_SHAPE, "reduce_sum_multi: count %d outside 1..%d", count,
+                DMLHIP_MULTI_MAX);
+    DML_REQUIRE(rows && cols, DMLHIP_ERR_NULL, "reduce_sum_multi: NULL extents");
+    part_floats = 0;
+    max_splits = 1;
+    max_cols = 0;
+    a.count = count;
+    for (int t = 0; t < count; ++t) {
+        DML_REQUIRE(rows[t] >= 0 && cols[t] >= 0 && rows[t] <= (1LL << 40) && cols[t] <= (1LL << 31), DMLHIP_ERR_SHAPE,
+                    "reduce_sum_multi: bad extent");
+        a.rows[t] = rows[t];
+        a.cols[t] = cols[t];
+        long long splits = ceil_div(rows[t] > 0 ? rows[t] : 1, 64);   // 64 rows (16 per wavefront) per workgroup
+        if (splits > 256) splits = 256;
+        a.rows_per_split[t] = ceil_div(rows[t] > 0 ? rows[t] : 1, splits);
+        a.splits[t] = (int)ceil_div(rows[t] > 0 ? rows[t] : 1, a.rows_per_split[t]);
+        a.part_off[t] = part_floats;
+        part_floats += (long long)a.splits[t] * cols[t];
+        if (a.splits[t] > max_splits) max_splits = a.splits[t];
+        if (cols[t] > max_cols) max_cols = cols[t];
+    }
+    return 0;
+}
+
+template <typename TIn>
+int reduce_sum_multi_impl(int count, const void* const* x, void* const* y, int out_dtype, const int64_t* rows,
+                          const int64_t* cols, void* ws, size_t ws_bytes, void* stream) {
+    DML_REQUIRE(out_dtype == DMLHIP_F16 || out_dtype == DMLHIP_F32, DMLHIP_ERR_ENUM, "reduce_sum_multi: unknown out_dtype");
+    DML_REQUIRE(x && y, DMLHIP_ERR_NULL, "reduce_sum_multi: NULL pointer table");
+    MultiRedArgs a = {};
+    long long part_floats, max_cols;
+    int max_splits;
+    if (int e = multi_plan(count, rows, cols, a, part_floats, max_splits, max_cols)) return e;
+    constexpr int V = VecOf<TIn>::n;
+    for (int t = 0; t < count; ++t) {
+        DML_REQUIRE(y[t] && (x[t] || rows[t] == 0 || cols[t] == 0), DMLHIP_ERR_NULL, "reduce_sum_multi: NULL tensor %d", t);
+        DML_REQUIRE(cols[t] % V == 0 && aligned16(x[t]), DMLHIP_ERR_ALIGN,
+                    "reduce_sum_multi: matrix %d needs 16-byte aligned rows (cols %% %d == 0)", t, V);
+        a.x[t] = x[t];
+        a.y[t] = y[t];
+    }
+    if (max_cols == 0) return 0;
+    DML_REQUIRE(ws && ws_bytes >= (size_t)part_floats * sizeof(float), DMLHIP_ERR_WORKSPACE,
+                "reduce_sum_multi: workspace of %zu bytes needed, %zu given", (size_t)part_floats * sizeof(float), ws_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL((multi_col_sum_kernel<TIn>), dim3((unsigned)ceil_div(max_cols, (int64_t)kWave * V), (unsigned)max_splits,
+                                                         (unsigned)count),
+                       kRedBlock, 0, st, a, (float*)ws);
+    if (int e = launch_status("reduce_sum_multi(stage 1)")) return e;
+    const dim3 g2((unsigned)ceil_div(max_cols, kWave), (unsigned)count);
+    if (out_dtype == DMLHIP_F32) hipLaunchKernelGGL((multi_partials_kernel<float>), g2, 1024, 0, st, a, (const float*)ws);
+    else hipLaunchKernelGGL((multi_partials_kernel<_Float16>), g2, 1024, 0, st, a, (const float*)ws);
+    return launch_status("reduce_sum_multi(stage 2)");
+}
+
 template <typename TIn>
 int reduce_impl(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r, int64_t inner, void* ws,
                 size_t ws_bytes, void* stream) {
@@ -211,6 +350,22 @@ size_t dmlhip_reduce_workspace_bytes(int64_t outer, int64_t r, int64_t inner) {
     if (splits > max_splits) splits = max_splits;
     if (splits <= 1) return 0;
     return (size_t)(splits + 1) * outer * inner * sizeof(float);
+}
+
+size_t dmlhip_reduce_sum_multi_workspace_bytes(int count, const int64_t* rows, const int64_t* cols) {
+    MultiRedArgs a = {};
+    long long part_floats = 0, max_cols;
+    int max_splits;
+    if (multi_plan(count, rows, cols, a, part_floats, max_splits, max_cols)) return 0;
+    return (size_t)part_floats * sizeof(float);
+}
+int dmlhip_reduce_sum_multi_f16(int count, const void* const* x, void* const* y, int out_dtype, const int64_t* rows,
+                                const int64_t* cols, void* workspace, size_t workspace_bytes, void* stream) {
+    return reduce_sum_multi_impl<_Float16>(count, x, y, out_dtype, rows, cols, workspace, workspace_bytes, stream);
+}
+int dmlhip_reduce_sum_multi_f32(int count, const void* const* x, void* const* y, int out_dtype, const int64_t* rows,
+                                const int64_t* cols, void* workspace, size_t workspace_bytes, void* stream) {
+    return reduce_sum_multi_impl<float>(count, x, y, out_dtype, rows, cols, workspace, workspace_bytes, stream);
 }
 
 int dmlhip_reduce_f16(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r, int64_t inner,

@@ -464,3 +464,22 @@ def attention_backward(q, k, v, out, lse, dout, scale):
                                               _ptr(lse), _ptr(dout), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(),
                                               _stream()))
     return dq, dk, dv
+
+
+def reduce_sum_multi(xs: Sequence[torch.Tensor], out_dtype: Optional[torch.dtype] = None):
+    """[x.sum over all axes but the last for x in xs] in one launch pair (at most eight tensors)."""
+    _check(*xs, dtype=xs[0].dtype)
+    xs = [_dense(x) for x in xs]
+    odt = out_dtype or xs[0].dtype
+    ys = [torch.empty((x.shape[-1], ), dtype=odt, device=x.device) for x in xs]
+    n = len(xs)
+    rows = (ctypes.c_int64 * n)(*[x.numel() // max(x.shape[-1], 1) for x in xs])
+    cols = (ctypes.c_int64 * n)(*[x.shape[-1] for x in xs])
+    xp = (ctypes.c_void_p * n)(*[x.data_ptr() for x in xs])
+    yp = (ctypes.c_void_p * n)(*[y.data_ptr() for y in ys])
+    lib = L.load()
+    need = lib.dmlhip_reduce_sum_multi_workspace_bytes(n, rows, cols)
+    ws = workspace(need, xs[0].device)
+    L.check(_fn("reduce_sum_multi", xs[0].dtype)(n, xp, yp, L.F16 if odt == torch.float16 else L.F32, rows, cols, _ptr(ws),
+                                                  ws.numel(), _stream()))
+    return ys

@@ -130,6 +130,9 @@ SCHEMAS = [
             v_perm=REQUIRED, o_perm=REQUIRED),
     _schema("FusedAttentionGrad", "Q K V O LogSumExp dO", "dQ dK dV", since=1, scale=1.0, q_perm=REQUIRED,
             k_perm=REQUIRED, v_perm=REQUIRED, o_perm=REQUIRED),
+    # several independent ReduceSum(all leading axes, keepdims=0) nodes in one launch pair: reduced__i = sum of
+    # data__i over every axis but the last (the bias gradients of a backward pass)
+    _schema("MultiReduceSum", "data*", "reduced*", since=1),
     # backward nodes emitted by the "hip" BackwardImplementations (names follow the ONNX Runtime
     # training contrib ops)
     _schema("SoftmaxGrad", "dY Y", "dX", since=1, axis=-1),

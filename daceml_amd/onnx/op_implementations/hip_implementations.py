@@ -1007,3 +1007,50 @@ class HipFusedAttentionGrad(ONNXForward):
                        
                         bytes_moved=_nbytes(ins["Q"], ins["K"], ins["V"], ins["O"], ins["dO"], outs["dQ"], outs["dK"],
                                             outs["dV"]), kind="attention_backward")
+
+
+# ----------------------------------------------------------------------------- several ReduceSum nodes at once
+@op_implementation(op="MultiReduceSum", name=IMPL)
+class HipMultiReduceSum(ONNXForward):
+    """reduced__i = np.sum(data__i, axis=all but the last) (ReduceSum, pure_implementations.py:294-306, keepdims 0)
+    for up to eight tensors in one pair of launches."""
+    @staticmethod
+    def _pairs(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        n = len(ins)
+        return [(ins["data__%d" % i], outs["reduced__%d" % i]) for i in range(n)]
+
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            pairs = HipMultiReduceSum._pairs(node, state, sdfg)
+            if not 1 <= len(pairs) <= L.MULTI_MAX:
+                return False
+            dt, odt = pairs[0][0].dtype, pairs[0][1].dtype
+            vec = 8 if dt == torch.float16 else 4
+            for x, y in pairs:
+                if x.dtype != dt or y.dtype != odt or dt not in FLOAT_DTYPES or odt not in FLOAT_DTYPES:
+                    return False
+                if not (x.is_contiguous() and y.is_contiguous()) or len(x.shape) < 1:
+                    return False
+                if y.total_size != x.shape[-1] or x.shape[-1] % vec:
+                    return False
+            return True
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        import ctypes
+        pairs = HipMultiReduceSum._pairs(node, state, sdfg)
+        n = len(pairs)
+        rows = tuple(_prod(x.shape[:-1]) for x, _ in pairs)
+        cols = tuple(int(x.shape[-1]) for x, _ in pairs)
+        r_arr, c_arr = (ctypes.c_int64 * n)(*rows), (ctypes.c_int64 * n)(*cols)
+        ws = L.load().dmlhip_reduce_sum_multi_workspace_bytes(n, r_arr, c_arr)
+        call = HipCall("dmlhip_reduce_sum_multi_" + _SFX[pairs[0][0].dtype],
+                       [I32(n), PtrArray(tuple("data__%d" % i for i in range(n))),
+                        PtrArray(tuple("reduced__%d" % i for i in range(n))), I32(_CODE[pairs[0][1].dtype]),
+                        I64Array(rows), I64Array(cols), Workspace(), WorkspaceBytes(), Stream()])
+        return _tasklet(node, state, [call], workspace_bytes=ws,
+                        bytes_moved=sum(_nbytes(x, y) for x, y in pairs), kind="reduce")

@@ -18,6 +18,7 @@ expansions it replaces (that composition is the oracle of the fused kernels).
                              [Add residual]                               -> FusedEinsum
     fuse_skip_layernorm      Add, LayerNormalization                      -> SkipLayerNormalization
     fuse_attention           Einsum(Q,K)[*scale], Softmax, Einsum(P,V)    -> FusedAttention
+    fuse_reductions          independent ReduceSum(leading axes) nodes    -> MultiReduceSum (one launch pair)
     fuse_conv_activation     Conv, Swish | Sigmoid | Relu                 -> Conv(_activation)
 """
 import math
@@ -636,6 +637,47 @@ def fuse_attention(sdfg: SDFG) -> int:
     if count:
         _drop_unused_arrays(sdfg)
     return count
+
+
+def fuse_reductions(sdfg: SDFG, max_group: int = 8) -> int:
+    """Horizontal fusion (cf. HorizontalEinsumFusion, daceml/transformation/einsum_fusion.py:102-151) of ReduceSum
+    nodes that sum over every axis but the last with keepdims=0 and whose results nobody in the state reads
+    (bias gradients): each is a latency-bound pair of tiny launches on its own. Returns the number of nodes
+    that were merged away."""
+    merged = 0
+    for state in sdfg.states():
+        cands = {}
+        for n in state.nodes():
+            if not _is_op(n, "ReduceSum") or n.keepdims:
+                continue
+            x, y = _in_array(state, n, "data"), _out_array(state, n, "reduced")
+            xd, yd = sdfg.arrays[x], sdfg.arrays[y]
+            nd = len(xd.shape)
+            axes = sorted(a % nd for a in (n.axes if n.axes is not None else range(nd)))
+            if nd < 2 or axes != list(range(nd - 1)) or _consumers(state, y):
+                continue
+            vec = 8 if xd.dtype == torch.float16 else 4
+            if not (xd.is_contiguous() and yd.is_contiguous()) or xd.shape[-1] % vec or xd.dtype not in (torch.float16, torch.float32):
+                continue
+            cands.setdefault((xd.dtype, yd.dtype), []).append((n, x, y))
+        for group in cands.values():
+            for i in range(0, len(group), max_group):
+                part = group[i:i + max_group]
+                if len(part) < 2:
+                    continue
+                ins = {"data__%d" % j: x for j, (_, x, _) in enumerate(part)}
+                outs = {"reduced__%d" % j: y for j, (_, _, y) in enumerate(part)}
+                for n, _, _ in part:
+                    _remove_node(state, n)
+                _add_node(sdfg, state, "MultiReduceSum", "multi_" + part[0][0].label, ins, outs)
+                merged += len(part) - 1
+    return merged
+
+
+def optimize_backward(sdfg: SDFG) -> Dict[str, int]:
+    """Rewrites for the state(s) autodiff added — what a ``post_autodiff_hooks`` entry of the reference's module
+    wrapper would run (daceml/torch/module.py:46-365)."""
+    return {"reductions": fuse_reductions(sdfg)}
 
 
 def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True) -> Dict[str, int]:

@@ -151,6 +151,20 @@ int dmlhip_reduce_f16(int op, const void* x, void* y, int out_dtype, int64_t out
                       int64_t inner, void* workspace, size_t workspace_bytes, void* stream);
 int dmlhip_reduce_f32(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r,
                       int64_t inner, void* workspace, size_t workspace_bytes, void* stream);
+/* Several independent ReduceSum nodes over all leading axes (keepdims = 0) in one launch pair:
+ * y[t][c] = sum_r x[t][r, c] for count <= DMLHIP_MULTI_MAX row-major matrices [rows[t], cols[t]].
+ * This is the shape of the bias gradients DefaultEinsumBackward's callers need
+ * (autodiff/implementations/onnx_ops.py:54-138 leaves them to ReduceSum, pure_implementations.py:
+ * 294-306); each alone is two latency-bound launches. cols[t] must keep rows 16-byte aligned.
+ * All outputs have element type out_dtype. */
+#define DMLHIP_MULTI_MAX 8
+size_t dmlhip_reduce_sum_multi_workspace_bytes(int count, const int64_t* rows, const int64_t* cols);
+int dmlhip_reduce_sum_multi_f16(int count, const void* const* x, void* const* y, int out_dtype,
+                                const int64_t* rows, const int64_t* cols, void* workspace,
+                                size_t workspace_bytes, void* stream);
+int dmlhip_reduce_sum_multi_f32(int count, const void* const* x, void* const* y, int out_dtype,
+                                const int64_t* rows, const int64_t* cols, void* workspace,
+                                size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ Transpose
  * Transpose "pure"/"einsum": pure_implementations.py:322-326,746-778.

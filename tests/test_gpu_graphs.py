@@ -71,10 +71,12 @@ def test_bert_layer_backward(dtype, attention):
     fusion.auto_optimize(sdfg, training=True, attention=attention)
     grads = add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + OB.PARAM_NAMES,
                               grad_dtypes={n: torch.float32 for n in OB.PARAM_NAMES})
+    if attention:
+        assert fusion.optimize_backward(sdfg)["reductions"] == 5   # six bias gradients -> one MultiReduceSum
     # the backward state contains only nodes with hand-written kernels
     bnames = {n.schema.name for n in sdfg.states()[1].library_nodes()}
     if attention:
-        assert bnames == {"FusedEinsum", "FusedAttentionGrad", "LayerNormalizationGrad", "GeluGrad", "ReduceSum", "Sum"}
+        assert bnames == {"FusedEinsum", "FusedAttentionGrad", "LayerNormalizationGrad", "GeluGrad", "MultiReduceSum", "Sum"}
     else:
         assert bnames == {"FusedEinsum", "SoftmaxGrad", "LayerNormalizationGrad", "GeluGrad", "ReduceSum", "Sum"}
     prog = _compile(sdfg)

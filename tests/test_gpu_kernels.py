@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from oracle import ops as O
-from tests.util import assert_close, dev, host, rng
+from tests.util import assert_close, dev, host, rng, tol
 
 pytestmark = pytest.mark.gpu
 
@@ -478,3 +478,22 @@ def test_attention_backward(b0, b1, sq, sk, layout):
         s = max(1.0, float(np.abs(want).max()))
         assert_close(host(got), want, torch.float16, "attention backward %s %s" % (name, (b0, b1, sq, sk, layout)),
                      atol=1e-2 * s)
+
+
+# ----------------------------------------------------------------------------- several column sums in one launch
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_reduce_sum_multi(dtype):
+    from daceml_amd import kernels as K
+    shapes = [(4096, 1024), (2, 300, 64), (1, 8), (777, 4096), (5, 3, 7, 128), (64, 8), (16000, 16), (3, 24)]
+    pairs = [_inputs(200 + i, s, dtype) for i, s in enumerate(shapes)]
+    got = K.reduce_sum_multi([dev(x) for x, _ in pairs], out_dtype=torch.float32)
+    for (x, x64), g, s in zip(pairs, got, shapes):
+        want = O.reduce_sum(x64, list(range(len(s) - 1)), 0)
+        n = x.size // s[-1]
+        assert_close(host(g), want, torch.float32, "reduce_sum_multi %s" % (s, ), rtol=1e-5, atol=1e-6 * max(1.0, np.sqrt(n)))
+    # a single tensor, output in the input type
+    one = K.reduce_sum_multi([dev(pairs[1][0])])
+    assert one[0].dtype == dtype
+    r, a = tol(dtype)
+    assert_close(host(one[0]), O.reduce_sum(pairs[1][1], [0, 1], 0), dtype, "reduce_sum_multi single",
+                 atol=a * np.sqrt(600))  # sums of 600 terms

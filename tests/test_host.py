@@ -348,6 +348,14 @@ def test_attention_fusion_roles_and_graph():
     assert len(back) == 1
     ins = {e.dst_conn for e in sdfg.states()[1].in_edges(back[0])}
     assert ins == {"Q", "K", "V", "O", "LogSumExp", "dO"}
+    # the six bias gradients become one node; nothing else in the state changes
+    n_before = len(sdfg.states()[1].library_nodes())
+    assert fusion.optimize_backward(sdfg) == {"reductions": 5}
+    bnodes = sdfg.states()[1].library_nodes()
+    assert len(bnodes) == n_before - 5 and not any(n.schema.name == "ReduceSum" for n in bnodes)
+    multi = [n for n in bnodes if n.schema.name == "MultiReduceSum"][0]
+    outs = sorted(e.data.data for e in sdfg.states()[1].out_edges(multi))
+    assert outs == sorted("gradient_%s_b" % p for p in ("q", "k", "v", "o", "ffn1", "ffn2"))
     # the forward node now also emits the log-sum-exp rows
     assert "LogSumExp" in {e.src_conn for e in st.out_edges(att)}
     # fp32 graphs keep the unfused chain (the kernel is fp16 only)
