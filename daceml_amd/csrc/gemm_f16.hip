@@ -259,25 +259,21 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_kernel(const _Float16* __re
         char* cur = lds + (kt & 1) * (A_BYTES + B_BYTES);
         char* nxt = lds + ((kt + 1) & 1) * (A_BYTES + B_BYTES);
         const bool more = kt + 1 < nk;
-#ifndef LAB_NO_GLOBAL
         if (more) {
             if constexpr (AMODE == 3) la.issue(A, (kt + 1) * BK, nxt);
             if constexpr (BMODE == 3) lb.issue(B, (kt + 1) * BK, nxt + A_BYTES);
             la.load(A, g.sak, (kt + 1) * BK, g.k);
             lb.load(B, g.sbk, (kt + 1) * BK, g.k);
         }
-#endif
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
             if (kk + 1 < BK / 16) {
                 read_frags(cur, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
             } else {
-#ifndef LAB_NO_STORE
                 if (more) {
                     la.store(nxt);
                     lb.store(nxt + A_BYTES);
                 }
-#endif
                 __syncthreads();
                 if (more) read_frags(nxt, 0, af[0], bf[0]);
             }

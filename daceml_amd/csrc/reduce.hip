@@ -195,13 +195,18 @@ __global__ __launch_bounds__(kRedBlock) void multi_col_sum_kernel(const MultiRed
     if (col < cols) {
         const TIn* base = reinterpret_cast<const TIn*>(a.x[t]) + col;
         long long i = r0 + wave;
-        for (; i + 3 * kRedWaves < r1; i += 4 * kRedWaves) {
-            const vec_t v0 = *reinterpret_cast<const vec_t*>(base + i * cols);
-            const vec_t v1 = *reinterpret_cast<const vec_t*>(base + (i + kRedWaves) * cols);
-            const vec_t v2 = *reinterpret_cast<const vec_t*>(base + (i + 2 * kRedWaves) * cols);
-            const vec_t v3 = *reinterpret_cast<const vec_t*>(base + (i + 3 * kRedWaves) * cols);
+        constexpr int U = 8;  // independent 16-byte loads in flight per lane
+        for (; i + (U - 1) * kRedWaves < r1; i += U * kRedWaves) {
+            vec_t v[U];
 #pragma unroll
-            for (int e = 0; e < V; ++e) acc[e] += (to_f32(v0[e]) + to_f32(v1[e])) + (to_f32(v2[e]) + to_f32(v3[e]));
+            for (int u = 0; u < U; ++u) v[u] = *reinterpret_cast<const vec_t*>(base + (i + u * kRedWaves) * cols);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                float s = 0.f;
+#pragma unroll
+                for (int u = 0; u < U; ++u) s += to_f32(v[u][e]);
+                acc[e] += s;
+            }
         }
         for (; i < r1; i += kRedWaves) {
             const vec_t v = *reinterpret_cast<const vec_t*>(base + i * cols);
@@ -261,7 +266,7 @@ int multi_plan(int count, const int64_t* rows, const int64_t* cols, MultiRedArgs
                     "reduce_sum_multi: bad extent");
         a.rows[t] = rows[t];
         a.cols[t] = cols[t];
-        long long splits = ceil_div(rows[t] > 0 ? rows[t] : 1, 64);   // 64 rows (16 per wavefront) per workgroup
+        long long splits = ceil_div(rows[t] > 0 ? rows[t] : 1, 128);   // 128 rows (32 per wavefront) per workgroup
         if (splits > 256) splits = 256;
         a.rows_per_split[t] = ceil_div(rows[t] > 0 ? rows[t] : 1, splits);
         a.splits[t] = (int)ceil_div(rows[t] > 0 ? rows[t] : 1, a.rows_per_split[t]);
