@@ -101,8 +101,117 @@ def cpu_baseline(OB, x, dy, p, budget_s=25.0):
                       "expansions in fp32, best of them" % len(times)}
 
 
+# ----------------------------------------------------------------------------- the other configurations
+def _time_program(prog, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        prog.launch()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        prog.launch()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
+def secondary_workload(name, device, steps, warmup, verbose):
+    """BASELINE.json configs[0..3]: parity-test cases that are also worth a measured line. Same JSON keys as the
+    headline; `roofline` is that of the launch that takes the most time."""
+    import numpy as np
+    import torch
+    from daceml_amd import graphs
+    from daceml_amd.runtime import CompiledSDFG
+    from daceml_amd.transformation import fusion
+    rng = np.random.default_rng(1234)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    if name == "bert_fwd":
+        from oracle import bert_layer as OB
+        sdfg = graphs.bert_encoder_layer(B, S, H, HEADS, FFN, torch.float16, eps=1e-12)
+        fusion.auto_optimize(sdfg)
+        p = OB.init_params(H, FFN, 1234 + 2, np.float32)
+        args = {n: dev(p[n].astype(np.float16)) for n in OB.PARAM_NAMES}
+        args["x"] = dev(rng.standard_normal((B, S, H)).astype(np.float16))
+        args["y"] = torch.empty((B, S, H), dtype=torch.float16, device=device)
+        what, dtype = "BERT-large encoder layer forward, B=8 S=512, fp16 (BASELINE.json configs[2])", "f16"
+    elif name == "nodes":
+        g = graphs.GraphBuilder("memory_bound_nodes", torch.float16)
+        sc = g.input("scores", (8, 16, 512, 512))
+        pr = g.node("Softmax", {"input": sc}, {"output": (8, 16, 512, 512)}, label="softmax", axis=-1)["output"]
+        g.output(pr, "probs")
+        xin = g.input("x", (8, 512, 1024))
+        g.input("gamma", (1024, ))
+        g.input("beta", (1024, ))
+        g.output(g.layer_norm(xin, "gamma", "beta", 1e-5, "ln"), "y")
+        sdfg = g.sdfg
+        fusion.auto_optimize(sdfg)
+        args = {"scores": dev(rng.standard_normal((8, 16, 512, 512)).astype(np.float16)),
+                "probs": torch.empty((8, 16, 512, 512), dtype=torch.float16, device=device),
+                "x": dev(rng.standard_normal((8, 512, 1024)).astype(np.float16)),
+                "gamma": dev(rng.uniform(0.5, 1.5, 1024).astype(np.float16)),
+                "beta": dev((rng.standard_normal(1024) * 0.1).astype(np.float16)),
+                "y": torch.empty((8, 512, 1024), dtype=torch.float16, device=device)}
+        what, dtype = "Softmax [8,16,512,512] and LayerNorm chain [8,512,1024], fp16 (BASELINE.json configs[1])", "f16"
+    elif name == "mbconv":
+        sdfg = graphs.mbconv_block(96, 32, 112)
+        fusion.auto_optimize(sdfg)
+        shapes = {"expand": (192, 32, 1, 1), "dw": (192, 1, 3, 3), "se1": (8, 192, 1, 1), "se2": (192, 8, 1, 1),
+                  "proj": (48, 192, 1, 1)}
+        args = {"x": dev(rng.standard_normal((96, 32, 112, 112)).astype(np.float32)),
+                "y": torch.empty((96, 48, 56, 56), dtype=torch.float32, device=device)}
+        for n, shp in shapes.items():
+            fan_in = shp[1] * shp[2] * shp[3]
+            args[n + "_w"] = dev((rng.standard_normal(shp) * np.sqrt(2.0 / fan_in)).astype(np.float32))
+            args[n + "_b"] = dev((rng.standard_normal(shp[0]) * 0.1).astype(np.float32))
+        what, dtype = "EfficientNet-B0 MBConv block, batch 96, [96,32,112,112], fp32 (BASELINE.json configs[3])", "f32"
+    elif name == "conv":
+        g = graphs.GraphBuilder("conv_c1", torch.float32)
+        xin = g.input("x", (5, 3, 10, 10))
+        g.input("w", (16, 3, 3, 3))
+        g.output(g.node("Conv", {"X": xin, "W": "w"}, {"Y": (5, 16, 4, 4)}, label="conv", kernel_shape=[3, 3],
+                        strides=[2, 2])["Y"], "y")
+        sdfg = g.sdfg
+        args = {"x": dev(rng.uniform(0, 1, (5, 3, 10, 10)).astype(np.float32)),
+                "w": dev(rng.uniform(0, 1, (16, 3, 3, 3)).astype(np.float32)),
+                "y": torch.empty((5, 16, 4, 4), dtype=torch.float32, device=device)}
+        what, dtype = "single Conv fp32 X[5,3,10,10] W[16,3,3,3] stride 2 (BASELINE.json configs[0]; launch latency)", "f32"
+    else:
+        sys.exit("unknown workload %r" % name)
+    prog = CompiledSDFG(sdfg, device=device)
+    prog(**args)
+    ms = _time_program(prog, steps, warmup)
+    rows = kernel_breakdown(prog)
+    launches = []
+    for l, t in rows:
+        e = {"label": l.label, "kind": l.kind, "us": round(t * 1e3, 2)}
+        if l.flops:
+            e["TFLOP/s"] = round(l.flops / (t * 1e-3) / 1e12, 2)
+        if l.bytes_moved:
+            e["GB/s"] = round(l.bytes_moved / (t * 1e-3) / 1e9, 1)
+        launches.append(e)
+        if verbose:
+            sys.stderr.write("%-28s %-40s %8.1f us %s\n" % (l.kind, l.label[:40], t * 1e3, {k: v for k, v in e.items()
+                                                                                             if "/s" in k}))
+    top, top_t = max(rows, key=lambda r: r[1])
+    if top.kind in ("gemm", "attention") and dtype == "f16":
+        roof = {"bound": "mfma", "achieved": round(top.flops / (top_t * 1e-3) / 1e12, 1), "peak": PEAK_FP16_TFLOPS,
+                "unit": "TFLOP/s"}
+    else:
+        roof = {"bound": "hbm", "achieved": round(top.bytes_moved / (top_t * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                "unit": "GB/s"}
+    roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
+    roof["traffic"] = None
+    roof["kernel"] = top.label
+    print(json.dumps({"metric": what + " ms/iter at 1 GPU", "value": round(ms, 4), "unit": "ms/iter", "n_gpus": 1,
+                      "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
+                      "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+                      "config": {"workload": what, "launches_per_step": len(prog.launches)}, "roofline": roof,
+                      "launches": launches}))
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--workload", default="bert_fwd_bwd", choices=["bert_fwd_bwd", "bert_fwd", "nodes", "mbconv", "conv"],
+                    help="bert_fwd_bwd is the headline (default); the others are BASELINE.json's remaining configs")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
@@ -120,6 +229,9 @@ def main():
         sys.exit("bench.py needs a GPU")
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
+
+    if a.workload != "bert_fwd_bwd":
+        return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose)
 
     prog, OB = build_program(device)
     args, x, dy, p = synthetic_inputs(OB, device)

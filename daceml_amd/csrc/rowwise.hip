@@ -282,18 +282,37 @@ __global__ __launch_bounds__(kRowBlock) void layernorm_bwd_wave_kernel(
 #pragma unroll
         for (int e = 0; e < VN; ++e) { g[j][e] = to_f32(t[e]); accg[j][e] = 0.f; accb[j][e] = 0.f; }
     }
-    for (int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + wave; row < rows;
-         row += (int64_t)gridDim.x * kRowsPerBlock) {
-        const float mu = mean[row], inv = rstd[row];
-        const V* xr = reinterpret_cast<const V*>(x + row * cols);
-        const V* gr = reinterpret_cast<const V*>(dy + row * cols);
+    // The rows of a wavefront are software-pipelined: the loads of its next row are issued before the current
+    // row is reduced, so a workgroup's short chain of rows is not a chain of full memory round trips.
+    const int64_t row_step = (int64_t)gridDim.x * kRowsPerBlock;
+    int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + wave;
+    V a_nxt[VPL], b_nxt[VPL];
+    float mu_nxt = 0.f, inv_nxt = 0.f;
+    auto fetch = [&](int64_t r) {
+        mu_nxt = mean[r];
+        inv_nxt = rstd[r];
+        const V* xr = reinterpret_cast<const V*>(x + r * cols);
+        const V* gr = reinterpret_cast<const V*>(dy + r * cols);
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const int vi = lane + j * kWave;
+            if (vi < nvec) { a_nxt[j] = xr[vi]; b_nxt[j] = gr[vi]; }
+        }
+    };
+    if (row < rows) fetch(row);
+    for (; row < rows; row += row_step) {
+        const float mu = mu_nxt, inv = inv_nxt;
+        V a_cur[VPL], b_cur[VPL];
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) { a_cur[j] = a_nxt[j]; b_cur[j] = b_nxt[j]; }
+        if (row + row_step < rows) fetch(row + row_step);
         float xh[VPL][VN], gd[VPL][VN];
         float s1 = 0.f, s2 = 0.f;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
             const int vi = lane + j * kWave;
             if (vi < nvec) {
-                V a = xr[vi], b = gr[vi];
+                const V a = a_cur[j], b = b_cur[j];
 #pragma unroll
                 for (int e = 0; e < VN; ++e) {
                     const float d = to_f32(b[e]);
