@@ -156,6 +156,12 @@ __device__ __forceinline__ float gelu_grad_f(float x) {
     return cdf + x * pdf;
 }
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+// Sigmoid for fused epilogues, on the hardware exp2 and reciprocal (each accurate to about one ulp, so the result
+// is within a few 1e-7 relative of sigmoid_f): an epilogue runs once per output element while the matrix pipe waits,
+// and the library expf plus a true division cost several times the arithmetic of the product itself there.
+__device__ __forceinline__ float sigmoid_epilogue_f(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * x));
+}
 
 // GELU for fp16 tensors: erf by Abramowitz-Stegun 7.1.26 (absolute error < 1.5e-7, far below the
 // half-precision rounding of the result) on the hardware exp2 / reciprocal. Not used on fp32 paths.
@@ -180,8 +186,8 @@ __device__ __forceinline__ float apply_act_half(int act, float v) {
 __device__ __forceinline__ float apply_act(int act, float v) {
     switch (act) {
         case DMLHIP_ACT_GELU: return gelu_f(v);
-        case DMLHIP_ACT_SWISH: return v * sigmoid_f(v);
-        case DMLHIP_ACT_SIGMOID: return sigmoid_f(v);
+        case DMLHIP_ACT_SWISH: return v * sigmoid_epilogue_f(v);
+        case DMLHIP_ACT_SIGMOID: return sigmoid_epilogue_f(v);
         case DMLHIP_ACT_RELU: return fmaxf(v, 0.f);
         default: return v;
     }

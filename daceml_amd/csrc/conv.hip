@@ -8,6 +8,8 @@
 //     sequentially in fp32 — the summation order of the reference's pure expansion.
 #include "common.h"
 
+#include <type_traits>
+
 namespace dml {
 namespace {
 
@@ -147,6 +149,139 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const float* __res
     if (threadIdx.x == 0) dw[blockIdx.x] = acc;
 }
 
+
+// ---------------------------------------------------------------- pointwise (1x1) convolution, fp32
+// Y[n, m, p] = act(sum_c W[m, c] * s[n, c] * X[n, c, p] + b[m]) with p running over the h*w pixels: per image a
+// GEMM with a short K (the input channels) and a very long, contiguous N. It is bound by the output write, so the
+// kernel is organised around reading X exactly once and writing Y in full 128-byte rows: a workgroup takes 256
+// pixels of one image and up to 192 output channels; X goes through LDS in chunks of 32 channels, W chunk by chunk
+// as well; every wavefront multiplies all output channels with its 64 pixels on v_mfma_f32_32x32x2f32 (true fp32).
+// A = W (rows = output channels), B = X (columns = pixels): a lane's accumulators are 16 output channels of ONE
+// pixel, so stores of a wavefront run along the pixels. `in_scale` (optional) is a per-image, per-input-channel
+// factor applied to X on its way into LDS (the squeeze-excite gate in front of a projection).
+template <int MT, int PT>  // 32-channel blocks per workgroup; 32-pixel blocks per wavefront
+__global__ __launch_bounds__(256, 2) void conv_pointwise_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                    const float* __restrict__ bias,
+                                                                    const float* __restrict__ in_scale, float* __restrict__ y,
+                                                                    int cin, int cout, int64_t hw, int act) {
+    constexpr int PX = 128 * PT, KC = 32, XP = PX + 32, WP = KC + 1;
+    extern __shared__ float pw_lds[];
+    float* xs = pw_lds;                 // [KC][XP]   pitch: rows k and k+1 land in different bank halves
+    float* ws = xs + KC * XP;           // [MT*32][WP]
+    float* bs = ws + MT * 32 * WP;      // [MT*32]
+    const int n = blockIdx.y;
+    const int64_t p0 = (int64_t)blockIdx.x * PX;
+    const int m0 = blockIdx.z * MT * 32;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int pwv = wave * 32 * PT;
+
+    floatx16 acc[MT][PT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < PT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    if (threadIdx.x < MT * 32) bs[threadIdx.x] = (bias && m0 + (int)threadIdx.x < cout) ? bias[m0 + threadIdx.x] : 0.f;
+    const float* xn = x + (int64_t)n * cin * hw;
+    for (int kc = 0; kc < cin; kc += KC) {
+        __syncthreads();  // the previous chunk has been consumed
+        // all loads of the chunk are issued before the first one is used (branch-free: out-of-range pixels read
+        // a clamped address and are zeroed afterwards), so the chunk costs one memory round trip, not eight
+        constexpr int XL = KC * (PX / 4) / 256, WL = (MT * 32 * (KC / 4) + 255) / 256;
+        floatx4 xv[XL], wv[WL];
+#pragma unroll
+        for (int r = 0; r < XL; ++r) {
+            const int idx = r * 256 + threadIdx.x, row = idx / (PX / 4), c4 = idx % (PX / 4);
+            const int64_t p = p0 + c4 * 4 < hw ? p0 + c4 * 4 : hw - 4;
+            xv[r] = *reinterpret_cast<const floatx4*>(xn + (int64_t)(kc + row) * hw + p);
+        }
+#pragma unroll
+        for (int r = 0; r < WL; ++r) {
+            const int idx = r * 256 + threadIdx.x, row = min(idx / (KC / 4), MT * 32 - 1), c4 = idx % (KC / 4);
+            wv[r] = *reinterpret_cast<const floatx4*>(w + (int64_t)min(m0 + row, cout - 1) * cin + kc + c4 * 4);
+        }
+#pragma unroll
+        for (int r = 0; r < XL; ++r) {
+            const int idx = r * 256 + threadIdx.x, row = idx / (PX / 4), c4 = idx % (PX / 4);
+            floatx4 v = xv[r];
+            if (in_scale) v *= in_scale[(int64_t)n * cin + kc + row];
+            if (!(p0 + c4 * 4 < hw)) v = floatx4{0.f, 0.f, 0.f, 0.f};
+            *reinterpret_cast<floatx4*>(xs + row * XP + c4 * 4) = v;
+        }
+#pragma unroll
+        for (int r = 0; r < WL; ++r) {
+            const int idx = r * 256 + threadIdx.x, row = idx / (KC / 4), c4 = idx % (KC / 4);
+            if (idx < MT * 32 * (KC / 4)) {
+                const bool ok = m0 + row < cout;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ws[row * WP + c4 * 4 + e] = ok ? wv[r][e] : 0.f;
+            }
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int kk = 0; kk < KC / 2; ++kk) {
+            float b[PT];
+#pragma unroll
+            for (int j = 0; j < PT; ++j) b[j] = xs[(2 * kk + h) * XP + pwv + j * 32 + l32];
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const float a = ws[(i * 32 + l32) * WP + 2 * kk + h];
+#pragma unroll
+                for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[j], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+    float* yn = y + (int64_t)n * cout * hw;
+    // the activation is selected once, outside the 32*MT stores of a lane
+    auto store_all = [&](auto actc) {
+        constexpr int ACT = decltype(actc)::value;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < PT; ++j) {
+                const int64_t p = p0 + pwv + j * 32 + l32;
+                if (p >= hw) continue;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int ml = i * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
+                    if (m0 + ml < cout) yn[(int64_t)(m0 + ml) * hw + p] = apply_act(ACT, acc[i][j][e] + bs[ml]);
+                }
+            }
+    };
+    switch (act) {
+        case DMLHIP_ACT_GELU: store_all(std::integral_constant<int, DMLHIP_ACT_GELU>{}); break;
+        case DMLHIP_ACT_SWISH: store_all(std::integral_constant<int, DMLHIP_ACT_SWISH>{}); break;
+        case DMLHIP_ACT_SIGMOID: store_all(std::integral_constant<int, DMLHIP_ACT_SIGMOID>{}); break;
+        case DMLHIP_ACT_RELU: store_all(std::integral_constant<int, DMLHIP_ACT_RELU>{}); break;
+        default: store_all(std::integral_constant<int, DMLHIP_ACT_NONE>{}); break;
+    }
+}
+
+int launch_pointwise_f32(const float* x, const float* w, const float* bias, const float* in_scale, float* y, int n, int cin,
+                         int cout, int64_t hw, int act, hipStream_t st) {
+    int mt = (int)ceil_div(cout, 32);
+    if (mt > 6) mt = 6;
+    // many output channels: 32 pixels per wavefront keep the accumulators (16 registers per 32x32 block) and the
+    // load registers within what two resident workgroups per CU may use
+    const int pt = mt >= 5 ? 1 : 2;
+    const dim3 grid((unsigned)ceil_div(hw, 128 * pt), (unsigned)n, (unsigned)ceil_div(cout, mt * 32));
+    const size_t lds = (size_t)(32 * (128 * pt + 32) + mt * 32 * 33 + mt * 32) * sizeof(float);
+#define DML_PW(MT, PT)                                                                                                 \
+    case MT:                                                                                                           \
+        hipLaunchKernelGGL((conv_pointwise_f32_kernel<MT, PT>), grid, 256, lds, st, x, w, bias, in_scale, y, cin, cout, hw, \
+                           act);                                                                                       \
+        break
+    switch (mt) {
+        DML_PW(1, 2); DML_PW(2, 2); DML_PW(3, 2); DML_PW(4, 2); DML_PW(5, 1);
+        default: DML_PW(6, 1);
+    }
+#undef DML_PW
+    return launch_status("conv2d(pointwise)");
+}
+
 // ---------------------------------------------------------------- host side
 int make_geom(const dmlhip_conv2d_desc* d, ConvGeom* g, const char* what) {
     DML_REQUIRE(d, DMLHIP_ERR_NULL, "%s: NULL descriptor", what);
@@ -194,8 +329,14 @@ int conv_forward(const dmlhip_conv2d_desc* d, const void* x, const void* w, cons
 
     // 1x1, stride 1, no pad, group 1: Y[b] (M x HW) = W (M x C) . X[b] (C x HW)
     if (g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1 && g.c > 0) {
-        dmlhip_gemm_desc gd = {};
         const int64_t hw = (int64_t)g.h * g.w;
+        if constexpr (sizeof(T) == 4) {
+            // many pixels, few channels: the streaming kernel (reads X once, writes Y in full rows)
+            if (g.c % 32 == 0 && hw % 4 == 0 && hw >= 128 && g.n <= 65535 && aligned16(x) && aligned16(w))
+                return launch_pointwise_f32((const float*)x, (const float*)w, (const float*)bias, nullptr, (float*)y, g.n,
+                                            g.c, g.m, hw, g.act, st);
+        }
+        dmlhip_gemm_desc gd = {};
         gd.m = g.m; gd.n = hw; gd.k = g.c;
         gd.batch[0] = 1; gd.batch[1] = 1; gd.batch[2] = g.n;
         gd.a_stride_m = g.c; gd.a_stride_k = 1;

@@ -376,6 +376,8 @@ CONV_CASES = [
     ((2, 8, 9, 9), (4, 4, 3, 3), (1, 1), (1, 1), (1, 1), 2, True),          # grouped
     ((1, 2, 12, 12), (3, 2, 3, 3), (1, 1), (2, 2), (2, 2), 1, False),       # dilated
     ((2, 4, 8, 8), (6, 4, 1, 1), (2, 2), (0, 0), (1, 1), 1, True),          # 1x1 strided -> direct
+    ((2, 192, 20, 26), (48, 192, 1, 1), (1, 1), (0, 0), (1, 1), 1, True),   # MBConv project: pointwise, 6 K chunks
+    ((2, 64, 17, 20), (200, 64, 1, 1), (1, 1), (0, 0), (1, 1), 1, False),   # pointwise, ragged channels and pixels
 ]
 
 
@@ -395,6 +397,7 @@ def test_conv2d_f32(xs, ws, st, pd, dl, grp, has_bias):
 def test_conv2d_f32_swish_epilogue():
     from daceml_amd import _lib as L, kernels as K
     for xs, ws, st, pd, grp in [((2, 16, 12, 12), (24, 16, 1, 1), (1, 1), (0, 0), 1),
+                                ((2, 32, 20, 20), (192, 32, 1, 1), (1, 1), (0, 0), 1),   # the pointwise kernel
                                 ((2, 24, 12, 12), (24, 1, 3, 3), (2, 2), (1, 1), 24)]:
         x = rng(93).standard_normal(xs).astype(np.float32)
         w = (rng(94).standard_normal(ws) * np.sqrt(2.0 / np.prod(ws[1:]))).astype(np.float32)
