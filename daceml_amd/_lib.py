@@ -93,6 +93,7 @@ SIGNATURES = {
     "dmlhip_conv2d_out_shape": (c_int, [POINTER(Conv2dDesc), _I64P, _I64P]),
     "dmlhip_conv2d_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, _P]),
     "dmlhip_conv2d_f16": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, _P]),
+    "dmlhip_conv2d_gated_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, _P, _P]),
     "dmlhip_conv2d_backward_data_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P]),
     "dmlhip_conv2d_backward_weight_workspace_bytes": (c_size_t, [POINTER(Conv2dDesc)]),
     "dmlhip_conv2d_backward_weight_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, c_size_t, _P]),

@@ -48,28 +48,57 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const T* __restrict__ 
 }
 
 // ---------------------------------------------------------------- depthwise forward
-// One workgroup per (image, channel, strip of ROWS output rows). LDS holds the input rows of the
-// strip, zero-padded left/right, so the stencil needs no bounds checks along x.
-template <typename T, int KH, int KW>
-__global__ __launch_bounds__(256) void conv_depthwise_kernel(const T* __restrict__ x, const T* __restrict__ w,
-                                                             const T* __restrict__ bias, T* __restrict__ y, ConvGeom g,
-                                                             int rows_per_strip, int strips) {
-    extern __shared__ float tile[];  // [in_rows][wp]
+// One workgroup per (image, channel, strip of output rows). LDS holds the input rows of the strip with the data
+// of a row starting at a 16-byte aligned column (left margin kLeft >= pad, zero-filled like the right margin), so
+// the stencil needs no bounds checks along x, global loads are 128-bit when the row length allows, and the
+// output loop has no integer divisions: lanes run along x, wavefronts along y.
+constexpr int kDwLeft = 4;
+
+__host__ __device__ inline int dw_pitch(int w, int pw) { return ((kDwLeft + w + pw + 3) / 4) * 4; }
+
+template <typename T, int KH, int KW, int ACT>
+__device__ __forceinline__ void depthwise_body(const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias,
+                                               T* __restrict__ y, const ConvGeom& g, int rows_per_strip, int strips,
+                                               float* tile) {
     const int strip = blockIdx.x % strips;
     const int64_t plane = blockIdx.x / strips;  // b * C + c
     const int c = (int)(plane % g.c);
     const int oy0 = strip * rows_per_strip;
     const int oy1 = min(oy0 + rows_per_strip, g.oh);
-    const int wp = g.w + 2 * g.pw;
+    const int pitch = dw_pitch(g.w, g.pw);
     const int iy0 = oy0 * g.sh - g.ph;
     const int in_rows = (oy1 - oy0 - 1) * g.sh + (KH - 1) * g.dh + 1;
     const T* xp = x + plane * g.h * g.w;
-    for (int i = threadIdx.x; i < in_rows * wp; i += 256) {
-        const int r = i / wp, col = i % wp - g.pw;
-        const int iy = iy0 + r;
-        float v = 0.f;
-        if (iy >= 0 && iy < g.h && col >= 0 && col < g.w) v = to_f32(xp[(int64_t)iy * g.w + col]);
-        tile[i] = v;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // margins: kDwLeft columns on the left, the rest of the pitch on the right
+    const int right0 = kDwLeft + g.w, margin = kDwLeft + pitch - right0;
+    for (int i = threadIdx.x; i < in_rows * margin; i += 256) {
+        const int r = i / margin, m = i % margin;
+        tile[r * pitch + (m < kDwLeft ? m : right0 + m - kDwLeft)] = 0.f;
+    }
+    if constexpr (sizeof(T) == 4) {
+        if (g.w % 4 == 0 && (reinterpret_cast<uintptr_t>(xp) & 15) == 0) {
+            const int vec = g.w / 4;
+            for (int i = threadIdx.x; i < in_rows * vec; i += 256) {
+                const int r = i / vec, c4 = i % vec;
+                const int iy = iy0 + r;
+                floatx4 v = {0.f, 0.f, 0.f, 0.f};
+                if (iy >= 0 && iy < g.h) v = *reinterpret_cast<const floatx4*>(xp + (int64_t)iy * g.w + c4 * 4);
+                *reinterpret_cast<floatx4*>(tile + r * pitch + kDwLeft + c4 * 4) = v;
+            }
+        } else {
+            for (int r = wave; r < in_rows; r += 4) {
+                const int iy = iy0 + r;
+                for (int col = lane; col < g.w; col += 64)
+                    tile[r * pitch + kDwLeft + col] = (iy >= 0 && iy < g.h) ? to_f32(xp[(int64_t)iy * g.w + col]) : 0.f;
+            }
+        }
+    } else {
+        for (int r = wave; r < in_rows; r += 4) {
+            const int iy = iy0 + r;
+            for (int col = lane; col < g.w; col += 64)
+                tile[r * pitch + kDwLeft + col] = (iy >= 0 && iy < g.h) ? to_f32(xp[(int64_t)iy * g.w + col]) : 0.f;
+        }
     }
     float wr[KH * KW];
 #pragma unroll
@@ -77,16 +106,30 @@ __global__ __launch_bounds__(256) void conv_depthwise_kernel(const T* __restrict
     const float bv = bias ? to_f32(bias[c]) : 0.f;
     __syncthreads();
     T* yp = y + plane * g.oh * g.ow;
-    const int outs = (oy1 - oy0) * g.ow;
-    for (int i = threadIdx.x; i < outs; i += 256) {
-        const int oy = i / g.ow, ox = i % g.ow;
-        const float* tp = tile + (oy * g.sh) * wp + ox * g.sw;
-        float acc = bv;
+    for (int oy = wave; oy < oy1 - oy0; oy += 4) {
+        for (int ox = lane; ox < g.ow; ox += 64) {
+            const float* tp = tile + (oy * g.sh) * pitch + kDwLeft - g.pw + ox * g.sw;
+            float acc = bv;
 #pragma unroll
-        for (int hy = 0; hy < KH; ++hy)
+            for (int hy = 0; hy < KH; ++hy)
 #pragma unroll
-            for (int hx = 0; hx < KW; ++hx) acc += wr[hy * KW + hx] * tp[hy * g.dh * wp + hx * g.dw];
-        yp[(int64_t)(oy0 + oy) * g.ow + ox] = from_f32<T>(apply_act(g.act, acc));
+                for (int hx = 0; hx < KW; ++hx) acc += wr[hy * KW + hx] * tp[hy * g.dh * pitch + hx * g.dw];
+            yp[(int64_t)(oy0 + oy) * g.ow + ox] = from_f32<T>(apply_act(ACT, acc));
+        }
+    }
+}
+
+template <typename T, int KH, int KW>
+__global__ __launch_bounds__(256) void conv_depthwise_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                             const T* __restrict__ bias, T* __restrict__ y, ConvGeom g,
+                                                             int rows_per_strip, int strips) {
+    extern __shared__ float tile[];  // [in_rows][pitch]
+    switch (g.act) {  // the activation is selected once per workgroup, not once per output
+        case DMLHIP_ACT_SWISH: depthwise_body<T, KH, KW, DMLHIP_ACT_SWISH>(x, w, bias, y, g, rows_per_strip, strips, tile); break;
+        case DMLHIP_ACT_SIGMOID: depthwise_body<T, KH, KW, DMLHIP_ACT_SIGMOID>(x, w, bias, y, g, rows_per_strip, strips, tile); break;
+        case DMLHIP_ACT_RELU: depthwise_body<T, KH, KW, DMLHIP_ACT_RELU>(x, w, bias, y, g, rows_per_strip, strips, tile); break;
+        case DMLHIP_ACT_GELU: depthwise_body<T, KH, KW, DMLHIP_ACT_GELU>(x, w, bias, y, g, rows_per_strip, strips, tile); break;
+        default: depthwise_body<T, KH, KW, DMLHIP_ACT_NONE>(x, w, bias, y, g, rows_per_strip, strips, tile); break;
     }
 }
 
@@ -260,6 +303,32 @@ __global__ __launch_bounds__(256, 2) void conv_pointwise_f32_kernel(const float*
     }
 }
 
+// Squeeze-excite sized products ([n, c, 1, 1] inputs): Y[n, m] = act(b[m] + sum_c X[n, c] W[m, c]). A few hundred
+// outputs with a short dot product each: one wavefront per output, lanes along c, so the whole product is one
+// memory round trip plus a wavefront reduction instead of a tiled GEMM's chain of synchronised K steps.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_1x1_spatial1_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                const T* __restrict__ bias, T* __restrict__ y, int n, int c,
+                                                                int m, int act) {
+    const int lane = threadIdx.x & 63;
+    const int64_t o = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (o >= (int64_t)n * m) return;
+    const int in = (int)(o / m), im = (int)(o % m);
+    const T* xr = x + (int64_t)in * c;
+    const T* wr = w + (int64_t)im * c;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int k = lane;
+    for (; k + 192 < c; k += 256) {
+        a0 += to_f32(xr[k]) * to_f32(wr[k]);
+        a1 += to_f32(xr[k + 64]) * to_f32(wr[k + 64]);
+        a2 += to_f32(xr[k + 128]) * to_f32(wr[k + 128]);
+        a3 += to_f32(xr[k + 192]) * to_f32(wr[k + 192]);
+    }
+    for (; k < c; k += 64) a0 += to_f32(xr[k]) * to_f32(wr[k]);
+    const float s = wave_reduce<OpSum>((a0 + a1) + (a2 + a3));
+    if (lane == 0) y[o] = from_f32<T>(apply_act(act, s + (bias ? to_f32(bias[im]) : 0.f)));
+}
+
 int launch_pointwise_f32(const float* x, const float* w, const float* bias, const float* in_scale, float* y, int n, int cin,
                          int cout, int64_t hw, int act, hipStream_t st) {
     int mt = (int)ceil_div(cout, 32);
@@ -337,6 +406,11 @@ int conv_forward(const dmlhip_conv2d_desc* d, const void* x, const void* w, cons
                                             g.c, g.m, hw, g.act, st);
         }
         dmlhip_gemm_desc gd = {};
+        if (hw == 1 && (int64_t)g.n * g.m <= (1 << 22)) {
+            hipLaunchKernelGGL((conv_1x1_spatial1_kernel<T>), (unsigned)ceil_div((int64_t)g.n * g.m, 4), 256, 0, st,
+                               (const T*)x, (const T*)w, (const T*)bias, (T*)y, g.n, g.c, g.m, g.act);
+            return launch_status("conv2d(1x1 on 1x1)");
+        }
         gd.m = g.m; gd.n = hw; gd.k = g.c;
         gd.batch[0] = 1; gd.batch[1] = 1; gd.batch[2] = g.n;
         gd.a_stride_m = g.c; gd.a_stride_k = 1;
@@ -352,7 +426,8 @@ int conv_forward(const dmlhip_conv2d_desc* d, const void* x, const void* w, cons
     }
     // depthwise with a small square-ish stencil
     if (g.group == g.c && g.m == g.c && ((g.kh == 3 && g.kw == 3) || (g.kh == 5 && g.kw == 5))) {
-        const int wp = g.w + 2 * g.pw;
+        if (g.pw > kDwLeft) goto direct;
+        const int wp = dw_pitch(g.w, g.pw);
         // rows per strip: keep the LDS tile under 32 KiB so several workgroups share a CU
         int rows = g.oh;
         while (rows > 1 && (size_t)((rows - 1) * g.sh + (g.kh - 1) * g.dh + 1) * wp * sizeof(float) > 32 * 1024)
@@ -371,6 +446,7 @@ int conv_forward(const dmlhip_conv2d_desc* d, const void* x, const void* w, cons
             return launch_status("conv2d(depthwise)");
         }
     }
+direct:
     hipLaunchKernelGGL((conv_direct_kernel<T>), grid_for(total), 256, 0, st, (const T*)x, (const T*)w, (const T*)bias,
                        (T*)y, g, total);
     return launch_status("conv2d(direct)");
@@ -395,6 +471,22 @@ int dmlhip_conv2d_out_shape(const dmlhip_conv2d_desc* d, int64_t* oh, int64_t* o
 int dmlhip_conv2d_f32(const dmlhip_conv2d_desc* d, const void* x, const void* w, const void* bias, void* y,
                       void* stream) {
     return conv_forward<float>(d, x, w, bias, y, stream);
+}
+
+int dmlhip_conv2d_gated_f32(const dmlhip_conv2d_desc* d, const void* x, const void* gate, const void* w, const void* bias,
+                            void* y, void* stream) {
+    ConvGeom g;
+    if (int e = make_geom(d, &g, "conv2d_gated")) return e;
+    const int64_t hw = (int64_t)g.h * g.w;
+    DML_REQUIRE(g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1,
+                DMLHIP_ERR_UNSUPPORTED, "conv2d_gated: only 1x1, stride 1, no padding, group 1");
+    DML_REQUIRE(g.c > 0 && g.c % 32 == 0 && hw % 4 == 0 && hw >= 128 && g.n <= 65535, DMLHIP_ERR_UNSUPPORTED,
+                "conv2d_gated: needs channels %% 32 == 0, h*w %% 4 == 0, h*w >= 128, n <= 65535");
+    if ((int64_t)g.n * g.m == 0) return 0;
+    DML_REQUIRE(x && gate && w && y, DMLHIP_ERR_NULL, "conv2d_gated: NULL tensor pointer");
+    DML_REQUIRE(aligned16(x) && aligned16(w), DMLHIP_ERR_ALIGN, "conv2d_gated: x and w must be 16-byte aligned");
+    return launch_pointwise_f32((const float*)x, (const float*)w, (const float*)bias, (const float*)gate, (float*)y, g.n, g.c,
+                                g.m, hw, g.act, (hipStream_t)stream);
 }
 
 int dmlhip_conv2d_f16(const dmlhip_conv2d_desc* d, const void* x, const void* w, const void* bias, void* y,

@@ -130,6 +130,9 @@ SCHEMAS = [
             v_perm=REQUIRED, o_perm=REQUIRED),
     _schema("FusedAttentionGrad", "Q K V O LogSumExp dO", "dQ dK dV", since=1, scale=1.0, q_perm=REQUIRED,
             k_perm=REQUIRED, v_perm=REQUIRED, o_perm=REQUIRED),
+    # Conv 1x1 whose input is first multiplied by a per-image, per-channel factor Gate [n, c, 1, 1] (squeeze-excite)
+    _schema("GatedConv", "X Gate W B?", "Y", since=1, auto_pad="NOTSET", dilations=None, group=1, kernel_shape=None,
+            pads=None, strides=None),
     # several independent ReduceSum(all leading axes, keepdims=0) nodes in one launch pair: reduced__i = sum of
     # data__i over every axis but the last (the bias gradients of a backward pass)
     _schema("MultiReduceSum", "data*", "reduced*", since=1),

@@ -845,6 +845,42 @@ class HipConv(ONNXForward):
         return _tasklet(node, state, [call], flops=flops, bytes_moved=_nbytes(x, w, y), kind="conv")
 
 
+@op_implementation(op="GatedConv", name=IMPL)
+class HipGatedConv(ONNXForward):
+    """Mul(X, Gate[n, c, 1, 1]) followed by a pointwise Conv (pure_implementations.py:86-88 +
+    img_op_implementations.py:164-330) in one kernel: the gate scales X on its way into LDS. fp32."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, gt, w, y = ins["X"], ins["Gate"], ins["W"], outs["Y"]
+            if x.dtype != torch.float32 or not (_float_ok(x, gt, w, y) and _dense(x, gt, w, y)):
+                return False
+            if tuple(gt.shape) != (x.shape[0], x.shape[1], 1, 1) or tuple(w.shape[2:]) != (1, 1):
+                return False
+            if "B" in ins and not (ins["B"].dtype == x.dtype and ins["B"].is_contiguous()
+                                   and ins["B"].total_size == w.shape[0]):
+                return False
+            d = _conv_struct(node, x, w)
+            if d is None or (d.stride_h, d.stride_w, d.pad_h, d.pad_w, d.group) != (1, 1, 0, 0, 1):
+                return False
+            hw = x.shape[2] * x.shape[3]
+            return (x.shape[1] % 32 == 0 and hw % 4 == 0 and hw >= 128 and x.shape[0] <= 65535
+                    and tuple(y.shape) == (x.shape[0], w.shape[0], x.shape[2], x.shape[3]))
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        x, w, y = ins["X"], ins["W"], outs["Y"]
+        d = _conv_struct(node, x, w, _ACT[getattr(node, "_activation", "none")])
+        call = HipCall("dmlhip_conv2d_gated_f32", [Struct(d, "dmlhip_conv2d_desc"), Ptr("X"), Ptr("Gate"), Ptr("W"),
+                                                   _opt(node, state, "B"), Ptr("Y"), Stream()])
+        return _tasklet(node, state, [call], flops=2 * y.total_size * w.shape[1] + x.total_size,
+                        bytes_moved=_nbytes(x, ins["Gate"], w, y), kind="conv")
+
+
 @op_implementation(op="ConvGrad", name=IMPL)
 class HipConvGrad(ONNXForward):
     """cudnnConvolutionBackwardData / BackwardFilter / BackwardBias

@@ -20,6 +20,7 @@ expansions it replaces (that composition is the oracle of the fused kernels).
     fuse_attention           Einsum(Q,K)[*scale], Softmax, Einsum(P,V)    -> FusedAttention
     fuse_reductions          independent ReduceSum(leading axes) nodes    -> MultiReduceSum (one launch pair)
     fuse_conv_activation     Conv, Swish | Sigmoid | Relu                 -> Conv(_activation)
+    fuse_gate_into_conv      Mul(X, gate[n,c,1,1]), Conv 1x1              -> GatedConv (inference graphs)
 """
 import math
 from typing import Dict, List, Optional, Tuple
@@ -299,6 +300,52 @@ def fuse_conv_activation(sdfg: SDFG) -> int:
             conv._activation = names[act.schema.name]
             count += 1
     _drop_unused_arrays(sdfg)
+    return count
+
+
+def fuse_gate_into_conv(sdfg: SDFG) -> int:
+    """Squeeze-excite: Mul(X[n,c,h,w], gate[n,c,1,1]) read only by a pointwise Conv becomes one GatedConv, which
+    saves a full read and write of X. Forward graphs only (GatedConv has no backward implementation)."""
+    count = 0
+    for state in sdfg.states():
+        for conv in [n for n in state.nodes() if _is_op(n, "Conv")]:
+            xa = _in_array(state, conv, "X")
+            prod = _producer(state, xa)
+            if prod is None or not _is_op(prod[0], "Mul") or not _internal(sdfg, state, xa):
+                continue
+            mul = prod[0]
+            a, b = _in_array(state, mul, "A"), _in_array(state, mul, "B")
+            xd = sdfg.arrays[xa]
+            if len(xd.shape) != 4 or xd.dtype != torch.float32:
+                continue
+            gate_shape = (xd.shape[0], xd.shape[1], 1, 1)
+            if tuple(sdfg.arrays[b].shape) == gate_shape and tuple(sdfg.arrays[a].shape) == tuple(xd.shape):
+                data, gate = a, b
+            elif tuple(sdfg.arrays[a].shape) == gate_shape and tuple(sdfg.arrays[b].shape) == tuple(xd.shape):
+                data, gate = b, a
+            else:
+                continue
+            wd = sdfg.arrays[_in_array(state, conv, "W")]
+            hw = xd.shape[2] * xd.shape[3]
+            attrs = {k: getattr(conv, k) for k in ("auto_pad", "dilations", "group", "kernel_shape", "pads", "strides")}
+            plain = (tuple(wd.shape[2:]) == (1, 1) and attrs["group"] == 1
+                     and all(v == 1 for v in (attrs["strides"] or [1, 1])) and not any(attrs["pads"] or [0]))
+            if not plain or xd.shape[1] % 32 or hw % 4 or hw < 128:
+                continue
+            ins = {"X": data, "Gate": gate, "W": _in_array(state, conv, "W")}
+            bias = _in_array(state, conv, "B")
+            if bias is not None:
+                ins["B"] = bias
+            y = _out_array(state, conv, "Y")
+            act = getattr(conv, "_activation", "none")
+            label = conv.label
+            _remove_node(state, conv)
+            _remove_node(state, mul)
+            node = _add_node(sdfg, state, "GatedConv", label, ins, {"Y": y}, **attrs)
+            node._activation = act
+            count += 1
+    if count:
+        _drop_unused_arrays(sdfg)
     return count
 
 
@@ -688,6 +735,7 @@ def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True) ->
     stats["layernorm"] = fuse_layernorm(sdfg)
     stats["swish"] = fuse_swish(sdfg)
     stats["conv_activation"] = fuse_conv_activation(sdfg)
+    stats["gated_conv"] = 0 if training else fuse_gate_into_conv(sdfg)
     stats["matmul_to_einsum"] = lower_matmul(sdfg)
     stats["views"] = fold_views(sdfg)
     stats["epilogues"] = fuse_epilogues(sdfg, keep_preactivation=training)

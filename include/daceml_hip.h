@@ -238,6 +238,12 @@ int dmlhip_conv2d_f32(const dmlhip_conv2d_desc* d, const void* x, const void* w,
                       const void* bias, void* y, void* stream);
 int dmlhip_conv2d_f16(const dmlhip_conv2d_desc* d, const void* x, const void* w,
                       const void* bias, void* y, void* stream);
+/* Y = Conv1x1(X * gate) with gate [n, c] (the [n, c, 1, 1] squeeze-excite factor broadcast over the pixels):
+ * the Mul node (pure_implementations.py:86-88) in front of a pointwise Conv folded into the conv's read of X.
+ * Only 1x1 / stride 1 / no padding / group 1 with c % 32 == 0, h*w % 4 == 0, h*w >= 128 (DMLHIP_ERR_UNSUPPORTED
+ * otherwise: the caller keeps Mul and Conv separate). */
+int dmlhip_conv2d_gated_f32(const dmlhip_conv2d_desc* d, const void* x, const void* gate,
+                            const void* w, const void* bias, void* y, void* stream);
 /* cudnnConvolutionBackwardData / BackwardFilter (autodiff/implementations/onnx_ops.py:663-703)
  * and the ATen depthwise backward (onnx_ops.py:1201-1231). dw is overwritten. The bias
  * gradient is dmlhip_reduce over [n, m, oh*ow] done by the caller (two reduce calls). */

@@ -123,7 +123,9 @@ def test_mbconv_block_forward():
         else:
             params[name] = (r.standard_normal(desc.shape) * 0.1).astype(np.float32)
     stats = fusion.auto_optimize(sdfg)
-    assert stats["swish"] == 3 and stats["conv_activation"] == 4
+    assert stats["swish"] == 3 and stats["conv_activation"] == 4 and stats["gated_conv"] == 1
+    names = [n.schema.name for n in sdfg.states()[0].library_nodes()]
+    assert names.count("GatedConv") == 1 and "Mul" not in names   # the squeeze-excite Mul went into the projection
     prog = _compile(sdfg)
     oh = (hw + 2 - 3) // 2 + 1
     y = torch.empty((b, cout, oh, oh), dtype=torch.float32, device="cuda")

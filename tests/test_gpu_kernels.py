@@ -378,6 +378,8 @@ CONV_CASES = [
     ((2, 4, 8, 8), (6, 4, 1, 1), (2, 2), (0, 0), (1, 1), 1, True),          # 1x1 strided -> direct
     ((2, 192, 20, 26), (48, 192, 1, 1), (1, 1), (0, 0), (1, 1), 1, True),   # MBConv project: pointwise, 6 K chunks
     ((2, 64, 17, 20), (200, 64, 1, 1), (1, 1), (0, 0), (1, 1), 1, False),   # pointwise, ragged channels and pixels
+    ((96, 192, 1, 1), (8, 192, 1, 1), (1, 1), (0, 0), (1, 1), 1, True),     # squeeze-excite reduce: one product
+    ((5, 8, 1, 1), (192, 8, 1, 1), (1, 1), (0, 0), (1, 1), 1, True),        # squeeze-excite expand
 ]
 
 

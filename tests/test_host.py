@@ -299,7 +299,7 @@ def test_fusion_pipeline_on_bert_layer():
     before = [n.schema.name for n in st.library_nodes()]
     assert before.count("MatMul") == 8 and before.count("Erf") == 1 and before.count("ReduceMean") == 4
     stats = fusion.auto_optimize(sdfg, training=True)
-    assert stats == {"gelu": 1, "layernorm": 2, "swish": 0, "conv_activation": 0, "matmul_to_einsum": 8,
+    assert stats == {"gelu": 1, "layernorm": 2, "swish": 0, "conv_activation": 0, "gated_conv": 0, "matmul_to_einsum": 8,
                      "views": 15, "epilogues": 7, "skip_layernorm": 0, "attention": 0}  # head dim 32: not fused
     after = {n.label: n for n in st.library_nodes()}
     assert sorted(n.schema.name for n in after.values()) == ["Einsum"] + ["FusedEinsum"] * 7 + \
