@@ -14,59 +14,80 @@ template <typename T> struct ExpFn;
 // fp16 I/O: the result is rounded to 11 bits, so the hardware exp2 is exact enough.
 template <> struct ExpFn<_Float16> {
     __device__ __forceinline__ static float f(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+    // exp(v - m) with the subtraction and the base change in one fma; m2 = m * log2(e)
+    __device__ __forceinline__ static float prep(float m) { return m * 1.44269504088896340736f; }
+    __device__ __forceinline__ static float shifted(float v, float m2) {
+        return __builtin_amdgcn_exp2f(__builtin_fmaf(v, 1.44269504088896340736f, -m2));
+    }
 };
 template <> struct ExpFn<float> {
     __device__ __forceinline__ static float f(float x) { return expf(x); }
+    __device__ __forceinline__ static float prep(float m) { return m; }
+    __device__ __forceinline__ static float shifted(float v, float m) { return expf(v - m); }
 };
 
 // ------------------------------------------------------------------ softmax, wave per row
-template <typename T, int VPL>
+// RPW rows per wavefront: the loads of all its rows are issued before the first reduction, so a wavefront keeps
+// RPW * VPL 16-byte loads in flight per lane instead of VPL (short rows otherwise leave the memory system idle
+// between a row's load and its store).
+template <typename T, int VPL, int RPW>
 __global__ __launch_bounds__(kRowBlock) void softmax_wave_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                  int64_t rows, int cols) {
     using V = typename VecOf<T>::type;
     constexpr int VN = VecOf<T>::n;
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave;
-    if (row >= rows) return;
-    const V* xr = reinterpret_cast<const V*>(x + row * cols);
-    V* yr = reinterpret_cast<V*>(y + row * cols);
+    const int64_t row0 = ((int64_t)blockIdx.x * kRowsPerBlock + threadIdx.x / kWave) * RPW;
+    if (row0 >= rows) return;
     const int nvec = cols / VN;
 
-    float v[VPL][VN];
-    float m = -INFINITY;
+    V raw[RPW][VPL];
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-        const int vi = lane + j * kWave;
-        if (vi < nvec) {
-            V t = __builtin_nontemporal_load(xr + vi);
+    for (int r = 0; r < RPW; ++r) {
+        const int64_t row = row0 + r < rows ? row0 + r : rows - 1;
+        const V* xr = reinterpret_cast<const V*>(x + row * cols);
 #pragma unroll
-            for (int e = 0; e < VN; ++e) {
-                v[j][e] = to_f32(t[e]);
-                m = fmaxf(m, v[j][e]);
-            }
-        } else {
-#pragma unroll
-            for (int e = 0; e < VN; ++e) v[j][e] = -INFINITY;
+        for (int j = 0; j < VPL; ++j) {
+            const int vi = lane + j * kWave;
+            if (vi < nvec) raw[r][j] = __builtin_nontemporal_load(xr + vi);
         }
     }
-    m = wave_reduce<OpMax>(m);
-    float s = 0.f;
 #pragma unroll
-    for (int j = 0; j < VPL; ++j)
+    for (int r = 0; r < RPW; ++r) {
+        if (row0 + r >= rows) break;
+        float v[VPL][VN];
+        float m = -INFINITY;
 #pragma unroll
-        for (int e = 0; e < VN; ++e) {
-            v[j][e] = ExpFn<T>::f(v[j][e] - m);
-            s += v[j][e];
+        for (int j = 0; j < VPL; ++j) {
+            const int vi = lane + j * kWave;
+#pragma unroll
+            for (int e = 0; e < VN; ++e) {
+                v[j][e] = vi < nvec ? to_f32(raw[r][j][e]) : -INFINITY;
+                m = fmaxf(m, v[j][e]);
+            }
         }
-    s = wave_reduce<OpSum>(s);
+        m = ExpFn<T>::prep(wave_reduce<OpMax>(m));
+        float s = 0.f;
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-        const int vi = lane + j * kWave;
-        if (vi < nvec) {
-            V t;
+        for (int j = 0; j < VPL; ++j)
 #pragma unroll
-            for (int e = 0; e < VN; ++e) t[e] = from_f32<T>(v[j][e] / s);
-            __builtin_nontemporal_store(t, yr + vi);
+            for (int e = 0; e < VN; ++e) {
+                v[j][e] = ExpFn<T>::shifted(v[j][e], m);
+                s += v[j][e];
+            }
+        s = wave_reduce<OpSum>(s);
+        // one true division per row; each element is then scaled (fp16 results: the hardware reciprocal would do,
+        // but the row total is shared by fp32 outputs that must hold 1e-5)
+        const float inv = 1.0f / s;
+        V* yr = reinterpret_cast<V*>(y + (row0 + r) * cols);
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const int vi = lane + j * kWave;
+            if (vi < nvec) {
+                V t;
+#pragma unroll
+                for (int e = 0; e < VN; ++e) t[e] = from_f32<T>(v[j][e] * inv);
+                __builtin_nontemporal_store(t, yr + vi);
+            }
         }
     }
 }
@@ -442,11 +463,20 @@ int softmax_impl(const void* x, void* y, int64_t rows, int64_t cols, void* strea
     const unsigned grid = (unsigned)ceil_div(rows, kRowsPerBlock);
     if (wave_path_ok<T>(cols, 4) && aligned16(x) && aligned16(y)) {
         const int vpl = (int)ceil_div(cols, kWave * VN);
+        // short rows and many of them: several rows per wavefront
+        const bool many = rows >= 16384;
+        const unsigned grid4 = (unsigned)ceil_div(rows, kRowsPerBlock * 4), grid2 = (unsigned)ceil_div(rows, kRowsPerBlock * 2);
         switch (vpl) {
-            case 1: hipLaunchKernelGGL((softmax_wave_kernel<T, 1>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
-            case 2: hipLaunchKernelGGL((softmax_wave_kernel<T, 2>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
-            case 3: hipLaunchKernelGGL((softmax_wave_kernel<T, 3>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
-            default: hipLaunchKernelGGL((softmax_wave_kernel<T, 4>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
+            case 1:
+                if (many) hipLaunchKernelGGL((softmax_wave_kernel<T, 1, 4>), grid4, kRowBlock, 0, st, xp, yp, rows, (int)cols);
+                else hipLaunchKernelGGL((softmax_wave_kernel<T, 1, 1>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols);
+                break;
+            case 2:
+                if (many) hipLaunchKernelGGL((softmax_wave_kernel<T, 2, 2>), grid2, kRowBlock, 0, st, xp, yp, rows, (int)cols);
+                else hipLaunchKernelGGL((softmax_wave_kernel<T, 2, 1>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols);
+                break;
+            case 3: hipLaunchKernelGGL((softmax_wave_kernel<T, 3, 1>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
+            default: hipLaunchKernelGGL((softmax_wave_kernel<T, 4, 1>), grid, kRowBlock, 0, st, xp, yp, rows, (int)cols); break;
         }
     } else {
         DML_REQUIRE(rows <= 2147483647, DMLHIP_ERR_SHAPE, "softmax: too many rows for the generic path");
