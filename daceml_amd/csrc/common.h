@@ -173,6 +173,17 @@ __device__ __forceinline__ float gelu_half_f(float x) {
     return 0.5f * x * (1.0f + copysignf(e, x));
 }
 
+// Derivative of the exact GELU for fp16 tensors, cdf(x) + x * pdf(x), with the same erf approximation and the
+// hardware exp2 (the result is rounded to 11 bits; the library erff + expf make the kernel compute bound).
+__device__ __forceinline__ float gelu_grad_half_f(float x) {
+    const float z = fabsf(x) * 0.70710678118654752440f;
+    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
+    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+    const float ex = __builtin_amdgcn_exp2f(-z * z * 1.44269504088896340736f);  // exp(-x^2 / 2)
+    const float cdf = 0.5f * (1.0f + copysignf(1.0f - poly * ex, x));
+    return cdf + x * 0.39894228040143267794f * ex;
+}
+
 __device__ __forceinline__ float apply_act_half(int act, float v) {
     switch (act) {
         case DMLHIP_ACT_GELU: return gelu_half_f(v);

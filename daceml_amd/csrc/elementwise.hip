@@ -131,7 +131,10 @@ __global__ __launch_bounds__(kEwBlock) void unary_kernel(const T* __restrict__ x
         V yv;
 #pragma unroll
         for (int e = 0; e < VN; ++e) {
-            if constexpr (GRAD) yv[e] = from_f32<T>(to_f32(gv[e]) * unary_grad<OP>(to_f32(xv[e]), p));
+            if constexpr (GRAD && OP == DMLHIP_GELU && sizeof(T) == 2)
+                yv[e] = from_f32<T>(to_f32(gv[e]) * gelu_grad_half_f(to_f32(xv[e])));
+            else if constexpr (GRAD) yv[e] = from_f32<T>(to_f32(gv[e]) * unary_grad<OP>(to_f32(xv[e]), p));
+            else if constexpr (OP == DMLHIP_GELU && sizeof(T) == 2) yv[e] = from_f32<T>(gelu_half_f(to_f32(xv[e])));
             else yv[e] = from_f32<T>(unary_apply<OP>(to_f32(xv[e]), p));
         }
         reinterpret_cast<V*>(y)[i] = yv;
