@@ -39,15 +39,17 @@ def test_bert_layer_forward(dtype, fused):
     x, p = _bert_inputs(b, s, h, ffn, dtype)
     sdfg = graphs.bert_encoder_layer(b, s, h, heads, ffn, dtype, eps=1e-5)
     if fused:
-        stats = fusion.auto_optimize(sdfg, attention=fused == "attention")
+        # "attention": the default pipeline (fused attention, Gelu as its own kernel); True: Gelu in the GEMM epilogue
+        stats = fusion.auto_optimize(sdfg, attention=fused == "attention", gelu_epilogue=fused is True)
         assert stats["layernorm"] == 2 and stats["gelu"] == 1 and stats["epilogues"] == 7
         names = [n.schema.name for n in sdfg.states()[0].library_nodes()]
         if fused == "attention" and dtype == torch.float16:  # the fused kernel is fp16 only
             assert stats["attention"] == 1
-            assert sorted(set(names)) == ["FusedAttention", "FusedEinsum", "LayerNormalization"]
+            assert sorted(set(names)) == ["FusedAttention", "FusedEinsum", "Gelu", "LayerNormalization"]
         else:
             assert stats["attention"] == 0
-            assert sorted(set(names)) == ["Einsum", "FusedEinsum", "LayerNormalization", "Softmax"]
+            extra = ["Gelu"] if fused == "attention" else []
+            assert sorted(set(names)) == sorted(["Einsum", "FusedEinsum", "LayerNormalization", "Softmax"] + extra)
     prog = _compile(sdfg)
     y = torch.empty((b, s, h), dtype=dtype, device="cuda")
     prog(x=dev(x), y=y, **{k: dev(v) for k, v in p.items()})
@@ -68,7 +70,7 @@ def test_bert_layer_backward(dtype, attention):
     x, p = _bert_inputs(b, s, h, ffn, dtype)
     dy = rng(77).standard_normal((b, s, h)).astype(x.dtype)
     sdfg = graphs.bert_encoder_layer(b, s, h, heads, ffn, dtype, eps=1e-5)
-    fusion.auto_optimize(sdfg, training=True, attention=attention)
+    fusion.auto_optimize(sdfg, training=True, attention=attention, gelu_epilogue=not attention)
     grads = add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + OB.PARAM_NAMES,
                               grad_dtypes={n: torch.float32 for n in OB.PARAM_NAMES})
     if attention:
