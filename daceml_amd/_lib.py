@@ -15,6 +15,7 @@ ERR_NULL, ERR_SHAPE, ERR_UNSUPPORTED, ERR_ALIGN, ERR_WORKSPACE, ERR_ENUM = -1, -
 F16, F32 = 0, 1
 ADD, SUB, MUL, DIV, POW = range(5)
 MULTI_MAX = 8  # DMLHIP_MULTI_MAX
+GROUP_MAX = 4  # DMLHIP_GROUP_MAX
 (ERF, SQRT, EXP, LOG, TANH, RELU, SIGMOID, RECIPROCAL, GELU, SWISH, SCALE, IDENTITY) = range(12)
 RSUM, RMAX, RMIN, RMEAN = range(4)
 ACT_NONE, ACT_GELU, ACT_SWISH, ACT_SIGMOID, ACT_RELU = range(5)
@@ -89,6 +90,8 @@ SIGNATURES = {
     "dmlhip_gemm_f16": (c_int, [POINTER(GemmDesc), _P, _P, _P, _P, _P, _P, _P]),
     "dmlhip_gemm_f16_workspace_bytes": (c_size_t, [POINTER(GemmDesc)]),
     "dmlhip_gemm_f16_ws": (c_int, [POINTER(GemmDesc), _P, _P, _P, _P, _P, _P, _P, c_size_t, _P]),
+    "dmlhip_gemm_f16_grouped": (c_int, [POINTER(GemmDesc), c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                        POINTER(c_void_p), _P, c_size_t, _P]),
     "dmlhip_gemm_f32": (c_int, [POINTER(GemmDesc), _P, _P, _P, _P, _P, _P, _P]),
     "dmlhip_conv2d_out_shape": (c_int, [POINTER(Conv2dDesc), _I64P, _I64P]),
     "dmlhip_conv2d_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, _P]),
@@ -111,6 +114,7 @@ SIGNATURES = {
 # exported for the test-suite only (not declared in the public header)
 DEBUG_SIGNATURES = {
     "dmlhip_debug_force_gemm_config": (None, [c_int]),
+    "dmlhip_debug_grouped_single_launches": (ctypes.c_longlong, []),
 }
 
 _lib = None

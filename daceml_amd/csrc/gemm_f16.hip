@@ -376,9 +376,22 @@ extern "C" {
 // Not part of the public header: lets the tests exercise every tile configuration.
 void dmlhip_debug_force_gemm_config(int cfg) { g_force_cfg = cfg; }
 void dmlhip_debug_gemm_direct_lds(int on) { g_direct_lds = on; }
+static long long g_grouped_single_launches = 0;
+// Number of grouped calls that went out as ONE launch (tests check that grouping really happens).
+long long dmlhip_debug_grouped_single_launches() { return g_grouped_single_launches; }
 
+struct GemmGroup {
+    int count;
+    const void* const* a;
+    const void* const* b;
+    void* const* c;
+    const void* const* bias;
+};
+
+// grp != nullptr: a / b / c / bias are those of group 0 (used for the layout checks, which the caller has made sure
+// hold for every group); returns DMLHIP_ERR_UNSUPPORTED when the grouped launch is not possible.
 static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, void* c, const void* bias,
-                        const void* residual, void* pre_out, void* stream) {
+                        const void* residual, void* pre_out, void* stream, const GemmGroup* grp = nullptr) {
     DML_REQUIRE(d, DMLHIP_ERR_NULL, "gemm_f16: NULL descriptor");
     DML_REQUIRE(d->m >= 0 && d->n >= 0 && d->k >= 0, DMLHIP_ERR_SHAPE, "gemm_f16: negative extent");
     DML_REQUIRE(d->m <= 2147483647 / 2 && d->n <= 2147483647 / 2 && d->k <= 2147483647 / 2, DMLHIP_ERR_SHAPE,
@@ -403,6 +416,17 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
     DML_REQUIRE(d->k == 0 || (a && b), DMLHIP_ERR_NULL, "gemm_f16: NULL operand");
 
     GemmArgs g;
+    g.groups = 0;
+    if (grp) {
+        g.groups = grp->count;
+        batch *= grp->count;
+        for (int i = 0; i < grp->count; ++i) {
+            g.ga[i] = (const _Float16*)grp->a[i];
+            g.gb[i] = (const _Float16*)grp->b[i];
+            g.gc[i] = grp->c[i];
+            g.gbias[i] = grp->bias ? grp->bias[i] : nullptr;
+        }
+    }
     g.m = (int)d->m; g.n = (int)d->n; g.k = (int)d->k;
     g.sam = d->a_stride_m; g.sak = d->a_stride_k; g.sbn = d->b_stride_n; g.sbk = d->b_stride_k;
     g.scm = d->c_stride_m;
@@ -447,6 +471,7 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
         return launch_pipelined(g, (const _Float16*)a, (const _Float16*)b, c, bias, residual, pre_out, amode == 1 ? 4 : 3,
                                 bmode == 1 ? 4 : 3, cfg, batch, st);
     }
+    if (grp) return DMLHIP_ERR_UNSUPPORTED;  // only the pipelined kernel takes pointer groups
     if (cfg < 0 || cfg > 2) {
         // Largest tile that still yields at least one workgroup per CU.
         auto blocks = [&](int bm, int bn) { return (long long)ceil_div(d->m, bm) * ceil_div(d->n, bn) * batch; };
@@ -527,6 +552,36 @@ int dmlhip_gemm_f16_ws(const dmlhip_gemm_desc* d, const void* a, const void* b, 
 int dmlhip_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, void* c, const void* bias,
                     const void* residual, void* pre_out, void* stream) {
     return run_gemm_f16(d, a, b, c, bias, residual, pre_out, stream);
+}
+
+int dmlhip_gemm_f16_grouped(const dmlhip_gemm_desc* d, int groups, const void* const* a, const void* const* b,
+                            void* const* c, const void* const* bias, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+    DML_REQUIRE(d, DMLHIP_ERR_NULL, "gemm_f16_grouped: NULL descriptor");
+    DML_REQUIRE(groups >= 1 && groups <= DMLHIP_GROUP_MAX, DMLHIP_ERR_SHAPE, "gemm_f16_grouped: %d groups outside 1..%d",
+                groups, DMLHIP_GROUP_MAX);
+    DML_REQUIRE(a && b && c, DMLHIP_ERR_NULL, "gemm_f16_grouped: NULL pointer table");
+    DML_REQUIRE(d->batch[0] == 1, DMLHIP_ERR_SHAPE, "gemm_f16_grouped: the outer batch extent must be 1");
+    for (int i = 0; i < groups; ++i) DML_REQUIRE(c[i], DMLHIP_ERR_NULL, "gemm_f16_grouped: NULL output %d", i);
+    // one launch when every group has the alignment of group 0 and the pipelined kernel applies
+    bool same = d->k > 0 && d->beta == 0.f;
+    for (int i = 0; i < groups && same; ++i) {
+        same = a[i] && b[i] && aligned16(a[i]) && aligned16(b[i]) && reinterpret_cast<uintptr_t>(c[i]) % 32 == 0 &&
+               (!bias == !(bias && bias[i])) && (!bias || aligned16(bias[i]));
+    }
+    if (same && groups > 1) {
+        dmlhip_gemm_desc p = *d;
+        p.a_stride_batch[0] = p.b_stride_batch[0] = p.c_stride_batch[0] = 0;   // the outer batch index selects the group
+        GemmGroup grp = {groups, a, b, c, bias};
+        const int e = run_gemm_f16(&p, a[0], b[0], c[0], bias ? bias[0] : nullptr, nullptr, nullptr, stream, &grp);
+        if (e == 0) ++g_grouped_single_launches;
+        if (e != DMLHIP_ERR_UNSUPPORTED) return e;
+    }
+    for (int i = 0; i < groups; ++i)
+        if (int e = dmlhip_gemm_f16_ws(d, a[i], b[i], c[i], bias ? bias[i] : nullptr, nullptr, nullptr, workspace,
+                                       workspace_bytes, stream))
+            return e;
+    return 0;
 }
 
 }  // extern "C"

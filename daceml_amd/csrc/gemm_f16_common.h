@@ -23,6 +23,13 @@ struct GemmArgs {
     int out_f32, bias_f32, act, bias_m, c_vec;
     int tiles_m, tiles_n;
     long long total_blocks;
+    // grouped launch: the outer batch index selects one of `groups` independent problems of identical shape and
+    // strides (0 = an ordinary launch, pointers come from the kernel parameters)
+    int groups;
+    const _Float16* ga[DMLHIP_GROUP_MAX];
+    const _Float16* gb[DMLHIP_GROUP_MAX];
+    void* gc[DMLHIP_GROUP_MAX];
+    const void* gbias[DMLHIP_GROUP_MAX];
 };
 
 template <int I, int N, typename F>

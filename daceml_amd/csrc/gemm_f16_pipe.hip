@@ -126,8 +126,7 @@ __device__ unsigned* dml_gemm_trace_buf;
 
 // ---------------------------------------------------------------- kernel
 template <int BM, int BN, int WM, int WN, int AKIND, int BKIND, int NSTAGE, int EPI>
-__global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16* __restrict__ a_ptr,
-                                                                 const _Float16* __restrict__ b_ptr, void* c_ptr,
+__global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16* a_ptr, const _Float16* b_ptr, void* c_ptr,
                                                                  const void* bias_ptr, const void* res_ptr,
                                                                  void* pre_ptr, const GemmArgs g) {
     static_assert((BM / WM) * (BN / WN) == kThreads / kWave, "four wavefronts per workgroup");
@@ -161,6 +160,12 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     const int z2 = (int)(batch % g.batch2);
     const int z1 = (int)((batch / g.batch2) % g.batch1);
     const int z0 = (int)(batch / ((long long)g.batch2 * g.batch1));
+    if (g.groups) {  // uniform: one of several same-shaped problems (host sets the outer batch strides to 0)
+        a_ptr = g.ga[z0];
+        b_ptr = g.gb[z0];
+        c_ptr = g.gc[z0];
+        bias_ptr = g.gbias[z0];
+    }
     const _Float16* A = a_ptr + z0 * g.sab[0] + z1 * g.sab[1] + z2 * g.sab[2];
     const _Float16* B = b_ptr + z0 * g.sbb[0] + z1 * g.sbb[1] + z2 * g.sbb[2];
     const int64_t coff = z0 * g.scb[0] + z1 * g.scb[1] + z2 * g.scb[2];

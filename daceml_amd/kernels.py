@@ -483,3 +483,36 @@ def reduce_sum_multi(xs: Sequence[torch.Tensor], out_dtype: Optional[torch.dtype
     L.check(_fn("reduce_sum_multi", xs[0].dtype)(n, xp, yp, L.F16 if odt == torch.float16 else L.F32, rows, cols, _ptr(ws),
                                                   ws.numel(), _stream()))
     return ys
+
+
+def einsum_grouped(equation: str, a_list: Sequence[torch.Tensor], b_list: Sequence[torch.Tensor], *,
+                   out_dtype: Optional[torch.dtype] = None, alpha: float = 1.0,
+                   bias_list: Optional[Sequence[torch.Tensor]] = None):
+    """Several fp16 two-operand einsums with the same equation, shapes and strides in one launch (at most four).
+    Tensors of different groups are independent allocations; an operand may repeat (a shared input)."""
+    from . import contraction as C
+    n = len(a_list)
+    if n != len(b_list) or (bias_list is not None and len(bias_list) != n):
+        raise ValueError("einsum_grouped: lists differ in length")
+    _check(*a_list, *b_list, *(bias_list or []), dtype=None)
+    a0, b0 = a_list[0], b_list[0]
+    if a0.dtype != torch.float16:
+        raise TypeError("einsum_grouped is implemented for fp16 operands")
+    for a, b in zip(a_list, b_list):
+        if a.shape != a0.shape or a.stride() != a0.stride() or b.shape != b0.shape or b.stride() != b0.stride() \
+                or a.dtype != a0.dtype or b.dtype != a0.dtype:
+            raise ValueError("einsum_grouped: every group needs the shapes, strides and dtype of group 0")
+    out_dtype = out_dtype or a0.dtype
+    plan = C.plan_contraction(equation, a0.shape, a0.stride(), b0.shape, b0.stride())
+    if plan.batch[0] != 1:
+        raise C.NotApplicable("einsum_grouped: three batch dimensions leave no slot for the group index")
+    outs = [torch.empty(plan.out_shape, dtype=out_dtype, device=a0.device) for _ in range(n)]
+    xs, ys = (b_list, a_list) if plan.swapped else (a_list, b_list)
+    desc = _fill_desc(plan, alpha, 0.0, out_dtype, bias_list[0] if bias_list else None, L.ACT_NONE)
+    arr = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])  # noqa: E731
+    lib = L.load()
+    need = lib.dmlhip_gemm_f16_workspace_bytes(ctypes.byref(desc))
+    ws = workspace(need, a0.device)
+    L.check(lib.dmlhip_gemm_f16_grouped(ctypes.byref(desc), n, arr(xs), arr(ys), arr(outs),
+                                        arr(bias_list) if bias_list else None, _ptr(ws), ws.numel(), _stream()))
+    return outs

@@ -45,7 +45,7 @@ def parse_variadic_param(param: str) -> Tuple[str, int]:
 @dataclasses.dataclass
 class ONNXParameter:
     name: str
-    kind: str = "single"  # single | optional | variadic
+    kind: str = "single"  # single | optional | variadic | variadic?
 
 
 @dataclasses.dataclass
@@ -57,16 +57,16 @@ class ONNXSchema:
     since_version: int = 12
 
     def non_variadic_inputs(self):
-        return [p.name for p in self.inputs if p.kind != "variadic"]
+        return [p.name for p in self.inputs if not p.kind.startswith("variadic")]
 
     def variadic_inputs(self):
-        return [p.name for p in self.inputs if p.kind == "variadic"]
+        return [p.name for p in self.inputs if p.kind.startswith("variadic")]
 
     def non_variadic_outputs(self):
-        return [p.name for p in self.outputs if p.kind != "variadic"]
+        return [p.name for p in self.outputs if not p.kind.startswith("variadic")]
 
     def variadic_outputs(self):
-        return [p.name for p in self.outputs if p.kind == "variadic"]
+        return [p.name for p in self.outputs if p.kind.startswith("variadic")]
 
 
 REQUIRED = object()
@@ -75,7 +75,9 @@ REQUIRED = object()
 def _p(spec: str) -> List[ONNXParameter]:
     out = []
     for tok in spec.split():
-        if tok.endswith("?"):
+        if tok.endswith("*?"):
+            out.append(ONNXParameter(tok[:-2], "variadic?"))   # variadic, and allowed to be absent altogether
+        elif tok.endswith("?"):
             out.append(ONNXParameter(tok[:-1], "optional"))
         elif tok.endswith("*"):
             out.append(ONNXParameter(tok[:-1], "variadic"))
@@ -133,6 +135,9 @@ SCHEMAS = [
     # Conv 1x1 whose input is first multiplied by a per-image, per-channel factor Gate [n, c, 1, 1] (squeeze-excite)
     _schema("GatedConv", "X Gate W B?", "Y", since=1, auto_pad="NOTSET", dilations=None, group=1, kernel_shape=None,
             pads=None, strides=None),
+    # several FusedEinsum nodes of identical equation, shapes, strides and scale, independent of each other, in one
+    # launch: Output__i = alpha * einsum(equation, A__i, B__i) [+ Bias__i]
+    _schema("GroupedEinsum", "A* B* Bias*?", "Output*", since=1, equation=REQUIRED, alpha=1.0),
     # several independent ReduceSum(all leading axes, keepdims=0) nodes in one launch pair: reduced__i = sum of
     # data__i over every axis but the last (the bias gradients of a backward pass)
     _schema("MultiReduceSum", "data*", "reduced*", since=1),
@@ -220,20 +225,22 @@ class ONNXOp(Node):
                 base = conn
                 if "__" in conn:
                     base, idx = parse_variadic_param(conn)
-                    if base not in names or names[base].kind != "variadic":
+                    if base not in names or not names[base].kind.startswith("variadic"):
                         raise ValueError("{}: '{}' is not a variadic parameter of {}".format(
                             self.label, base, self.schema.name))
                     seen.setdefault(base, []).append(idx)
                 elif base not in names:
                     raise ValueError("{}: unknown connector '{}' for {}".format(self.label, conn, self.schema.name))
-                elif names[base].kind == "variadic":
+                elif names[base].kind.startswith("variadic"):
                     raise ValueError("{}: variadic parameter '{}' must be numbered".format(self.label, base))
             for p in params:
                 if p.kind == "single" and p.name not in edge_conns:
                     raise ValueError("{}: required {} connector '{}' of {} is not connected".format(
                         self.label, "input" if is_input else "output", p.name, self.schema.name))
-                if p.kind == "variadic":
+                if p.kind.startswith("variadic"):
                     idxs = sorted(seen.get(p.name, []))
+                    if not idxs and p.kind == "variadic?":
+                        continue
                     if not idxs:
                         raise ValueError("{}: variadic parameter '{}' needs at least one edge".format(
                             self.label, p.name))

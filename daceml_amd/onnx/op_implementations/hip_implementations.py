@@ -1090,3 +1090,67 @@ class HipMultiReduceSum(ONNXForward):
                         I64Array(rows), I64Array(cols), Workspace(), WorkspaceBytes(), Stream()])
         return _tasklet(node, state, [call], workspace_bytes=ws,
                         bytes_moved=sum(_nbytes(x, y) for x, y in pairs), kind="reduce")
+
+
+# ----------------------------------------------------------------------------- several equal contractions at once
+@op_implementation(op="GroupedEinsum", name=IMPL)
+class HipGroupedEinsum(ONNXForward):
+    """Up to four PureEinsum contractions (pure_implementations.py:219-252) of identical equation, shapes and
+    strides in one grouped GEMM launch — the effect HorizontalEinsumFusion (transformation/einsum_fusion.py:102-151)
+    has on the Q/K/V projections, without requiring the operands to be adjacent in memory."""
+    @staticmethod
+    def _groups(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        n = len(outs)
+        a = [ins["A__%d" % i] for i in range(n)]
+        b = [ins["B__%d" % i] for i in range(n)]
+        bias = [ins["Bias__%d" % i] for i in range(n)] if "Bias__0" in ins else None
+        out = [outs["Output__%d" % i] for i in range(n)]
+        return n, a, b, bias, out
+
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            n, a, b, bias, out = HipGroupedEinsum._groups(node, state, sdfg)
+            if not 2 <= n <= L.GROUP_MAX or a[0].dtype != torch.float16:
+                return False
+            eq = node.equation.replace(" ", "")
+            for i in range(n):
+                if (a[i].shape, a[i].strides, a[i].dtype) != (a[0].shape, a[0].strides, a[0].dtype):
+                    return False
+                if (b[i].shape, b[i].strides, b[i].dtype) != (b[0].shape, b[0].strides, a[0].dtype):
+                    return False
+                if (out[i].shape, out[i].dtype) != (out[0].shape, out[0].dtype):
+                    return False
+                if not _einsum_can_apply(eq, [a[i], b[i]], out[i], allow_f32_out=True):
+                    return False
+            plan = _einsum_plan(eq, a[0], b[0])
+            if plan is None or plan.batch[0] != 1:
+                return False
+            if bias is not None:
+                for t in bias:
+                    if not (t.dtype == bias[0].dtype and t.dtype in FLOAT_DTYPES and t.is_contiguous()
+                            and t.total_size == plan.n and t.shape[-1] == plan.n):
+                        return False
+            return True
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        import ctypes
+        n, a, b, bias, out = HipGroupedEinsum._groups(node, state, sdfg)
+        eq = node.equation.replace(" ", "")
+        plan = C.plan_contraction(eq, a[0].shape, a[0].strides, b[0].shape, b[0].strides)
+        desc = _gemm_struct(plan, node.alpha, 0.0, out[0].dtype, bias[0].dtype if bias else out[0].dtype, L.ACT_NONE)
+        xa, xb = ("B", "A") if plan.swapped else ("A", "B")
+        ws = L.load().dmlhip_gemm_f16_workspace_bytes(ctypes.byref(desc))
+        call = HipCall("dmlhip_gemm_f16_grouped",
+                       [Struct(desc, "dmlhip_gemm_desc"), I32(n), PtrArray(tuple("%s__%d" % (xa, i) for i in range(n))),
+                        PtrArray(tuple("%s__%d" % (xb, i) for i in range(n))),
+                        PtrArray(tuple("Output__%d" % i for i in range(n))),
+                        PtrArray(tuple("Bias__%d" % i for i in range(n))) if bias else Null(), Workspace(),
+                        WorkspaceBytes(), Stream()])
+        extra = bias or []
+        return _tasklet(node, state, [call], workspace_bytes=ws, flops=plan.flops * n,
+                        bytes_moved=sum(_nbytes(a[i], b[i], out[i]) for i in range(n)) + _nbytes(*extra), kind="gemm")

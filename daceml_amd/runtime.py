@@ -148,7 +148,9 @@ class CompiledSDFG:
                     else:
                         args.append(self._ptr[name])
                 elif isinstance(a, T.Null):
-                    args.append(ctypes.c_void_p(0))
+                    # None, not c_void_p(0): for a POINTER(c_void_p) parameter ctypes would pass the ADDRESS of a
+                    # c_void_p instance (a non-NULL pointer table with one NULL entry)
+                    args.append(None)
                 elif isinstance(a, T.I64):
                     args.append(ctypes.c_int64(a.value))
                 elif isinstance(a, T.I32):

@@ -19,6 +19,7 @@ expansions it replaces (that composition is the oracle of the fused kernels).
     fuse_skip_layernorm      Add, LayerNormalization                      -> SkipLayerNormalization
     fuse_attention           Einsum(Q,K)[*scale], Softmax, Einsum(P,V)    -> FusedAttention
     fuse_reductions          independent ReduceSum(leading axes) nodes    -> MultiReduceSum (one launch pair)
+    group_einsums            independent, identically shaped FusedEinsums -> GroupedEinsum (one launch)
     fuse_conv_activation     Conv, Swish | Sigmoid | Relu                 -> Conv(_activation)
     fuse_gate_into_conv      Mul(X, gate[n,c,1,1]), Conv 1x1              -> GatedConv (inference graphs)
 """
@@ -723,10 +724,102 @@ def fuse_reductions(sdfg: SDFG, max_group: int = 8) -> int:
     return merged
 
 
+def _reachable(sdfg: SDFG, state: SDFGState, src) -> set:
+    """Nodes reachable from `src` along the state's edges."""
+    succ = {}
+    for e in state.edges():
+        succ.setdefault(e.src, []).append(e.dst)
+
+    def root(name):
+        while sdfg.arrays[name].view_of is not None:
+            name = sdfg.arrays[name].view_of
+        return name
+
+    # access nodes of one buffer are distinct objects per use, and views alias their base: join them by root array
+    by_array = {}
+    for n in state.nodes():
+        if isinstance(n, AccessNode):
+            by_array.setdefault(root(n.data), []).append(n)
+    seen, stack = set(), [src]
+    while stack:
+        n = stack.pop()
+        nxt = list(succ.get(n, []))
+        if isinstance(n, AccessNode):
+            nxt += [m for m in by_array[root(n.data)] if m is not n]
+        for m in nxt:
+            if m not in seen:
+                seen.add(m)
+                stack.append(m)
+    return seen
+
+
+def group_einsums(sdfg: SDFG, max_group: int = 4) -> int:
+    """Horizontal fusion of contractions (cf. HorizontalEinsumFusion, daceml/transformation/einsum_fusion.py:102-151):
+    FusedEinsum nodes with the same equation, scale, operand shapes / strides / types (optionally a bias each, no
+    residual, activation or accumulation) and no data dependence on each other become one GroupedEinsum — the
+    Q/K/V projections of an attention block, and in the backward pass their input and weight gradients. Works on
+    every state, so it is run after autodiff. Returns the number of nodes merged away."""
+    merged = 0
+    for state in sdfg.states():
+        buckets = {}
+        for n in state.nodes():
+            if not _is_op(n, "FusedEinsum") or n.activation != "none" or n.accumulate:
+                continue
+            conns = {e.dst_conn for e in state.in_edges(n)} | {e.src_conn for e in state.out_edges(n)}
+            if conns - {"Inputs__0", "Inputs__1", "Bias", "Output"} or not {"Inputs__0", "Inputs__1", "Output"} <= conns:
+                continue
+            a = sdfg.arrays[_in_array(state, n, "Inputs__0")]
+            b = sdfg.arrays[_in_array(state, n, "Inputs__1")]
+            o = sdfg.arrays[_out_array(state, n, "Output")]
+            if a.dtype != torch.float16 or b.dtype != torch.float16 or not o.is_contiguous():
+                continue
+            bias = _in_array(state, n, "Bias")
+            key = (n.equation.replace(" ", ""), float(n.alpha), tuple(a.shape), tuple(a.strides), tuple(b.shape),
+                   tuple(b.strides), tuple(o.shape), o.dtype, None if bias is None else sdfg.arrays[bias].dtype)
+            buckets.setdefault(key, []).append(n)
+        for key, nodes in buckets.items():
+            if len(nodes) < 2:
+                continue
+            nodes.sort(key=lambda n: n.label)   # the result must not depend on the order the state lists its nodes in
+            try:
+                plan = C.plan_contraction(key[0], key[2], key[3], key[4], key[5])
+            except (C.NotApplicable, ValueError):
+                continue
+            if plan.batch[0] != 1:
+                continue
+            # greedy grouping of mutually independent nodes
+            reach = {n: _reachable(sdfg, state, n) for n in nodes}
+            groups: List[List[ONNXOp]] = []
+            for n in nodes:
+                for grp in groups:
+                    if len(grp) < max_group and all(n not in reach[m] and m not in reach[n] for m in grp):
+                        grp.append(n)
+                        break
+                else:
+                    groups.append([n])
+            for grp in groups:
+                if len(grp) < 2:
+                    continue
+                ins, outs = {}, {}
+                for i, n in enumerate(grp):
+                    ins["A__%d" % i] = _in_array(state, n, "Inputs__0")
+                    ins["B__%d" % i] = _in_array(state, n, "Inputs__1")
+                    bias = _in_array(state, n, "Bias")
+                    if bias is not None:
+                        ins["Bias__%d" % i] = bias
+                    outs["Output__%d" % i] = _out_array(state, n, "Output")
+                label = "grouped_" + "_".join(n.label.replace("_matmul_fused", "") for n in grp)
+                for n in grp:
+                    _remove_node(state, n)
+                _add_node(sdfg, state, "GroupedEinsum", label, ins, outs, equation=key[0], alpha=key[1])
+                merged += len(grp) - 1
+    return merged
+
+
 def optimize_backward(sdfg: SDFG) -> Dict[str, int]:
     """Rewrites for the state(s) autodiff added — what a ``post_autodiff_hooks`` entry of the reference's module
     wrapper would run (daceml/torch/module.py:46-365)."""
-    return {"reductions": fuse_reductions(sdfg)}
+    return {"reductions": fuse_reductions(sdfg), "grouped_einsums": group_einsums(sdfg)}
 
 
 def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True,

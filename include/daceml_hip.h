@@ -215,6 +215,16 @@ int dmlhip_gemm_f16_ws(const dmlhip_gemm_desc* desc, const void* a, const void* 
                        const void* bias, const void* residual, void* pre_out, void* workspace,
                        size_t workspace_bytes, void* stream);
 /* inputs fp32, true fp32 MFMA (no reduced-precision path); out_dtype must be DMLHIP_F32 */
+/* Several products of identical shape, strides and epilogue (alpha, column bias) on different tensors in one
+ * launch: groups <= DMLHIP_GROUP_MAX, tensor i uses a[i], b[i], c[i], bias[i] (bias may be NULL: none). This is
+ * HorizontalEinsumFusion's purpose (daceml/transformation/einsum_fusion.py:102-151: the three Q/K/V projections of
+ * an attention block as one contraction) without requiring the operands to be adjacent in memory. d->batch[0]
+ * must be 1 and d->beta 0; no residual / pre-activation / activation. Falls back to `groups` separate calls of
+ * dmlhip_gemm_f16_ws (with the given workspace) when one launch is not possible. */
+#define DMLHIP_GROUP_MAX 4
+int dmlhip_gemm_f16_grouped(const dmlhip_gemm_desc* d, int groups, const void* const* a,
+                            const void* const* b, void* const* c, const void* const* bias,
+                            void* workspace, size_t workspace_bytes, void* stream);
 int dmlhip_gemm_f32(const dmlhip_gemm_desc* desc, const void* a, const void* b, void* c,
                     const void* bias, const void* residual, void* pre_out, void* stream);
 

@@ -502,3 +502,28 @@ def test_reduce_sum_multi(dtype):
     r, a = tol(dtype)
     assert_close(host(one[0]), O.reduce_sum(pairs[1][1], [0, 1], 0), dtype, "reduce_sum_multi single",
                  atol=a * np.sqrt(600))  # sums of 600 terms
+
+
+# ----------------------------------------------------------------------------- grouped contractions
+@pytest.mark.parametrize("eq,sa,sb,with_bias,out_dtype", [
+    ("aik,jk->aij", (2, 256, 128), (192, 128), True, torch.float16),     # Q/K/V projections of one input
+    ("aij,jk->aik", (2, 128, 192), (192, 256), False, torch.float16),    # their input gradients
+    ("aij,aik->jk", (2, 256, 128), (2, 256, 64), False, torch.float32),  # their weight gradients (fp32 masters)
+    ("ik,kj->ij", (100, 72), (72, 50), True, torch.float16),             # K % 64 != 0: falls back to separate launches
+])
+def test_einsum_grouped(eq, sa, sb, with_bias, out_dtype):
+    from daceml_amd import contraction as C, kernels as K
+    n = 3
+    plan_n = C.plan_contraction(eq, sa, C.contiguous_strides(sa), sb, C.contiguous_strides(sb)).out_shape[-1]
+    a = [_inputs(300 + i, sa, torch.float16) for i in range(n)]
+    b = [_inputs(310 + i, sb, torch.float16, 0.2) for i in range(n)]
+    bias = [_inputs(320 + i, (plan_n, ), torch.float16) for i in range(n)] if with_bias else None
+    a[1] = a[0]  # a shared operand (the layer input of the three projections)
+    got = K.einsum_grouped(eq, [dev(x) for x, _ in a], [dev(x) for x, _ in b], out_dtype=out_dtype,
+                           bias_list=[dev(x) for x, _ in bias] if bias else None)
+    for i in range(n):
+        want = O.einsum(eq, a[i][1], b[i][1])
+        if bias:
+            want = want + bias[i][1]
+        assert got[i].dtype == out_dtype
+        assert_close(host(got[i]), want, torch.float16, "grouped einsum %s group %d" % (eq, i))

@@ -351,9 +351,17 @@ def test_attention_fusion_roles_and_graph():
     assert ins == {"Q", "K", "V", "O", "LogSumExp", "dO"}
     # the six bias gradients become one node; nothing else in the state changes
     n_before = len(sdfg.states()[1].library_nodes())
-    assert fusion.optimize_backward(sdfg) == {"reductions": 5}
+    assert fusion.optimize_backward(sdfg) == {"reductions": 5, "grouped_einsums": 7}
     bnodes = sdfg.states()[1].library_nodes()
-    assert len(bnodes) == n_before - 5 and not any(n.schema.name == "ReduceSum" for n in bnodes)
+    # five reductions and five contractions fewer (q/k/v input gradients: 3 -> 1; o/q/k/v weight gradients: 4 -> 1)
+    assert len(bnodes) == n_before - 10 and not any(n.schema.name == "ReduceSum" for n in bnodes)
+    grouped = sorted(n.label for st_ in sdfg.states() for n in st_.library_nodes() if n.schema.name == "GroupedEinsum")
+    assert grouped == ["grouped_k_grad_0_q_grad_0_v_grad_0", "grouped_k_grad_1_o_grad_1_q_grad_1_v_grad_1", "grouped_k_q_v"]
+    # grouping respects data dependences, also through views: o's input gradient feeds the attention backward
+    # whose outputs the q/k/v gradients read, so it stays on its own; the states still sort topologically
+    assert any(n.label == "o_matmul_fused_grad_0" for n in bnodes)
+    for st_ in sdfg.states():
+        st_.topological_sort()
     multi = [n for n in bnodes if n.schema.name == "MultiReduceSum"][0]
     outs = sorted(e.data.data for e in sdfg.states()[1].out_edges(multi))
     assert outs == sorted("gradient_%s_b" % p for p in ("q", "k", "v", "o", "ffn1", "ffn2"))
