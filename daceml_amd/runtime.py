@@ -184,11 +184,13 @@ class CompiledSDFG:
                                           node.bytes_moved if first else 0, node.kind, state.label))
 
     # -- execution -----------------------------------------------------------
-    def _bind_arguments(self, kwargs: Dict[str, torch.Tensor]):
+    def _bind_arguments(self, kwargs: Dict[str, torch.Tensor], partial: bool = False):
         for name, desc in self.sdfg.arrays.items():
             if desc.transient or name in self.sdfg.constants or desc.view_of is not None:
                 continue
             if name not in kwargs:
+                if partial:
+                    continue
                 raise TypeError("missing argument %r (arrays to pass: %s)" % (name, sorted(self.arglist())))
             t = kwargs[name]
             if not isinstance(t, torch.Tensor) or t.device != self.device:
@@ -211,6 +213,12 @@ class CompiledSDFG:
     def __call__(self, **kwargs):
         self._bind_arguments(kwargs)
         self.launch()
+
+    def bind(self, tensors: Dict[str, torch.Tensor]):
+        """Bind some of the caller-owned arrays; the others keep the pointers of their last binding. For callers
+        that run the states separately (forward now, backward later) with ``launch(states)``; the tensors must stay
+        alive until the launches that use them have been enqueued."""
+        self._bind_arguments(tensors, partial=True)
 
     def launch(self, states: Optional[Sequence[str]] = None):
         """Enqueue every kernel (of the named states) on the current stream, with the pointers of the

@@ -216,7 +216,19 @@ def _match_layernorm(sdfg, state, sqrt):
         return None
     cen_arr = _in_array(state, powr, "X")
     sub = single(cen_arr, "Sub")
-    if sub is None or not _internal(sdfg, state, cen_arr, 2):
+    casts = []
+    if sub is None:
+        # a half-precision LayerNorm is exported with the variance computed in a wider type: Sub -> Cast -> Pow ...
+        # Div -> Cast -> Mul. The fused kernel does all of its arithmetic in fp32, so the casts fold away.
+        cast_in = single(cen_arr, "Cast")
+        if cast_in is None:
+            return None
+        narrow = _in_array(state, cast_in, "input")
+        sub = single(narrow, "Sub")
+        if sub is None or not _internal(sdfg, state, narrow):
+            return None
+        casts.append(cast_in)
+    if not _internal(sdfg, state, cen_arr, 2):
         return None
     x, mean_arr = _binary_operands(state, sub)
     mean = single(mean_arr, "ReduceMean")
@@ -236,6 +248,14 @@ def _match_layernorm(sdfg, state, sqrt):
         return None
     nrm = _out_array(state, div, "C")
     cons = _consumers(state, nrm)
+    if casts:
+        if len(cons) != 1 or not _is_op(cons[0][0], "Cast") or not _internal(sdfg, state, nrm):
+            return None
+        casts.append(cons[0][0])
+        nrm = _out_array(state, cons[0][0], "output")
+        if sdfg.arrays[nrm].dtype != sdfg.arrays[x].dtype:
+            return None
+        cons = _consumers(state, nrm)
     if len(cons) != 1 or not _is_op(cons[0][0], "Mul") or not _internal(sdfg, state, nrm):
         return None
     mul = cons[0][0]
@@ -250,7 +270,7 @@ def _match_layernorm(sdfg, state, sqrt):
     if len(beta) != 1 or sdfg.arrays[gamma[0]].total_size != h or sdfg.arrays[beta[0]].total_size != h:
         return None
     out = _out_array(state, add, "C")
-    return x, gamma[0], beta[0], eps, out, [mean, sub, powr, var, addeps, sqrt, div, mul, add]
+    return x, gamma[0], beta[0], eps, out, [mean, sub, powr, var, addeps, sqrt, div, mul, add] + casts
 
 
 # ----------------------------------------------------------------------------- Swish

@@ -1,0 +1,305 @@
+"""The PyTorch-facing side of the path: ONNX wire reader, importer, DaceModule (cf. the reference's
+tests/pytorch/test_module_api.py, tests/pytorch/test_bert_encoder.py, tests/test_models/test_efficientnet.py:
+wrap a torch module, call it, compare with the module itself)."""
+import collections
+import copy
+import struct
+import warnings
+
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+from daceml_amd.onnx import proto
+from daceml_amd.onnx.onnx_importer import ONNXModel, UnsupportedModel, clean_onnx_name
+from daceml_amd.torch import DaceModule, dace_module
+from daceml_amd.torch.export import export_onnx
+from util import assert_close, host
+
+
+# ----------------------------------------------------------------------------- modules under test
+class SmallEncoder(nn.Module):
+    """Linear + GELU + LayerNorm + a 4-head attention with head size 4 + Linear + residual."""
+    def __init__(self):
+        super().__init__()
+        self.l1 = nn.Linear(8, 16)
+        self.ln = nn.LayerNorm(16)
+        self.l2 = nn.Linear(16, 8)
+
+    def forward(self, x):
+        h = self.ln(nn.functional.gelu(self.l1(x)))
+        b, t, _ = h.shape
+        h = h.view(b, t, 4, 4).permute(0, 2, 1, 3)
+        a = torch.softmax(torch.matmul(h, h.transpose(-1, -2)) / 2.0, dim=-1)
+        h = torch.matmul(a, h).permute(0, 2, 1, 3).contiguous().view(b, t, 16)
+        return self.l2(h) + x
+
+
+class MBConv(nn.Module):
+    """EfficientNet-style block with folded BatchNorm: 1x1 expand, depthwise 3x3 stride 2, squeeze-excite, 1x1 project
+    (swish written as x * sigmoid(x), as efficientnet_pytorch's MemoryEfficientSwish exports)."""
+    def __init__(self, cin=8, mid=32, cout=16, se=4):
+        super().__init__()
+        self.expand = nn.Conv2d(cin, mid, 1)
+        self.dw = nn.Conv2d(mid, mid, 3, stride=2, padding=1, groups=mid)
+        self.se1 = nn.Conv2d(mid, se, 1)
+        self.se2 = nn.Conv2d(se, mid, 1)
+        self.proj = nn.Conv2d(mid, cout, 1)
+
+    def forward(self, x):
+        x = self.expand(x)
+        x = x * torch.sigmoid(x)
+        x = self.dw(x)
+        x = x * torch.sigmoid(x)
+        s = nn.functional.adaptive_avg_pool2d(x, 1)
+        s = self.se1(s)
+        s = s * torch.sigmoid(s)
+        s = self.se2(s)
+        x = torch.sigmoid(s) * x
+        return self.proj(x)
+
+
+class BertLayerOutput(nn.Module):
+    """HuggingFace BertLayer (what tests/pytorch/test_bert_encoder.py wraps), returning the hidden states only."""
+    def __init__(self, hidden, heads, ffn):
+        super().__init__()
+        from transformers import BertConfig
+        from transformers.models.bert.modeling_bert import BertLayer
+        cfg = BertConfig(hidden_size=hidden, num_attention_heads=heads, intermediate_size=ffn,
+                         hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0)
+        cfg._attn_implementation = "eager"
+        self.layer = BertLayer(cfg)
+
+    def forward(self, x):
+        out = self.layer(x)
+        return out[0] if isinstance(out, (tuple, list)) else out
+
+
+def _kinds(sdfg):
+    return collections.Counter(n.schema.name for st in sdfg.states() for n in st.library_nodes())
+
+
+# ----------------------------------------------------------------------------- wire reader
+def _varint(v):
+    v &= (1 << 64) - 1
+    out = bytearray()
+    while True:
+        b = v & 0x7F
+        v >>= 7
+        out.append(b | (0x80 if v else 0))
+        if not v:
+            return bytes(out)
+
+
+def _ld(num, payload):
+    return _varint(num << 3 | 2) + _varint(len(payload)) + payload
+
+
+def test_wire_reader_decodes_hand_built_messages():
+    # a TensorProto with dims [2, 2], int64 data given unpacked (one of them negative) and a name
+    t = _ld(1, _varint(2) + _varint(2)) + _varint(2 << 3) + _varint(7) + b"".join(
+        _varint(7 << 3) + _varint(v) for v in (1, -2, 3, 1 << 40)) + _ld(8, b"t0")
+    tp = proto.TensorProto(t)
+    assert tp.name == "t0" and tp.array.dtype == np.int64 and tp.array.tolist() == [[1, -2], [3, 1 << 40]]
+    # fp16 values travel as bit patterns in int32_data (packed here)
+    bits = np.array([1.5, -0.25], np.float16).view(np.uint16).tolist()
+    t = _ld(1, _varint(2)) + _varint(2 << 3) + _varint(10) + _ld(5, b"".join(_varint(b) for b in bits))
+    assert proto.TensorProto(t).array.tolist() == [1.5, -0.25]
+    # raw_data, float
+    t = _ld(1, _varint(3)) + _varint(2 << 3) + _varint(1) + _ld(9, struct.pack("<3f", 1.0, 2.0, -3.5))
+    assert proto.TensorProto(t).array.tolist() == [1.0, 2.0, -3.5]
+    # attributes: INT (negative), FLOAT, INTS packed, STRING
+    a = proto.AttributeProto(_ld(1, b"axis") + _varint(3 << 3) + _varint(-1) + _varint(20 << 3) + _varint(2))
+    assert (a.name, a.value) == ("axis", -1)
+    a = proto.AttributeProto(_ld(1, b"alpha") + _varint(2 << 3 | 5) + struct.pack("<f", 0.5) + _varint(20 << 3) + _varint(1))
+    assert a.value == 0.5
+    a = proto.AttributeProto(_ld(1, b"perm") + _ld(8, _varint(0) + _varint(2) + _varint(1)) + _varint(20 << 3) + _varint(7))
+    assert a.value == [0, 2, 1]
+    a = proto.AttributeProto(_ld(1, b"auto_pad") + _ld(4, b"NOTSET") + _varint(20 << 3) + _varint(3))
+    assert a.value == "NOTSET"
+    with pytest.raises(proto.ProtoError):
+        proto.TensorProto(t[:-3])                      # truncated
+    with pytest.raises(proto.ProtoError):
+        proto.load_model(_varint(1 << 3) + _varint(7))   # no graph
+
+
+def test_wire_reader_on_an_exported_model():
+    m = nn.Sequential(nn.Linear(8, 16), nn.GELU(), nn.LayerNorm(16))
+    model = proto.load_model(export_onnx(m, (torch.randn(2, 4, 8), )))
+    assert model.opset_import[""] == 12 and model.producer_name == "pytorch"
+    g = model.graph
+    ops = [n.op_type for n in g.node if n.op_type != "Constant"]
+    # nn.Linear = Transpose, MatMul, Add; exact GELU = Div, Erf, Add, Mul, Mul; LayerNorm = the nine-node chain
+    assert ops == ["Transpose", "MatMul", "Add", "Div", "Erf", "Add", "Mul", "Mul", "ReduceMean", "Sub", "Pow",
+                   "ReduceMean", "Add", "Sqrt", "Div", "Mul", "Add"]
+    inits = {t.name: t.array for t in g.initializer}
+    sd = m.state_dict()
+    assert set(inits) == set(sd)
+    for k, v in sd.items():
+        assert np.array_equal(inits[k], v.numpy())
+    x = [i for i in g.input if i.name not in inits]
+    assert len(x) == 1 and x[0].shape == [2, 4, 8] and x[0].elem_type == 1
+    consts = [n.attribute[0].value for n in g.node if n.op_type == "Constant"]
+    assert [round(float(c), 5) for c in consts] == [1.41421, 1.0, 0.5, 2.0, 1e-05]
+
+
+# ----------------------------------------------------------------------------- importer
+def test_importer_names_shapes_and_folding():
+    net = SmallEncoder()
+    model = ONNXModel("enc", export_onnx(net, (torch.randn(2, 4, 8), )), auto_optimize=False)
+    sdfg = model.sdfg
+    assert model.outputs == ["__return"] and len(model.inputs) == 1
+    assert set(model.weights) == set(net.state_dict())
+    assert clean_onnx_name("l1.weight") == "l1DOTweight" and clean_onnx_name("0.bias") == "ONNX_0DOTbias"
+    assert sdfg.arrays["l1DOTweight"].shape == (16, 8) and not sdfg.arrays["l1DOTweight"].transient
+    assert sdfg.arrays["__return"].shape == (2, 4, 8)
+    kinds = _kinds(sdfg)
+    # the Shape / Gather / Unsqueeze / Concat chains around view() are evaluated at import
+    assert not {"Shape", "Gather", "Unsqueeze", "Concat", "Constant"} & set(kinds)
+    assert kinds["Reshape"] == 2 and kinds["Softmax"] == 1 and kinds["MatMul"] == 4 and kinds["Transpose"] == 5
+    reshapes = [n for n in model.state.library_nodes() if n.schema.name == "Reshape"]
+    shapes = sorted(sdfg.arrays[e.data.data].shape for r in reshapes for e in model.state.out_edges(r))
+    assert shapes == [(2, 4, 4, 4), (2, 4, 16)]
+    stats = model.auto_optimize()
+    assert stats["gelu"] == 1 and stats["layernorm"] == 1 and stats["matmul_to_einsum"] == 4
+    assert _kinds(sdfg) == {"FusedEinsum": 3, "Einsum": 1, "Softmax": 1, "Gelu": 1, "LayerNormalization": 1}
+
+
+def test_importer_refuses_what_it_cannot_run():
+    class Odd(nn.Module):
+        def forward(self, x):
+            return torch.cumsum(x, dim=1)
+
+    with pytest.raises(UnsupportedModel, match="Unsupported ONNX operator: 'CumSum'"):
+        ONNXModel("odd", export_onnx(Odd(), (torch.randn(2, 3), )))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_huggingface_bert_layer_imports_to_the_fused_graph(dtype):
+    """The decomposition the real exporter emits for BertLayer is the one the hand-built bench graph assumes: after
+    the fusion pipeline both consist of the same library nodes."""
+    from daceml_amd import graphs
+    from daceml_amd.transformation import fusion
+    b, s, h, heads, ffn = 2, 64, 256, 4, 512
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        m = DaceModule(BertLayerOutput(h, heads, ffn).eval().to(dtype), backward=True)
+        model = m._import((torch.randn(b, s, h).to(dtype), ))
+    want = graphs.bert_encoder_layer(b, s, h, heads, ffn, dtype, eps=1e-12)
+    want_stats = fusion.auto_optimize(want, training=True)
+    assert _kinds(model.sdfg) == _kinds(want)
+    for k in ("gelu", "layernorm", "attention", "epilogues", "skip_layernorm"):
+        assert m.optimization_stats[k] == want_stats[k], k
+    if dtype == torch.float16:
+        assert _kinds(model.sdfg)["FusedAttention"] == 1
+    # parameters are graph inputs under their state_dict names
+    assert "layer.attention.self.query.weight" in model.inputs and not model.weights
+
+
+def test_module_hooks_and_decorator():
+    calls = []
+    m = DaceModule(SmallEncoder(), auto_optimize=False)
+    m.append_post_onnx_hook("b", lambda mod: calls.append("b"))
+    m.prepend_post_onnx_hook("a", lambda mod: calls.append("a"))
+    m.append_post_onnx_hook("b", lambda mod: calls.append("b2"))       # same name: made unique, both run
+    assert list(m.post_onnx_hooks) == ["a", "b", "b_0"]
+    m._import((torch.randn(2, 4, 8), ))
+    assert calls == ["a", "b", "b2"]
+    assert _kinds(m.sdfg)["MatMul"] == 4                                # nothing was fused
+    auto = DaceModule(SmallEncoder(), backward=True)
+    assert list(auto.post_onnx_hooks) == ["auto_optimize"] and list(auto.post_autodiff_hooks) == ["auto_optimize"]
+    with pytest.raises(ValueError):
+        DaceModule(SmallEncoder(), cuda=False)
+
+    @dace_module(backward=True)
+    class Wrapped(nn.Module):
+        def __init__(self, n):
+            super().__init__()
+            self.fc = nn.Linear(n, n)
+
+        def forward(self, x):
+            return self.fc(x)
+
+    w = Wrapped(4)
+    assert isinstance(w, DaceModule) and isinstance(w.model.fc, nn.Linear) and w.backward
+
+
+# ----------------------------------------------------------------------------- on the GPU
+def _compare_module(module, x, dtype, backward, rtol=None, atol=None, grad_rtol=None, grad_atol=None):
+    module = module.cuda().to(dtype)
+    ref = copy.deepcopy(module).double()
+    x = x.cuda().to(dtype)
+    wrapped = DaceModule(module, backward=backward)
+    xr = x.detach().double().requires_grad_(backward)
+    xs = x.detach().clone().requires_grad_(backward)
+    y = wrapped(xs)
+    want = ref(xr)
+    assert y.dtype == dtype and y.shape == want.shape
+    assert_close(host(y), want.detach().cpu().numpy(), dtype, "forward", rtol=rtol, atol=atol)
+    if not backward:
+        return wrapped
+    g = torch.randn(want.shape, generator=torch.Generator().manual_seed(5)).cuda()
+    y.backward(g.to(dtype))
+    want.backward(g.to(dtype).double())
+    assert_close(host(xs.grad), xr.grad.cpu().numpy(), dtype, "input gradient", rtol=grad_rtol, atol=grad_atol)
+    for (n, p), (_, pr) in zip(module.named_parameters(), ref.named_parameters()):
+        assert p.grad is not None, n
+        scale = float(pr.grad.abs().max())
+        a = (grad_atol if grad_atol is not None else (1e-2 if dtype == torch.float16 else 1e-6))
+        assert_close(host(p.grad), pr.grad.cpu().numpy(), dtype, "gradient of " + n, rtol=grad_rtol,
+                     atol=a * max(scale, 1.0))
+    return wrapped
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("backward", [False, True])
+def test_small_encoder_module(backward):
+    torch.manual_seed(0)
+    # a chain of seven fp32 nodes: rounding accumulates beyond one node's 1e-5 / 1e-6
+    w = _compare_module(SmallEncoder(), torch.randn(2, 4, 8), torch.float32, backward, rtol=1e-4, atol=1e-5,
+                        grad_rtol=1e-4, grad_atol=1e-5)
+    assert w.optimization_stats["gelu"] == 1 and w.optimization_stats["layernorm"] == 1
+    # a second call reuses the bound program and sees updated parameters
+    with torch.no_grad():
+        w.model.l2.bias.add_(1.0)
+    x = torch.randn(2, 4, 8, device="cuda")
+    assert_close(host(w(x)), host(w.model(x)), torch.float32, "second call", rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,backward", [(torch.float32, False), (torch.float16, False), (torch.float16, True)])
+def test_huggingface_bert_layer_module(dtype, backward):
+    torch.manual_seed(1)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        layer = BertLayerOutput(256, 4, 512).eval()
+        kw = dict(rtol=1e-4, atol=2e-5) if dtype == torch.float32 else {}
+        w = _compare_module(layer, torch.randn(2, 128, 256), dtype, backward, **kw)
+    kinds = {l.kind for l in w.compiled.launches}
+    if dtype == torch.float16:
+        assert "attention" in kinds and w.optimization_stats["attention"] == 1
+        if backward:
+            assert "attention_backward" in kinds and w.optimization_stats["grouped_einsums"] > 0
+
+
+@pytest.mark.gpu
+def test_mbconv_module():
+    torch.manual_seed(2)
+    w = _compare_module(MBConv(), torch.randn(3, 8, 32, 32), torch.float32, False, rtol=1e-4, atol=1e-5)
+    assert w.optimization_stats["swish"] == 3 and w.optimization_stats["gated_conv"] == 1
+
+
+@pytest.mark.gpu
+def test_onnx_model_call_passes_its_own_weights():
+    """ONNXModel on its own (daceml/onnx/onnx_importer.py:482-560): initializers become ``weights`` that every call
+    passes; inputs positionally or by name."""
+    torch.manual_seed(3)
+    net = SmallEncoder()
+    model = ONNXModel("enc", export_onnx(net, (torch.randn(2, 4, 8), )))
+    x = torch.randn(2, 4, 8)
+    want = net(x).detach().numpy()
+    assert_close(host(model(x.cuda())), want, torch.float32, "positional", rtol=1e-4, atol=1e-5)
+    assert_close(host(model(**{model.inputs[0]: x.cuda()})), want, torch.float32, "by name", rtol=1e-4, atol=1e-5)
+    with pytest.raises(TypeError):
+        model()
