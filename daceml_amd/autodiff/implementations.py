@@ -255,6 +255,31 @@ class HipLayerNormalizationBackward(BackwardImplementation):
                                  given_grad_names={"Y": "Y_grad"})
 
 
+@autoregister_params(op="BatchNormalization", name=NAME)
+class HipBatchNormalizationBackward(BackwardImplementation):
+    """Training-mode BatchNormalization: one BatchNormalizationGrad node reading X, scale and the statistics the
+    forward node saved (CuDNNBatchNormBackward, daceml/autodiff/implementations/onnx_ops.py:1268-1510). The
+    running statistics carry no gradient."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        outs = {e.src_conn for e in state.out_edges(node)}
+        return {"saved_mean", "saved_var"} <= outs
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        g = _new(context, "BatchNormalizationGrad", forward_node.label + "_backward", epsilon=forward_node.epsilon)
+        connect_input_from_forward(forward_node, g, context, "X")
+        connect_input_from_forward(forward_node, g, context, "scale")
+        connect_output_from_forward(forward_node, g, context, "saved_mean")
+        connect_output_from_forward(forward_node, g, context, "saved_var")
+        req = {"X": "dX", "scale": "dscale", "B": "dB"}
+        for c in required_gradients:
+            if c in req:
+                g.add_out_connector(req[c])
+        return g, BackwardResult(required_grad_names={c: req[c] for c in required_gradients if c in req},
+                                 given_grad_names={"Y": "dY"})
+
+
 # ----------------------------------------------------------------------------- elementwise
 def _make_unary_backward(op: str, grad_op: str, in_conn: str, out_conn: str):
     class _B(BackwardImplementation):

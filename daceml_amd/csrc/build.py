@@ -25,6 +25,7 @@ SOURCES = [
     "gemm_f32.hip",
     "conv.hip",
     "attention.hip",
+    "batchnorm.hip",
 ]
 
 # -packed-fp32-ops: keep the compiler from forming packed-fp32 VALU instructions.

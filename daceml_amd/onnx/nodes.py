@@ -115,6 +115,10 @@ SCHEMAS = [
     _schema("Conv", "X W B?", "Y", auto_pad="NOTSET", dilations=None, group=1, kernel_shape=None, pads=None,
             strides=None),
     _schema("GlobalAveragePool", "X", "Y"),
+    # "mean" / "var" name both inputs and outputs in ONNX; the connectors carry the in_ / out_ prefixes of the
+    # reference (tests/test_shared_input_output.py)
+    _schema("BatchNormalization", "X scale B in_mean in_var", "Y out_mean? out_var? saved_mean? saved_var?",
+            since=9, epsilon=1e-5, momentum=0.9),
     # fused nodes (not in opset 12)
     _schema("LayerNormalization", "X Scale B?", "Y Mean? InvStdDev?", since=17, axis=-1, epsilon=1e-5),
     _schema("SkipLayerNormalization", "input skip gamma beta?", "output mean? inv_std_var? input_skip_bias_sum?",
@@ -144,6 +148,7 @@ SCHEMAS = [
     # backward nodes emitted by the "hip" BackwardImplementations (names follow the ONNX Runtime
     # training contrib ops)
     _schema("SoftmaxGrad", "dY Y", "dX", since=1, axis=-1),
+    _schema("BatchNormalizationGrad", "dY X scale saved_mean saved_var", "dX? dscale? dB?", since=1, epsilon=1e-5),
     _schema("LayerNormalizationGrad", "Y_grad X scale mean inv_std_var", "X_grad scale_grad bias_grad", since=1,
             axis=-1),
     _schema("GeluGrad", "dY X", "dX", since=1),

@@ -228,6 +228,8 @@ class ONNXModel:
                 raise UnsupportedModel("Unsupported ONNX operator: '%s'" % op)
             out_shapes, out_dtypes, ins, attrs = self._infer(op, node, ins, attrs)
 
+        if op == "BatchNormalization":
+            attrs = {k: v for k, v in attrs.items() if k in ("epsilon", "momentum")}   # drops opset-7 `spatial`
         label = clean_onnx_name(node.name) if node.name else "%s_%d" % (op, idx)
         cls = donnx.get_onnx_node(op)
         op_node = cls(label, **attrs)
@@ -391,8 +393,12 @@ class ONNXModel:
             return [(x[0], w[0]) + tuple(out)], [dt], ins, attrs
         if op == "GlobalAveragePool":
             return [tuple(shp[0][:2]) + (1, ) * (len(shp[0]) - 2)], [dt], ins, attrs
-        if op in ("LayerNormalization", "BatchNormalization"):
+        if op == "LayerNormalization":
             return [shp[0]], [dt], ins, attrs
+        if op == "BatchNormalization":
+            # Y, then out_mean, out_var, saved_mean, saved_var when the node is in its training form
+            n_out = 5 if len([o for o in node.output if o]) > 1 else 1
+            return [shp[0]] + [(shp[0][1], )] * (n_out - 1), [dt] * n_out, ins, attrs
         raise UnsupportedModel("no shape rule for ONNX operator '%s' (node %r)" % (op, node.name))
 
     # ------------------------------------------------------------------ execution

@@ -773,6 +773,95 @@ class HipReshape(ONNXForward):
         return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="elementwise")
 
 
+# ----------------------------------------------------------------------------- batch normalisation
+def _bn_ok(x, *vectors) -> bool:
+    if len(x.shape) < 2 or not (_float_ok(x) and _dense(x)):
+        return False
+    return all(v.dtype == x.dtype and v.is_contiguous() and v.total_size == x.shape[1] for v in vectors)
+
+
+def _bn_dims(x):
+    n, c = x.shape[0], x.shape[1]
+    return n, c, x.total_size // max(n * c, 1)
+
+
+@op_implementation(op="BatchNormalization", name=IMPL)
+class HipBatchNormalization(ONNXForward):
+    """Inference (only Y connected) and training (all five outputs connected) forms of PureBatchNormalization
+    (img_op_implementations.py:333-412; cuDNN variant cudnn_implementations.py:444-649): biased batch variance,
+    running statistics updated as ``in * momentum + saved * (1 - momentum)``. As in the reference (:392-410) the
+    updated running statistics are also written back to the arrays they came from, when those are caller-owned
+    buffers."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, y = ins["X"], outs["Y"]
+            stats = [outs.get(k) for k in ("out_mean", "out_var", "saved_mean", "saved_var")]
+            if any(s is None for s in stats) and any(s is not None for s in stats):
+                return False
+            return (_dense(y) and y.shape == x.shape and y.dtype == x.dtype and node.epsilon >= 0
+                    and _bn_ok(x, ins["scale"], ins["B"], ins["in_mean"], ins["in_var"], *[s for s in stats if s]))
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "X")
+        n, c, hw = _bn_dims(x)
+        sfx = _SFX[x.dtype]
+        training = "saved_mean" in {e.src_conn for e in state.out_edges(node)}
+        if not training:
+            call = HipCall("dmlhip_batchnorm_inference_" + sfx,
+                           [Ptr("X"), Ptr("scale"), Ptr("B"), Ptr("in_mean"), Ptr("in_var"), Ptr("Y"), I64(n), I64(c),
+                            I64(hw), F32(node.epsilon), Stream()])
+            return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="batchnorm")
+        ws = L.load().dmlhip_batchnorm_workspace_bytes(n, c, hw)
+        calls = [HipCall("dmlhip_batchnorm_training_" + sfx,
+                         [Ptr("X"), Ptr("scale"), Ptr("B"), Ptr("in_mean"), Ptr("in_var"), Ptr("Y"), Ptr("out_mean"),
+                          Ptr("out_var"), Ptr("saved_mean"), Ptr("saved_var"), I64(n), I64(c), I64(hw),
+                          F32(node.epsilon), F32(node.momentum), Workspace(), WorkspaceBytes(), Stream()])]
+        for src, dst in (("out_mean", "in_mean"), ("out_var", "in_var")):
+            arr = next(iter(state.in_edges_by_connector(node, dst))).data.data
+            if not sdfg.arrays[arr].transient and arr not in sdfg.constants:
+                calls.append(HipCall("dmlhip_unary_" + sfx, [I32(L.IDENTITY), Ptr(src), Ptr(dst), I64(c), F32(0.0),
+                                                             Stream()]))
+        return _tasklet(node, state, calls, workspace_bytes=ws, bytes_moved=3 * _nbytes(x), kind="batchnorm")
+
+
+@op_implementation(op="BatchNormalizationGrad", name=IMPL)
+class HipBatchNormalizationGrad(ONNXForward):
+    """Backward of training-mode BatchNormalization (CuDNNBatchNormBackward,
+    autodiff/implementations/onnx_ops.py:1268-1510): dX in the tensor type, dscale / dB in fp32."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, dy = ins["X"], ins["dY"]
+            if not (_bn_ok(x, ins["scale"], ins["saved_mean"], ins["saved_var"]) and _dense(dy)
+                    and dy.shape == x.shape and dy.dtype == x.dtype and outs):
+                return False
+            dx = outs.get("dX")
+            if dx is not None and not (_dense(dx) and dx.shape == x.shape and dx.dtype == x.dtype):
+                return False
+            return all(d is None or (d.dtype == torch.float32 and d.is_contiguous() and d.total_size == x.shape[1])
+                       for d in (outs.get("dscale"), outs.get("dB")))
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "X")
+        n, c, hw = _bn_dims(x)
+        ws = L.load().dmlhip_batchnorm_workspace_bytes(n, c, hw)
+        call = HipCall("dmlhip_batchnorm_backward_" + _SFX[x.dtype],
+                       [Ptr("dY"), Ptr("X"), Ptr("scale"), Ptr("saved_mean"), Ptr("saved_var"),
+                        _opt(node, state, "dX", False), _opt(node, state, "dscale", False),
+                        _opt(node, state, "dB", False), I64(n), I64(c), I64(hw), F32(node.epsilon), Workspace(),
+                        WorkspaceBytes(), Stream()])
+        return _tasklet(node, state, [call], workspace_bytes=ws, bytes_moved=5 * _nbytes(x), kind="batchnorm_backward")
+
+
 # ----------------------------------------------------------------------------- convolution
 def _conv_struct(node, x: Array, w: Array, act=L.ACT_NONE) -> Optional[L.Conv2dDesc]:
     """Attribute handling of CudnnConvolution (cudnn_implementations.py:148-275): 2-D, symmetric pads,

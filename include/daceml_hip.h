@@ -292,6 +292,42 @@ int dmlhip_attention_backward_f16(const dmlhip_attention_desc* d,
                                   const void* d_o, void* dq, void* dk, void* dv,
                                   void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- BatchNormalization (NCHW) ------------------------------------------------------------------
+ * Replaces PureBatchNormalization (daceml/onnx/op_implementations/img_op_implementations.py:333-412) and
+ * CudnnBatchNormalizationTraining (daceml/onnx/op_implementations/cudnn_implementations.py:444-649);
+ * backward replaces CuDNNBatchNormBackward (daceml/autodiff/implementations/onnx_ops.py:1268-1510).
+ * x, y: [n, c, hw] dense; scale, bias and every statistic: [c] in the tensor's element type.
+ * inference: y = (x - mean) / sqrt(var + eps) * scale + bias with the given statistics.
+ * training:  saved_mean / saved_var = batch mean and biased batch variance per channel; y from those;
+ *            out_mean = in_mean * momentum + saved_mean * (1 - momentum), likewise out_var (ONNX convention:
+ *            `momentum` weighs the running value). out_* may alias in_*.
+ * backward:  dx (tensor type, may be NULL), dscale / dbias (fp32, overwritten, may be NULL) from dy, x and the
+ *            statistics saved by the training call.
+ * training and backward need a workspace of dmlhip_batchnorm_workspace_bytes(n, c, hw) bytes. */
+size_t dmlhip_batchnorm_workspace_bytes(int64_t n, int64_t c, int64_t hw);
+int dmlhip_batchnorm_inference_f16(const void* x, const void* scale, const void* bias, const void* mean,
+                                   const void* var, void* y, int64_t n, int64_t c, int64_t hw, float eps,
+                                   void* stream);
+int dmlhip_batchnorm_inference_f32(const void* x, const void* scale, const void* bias, const void* mean,
+                                   const void* var, void* y, int64_t n, int64_t c, int64_t hw, float eps,
+                                   void* stream);
+int dmlhip_batchnorm_training_f16(const void* x, const void* scale, const void* bias, const void* in_mean,
+                                  const void* in_var, void* y, void* out_mean, void* out_var, void* saved_mean,
+                                  void* saved_var, int64_t n, int64_t c, int64_t hw, float eps, float momentum,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+int dmlhip_batchnorm_training_f32(const void* x, const void* scale, const void* bias, const void* in_mean,
+                                  const void* in_var, void* y, void* out_mean, void* out_var, void* saved_mean,
+                                  void* saved_var, int64_t n, int64_t c, int64_t hw, float eps, float momentum,
+                                  void* workspace, size_t workspace_bytes, void* stream);
+int dmlhip_batchnorm_backward_f16(const void* dy, const void* x, const void* scale, const void* saved_mean,
+                                  const void* saved_var, void* dx, float* dscale, float* dbias, int64_t n,
+                                  int64_t c, int64_t hw, float eps, void* workspace, size_t workspace_bytes,
+                                  void* stream);
+int dmlhip_batchnorm_backward_f32(const void* dy, const void* x, const void* scale, const void* saved_mean,
+                                  const void* saved_var, void* dx, float* dscale, float* dbias, int64_t n,
+                                  int64_t c, int64_t hw, float eps, void* workspace, size_t workspace_bytes,
+                                  void* stream);
+
 #ifdef __cplusplus
 }
 #endif

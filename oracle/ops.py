@@ -240,6 +240,50 @@ def layernorm_backward(dy, x, gamma, eps=1e-5):
     return dx, dgamma, dbeta
 
 
+def batchnorm_training(X, scale, B, in_mean, in_var, epsilon=1e-5, momentum=0.9):
+    """PureBatchNormalization, training form: img_op_implementations.py:369-390, statement by statement.
+    Returns (Y, out_mean, out_var, saved_mean, saved_var); the variance is the biased one and ``momentum``
+    weighs the running value."""
+    axis = tuple(i for i in range(X.ndim) if i != 1)
+    N = 1
+    for i in axis:
+        N *= X.shape[i]
+    bshape = [X.shape[1]] + [1] * (X.ndim - 2)
+    saved_mean = np.add.reduce(X, axis=axis) / N
+    X_minus_mean = X - saved_mean.reshape(bshape)
+    saved_var = np.add.reduce(X_minus_mean * X_minus_mean, axis=axis) / N
+    saved_var_eps = np.reshape(saved_var + epsilon, bshape)
+    normalized = X_minus_mean * (1.0 / np.sqrt(saved_var_eps))
+    Y = normalized * np.reshape(scale, bshape) + np.reshape(B, bshape)
+    out_mean = in_mean * momentum + saved_mean * (1 - momentum)
+    out_var = in_var * momentum + saved_var * (1 - momentum)
+    return Y, out_mean, out_var, saved_mean, saved_var
+
+
+def batchnorm_inference(X, scale, B, mean, var, epsilon=1e-5):
+    """BatchNormalization with only Y connected (ONNX inference form; what tests/test_shared_input_output.py:19-43
+    compares with ``F.batch_norm(X, mean, var, scale, B)``)."""
+    bshape = [X.shape[1]] + [1] * (X.ndim - 2)
+    return (X - np.reshape(mean, bshape)) / np.sqrt(np.reshape(var, bshape) + epsilon) * np.reshape(scale, bshape) \
+        + np.reshape(B, bshape)
+
+
+def batchnorm_backward(dY, X, scale, saved_mean, saved_var, epsilon=1e-5):
+    """What cudnnBatchNormalizationBackwardEx returns for CuDNNBatchNormBackward
+    (autodiff/implementations/onnx_ops.py:1397-1440): (dX, dscale, dB) of the training-form forward."""
+    axis = tuple(i for i in range(X.ndim) if i != 1)
+    N = 1
+    for i in axis:
+        N *= X.shape[i]
+    bshape = [X.shape[1]] + [1] * (X.ndim - 2)
+    invstd = 1.0 / np.sqrt(saved_var + epsilon)
+    xhat = (X - saved_mean.reshape(bshape)) * invstd.reshape(bshape)
+    dB = np.add.reduce(dY, axis=axis)
+    dscale = np.add.reduce(dY * xhat, axis=axis)
+    dX = (scale * invstd).reshape(bshape) / N * (N * dY - dB.reshape(bshape) - xhat * dscale.reshape(bshape))
+    return dX, dscale, dB
+
+
 def gelu_chain(x):
     """GELU as exported at opset 12: Div(x, sqrt 2), Erf, Add 1, Mul x, Mul 0.5
     (pure_implementations.py:91-93,106-108,76-78,86-88). Exact erf, not the tanh form."""

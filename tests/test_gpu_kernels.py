@@ -3,6 +3,8 @@
 fp32 paths: rtol 1e-5 / atol 1e-6. fp16 paths (fp32 accumulation): rtol 2e-2 / atol 1e-2 against the
 oracle evaluated in fp64 on the fp16-rounded inputs. All calls go through the C ABI (ctypes).
 """
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -124,6 +126,90 @@ def test_layernorm_backward(dtype, shape):
     # column sums over `rows` terms: fp32 accumulation error grows with sqrt(rows)
     assert_close(host(dg), wdg, torch.float32, "ln dgamma", rtol=1e-4, atol=1e-5 * np.sqrt(rows))
     assert_close(host(db), wdb, torch.float32, "ln dbeta", rtol=1e-4, atol=1e-5 * np.sqrt(rows))
+
+
+# ----------------------------------------------------------------------------- batch normalisation
+# shapes: the reference's own case (tests/test_shared_input_output.py: [8, 3, 32, 32]), an MBConv expand output slice,
+# ragged spatial sizes (scalar path), a single image, 2-D input [N, C], segments longer than one chunk
+BN_SHAPES = [(8, 3, 32, 32), (4, 192, 28, 28), (5, 7, 9, 11), (1, 16, 8, 8), (64, 24), (2, 5, 96, 96)]
+
+
+def _bn_inputs(shape, dtype, seed):
+    c = shape[1]
+    x, x64 = _inputs(seed, shape, dtype)
+    x = (x * 2 + 1.5).astype(_np(dtype))          # a mean that is not small against the spread
+    vecs = [rng(seed + 1).uniform(0.5, 1.5, c), rng(seed + 2).standard_normal(c) * 0.3,
+            rng(seed + 3).standard_normal(c) * 0.5, rng(seed + 4).uniform(0.5, 2.0, c)]
+    vecs = [v.astype(_np(dtype)) for v in vecs]
+    return x, x.astype(np.float64), vecs, [v.astype(np.float64) for v in vecs]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", BN_SHAPES)
+def test_batchnorm_inference(dtype, shape):
+    from daceml_amd import kernels as K
+    x, x64, v, v64 = _bn_inputs(shape, dtype, 300)
+    y = K.batchnorm_inference(dev(x), *[dev(t) for t in v], eps=1e-5)
+    want = O.batchnorm_inference(x64, *v64, 1e-5)
+    assert_close(host(y), want, dtype, "bn inference", rtol=None if dtype == torch.float16 else 2e-5,
+                 atol=None if dtype == torch.float16 else 2e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", BN_SHAPES)
+def test_batchnorm_training_and_backward(dtype, shape):
+    from daceml_amd import kernels as K
+    x, x64, v, v64 = _bn_inputs(shape, dtype, 310)
+    y, om, ov, sm, sv = K.batchnorm_training(dev(x), *[dev(t) for t in v], eps=1e-5, momentum=0.9)
+    wy, wom, wov, wsm, wsv = O.batchnorm_training(x64, *v64, 1e-5, 0.9)
+    f32 = dtype != torch.float16
+    kw = dict(rtol=1e-4, atol=1e-5) if f32 else {}
+    assert_close(host(y), wy, dtype, "bn y", **kw)
+    for got, want, what in ((om, wom, "out_mean"), (ov, wov, "out_var"), (sm, wsm, "saved_mean"), (sv, wsv, "saved_var")):
+        assert got.dtype == dtype and tuple(got.shape) == (shape[1], )
+        assert_close(host(got), want, dtype, what, **kw)
+    dy, dy64 = _inputs(320, shape, dtype)
+    dx, ds, db = K.batchnorm_backward(dev(dy), dev(x), dev(v[0]), sm, sv, eps=1e-5)
+    # the oracle differentiates at the statistics the kernel saved (rounded to the tensor type for fp16)
+    wdx, wds, wdb = O.batchnorm_backward(dy64, x64, v64[0], host(sm).astype(np.float64), host(sv).astype(np.float64),
+                                         1e-5)
+    assert ds.dtype == torch.float32 and db.dtype == torch.float32
+    cnt = x.size // shape[1]
+    assert_close(host(dx), wdx, dtype, "bn dx", **kw)
+    assert_close(host(ds), wds, torch.float32, "bn dscale", rtol=1e-4 if f32 else 2e-2,
+                 atol=(1e-5 if f32 else 1e-2) * np.sqrt(cnt))
+    assert_close(host(db), wdb, torch.float32, "bn dbias", rtol=1e-4 if f32 else 2e-2,
+                 atol=(1e-5 if f32 else 1e-2) * np.sqrt(cnt))
+
+
+def test_batchnorm_large_mean_keeps_precision():
+    """fp32, mean 1000 with unit spread: the shifted sums and the centre-then-scale output keep 1e-4 relative
+    accuracy of the variance where E[x^2] - E[x]^2 would lose every digit."""
+    from daceml_amd import kernels as K
+    shape = (16, 8, 24, 24)
+    x = (rng(330).standard_normal(shape) + 1000.0).astype(np.float32)
+    c = shape[1]
+    ones, zeros = np.ones(c, np.float32), np.zeros(c, np.float32)
+    y, _, _, sm, sv = K.batchnorm_training(dev(x), dev(ones), dev(zeros), dev(zeros), dev(ones), eps=1e-5)
+    wy, _, _, wsm, wsv = O.batchnorm_training(x.astype(np.float64), ones, zeros, zeros, ones, 1e-5, 0.9)
+    assert_close(host(sv), wsv, torch.float32, "variance", rtol=1e-4, atol=0)
+    assert_close(host(y), wy, torch.float32, "y", rtol=1e-3, atol=2e-4)   # x itself carries 6e-5 of rounding
+
+
+def test_batchnorm_argument_errors():
+    from daceml_amd import _lib as L, kernels as K
+    x = torch.zeros((2, 3, 4, 4), device="cuda")
+    v = torch.ones(3, device="cuda")
+    lib = L.load()
+    p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    assert lib.dmlhip_batchnorm_inference_f32(p(x), p(v), p(v), p(v), None, p(x), 2, 3, 16, 1e-5, None) == L.ERR_NULL
+    assert lib.dmlhip_batchnorm_training_f32(p(x), p(v), p(v), p(v), p(v), p(x), p(v), p(v), p(v), p(v), 2, 3, 16, 1e-5,
+                                             0.9, None, 0, None) == L.ERR_WORKSPACE
+    assert lib.dmlhip_batchnorm_backward_f32(p(x), p(x), p(v), p(v), p(v), None, None, None, 2, 3, 16, 1e-5, p(x), 4096,
+                                             None) == L.ERR_NULL
+    assert lib.dmlhip_batchnorm_inference_f32(p(x), p(v), p(v), p(v), p(v), p(x), 0, 3, 16, 1e-5, None) == L.ERR_SHAPE
+    with pytest.raises(ValueError):
+        K.batchnorm_inference(torch.zeros(4, device="cuda"), v, v, v, v)
 
 
 # ----------------------------------------------------------------------------- elementwise

@@ -344,3 +344,43 @@ def test_bert_layer_matches_huggingface_bertlayer():
         out = layer(torch.tensor(x))
     out = out[0] if isinstance(out, (tuple, list)) else out
     np.testing.assert_allclose(OB.forward(x, p, heads, eps=cfg.layer_norm_eps), out.numpy(), rtol=1e-9, atol=1e-11)
+
+
+def test_batchnorm_matches_torch_running_stats_and_autograd():
+    """Training form against F.batch_norm(training=True): output, saved statistics, autograd gradients; the running
+    variance through torch's own update rule (torch blends the UNBIASED variance with weight 1 - momentum_onnx;
+    the reference blends the biased one, img_op_implementations.py:373-390), so a dropped Bessel factor, a swapped
+    momentum or a missing eps each fail a check."""
+    n, c, h, w = 5, 3, 4, 6
+    x = rng(40).standard_normal((n, c, h, w)) * 2 + 3
+    scale, b = rng(41).uniform(0.5, 1.5, c), rng(42).standard_normal(c)
+    rm, rv = rng(43).standard_normal(c), rng(44).uniform(0.5, 2.0, c)
+    momentum_onnx = 0.9
+    y, om, ov, sm, sv = O.batchnorm_training(x, scale, b, rm, rv, 1e-5, momentum_onnx)
+    xt = torch.tensor(x, requires_grad=True)
+    st, bt = torch.tensor(scale, requires_grad=True), torch.tensor(b, requires_grad=True)
+    trm, trv = torch.tensor(rm), torch.tensor(rv)
+    yt = F.batch_norm(xt, trm, trv, st, bt, training=True, momentum=1 - momentum_onnx, eps=1e-5)
+    np.testing.assert_allclose(y, yt.detach().numpy(), rtol=1e-10, atol=1e-12)
+    cnt = n * h * w
+    np.testing.assert_allclose(sm, x.mean(axis=(0, 2, 3)), rtol=1e-12)
+    np.testing.assert_allclose(sv, x.var(axis=(0, 2, 3)), rtol=1e-12)            # biased (ddof = 0)
+    np.testing.assert_allclose(om, trm.numpy(), rtol=1e-12)                        # torch updated rm in place
+    unbiased = (trv.numpy() - momentum_onnx * rv) / (1 - momentum_onnx)            # invert torch's update
+    np.testing.assert_allclose(ov, momentum_onnx * rv + (1 - momentum_onnx) * unbiased * (cnt - 1) / cnt, rtol=1e-10)
+    dy = rng(45).standard_normal((n, c, h, w))
+    yt.backward(torch.tensor(dy))
+    dx, ds, db = O.batchnorm_backward(dy, x, scale, sm, sv, 1e-5)
+    np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(ds, st.grad.numpy(), rtol=1e-10)
+    np.testing.assert_allclose(db, bt.grad.numpy(), rtol=1e-10)
+    # inference form: what tests/test_shared_input_output.py:41-43 compares with
+    yi = O.batchnorm_inference(x, scale, b, rm, rv, 1e-5)
+    np.testing.assert_allclose(yi, F.batch_norm(torch.tensor(x), torch.tensor(rm), torch.tensor(rv), torch.tensor(scale),
+                                                torch.tensor(b), training=False, eps=1e-5).numpy(), rtol=1e-11)
+    # invariants: unit scale / zero shift gives zero mean and unit variance per channel; a constant channel gives B
+    y1 = O.batchnorm_training(x, np.ones(c), np.zeros(c), rm, rv, 0.0, 0.9)[0]
+    np.testing.assert_allclose(y1.mean(axis=(0, 2, 3)), 0.0, atol=1e-13)
+    np.testing.assert_allclose(y1.var(axis=(0, 2, 3)), 1.0, rtol=1e-12)
+    yc = O.batchnorm_training(np.full((2, c, 3, 3), 7.0), scale, b, rm, rv, 1e-5, 0.9)[0]
+    np.testing.assert_allclose(yc, np.broadcast_to(b.reshape(1, c, 1, 1), yc.shape), atol=1e-12)

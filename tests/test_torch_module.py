@@ -76,6 +76,18 @@ class BertLayerOutput(nn.Module):
         return out[0] if isinstance(out, (tuple, list)) else out
 
 
+class ConvBN(nn.Module):
+    """Conv -> BatchNorm -> ReLU -> Conv, the un-folded form of an EfficientNet stem."""
+    def __init__(self, track=True):
+        super().__init__()
+        self.conv = nn.Conv2d(3, 8, 3, padding=1)
+        self.bn = nn.BatchNorm2d(8, track_running_stats=track)
+        self.out = nn.Conv2d(8, 4, 1)
+
+    def forward(self, x):
+        return self.out(torch.relu(self.bn(self.conv(x))))
+
+
 def _kinds(sdfg):
     return collections.Counter(n.schema.name for st in sdfg.states() for n in st.library_nodes())
 
@@ -197,6 +209,24 @@ def test_huggingface_bert_layer_imports_to_the_fused_graph(dtype):
     assert "layer.attention.self.query.weight" in model.inputs and not model.weights
 
 
+def test_batchnorm_import_forms():
+    """eval -> inference form (Y only); training -> all five outputs, with the running statistics as graph inputs
+    under their buffer names (so that the node's write-back updates the module's buffers)."""
+    x = torch.randn(2, 3, 8, 8)
+    m = DaceModule(ConvBN().eval(), auto_optimize=False)
+    model = m._import((x, ))
+    bn = [n for n in model.state.library_nodes() if n.schema.name == "BatchNormalization"]
+    assert len(bn) == 1 and {e.src_conn for e in model.state.out_edges(bn[0])} == {"Y"}
+    assert {e.dst_conn for e in model.state.in_edges(bn[0])} == {"X", "scale", "B", "in_mean", "in_var"}
+    assert abs(bn[0].momentum - 0.9) < 1e-6 and abs(bn[0].epsilon - 1e-5) < 1e-9
+    m = DaceModule(ConvBN().train(), training=True, backward=True, auto_optimize=False)
+    model = m._import((x, ))
+    bn = [n for n in model.state.library_nodes() if n.schema.name == "BatchNormalization"]
+    assert {e.src_conn for e in model.state.out_edges(bn[0])} == {"Y", "out_mean", "out_var", "saved_mean", "saved_var"}
+    assert "bn.running_mean" in model.inputs and "bn.running_var" in model.inputs
+    assert model.sdfg.arrays["SLASHbnSLASHBatchNormalization_output_3"].shape == (8, )
+
+
 def test_module_hooks_and_decorator():
     calls = []
     m = DaceModule(SmallEncoder(), auto_optimize=False)
@@ -303,3 +333,37 @@ def test_onnx_model_call_passes_its_own_weights():
     assert_close(host(model(**{model.inputs[0]: x.cuda()})), want, torch.float32, "by name", rtol=1e-4, atol=1e-5)
     with pytest.raises(TypeError):
         model()
+
+
+@pytest.mark.gpu
+def test_batchnorm_module_training_and_eval():
+    """nn.BatchNorm2d inside a module (the reference's test_bn_in_import, tests/test_shared_input_output.py:46-68,
+    plus the backward pass and the running statistics)."""
+    torch.manual_seed(4)
+    net = ConvBN().cuda().train()
+    ref = copy.deepcopy(net).double()
+    w = DaceModule(net, training=True, backward=True)
+    x = torch.randn(6, 3, 16, 16, device="cuda")
+    xs = x.clone().requires_grad_(True)
+    xr = x.double().requires_grad_(True)
+    y, want = w(xs), ref(xr)
+    assert_close(host(y), want.detach().cpu().numpy(), torch.float32, "training forward", rtol=1e-4, atol=1e-5)
+    g = torch.randn_like(y)
+    y.backward(g)
+    want.backward(g.double())
+    assert_close(host(xs.grad), xr.grad.cpu().numpy(), torch.float32, "dx", rtol=1e-4, atol=1e-5)
+    for (n, p), (_, pr) in zip(net.named_parameters(), ref.named_parameters()):
+        scale = max(float(pr.grad.abs().max()), 1.0)
+        assert_close(host(p.grad), pr.grad.cpu().numpy(), torch.float32, "gradient of " + n, rtol=1e-4, atol=1e-5 * scale)
+    # running statistics were updated in the module's own buffers: the mean as torch does, the variance with the
+    # biased batch variance (the reference's rule) where torch uses the unbiased one
+    assert_close(host(net.bn.running_mean), ref.bn.running_mean.cpu().numpy(), torch.float32, "running mean",
+                 rtol=1e-4, atol=1e-6)
+    cnt = 6 * 16 * 16
+    unbiased = (ref.bn.running_var.cpu().numpy() - 0.9) / 0.1
+    assert_close(host(net.bn.running_var), 0.9 + 0.1 * unbiased * (cnt - 1) / cnt, torch.float32, "running var",
+                 rtol=1e-4, atol=1e-6)
+    # evaluation mode: the inference form with those statistics
+    net_eval = copy.deepcopy(net).eval()
+    we = DaceModule(copy.deepcopy(net_eval))
+    assert_close(host(we(x)), host(net_eval(x)), torch.float32, "eval forward", rtol=1e-4, atol=1e-5)
