@@ -384,8 +384,9 @@ struct GemmGroup {
     int count;
     const void* const* a;
     const void* const* b;
-    void* const* c;
-    const void* const* bias;
+    void* const* c;            // unused with ksum
+    const void* const* bias;   // unused with ksum
+    bool ksum;                 // concatenate the groups along K into one output instead of running them side by side
 };
 
 // grp != nullptr: a / b / c / bias are those of group 0 (used for the layout checks, which the caller has made sure
@@ -417,14 +418,17 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
 
     GemmArgs g;
     g.groups = 0;
+    g.ksum = 0;
     if (grp) {
         g.groups = grp->count;
-        batch *= grp->count;
-        for (int i = 0; i < grp->count; ++i) {
-            g.ga[i] = (const _Float16*)grp->a[i];
-            g.gb[i] = (const _Float16*)grp->b[i];
-            g.gc[i] = grp->c[i];
-            g.gbias[i] = grp->bias ? grp->bias[i] : nullptr;
+        g.ksum = grp->ksum;
+        if (!grp->ksum) batch *= grp->count;
+        for (int i = 0; i < DMLHIP_GROUP_MAX; ++i) {
+            const bool on = i < grp->count;
+            g.ga[i] = on ? (const _Float16*)grp->a[i] : nullptr;
+            g.gb[i] = on ? (const _Float16*)grp->b[i] : nullptr;
+            g.gc[i] = on && !grp->ksum ? grp->c[i] : nullptr;
+            g.gbias[i] = on && !grp->ksum && grp->bias ? grp->bias[i] : nullptr;
         }
     }
     g.m = (int)d->m; g.n = (int)d->n; g.k = (int)d->k;
@@ -572,7 +576,7 @@ int dmlhip_gemm_f16_grouped(const dmlhip_gemm_desc* d, int groups, const void* c
     if (same && groups > 1) {
         dmlhip_gemm_desc p = *d;
         p.a_stride_batch[0] = p.b_stride_batch[0] = p.c_stride_batch[0] = 0;   // the outer batch index selects the group
-        GemmGroup grp = {groups, a, b, c, bias};
+        GemmGroup grp = {groups, a, b, c, bias, false};
         const int e = run_gemm_f16(&p, a[0], b[0], c[0], bias ? bias[0] : nullptr, nullptr, nullptr, stream, &grp);
         if (e == 0) ++g_grouped_single_launches;
         if (e != DMLHIP_ERR_UNSUPPORTED) return e;
@@ -581,6 +585,33 @@ int dmlhip_gemm_f16_grouped(const dmlhip_gemm_desc* d, int groups, const void* c
         if (int e = dmlhip_gemm_f16_ws(d, a[i], b[i], c[i], bias ? bias[i] : nullptr, nullptr, nullptr, workspace,
                                        workspace_bytes, stream))
             return e;
+    return 0;
+}
+
+int dmlhip_gemm_f16_ksum(const dmlhip_gemm_desc* d, int groups, const void* const* a, const void* const* b, void* c,
+                         const void* bias, const void* residual, void* stream) {
+    DML_REQUIRE(d, DMLHIP_ERR_NULL, "gemm_f16_ksum: NULL descriptor");
+    DML_REQUIRE(groups >= 1 && groups <= DMLHIP_GROUP_MAX, DMLHIP_ERR_SHAPE, "gemm_f16_ksum: %d groups outside 1..%d",
+                groups, DMLHIP_GROUP_MAX);
+    DML_REQUIRE(a && b && c, DMLHIP_ERR_NULL, "gemm_f16_ksum: NULL pointer");
+    DML_REQUIRE(d->beta == 0.f && d->act == DMLHIP_ACT_NONE, DMLHIP_ERR_UNSUPPORTED,
+                "gemm_f16_ksum: beta and activations are not supported");
+    for (int i = 0; i < groups; ++i) DML_REQUIRE(a[i] && b[i], DMLHIP_ERR_NULL, "gemm_f16_ksum: NULL operand %d", i);
+    bool same = d->k > 0 && groups > 1;
+    for (int i = 0; i < groups && same; ++i) same = aligned16(a[i]) && aligned16(b[i]);
+    if (same) {
+        GemmGroup grp = {groups, a, b, nullptr, nullptr, true};
+        const int e = run_gemm_f16(d, a[0], b[0], c, bias, residual, nullptr, stream, &grp);
+        if (e == 0) ++g_grouped_single_launches;
+        if (e != DMLHIP_ERR_UNSUPPORTED) return e;
+    }
+    // one product after the other, accumulating in C (rounded to C's type in between)
+    dmlhip_gemm_desc p = *d;
+    for (int i = 0; i < groups; ++i) {
+        if (int e = run_gemm_f16(&p, a[i], b[i], c, i == 0 ? bias : nullptr, i == 0 ? residual : nullptr, nullptr, stream))
+            return e;
+        p.beta = 1.f;
+    }
     return 0;
 }
 

@@ -24,8 +24,9 @@ struct GemmArgs {
     int tiles_m, tiles_n;
     long long total_blocks;
     // grouped launch: the outer batch index selects one of `groups` independent problems of identical shape and
-    // strides (0 = an ordinary launch, pointers come from the kernel parameters)
-    int groups;
+    // strides (0 = an ordinary launch, pointers come from the kernel parameters). With `ksum` the groups are instead
+    // concatenated along K: one output C = sum over groups of A_g B_g (only ga / gb are used).
+    int groups, ksum;
     const _Float16* ga[DMLHIP_GROUP_MAX];
     const _Float16* gb[DMLHIP_GROUP_MAX];
     void* gc[DMLHIP_GROUP_MAX];

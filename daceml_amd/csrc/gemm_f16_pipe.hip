@@ -125,7 +125,9 @@ __device__ unsigned* dml_gemm_trace_buf;
 #endif
 
 // ---------------------------------------------------------------- kernel
-template <int BM, int BN, int WM, int WN, int AKIND, int BKIND, int NSTAGE, int EPI>
+// KSUM: the operand pairs g.ga[i] / g.gb[i] are concatenated along K (one output, see GemmArgs::ksum). A template
+// parameter, so that the ordinary kernels keep loop-invariant operand bases.
+template <int BM, int BN, int WM, int WN, int AKIND, int BKIND, int NSTAGE, int EPI, bool KSUM = false>
 __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16* a_ptr, const _Float16* b_ptr, void* c_ptr,
                                                                  const void* bias_ptr, const void* res_ptr,
                                                                  void* pre_ptr, const GemmArgs g) {
@@ -160,14 +162,16 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     const int z2 = (int)(batch % g.batch2);
     const int z1 = (int)((batch / g.batch2) % g.batch1);
     const int z0 = (int)(batch / ((long long)g.batch2 * g.batch1));
-    if (g.groups) {  // uniform: one of several same-shaped problems (host sets the outer batch strides to 0)
+    if (!KSUM && g.groups) {  // uniform: one of several same-shaped problems (host sets the outer batch strides to 0)
         a_ptr = g.ga[z0];
         b_ptr = g.gb[z0];
         c_ptr = g.gc[z0];
         bias_ptr = g.gbias[z0];
     }
-    const _Float16* A = a_ptr + z0 * g.sab[0] + z1 * g.sab[1] + z2 * g.sab[2];
-    const _Float16* B = b_ptr + z0 * g.sbb[0] + z1 * g.sbb[1] + z2 * g.sbb[2];
+    const int64_t aoff = z0 * g.sab[0] + z1 * g.sab[1] + z2 * g.sab[2];
+    const int64_t boff = z0 * g.sbb[0] + z1 * g.sbb[1] + z2 * g.sbb[2];
+    const _Float16* A = a_ptr + aoff;
+    const _Float16* B = b_ptr + boff;
     const int64_t coff = z0 * g.scb[0] + z1 * g.scb[1] + z2 * g.scb[2];
     const int m0 = tm * BM, n0 = tn * BN;
 
@@ -191,13 +195,33 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     constexpr int READS = Stream<BM, AKIND, TM>::READS + Stream<BN, BKIND, TN>::READS;
     constexpr int READS_W = READS > 15 ? 15 : READS;  // lgkmcnt saturates at 15: waiting for one more is harmless
 
-    const int nk = g.k / BK;
+    // K steps: g.k / BK per operand pair; with ksum the pairs follow each other (the accumulators simply keep
+    // running), and the fill cursor (fa, fb, fk) walks pair by pair.
+    const int nkg = g.k / BK;
+    const int nk = KSUM ? nkg * g.groups : nkg;
+    const _Float16* fa = A;
+    const _Float16* fb = B;
+    int fk = 0, fgrp = 0;
+    auto advance = [&]() {
+        ++fk;
+        if constexpr (KSUM) {
+            if (fk == nkg && fgrp + 1 < g.groups) {
+                fk = 0;
+                ++fgrp;
+                // constant indices: the table stays in the kernel-argument segment, the choice in scalar registers
+                fa = (fgrp == 1 ? g.ga[1] : fgrp == 2 ? g.ga[2] : g.ga[3]) + aoff;
+                fb = (fgrp == 1 ? g.gb[1] : fgrp == 2 ? g.gb[2] : g.gb[3]) + boff;
+            }
+        }
+    };
+    static_assert(DMLHIP_GROUP_MAX == 4, "the operand-pair selection above lists four entries");
     // prologue: tiles 0 .. NSTAGE-2 in flight
 #pragma unroll
     for (int s = 0; s < NSTAGE - 1; ++s) {
         if (s < nk) {
-            sa.issue(A, g.sak, s * BK, lds + s * STAGE, wave);
-            sb.issue(B, g.sbk, s * BK, lds + s * STAGE + A_BYTES, wave);
+            sa.issue(KSUM ? fa : A, g.sak, (KSUM ? fk : s) * BK, lds + s * STAGE, wave);
+            sb.issue(KSUM ? fb : B, g.sbk, (KSUM ? fk : s) * BK, lds + s * STAGE + A_BYTES, wave);
+            if constexpr (KSUM) advance();
         }
     }
     DML_TR(1);
@@ -227,10 +251,14 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
         const int fill = kt + NSTAGE - 1;
         const int fs = cur_stage == 0 ? NSTAGE - 1 : cur_stage - 1;
         char* fill_tile = lds + fs * STAGE;
+        const _Float16* const fill_a = KSUM ? fa : A;
+        const _Float16* const fill_b = KSUM ? fb : B;
+        const int fill_k = (KSUM ? fk : fill) * BK;
+        if (KSUM && fill < nk) advance();
         if constexpr (!SPREAD) {
             if (fill < nk) {
-                sa.issue(A, g.sak, fill * BK, fill_tile, wave);
-                sb.issue(B, g.sbk, fill * BK, fill_tile + A_BYTES, wave);
+                sa.issue(fill_a, g.sak, fill_k, fill_tile, wave);
+                sb.issue(fill_b, g.sbk, fill_k, fill_tile + A_BYTES, wave);
             }
         }
         const bool more = kt + 1 < nk;
@@ -269,8 +297,8 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
                     constexpr int NA = BM / 32;
                     static_for<kk * LPT / 3, (kk + 1) * LPT / 3>([&](auto jc) {
                         constexpr int j = decltype(jc)::value;
-                        if constexpr (j < NA) sa.template issue_one<j>(A, g.sak, fill * BK, fill_tile, wave);
-                        else sb.template issue_one<j - NA>(B, g.sbk, fill * BK, fill_tile + A_BYTES, wave);
+                        if constexpr (j < NA) sa.template issue_one<j>(fill_a, g.sak, fill_k, fill_tile, wave);
+                        else sb.template issue_one<j - NA>(fill_b, g.sbk, fill_k, fill_tile + A_BYTES, wave);
                     });
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -302,7 +330,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
 #endif
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE>
+template <int BM, int BN, int WM, int WN, int NSTAGE, bool KSUM = false>
 int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, const void* bias, const void* res, void* pre,
                 int akind, int bkind, long long batch, hipStream_t st) {
     g.tiles_m = (g.m + BM - 1) / BM;
@@ -320,7 +348,7 @@ int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, cons
     }
 #define DML_PIPE_CASE(AK, BKD, ACTV)                                                                          \
     if (akind == AK && bkind == BKD && ek == ACTV) {                                                          \
-        auto kern = gemm_f16_pipe_kernel<BM, BN, WM, WN, AK, BKD, NSTAGE, ACTV>;                              \
+        auto kern = gemm_f16_pipe_kernel<BM, BN, WM, WN, AK, BKD, NSTAGE, ACTV, KSUM>;                        \
         if (lds > 64 * 1024) {                                                                                \
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
                                                (int)lds);                                                     \
@@ -333,7 +361,9 @@ int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, cons
         return launch_status("gemm_f16(pipelined)");                                                          \
     }
     DML_PIPE_CASE(0, 0, EPI_PLAIN) DML_PIPE_CASE(0, 1, EPI_PLAIN) DML_PIPE_CASE(1, 0, EPI_PLAIN) DML_PIPE_CASE(1, 1, EPI_PLAIN)
-    DML_PIPE_CASE(0, 0, EPI_ACT) DML_PIPE_CASE(0, 1, EPI_ACT) DML_PIPE_CASE(1, 0, EPI_ACT) DML_PIPE_CASE(1, 1, EPI_ACT)
+    if constexpr (!KSUM) {
+        DML_PIPE_CASE(0, 0, EPI_ACT) DML_PIPE_CASE(0, 1, EPI_ACT) DML_PIPE_CASE(1, 0, EPI_ACT) DML_PIPE_CASE(1, 1, EPI_ACT)
+    }
     DML_PIPE_CASE(0, 0, EPI_GENERAL) DML_PIPE_CASE(0, 1, EPI_GENERAL) DML_PIPE_CASE(1, 0, EPI_GENERAL)
     DML_PIPE_CASE(1, 1, EPI_GENERAL)
 #undef DML_PIPE_CASE
@@ -346,6 +376,10 @@ int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, cons
 int launch_pipelined(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, const void* bias, const void* residual,
                      void* pre, int amode, int bmode, int cfg, long long batch, hipStream_t st) {
     const int ak = amode == 4 ? 1 : 0, bk = bmode == 4 ? 1 : 0;
+    if (g.ksum) {  // K-concatenated operand pairs: the two 128x128 configurations only
+        if (cfg == 3) return launch_tile<128, 128, 64, 64, 2, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+        return launch_tile<128, 128, 64, 64, 4, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+    }
     switch (cfg) {
         case 2: return launch_tile<256, 256, 128, 128, 2>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
         case 1: return launch_tile<256, 128, 128, 64, 3>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);

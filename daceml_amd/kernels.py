@@ -534,6 +534,36 @@ def reduce_sum_multi(xs: Sequence[torch.Tensor], out_dtype: Optional[torch.dtype
     return ys
 
 
+def einsum_sum(equation: str, a_list: Sequence[torch.Tensor], b_list: Sequence[torch.Tensor], *,
+               out_dtype: Optional[torch.dtype] = None, alpha: float = 1.0, bias: Optional[torch.Tensor] = None,
+               residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """alpha * sum_i einsum(equation, a_i, b_i) (+ bias) (+ residual) for fp16 operand pairs of identical shapes and
+    strides (at most four), accumulated inside one launch."""
+    from . import contraction as C
+    n = len(a_list)
+    if n != len(b_list) or n < 1:
+        raise ValueError("einsum_sum: lists differ in length")
+    _check(*a_list, *b_list, bias, residual, dtype=None)
+    a0, b0 = a_list[0], b_list[0]
+    if a0.dtype != torch.float16:
+        raise TypeError("einsum_sum is implemented for fp16 operands")
+    for a, b in zip(a_list, b_list):
+        if a.shape != a0.shape or a.stride() != a0.stride() or b.shape != b0.shape or b.stride() != b0.stride() \
+                or a.dtype != a0.dtype or b.dtype != a0.dtype:
+            raise ValueError("einsum_sum: every pair needs the shapes, strides and dtype of pair 0")
+    out_dtype = out_dtype or a0.dtype
+    plan = C.plan_contraction(equation, a0.shape, a0.stride(), b0.shape, b0.stride())
+    out = torch.empty(plan.out_shape, dtype=out_dtype, device=a0.device)
+    if residual is not None and (residual.shape != out.shape or residual.dtype != out_dtype):
+        raise ValueError("einsum_sum: the residual needs the output's shape and dtype")
+    xs, ys = (b_list, a_list) if plan.swapped else (a_list, b_list)
+    desc = _fill_desc(plan, alpha, 0.0, out_dtype, bias, L.ACT_NONE)
+    arr = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])  # noqa: E731
+    L.check(L.load().dmlhip_gemm_f16_ksum(ctypes.byref(desc), n, arr(xs), arr(ys), _ptr(out), _ptr(bias),
+                                          _ptr(_dense(residual) if residual is not None else None), _stream()))
+    return out
+
+
 def einsum_grouped(equation: str, a_list: Sequence[torch.Tensor], b_list: Sequence[torch.Tensor], *,
                    out_dtype: Optional[torch.dtype] = None, alpha: float = 1.0,
                    bias_list: Optional[Sequence[torch.Tensor]] = None):

@@ -144,6 +144,7 @@ SCHEMAS = [
     _schema("GroupedEinsum", "A* B* Bias*?", "Output*", since=1, equation=REQUIRED, alpha=1.0),
     # several independent ReduceSum(all leading axes, keepdims=0) nodes in one launch pair: reduced__i = sum of
     # data__i over every axis but the last (the bias gradients of a backward pass)
+    _schema("EinsumSum", "A* B* Residual?", "Output", since=1, equation=REQUIRED, alpha=1.0),
     _schema("MultiReduceSum", "data*", "reduced*", since=1),
     # backward nodes emitted by the "hip" BackwardImplementations (names follow the ONNX Runtime
     # training contrib ops)

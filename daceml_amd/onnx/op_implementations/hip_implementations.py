@@ -1243,3 +1243,52 @@ class HipGroupedEinsum(ONNXForward):
         extra = bias or []
         return _tasklet(node, state, [call], workspace_bytes=ws, flops=plan.flops * n,
                         bytes_moved=sum(_nbytes(a[i], b[i], out[i]) for i in range(n)) + _nbytes(*extra), kind="gemm")
+
+
+@op_implementation(op="EinsumSum", name=IMPL)
+class HipEinsumSum(ONNXForward):
+    """Sum of up to four PureEinsum contractions (pure_implementations.py:219-252) of identical equation, shapes and
+    strides, optionally plus a residual of the output's shape: the ONNXSum with which autodiff accumulates gradient
+    contributions (autodiff/backward_pass_generator.py:715-752) folded into the contractions that produce them.
+    The operand pairs are concatenated along K in one launch; the accumulation stays in fp32."""
+    @staticmethod
+    def _pairs(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        n = len([k for k in ins if k.startswith("A__")])
+        return n, [ins["A__%d" % i] for i in range(n)], [ins["B__%d" % i] for i in range(n)], ins.get("Residual"), \
+            outs["Output"]
+
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            n, a, b, res, out = HipEinsumSum._pairs(node, state, sdfg)
+            if not 1 <= n <= L.GROUP_MAX or a[0].dtype != torch.float16:
+                return False
+            eq = node.equation.replace(" ", "")
+            for i in range(n):
+                if (a[i].shape, a[i].strides, a[i].dtype) != (a[0].shape, a[0].strides, a[0].dtype):
+                    return False
+                if (b[i].shape, b[i].strides, b[i].dtype) != (b[0].shape, b[0].strides, a[0].dtype):
+                    return False
+                if not _einsum_can_apply(eq, [a[i], b[i]], out, allow_f32_out=True):
+                    return False
+            if res is not None and not (res.shape == out.shape and res.dtype == out.dtype and res.strides == out.strides):
+                return False
+            return _einsum_plan(eq, a[0], b[0]) is not None
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        n, a, b, res, out = HipEinsumSum._pairs(node, state, sdfg)
+        eq = node.equation.replace(" ", "")
+        plan = C.plan_contraction(eq, a[0].shape, a[0].strides, b[0].shape, b[0].strides)
+        desc = _gemm_struct(plan, node.alpha, 0.0, out.dtype, out.dtype, L.ACT_NONE)
+        xa, xb = ("B", "A") if plan.swapped else ("A", "B")
+        call = HipCall("dmlhip_gemm_f16_ksum",
+                       [Struct(desc, "dmlhip_gemm_desc"), I32(n), PtrArray(tuple("%s__%d" % (xa, i) for i in range(n))),
+                        PtrArray(tuple("%s__%d" % (xb, i) for i in range(n))), Ptr("Output"), Null(),
+                        Ptr("Residual") if res is not None else Null(), Stream()])
+        extra = [res] if res is not None else []
+        return _tasklet(node, state, [call], flops=plan.flops * n,
+                        bytes_moved=sum(_nbytes(a[i], b[i]) for i in range(n)) + _nbytes(out, *extra), kind="gemm")

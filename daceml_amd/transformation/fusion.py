@@ -836,10 +836,103 @@ def group_einsums(sdfg: SDFG, max_group: int = 4) -> int:
     return merged
 
 
+def fuse_einsum_sums(sdfg: SDFG, max_group: int = 4) -> int:
+    """Gradient accumulation folded into the contractions that feed it. Autodiff sums the contributions of an
+    array's consumers with an ONNXSum (daceml/autodiff/backward_pass_generator.py:715-752); when contributions are
+    plain contractions of one shape (the input gradients of the Q/K/V projections) they become one EinsumSum —
+    operand pairs concatenated along K, partial products never written — and a single remaining summand rides
+    along as the residual of the epilogue. A Sum of one contraction and one other array becomes that contraction
+    with a Residual. Returns the number of Sum operands that no longer pass through memory."""
+    saved = 0
+    for state in sdfg.states():
+        for sm in [n for n in state.nodes() if _is_op(n, "Sum")]:
+            arrays = [e.data.data for e in state.in_edges(sm)]
+            out = _out_array(state, sm, "sum")
+            od = sdfg.arrays[out]
+            if od.dtype != torch.float16 or not od.is_contiguous() or len(set(arrays)) != len(arrays):
+                continue
+            viewed = {d.view_of for d in sdfg.arrays.values() if d.view_of is not None}
+            buckets, producer_of = {}, {}
+            for arr in arrays:
+                prod = _producer(state, arr)
+                d = sdfg.arrays[arr]
+                if prod is None or not _is_op(prod[0], "FusedEinsum") or not _internal(sdfg, state, arr) or arr in viewed \
+                        or (d.shape, d.strides, d.dtype) != (od.shape, od.strides, od.dtype):
+                    continue
+                n = prod[0]
+                conns = {e.dst_conn for e in state.in_edges(n)} | {e.src_conn for e in state.out_edges(n)}
+                if conns != {"Inputs__0", "Inputs__1", "Output"} or n.activation != "none" or n.accumulate:
+                    continue
+                a = sdfg.arrays[_in_array(state, n, "Inputs__0")]
+                b = sdfg.arrays[_in_array(state, n, "Inputs__1")]
+                if a.dtype != torch.float16 or b.dtype != torch.float16:
+                    continue
+                key = (n.equation.replace(" ", ""), float(n.alpha), tuple(a.shape), tuple(a.strides), tuple(b.shape),
+                       tuple(b.strides))
+                buckets.setdefault(key, []).append(arr)
+                producer_of[arr] = n
+            if not buckets:
+                continue
+            key, grp = max(buckets.items(), key=lambda kv: len(kv[1]))
+            grp = sorted(grp, key=lambda arr: producer_of[arr].label)[:max_group]
+            others = [arr for arr in arrays if arr not in grp]
+            residual = others[0] if len(others) == 1 else None
+            if residual is not None:
+                rd = sdfg.arrays[residual]
+                if (rd.shape, rd.strides, rd.dtype) != (od.shape, od.strides, od.dtype):
+                    residual = None
+            if len(grp) == 1:
+                if residual is None:
+                    continue
+                # the contraction writes the sum itself
+                n = producer_of[grp[0]]
+                ins = {"Inputs__0": _in_array(state, n, "Inputs__0"), "Inputs__1": _in_array(state, n, "Inputs__1"),
+                       "Residual": residual}
+                attrs = dict(equation=n.equation, alpha=n.alpha, activation="none", accumulate=0)
+                label = n.label
+                _remove_node(state, sm)
+                _remove_node(state, n)
+                _add_node(sdfg, state, "FusedEinsum", label, ins, {"Output": out}, **attrs)
+                saved += 2
+                continue
+            try:
+                C.plan_contraction(key[0], key[2], key[3], key[4], key[5])
+            except (C.NotApplicable, ValueError):
+                continue
+            ins = {}
+            for i, arr in enumerate(grp):
+                n = producer_of[arr]
+                ins["A__%d" % i] = _in_array(state, n, "Inputs__0")
+                ins["B__%d" % i] = _in_array(state, n, "Inputs__1")
+            label = "sum_" + "_".join(producer_of[arr].label.replace("_matmul_fused", "") for arr in grp)
+            sum_label = sm.label
+            rest = [arr for arr in others if arr != residual] if residual is not None else others
+            _remove_node(state, sm)
+            for arr in grp:
+                _remove_node(state, producer_of[arr])
+            if residual is not None:
+                ins["Residual"] = residual
+            if rest:
+                target, _ = sdfg.add_transient(label + "_out", od.shape, od.dtype)
+            else:
+                target = out
+            _add_node(sdfg, state, "EinsumSum", label, ins, {"Output": target}, equation=key[0], alpha=key[1])
+            if rest:
+                _add_node(sdfg, state, "Sum", sum_label, {"data_0__%d" % i: arr for i, arr in enumerate([target] + rest)},
+                          {"sum": out})
+            saved += len(grp) + (1 if residual is not None else 0) - (1 if rest else 0)
+    if saved:
+        _drop_unused_arrays(sdfg)
+    return saved
+
+
 def optimize_backward(sdfg: SDFG) -> Dict[str, int]:
     """Rewrites for the state(s) autodiff added — what a ``post_autodiff_hooks`` entry of the reference's module
     wrapper would run (daceml/torch/module.py:46-365)."""
-    return {"reductions": fuse_reductions(sdfg), "grouped_einsums": group_einsums(sdfg)}
+    stats = {"reductions": fuse_reductions(sdfg)}
+    stats["einsum_sums"] = fuse_einsum_sums(sdfg)      # before grouping: a summed group needs no separate outputs
+    stats["grouped_einsums"] = group_einsums(sdfg)
+    return stats
 
 
 def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True,

@@ -225,6 +225,14 @@ int dmlhip_gemm_f16_ws(const dmlhip_gemm_desc* desc, const void* a, const void* 
 int dmlhip_gemm_f16_grouped(const dmlhip_gemm_desc* d, int groups, const void* const* a,
                             const void* const* b, void* const* c, const void* const* bias,
                             void* workspace, size_t workspace_bytes, void* stream);
+/* c = alpha * sum_i a[i] b[i] (+ column bias) (+ residual): `groups` products of identical shape and strides that
+ * are summed — the operand pairs are concatenated along K inside one launch, so the partial products never reach
+ * memory. This is what autodiff's gradient accumulation (an ONNXSum over the contributions of several consumers,
+ * daceml/autodiff/backward_pass_generator.py:715-752) amounts to when the contributions are contractions, e.g. the
+ * input gradient of the Q/K/V projections. d->beta must be 0 and d->act NONE. Falls back to `groups` accumulating
+ * calls of dmlhip_gemm_f16 when one launch is not possible. */
+int dmlhip_gemm_f16_ksum(const dmlhip_gemm_desc* d, int groups, const void* const* a, const void* const* b,
+                         void* c, const void* bias, const void* residual, void* stream);
 int dmlhip_gemm_f32(const dmlhip_gemm_desc* desc, const void* a, const void* b, void* c,
                     const void* bias, const void* residual, void* pre_out, void* stream);
 

@@ -78,11 +78,11 @@ def test_bert_layer_backward(dtype, attention):
     # the backward state contains only nodes with hand-written kernels
     bnames = {n.schema.name for n in sdfg.states()[1].library_nodes()}
     if attention:
-        assert bnames == {"FusedEinsum", "GroupedEinsum", "FusedAttentionGrad", "LayerNormalizationGrad", "GeluGrad",
-                          "MultiReduceSum", "Sum"}
+        assert bnames == {"FusedEinsum", "GroupedEinsum", "EinsumSum", "FusedAttentionGrad", "LayerNormalizationGrad",
+                          "GeluGrad", "MultiReduceSum"}
     else:
         assert bnames == {"FusedEinsum", "SoftmaxGrad", "LayerNormalizationGrad", "GeluGrad", "ReduceSum", "Sum"}
-    n_grouped = sum(n.schema.name == "GroupedEinsum" for st in sdfg.states() for n in st.library_nodes())
+    n_grouped = sum(n.schema.name in ("GroupedEinsum", "EinsumSum") for st in sdfg.states() for n in st.library_nodes())
     prog = _compile(sdfg)   # expands the library nodes in place
     args = {"x": dev(x), "y": torch.empty((b, s, h), dtype=dtype, device="cuda"), "gradient_y": dev(dy)}
     args.update({k: dev(v) for k, v in p.items()})
@@ -94,8 +94,8 @@ def test_bert_layer_backward(dtype, attention):
     before = single()
     prog(**args, **out)
     if attention:
-        # q/k/v projections, their input gradients and the o/q/k/v weight gradients: one launch each, also for
-        # the two backward groups, which carry no bias table
+        # q/k/v projections, the sum of their input gradients and the o/q/k/v weight gradients: one launch each, also
+        # for the two backward nodes, which carry no bias table
         assert n_grouped == 3 and single() - before == 3
     x64 = x.astype(np.float64)
     p64 = {k: v.astype(np.float64) for k, v in p.items()}

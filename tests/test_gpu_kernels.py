@@ -598,6 +598,38 @@ def test_reduce_sum_multi(dtype):
     ("ik,kj->ij", (100, 72), (72, 50), True, torch.float16),             # K % 64 != 0: falls back to separate launches
 ])
 def test_einsum_grouped(eq, sa, sb, with_bias, out_dtype):
+    _einsum_grouped_case(eq, sa, sb, with_bias, out_dtype)
+
+
+@pytest.mark.parametrize("eq,sa,sb,n,with_res,out_dtype,single", [
+    ("aij,jk->aik", (2, 256, 128), (128, 192), 3, True, torch.float16, True),    # q/k/v input gradients + residual path
+    ("aij,jk->aik", (2, 256, 128), (128, 192), 2, False, torch.float16, True),
+    ("aik,jk->aij", (2, 128, 256), (128, 256), 4, True, torch.float16, True),    # four stages deep, K-contiguous operands
+    ("aij,aik->jk", (2, 256, 128), (2, 256, 64), 3, False, torch.float32, True),
+    ("ik,kj->ij", (100, 72), (72, 50), 3, True, torch.float16, False),           # K % 64 != 0: accumulating launches
+    ("aij,jk->aik", (2, 256, 128), (128, 192), 1, True, torch.float16, False),   # a single pair
+])
+def test_einsum_sum(eq, sa, sb, n, with_res, out_dtype, single):
+    """sum_i einsum(a_i, b_i) (+ residual): the operand pairs are concatenated along K in one launch."""
+    from daceml_amd import _lib as L, kernels as K
+    a = [_inputs(400 + i, sa, torch.float16) for i in range(n)]
+    b = [_inputs(410 + i, sb, torch.float16, 0.2) for i in range(n)]
+    want = sum(O.einsum(eq, a[i][1], b[i][1]) for i in range(n))
+    res = None
+    if with_res:
+        r, r64 = _inputs(420, want.shape, torch.float16)
+        res = dev(r).to(out_dtype)
+        want = want + r64
+    count = L.load().dmlhip_debug_grouped_single_launches
+    before = count()
+    got = K.einsum_sum(eq, [dev(x) for x, _ in a], [dev(x) for x, _ in b], out_dtype=out_dtype, residual=res)
+    assert count() - before == (1 if single else 0)
+    assert got.dtype == out_dtype
+    k_total = n * (sa[-1] if eq.startswith("aik") or eq.startswith("ik") else sa[-2] if eq.startswith("aij,jk") else sa[0] * sa[1])
+    assert_close(host(got), want, torch.float16, "einsum sum %s x%d" % (eq, n), atol=1e-2 * max(1.0, np.sqrt(k_total / 256)))
+
+
+def _einsum_grouped_case(eq, sa, sb, with_bias, out_dtype):
     from daceml_amd import contraction as C, kernels as K
     n = 3
     plan_n = C.plan_contraction(eq, sa, C.contiguous_strides(sa), sb, C.contiguous_strides(sb)).out_shape[-1]

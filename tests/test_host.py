@@ -315,6 +315,10 @@ def test_fusion_pipeline_on_bert_layer():
                for e in st.in_edges(after["q_matmul_fused"]))           # weight used as stored, no Transpose
 
 
+def _out(state, node, conn):
+    return next(iter(state.out_edges_by_connector(node, conn))).data.data
+
+
 def test_attention_fusion_roles_and_graph():
     from daceml_amd import graphs
     from daceml_amd.autodiff import add_backward_pass
@@ -351,12 +355,17 @@ def test_attention_fusion_roles_and_graph():
     assert ins == {"Q", "K", "V", "O", "LogSumExp", "dO"}
     # the six bias gradients become one node; nothing else in the state changes
     n_before = len(sdfg.states()[1].library_nodes())
-    assert fusion.optimize_backward(sdfg) == {"reductions": 5, "grouped_einsums": 7}
+    assert fusion.optimize_backward(sdfg) == {"reductions": 5, "einsum_sums": 6, "grouped_einsums": 5}
     bnodes = sdfg.states()[1].library_nodes()
-    # five reductions and five contractions fewer (q/k/v input gradients: 3 -> 1; o/q/k/v weight gradients: 4 -> 1)
-    assert len(bnodes) == n_before - 10 and not any(n.schema.name == "ReduceSum" for n in bnodes)
+    # five reductions, two gradient sums and five contractions fewer (q/k/v input gradients: 3 -> 1 EinsumSum that also
+    # adds the residual path; o/q/k/v weight gradients: 4 -> 1; the other Sum rides on a contraction as its Residual)
+    assert len(bnodes) == n_before - 12 and not any(n.schema.name in ("ReduceSum", "Sum") for n in bnodes)
+    es = [n for n in bnodes if n.schema.name == "EinsumSum"]
+    assert len(es) == 1 and es[0].label == "sum_k_grad_0_q_grad_0_v_grad_0"
+    assert _out(sdfg.states()[1], es[0], "Output") == "gradient_x"
+    assert {e.dst_conn for e in sdfg.states()[1].in_edges(es[0])} == {"A__0", "B__0", "A__1", "B__1", "A__2", "B__2", "Residual"}
     grouped = sorted(n.label for st_ in sdfg.states() for n in st_.library_nodes() if n.schema.name == "GroupedEinsum")
-    assert grouped == ["grouped_k_grad_0_q_grad_0_v_grad_0", "grouped_k_grad_1_o_grad_1_q_grad_1_v_grad_1", "grouped_k_q_v"]
+    assert grouped == ["grouped_k_grad_1_o_grad_1_q_grad_1_v_grad_1", "grouped_k_q_v"]
     # grouping respects data dependences, also through views: o's input gradient feeds the attention backward
     # whose outputs the q/k/v gradients read, so it stays on its own; the states still sort topologically
     assert any(n.label == "o_matmul_fused_grad_0" for n in bnodes)
