@@ -99,6 +99,9 @@ SIGNATURES = {
     "dmlhip_gemm_f16_ws": (c_int, [POINTER(GemmDesc), _P, _P, _P, _P, _P, _P, _P, c_size_t, _P]),
     "dmlhip_gemm_f16_grouped": (c_int, [POINTER(GemmDesc), c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                         POINTER(c_void_p), _P, c_size_t, _P]),
+    "dmlhip_gemm_f16_grouped_asum_workspace_bytes": (c_size_t, [POINTER(GemmDesc)]),
+    "dmlhip_gemm_f16_grouped_asum": (c_int, [POINTER(GemmDesc), c_int, POINTER(c_void_p), POINTER(c_void_p),
+                                             POINTER(c_void_p), POINTER(c_void_p), c_int, _P, c_size_t, _P]),
     "dmlhip_gemm_f16_ksum": (c_int, [POINTER(GemmDesc), c_int, POINTER(c_void_p), POINTER(c_void_p), _P, _P, _P, _P]),
     "dmlhip_gemm_f32": (c_int, [POINTER(GemmDesc), _P, _P, _P, _P, _P, _P, _P]),
     "dmlhip_conv2d_out_shape": (c_int, [POINTER(Conv2dDesc), _I64P, _I64P]),

@@ -392,7 +392,8 @@ struct GemmGroup {
 // grp != nullptr: a / b / c / bias are those of group 0 (used for the layout checks, which the caller has made sure
 // hold for every group); returns DMLHIP_ERR_UNSUPPORTED when the grouped launch is not possible.
 static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b, void* c, const void* bias,
-                        const void* residual, void* pre_out, void* stream, const GemmGroup* grp = nullptr) {
+                        const void* residual, void* pre_out, void* stream, const GemmGroup* grp = nullptr,
+                        void* const* asum = nullptr, int asum_f32 = 0) {
     DML_REQUIRE(d, DMLHIP_ERR_NULL, "gemm_f16: NULL descriptor");
     DML_REQUIRE(d->m >= 0 && d->n >= 0 && d->k >= 0, DMLHIP_ERR_SHAPE, "gemm_f16: negative extent");
     DML_REQUIRE(d->m <= 2147483647 / 2 && d->n <= 2147483647 / 2 && d->k <= 2147483647 / 2, DMLHIP_ERR_SHAPE,
@@ -419,6 +420,9 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
     GemmArgs g;
     g.groups = 0;
     g.ksum = 0;
+    g.asum = !grp && asum ? asum[0] : nullptr;
+    g.asum_f32 = asum_f32;
+    for (int i = 0; i < DMLHIP_GROUP_MAX; ++i) g.gasum[i] = grp && asum && i < grp->count ? asum[i] : nullptr;
     if (grp) {
         g.groups = grp->count;
         g.ksum = grp->ksum;
@@ -475,7 +479,7 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
         return launch_pipelined(g, (const _Float16*)a, (const _Float16*)b, c, bias, residual, pre_out, amode == 1 ? 4 : 3,
                                 bmode == 1 ? 4 : 3, cfg, batch, st);
     }
-    if (grp) return DMLHIP_ERR_UNSUPPORTED;  // only the pipelined kernel takes pointer groups
+    if (grp || asum) return DMLHIP_ERR_UNSUPPORTED;  // only the pipelined kernel takes pointer groups / makes row sums
     if (cfg < 0 || cfg > 2) {
         // Largest tile that still yields at least one workgroup per CU.
         auto blocks = [&](int bm, int bn) { return (long long)ceil_div(d->m, bm) * ceil_div(d->n, bn) * batch; };
@@ -585,6 +589,58 @@ int dmlhip_gemm_f16_grouped(const dmlhip_gemm_desc* d, int groups, const void* c
         if (int e = dmlhip_gemm_f16_ws(d, a[i], b[i], c[i], bias ? bias[i] : nullptr, nullptr, nullptr, workspace,
                                        workspace_bytes, stream))
             return e;
+    return 0;
+}
+
+size_t dmlhip_gemm_f16_grouped_asum_workspace_bytes(const dmlhip_gemm_desc* d) {
+    if (!d) return 0;
+    const size_t g = dmlhip_gemm_f16_workspace_bytes(d);
+    const size_t r = dmlhip_reduce_workspace_bytes(1, d->k, d->m);
+    return g > r ? g : r;
+}
+
+int dmlhip_gemm_f16_grouped_asum(const dmlhip_gemm_desc* d, int groups, const void* const* a, const void* const* b,
+                                 void* const* c, void* const* asum, int asum_dtype, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+    DML_REQUIRE(d, DMLHIP_ERR_NULL, "gemm_f16_grouped_asum: NULL descriptor");
+    DML_REQUIRE(groups >= 1 && groups <= DMLHIP_GROUP_MAX, DMLHIP_ERR_SHAPE,
+                "gemm_f16_grouped_asum: %d groups outside 1..%d", groups, DMLHIP_GROUP_MAX);
+    DML_REQUIRE(a && b && c && asum, DMLHIP_ERR_NULL, "gemm_f16_grouped_asum: NULL pointer table");
+    DML_REQUIRE(asum_dtype == DMLHIP_F16 || asum_dtype == DMLHIP_F32, DMLHIP_ERR_ENUM,
+                "gemm_f16_grouped_asum: bad asum_dtype");
+    DML_REQUIRE(d->batch[0] == 1 && d->batch[1] == 1 && d->batch[2] == 1, DMLHIP_ERR_SHAPE,
+                "gemm_f16_grouped_asum: batched products are not supported");
+    DML_REQUIRE(d->beta == 0.f && d->act == DMLHIP_ACT_NONE, DMLHIP_ERR_UNSUPPORTED,
+                "gemm_f16_grouped_asum: beta and activations are not supported");
+    DML_REQUIRE(d->a_stride_m == 1 && d->a_stride_k == d->m, DMLHIP_ERR_UNSUPPORTED,
+                "gemm_f16_grouped_asum: A must be stored as a dense [k, m] matrix");
+    for (int i = 0; i < groups; ++i)
+        DML_REQUIRE(c[i] && asum[i] && (d->k == 0 || (a[i] && b[i])), DMLHIP_ERR_NULL,
+                    "gemm_f16_grouped_asum: NULL tensor in group %d", i);
+    bool same = d->k > 0;
+    for (int i = 0; i < groups && same; ++i)
+        same = aligned16(a[i]) && aligned16(b[i]) && reinterpret_cast<uintptr_t>(c[i]) % 32 == 0;
+    if (same) {
+        int e;
+        if (groups > 1) {
+            dmlhip_gemm_desc p = *d;
+            p.a_stride_batch[0] = p.b_stride_batch[0] = p.c_stride_batch[0] = 0;
+            GemmGroup grp = {groups, a, b, c, nullptr, false};
+            e = run_gemm_f16(&p, a[0], b[0], c[0], nullptr, nullptr, nullptr, stream, &grp, asum, asum_dtype == DMLHIP_F32);
+        } else {
+            e = run_gemm_f16(d, a[0], b[0], c[0], nullptr, nullptr, nullptr, stream, nullptr, asum, asum_dtype == DMLHIP_F32);
+        }
+        if (e == 0) ++g_grouped_single_launches;
+        if (e != DMLHIP_ERR_UNSUPPORTED) return e;
+    }
+    // products and column sums of the stored [k, m] matrices one after the other
+    for (int i = 0; i < groups; ++i) {
+        if (int e = dmlhip_gemm_f16_ws(d, a[i], b[i], c[i], nullptr, nullptr, nullptr, workspace, workspace_bytes, stream))
+            return e;
+        if (int e = dmlhip_reduce_f16(DMLHIP_RSUM, a[i], asum[i], asum_dtype, 1, d->k, d->m, workspace, workspace_bytes,
+                                      stream))
+            return e;
+    }
     return 0;
 }
 

@@ -27,6 +27,11 @@ struct GemmArgs {
     // strides (0 = an ordinary launch, pointers come from the kernel parameters). With `ksum` the groups are instead
     // concatenated along K: one output C = sum over groups of A_g B_g (only ga / gb are used).
     int groups, ksum;
+    // optional second result: asum[m] = sum over k of A[m, k] (per group: gasum), written by the workgroups of the
+    // first tile column; fp32 or fp16 elements
+    void* asum;
+    void* gasum[DMLHIP_GROUP_MAX];
+    int asum_f32;
     const _Float16* ga[DMLHIP_GROUP_MAX];
     const _Float16* gb[DMLHIP_GROUP_MAX];
     void* gc[DMLHIP_GROUP_MAX];

@@ -127,7 +127,10 @@ __device__ unsigned* dml_gemm_trace_buf;
 // ---------------------------------------------------------------- kernel
 // KSUM: the operand pairs g.ga[i] / g.gb[i] are concatenated along K (one output, see GemmArgs::ksum). A template
 // parameter, so that the ordinary kernels keep loop-invariant operand bases.
-template <int BM, int BN, int WM, int WN, int AKIND, int BKIND, int NSTAGE, int EPI, bool KSUM = false>
+// ASUM: the workgroups of tile column 0 also produce asum[m] = sum_k A[m, k] (GemmArgs::asum) — the bias gradient
+// that accompanies a weight gradient — from the A fragments they hold anyway: four packed dot products against ones
+// per fragment, vector instructions that issue while the matrix pipe works on the MFMAs of the same sub-step.
+template <int BM, int BN, int WM, int WN, int AKIND, int BKIND, int NSTAGE, int EPI, bool KSUM = false, bool ASUM = false>
 __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16* a_ptr, const _Float16* b_ptr, void* c_ptr,
                                                                  const void* bias_ptr, const void* res_ptr,
                                                                  void* pre_ptr, const GemmArgs g) {
@@ -162,11 +165,13 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     const int z2 = (int)(batch % g.batch2);
     const int z1 = (int)((batch / g.batch2) % g.batch1);
     const int z0 = (int)(batch / ((long long)g.batch2 * g.batch1));
+    void* asum_ptr = g.asum;
     if (!KSUM && g.groups) {  // uniform: one of several same-shaped problems (host sets the outer batch strides to 0)
         a_ptr = g.ga[z0];
         b_ptr = g.gb[z0];
         c_ptr = g.gc[z0];
         bias_ptr = g.gbias[z0];
+        asum_ptr = g.gasum[z0];
     }
     const int64_t aoff = z0 * g.sab[0] + z1 * g.sab[1] + z2 * g.sab[2];
     const int64_t boff = z0 * g.sbb[0] + z1 * g.sbb[1] + z2 * g.sbb[2];
@@ -186,6 +191,16 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    // wave-uniform: the wavefronts of tile column 0 sum the A rows they multiply; wn = 0 writes the result
+    static_assert(!ASUM || BN / WN == 2, "the row sums are shared by two wavefronts per row block");
+    const bool do_asum = ASUM && tn == 0 && asum_ptr != nullptr;
+    const int asum_parity = do_asum ? wn : -1;
+    float acc_sum[ASUM ? TM : 1];   // per lane: row lane % 32 of block i, the k half lane / 32 of every sub-step
+    if constexpr (ASUM) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) acc_sum[i] = 0.f;
+    }
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
     Stream<BM, AKIND, TM> sa;
@@ -291,6 +306,21 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][j], af[kk & 1][i], acc[i][j], 0, 0, 0);
+            if constexpr (ASUM) {
+                // the two wavefronts that share these A rows (wn = 0, 1) take alternate sub-steps
+                if (asum_parity == (kk & 1)) {
+                    const half2v one2 = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) {
+                        const half8 f = af[kk & 1][i];
+#pragma unroll
+                        for (int e = 0; e < 8; e += 2) {
+                            const half2v p = {f[e], f[e + 1]};
+                            acc_sum[i] = __builtin_amdgcn_fdot2(p, one2, acc_sum[i], false);
+                        }
+                    }
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (SPREAD && kk < 3) {
                 if (fill < nk) {
@@ -324,13 +354,37 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
         else store_strip<_Float16, WN, EPI>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, bias_n, strip, mb, nb, coff, lane);
         __builtin_amdgcn_wave_barrier();
     });
+    if constexpr (ASUM) {
+        // lanes l and l + 32 hold the two k halves of row l; wavefront wn = 1 hands its share over through LDS
+        __syncthreads();   // the epilogue strips in LDS are done with
+        float* hand = reinterpret_cast<float*>(lds) + wm * (TM * 32);
+        float v[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int other = __builtin_amdgcn_ds_bpermute(((lane + 32) & 63) << 2, __builtin_bit_cast(int, acc_sum[i]));
+            v[i] = acc_sum[i] + __builtin_bit_cast(float, other);
+            if (do_asum && wn == 1 && lane < 32) hand[i * 32 + lane] = v[i];
+        }
+        __syncthreads();
+        if (do_asum && wn == 0 && lane < 32) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int m = m0 + wm * WM + i * 32 + lane;
+                const float r = v[i] + hand[i * 32 + lane];
+                if (m < g.m) {
+                    if (g.asum_f32) reinterpret_cast<float*>(asum_ptr)[m] = r;
+                    else reinterpret_cast<_Float16*>(asum_ptr)[m] = (_Float16)r;
+                }
+            }
+        }
+    }
 #ifdef DML_GEMM_TRACE
     DML_TR(63);
     if (dml_gemm_trace_buf) dml_gemm_trace_buf[((size_t)blockIdx.x * 4 + wave) * 64 + lane] = (unsigned)trace_v;
 #endif
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE, bool KSUM = false>
+template <int BM, int BN, int WM, int WN, int NSTAGE, bool KSUM = false, bool ASUM = false>
 int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, const void* bias, const void* res, void* pre,
                 int akind, int bkind, long long batch, hipStream_t st) {
     g.tiles_m = (g.m + BM - 1) / BM;
@@ -348,7 +402,7 @@ int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, cons
     }
 #define DML_PIPE_CASE(AK, BKD, ACTV)                                                                          \
     if (akind == AK && bkind == BKD && ek == ACTV) {                                                          \
-        auto kern = gemm_f16_pipe_kernel<BM, BN, WM, WN, AK, BKD, NSTAGE, ACTV, KSUM>;                        \
+        auto kern = gemm_f16_pipe_kernel<BM, BN, WM, WN, AK, BKD, NSTAGE, ACTV, KSUM, ASUM>;                  \
         if (lds > 64 * 1024) {                                                                                \
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
                                                (int)lds);                                                     \
@@ -361,14 +415,19 @@ int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, cons
         return launch_status("gemm_f16(pipelined)");                                                          \
     }
     DML_PIPE_CASE(0, 0, EPI_PLAIN) DML_PIPE_CASE(0, 1, EPI_PLAIN) DML_PIPE_CASE(1, 0, EPI_PLAIN) DML_PIPE_CASE(1, 1, EPI_PLAIN)
-    if constexpr (!KSUM) {
-        DML_PIPE_CASE(0, 0, EPI_ACT) DML_PIPE_CASE(0, 1, EPI_ACT) DML_PIPE_CASE(1, 0, EPI_ACT) DML_PIPE_CASE(1, 1, EPI_ACT)
+    if constexpr (ASUM) {
+        set_error("gemm_f16: the row-sum result needs a plain epilogue");
+        return DMLHIP_ERR_UNSUPPORTED;
+    } else {
+        if constexpr (!KSUM) {
+            DML_PIPE_CASE(0, 0, EPI_ACT) DML_PIPE_CASE(0, 1, EPI_ACT) DML_PIPE_CASE(1, 0, EPI_ACT) DML_PIPE_CASE(1, 1, EPI_ACT)
+        }
+        DML_PIPE_CASE(0, 0, EPI_GENERAL) DML_PIPE_CASE(0, 1, EPI_GENERAL) DML_PIPE_CASE(1, 0, EPI_GENERAL)
+        DML_PIPE_CASE(1, 1, EPI_GENERAL)
+        set_error("gemm_f16: no pipelined kernel for operand kinds %d/%d", akind, bkind);
+        return DMLHIP_ERR_UNSUPPORTED;
     }
-    DML_PIPE_CASE(0, 0, EPI_GENERAL) DML_PIPE_CASE(0, 1, EPI_GENERAL) DML_PIPE_CASE(1, 0, EPI_GENERAL)
-    DML_PIPE_CASE(1, 1, EPI_GENERAL)
 #undef DML_PIPE_CASE
-    set_error("gemm_f16: no pipelined kernel for operand kinds %d/%d", akind, bkind);
-    return DMLHIP_ERR_UNSUPPORTED;
 }
 
 }  // namespace
@@ -376,6 +435,14 @@ int launch_tile(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, cons
 int launch_pipelined(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, const void* bias, const void* residual,
                      void* pre, int amode, int bmode, int cfg, long long batch, hipStream_t st) {
     const int ak = amode == 4 ? 1 : 0, bk = bmode == 4 ? 1 : 0;
+    if (g.asum || (g.groups && g.gasum[0])) {  // row sums of A alongside: the two 128x128 configurations only
+        if (g.ksum) {
+            set_error("gemm_f16: row sums are not combined with K-concatenated operand pairs");
+            return DMLHIP_ERR_UNSUPPORTED;
+        }
+        if (cfg == 3) return launch_tile<128, 128, 64, 64, 2, false, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+        return launch_tile<128, 128, 64, 64, 4, false, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+    }
     if (g.ksum) {  // K-concatenated operand pairs: the two 128x128 configurations only
         if (cfg == 3) return launch_tile<128, 128, 64, 64, 2, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
         return launch_tile<128, 128, 64, 64, 4, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);

@@ -534,6 +534,40 @@ def reduce_sum_multi(xs: Sequence[torch.Tensor], out_dtype: Optional[torch.dtype
     return ys
 
 
+def einsum_grouped_asum(equation: str, a_list: Sequence[torch.Tensor], b_list: Sequence[torch.Tensor], *,
+                        out_dtype: Optional[torch.dtype] = None, sum_dtype: torch.dtype = torch.float32,
+                        alpha: float = 1.0):
+    """Like einsum_grouped (one or more pairs, no bias), and per pair the sum of the first operand over the contracted
+    indices: for a weight gradient ``einsum("aij,aik->jk", dY, X)`` that is the bias gradient ``dY.sum((0, 1))``.
+    Returns (outputs, sums)."""
+    from . import contraction as C
+    n = len(a_list)
+    if n != len(b_list) or n < 1:
+        raise ValueError("einsum_grouped_asum: lists differ in length")
+    _check(*a_list, *b_list, dtype=None)
+    a0, b0 = a_list[0], b_list[0]
+    if a0.dtype != torch.float16:
+        raise TypeError("einsum_grouped_asum is implemented for fp16 operands")
+    for a, b in zip(a_list, b_list):
+        if a.shape != a0.shape or a.stride() != a0.stride() or b.shape != b0.shape or b.stride() != b0.stride() \
+                or a.dtype != a0.dtype or b.dtype != a0.dtype:
+            raise ValueError("einsum_grouped_asum: every pair needs the shapes, strides and dtype of pair 0")
+    out_dtype = out_dtype or a0.dtype
+    plan = C.plan_contraction(equation, a0.shape, a0.stride(), b0.shape, b0.stride())
+    if plan.swapped or any(e != 1 for e in plan.batch):
+        raise C.NotApplicable("einsum_grouped_asum: the summed operand must be the unbatched row operand of the product")
+    outs = [torch.empty(plan.out_shape, dtype=out_dtype, device=a0.device) for _ in range(n)]
+    sums = [torch.empty(plan.m, dtype=sum_dtype, device=a0.device) for _ in range(n)]
+    desc = _fill_desc(plan, alpha, 0.0, out_dtype, None, L.ACT_NONE)
+    arr = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])  # noqa: E731
+    lib = L.load()
+    ws = workspace(lib.dmlhip_gemm_f16_grouped_asum_workspace_bytes(ctypes.byref(desc)), a0.device)
+    L.check(lib.dmlhip_gemm_f16_grouped_asum(ctypes.byref(desc), n, arr(a_list), arr(b_list), arr(outs), arr(sums),
+                                             L.F32 if sum_dtype == torch.float32 else L.F16, _ptr(ws), ws.numel(),
+                                             _stream()))
+    return outs, sums
+
+
 def einsum_sum(equation: str, a_list: Sequence[torch.Tensor], b_list: Sequence[torch.Tensor], *,
                out_dtype: Optional[torch.dtype] = None, alpha: float = 1.0, bias: Optional[torch.Tensor] = None,
                residual: Optional[torch.Tensor] = None) -> torch.Tensor:

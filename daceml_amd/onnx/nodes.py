@@ -128,7 +128,8 @@ SCHEMAS = [
     _schema("Swish", "X", "Y", since=1),
     # a contraction with its neighbours folded in (scale, bias Add, activation, residual Add);
     # produced by the fusion pass, never by an importer
-    _schema("FusedEinsum", "Inputs* Bias? Residual?", "Output PreActivation?", since=1, equation=REQUIRED,
+    # InputSum: Inputs__0 summed over the contracted indices (the bias gradient beside a weight gradient)
+    _schema("FusedEinsum", "Inputs* Bias? Residual?", "Output PreActivation? InputSum?", since=1, equation=REQUIRED,
             alpha=1.0, activation="none", accumulate=0),
     # Einsum(Q,K) [* scale] -> Softmax(last axis) -> Einsum(P,V) as one node (the scores never reach memory).
     # *_perm: which dimension of that tensor is (batch0, batch1, sequence, head); -1 for an absent batch dim.
@@ -141,7 +142,7 @@ SCHEMAS = [
             pads=None, strides=None),
     # several FusedEinsum nodes of identical equation, shapes, strides and scale, independent of each other, in one
     # launch: Output__i = alpha * einsum(equation, A__i, B__i) [+ Bias__i]
-    _schema("GroupedEinsum", "A* B* Bias*?", "Output*", since=1, equation=REQUIRED, alpha=1.0),
+    _schema("GroupedEinsum", "A* B* Bias*?", "Output* InputSum*?", since=1, equation=REQUIRED, alpha=1.0),
     # several independent ReduceSum(all leading axes, keepdims=0) nodes in one launch pair: reduced__i = sum of
     # data__i over every axis but the last (the bias gradients of a backward pass)
     _schema("EinsumSum", "A* B* Residual?", "Output", since=1, equation=REQUIRED, alpha=1.0),

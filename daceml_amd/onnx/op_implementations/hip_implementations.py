@@ -173,6 +173,28 @@ class HipEinsum(ONNXForward):
         return _einsum_tasklet(node, state, eq, "Inputs__0", "Inputs__1", "Output", ins[0], ins[1], out)
 
 
+def _input_sum_ok(plan, a: Array, s: Array) -> bool:
+    """The row-sum result of the contraction kernel: the summed operand is the unbatched row operand A, stored as a
+    dense [k, m] matrix; the sums are a dense vector of m fp16 / fp32 values."""
+    return (plan is not None and not plan.swapped and all(e == 1 for e in plan.batch) and a.dtype == torch.float16
+            and a.is_contiguous() and a.shape[-1] == plan.m and a.total_size == plan.m * plan.k
+            and s.dtype in FLOAT_DTYPES and s.is_contiguous() and s.total_size == plan.m)
+
+
+def _asum_tasklet(node, state, eq, alpha, a, b, out, sum_desc, a_conns, b_conns, out_conns, sum_conns):
+    import ctypes
+    n = len(a)
+    plan = C.plan_contraction(eq, a[0].shape, a[0].strides, b[0].shape, b[0].strides)
+    desc = _gemm_struct(plan, alpha, 0.0, out[0].dtype, out[0].dtype, L.ACT_NONE)
+    ws = L.load().dmlhip_gemm_f16_grouped_asum_workspace_bytes(ctypes.byref(desc))
+    call = HipCall("dmlhip_gemm_f16_grouped_asum",
+                   [Struct(desc, "dmlhip_gemm_desc"), I32(n), PtrArray(tuple(a_conns)), PtrArray(tuple(b_conns)),
+                    PtrArray(tuple(out_conns)), PtrArray(tuple(sum_conns)), I32(_CODE[sum_desc.dtype]), Workspace(),
+                    WorkspaceBytes(), Stream()])
+    return _tasklet(node, state, [call], workspace_bytes=ws, flops=plan.flops * n,
+                    bytes_moved=sum(_nbytes(a[i], b[i], out[i]) for i in range(n)), kind="gemm")
+
+
 @op_implementation(op="FusedEinsum", name=IMPL)
 class HipFusedEinsum(ONNXForward):
     """A contraction with the scale / bias Add / activation / residual Add that followed it in the
@@ -200,6 +222,11 @@ class HipFusedEinsum(ONNXForward):
                 if d is not None and not (d.is_contiguous() and tuple(d.shape) == tuple(out.shape)
                                           and d.dtype == out.dtype):
                     return False
+            if "InputSum" in outs:
+                plain = set(ins) == {"Inputs__0", "Inputs__1"} and set(outs) == {"Output", "InputSum"}
+                if not (plain and node.activation == "none" and not node.accumulate
+                        and _input_sum_ok(plan, ins["Inputs__0"], outs["InputSum"])):
+                    return False
             return True
         except Exception:
             return False
@@ -207,6 +234,10 @@ class HipFusedEinsum(ONNXForward):
     @staticmethod
     def forward(node, state, sdfg):
         ins, outs = _descs(node, state, sdfg)
+        if "InputSum" in outs:
+            return _asum_tasklet(node, state, node.equation.replace(" ", ""), node.alpha, [ins["Inputs__0"]],
+                                 [ins["Inputs__1"]], [outs["Output"]], outs["InputSum"], ["Inputs__0"], ["Inputs__1"],
+                                 ["Output"], ["InputSum"])
         return _einsum_tasklet(node, state, node.equation.replace(" ", ""), "Inputs__0", "Inputs__1", "Output",
                                ins["Inputs__0"], ins["Inputs__1"], outs["Output"], alpha=node.alpha,
                                beta=1.0 if node.accumulate else 0.0, act=_ACT[node.activation],
@@ -1190,12 +1221,19 @@ class HipGroupedEinsum(ONNXForward):
     @staticmethod
     def _groups(node, state, sdfg):
         ins, outs = _descs(node, state, sdfg)
-        n = len(outs)
+        n = len([k for k in outs if k.startswith("Output__")])
         a = [ins["A__%d" % i] for i in range(n)]
         b = [ins["B__%d" % i] for i in range(n)]
         bias = [ins["Bias__%d" % i] for i in range(n)] if "Bias__0" in ins else None
         out = [outs["Output__%d" % i] for i in range(n)]
         return n, a, b, bias, out
+
+    @staticmethod
+    def _sums(node, state, sdfg, n):
+        _, outs = _descs(node, state, sdfg)
+        if "InputSum__0" not in outs:
+            return None
+        return [outs["InputSum__%d" % i] for i in range(n)]
 
     @staticmethod
     def forward_can_be_applied(node, state, sdfg) -> bool:
@@ -1221,6 +1259,12 @@ class HipGroupedEinsum(ONNXForward):
                     if not (t.dtype == bias[0].dtype and t.dtype in FLOAT_DTYPES and t.is_contiguous()
                             and t.total_size == plan.n and t.shape[-1] == plan.n):
                         return False
+            sums = HipGroupedEinsum._sums(node, state, sdfg, n)
+            if sums is not None:
+                if bias is not None or any(t.dtype != sums[0].dtype for t in sums):
+                    return False
+                if not all(_input_sum_ok(plan, a[i], sums[i]) for i in range(n)):
+                    return False
             return True
         except Exception:
             return False
@@ -1230,6 +1274,12 @@ class HipGroupedEinsum(ONNXForward):
         import ctypes
         n, a, b, bias, out = HipGroupedEinsum._groups(node, state, sdfg)
         eq = node.equation.replace(" ", "")
+        sums = HipGroupedEinsum._sums(node, state, sdfg, n)
+        if sums is not None:
+            rng_ = range(n)
+            return _asum_tasklet(node, state, eq, node.alpha, a, b, out, sums[0], ["A__%d" % i for i in rng_],
+                                 ["B__%d" % i for i in rng_], ["Output__%d" % i for i in rng_],
+                                 ["InputSum__%d" % i for i in rng_])
         plan = C.plan_contraction(eq, a[0].shape, a[0].strides, b[0].shape, b[0].strides)
         desc = _gemm_struct(plan, node.alpha, 0.0, out[0].dtype, bias[0].dtype if bias else out[0].dtype, L.ACT_NONE)
         xa, xb = ("B", "A") if plan.swapped else ("A", "B")

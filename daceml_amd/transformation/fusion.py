@@ -709,6 +709,50 @@ def fuse_attention(sdfg: SDFG) -> int:
     return count
 
 
+def fuse_bias_gradients(sdfg: SDFG) -> int:
+    """A ReduceSum of dY over every axis but the last (a bias gradient; the third node DefaultEinsumBackward's
+    callers emit, daceml/autodiff/implementations/onnx_ops.py:54-138) next to a contraction whose first operand is
+    the same dY summed over the same indices (the weight gradient) becomes that contraction's InputSum output: the
+    kernel adds up the operand tiles it multiplies anyway, and dY is not read a second time."""
+    count = 0
+    for state in sdfg.states():
+        for red in [n for n in state.nodes() if _is_op(n, "ReduceSum")]:
+            if red.keepdims:
+                continue
+            x, y = _in_array(state, red, "data"), _out_array(state, red, "reduced")
+            xd, yd = sdfg.arrays[x], sdfg.arrays[y]
+            nd = len(xd.shape)
+            axes = sorted(a % nd for a in (red.axes if red.axes is not None else range(nd)))
+            if nd < 2 or axes != list(range(nd - 1)) or _consumers(state, y) or xd.dtype != torch.float16 \
+                    or not (xd.is_contiguous() and yd.is_contiguous()) or yd.dtype not in (torch.float16, torch.float32):
+                continue
+            for node, conn in _consumers(state, x):
+                if not _is_op(node, "FusedEinsum") or conn != "Inputs__0" or node.activation != "none" or node.accumulate:
+                    continue
+                conns = {e.dst_conn for e in state.in_edges(node)} | {e.src_conn for e in state.out_edges(node)}
+                if conns != {"Inputs__0", "Inputs__1", "Output"}:
+                    continue
+                b = sdfg.arrays[_in_array(state, node, "Inputs__1")]
+                eq = node.equation.replace(" ", "")
+                terms, res = eq.split("->")[0].split(","), eq.split("->")[1]
+                # the last axis of dY survives into the result, every other axis of it is contracted with the other operand
+                if len(terms) != 2 or terms[0][-1] not in res or any(l in res or l not in terms[1] for l in terms[0][:-1]):
+                    continue
+                try:
+                    plan = C.plan_contraction(eq, xd.shape, xd.strides, b.shape, b.strides)
+                except (C.NotApplicable, ValueError):
+                    continue
+                if plan.swapped or any(e != 1 for e in plan.batch) or plan.m != xd.shape[-1] \
+                        or plan.m * plan.k != xd.total_size or plan.k % 64 or b.dtype != torch.float16:
+                    continue
+                _remove_node(state, red)
+                node.add_out_connector("InputSum")
+                state.add_edge(node, "InputSum", state.add_write(y), None, sdfg.make_array_memlet(y))
+                count += 1
+                break
+    return count
+
+
 def fuse_reductions(sdfg: SDFG, max_group: int = 8) -> int:
     """Horizontal fusion (cf. HorizontalEinsumFusion, daceml/transformation/einsum_fusion.py:102-151) of ReduceSum
     nodes that sum over every axis but the last with keepdims=0 and whose results nobody in the state reads
@@ -786,7 +830,8 @@ def group_einsums(sdfg: SDFG, max_group: int = 4) -> int:
             if not _is_op(n, "FusedEinsum") or n.activation != "none" or n.accumulate:
                 continue
             conns = {e.dst_conn for e in state.in_edges(n)} | {e.src_conn for e in state.out_edges(n)}
-            if conns - {"Inputs__0", "Inputs__1", "Bias", "Output"} or not {"Inputs__0", "Inputs__1", "Output"} <= conns:
+            if conns - {"Inputs__0", "Inputs__1", "Bias", "Output", "InputSum"} \
+                    or not {"Inputs__0", "Inputs__1", "Output"} <= conns:
                 continue
             a = sdfg.arrays[_in_array(state, n, "Inputs__0")]
             b = sdfg.arrays[_in_array(state, n, "Inputs__1")]
@@ -794,8 +839,10 @@ def group_einsums(sdfg: SDFG, max_group: int = 4) -> int:
             if a.dtype != torch.float16 or b.dtype != torch.float16 or not o.is_contiguous():
                 continue
             bias = _in_array(state, n, "Bias")
+            isum = _out_array(state, n, "InputSum")
             key = (n.equation.replace(" ", ""), float(n.alpha), tuple(a.shape), tuple(a.strides), tuple(b.shape),
-                   tuple(b.strides), tuple(o.shape), o.dtype, None if bias is None else sdfg.arrays[bias].dtype)
+                   tuple(b.strides), tuple(o.shape), o.dtype, None if bias is None else sdfg.arrays[bias].dtype,
+                   None if isum is None else sdfg.arrays[isum].dtype)
             buckets.setdefault(key, []).append(n)
         for key, nodes in buckets.items():
             if len(nodes) < 2:
@@ -828,6 +875,9 @@ def group_einsums(sdfg: SDFG, max_group: int = 4) -> int:
                     if bias is not None:
                         ins["Bias__%d" % i] = bias
                     outs["Output__%d" % i] = _out_array(state, n, "Output")
+                    isum = _out_array(state, n, "InputSum")
+                    if isum is not None:
+                        outs["InputSum__%d" % i] = isum
                 label = "grouped_" + "_".join(n.label.replace("_matmul_fused", "") for n in grp)
                 for n in grp:
                     _remove_node(state, n)
@@ -929,7 +979,8 @@ def fuse_einsum_sums(sdfg: SDFG, max_group: int = 4) -> int:
 def optimize_backward(sdfg: SDFG) -> Dict[str, int]:
     """Rewrites for the state(s) autodiff added — what a ``post_autodiff_hooks`` entry of the reference's module
     wrapper would run (daceml/torch/module.py:46-365)."""
-    stats = {"reductions": fuse_reductions(sdfg)}
+    stats = {"bias_gradients": fuse_bias_gradients(sdfg)}
+    stats["reductions"] = fuse_reductions(sdfg)
     stats["einsum_sums"] = fuse_einsum_sums(sdfg)      # before grouping: a summed group needs no separate outputs
     stats["grouped_einsums"] = group_einsums(sdfg)
     return stats

@@ -225,6 +225,17 @@ int dmlhip_gemm_f16_ws(const dmlhip_gemm_desc* desc, const void* a, const void* 
 int dmlhip_gemm_f16_grouped(const dmlhip_gemm_desc* d, int groups, const void* const* a,
                             const void* const* b, void* const* c, const void* const* bias,
                             void* workspace, size_t workspace_bytes, void* stream);
+/* dmlhip_gemm_f16_grouped without bias, plus a second result per group: asum[i][m] = sum over k of a[i][m, k]
+ * (element type asum_dtype). For a weight gradient dW = dY^T X this is the bias gradient, i.e. the ReduceSum node
+ * that accompanies the two Einsum nodes of DefaultEinsumBackward's callers
+ * (daceml/autodiff/implementations/onnx_ops.py:54-138) — produced inside the contraction from the operand tiles
+ * that are in LDS anyway instead of by another pass over dY. groups may be 1. Unbatched products only; a[i] must be
+ * stored as a dense [k, m] matrix (a_stride_m == 1, a_stride_k == m). Needs a workspace of
+ * dmlhip_gemm_f16_grouped_asum_workspace_bytes(d) for the case that one launch is not possible. */
+size_t dmlhip_gemm_f16_grouped_asum_workspace_bytes(const dmlhip_gemm_desc* d);
+int dmlhip_gemm_f16_grouped_asum(const dmlhip_gemm_desc* d, int groups, const void* const* a,
+                                 const void* const* b, void* const* c, void* const* asum, int asum_dtype,
+                                 void* workspace, size_t workspace_bytes, void* stream);
 /* c = alpha * sum_i a[i] b[i] (+ column bias) (+ residual): `groups` products of identical shape and strides that
  * are summed — the operand pairs are concatenated along K inside one launch, so the partial products never reach
  * memory. This is what autodiff's gradient accumulation (an ONNXSum over the contributions of several consumers,

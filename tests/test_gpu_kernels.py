@@ -629,6 +629,33 @@ def test_einsum_sum(eq, sa, sb, n, with_res, out_dtype, single):
     assert_close(host(got), want, torch.float16, "einsum sum %s x%d" % (eq, n), atol=1e-2 * max(1.0, np.sqrt(k_total / 256)))
 
 
+@pytest.mark.parametrize("sa,sb,n,sum_dtype,single", [
+    ((2, 256, 128), (2, 256, 64), 1, torch.float32, True),     # one weight gradient [128, 64] with its bias gradient
+    ((2, 256, 256), (2, 256, 128), 3, torch.float32, True),    # grouped; two tile rows
+    ((4, 128, 384), (4, 128, 192), 4, torch.float16, True),    # three tile rows, two tile columns
+    ((2, 256, 200), (2, 256, 72), 2, torch.float32, True),     # ragged m and n: clamped rows must not reach the sums
+    ((3, 50, 128), (3, 50, 64), 2, torch.float32, False),      # K = 150: separate products and column reductions
+])
+def test_einsum_grouped_asum(sa, sb, n, sum_dtype, single):
+    """dW_i = einsum("aij,aik->jk", dY_i, X_i) together with db_i = dY_i.sum((0, 1)) from the same launch."""
+    from daceml_amd import _lib as L, kernels as K
+    eq = "aij,aik->jk"
+    a = [_inputs(500 + i, sa, torch.float16) for i in range(n)]
+    b = [_inputs(510 + i, sb, torch.float16) for i in range(n)]
+    count = L.load().dmlhip_debug_grouped_single_launches
+    before = count()
+    outs, sums = K.einsum_grouped_asum(eq, [dev(x) for x, _ in a], [dev(x) for x, _ in b], out_dtype=torch.float32,
+                                       sum_dtype=sum_dtype)
+    assert count() - before == (1 if single else 0)
+    k_total = sa[0] * sa[1]
+    for i in range(n):
+        assert outs[i].dtype == torch.float32 and sums[i].dtype == sum_dtype and tuple(sums[i].shape) == (sa[2], )
+        assert_close(host(outs[i]), O.einsum(eq, a[i][1], b[i][1]), torch.float16, "weight gradient %d" % i,
+                     atol=1e-2 * max(1.0, np.sqrt(k_total / 256)))
+        assert_close(host(sums[i]), O.reduce_sum(a[i][1], axes=[0, 1], keepdims=0), torch.float16, "bias gradient %d" % i,
+                     atol=1e-2 * max(1.0, np.sqrt(k_total / 64)))
+
+
 def _einsum_grouped_case(eq, sa, sb, with_bias, out_dtype):
     from daceml_amd import contraction as C, kernels as K
     n = 3

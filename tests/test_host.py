@@ -355,11 +355,15 @@ def test_attention_fusion_roles_and_graph():
     assert ins == {"Q", "K", "V", "O", "LogSumExp", "dO"}
     # the six bias gradients become one node; nothing else in the state changes
     n_before = len(sdfg.states()[1].library_nodes())
-    assert fusion.optimize_backward(sdfg) == {"reductions": 5, "einsum_sums": 6, "grouped_einsums": 5}
+    assert fusion.optimize_backward(sdfg) == {"bias_gradients": 6, "reductions": 0, "einsum_sums": 6, "grouped_einsums": 5}
     bnodes = sdfg.states()[1].library_nodes()
-    # five reductions, two gradient sums and five contractions fewer (q/k/v input gradients: 3 -> 1 EinsumSum that also
-    # adds the residual path; o/q/k/v weight gradients: 4 -> 1; the other Sum rides on a contraction as its Residual)
-    assert len(bnodes) == n_before - 12 and not any(n.schema.name in ("ReduceSum", "Sum") for n in bnodes)
+    # six bias-gradient reductions (now InputSum outputs of the weight-gradient contractions), two gradient sums and five
+    # contractions fewer (q/k/v input gradients: 3 -> 1 EinsumSum that also adds the residual path; o/q/k/v weight
+    # gradients: 4 -> 1; the other Sum rides on a contraction as its Residual)
+    assert len(bnodes) == n_before - 13 and not any(n.schema.name in ("ReduceSum", "MultiReduceSum", "Sum") for n in bnodes)
+    wg = [n for n in bnodes if n.schema.name == "GroupedEinsum"]
+    assert len(wg) == 1 and {_out(sdfg.states()[1], wg[0], "InputSum__%d" % i) for i in range(4)} == \
+        {"gradient_%s_b" % p for p in "koqv"}
     es = [n for n in bnodes if n.schema.name == "EinsumSum"]
     assert len(es) == 1 and es[0].label == "sum_k_grad_0_q_grad_0_v_grad_0"
     assert _out(sdfg.states()[1], es[0], "Output") == "gradient_x"
@@ -371,8 +375,16 @@ def test_attention_fusion_roles_and_graph():
     assert any(n.label == "o_matmul_fused_grad_0" for n in bnodes)
     for st_ in sdfg.states():
         st_.topological_sort()
-    multi = [n for n in bnodes if n.schema.name == "MultiReduceSum"][0]
-    outs = sorted(e.data.data for e in sdfg.states()[1].out_edges(multi))
+    sums = sorted(e.data.data for n in bnodes for e in sdfg.states()[1].out_edges(n) if e.src_conn.startswith("InputSum"))
+    assert sums == sorted("gradient_%s_b" % p for p in ("q", "k", "v", "o", "ffn1", "ffn2"))
+    # without the contraction route the six reductions still merge into one MultiReduceSum
+    s2 = graphs.bert_encoder_layer(2, 64, 256, 4, 512, torch.float16)
+    fusion.auto_optimize(s2, training=True)
+    add_backward_pass(s2, s2.states()[0], ["y"], ["x"] + OB.PARAM_NAMES,
+                      grad_dtypes={n: torch.float32 for n in OB.PARAM_NAMES})
+    assert fusion.fuse_reductions(s2) == 5
+    multi = [n for n in s2.states()[1].library_nodes() if n.schema.name == "MultiReduceSum"][0]
+    outs = sorted(e.data.data for e in s2.states()[1].out_edges(multi))
     assert outs == sorted("gradient_%s_b" % p for p in ("q", "k", "v", "o", "ffn1", "ffn2"))
     # the forward node now also emits the log-sum-exp rows
     assert "LogSumExp" in {e.src_conn for e in st.out_edges(att)}
