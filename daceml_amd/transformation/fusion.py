@@ -1006,4 +1006,7 @@ def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True,
     stats["epilogues"] = fuse_epilogues(sdfg, keep_preactivation=training, activation_in_epilogue=gelu_epilogue)
     stats["skip_layernorm"] = fuse_skip_layernorm(sdfg)
     stats["attention"] = fuse_attention(sdfg) if attention else 0
+    # with a backward pass to come, grouping waits until after autodiff (optimize_backward): the backward
+    # implementations differentiate the single contractions
+    stats["grouped_einsums"] = 0 if training else group_einsums(sdfg)
     return stats

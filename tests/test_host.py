@@ -300,7 +300,8 @@ def test_fusion_pipeline_on_bert_layer():
     assert before.count("MatMul") == 8 and before.count("Erf") == 1 and before.count("ReduceMean") == 4
     stats = fusion.auto_optimize(sdfg, training=True, gelu_epilogue=True)
     assert stats == {"gelu": 1, "layernorm": 2, "swish": 0, "conv_activation": 0, "gated_conv": 0, "matmul_to_einsum": 8,
-                     "views": 15, "epilogues": 7, "skip_layernorm": 0, "attention": 0}  # head dim 32: not fused
+                     "views": 15, "epilogues": 7, "skip_layernorm": 0, "attention": 0,   # head dim 32: not fused
+                     "grouped_einsums": 0}                                               # training: after autodiff
     after = {n.label: n for n in st.library_nodes()}
     assert sorted(n.schema.name for n in after.values()) == ["Einsum"] + ["FusedEinsum"] * 7 + \
         ["LayerNormalization"] * 2 + ["Softmax"]
@@ -313,6 +314,10 @@ def test_fusion_pipeline_on_bert_layer():
     assert after["ln1_fused"].epsilon == 1e-12                          # not the fp16-rounded 0.0
     assert all(e.dst_conn != "Inputs__1" or sdfg.arrays[e.data.data].shape == (128, 128)
                for e in st.in_edges(after["q_matmul_fused"]))           # weight used as stored, no Transpose
+    # an inference graph also gets its three projections grouped into one launch
+    inf = graphs.bert_encoder_layer(2, 64, 128, 4, 512, torch.float16)
+    assert fusion.auto_optimize(inf)["grouped_einsums"] == 2
+    assert "grouped_k_q_v" in {n.label for n in inf.states()[0].library_nodes()}
 
 
 def _out(state, node, conn):
