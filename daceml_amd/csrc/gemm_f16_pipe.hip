@@ -144,27 +144,38 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     int trace_v = 0;
 #endif
     DML_TR(0);
-    long long bid = blockIdx.x;
+    // All of this is wave-uniform integer arithmetic in 32 bits (the host checks total_blocks < 2^31): 64-bit
+    // divisions are long software sequences, and this prologue runs before the first load can be issued.
+    uint32_t bid = blockIdx.x;
     {
-        const long long total = g.total_blocks;
-        const long long xcd = bid % kXcds, idx = bid / kXcds;
-        const long long base = total / kXcds, rem = total % kXcds;
+        const uint32_t total = (uint32_t)g.total_blocks;
+        const uint32_t xcd = bid % kXcds, idx = bid / kXcds;
+        const uint32_t base = total / kXcds, rem = total % kXcds;
         bid = xcd * base + (xcd < rem ? xcd : rem) + idx;
     }
-    const int tiles = g.tiles_m * g.tiles_n;
-    const long long batch = bid / tiles;
-    const int tile = (int)(bid % tiles);
+    const uint32_t tiles = (uint32_t)(g.tiles_m * g.tiles_n);
+    uint32_t batch = 0, tile = bid;
+    if (bid >= tiles) {   // more than one batch entry / group
+        batch = bid / tiles;
+        tile = bid - batch * tiles;
+    }
     // Tiles are walked in groups of kGroupM tile rows, column by column inside a group: the workgroups that
     // are resident together (and the contiguous run of tiles an XCD gets) then cover a squarish patch of C and
     // share few rows of A and few columns of B, which is what fits an XCD's 4 MB L2.
-    constexpr int kGroupM = 8;
-    const int per_group = kGroupM * g.tiles_n;
-    const int group = tile / per_group, in_group = tile % per_group;
-    const int rows_here = min(g.tiles_m - group * kGroupM, kGroupM);
-    const int tm = group * kGroupM + in_group % rows_here, tn = in_group / rows_here;
-    const int z2 = (int)(batch % g.batch2);
-    const int z1 = (int)((batch / g.batch2) % g.batch1);
-    const int z0 = (int)(batch / ((long long)g.batch2 * g.batch1));
+    constexpr uint32_t kGroupM = 8;
+    const uint32_t per_group = kGroupM * (uint32_t)g.tiles_n;
+    const uint32_t group = tile / per_group, in_group = tile - group * per_group;
+    const uint32_t rows_here = min((uint32_t)g.tiles_m - group * kGroupM, kGroupM);
+    const uint32_t tn_u = in_group / rows_here;
+    const int tm = (int)(group * kGroupM + (in_group - tn_u * rows_here)), tn = (int)tn_u;
+    int z0 = 0, z1 = 0, z2 = 0;
+    if (batch != 0) {
+        const uint32_t b2 = (uint32_t)g.batch2, b1 = (uint32_t)g.batch1;
+        const uint32_t q = batch / b2;
+        z2 = (int)(batch - q * b2);
+        z0 = (int)(q / b1);
+        z1 = (int)(q - (uint32_t)z0 * b1);
+    }
     void* asum_ptr = g.asum;
     if (!KSUM && g.groups) {  // uniform: one of several same-shaped problems (host sets the outer batch strides to 0)
         a_ptr = g.ga[z0];

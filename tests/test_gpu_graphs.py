@@ -45,10 +45,12 @@ def test_bert_layer_forward(dtype, fused):
         names = [n.schema.name for n in sdfg.states()[0].library_nodes()]
         if fused == "attention" and dtype == torch.float16:  # the fused kernel is fp16 only
             assert stats["attention"] == 1
-            assert sorted(set(names)) == ["FusedAttention", "FusedEinsum", "Gelu", "LayerNormalization"]
+            assert sorted(set(names)) == ["FusedAttention", "FusedEinsum", "Gelu", "GroupedEinsum", "LayerNormalization"]
         else:
             assert stats["attention"] == 0
             extra = ["Gelu"] if fused == "attention" else []
+            # the three projections run as one grouped launch where the grouped kernel exists (fp16)
+            extra += ["GroupedEinsum"] if dtype == torch.float16 else []
             assert sorted(set(names)) == sorted(["Einsum", "FusedEinsum", "LayerNormalization", "Softmax"] + extra)
     prog = _compile(sdfg)
     y = torch.empty((b, s, h), dtype=dtype, device="cuda")
