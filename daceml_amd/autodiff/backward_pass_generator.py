@@ -171,7 +171,7 @@ class BackwardPassGenerator:
 
     def _targets(self, rev: Node, conn: str) -> List[Tuple[Node, str]]:
         if isinstance(rev, BackwardGroup):
-            return rev.inputs[conn]
+            return rev.inputs.get(conn, [])   # empty when every input gradient is a pass-through of the given one
         return [(rev, conn)]
 
     def _source(self, rev: Node, conn: str) -> Tuple[Node, str]:

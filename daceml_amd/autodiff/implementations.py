@@ -344,6 +344,136 @@ class HipAddBackward(BackwardImplementation):
                                      passthrough=passthrough)
 
 
+def _broadcast_ok(node, state, sdfg) -> bool:
+    """Operands have the output's shape or its trailing dims (the broadcasts the exporter emits: bias vectors,
+    per-row scalars come as [.., 1] and are not covered)."""
+    return HipAddBackward.backward_can_be_applied(node, state, sdfg)
+
+
+def _minus_one(ctx, dtype) -> str:
+    sdfg = ctx.forward_sdfg
+    name = "autodiff_minus_one_%s" % str(dtype).split(".")[-1]
+    if name not in sdfg.arrays:
+        sdfg.add_array(name, (), dtype)
+        sdfg.add_constant(name, torch.tensor(-1.0, dtype=dtype))
+        sdfg.constants_exact[name] = -1.0
+    return name
+
+
+class _ElementwiseBackward:
+    """Builds the reverse of a broadcasting binary op out of the same elementwise library nodes (what the SymPy
+    tasklet reversal of daceml/autodiff/backward_pass_generator.py:1284-1421 produces as generated maps, plus
+    ReverseReduce, dace_nodes.py:13-105, for a broadcast operand)."""
+    def __init__(self, forward_node, ctx):
+        self.node, self.ctx = forward_node, ctx
+        self.sdfg = ctx.forward_sdfg
+        self.out = _out_arr(ctx, forward_node, "C")
+        self.od = self.sdfg.arrays[self.out]
+        self.group = BackwardGroup(forward_node.label + "_backward")
+        self.n = 0
+
+    def op(self, kind, a, b):
+        """A binary node; an operand is an array name, or None for the given gradient. Returns (node, out conn)."""
+        self.n += 1
+        node = _new(self.ctx, kind, "%s_grad_%s_%d" % (self.node.label, kind.lower(), self.n))
+        for conn, src in (("A", a), ("B", b)):
+            node.add_in_connector(conn)
+            if src is None:
+                self.group.map_input("C_grad", node, conn)
+            elif isinstance(src, tuple):
+                tmp, _ = self.sdfg.add_transient("%s_tmp_%d" % (self.group.label, self.n), self.od.shape, self.od.dtype)
+                _write(self.ctx, src[0], src[1], tmp)
+                _read(self.ctx, tmp, node, conn)
+            else:
+                _read(self.ctx, src, node, conn)
+        node.add_out_connector("C")
+        return node, "C"
+
+    def finish(self, conn, produced):
+        """Route a full-shape gradient (node, connector) to input `conn`, reducing over broadcast dims if needed."""
+        shp = self.sdfg.arrays[_in_arr(self.ctx, self.node, conn)].shape
+        if tuple(shp) == tuple(self.od.shape):
+            self.group.map_output(conn + "_grad", produced[0], produced[1])
+            return
+        self.n += 1
+        tmp, _ = self.sdfg.add_transient("%s_full_%s" % (self.group.label, conn), self.od.shape, self.od.dtype)
+        _write(self.ctx, produced[0], produced[1], tmp)
+        rs = _new(self.ctx, "ReduceSum", "%s_%s_grad" % (self.node.label, conn),
+                  axes=list(range(len(self.od.shape) - len(shp))), keepdims=0)
+        _read(self.ctx, tmp, rs, "data")
+        self.group.map_output(conn + "_grad", rs, "reduced")
+
+
+@autoregister_params(op="Mul", name=NAME)
+class HipMulBackward(BackwardImplementation):
+    """C = A * B: dA = dC * B, dB = dC * A (summed over broadcast dims)."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        return _broadcast_ok(node, state, sdfg)
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        b = _ElementwiseBackward(forward_node, context)
+        req = {}
+        for conn in required_gradients:
+            other = _in_arr(context, forward_node, "B" if conn == "A" else "A")
+            b.finish(conn, b.op("Mul", None, other))
+            req[conn] = conn + "_grad"
+        return b.group, BackwardResult(required_grad_names=req, given_grad_names={"C": "C_grad"})
+
+
+@autoregister_params(op="Sub", name=NAME)
+class HipSubBackward(BackwardImplementation):
+    """C = A - B: dA = dC (passed through when shapes agree), dB = -dC."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        return _broadcast_ok(node, state, sdfg)
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        b = _ElementwiseBackward(forward_node, context)
+        req, passthrough = {}, {}
+        for conn in required_gradients:
+            shp = b.sdfg.arrays[_in_arr(context, forward_node, conn)].shape
+            if conn == "A" and tuple(shp) == tuple(b.od.shape):
+                passthrough[conn] = "C"
+                continue
+            if conn == "A":
+                rs = _new(context, "ReduceSum", "%s_A_grad" % forward_node.label,
+                          axes=list(range(len(b.od.shape) - len(shp))), keepdims=0)
+                rs.add_in_connector("data")
+                b.group.map_input("C_grad", rs, "data")
+                b.group.map_output("A_grad", rs, "reduced")
+            else:
+                b.finish(conn, b.op("Mul", None, _minus_one(context, b.od.dtype)))
+            req[conn] = conn + "_grad"
+        return b.group, BackwardResult(required_grad_names=req, given_grad_names={"C": "C_grad"},
+                                       passthrough=passthrough)
+
+
+@autoregister_params(op="Div", name=NAME)
+class HipDivBackward(BackwardImplementation):
+    """C = A / B: dA = dC / B, dB = -(dC * C) / B with the forward output C."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        return _broadcast_ok(node, state, sdfg)
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        b = _ElementwiseBackward(forward_node, context)
+        den = _in_arr(context, forward_node, "B")
+        req = {}
+        for conn in required_gradients:
+            if conn == "A":
+                b.finish(conn, b.op("Div", None, den))
+            else:
+                t = b.op("Mul", None, b.out)
+                t = b.op("Div", t, den)
+                b.finish(conn, b.op("Mul", t, _minus_one(context, b.od.dtype)))
+            req[conn] = conn + "_grad"
+        return b.group, BackwardResult(required_grad_names=req, given_grad_names={"C": "C_grad"})
+
+
 # ----------------------------------------------------------------------------- convolution
 @autoregister_params(op="Conv", name=NAME)
 class HipConvBackward(BackwardImplementation):

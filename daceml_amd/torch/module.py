@@ -158,6 +158,9 @@ class DaceModule(nn.Module):
 
         grads: Dict[str, str] = {}
         if self.backward:
+            # differentiation works on contractions (as in the reference, where PureMatMul / PureGemm have expanded
+            # to Einsum nodes before the backward pass is generated); a no-op after auto_optimize
+            fusion.lower_matmul(sdfg)
             # gradients for every input that is not a buffer or skipped, and every parameter that requires one
             # (module.py:333-346)
             buffers = {n for n, _ in self.model.named_buffers()}

@@ -372,7 +372,7 @@ def fuse_gate_into_conv(sdfg: SDFG) -> int:
 
 # ----------------------------------------------------------------------------- contractions
 def lower_matmul(sdfg: SDFG) -> int:
-    """MatMul -> Einsum with the equation PureMatMul builds (pure_implementations.py:132-191)."""
+    """MatMul -> Einsum with the equation PureMatMul builds (pure_implementations.py:132-191); Gemm likewise."""
     count = 0
     for state in sdfg.states():
         for mm in [n for n in state.nodes() if _is_op(n, "MatMul")]:
@@ -384,6 +384,28 @@ def lower_matmul(sdfg: SDFG) -> int:
             eq = C.matmul_equation(ra, rb)
             _remove_node(state, mm)
             _add_node(sdfg, state, "Einsum", mm.label, {"Inputs__0": a, "Inputs__1": b}, {"Output": y}, equation=eq)
+            count += 1
+        # Gemm (how nn.Linear on a 2-D input is exported: transB = 1, C = the bias) -> the contraction PureGemm builds
+        # (pure_implementations.py:455-553) with alpha and the bias vector folded in
+        for gm in [n for n in state.nodes() if _is_op(n, "Gemm")]:
+            a, b, c = _in_array(state, gm, "A"), _in_array(state, gm, "B"), _in_array(state, gm, "C")
+            y = _out_array(state, gm, "Y")
+            if len(sdfg.arrays[a].shape) != 2 or len(sdfg.arrays[b].shape) != 2:
+                continue
+            n_out = sdfg.arrays[y].shape[-1]
+            if c is not None and not (float(gm.beta) == 1.0 and sdfg.arrays[c].total_size == n_out
+                                      and sdfg.arrays[c].shape[-1] == n_out and sdfg.arrays[c].is_contiguous()):
+                continue
+            eq = "%s,%s->ij" % ("ki" if gm.transA else "ik", "jk" if gm.transB else "kj")
+            ins = {"Inputs__0": a, "Inputs__1": b}
+            if c is not None:
+                ins["Bias"] = c
+            _remove_node(state, gm)
+            if c is None and float(gm.alpha) == 1.0:
+                _add_node(sdfg, state, "Einsum", gm.label, ins, {"Output": y}, equation=eq)
+            else:
+                _add_node(sdfg, state, "FusedEinsum", gm.label, ins, {"Output": y}, equation=eq, alpha=float(gm.alpha),
+                          activation="none", accumulate=0)
             count += 1
     return count
 

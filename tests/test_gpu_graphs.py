@@ -176,3 +176,36 @@ def test_selection_levels_and_refusal():
         expand_onnx_nodes(sdfg)
     node.implementation = None
     assert expand_onnx_nodes(sdfg) == 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_elementwise_backward_with_broadcast(dtype):
+    """Mul / Sub / Div reversed as elementwise nodes plus a reduction for the broadcast operand (what the reference
+    gets from symbolic tasklet reversal and ReverseReduce), against autograd."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    g = graphs.GraphBuilder("elementwise_backward", dtype)
+    a, b, c = g.input("a", (6, 5, 32)), g.input("b", (32, )), g.input("c", (6, 5, 32))
+    m = g.node("Mul", {"A": a, "B": b}, {"C": (6, 5, 32)}, label="m")["C"]
+    s_ = g.node("Sub", {"A": m, "B": c}, {"C": (6, 5, 32)}, label="s")["C"]
+    d = g.node("Div", {"A": s_, "B": b}, {"C": (6, 5, 32)}, label="d")["C"]
+    t = g.node("Sub", {"A": b, "B": d}, {"C": (6, 5, 32)}, label="t")["C"]     # broadcast operand first
+    g.output(t, "y")
+    grads = add_backward_pass(g.sdfg, g.state, ["y"], ["a", "b", "c"])
+    assert grads == {"a": "gradient_a", "b": "gradient_b", "c": "gradient_c"}
+    prog = _compile(g.sdfg)
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    av = rng(1).standard_normal((6, 5, 32)).astype(npdt)
+    bv = (rng(2).uniform(0.5, 1.5, 32)).astype(npdt)
+    cv = rng(3).standard_normal((6, 5, 32)).astype(npdt)
+    dyv = rng(4).standard_normal((6, 5, 32)).astype(npdt)
+    out = {n: torch.empty(s, dtype=dtype, device="cuda") for n, s in
+           (("y", (6, 5, 32)), ("gradient_a", (6, 5, 32)), ("gradient_b", (32, )), ("gradient_c", (6, 5, 32)))}
+    prog(a=dev(av), b=dev(bv), c=dev(cv), gradient_y=dev(dyv), **out)
+    ta, tb, tc = (torch.tensor(v.astype(np.float64), requires_grad=True) for v in (av, bv, cv))
+    ty = tb - (ta * tb - tc) / tb
+    ty.backward(torch.tensor(dyv.astype(np.float64)))
+    assert_close(host(out["y"]), ty.detach().numpy(), dtype, "forward")
+    for name, want in (("a", ta.grad), ("b", tb.grad), ("c", tc.grad)):
+        kw = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(atol=0.1 if name == "b" else 1e-2)
+        assert_close(host(out["gradient_" + name]), want.numpy(), dtype, "gradient of " + name, **kw)

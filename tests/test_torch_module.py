@@ -367,3 +367,47 @@ def test_batchnorm_module_training_and_eval():
     net_eval = copy.deepcopy(net).eval()
     we = DaceModule(copy.deepcopy(net_eval))
     assert_close(host(we(x)), host(net_eval(x)), torch.float32, "eval forward", rtol=1e-4, atol=1e-5)
+
+
+class TwoInTwoOut(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc = nn.Linear(16, 16)
+
+    def forward(self, a, b):
+        h = self.fc(a) * torch.sigmoid(b)
+        return h + a, torch.tanh(h)
+
+
+@pytest.mark.gpu
+def test_module_with_two_inputs_two_outputs_and_a_skipped_gradient():
+    """Several inputs and outputs, one input excluded from differentiation (`inputs_to_skip`,
+    daceml/torch/module.py:59-60): its gradient comes back as None, everything else matches autograd."""
+    torch.manual_seed(6)
+    net = TwoInTwoOut().cuda()
+    ref = copy.deepcopy(net).double()
+    probe = DaceModule(copy.deepcopy(net))
+    model = probe._import((torch.randn(4, 16, device="cuda"), torch.randn(4, 16, device="cuda")))
+    assert len(model.inputs) == 2 + 2 and model.outputs == ["__return_0", "__return_1"]
+    skip = model.inputs[1]
+    w = DaceModule(net, backward=True, inputs_to_skip=[skip])
+    a = torch.randn(4, 16, device="cuda", requires_grad=True)
+    b = torch.randn(4, 16, device="cuda", requires_grad=True)
+    ar, br = a.detach().double().requires_grad_(True), b.detach().double().requires_grad_(True)
+    y0, y1 = w(a, b)
+    r0, r1 = ref(ar, br)
+    assert_close(host(y0), r0.detach().cpu().numpy(), torch.float32, "first output", rtol=1e-4, atol=1e-5)
+    assert_close(host(y1), r1.detach().cpu().numpy(), torch.float32, "second output", rtol=1e-4, atol=1e-5)
+    g0, g1 = torch.randn_like(y0), torch.randn_like(y1)
+    torch.autograd.backward([y0, y1], [g0, g1])
+    torch.autograd.backward([r0, r1], [g0.double(), g1.double()])
+    assert b.grad is None
+    assert_close(host(a.grad), ar.grad.cpu().numpy(), torch.float32, "gradient of the first input", rtol=1e-4, atol=1e-5)
+    for (n, p_), (_, pr) in zip(net.named_parameters(), ref.named_parameters()):
+        assert_close(host(p_.grad), pr.grad.cpu().numpy(), torch.float32, "gradient of " + n, rtol=1e-4, atol=1e-5)
+    # only one of the two output gradients given: the other counts as zero
+    a2 = a.detach().clone().requires_grad_(True)
+    ar2 = a.detach().double().requires_grad_(True)
+    w(a2, b.detach())[1].sum().backward()
+    ref(ar2, b.detach().double())[1].sum().backward()
+    assert_close(host(a2.grad), ar2.grad.cpu().numpy(), torch.float32, "partial output gradient", rtol=1e-4, atol=1e-5)
