@@ -1021,12 +1021,14 @@ def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True,
     stats["gelu"] = fuse_gelu(sdfg)
     stats["layernorm"] = fuse_layernorm(sdfg)
     stats["swish"] = fuse_swish(sdfg)
-    stats["conv_activation"] = fuse_conv_activation(sdfg)
+    # a Conv with a folded activation, GatedConv and SkipLayerNormalization have no backward implementation: graphs that
+    # will be differentiated keep those nodes apart
+    stats["conv_activation"] = 0 if training else fuse_conv_activation(sdfg)
     stats["gated_conv"] = 0 if training else fuse_gate_into_conv(sdfg)
     stats["matmul_to_einsum"] = lower_matmul(sdfg)
     stats["views"] = fold_views(sdfg)
     stats["epilogues"] = fuse_epilogues(sdfg, keep_preactivation=training, activation_in_epilogue=gelu_epilogue)
-    stats["skip_layernorm"] = fuse_skip_layernorm(sdfg)
+    stats["skip_layernorm"] = 0 if training else fuse_skip_layernorm(sdfg)
     stats["attention"] = fuse_attention(sdfg) if attention else 0
     # with a backward pass to come, grouping waits until after autodiff (optimize_backward): the backward
     # implementations differentiate the single contractions

@@ -398,6 +398,32 @@ def test_attention_fusion_roles_and_graph():
     assert fusion.auto_optimize(s32)["attention"] == 0
 
 
+def test_training_graphs_keep_differentiable_nodes():
+    """Conv + activation stays two nodes when a backward pass is to come (ConvGrad differentiates a plain Conv), and
+    the backward pass then builds."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.transformation import fusion
+
+    def build():
+        g = graphs.GraphBuilder("convnet", torch.float32)
+        x = g.input("x", (2, 3, 8, 8))
+        g.input("w", (4, 3, 3, 3))
+        g.input("b", (4, ))
+        y = g.node("Conv", {"X": x, "W": "w", "B": "b"}, {"Y": (2, 4, 6, 6)}, label="conv", kernel_shape=[3, 3])["Y"]
+        r = g.node("Relu", {"X": y}, {"Y": (2, 4, 6, 6)}, label="relu")["Y"]
+        g.output(r, "y")
+        return g
+
+    g = build()
+    assert fusion.auto_optimize(g.sdfg, training=False)["conv_activation"] == 1
+    g = build()
+    assert fusion.auto_optimize(g.sdfg, training=True)["conv_activation"] == 0
+    grads = add_backward_pass(g.sdfg, g.state, ["y"], ["x", "w", "b"])
+    assert grads == {"x": "gradient_x", "w": "gradient_w", "b": "gradient_b"}
+    assert sorted(n.schema.name for n in g.sdfg.states()[1].library_nodes()) == ["ConvGrad", "ReluGrad"]
+
+
 def test_fusion_leaves_non_matching_chains_alone():
     from daceml_amd import graphs
     from daceml_amd.transformation import fusion
