@@ -313,11 +313,7 @@ class HipAddBackward(BackwardImplementation):
             oshape = sdfg.arrays[out].shape
             for conn in ("A", "B"):
                 arr = next(iter(state.in_edges_by_connector(node, conn))).data.data
-                shp = sdfg.arrays[arr].shape
-                if shp == oshape:
-                    continue
-                k = len(shp)
-                if not (k <= len(oshape) and tuple(oshape[len(oshape) - k:]) == tuple(shp)):
+                if _reduction_for(sdfg.arrays[arr].shape, oshape) is False:
                     return False
             return True
         except StopIteration:
@@ -331,11 +327,11 @@ class HipAddBackward(BackwardImplementation):
         req, passthrough = {}, {}
         for conn in required_gradients:
             shp = sdfg.arrays[_in_arr(context, forward_node, conn)].shape
-            if shp == oshape:
+            red = _reduction_for(shp, oshape)
+            if red is None:
                 passthrough[conn] = "C"
             else:
-                rs = _new(context, "ReduceSum", "%s_%s_grad" % (forward_node.label, conn),
-                          axes=list(range(len(oshape) - len(shp))), keepdims=0)
+                rs = _new(context, "ReduceSum", "%s_%s_grad" % (forward_node.label, conn), axes=red[0], keepdims=red[1])
                 rs.add_in_connector("data")
                 group.map_input("C_grad", rs, "data")
                 group.map_output(conn + "_grad", rs, "reduced")
@@ -344,10 +340,34 @@ class HipAddBackward(BackwardImplementation):
                                      passthrough=passthrough)
 
 
+def _reduction_for(shp, oshape):
+    """How the gradient of a broadcast operand is summed back: (axes, keepdims), None when the shapes agree, or
+    False when this form of broadcast is not covered. Covered: the operand has the output's trailing dims (bias
+    vectors), or the output's rank with one adjacent run of size-1 dims (a per-channel gate [N, C, 1, 1])."""
+    shp, oshape = tuple(shp), tuple(oshape)
+    if shp == oshape:
+        return None
+    k = len(shp)
+    if k < len(oshape) and oshape[len(oshape) - k:] == shp:
+        return list(range(len(oshape) - k)), 0
+    if k == len(oshape) and all(a == b or a == 1 for a, b in zip(shp, oshape)):
+        axes = [i for i, (a, b) in enumerate(zip(shp, oshape)) if a == 1 and b != 1]
+        if axes and axes == list(range(axes[0], axes[-1] + 1)):
+            return axes, 1
+    return False
+
+
 def _broadcast_ok(node, state, sdfg) -> bool:
-    """Operands have the output's shape or its trailing dims (the broadcasts the exporter emits: bias vectors,
-    per-row scalars come as [.., 1] and are not covered)."""
-    return HipAddBackward.backward_can_be_applied(node, state, sdfg)
+    try:
+        out = next(iter(state.out_edges_by_connector(node, "C"))).data.data
+        oshape = sdfg.arrays[out].shape
+        for conn in ("A", "B"):
+            arr = next(iter(state.in_edges_by_connector(node, conn))).data.data
+            if _reduction_for(sdfg.arrays[arr].shape, oshape) is False:
+                return False
+        return True
+    except StopIteration:
+        return False
 
 
 def _minus_one(ctx, dtype) -> str:
@@ -392,14 +412,14 @@ class _ElementwiseBackward:
     def finish(self, conn, produced):
         """Route a full-shape gradient (node, connector) to input `conn`, reducing over broadcast dims if needed."""
         shp = self.sdfg.arrays[_in_arr(self.ctx, self.node, conn)].shape
-        if tuple(shp) == tuple(self.od.shape):
+        red = _reduction_for(shp, self.od.shape)
+        if red is None:
             self.group.map_output(conn + "_grad", produced[0], produced[1])
             return
         self.n += 1
         tmp, _ = self.sdfg.add_transient("%s_full_%s" % (self.group.label, conn), self.od.shape, self.od.dtype)
         _write(self.ctx, produced[0], produced[1], tmp)
-        rs = _new(self.ctx, "ReduceSum", "%s_%s_grad" % (self.node.label, conn),
-                  axes=list(range(len(self.od.shape) - len(shp))), keepdims=0)
+        rs = _new(self.ctx, "ReduceSum", "%s_%s_grad" % (self.node.label, conn), axes=red[0], keepdims=red[1])
         _read(self.ctx, tmp, rs, "data")
         self.group.map_output(conn + "_grad", rs, "reduced")
 
@@ -435,12 +455,12 @@ class HipSubBackward(BackwardImplementation):
         req, passthrough = {}, {}
         for conn in required_gradients:
             shp = b.sdfg.arrays[_in_arr(context, forward_node, conn)].shape
-            if conn == "A" and tuple(shp) == tuple(b.od.shape):
+            red = _reduction_for(shp, b.od.shape)
+            if conn == "A" and red is None:
                 passthrough[conn] = "C"
                 continue
             if conn == "A":
-                rs = _new(context, "ReduceSum", "%s_A_grad" % forward_node.label,
-                          axes=list(range(len(b.od.shape) - len(shp))), keepdims=0)
+                rs = _new(context, "ReduceSum", "%s_A_grad" % forward_node.label, axes=red[0], keepdims=red[1])
                 rs.add_in_connector("data")
                 b.group.map_input("C_grad", rs, "data")
                 b.group.map_output("A_grad", rs, "reduced")
@@ -472,6 +492,28 @@ class HipDivBackward(BackwardImplementation):
                 b.finish(conn, b.op("Mul", t, _minus_one(context, b.od.dtype)))
             req[conn] = conn + "_grad"
         return b.group, BackwardResult(required_grad_names=req, given_grad_names={"C": "C_grad"})
+
+
+@autoregister_params(op="GlobalAveragePool", name=NAME)
+class HipGlobalAveragePoolBackward(BackwardImplementation):
+    """Y = mean of X over the spatial dims (img_op_implementations.py:415-417): dX = dY / (H*W), broadcast back over
+    them — one ScaledExpand node."""
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        sdfg = context.forward_sdfg
+        xd = sdfg.arrays[_in_arr(context, forward_node, "X")]
+        count = 1
+        for e in xd.shape[2:]:
+            count *= e
+        name = "%s_inv_count" % forward_node.label
+        sdfg.add_array(name, (), xd.dtype)
+        sdfg.add_constant(name, torch.tensor(1.0 / count, dtype=xd.dtype))
+        sdfg.constants_exact[name] = 1.0 / count
+        g = _new(context, "ScaledExpand", forward_node.label + "_backward")
+        g.add_in_connector("X")
+        _read(context, name, g, "Scale")
+        g.add_out_connector("Y")
+        return g, BackwardResult(required_grad_names={"X": "Y"}, given_grad_names={"Y": "X"})
 
 
 # ----------------------------------------------------------------------------- convolution

@@ -55,7 +55,8 @@ def render_tasklet_code(tasklet: T.HipTasklet, conn_ptr=lambda c: "_" + c):
             elif isinstance(a, T.PtrArray):
                 name = "__dml_ptrs%d" % n
                 n += 1
-                lines.append("const void* %s[] = {%s};" % (name, ", ".join(conn_ptr(c) for c in a.conns)))
+                # void*[]: converts to both `const void* const*` (inputs) and `void* const*` (outputs)
+                lines.append("void* %s[] = {%s};" % (name, ", ".join("(void*)" + conn_ptr(c) for c in a.conns)))
                 args.append(name)
             elif isinstance(a, T.Struct):
                 name = "__dml_desc%d" % n

@@ -150,6 +150,9 @@ SCHEMAS = [
     # backward nodes emitted by the "hip" BackwardImplementations (names follow the ONNX Runtime
     # training contrib ops)
     _schema("SoftmaxGrad", "dY Y", "dX", since=1, axis=-1),
+    # Y = broadcast(X) * Scale to the shape of Y's descriptor (X has Y's rank with extents equal or 1; Scale is one
+    # element): the reverse of a mean / sum reduction (ReverseReduce, daceml/autodiff/implementations/dace_nodes.py:13-105)
+    _schema("ScaledExpand", "X Scale", "Y", since=1),
     _schema("BatchNormalizationGrad", "dY X scale saved_mean saved_var", "dX? dscale? dB?", since=1, epsilon=1e-5),
     _schema("LayerNormalizationGrad", "Y_grad X scale mean inv_std_var", "X_grad scale_grad bias_grad", since=1,
             axis=-1),

@@ -1342,3 +1342,30 @@ class HipEinsumSum(ONNXForward):
         extra = [res] if res is not None else []
         return _tasklet(node, state, [call], flops=plan.flops * n,
                         bytes_moved=sum(_nbytes(a[i], b[i]) for i in range(n)) + _nbytes(out, *extra), kind="gemm")
+
+
+@op_implementation(op="ScaledExpand", name=IMPL)
+class HipScaledExpand(ONNXForward):
+    """Broadcast X along its size-1 dims to Y's shape and multiply by a one-element Scale: what ReverseReduce
+    (daceml/autodiff/implementations/dace_nodes.py:13-105) does for a Sum reduction, times the 1/n of a mean —
+    one pass of the broadcasting elementwise kernel."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, sc, y = ins["X"], ins["Scale"], outs["Y"]
+            return (_float_ok(x, sc, y) and x.dtype == y.dtype == sc.dtype and sc.total_size == 1 and y.is_contiguous()
+                    and x.is_contiguous() and len(x.shape) == len(y.shape) <= L.MAX_DIMS
+                    and all(a == b or a == 1 for a, b in zip(x.shape, y.shape)))
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        x, y = ins["X"], outs["Y"]
+        shape = tuple(y.shape)
+        call = HipCall("dmlhip_binary_" + _SFX[y.dtype],
+                       [I32(L.MUL), Ptr("X"), Ptr("Scale"), Ptr("Y"), I32(len(shape)), I64Array(shape),
+                        I64Array(tuple(_bcast_strides(x, shape))), I64Array((0, ) * len(shape)), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=_nbytes(x, y), kind="elementwise")

@@ -411,3 +411,47 @@ def test_module_with_two_inputs_two_outputs_and_a_skipped_gradient():
     w(a2, b.detach())[1].sum().backward()
     ref(ar2, b.detach().double())[1].sum().backward()
     assert_close(host(a2.grad), ar2.grad.cpu().numpy(), torch.float32, "partial output gradient", rtol=1e-4, atol=1e-5)
+
+
+class MBConvBN(nn.Module):
+    """MBConv block as efficientnet_pytorch builds it (what tests/autodiff/torch/test_efficientnet_block_backward.py
+    trains): every conv without bias followed by BatchNorm, swish as x * sigmoid(x), squeeze-excite with biases."""
+    def __init__(self, cin=8, mid=32, cout=16, se=4):
+        super().__init__()
+        self.expand, self.bn0 = nn.Conv2d(cin, mid, 1, bias=False), nn.BatchNorm2d(mid)
+        self.dw, self.bn1 = nn.Conv2d(mid, mid, 3, stride=1, padding=1, groups=mid, bias=False), nn.BatchNorm2d(mid)
+        self.se1, self.se2 = nn.Conv2d(mid, se, 1), nn.Conv2d(se, mid, 1)
+        self.proj, self.bn2 = nn.Conv2d(mid, cout, 1, bias=False), nn.BatchNorm2d(cout)
+
+    def forward(self, x):
+        x = self.bn0(self.expand(x))
+        x = x * torch.sigmoid(x)
+        x = self.bn1(self.dw(x))
+        x = x * torch.sigmoid(x)
+        s = nn.functional.adaptive_avg_pool2d(x, 1)
+        s = self.se1(s)
+        s = s * torch.sigmoid(s)
+        s = self.se2(s)
+        x = torch.sigmoid(s) * x
+        return self.bn2(self.proj(x))
+
+
+@pytest.mark.gpu
+def test_mbconv_block_training_through_the_wrapper():
+    torch.manual_seed(7)
+    net = MBConvBN().cuda().train()
+    ref = copy.deepcopy(net).double()
+    w = DaceModule(net, training=True, backward=True)
+    x = torch.randn(4, 8, 12, 12, device="cuda")
+    xs, xr = x.clone().requires_grad_(True), x.double().requires_grad_(True)
+    y, want = w(xs), ref(xr)
+    assert_close(host(y), want.detach().cpu().numpy(), torch.float32, "forward", rtol=2e-4, atol=2e-5)
+    g = torch.randn_like(y)
+    y.backward(g)
+    want.backward(g.double())
+    kinds = {l.kind for l in w.compiled.launches}
+    assert {"batchnorm", "batchnorm_backward", "conv"} <= kinds
+    assert_close(host(xs.grad), xr.grad.cpu().numpy(), torch.float32, "dx", rtol=1e-3, atol=1e-4)
+    for (n, p_), (_, pr) in zip(net.named_parameters(), ref.named_parameters()):
+        scale = max(float(pr.grad.abs().max()), 1.0)
+        assert_close(host(p_.grad), pr.grad.cpu().numpy(), torch.float32, "gradient of " + n, rtol=1e-3, atol=1e-4 * scale)
