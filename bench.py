@@ -208,9 +208,67 @@ def secondary_workload(name, device, steps, warmup, verbose):
                       "launches": launches}))
 
 
+def module_workload(device, steps, warmup):
+    """HuggingFace BertLayer (BERT-large sizes, fp16, no dropout) wrapped in DaceModule: forward + backward through
+    torch.autograd, next to the same module run by PyTorch itself on the same GPU. Includes everything a user of
+    the wrapper pays per call (autograd bookkeeping, output allocation, gradient casts)."""
+    import copy
+    import warnings
+    import torch
+    from transformers import BertConfig
+    from transformers.models.bert.modeling_bert import BertLayer
+    from daceml_amd.torch import DaceModule
+
+    class Layer(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            cfg = BertConfig(hidden_size=H, num_attention_heads=HEADS, intermediate_size=FFN, hidden_dropout_prob=0.0,
+                             attention_probs_dropout_prob=0.0)
+            cfg._attn_implementation = "eager"
+            self.layer = BertLayer(cfg)
+
+        def forward(self, x):
+            out = self.layer(x)
+            return out[0] if isinstance(out, (tuple, list)) else out
+
+    torch.manual_seed(1234)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        eager = Layer().to(device).half().eval()
+        wrapped = DaceModule(copy.deepcopy(eager), backward=True)
+        x = torch.randn(B, S, H, device=device, dtype=torch.float16, requires_grad=True)
+        dy = torch.randn(B, S, H, device=device, dtype=torch.float16)
+        wrapped(x)   # traces, imports, fuses, binds
+
+    def step(mod):
+        x.grad = None
+        for p_ in mod.parameters():
+            p_.grad = None
+        mod(x).backward(dy)
+
+    def timed(mod):
+        for _ in range(warmup):
+            step(mod)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(mod)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    ms, ms_eager = timed(wrapped), timed(eager)
+    what = "HuggingFace BertLayer (BERT-large sizes, B=8 S=512, fp16) forward + backward through DaceModule"
+    print(json.dumps({"metric": what + " ms/iter at 1 GPU", "value": round(ms, 4), "unit": "ms/iter", "n_gpus": 1,
+                      "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+                      "config": {"workload": what, "launches_per_step": len(wrapped.compiled.launches)},
+                      "pytorch_eager_ms": round(ms_eager, 4), "speedup_over_pytorch_eager": round(ms_eager / ms, 2),
+                      "optimization_stats": wrapped.optimization_stats}))
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="bert_fwd_bwd", choices=["bert_fwd_bwd", "bert_fwd", "nodes", "mbconv", "conv"],
+    ap.add_argument("--workload", default="bert_fwd_bwd", choices=["bert_fwd_bwd", "bert_fwd", "nodes", "mbconv", "conv", "module_bert"],
                     help="bert_fwd_bwd is the headline (default); the others are BASELINE.json's remaining configs")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
@@ -230,6 +288,8 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
+    if a.workload == "module_bert":
+        return module_workload(device, a.steps, a.warmup)
     if a.workload != "bert_fwd_bwd":
         return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose)
 
