@@ -24,7 +24,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # --pmc WRITE_SIZE (one run each, of `bench.py --steps 3 --warmup 2 --no-cpu-baseline --calibrate-copy`), each
 # scaled by what the same counter reads for the 128 MiB copy kernel of --calibrate-copy (FETCH_SIZE x 2.000,
 # WRITE_SIZE x 1.000). Measured, not computed here: it goes stale when the GEMM tiling changes.
-GEMM_TRAFFIC_BYTES_PER_STEP = {"fetched": 867.1e6, "written": 184.6e6}
+GEMM_TRAFFIC_BYTES_PER_STEP = {"fetched": 866.6e6, "written": 184.6e6}
 
 METRIC = "BERT-large encoder layer fp16 fwd+bwd ms/iter at 1 GPU; % MFMA & HBM roofline"
 B, S, H, HEADS, FFN = 8, 512, 1024, 16, 4096
