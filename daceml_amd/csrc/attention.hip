@@ -239,23 +239,22 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
 
         // ---- online softmax over the key axis; the lane's query is lane%32, its keys are
         // 64*j + 32*blk + 8*(e/4) + 4*h + e%4
-        float x[2][16];
+        // (scale > 0, checked on the host: the maximum is taken over the raw scores and scaled once, and scale and
+        // shift of the exponent's argument are one fused multiply-add per score)
         float mt = -INFINITY;
         const bool ragged = (j + 1) * 64 > a.seq_k;
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                float v = sacc[blk][e] * a.scale_log2;
                 if (ragged) {
                     const int key = j * 64 + blk * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-                    if (key >= a.seq_k) v = -INFINITY;
+                    if (key >= a.seq_k) sacc[blk][e] = -INFINITY;
                 }
-                x[blk][e] = v;
-                mt = fmaxf(mt, v);
+                mt = fmaxf(mt, sacc[blk][e]);
             }
         mt = cross_half_max(mt);
-        const float m_new = fmaxf(m_run, mt);
+        const float m_new = fmaxf(m_run, mt * a.scale_log2);
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         m_run = m_new;
         float psum = 0.f;
@@ -264,15 +263,18 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const float p = __builtin_amdgcn_exp2f(x[blk][e] - m_new);
+                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], a.scale_log2, -m_new));
                 psum += p;
                 pf[blk * 2 + (e >> 3)][e & 7] = (_Float16)p;
             }
         l_run = l_run * alpha + psum;
+        // once the running maxima have settled every alpha is 1 and the accumulators need no rescaling
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
+            for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) oacc[blk][e] *= alpha;
+                for (int e = 0; e < 16; ++e) oacc[blk][e] *= alpha;
+        }
 
         // ---- O^T += V^T P^T
         wait_lgkm<0>();
@@ -608,6 +610,7 @@ int fill_args(const dmlhip_attention_desc* d, const dmlhip_attention_desc* g, At
             else { a.dqs[i] = s4[0]; a.dks[i] = s4[1]; a.dvs[i] = s4[2]; a.dos[i] = s4[3]; }
         }
     }
+    DML_REQUIRE(d->scale > 0.f, DMLHIP_ERR_SHAPE, "%s: the scale must be positive, got %g", what, (double)d->scale);
     a.scale = d->scale;
     a.scale_log2 = d->scale * 1.44269504088896340736f;
     return 0;

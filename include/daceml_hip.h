@@ -293,7 +293,7 @@ int dmlhip_conv2d_backward_weight_f32(const dmlhip_conv2d_desc* d, const void* x
  * Tensors are [batch0, batch1, seq, head_dim] views: element strides for batch0, batch1 and
  * seq are given per tensor (multiples of 8), head_dim is contiguous and must be 64.
  * lse (optional in forward, required by backward): fp32 [batch0, batch1, seq_q] dense,
- * lse = log(sum_k exp(scale * q.k)) per query row. */
+ * lse = log(sum_k exp(scale * q.k)) per query row. scale must be positive. */
 typedef struct dmlhip_attention_desc {
     int64_t batch[2];
     int64_t seq_q, seq_k, head_dim;
