@@ -85,6 +85,55 @@ def test_argument_errors_need_no_gpu(lib):
     assert (oh.value, ow.value) == (4, 4)
 
 
+def test_argument_errors_of_the_grouped_and_fused_entry_points(lib):
+    """Grouped / K-summed / row-sum contractions, attention and BatchNormalization validate on the host too."""
+    from daceml_amd import _lib as L
+    p = ctypes.c_void_p(32)
+    table = (ctypes.c_void_p * 4)(32, 32, 32, 32)
+    holes = (ctypes.c_void_p * 4)(32, 0, 32, 32)
+    d = L.GemmDesc()
+    d.m, d.n, d.k = 128, 128, 64
+    d.batch[0] = d.batch[1] = d.batch[2] = 1
+    d.a_stride_m, d.a_stride_k, d.b_stride_k, d.b_stride_n, d.c_stride_m = 64, 1, 1, 64, 128
+    d.alpha = 1.0
+    ref = ctypes.byref(d)
+    assert lib.dmlhip_gemm_f16_grouped(ref, 0, table, table, table, None, None, 0, None) == L.ERR_SHAPE
+    assert lib.dmlhip_gemm_f16_grouped(ref, 5, table, table, table, None, None, 0, None) == L.ERR_SHAPE
+    assert lib.dmlhip_gemm_f16_grouped(ref, 2, None, table, table, None, None, 0, None) == L.ERR_NULL
+    assert lib.dmlhip_gemm_f16_grouped(ref, 3, table, table, holes, None, None, 0, None) == L.ERR_NULL
+    assert lib.dmlhip_gemm_f16_ksum(ref, 5, table, table, p, None, None, None) == L.ERR_SHAPE
+    assert lib.dmlhip_gemm_f16_ksum(ref, 3, table, holes, p, None, None, None) == L.ERR_NULL
+    assert lib.dmlhip_gemm_f16_ksum(ref, 2, table, table, None, None, None, None) == L.ERR_NULL
+    d.beta = 1.0
+    assert lib.dmlhip_gemm_f16_ksum(ref, 2, table, table, p, None, None, None) == L.ERR_UNSUPPORTED
+    d.beta = 0.0
+    # row sums: A must be a dense [k, m] matrix, the product unbatched, the sums fp16 / fp32
+    assert lib.dmlhip_gemm_f16_grouped_asum(ref, 1, table, table, table, table, L.F32, None, 0, None) == L.ERR_UNSUPPORTED
+    d.a_stride_m, d.a_stride_k = 1, 128
+    assert lib.dmlhip_gemm_f16_grouped_asum(ref, 1, table, table, table, table, 7, None, 0, None) == L.ERR_ENUM
+    assert lib.dmlhip_gemm_f16_grouped_asum(ref, 1, table, table, table, None, L.F32, None, 0, None) == L.ERR_NULL
+    d.batch[1] = 2
+    assert lib.dmlhip_gemm_f16_grouped_asum(ref, 1, table, table, table, table, L.F32, None, 0, None) == L.ERR_SHAPE
+    d.batch[1] = 1
+    assert lib.dmlhip_gemm_f16_grouped_asum_workspace_bytes(ref) >= 0
+    a = L.AttentionDesc()
+    a.batch[0], a.batch[1], a.seq_q, a.seq_k, a.head_dim = 1, 2, 64, 64, 64
+    for arr in (a.q_stride, a.k_stride, a.v_stride, a.o_stride):
+        arr[0], arr[1], arr[2] = 2 * 64 * 64, 64 * 64, 64
+    a.scale = 0.125
+    assert lib.dmlhip_attention_f16(ctypes.byref(a), p, p, None, p, None, None) == L.ERR_NULL
+    a.scale = -1.0
+    assert lib.dmlhip_attention_f16(ctypes.byref(a), p, p, p, p, None, None) == L.ERR_SHAPE
+    assert "scale" in L.last_error()
+    a.scale, a.head_dim = 0.125, 32
+    assert lib.dmlhip_attention_f16(ctypes.byref(a), p, p, p, p, None, None) == L.ERR_UNSUPPORTED
+    assert lib.dmlhip_batchnorm_inference_f32(p, p, p, p, p, p, 2, 0, 16, 1e-5, None) == L.ERR_SHAPE
+    assert lib.dmlhip_batchnorm_training_f16(p, p, p, p, p, p, p, p, p, p, 2, 3, 16, 1e-5, 0.9, None, 0, None) == \
+        L.ERR_WORKSPACE
+    assert lib.dmlhip_batchnorm_backward_f32(p, p, p, p, p, None, None, None, 2, 3, 16, 1e-5, p, 1 << 20, None) == L.ERR_NULL
+    assert lib.dmlhip_batchnorm_workspace_bytes(8, 3, 1024) > 0
+
+
 def test_kernels_refuse_host_tensors():
     from daceml_amd import kernels as K
     with pytest.raises(ValueError):
