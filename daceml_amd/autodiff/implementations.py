@@ -494,6 +494,60 @@ class HipDivBackward(BackwardImplementation):
         return b.group, BackwardResult(required_grad_names=req, given_grad_names={"C": "C_grad"})
 
 
+def _scalar_constant(ctx, name: str, value: float, dtype) -> str:
+    sdfg = ctx.forward_sdfg
+    if name not in sdfg.arrays:
+        sdfg.add_array(name, (), dtype)
+        sdfg.add_constant(name, torch.tensor(value, dtype=dtype))
+        sdfg.constants_exact[name] = float(value)
+    return name
+
+
+def _make_reduce_backward(op: str, mean: bool):
+    class _B(BackwardImplementation):
+        @staticmethod
+        def backward(forward_node, context, given_gradients, required_gradients):
+            sdfg = context.forward_sdfg
+            xd = sdfg.arrays[_in_arr(context, forward_node, "data")]
+            nd = len(xd.shape)
+            axes = sorted(a % nd for a in (forward_node.axes if forward_node.axes is not None else range(nd)))
+            count = 1
+            for a in axes:
+                count *= xd.shape[a]
+            kept = tuple(1 if i in axes else d for i, d in enumerate(xd.shape))
+            scale = _scalar_constant(context, "%s_backward_scale" % forward_node.label, 1.0 / count if mean else 1.0,
+                                     xd.dtype)
+            g = _new(context, "ScaledExpand", forward_node.label + "_backward", x_shape=list(kept))
+            g.add_in_connector("X")
+            _read(context, scale, g, "Scale")
+            g.add_out_connector("Y")
+            return g, BackwardResult(required_grad_names={"data": "Y"}, given_grad_names={"reduced": "X"})
+
+    _B.__name__ = "Hip%sBackward" % op
+    _B.__doc__ = ("The gradient of %s is the given gradient broadcast back over the reduced axes%s (ReverseReduce, "
+                  "daceml/autodiff/implementations/dace_nodes.py:13-105): one ScaledExpand node." %
+                  (op, ", divided by their extent" if mean else ""))
+    return autoregister_params(op=op, name=NAME)(_B)
+
+
+HipReduceSumBackward = _make_reduce_backward("ReduceSum", False)
+HipReduceMeanBackward = _make_reduce_backward("ReduceMean", True)
+
+
+@autoregister_params(op="Transpose", name=NAME)
+class HipTransposeBackward(BackwardImplementation):
+    """The gradient of a Transpose is the Transpose of the gradient with the inverse permutation."""
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        nd = len(context.forward_sdfg.arrays[_in_arr(context, forward_node, "data")].shape)
+        perm = list(reversed(range(nd))) if forward_node.perm is None else [p % nd for p in forward_node.perm]
+        inverse = [perm.index(i) for i in range(nd)]
+        g = _new(context, "Transpose", forward_node.label + "_backward", perm=inverse)
+        g.add_in_connector("data")
+        g.add_out_connector("transposed")
+        return g, BackwardResult(required_grad_names={"data": "transposed"}, given_grad_names={"transposed": "data"})
+
+
 @autoregister_params(op="GlobalAveragePool", name=NAME)
 class HipGlobalAveragePoolBackward(BackwardImplementation):
     """Y = mean of X over the spatial dims (img_op_implementations.py:415-417): dX = dY / (H*W), broadcast back over
@@ -505,10 +559,7 @@ class HipGlobalAveragePoolBackward(BackwardImplementation):
         count = 1
         for e in xd.shape[2:]:
             count *= e
-        name = "%s_inv_count" % forward_node.label
-        sdfg.add_array(name, (), xd.dtype)
-        sdfg.add_constant(name, torch.tensor(1.0 / count, dtype=xd.dtype))
-        sdfg.constants_exact[name] = 1.0 / count
+        name = _scalar_constant(context, "%s_inv_count" % forward_node.label, 1.0 / count, xd.dtype)
         g = _new(context, "ScaledExpand", forward_node.label + "_backward")
         g.add_in_connector("X")
         _read(context, name, g, "Scale")

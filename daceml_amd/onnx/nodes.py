@@ -152,7 +152,8 @@ SCHEMAS = [
     _schema("SoftmaxGrad", "dY Y", "dX", since=1, axis=-1),
     # Y = broadcast(X) * Scale to the shape of Y's descriptor (X has Y's rank with extents equal or 1; Scale is one
     # element): the reverse of a mean / sum reduction (ReverseReduce, daceml/autodiff/implementations/dace_nodes.py:13-105)
-    _schema("ScaledExpand", "X Scale", "Y", since=1),
+    # x_shape: the shape X is read with when its descriptor has the size-1 dims squeezed out (keepdims = 0)
+    _schema("ScaledExpand", "X Scale", "Y", since=1, x_shape=None),
     _schema("BatchNormalizationGrad", "dY X scale saved_mean saved_var", "dX? dscale? dB?", since=1, epsilon=1e-5),
     _schema("LayerNormalizationGrad", "Y_grad X scale mean inv_std_var", "X_grad scale_grad bias_grad", since=1,
             axis=-1),

@@ -1354,18 +1354,26 @@ class HipScaledExpand(ONNXForward):
         try:
             ins, outs = _descs(node, state, sdfg)
             x, sc, y = ins["X"], ins["Scale"], outs["Y"]
+            xs = HipScaledExpand._x_shape(node, x)
             return (_float_ok(x, sc, y) and x.dtype == y.dtype == sc.dtype and sc.total_size == 1 and y.is_contiguous()
-                    and x.is_contiguous() and len(x.shape) == len(y.shape) <= L.MAX_DIMS
-                    and all(a == b or a == 1 for a, b in zip(x.shape, y.shape)))
+                    and x.is_contiguous() and _prod(xs) == x.total_size and len(xs) == len(y.shape) <= L.MAX_DIMS
+                    and all(a == b or a == 1 for a, b in zip(xs, y.shape)))
         except Exception:
             return False
+
+    @staticmethod
+    def _x_shape(node, x):
+        return tuple(int(d) for d in node.x_shape) if node.x_shape is not None else tuple(x.shape)
 
     @staticmethod
     def forward(node, state, sdfg):
         ins, outs = _descs(node, state, sdfg)
         x, y = ins["X"], outs["Y"]
         shape = tuple(y.shape)
+        xs = HipScaledExpand._x_shape(node, x)
+        dense = C.contiguous_strides(xs)
+        x_strides = tuple(0 if e == 1 else s for e, s in zip(xs, dense))
         call = HipCall("dmlhip_binary_" + _SFX[y.dtype],
                        [I32(L.MUL), Ptr("X"), Ptr("Scale"), Ptr("Y"), I32(len(shape)), I64Array(shape),
-                        I64Array(tuple(_bcast_strides(x, shape))), I64Array((0, ) * len(shape)), Stream()])
+                        I64Array(x_strides), I64Array((0, ) * len(shape)), Stream()])
         return _tasklet(node, state, [call], bytes_moved=_nbytes(x, y), kind="elementwise")

@@ -209,3 +209,35 @@ def test_elementwise_backward_with_broadcast(dtype):
     for name, want in (("a", ta.grad), ("b", tb.grad), ("c", tc.grad)):
         kw = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(atol=0.1 if name == "b" else 1e-2)
         assert_close(host(out["gradient_" + name]), want.numpy(), dtype, "gradient of " + name, **kw)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_reduce_and_transpose_backward(dtype):
+    """ReduceMean (keepdims 1), ReduceSum (keepdims 0) and Transpose reversed with ScaledExpand / Transpose nodes,
+    against autograd: y = transpose(x - mean(x, -1, keepdim)) * sum(x, (0, 1))."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    g = graphs.GraphBuilder("reduce_backward", dtype)
+    x = g.input("x", (4, 6, 16))
+    mean = g.node("ReduceMean", {"data": x}, {"reduced": (4, 6, 1)}, label="mean", axes=[-1], keepdims=1)["reduced"]
+    cen = g.node("Sub", {"A": x, "B": mean}, {"C": (4, 6, 16)}, label="cen")["C"]
+    tr = g.node("Transpose", {"data": cen}, {"transposed": (6, 4, 16)}, label="tr", perm=[1, 0, 2])["transposed"]
+    tot = g.node("ReduceSum", {"data": x}, {"reduced": (16, )}, label="tot", axes=[0, 1], keepdims=0)["reduced"]
+    y = g.node("Mul", {"A": tr, "B": tot}, {"C": (6, 4, 16)}, label="scale")["C"]
+    g.output(y, "y")
+    assert add_backward_pass(g.sdfg, g.state, ["y"], ["x"]) == {"x": "gradient_x"}
+    kinds = sorted(n.schema.name for n in g.sdfg.states()[1].library_nodes())
+    assert kinds.count("ScaledExpand") == 2 and kinds.count("Transpose") == 1
+    prog = _compile(g.sdfg)
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    xv = rng(11).standard_normal((4, 6, 16)).astype(npdt)
+    dyv = rng(12).standard_normal((6, 4, 16)).astype(npdt)
+    out = {"y": torch.empty((6, 4, 16), dtype=dtype, device="cuda"),
+           "gradient_x": torch.empty((4, 6, 16), dtype=dtype, device="cuda")}
+    prog(x=dev(xv), gradient_y=dev(dyv), **out)
+    tx = torch.tensor(xv.astype(np.float64), requires_grad=True)
+    ty = (tx - tx.mean(-1, keepdim=True)).permute(1, 0, 2) * tx.sum((0, 1))
+    ty.backward(torch.tensor(dyv.astype(np.float64)))
+    kw = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=3e-2, atol=0.15)
+    assert_close(host(out["y"]), ty.detach().numpy(), dtype, "forward", **kw)
+    assert_close(host(out["gradient_x"]), tx.grad.numpy(), dtype, "gradient of x", **kw)
