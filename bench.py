@@ -18,6 +18,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # Bytes that cross the L2 <-> fabric boundary for the 11 GEMM launches of one step: rocprofv3 --pmc FETCH_SIZE and
@@ -194,6 +195,11 @@ def secondary_workload(name, device, steps, warmup, verbose):
     top, top_t = max(rows, key=lambda r: r[1])
     if top.kind in ("gemm", "attention") and dtype == "f16":
         roof = {"bound": "mfma", "achieved": round(top.flops / (top_t * 1e-3) / 1e12, 1), "peak": PEAK_FP16_TFLOPS,
+                "unit": "TFLOP/s"}
+    elif dtype == "f32" and top.flops and top.bytes_moved and \
+            top.flops / top.bytes_moved > PEAK_FP32_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9):
+        # more flops per byte than the fp32 matrix pipe can absorb at full HBM rate (the fused expand + depthwise node)
+        roof = {"bound": "mfma", "achieved": round(top.flops / (top_t * 1e-3) / 1e12, 1), "peak": PEAK_FP32_TFLOPS,
                 "unit": "TFLOP/s"}
     else:
         roof = {"bound": "hbm", "achieved": round(top.bytes_moved / (top_t * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,

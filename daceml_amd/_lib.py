@@ -108,6 +108,7 @@ SIGNATURES = {
     "dmlhip_conv2d_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, _P]),
     "dmlhip_conv2d_f16": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, _P]),
     "dmlhip_conv2d_gated_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, _P, _P]),
+    "dmlhip_conv2d_expand_depthwise_f32": (c_int, [POINTER(Conv2dDesc), POINTER(Conv2dDesc), _P, _P, _P, _P, _P, _P, _P]),
     "dmlhip_conv2d_backward_data_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P]),
     "dmlhip_conv2d_backward_weight_workspace_bytes": (c_size_t, [POINTER(Conv2dDesc)]),
     "dmlhip_conv2d_backward_weight_f32": (c_int, [POINTER(Conv2dDesc), _P, _P, _P, _P, c_size_t, _P]),
@@ -126,6 +127,7 @@ SIGNATURES = {
 DEBUG_SIGNATURES = {
     "dmlhip_debug_force_gemm_config": (None, [c_int]),
     "dmlhip_debug_grouped_single_launches": (ctypes.c_longlong, []),
+    "dmlhip_debug_force_fused_strip": (None, [c_int]),
 }
 
 _lib = None

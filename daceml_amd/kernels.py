@@ -449,6 +449,22 @@ def conv2d(x, w, bias=None, strides=(1, 1), pads=(0, 0), dilations=(1, 1), group
     return y
 
 
+def conv2d_expand_depthwise(x, w_pw, b_pw, w_dw, b_dw, stride=1, act_pw: int = L.ACT_NONE, act_dw: int = L.ACT_NONE):
+    """act_dw(depthwise3x3(act_pw(conv1x1(x, w_pw) + b_pw), w_dw, stride, pad 1) + b_dw) in one kernel (fp32): the
+    expanded tensor is never written to memory."""
+    _check(x, w_pw, b_pw, w_dw, b_dw, dtype=torch.float32)
+    x, w_pw, w_dw = _dense(x), _dense(w_pw), _dense(w_dw)
+    d1 = _conv_desc(x.shape, w_pw.shape, (1, 1), (0, 0), (1, 1), 1, act_pw)
+    mid = (x.shape[0], w_pw.shape[0], x.shape[2], x.shape[3])
+    d2 = _conv_desc(mid, w_dw.shape, (stride, stride), (1, 1), (1, 1), w_pw.shape[0], act_dw)
+    oh, ow = conv_out_shape(d2)
+    y = torch.empty((d2.n, d2.m, oh, ow), dtype=x.dtype, device=x.device)
+    L.check(L.load().dmlhip_conv2d_expand_depthwise_f32(ctypes.byref(d1), ctypes.byref(d2), _ptr(x), _ptr(w_pw),
+                                                        _ptr(None if b_pw is None else _dense(b_pw)), _ptr(w_dw),
+                                                        _ptr(None if b_dw is None else _dense(b_dw)), _ptr(y), _stream()))
+    return y
+
+
 def conv2d_backward(x, w, dy, strides=(1, 1), pads=(0, 0), dilations=(1, 1), group=1, need_dx=True, need_dw=True):
     """Returns (dx or None, dw or None); fp32 only."""
     _check(x, w, dy, dtype=torch.float32)

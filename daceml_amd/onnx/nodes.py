@@ -140,6 +140,9 @@ SCHEMAS = [
     # Conv 1x1 whose input is first multiplied by a per-image, per-channel factor Gate [n, c, 1, 1] (squeeze-excite)
     _schema("GatedConv", "X Gate W B?", "Y", since=1, auto_pad="NOTSET", dilations=None, group=1, kernel_shape=None,
             pads=None, strides=None),
+    # pointwise Conv (W_pw [m, c, 1, 1]) + activation followed by a 3x3 depthwise Conv (W_dw [m, 1, 3, 3], padding 1,
+    # stride `strides`) + activation: the expanded tensor of an inverted-residual block never reaches memory
+    _schema("ExpandDepthwiseConv", "X W_pw B_pw? W_dw B_dw?", "Y", since=1, strides=None, act_pw="none", act_dw="none"),
     # several FusedEinsum nodes of identical equation, shapes, strides and scale, independent of each other, in one
     # launch: Output__i = alpha * einsum(equation, A__i, B__i) [+ Bias__i]
     _schema("GroupedEinsum", "A* B* Bias*?", "Output* InputSum*?", since=1, equation=REQUIRED, alpha=1.0),

@@ -1001,6 +1001,67 @@ class HipGatedConv(ONNXForward):
                         bytes_moved=_nbytes(x, ins["Gate"], w, y), kind="conv")
 
 
+@op_implementation(op="ExpandDepthwiseConv", name=IMPL)
+class HipExpandDepthwiseConv(ONNXForward):
+    """Pointwise Conv + activation + 3x3 depthwise Conv + activation (img_op_implementations.py:164-330 twice, with
+    the elementwise ops of pure_implementations.py:556-560 between) in one kernel; the expanded tensor stays in LDS.
+    fp32."""
+    @staticmethod
+    def _descs(node, x, w_pw, w_dw, y):
+        stride = int((node.strides or [1, 1])[0])
+        mid = (x.shape[0], w_pw.shape[0], x.shape[2], x.shape[3])
+        pw, dw = L.Conv2dDesc(), L.Conv2dDesc()
+        pw.n, pw.c, pw.h, pw.w = x.shape
+        pw.m, pw.kh, pw.kw = w_pw.shape[0], 1, 1
+        pw.stride_h = pw.stride_w = pw.dil_h = pw.dil_w = pw.group = 1
+        pw.pad_h = pw.pad_w = 0
+        pw.act = _ACT[node.act_pw]
+        dw.n, dw.c, dw.h, dw.w = mid
+        dw.m, dw.kh, dw.kw = mid[1], 3, 3
+        dw.stride_h = dw.stride_w = stride
+        dw.pad_h = dw.pad_w = dw.dil_h = dw.dil_w = 1
+        dw.group = mid[1]
+        dw.act = _ACT[node.act_dw]
+        oh, ow = (x.shape[2] - 1) // stride + 1, (x.shape[3] - 1) // stride + 1
+        return pw, dw, (x.shape[0], w_pw.shape[0], oh, ow)
+
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, w1, w2, y = ins["X"], ins["W_pw"], ins["W_dw"], outs["Y"]
+            if x.dtype != torch.float32 or not (_float_ok(x, w1, w2, y) and _dense(x, w1, w2, y)):
+                return False
+            if len(x.shape) != 4 or tuple(w1.shape) != (w1.shape[0], x.shape[1], 1, 1):
+                return False
+            if tuple(w2.shape) != (w1.shape[0], 1, 3, 3) or list(node.strides or [1, 1]) not in ([1, 1], [2, 2]):
+                return False
+            for b in ("B_pw", "B_dw"):
+                if b in ins and not (ins[b].dtype == x.dtype and ins[b].is_contiguous()
+                                     and ins[b].total_size == w1.shape[0]):
+                    return False
+            from daceml_amd.transformation.fusion import EXPAND_DEPTHWISE_ACTIVATIONS
+            if (node.act_pw, node.act_dw) not in EXPAND_DEPTHWISE_ACTIVATIONS:
+                return False
+            _, _, yshape = HipExpandDepthwiseConv._descs(node, x, w1, w2, y)
+            return (x.shape[1] % 16 == 0 and w1.shape[0] % 32 == 0 and tuple(y.shape) == yshape
+                    and 32 * 3 * (x.shape[3] + 2) * 4 <= 140 * 1024)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        x, w1, w2, y = ins["X"], ins["W_pw"], ins["W_dw"], outs["Y"]
+        pw, dw, _ = HipExpandDepthwiseConv._descs(node, x, w1, w2, y)
+        call = HipCall("dmlhip_conv2d_expand_depthwise_f32",
+                       [Struct(pw, "dmlhip_conv2d_desc"), Struct(dw, "dmlhip_conv2d_desc"), Ptr("X"), Ptr("W_pw"),
+                        _opt(node, state, "B_pw"), Ptr("W_dw"), _opt(node, state, "B_dw"), Ptr("Y"), Stream()])
+        mid = x.shape[0] * w1.shape[0] * x.shape[2] * x.shape[3]
+        return _tasklet(node, state, [call], flops=2 * mid * x.shape[1] + 18 * y.total_size,
+                        bytes_moved=_nbytes(x, w1, w2, y), kind="conv")
+
+
 @op_implementation(op="ConvGrad", name=IMPL)
 class HipConvGrad(ONNXForward):
     """cudnnConvolutionBackwardData / BackwardFilter / BackwardBias

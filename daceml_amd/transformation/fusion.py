@@ -370,6 +370,62 @@ def fuse_gate_into_conv(sdfg: SDFG) -> int:
     return count
 
 
+def fuse_expand_depthwise(sdfg: SDFG) -> int:
+    """Inverted-residual expansion: a pointwise Conv (+ activation) read only by a 3x3 depthwise Conv (+ activation)
+    becomes one ExpandDepthwiseConv, which keeps the expanded tensor (the widest of the block) out of memory. Runs
+    after fuse_conv_activation. Forward graphs only: a backward pass needs the expanded tensor."""
+    count = 0
+    for state in sdfg.states():
+        for dw in [n for n in state.nodes() if _is_op(n, "Conv")]:
+            mid = _in_array(state, dw, "X")
+            prod = _producer(state, mid)
+            if prod is None or not _is_op(prod[0], "Conv") or not _internal(sdfg, state, mid):
+                continue
+            pw = prod[0]
+            if len(_consumers(state, mid)) != 1:
+                continue
+            x = _in_array(state, pw, "X")
+            xd, md = sdfg.arrays[x], sdfg.arrays[mid]
+            w1, w2 = sdfg.arrays[_in_array(state, pw, "W")], sdfg.arrays[_in_array(state, dw, "W")]
+            if len(xd.shape) != 4 or any(d.dtype != torch.float32 for d in (xd, md, w1, w2)):
+                continue
+            pointwise = (tuple(w1.shape[2:]) == (1, 1) and pw.group == 1 and pw.auto_pad == "NOTSET"
+                         and all(v == 1 for v in (pw.strides or [1, 1])) and not any(pw.pads or [0])
+                         and all(v == 1 for v in (pw.dilations or [1, 1])))
+            strides = list(dw.strides or [1, 1])
+            depthwise = (tuple(w2.shape) == (md.shape[1], 1, 3, 3) and dw.group == md.shape[1]
+                         and dw.auto_pad == "NOTSET" and list(dw.pads or [0]) == [1, 1, 1, 1]
+                         and all(v == 1 for v in (dw.dilations or [1, 1]))
+                         and strides[0] == strides[1] and strides[0] in (1, 2))
+            acts = (getattr(pw, "_activation", "none"), getattr(dw, "_activation", "none"))
+            if not pointwise or not depthwise or acts not in EXPAND_DEPTHWISE_ACTIVATIONS:
+                continue
+            # the kernel's tiling: 16 input channels per step, 32 expanded channels per workgroup, and three expanded
+            # rows of 32 channels must fit LDS
+            if xd.shape[1] % 16 or md.shape[1] % 32 or 32 * 3 * (xd.shape[3] + 2) * 4 > 140 * 1024:
+                continue
+            ins = {"X": x, "W_pw": _in_array(state, pw, "W"), "W_dw": _in_array(state, dw, "W")}
+            for conn, node in (("B_pw", pw), ("B_dw", dw)):
+                bias = _in_array(state, node, "B")
+                if bias is not None:
+                    ins[conn] = bias
+            y = _out_array(state, dw, "Y")
+            label = dw.label
+            _remove_node(state, dw)
+            _remove_node(state, pw)
+            _add_node(sdfg, state, "ExpandDepthwiseConv", label, ins, {"Y": y}, strides=strides, act_pw=acts[0],
+                      act_dw=acts[1])
+            count += 1
+    if count:
+        _drop_unused_arrays(sdfg)
+    return count
+
+
+# (pointwise activation, depthwise activation) pairs the fused kernel is built for
+EXPAND_DEPTHWISE_ACTIVATIONS = {("swish", "swish"), ("none", "none"), ("relu", "relu"), ("swish", "none"),
+                                ("none", "swish"), ("relu", "none"), ("none", "relu")}
+
+
 # ----------------------------------------------------------------------------- contractions
 def lower_matmul(sdfg: SDFG) -> int:
     """MatMul -> Einsum with the equation PureMatMul builds (pure_implementations.py:132-191); Gemm likewise."""
@@ -1025,6 +1081,7 @@ def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True,
     # will be differentiated keep those nodes apart
     stats["conv_activation"] = 0 if training else fuse_conv_activation(sdfg)
     stats["gated_conv"] = 0 if training else fuse_gate_into_conv(sdfg)
+    stats["expand_depthwise"] = 0 if training else fuse_expand_depthwise(sdfg)
     stats["matmul_to_einsum"] = lower_matmul(sdfg)
     stats["views"] = fold_views(sdfg)
     stats["epilogues"] = fuse_epilogues(sdfg, keep_preactivation=training, activation_in_epilogue=gelu_epilogue)

@@ -273,6 +273,15 @@ int dmlhip_conv2d_f16(const dmlhip_conv2d_desc* d, const void* x, const void* w,
  * otherwise: the caller keeps Mul and Conv separate). */
 int dmlhip_conv2d_gated_f32(const dmlhip_conv2d_desc* d, const void* x, const void* gate,
                             const void* w, const void* bias, void* y, void* stream);
+/* A pointwise convolution + activation followed by a 3x3 depthwise convolution + activation — the expand and
+ * depthwise stages of an MBConv block, i.e. two Conv nodes (PureConv2D / CudnnConvolution,
+ * img_op_implementations.py:164-330, cudnn_implementations.py:123-410) with their Swish chains — in one kernel:
+ * the expanded tensor stays in LDS. pw: 1x1, stride 1, no padding, group 1, c % 16 == 0, m % 32 == 0; dw: the
+ * pointwise output as input, 3x3, padding 1, stride 1 or 2, group = channels. act of each descriptor: NONE, SWISH,
+ * RELU. DMLHIP_ERR_UNSUPPORTED otherwise (the caller keeps the two convolutions). fp32. */
+int dmlhip_conv2d_expand_depthwise_f32(const dmlhip_conv2d_desc* pw, const dmlhip_conv2d_desc* dw, const void* x,
+                                       const void* w_pw, const void* b_pw, const void* w_dw, const void* b_dw,
+                                       void* y, void* stream);
 /* cudnnConvolutionBackwardData / BackwardFilter (autodiff/implementations/onnx_ops.py:663-703)
  * and the ATen depthwise backward (onnx_ops.py:1201-1231). dw is overwritten. The bias
  * gradient is dmlhip_reduce over [n, m, oh*ow] done by the caller (two reduce calls). */

@@ -139,8 +139,10 @@ def test_mbconv_block_forward():
             params[name] = (r.standard_normal(desc.shape) * 0.1).astype(np.float32)
     stats = fusion.auto_optimize(sdfg)
     assert stats["swish"] == 3 and stats["conv_activation"] == 4 and stats["gated_conv"] == 1
+    assert stats["expand_depthwise"] == 1
     names = [n.schema.name for n in sdfg.states()[0].library_nodes()]
     assert names.count("GatedConv") == 1 and "Mul" not in names   # the squeeze-excite Mul went into the projection
+    assert names.count("ExpandDepthwiseConv") == 1                # the expanded tensor stays on chip
     prog = _compile(sdfg)
     oh = (hw + 2 - 3) // 2 + 1
     y = torch.empty((b, cout, oh, oh), dtype=torch.float32, device="cuda")

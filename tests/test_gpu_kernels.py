@@ -496,6 +496,48 @@ def test_conv2d_f32_swish_epilogue():
         assert_close(host(got), want, torch.float32, "conv+swish %s" % (ws, ))
 
 
+# n, cin, cmid, h, w, stride, activations, biases
+EXPAND_DEPTHWISE_CASES = [
+    (2, 16, 32, 9, 11, 2, ("swish", "swish"), True),      # odd sizes, stride 2: the last strip is short
+    (3, 32, 64, 14, 14, 1, ("none", "none"), True),
+    (2, 16, 96, 28, 28, 2, ("swish", "swish"), True),     # the MBConv block of the graph tests
+    (1, 48, 32, 7, 5, 1, ("relu", "none"), False),        # three input-channel steps, image narrower than a tile
+    (2, 32, 64, 5, 70, 2, ("none", "relu"), True),        # rows wider than a wavefront
+    (1, 16, 32, 1, 1, 1, ("swish", "none"), True),        # a single pixel: every neighbour is padding
+    (2, 32, 192, 40, 40, 1, ("relu", "relu"), False),
+]
+
+
+@pytest.mark.parametrize("n,cin,cmid,h,w,stride,acts,has_bias", EXPAND_DEPTHWISE_CASES)
+def test_conv2d_expand_depthwise(n, cin, cmid, h, w, stride, acts, has_bias):
+    """The fused pointwise + depthwise kernel against the composition of the two oracle convolutions, at the strip
+    height the library picks and at pinned ones (strips of 1 and 4 output rows recompute different halo rows)."""
+    from daceml_amd import _lib as L, kernels as K
+    code = {"none": L.ACT_NONE, "swish": L.ACT_SWISH, "relu": L.ACT_RELU}
+    fn = {"none": lambda t: t, "swish": O.swish, "relu": lambda t: np.maximum(t, 0.0)}
+    r = rng(140)
+    x = r.standard_normal((n, cin, h, w)).astype(np.float32)
+    w1 = (r.standard_normal((cmid, cin, 1, 1)) * np.sqrt(2.0 / cin)).astype(np.float32)
+    w2 = (r.standard_normal((cmid, 1, 3, 3)) * np.sqrt(2.0 / 9)).astype(np.float32)
+    b1 = (r.standard_normal(cmid) * 0.1).astype(np.float32) if has_bias else None
+    b2 = (r.standard_normal(cmid) * 0.1).astype(np.float32) if has_bias else None
+    f64 = lambda t: None if t is None else t.astype(np.float64)
+    mid = fn[acts[0]](O.conv2d(f64(x), f64(w1), f64(b1)))
+    want = fn[acts[1]](O.conv2d(mid, f64(w2), f64(b2), (stride, stride), (1, 1, 1, 1), (1, 1), cmid))
+    lib = L.load()
+    try:
+        for toh in (0, 1, 4):
+            lib.dmlhip_debug_force_fused_strip(toh)
+            got = K.conv2d_expand_depthwise(dev(x), dev(w1), None if b1 is None else dev(b1), dev(w2),
+                                            None if b2 is None else dev(b2), stride=stride, act_pw=code[acts[0]],
+                                            act_dw=code[acts[1]])
+            assert tuple(got.shape) == want.shape
+            # two chained fp32 convolutions: the first one's rounding passes through nine taps of the second
+            assert_close(host(got), want, torch.float32, "expand+depthwise strip %d" % toh, rtol=1e-5, atol=4e-6)
+    finally:
+        lib.dmlhip_debug_force_fused_strip(0)
+
+
 @pytest.mark.parametrize("xs,ws,st,pd,dl,grp,has_bias", CONV_CASES)
 def test_conv2d_backward_f32(xs, ws, st, pd, dl, grp, has_bias):
     from daceml_amd import kernels as K

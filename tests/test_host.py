@@ -132,6 +132,26 @@ def test_argument_errors_of_the_grouped_and_fused_entry_points(lib):
         L.ERR_WORKSPACE
     assert lib.dmlhip_batchnorm_backward_f32(p, p, p, p, p, None, None, None, 2, 3, 16, 1e-5, p, 1 << 20, None) == L.ERR_NULL
     assert lib.dmlhip_batchnorm_workspace_bytes(8, 3, 1024) > 0
+    # pointwise + depthwise in one kernel: the pair of descriptors must describe that chain
+    pw, dw = L.Conv2dDesc(), L.Conv2dDesc()
+    pw.n, pw.c, pw.h, pw.w, pw.m, pw.kh, pw.kw = 2, 16, 8, 8, 32, 1, 1
+    pw.stride_h = pw.stride_w = pw.dil_h = pw.dil_w = pw.group = 1
+    dw.n, dw.c, dw.h, dw.w, dw.m, dw.kh, dw.kw = 2, 32, 8, 8, 32, 3, 3
+    dw.stride_h = dw.stride_w = dw.pad_h = dw.pad_w = dw.dil_h = dw.dil_w = 1
+    dw.group = 32
+    fused = lambda *a: lib.dmlhip_conv2d_expand_depthwise_f32(ctypes.byref(pw), ctypes.byref(dw), *a)
+    assert fused(p, p, None, None, None, p, None) == L.ERR_NULL
+    dw.stride_h = dw.stride_w = 3
+    assert fused(p, p, None, p, None, p, None) == L.ERR_UNSUPPORTED
+    dw.stride_h = dw.stride_w = 1
+    dw.h = 9
+    assert fused(p, p, None, p, None, p, None) == L.ERR_SHAPE
+    dw.h = 8
+    pw.c = 8
+    assert fused(p, p, None, p, None, p, None) == L.ERR_UNSUPPORTED
+    pw.c = 16
+    pw.act = L.ACT_GELU
+    assert fused(p, p, None, p, None, p, None) == L.ERR_ENUM
 
 
 def test_kernels_refuse_host_tensors():
@@ -348,7 +368,8 @@ def test_fusion_pipeline_on_bert_layer():
     before = [n.schema.name for n in st.library_nodes()]
     assert before.count("MatMul") == 8 and before.count("Erf") == 1 and before.count("ReduceMean") == 4
     stats = fusion.auto_optimize(sdfg, training=True, gelu_epilogue=True)
-    assert stats == {"gelu": 1, "layernorm": 2, "swish": 0, "conv_activation": 0, "gated_conv": 0, "matmul_to_einsum": 8,
+    assert stats == {"gelu": 1, "layernorm": 2, "swish": 0, "conv_activation": 0, "gated_conv": 0, "expand_depthwise": 0,
+                     "matmul_to_einsum": 8,
                      "views": 15, "epilogues": 7, "skip_layernorm": 0, "attention": 0,   # head dim 32: not fused
                      "grouped_einsums": 0}                                               # training: after autodiff
     after = {n.label: n for n in st.library_nodes()}
@@ -466,6 +487,18 @@ def test_training_graphs_keep_differentiable_nodes():
 
     g = build()
     assert fusion.auto_optimize(g.sdfg, training=False)["conv_activation"] == 1
+
+    # pointwise + swish + depthwise + swish -> one node, in forward graphs only and only in the kernel's tiling
+    def block(cin):
+        return graphs.mbconv_block(2, cin, 32, expand=6, cout=24, se_reduce=4, stride=2, dtype=torch.float32)
+    sdfg = block(16)
+    assert fusion.auto_optimize(sdfg)["expand_depthwise"] == 1
+    fused = [n for n in sdfg.states()[0].library_nodes() if n.schema.name == "ExpandDepthwiseConv"]
+    assert len(fused) == 1 and (fused[0].act_pw, fused[0].act_dw, list(fused[0].strides)) == ("swish", "swish", [2, 2])
+    assert sorted(fused[0].in_connectors) == ["B_dw", "B_pw", "W_dw", "W_pw", "X"]
+    assert [n.schema.name for n in sdfg.states()[0].library_nodes()].count("Conv") == 2   # the squeeze-excite pair
+    assert fusion.auto_optimize(block(16), training=True)["expand_depthwise"] == 0
+    assert fusion.auto_optimize(block(24))["expand_depthwise"] == 0                      # 24 input channels: not tiled
     g = build()
     assert fusion.auto_optimize(g.sdfg, training=True)["conv_activation"] == 0
     grads = add_backward_pass(g.sdfg, g.state, ["y"], ["x", "w", "b"])
