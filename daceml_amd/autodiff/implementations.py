@@ -299,6 +299,11 @@ HipSwishBackward = _make_unary_backward("Swish", "SwishGrad", "X", "Y")
 HipSigmoidBackward = _make_unary_backward("Sigmoid", "SigmoidGrad", "X", "Y")
 HipReluBackward = _make_unary_backward("Relu", "ReluGrad", "X", "Y")
 HipTanhBackward = _make_unary_backward("Tanh", "TanhGrad", "input", "output")
+HipErfBackward = _make_unary_backward("Erf", "ErfGrad", "input", "output")
+HipSqrtBackward = _make_unary_backward("Sqrt", "SqrtGrad", "X", "Y")
+HipExpBackward = _make_unary_backward("Exp", "ExpGrad", "input", "output")
+HipLogBackward = _make_unary_backward("Log", "LogGrad", "input", "output")
+HipReciprocalBackward = _make_unary_backward("Reciprocal", "ReciprocalGrad", "X", "Y")
 
 
 @autoregister_params(op="Add", name=NAME)
@@ -492,6 +497,65 @@ class HipDivBackward(BackwardImplementation):
                 b.finish(conn, b.op("Mul", t, _minus_one(context, b.od.dtype)))
             req[conn] = conn + "_grad"
         return b.group, BackwardResult(required_grad_names=req, given_grad_names={"C": "C_grad"})
+
+
+@autoregister_params(op="Pow", name=NAME)
+class HipPowBackward(BackwardImplementation):
+    """Z = X ** p with p a scalar constant of the graph (the square of a decomposed LayerNormalization,
+    pure_implementations.py:39-41): dX = dZ * p * X ** (p - 1). A gradient for the exponent is not offered."""
+    @staticmethod
+    def _exponent(node, state, sdfg):
+        arr = next(iter(state.in_edges_by_connector(node, "Y"))).data.data
+        return sdfg.constants_exact.get(arr)
+
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            x = next(iter(state.in_edges_by_connector(node, "X"))).data.data
+            z = next(iter(state.out_edges_by_connector(node, "Z"))).data.data
+            return (HipPowBackward._exponent(node, state, sdfg) is not None
+                    and tuple(sdfg.arrays[x].shape) == tuple(sdfg.arrays[z].shape))
+        except StopIteration:
+            return False
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        if list(required_gradients) != ["X"]:
+            raise AutoDiffException("Pow: only the base can be differentiated (node %s)" % forward_node.label)
+        sdfg = context.forward_sdfg
+        x = _in_arr(context, forward_node, "X")
+        xd = sdfg.arrays[x]
+        p = HipPowBackward._exponent(forward_node, context.forward_state, sdfg)
+        group = BackwardGroup(forward_node.label + "_backward")
+        label = forward_node.label
+
+        def binary(kind, tag, a, b):
+            node = _new(context, kind, "%s_grad_%s" % (label, tag))
+            for conn, src in (("A", a), ("B", b)):
+                node.add_in_connector(conn)
+                if src is None:
+                    group.map_input("Z_grad", node, conn)
+                elif isinstance(src, tuple):
+                    tmp, _ = sdfg.add_transient("%s_backward_%s_%s" % (label, tag, conn), xd.shape, xd.dtype)
+                    _write(context, src[0], src[1], tmp)
+                    _read(context, tmp, node, conn)
+                else:
+                    _read(context, src, node, conn)
+            node.add_out_connector("C")
+            return node, "C"
+
+        if p == 2.0:
+            base = x                                     # X ** 1
+        else:
+            pw = _new(context, "Pow", "%s_grad_pow" % label)
+            _read(context, x, pw, "X")
+            _read(context, _scalar_constant(context, "%s_backward_exponent" % label, p - 1.0, xd.dtype), pw, "Y")
+            pw.add_out_connector("Z")
+            base = (pw, "Z")
+        t = binary("Mul", "times_base", None, base)
+        t = binary("Mul", "times_exponent", t, _scalar_constant(context, "%s_backward_factor" % label, p, xd.dtype))
+        group.map_output("X_grad", t[0], t[1])
+        return group, BackwardResult(required_grad_names={"X": "X_grad"}, given_grad_names={"Z": "Z_grad"})
 
 
 def _scalar_constant(ctx, name: str, value: float, dtype) -> str:

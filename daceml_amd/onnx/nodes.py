@@ -165,6 +165,9 @@ SCHEMAS = [
     _schema("SigmoidGrad", "dY X", "dX", since=1),
     _schema("ReluGrad", "dY X", "dX", since=1),
     _schema("TanhGrad", "dY X", "dX", since=1),
+    _schema("ErfGrad", "dY X", "dX", since=1), _schema("SqrtGrad", "dY X", "dX", since=1),
+    _schema("ExpGrad", "dY X", "dX", since=1), _schema("LogGrad", "dY X", "dX", since=1),
+    _schema("ReciprocalGrad", "dY X", "dX", since=1),
     _schema("ConvGrad", "dY X W", "dX? dW? dB?", since=1, auto_pad="NOTSET", dilations=None, group=1,
             kernel_shape=None, pads=None, strides=None),
 ]

@@ -609,6 +609,11 @@ HipSwishGrad = _make_unary_grad("SwishGrad", L.SWISH, _GRAD_DOC)
 HipSigmoidGrad = _make_unary_grad("SigmoidGrad", L.SIGMOID, _GRAD_DOC)
 HipReluGrad = _make_unary_grad("ReluGrad", L.RELU, _GRAD_DOC)
 HipTanhGrad = _make_unary_grad("TanhGrad", L.TANH, _GRAD_DOC)
+HipErfGrad = _make_unary_grad("ErfGrad", L.ERF, _GRAD_DOC)
+HipSqrtGrad = _make_unary_grad("SqrtGrad", L.SQRT, _GRAD_DOC)
+HipExpGrad = _make_unary_grad("ExpGrad", L.EXP, _GRAD_DOC)
+HipLogGrad = _make_unary_grad("LogGrad", L.LOG, _GRAD_DOC)
+HipReciprocalGrad = _make_unary_grad("ReciprocalGrad", L.RECIPROCAL, _GRAD_DOC)
 
 
 @op_implementation(op="BiasGelu", name=IMPL)

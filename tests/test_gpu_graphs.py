@@ -214,6 +214,47 @@ def test_elementwise_backward_with_broadcast(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_unfused_layernorm_and_gelu_chains_backward(dtype):
+    """The exporter's decomposed LayerNormalization (ReduceMean, Sub, Pow, ReduceMean, Add, Sqrt, Div, Mul, Add) and GELU
+    (Div, Erf, Add, Mul, Mul) differentiated node by node, without the fusion pass (the reference reverses these maps
+    symbolically, backward_pass_generator.py:1284-1421), against autograd on the same expression."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    g = graphs.GraphBuilder("chains_backward", dtype)
+    x = g.input("x", (3, 7, 64))
+    g.input("gamma", (64, ))
+    g.input("beta", (64, ))
+    ln = g.layer_norm(x, "gamma", "beta", 1e-5, "ln")
+    g.output(g.gelu(ln, "act"), "y")
+    grads = add_backward_pass(g.sdfg, g.state, ["y"], ["x", "gamma", "beta"])
+    assert grads == {"x": "gradient_x", "gamma": "gradient_gamma", "beta": "gradient_beta"}
+    kinds = [n.schema.name for n in g.sdfg.states()[1].library_nodes()]
+    assert "ErfGrad" in kinds and "SqrtGrad" in kinds and kinds.count("ScaledExpand") == 2
+    assert "LayerNormalizationGrad" not in kinds and "GeluGrad" not in kinds
+    prog = _compile(g.sdfg)
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    xv = rng(21).standard_normal((3, 7, 64)).astype(npdt)
+    gv = rng(22).uniform(0.5, 1.5, 64).astype(npdt)
+    bv = (rng(23).standard_normal(64) * 0.1).astype(npdt)
+    dyv = rng(24).standard_normal((3, 7, 64)).astype(npdt)
+    out = {"y": torch.empty((3, 7, 64), dtype=dtype, device="cuda"),
+           "gradient_x": torch.empty((3, 7, 64), dtype=dtype, device="cuda"),
+           "gradient_gamma": torch.empty((64, ), dtype=dtype, device="cuda"),
+           "gradient_beta": torch.empty((64, ), dtype=dtype, device="cuda")}
+    prog(x=dev(xv), gamma=dev(gv), beta=dev(bv), gradient_y=dev(dyv), **out)
+    tx, tg, tb = (torch.tensor(v.astype(np.float64), requires_grad=True) for v in (xv, gv, bv))
+    ty = torch.nn.functional.gelu(torch.nn.functional.layer_norm(tx, (64, ), tg, tb, 1e-5))
+    ty.backward(torch.tensor(dyv.astype(np.float64)))
+    # fourteen chained elementwise / reduction nodes: every fp16 intermediate is rounded to fp16
+    kw = dict(rtol=1e-4, atol=2e-5) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+    assert_close(host(out["y"]), ty.detach().numpy(), dtype, "forward", **kw)
+    assert_close(host(out["gradient_x"]), tx.grad.numpy(), dtype, "gradient of x", **kw)
+    kw = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=3e-2, atol=0.15)
+    assert_close(host(out["gradient_gamma"]), tg.grad.numpy(), dtype, "gradient of gamma", **kw)
+    assert_close(host(out["gradient_beta"]), tb.grad.numpy(), dtype, "gradient of beta", **kw)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_reduce_and_transpose_backward(dtype):
     """ReduceMean (keepdims 1), ReduceSum (keepdims 0) and Transpose reversed with ScaledExpand / Transpose nodes,
     against autograd: y = transpose(x - mean(x, -1, keepdim)) * sum(x, (0, 1))."""

@@ -254,14 +254,18 @@ def test_unary(dtype, name):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["gelu", "swish", "sigmoid", "relu", "tanh"])
+@pytest.mark.parametrize("name", ["gelu", "swish", "sigmoid", "relu", "tanh", "erf", "sqrt", "exp", "log", "reciprocal"])
 def test_unary_backward(dtype, name):
     from daceml_amd import _lib as L, kernels as K
     x, x64 = _inputs(17, (41, 64), dtype)
     dy, dy64 = _inputs(18, (41, 64), dtype)
+    if name in ("sqrt", "log", "reciprocal"):
+        x = (np.abs(x) + 0.5).astype(_np(dtype))
+        x64 = x.astype(np.float64)
     t = torch.tensor(x64, requires_grad=True)
     f = {"gelu": lambda v: torch.nn.functional.gelu(v), "swish": lambda v: v * torch.sigmoid(v),
-         "sigmoid": torch.sigmoid, "relu": torch.relu, "tanh": torch.tanh}[name]
+         "sigmoid": torch.sigmoid, "relu": torch.relu, "tanh": torch.tanh, "erf": torch.erf, "sqrt": torch.sqrt,
+         "exp": torch.exp, "log": torch.log, "reciprocal": torch.reciprocal}[name]
     f(t).backward(torch.tensor(dy64))
     got = K.unary_backward(getattr(L, name.upper()), dev(x), dev(dy))
     assert_close(host(got), t.grad.numpy(), dtype, name + " backward")

@@ -468,6 +468,32 @@ def test_attention_fusion_roles_and_graph():
     assert fusion.auto_optimize(s32)["attention"] == 0
 
 
+def test_pow_backward_needs_a_constant_exponent():
+    """X ** p reverses to dZ * p * X ** (p - 1) for a scalar constant p (p = 2: no Pow node left); an exponent that is
+    a run-time tensor has no backward and the generator says so."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.autodiff.base_abc import AutoDiffException
+
+    def build(exponent):
+        g = graphs.GraphBuilder("pow", torch.float32)
+        x = g.input("x", (4, 8))
+        e = g.input("e", (4, 8)) if exponent is None else g.constant("e", exponent)
+        g.output(g.node("Pow", {"X": x, "Y": e}, {"Z": (4, 8)}, label="p")["Z"], "y")
+        return g
+
+    g = build(3.0)
+    assert add_backward_pass(g.sdfg, g.state, ["y"], ["x"]) == {"x": "gradient_x"}
+    assert sorted(n.schema.name for n in g.sdfg.states()[1].library_nodes()) == ["Mul", "Mul", "Pow"]
+    assert g.sdfg.constants_exact["p_backward_exponent"] == 2.0 and g.sdfg.constants_exact["p_backward_factor"] == 3.0
+    g = build(2.0)
+    add_backward_pass(g.sdfg, g.state, ["y"], ["x"])
+    assert sorted(n.schema.name for n in g.sdfg.states()[1].library_nodes()) == ["Mul", "Mul"]
+    g = build(None)
+    with pytest.raises(AutoDiffException):
+        add_backward_pass(g.sdfg, g.state, ["y"], ["x"])
+
+
 def test_training_graphs_keep_differentiable_nodes():
     """Conv + activation stays two nodes when a backward pass is to come (ConvGrad differentiates a plain Conv), and
     the backward pass then builds."""
