@@ -11,6 +11,18 @@
 #include <type_traits>
 
 namespace dml {
+
+// conv_backward.hip
+bool depthwise_bwd_supported(int k, int s, int p);
+int launch_depthwise_bwd_data(const float* dy, const float* w, float* dx, int n, int c, int h, int wd, int oh, int ow, int k,
+                              int s, hipStream_t st);
+size_t depthwise_bwd_weight_partials(int n, int c, int k);
+int launch_depthwise_bwd_weight(const float* x, const float* dy, float* part, int n, int c, int h, int wd, int oh, int ow,
+                                int k, int s, int p, hipStream_t st);
+int64_t pointwise_bwd_weight_partials(int n, int m, int c, int64_t hw);
+int launch_pointwise_bwd_weight(const float* x, const float* dy, float* part, int n, int m, int c, int64_t hw,
+                                hipStream_t st);
+
 namespace {
 
 struct ConvGeom {
@@ -202,7 +214,9 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const float* __res
 // A = W (rows = output channels), B = X (columns = pixels): a lane's accumulators are 16 output channels of ONE
 // pixel, so stores of a wavefront run along the pixels. `in_scale` (optional) is a per-image, per-input-channel
 // factor applied to X on its way into LDS (the squeeze-excite gate in front of a projection).
-template <int MT, int PT>  // 32-channel blocks per workgroup; 32-pixel blocks per wavefront
+// WT: the weights are given transposed, as [cin][cout] (the data gradient of a pointwise convolution is a pointwise
+// convolution of dY with W^T); cin may then be any positive number, the last chunk is zero-filled.
+template <int MT, int PT, bool WT>  // 32-channel blocks per workgroup; 32-pixel blocks per wavefront
 __global__ __launch_bounds__(256, 2) void conv_pointwise_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                                     const float* __restrict__ bias,
                                                                     const float* __restrict__ in_scale, float* __restrict__ y,
@@ -233,34 +247,51 @@ __global__ __launch_bounds__(256, 2) void conv_pointwise_f32_kernel(const float*
         __syncthreads();  // the previous chunk has been consumed
         // all loads of the chunk are issued before the first one is used (branch-free: out-of-range pixels read
         // a clamped address and are zeroed afterwards), so the chunk costs one memory round trip, not eight
-        constexpr int XL = KC * (PX / 4) / 256, WL = (MT * 32 * (KC / 4) + 255) / 256;
-        floatx4 xv[XL], wv[WL];
+        constexpr int XL = KC * (PX / 4) / 256, WL = (MT * 32 * (KC / 4) + 255) / 256, WS = MT * 32 * KC / 256;
+        floatx4 xv[XL], wv[WT ? 1 : WL];
+        float wt[WT ? WS : 1];
 #pragma unroll
         for (int r = 0; r < XL; ++r) {
             const int idx = r * 256 + threadIdx.x, row = idx / (PX / 4), c4 = idx % (PX / 4);
             const int64_t p = p0 + c4 * 4 < hw ? p0 + c4 * 4 : hw - 4;
-            xv[r] = *reinterpret_cast<const floatx4*>(xn + (int64_t)(kc + row) * hw + p);
+            xv[r] = *reinterpret_cast<const floatx4*>(xn + (int64_t)min(kc + row, cin - 1) * hw + p);
         }
+        if constexpr (WT) {
 #pragma unroll
-        for (int r = 0; r < WL; ++r) {
-            const int idx = r * 256 + threadIdx.x, row = min(idx / (KC / 4), MT * 32 - 1), c4 = idx % (KC / 4);
-            wv[r] = *reinterpret_cast<const floatx4*>(w + (int64_t)min(m0 + row, cout - 1) * cin + kc + c4 * 4);
+            for (int r = 0; r < WS; ++r) {
+                const int idx = r * 256 + threadIdx.x, col = idx / (MT * 32), row = idx % (MT * 32);
+                wt[r] = w[(int64_t)min(kc + col, cin - 1) * cout + min(m0 + row, cout - 1)];
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < WL; ++r) {
+                const int idx = r * 256 + threadIdx.x, row = min(idx / (KC / 4), MT * 32 - 1), c4 = idx % (KC / 4);
+                wv[r] = *reinterpret_cast<const floatx4*>(w + (int64_t)min(m0 + row, cout - 1) * cin + kc + c4 * 4);
+            }
         }
 #pragma unroll
         for (int r = 0; r < XL; ++r) {
             const int idx = r * 256 + threadIdx.x, row = idx / (PX / 4), c4 = idx % (PX / 4);
             floatx4 v = xv[r];
-            if (in_scale) v *= in_scale[(int64_t)n * cin + kc + row];
-            if (!(p0 + c4 * 4 < hw)) v = floatx4{0.f, 0.f, 0.f, 0.f};
+            if (in_scale) v *= in_scale[(int64_t)n * cin + min(kc + row, cin - 1)];
+            if (!(p0 + c4 * 4 < hw) || kc + row >= cin) v = floatx4{0.f, 0.f, 0.f, 0.f};
             *reinterpret_cast<floatx4*>(xs + row * XP + c4 * 4) = v;
         }
+        if constexpr (WT) {
 #pragma unroll
-        for (int r = 0; r < WL; ++r) {
-            const int idx = r * 256 + threadIdx.x, row = idx / (KC / 4), c4 = idx % (KC / 4);
-            if (idx < MT * 32 * (KC / 4)) {
-                const bool ok = m0 + row < cout;
+            for (int r = 0; r < WS; ++r) {
+                const int idx = r * 256 + threadIdx.x, col = idx / (MT * 32), row = idx % (MT * 32);
+                ws[row * WP + col] = (kc + col < cin && m0 + row < cout) ? wt[r] : 0.f;
+            }
+        } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) ws[row * WP + c4 * 4 + e] = ok ? wv[r][e] : 0.f;
+            for (int r = 0; r < WL; ++r) {
+                const int idx = r * 256 + threadIdx.x, row = idx / (KC / 4), c4 = idx % (KC / 4);
+                if (idx < MT * 32 * (KC / 4)) {
+                    const bool ok = m0 + row < cout;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ws[row * WP + c4 * 4 + e] = ok ? wv[r][e] : 0.f;
+                }
             }
         }
         __syncthreads();
@@ -330,7 +361,7 @@ __global__ __launch_bounds__(256) void conv_1x1_spatial1_kernel(const T* __restr
 }
 
 int launch_pointwise_f32(const float* x, const float* w, const float* bias, const float* in_scale, float* y, int n, int cin,
-                         int cout, int64_t hw, int act, hipStream_t st) {
+                         int cout, int64_t hw, int act, hipStream_t st, bool w_transposed = false) {
     int mt = (int)ceil_div(cout, 32);
     if (mt > 6) mt = 6;
     // many output channels: 32 pixels per wavefront keep the accumulators (16 registers per 32x32 block) and the
@@ -340,8 +371,12 @@ int launch_pointwise_f32(const float* x, const float* w, const float* bias, cons
     const size_t lds = (size_t)(32 * (128 * pt + 32) + mt * 32 * 33 + mt * 32) * sizeof(float);
 #define DML_PW(MT, PT)                                                                                                 \
     case MT:                                                                                                           \
-        hipLaunchKernelGGL((conv_pointwise_f32_kernel<MT, PT>), grid, 256, lds, st, x, w, bias, in_scale, y, cin, cout, hw, \
-                           act);                                                                                       \
+        if (w_transposed)                                                                                              \
+            hipLaunchKernelGGL((conv_pointwise_f32_kernel<MT, PT, true>), grid, 256, lds, st, x, w, bias, in_scale, y, \
+                               cin, cout, hw, act);                                                                    \
+        else                                                                                                           \
+            hipLaunchKernelGGL((conv_pointwise_f32_kernel<MT, PT, false>), grid, 256, lds, st, x, w, bias, in_scale, y, \
+                               cin, cout, hw, act);                                                                    \
         break
     switch (mt) {
         DML_PW(1, 2); DML_PW(2, 2); DML_PW(3, 2); DML_PW(4, 2); DML_PW(5, 1);
@@ -379,6 +414,16 @@ int make_geom(const dmlhip_conv2d_desc* d, ConvGeom* g, const char* what) {
     g->group = (int)d->group; g->oh = (int)oh; g->ow = (int)ow;
     g->cg = g->c / g->group; g->mg = g->m / g->group; g->act = d->act;
     return 0;
+}
+
+inline bool is_pointwise(const ConvGeom& g) {
+    return g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1;
+}
+
+// depthwise with a stencil, stride and "same" padding the gradient kernels are built for
+inline bool is_depthwise_grad(const ConvGeom& g) {
+    return g.group == g.c && g.m == g.c && g.c > 0 && g.kh == g.kw && g.sh == g.sw && g.ph == g.pw && g.dh == 1 &&
+           g.dw == 1 && depthwise_bwd_supported(g.kh, g.sh, g.ph) && g.oh > 0 && g.ow > 0;
 }
 
 inline unsigned grid_for(int64_t total) {
@@ -505,8 +550,12 @@ int dmlhip_conv2d_backward_data_f32(const dmlhip_conv2d_desc* d, const void* dy,
     hipStream_t st = (hipStream_t)stream;
     if (g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1 && g.m > 0) {
         // dX[b] (C x HW) = W^T (C x M) . dY[b] (M x HW)
-        dmlhip_gemm_desc gd = {};
         const int64_t hw = (int64_t)g.h * g.w;
+        // many pixels: the streaming pointwise kernel with dY as its input and W read as [cin = M][cout = C]
+        if (hw % 4 == 0 && hw >= 128 && g.n <= 65535 && aligned16(dy) && aligned16(dx))
+            return launch_pointwise_f32((const float*)dy, (const float*)w, nullptr, nullptr, (float*)dx, g.n, g.m, g.c, hw,
+                                        DMLHIP_ACT_NONE, st, true);
+        dmlhip_gemm_desc gd = {};
         gd.m = g.c; gd.n = hw; gd.k = g.m;
         gd.batch[0] = 1; gd.batch[1] = 1; gd.batch[2] = g.n;
         gd.a_stride_m = 1; gd.a_stride_k = g.c;
@@ -515,6 +564,9 @@ int dmlhip_conv2d_backward_data_f32(const dmlhip_conv2d_desc* d, const void* dy,
         gd.alpha = 1.f; gd.out_dtype = DMLHIP_F32; gd.bias_dtype = DMLHIP_F32;
         return dmlhip_gemm_f32(&gd, w, dy, dx, nullptr, nullptr, nullptr, stream);
     }
+    if (is_depthwise_grad(g))
+        return launch_depthwise_bwd_data((const float*)dy, (const float*)w, (float*)dx, g.n, g.c, g.h, g.w, g.oh, g.ow, g.kh,
+                                         g.sh, st);
     hipLaunchKernelGGL(conv_bwd_data_kernel, grid_for(total), 256, 0, st, (const float*)dy, (const float*)w, (float*)dx,
                        g, total);
     return launch_status("conv2d_backward_data");
@@ -523,8 +575,22 @@ int dmlhip_conv2d_backward_data_f32(const dmlhip_conv2d_desc* d, const void* dy,
 size_t dmlhip_conv2d_backward_weight_workspace_bytes(const dmlhip_conv2d_desc* d) {
     ConvGeom g;
     if (make_geom(d, &g, "conv2d_backward_weight")) return 0;
-    if (g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1 && g.n > 1)
-        return (size_t)g.n * g.m * g.c * sizeof(float) + dmlhip_reduce_workspace_bytes(1, g.n, (int64_t)g.m * g.c);
+    if (is_pointwise(g) && g.n >= 1) {
+        // the larger of what the two paths need: per-workgroup results of the streaming kernel, or per-image
+        // products of the batched GEMM (taken when the streaming kernel does not apply or an operand is unaligned)
+        const int64_t mc = (int64_t)g.m * g.c;
+        size_t need = g.n > 1 ? (size_t)g.n * mc * sizeof(float) + dmlhip_reduce_workspace_bytes(1, g.n, mc) : 0;
+        const int64_t parts = pointwise_bwd_weight_partials(g.n, g.m, g.c, (int64_t)g.h * g.w);
+        if (parts > 1) {
+            const size_t streaming = (size_t)parts * mc * sizeof(float) + dmlhip_reduce_workspace_bytes(1, parts, mc);
+            if (streaming > need) need = streaming;
+        }
+        return need;
+    }
+    if (is_depthwise_grad(g) && g.n > 1) {
+        const int64_t per = (int64_t)g.c * g.kh * g.kw;
+        return (size_t)g.n * per * sizeof(float) + dmlhip_reduce_workspace_bytes(1, g.n, per);
+    }
     return 0;
 }
 
@@ -539,13 +605,38 @@ int dmlhip_conv2d_backward_weight_f32(const dmlhip_conv2d_desc* d, const void* x
     DML_REQUIRE(red == 0 || (x && dy), DMLHIP_ERR_NULL, "conv2d_backward_weight: NULL tensor pointer");
     DML_REQUIRE(total <= 2147483647LL, DMLHIP_ERR_SHAPE, "conv2d_backward_weight: too many weights");
     hipStream_t st = (hipStream_t)stream;
-    if (g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1 && red > 0) {
-        // per image: P[b] (M x C) = dY[b] (M x HW) . X[b]^T (HW x C); then dW = sum_b P[b]
+    if ((is_pointwise(g) || is_depthwise_grad(g)) && red > 0) {
         const size_t need = dmlhip_conv2d_backward_weight_workspace_bytes(d);
         DML_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), DMLHIP_ERR_WORKSPACE,
                     "conv2d_backward_weight: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-        dmlhip_gemm_desc gd = {};
+    }
+    if (is_depthwise_grad(g) && red > 0) {
+        // one result per (image, channel) plane, summed over the images in a fixed order
+        const int64_t per = (int64_t)g.c * g.kh * g.kw;
+        float* part = g.n > 1 ? (float*)workspace : (float*)dw;
+        if (int e = launch_depthwise_bwd_weight((const float*)x, (const float*)dy, part, g.n, g.c, g.h, g.w, g.oh, g.ow,
+                                                g.kh, g.sh, g.ph, st))
+            return e;
+        if (g.n == 1) return 0;
+        const size_t part_bytes = (size_t)g.n * per * sizeof(float);
+        return dmlhip_reduce_f32(DMLHIP_RSUM, part, dw, DMLHIP_F32, 1, g.n, per, (char*)workspace + part_bytes,
+                                 workspace_bytes - part_bytes, stream);
+    }
+    if (is_pointwise(g) && red > 0) {
         const int64_t hw = (int64_t)g.h * g.w;
+        const int64_t parts = pointwise_bwd_weight_partials(g.n, g.m, g.c, hw);
+        if (parts > 0 && aligned16(x) && aligned16(dy)) {
+            // streaming kernel: every workgroup's M x C result, then their sum in a fixed order
+            const int64_t mc = (int64_t)g.m * g.c;
+            float* part = parts > 1 ? (float*)workspace : (float*)dw;
+            if (int e = launch_pointwise_bwd_weight((const float*)x, (const float*)dy, part, g.n, g.m, g.c, hw, st)) return e;
+            if (parts == 1) return 0;
+            const size_t part_bytes = (size_t)parts * mc * sizeof(float);
+            return dmlhip_reduce_f32(DMLHIP_RSUM, part, dw, DMLHIP_F32, 1, parts, mc, (char*)workspace + part_bytes,
+                                     workspace_bytes - part_bytes, stream);
+        }
+        // per image: P[b] (M x C) = dY[b] (M x HW) . X[b]^T (HW x C); then dW = sum_b P[b]
+        dmlhip_gemm_desc gd = {};
         gd.m = g.m; gd.n = g.c; gd.k = hw;
         gd.batch[0] = 1; gd.batch[1] = 1; gd.batch[2] = g.n;
         gd.a_stride_m = hw; gd.a_stride_k = 1; gd.a_stride_batch[2] = (int64_t)g.m * hw;

@@ -463,6 +463,11 @@ CONV_CASES = [
     ((3, 32, 28, 28), (192, 32, 1, 1), (1, 1), (0, 0), (1, 1), 1, True),    # MBConv expand, small spatial
     ((2, 12, 30, 30), (12, 1, 3, 3), (2, 2), (1, 1), (1, 1), 12, True),     # depthwise s2 p1
     ((2, 6, 17, 19), (6, 1, 5, 5), (1, 1), (2, 2), (1, 1), 6, False),       # depthwise 5x5 odd sizes
+    ((2, 6, 17, 19), (6, 1, 5, 5), (2, 2), (2, 2), (1, 1), 6, True),        # depthwise 5x5 stride 2, odd sizes
+    ((1, 4, 9, 11), (4, 1, 3, 3), (2, 2), (1, 1), (1, 1), 4, False),        # depthwise 3x3 stride 2, odd sizes
+    ((2, 5, 13, 70), (5, 1, 3, 3), (1, 1), (1, 1), (1, 1), 5, True),        # depthwise 3x3 stride 1, wide rows
+    ((3, 3, 40, 40), (3, 1, 3, 3), (1, 1), (0, 0), (1, 1), 3, False),       # depthwise without padding: direct gradients
+    ((2, 40, 24, 24), (72, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1, False),    # pointwise, ragged blocks both ways
     ((2, 8, 9, 9), (4, 4, 3, 3), (1, 1), (1, 1), (1, 1), 2, True),          # grouped
     ((1, 2, 12, 12), (3, 2, 3, 3), (1, 1), (2, 2), (2, 2), 1, False),       # dilated
     ((2, 4, 8, 8), (6, 4, 1, 1), (2, 2), (0, 0), (1, 1), 1, True),          # 1x1 strided -> direct
