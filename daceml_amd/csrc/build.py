@@ -24,7 +24,7 @@ SOURCES = [
     "gemm_f16_pipe.hip",
     "gemm_f32.hip",
     "conv.hip",
-    "conv_fused.hip", "conv_backward.hip",
+    "conv_fused.hip", "conv_backward.hip", "conv_implicit.hip",
     "attention.hip",
     "batchnorm.hip",
 ]

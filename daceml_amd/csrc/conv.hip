@@ -7,6 +7,7 @@
 //   * everything else runs a direct kernel, one thread per output, accumulating c, hy, hx
 //     sequentially in fp32 — the summation order of the reference's pure expansion.
 #include "common.h"
+#include "conv_geom.h"
 
 #include <type_traits>
 
@@ -23,11 +24,11 @@ int64_t pointwise_bwd_weight_partials(int n, int m, int c, int64_t hw);
 int launch_pointwise_bwd_weight(const float* x, const float* dy, float* part, int n, int m, int c, int64_t hw,
                                 hipStream_t st);
 
-namespace {
+// conv_implicit.hip
+bool conv_implicit_applicable(const ConvGeom& g);
+int launch_conv_implicit_f32(const ConvGeom& g, const float* x, const float* w, const float* bias, float* y, hipStream_t st);
 
-struct ConvGeom {
-    int n, c, h, w, m, kh, kw, sh, sw, ph, pw, dh, dw, group, oh, ow, cg, mg, act;
-};
+namespace {
 
 // ---------------------------------------------------------------- direct forward
 template <typename T>
@@ -492,6 +493,11 @@ int conv_forward(const dmlhip_conv2d_desc* d, const void* x, const void* w, cons
         }
     }
 direct:
+    if constexpr (sizeof(T) == 4) {
+        // dense convolutions with enough work per output: implicit GEMM on the fp32 matrix pipe
+        if (conv_implicit_applicable(g))
+            return launch_conv_implicit_f32(g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, st);
+    }
     hipLaunchKernelGGL((conv_direct_kernel<T>), grid_for(total), 256, 0, st, (const T*)x, (const T*)w, (const T*)bias,
                        (T*)y, g, total);
     return launch_status("conv2d(direct)");
