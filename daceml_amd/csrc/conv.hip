@@ -27,6 +27,8 @@ int launch_pointwise_bwd_weight(const float* x, const float* dy, float* part, in
 // conv_implicit.hip
 bool conv_implicit_applicable(const ConvGeom& g);
 int launch_conv_implicit_f32(const ConvGeom& g, const float* x, const float* w, const float* bias, float* y, hipStream_t st);
+bool conv_implicit_bwd_data_applicable(const ConvGeom& g);
+int launch_conv_implicit_bwd_data_f32(const ConvGeom& g, const float* dy, const float* w, float* dx, hipStream_t st);
 
 namespace {
 
@@ -573,6 +575,8 @@ int dmlhip_conv2d_backward_data_f32(const dmlhip_conv2d_desc* d, const void* dy,
     if (is_depthwise_grad(g))
         return launch_depthwise_bwd_data((const float*)dy, (const float*)w, (float*)dx, g.n, g.c, g.h, g.w, g.oh, g.ow, g.kh,
                                          g.sh, st);
+    if (conv_implicit_bwd_data_applicable(g))
+        return launch_conv_implicit_bwd_data_f32(g, (const float*)dy, (const float*)w, (float*)dx, st);
     hipLaunchKernelGGL(conv_bwd_data_kernel, grid_for(total), 256, 0, st, (const float*)dy, (const float*)w, (float*)dx,
                        g, total);
     return launch_status("conv2d_backward_data");

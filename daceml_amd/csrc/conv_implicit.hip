@@ -21,6 +21,9 @@ struct ImplicitArgs {
     int prow, pwid, plane;    // rectangle rows / columns, and the per-channel pitch in LDS (== 32 mod 64: the two input
                               // channels a wavefront reads at once sit in different bank halves)
     int wpitch;               // LDS pitch of a weight row: kIgChunk * kh * kw + 1
+    // data-gradient mode: the input (dY) is read as if ids - 1 zeros stood between its rows / columns (the forward
+    // stride), and the weights as W[input channel][output channel] with the taps reversed
+    int ids_h, ids_w, wflip;
 };
 
 // a / b for 0 <= a < 2^22 and 0 < b: the float quotient is within one of the result, the remainder says which way
@@ -76,7 +79,8 @@ __global__ __launch_bounds__(256, (MT * PT <= 2 ? 4 : 2)) void conv_implicit_f32
     const float* xn = x + (size_t)n * g.c * g.h * g.w;
     const int rect = g.prow * g.pwid;
     const int wrow = kIgChunk * kk;     // weights of a chunk per output channel (contiguous in W)
-    const float inv_pwid = 1.0f / (float)g.pwid, inv_wrow = 1.0f / (float)wrow;
+    const float inv_pwid = 1.0f / (float)g.pwid, inv_wrow = 1.0f / (float)wrow, inv_kk = 1.0f / (float)kk;
+    const float inv_ids_h = 1.0f / (float)g.ids_h, inv_ids_w = 1.0f / (float)g.ids_w;
     const int in_plane = g.h * g.w;
     for (int kc = 0; kc < g.c; kc += kIgChunk) {
         __syncthreads();   // the previous chunk has been consumed
@@ -91,8 +95,15 @@ __global__ __launch_bounds__(256, (MT * PT <= 2 ? 4 : 2)) void conv_implicit_f32
             for (int u = 0; u < 2; ++u) {
                 pos[u] = i0 + u * 256 + (int)threadIdx.x;
                 const int row = fast_div(pos[u], g.pwid, inv_pwid), col = pos[u] - row * g.pwid;
-                const int iy = iy_first + row, ix = ix_first + col;
-                ok[u] = pos[u] < rect && iy >= 0 && iy < g.h && ix >= 0 && ix < g.w;
+                int iy = iy_first + row, ix = ix_first + col;
+                bool on_grid = iy >= 0 && ix >= 0;
+                if (g.ids_h > 1 || g.ids_w > 1) {     // only every ids-th position of the dilated input holds a value
+                    const int qy = fast_div(max(iy, 0), g.ids_h, inv_ids_h), qx = fast_div(max(ix, 0), g.ids_w, inv_ids_w);
+                    on_grid = on_grid && qy * g.ids_h == iy && qx * g.ids_w == ix;
+                    iy = qy;
+                    ix = qx;
+                }
+                ok[u] = pos[u] < rect && on_grid && iy < g.h && ix < g.w;
                 off[u] = ok[u] ? iy * g.w + ix : 0;
             }
             float v[2][kIgChunk];
@@ -118,7 +129,12 @@ __global__ __launch_bounds__(256, (MT * PT <= 2 ? 4 : 2)) void conv_implicit_f32
                 const int i = i0 + u * 256 + (int)threadIdx.x;
                 const int row = fast_div(i, wrow, inv_wrow), k = i - row * wrow;
                 const bool ok = i < wtotal && m0 + row < g.m && k < cl * kk;
-                v[u] = w[ok ? ((size_t)(m0 + row) * g.c + kc) * kk + k : 0];
+                size_t src = ((size_t)(m0 + row) * g.c + kc) * kk + k;
+                if (g.wflip) {
+                    const int ch = fast_div(k, kk, inv_kk), tap = k - ch * kk;
+                    src = ((size_t)(kc + ch) * g.m + m0 + row) * kk + (kk - 1 - tap);
+                }
+                v[u] = w[ok ? src : 0];
                 v[u] = ok ? v[u] : 0.f;
                 dst[u] = i < wtotal ? row * g.wpitch + k : -1;
             }
@@ -179,19 +195,24 @@ struct ImplicitPlan {
     dim3 grid;
 };
 
-bool plan_implicit(const ConvGeom& g, ImplicitPlan* pl) {
+// g describes the convolution the kernel runs: for a data gradient that is the stride-1 convolution of the
+// (zero-dilated) dY with the reversed weights, not the forward one.
+bool plan_implicit(const ConvGeom& g, int ids_h, int ids_w, int wflip, ImplicitPlan* pl) {
     if (g.group != 1 || g.c < 1 || g.m < 1 || g.oh < 1 || g.ow < 1 || g.n < 1 || g.n > 65535) return false;
     // worth the staging only with enough arithmetic per output; tiny products stay on the direct kernel
     const int64_t kdim = (int64_t)g.c * g.kh * g.kw;
     if (kdim < 32 || (int64_t)g.oh * g.ow < 64 || g.kh * g.kw > 121) return false;
     if ((int64_t)g.n * g.m * g.oh * g.ow * kdim < (1LL << 24)) return false;
     const int64_t ohw = (int64_t)g.oh * g.ow;
-    if (ohw > (1 << 28) || (int64_t)g.h * g.w > (1 << 28)) return false;
+    if (ohw > (1 << 22) || (int64_t)g.h * g.w > (1 << 28) || (int64_t)g.h * ids_h > (1 << 22) ||
+        (int64_t)g.w * ids_w > (1 << 22))
+        return false;
     int mt = (int)ceil_div(g.m, 32);
     mt = mt >= 4 ? 4 : (mt == 3 ? 4 : mt);
     ImplicitArgs& a = pl->a;
     a.c = g.c; a.h = g.h; a.w = g.w; a.m = g.m; a.kh = g.kh; a.kw = g.kw; a.sh = g.sh; a.sw = g.sw; a.ph = g.ph; a.pw = g.pw;
     a.dh = g.dh; a.dw = g.dw; a.oh = g.oh; a.ow = g.ow; a.act = g.act;
+    a.ids_h = ids_h; a.ids_w = ids_w; a.wflip = wflip;
     a.pwid = (g.ow - 1) * g.sw + (g.kw - 1) * g.dw + 1;
     a.wpitch = kIgChunk * g.kh * g.kw + 1;
     for (int pt = 2; pt >= 1; --pt) {
@@ -216,33 +237,68 @@ bool plan_implicit(const ConvGeom& g, ImplicitPlan* pl) {
     return false;
 }
 
-}  // namespace
-
-bool conv_implicit_applicable(const ConvGeom& g) {
-    ImplicitPlan pl;
-    return plan_implicit(g, &pl);
+// The data gradient of a dense convolution as a convolution: dX = conv(dY with s - 1 zeros between its elements,
+// W with input / output channels exchanged and the taps reversed, stride 1, padding (k - 1) d - p).
+bool data_gradient_problem(const ConvGeom& f, ConvGeom* b) {
+    const int ph = (f.kh - 1) * f.dh - f.ph, pw = (f.kw - 1) * f.dw - f.pw;
+    if (f.group != 1 || ph < 0 || pw < 0) return false;
+    *b = f;
+    b->c = f.m; b->m = f.c;            // channels exchanged
+    b->h = f.oh; b->w = f.ow;          // the input is dY ...
+    b->oh = f.h; b->ow = f.w;          // ... the output dX
+    b->sh = b->sw = 1;
+    b->ph = ph; b->pw = pw;
+    b->cg = b->c; b->mg = b->m;
+    b->act = DMLHIP_ACT_NONE;
+    return true;
 }
 
-int launch_conv_implicit_f32(const ConvGeom& g, const float* x, const float* w, const float* bias, float* y, hipStream_t st) {
-    ImplicitPlan pl;
-    DML_REQUIRE(plan_implicit(g, &pl), DMLHIP_ERR_UNSUPPORTED, "conv2d: the implicit-GEMM kernel does not apply");
+int launch_planned(const ImplicitPlan& pl, const float* x, const float* w, const float* bias, float* y, hipStream_t st,
+                   const char* what) {
 #define DML_IG(MT, PT)                                                                                                 \
     if (pl.mt == MT && pl.pt == PT) {                                                                                  \
         auto kern = conv_implicit_f32_kernel<MT, PT>;                                                                  \
         if (pl.lds > 64 * 1024) {                                                                                      \
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds); \
             if (e != hipSuccess) {                                                                                     \
-                set_error("conv2d: cannot reserve %zu bytes of LDS: %s", pl.lds, hipGetErrorString(e));               \
+                set_error("%s: cannot reserve %zu bytes of LDS: %s", what, pl.lds, hipGetErrorString(e));             \
                 return (int)e;                                                                                         \
             }                                                                                                          \
         }                                                                                                              \
         hipLaunchKernelGGL(kern, pl.grid, 256, pl.lds, st, x, w, bias, y, pl.a);                                       \
-        return launch_status("conv2d(implicit GEMM)");                                                                 \
+        return launch_status(what);                                                                                    \
     }
     DML_IG(1, 1) DML_IG(1, 2) DML_IG(2, 1) DML_IG(2, 2) DML_IG(4, 1) DML_IG(4, 2)
 #undef DML_IG
-    set_error("conv2d: no implicit-GEMM kernel for %d x %d blocks", pl.mt, pl.pt);
+    set_error("%s: no implicit-GEMM kernel for %d x %d blocks", what, pl.mt, pl.pt);
     return DMLHIP_ERR_UNSUPPORTED;
+}
+
+}  // namespace
+
+bool conv_implicit_applicable(const ConvGeom& g) {
+    ImplicitPlan pl;
+    return plan_implicit(g, 1, 1, 0, &pl);
+}
+
+int launch_conv_implicit_f32(const ConvGeom& g, const float* x, const float* w, const float* bias, float* y, hipStream_t st) {
+    ImplicitPlan pl;
+    DML_REQUIRE(plan_implicit(g, 1, 1, 0, &pl), DMLHIP_ERR_UNSUPPORTED, "conv2d: the implicit-GEMM kernel does not apply");
+    return launch_planned(pl, x, w, bias, y, st, "conv2d(implicit GEMM)");
+}
+
+bool conv_implicit_bwd_data_applicable(const ConvGeom& g) {
+    ConvGeom b;
+    ImplicitPlan pl;
+    return data_gradient_problem(g, &b) && plan_implicit(b, g.sh, g.sw, 1, &pl);
+}
+
+int launch_conv_implicit_bwd_data_f32(const ConvGeom& g, const float* dy, const float* w, float* dx, hipStream_t st) {
+    ConvGeom b;
+    ImplicitPlan pl;
+    DML_REQUIRE(data_gradient_problem(g, &b) && plan_implicit(b, g.sh, g.sw, 1, &pl), DMLHIP_ERR_UNSUPPORTED,
+                "conv2d_backward_data: the implicit-GEMM kernel does not apply");
+    return launch_planned(pl, dy, w, nullptr, dx, st, "conv2d_backward_data(implicit GEMM)");
 }
 
 }  // namespace dml
