@@ -20,6 +20,9 @@ int launch_depthwise_bwd_data(const float* dy, const float* w, float* dx, int n,
 size_t depthwise_bwd_weight_partials(int n, int c, int k);
 int launch_depthwise_bwd_weight(const float* x, const float* dy, float* part, int n, int c, int h, int wd, int oh, int ow,
                                 int k, int s, int p, hipStream_t st);
+int64_t dense_bwd_weight_partials(int n, int c, int m, int kh, int kw, int oh, int ow, int h, int w);
+int launch_dense_bwd_weight(const float* x, const float* dy, float* part, int n, int c, int h, int w, int m, int kh, int kw,
+                            int sh, int sw, int ph, int pw, int dh, int dw, int oh, int ow, hipStream_t st);
 int64_t pointwise_bwd_weight_partials(int n, int m, int c, int64_t hw);
 int launch_pointwise_bwd_weight(const float* x, const float* dy, float* part, int n, int m, int c, int64_t hw,
                                 hipStream_t st);
@@ -601,6 +604,11 @@ size_t dmlhip_conv2d_backward_weight_workspace_bytes(const dmlhip_conv2d_desc* d
         const int64_t per = (int64_t)g.c * g.kh * g.kw;
         return (size_t)g.n * per * sizeof(float) + dmlhip_reduce_workspace_bytes(1, g.n, per);
     }
+    if (g.group == 1) {
+        const int64_t parts = dense_bwd_weight_partials(g.n, g.c, g.m, g.kh, g.kw, g.oh, g.ow, g.h, g.w);
+        const int64_t per = (int64_t)g.m * g.c * g.kh * g.kw;
+        if (parts > 1) return (size_t)parts * per * sizeof(float) + dmlhip_reduce_workspace_bytes(1, parts, per);
+    }
     return 0;
 }
 
@@ -615,7 +623,10 @@ int dmlhip_conv2d_backward_weight_f32(const dmlhip_conv2d_desc* d, const void* x
     DML_REQUIRE(red == 0 || (x && dy), DMLHIP_ERR_NULL, "conv2d_backward_weight: NULL tensor pointer");
     DML_REQUIRE(total <= 2147483647LL, DMLHIP_ERR_SHAPE, "conv2d_backward_weight: too many weights");
     hipStream_t st = (hipStream_t)stream;
-    if ((is_pointwise(g) || is_depthwise_grad(g)) && red > 0) {
+    const int64_t dense_parts =
+        (!is_pointwise(g) && g.group == 1 && red > 0)
+            ? dense_bwd_weight_partials(g.n, g.c, g.m, g.kh, g.kw, g.oh, g.ow, g.h, g.w) : 0;
+    if ((is_pointwise(g) || is_depthwise_grad(g) || dense_parts > 0) && red > 0) {
         const size_t need = dmlhip_conv2d_backward_weight_workspace_bytes(d);
         DML_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), DMLHIP_ERR_WORKSPACE,
                     "conv2d_backward_weight: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
@@ -630,6 +641,17 @@ int dmlhip_conv2d_backward_weight_f32(const dmlhip_conv2d_desc* d, const void* x
         if (g.n == 1) return 0;
         const size_t part_bytes = (size_t)g.n * per * sizeof(float);
         return dmlhip_reduce_f32(DMLHIP_RSUM, part, dw, DMLHIP_F32, 1, g.n, per, (char*)workspace + part_bytes,
+                                 workspace_bytes - part_bytes, stream);
+    }
+    if (dense_parts > 0) {
+        // implicit GEMM over ranges of the (image, pixel) space, then their sum in a fixed order
+        float* part = dense_parts > 1 ? (float*)workspace : (float*)dw;
+        if (int e = launch_dense_bwd_weight((const float*)x, (const float*)dy, part, g.n, g.c, g.h, g.w, g.m, g.kh, g.kw,
+                                            g.sh, g.sw, g.ph, g.pw, g.dh, g.dw, g.oh, g.ow, st))
+            return e;
+        if (dense_parts == 1) return 0;
+        const size_t part_bytes = (size_t)dense_parts * total * sizeof(float);
+        return dmlhip_reduce_f32(DMLHIP_RSUM, part, dw, DMLHIP_F32, 1, dense_parts, total, (char*)workspace + part_bytes,
                                  workspace_bytes - part_bytes, stream);
     }
     if (is_pointwise(g) && red > 0) {

@@ -233,6 +233,164 @@ __global__ __launch_bounds__(256, 2) void pointwise_bwd_weight_kernel(const PwGr
     }
 }
 
+// ---------------------------------------------------------------- dense KxK, weight gradient
+// dW[m, j] = sum_{n, p} dY[n, m, p] * X[n, c(j), oy(p) s - pad + hy(j) d, ox(p) s - pad + hx(j) d] with j = (c, hy, hx)
+// flattened as in W. Same scheme as the pointwise kernel above — 64-pixel slabs, accumulators' rows = output
+// channels, columns = 32 consecutive j — but the slab of the second operand is gathered: row j of it is X shifted by
+// j's tap. A workgroup covers a range of images and a range of each image's pixels.
+struct DenseGradArgs {
+    const float* x;
+    const float* dy;
+    float* part;          // [groups of images * pixel ranges][m * c * kh * kw]
+    int n, c, h, w, m, kh, kw, sh, sw, ph, pw, dh, dw, oh, ow;
+    int imgs_per_group, chunk_px, chunks_per_img;
+    int a_groups, b_tiles;   // workgroups = a_groups * b_tiles * (image groups * pixel ranges); the first two vary fastest
+};
+
+__device__ __forceinline__ int small_div(int a, int b, float inv_b) {   // a / b for 0 <= a < 2^22
+    int q = (int)((float)a * inv_b);
+    const int r = a - q * b;
+    q += (r >= b) - (r < 0);
+    return q;
+}
+
+template <int TA>
+__global__ __launch_bounds__(256, 2) void dense_bwd_weight_kernel(const DenseGradArgs g) {
+    extern __shared__ __attribute__((aligned(16))) float dg_lds[];
+    constexpr int RA = TA * 8, RB = 8;               // rows of dY / of the gathered operand a thread moves per slab
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, hh = lane >> 5;
+    const int ytiles = g.a_groups * g.b_tiles;
+    const int yt = blockIdx.x % ytiles, xb = blockIdx.x / ytiles;
+    const int ag = yt % g.a_groups, bt = yt / g.a_groups;
+    const int grp = xb / g.chunks_per_img, chunk = xb - grp * g.chunks_per_img;
+    const int a0 = ag * TA * 32, b0 = bt * 32;
+    const int ohw = g.oh * g.ow, kk = g.kh * g.kw, jn = g.c * kk, in_plane = g.h * g.w;
+    const int p_begin = chunk * g.chunk_px, p_end = min(p_begin + g.chunk_px, ohw);
+    const int n_begin = grp * g.imgs_per_group, n_end = min(n_begin + g.imgs_per_group, g.n);
+    const float inv_ow = 1.0f / (float)g.ow, inv_kk = 1.0f / (float)kk, inv_kw = 1.0f / (float)g.kw;
+
+    // the rows of the gathered operand this thread fills: channel offset and tap shift of j = b0 + wave + 4 e
+    int coff[RB], tshift[RB];
+#pragma unroll
+    for (int e = 0; e < RB; ++e) {
+        const int j = b0 + wave + 4 * e;
+        const int ch = small_div(min(j, jn - 1), kk, inv_kk), tap = min(j, jn - 1) - ch * kk;
+        const int hy = small_div(tap, g.kw, inv_kw), hx = tap - hy * g.kw;
+        coff[e] = j < jn ? ch * in_plane : -1;
+        tshift[e] = ((hy * g.dh) << 16) | (hx * g.dw);
+    }
+
+    floatx16 acc[TA];
+#pragma unroll
+    for (int t = 0; t < TA; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+
+    float pa[RA], pb[RB];
+    auto fetch = [&](int img, int p0) {
+        const int p = p0 + lane;
+        const bool pok = p < p_end;
+        const int pc = pok ? p : p_begin;
+        const float* dyn = g.dy + (size_t)img * g.m * ohw + pc;
+#pragma unroll
+        for (int e = 0; e < RA; ++e) {
+            const int row = a0 + wave + 4 * e;
+            const bool ok = pok && row < g.m;
+            pa[e] = dyn[(size_t)(ok ? row : 0) * ohw];
+            pa[e] = ok ? pa[e] : 0.f;
+        }
+        const int oy = small_div(pc, g.ow, inv_ow), ox = pc - oy * g.ow;
+        const int by = oy * g.sh - g.ph, bx = ox * g.sw - g.pw;
+        const float* xn = g.x + (size_t)img * g.c * in_plane;
+#pragma unroll
+        for (int e = 0; e < RB; ++e) {
+            const int iy = by + (tshift[e] >> 16), ix = bx + (tshift[e] & 0xffff);
+            const bool ok = pok && coff[e] >= 0 && iy >= 0 && iy < g.h && ix >= 0 && ix < g.w;
+            pb[e] = xn[ok ? coff[e] + iy * g.w + ix : 0];
+            pb[e] = ok ? pb[e] : 0.f;
+        }
+    };
+    int img = n_begin, p0 = p_begin;
+    const bool any = n_begin < n_end && p_begin < p_end;
+    if (any) fetch(img, p0);
+    while (any && img < n_end) {
+        __syncthreads();      // the previous slab has been consumed
+#pragma unroll
+        for (int e = 0; e < RA; ++e) dg_lds[(wave + 4 * e) * kPitch + lane] = pa[e];
+#pragma unroll
+        for (int e = 0; e < RB; ++e) dg_lds[(TA * 32 + wave + 4 * e) * kPitch + lane] = pb[e];
+        __syncthreads();
+        p0 += kSlab;
+        if (p0 >= p_end) {
+            p0 = p_begin;
+            ++img;
+        }
+        if (img < n_end) fetch(img, p0);     // in flight while this slab is multiplied
+        const float* bl = dg_lds + (TA * 32 + l32) * kPitch + wave * 16 + hh;
+        const float* al = dg_lds + l32 * kPitch + wave * 16 + hh;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const float bv = bl[2 * ks];
+#pragma unroll
+            for (int t = 0; t < TA; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(al[t * 32 * kPitch + 2 * ks], bv, acc[t], 0, 0, 0);
+        }
+    }
+    float* out = g.part + (size_t)xb * g.m * jn;
+#pragma unroll
+    for (int t = 0; t < TA; ++t) {
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dg_lds[wave * 1024 + e * 64 + lane] = acc[t][e];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int q = r * 256 + threadIdx.x;
+            const float s = (dg_lds[q] + dg_lds[1024 + q]) + (dg_lds[2048 + q] + dg_lds[3072 + q]);
+            const int e = q >> 6, ln = q & 63;
+            const int row_a = a0 + t * 32 + (e >> 2) * 8 + (ln >> 5) * 4 + (e & 3);
+            const int row_b = b0 + (ln & 31);
+            if (row_a < g.m && row_b < jn) out[(size_t)row_a * jn + row_b] = s;
+        }
+    }
+}
+
+struct DenseGradPlan {
+    int ta, a_groups, b_tiles, imgs_per_group, chunk_px, chunks_per_img;
+    int64_t xblocks;
+};
+
+bool plan_dense_bwd_weight(int n, int c, int m, int kk, int oh, int ow, int h, int w, DenseGradPlan* pl) {
+    const int64_t ohw = (int64_t)oh * ow, jn = (int64_t)c * kk;
+    if (n < 1 || c < 1 || m < 1 || ohw < 64 || ohw > (1 << 22) || (int64_t)h * w > (1 << 28) || jn > (1 << 22)) return false;
+    if ((int64_t)n * ohw * m * jn < (1LL << 24)) return false;          // tiny: the direct kernel
+    const int tm = (int)ceil_div(m, 32);
+    pl->a_groups = (tm + 7) / 8;
+    pl->ta = (tm + pl->a_groups - 1) / pl->a_groups;
+    pl->b_tiles = (int)ceil_div(jn, (int64_t)32);
+    const int64_t ytiles = (int64_t)pl->a_groups * pl->b_tiles;
+    int64_t want = ceil_div((int64_t)2048, ytiles);                      // ranges of the (image, pixel) space
+    const int64_t cap = (64LL << 20) / ((int64_t)m * jn);                // at most 256 MiB of per-range results
+    if (want > cap) want = cap;
+    if (want < 1) want = 1;
+    if (want >= n) {
+        pl->imgs_per_group = 1;
+        int64_t per_img = want / n;
+        const int64_t max_per_img = ceil_div(ohw, (int64_t)256);
+        if (per_img > max_per_img) per_img = max_per_img;
+        pl->chunk_px = (int)(ceil_div(ceil_div(ohw, per_img), (int64_t)kSlab) * kSlab);
+        pl->chunks_per_img = (int)ceil_div(ohw, (int64_t)pl->chunk_px);
+        pl->xblocks = (int64_t)n * pl->chunks_per_img;
+    } else {
+        pl->imgs_per_group = (int)ceil_div((int64_t)n, want);
+        pl->chunk_px = (int)(ceil_div(ohw, (int64_t)kSlab) * kSlab);
+        pl->chunks_per_img = 1;
+        pl->xblocks = ceil_div((int64_t)n, (int64_t)pl->imgs_per_group);
+    }
+    return pl->xblocks * ytiles <= 2147483647LL && pl->xblocks * (int64_t)m * jn < (1LL << 31);
+}
+
 struct PwGradPlan {
     bool swap;            // a = X (rows = input channels) instead of a = dY
     int ta, a_groups, b_tiles, chunk_px, chunks_per_img;
@@ -309,6 +467,49 @@ int launch_depthwise_bwd_weight(const float* x, const float* dy, float* part, in
 #undef DML_DWW
     set_error("conv2d_backward_weight: no depthwise kernel for k %d stride %d", k, s);
     return DMLHIP_ERR_UNSUPPORTED;
+}
+
+// number of per-workgroup-range results (each m * c * kh * kw floats) of the dense weight gradient; 0 = not applicable
+int64_t dense_bwd_weight_partials(int n, int c, int m, int kh, int kw, int oh, int ow, int h, int w) {
+    DenseGradPlan pl;
+    return plan_dense_bwd_weight(n, c, m, kh * kw, oh, ow, h, w, &pl) ? pl.xblocks : 0;
+}
+
+int launch_dense_bwd_weight(const float* x, const float* dy, float* part, int n, int c, int h, int w, int m, int kh, int kw,
+                            int sh, int sw, int ph, int pw, int dh, int dw, int oh, int ow, hipStream_t st) {
+    DenseGradPlan pl;
+    DML_REQUIRE(plan_dense_bwd_weight(n, c, m, kh * kw, oh, ow, h, w, &pl), DMLHIP_ERR_UNSUPPORTED,
+                "conv2d_backward_weight: the implicit-GEMM kernel does not apply");
+    DML_REQUIRE(kh * dh < 32768 && kw * dw < 32768, DMLHIP_ERR_UNSUPPORTED, "conv2d_backward_weight: stencil too large");
+    DenseGradArgs g;
+    g.x = x; g.dy = dy; g.part = part;
+    g.n = n; g.c = c; g.h = h; g.w = w; g.m = m; g.kh = kh; g.kw = kw; g.sh = sh; g.sw = sw; g.ph = ph; g.pw = pw;
+    g.dh = dh; g.dw = dw; g.oh = oh; g.ow = ow;
+    g.imgs_per_group = pl.imgs_per_group; g.chunk_px = pl.chunk_px; g.chunks_per_img = pl.chunks_per_img;
+    g.a_groups = pl.a_groups; g.b_tiles = pl.b_tiles;
+    const unsigned blocks = (unsigned)(pl.xblocks * pl.a_groups * pl.b_tiles);
+    const size_t lds = (size_t)(pl.ta + 1) * 32 * kPitch * sizeof(float);
+#define DML_DG(TA)                                                                                                     \
+    case TA: {                                                                                                         \
+        auto kern = dense_bwd_weight_kernel<TA>;                                                                       \
+        if (lds > 64 * 1024) {                                                                                         \
+            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+            if (e != hipSuccess) {                                                                                     \
+                set_error("conv2d_backward_weight: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));  \
+                return (int)e;                                                                                         \
+            }                                                                                                          \
+        }                                                                                                              \
+        hipLaunchKernelGGL(kern, blocks, 256, lds, st, g);                                                             \
+        break;                                                                                                         \
+    }
+    switch (pl.ta) {
+        DML_DG(1) DML_DG(2) DML_DG(3) DML_DG(4) DML_DG(5) DML_DG(6) DML_DG(7) DML_DG(8)
+        default:
+            set_error("conv2d_backward_weight: bad block count %d", pl.ta);
+            return DMLHIP_ERR_UNSUPPORTED;
+    }
+#undef DML_DG
+    return launch_status("conv2d_backward_weight(implicit GEMM)");
 }
 
 // number of per-workgroup results (each m * c floats) the pointwise weight gradient writes; 0 = not applicable
