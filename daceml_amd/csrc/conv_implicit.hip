@@ -218,7 +218,7 @@ bool plan_implicit(const ConvGeom& g, int ids_h, int ids_w, int wflip, ImplicitP
     for (int pt = 2; pt >= 1; --pt) {
         const int px = 128 * pt;
         const int64_t blocks = ceil_div(ohw, (int64_t)px) * g.n * ceil_div(g.m, mt * 32);
-        if (pt == 2 && blocks < 768) continue;          // few workgroups: smaller ones fill the chip better
+        if (pt == 2 && blocks < 384) continue;          // few workgroups: smaller ones fill the chip better
         // output rows a block of px consecutive pixels can span, then the input rows under them
         const int span = (int)((px - 1 + g.ow - 1) / g.ow) + 1;
         const int rows = span < g.oh ? span : g.oh;
