@@ -88,6 +88,9 @@ __global__ __launch_bounds__(256, (MT * PT <= 2 ? 4 : 2)) void conv_implicit_f32
         // rectangle: kIgChunk channels x prow rows x pwid columns, zeros outside the image and past the last channel.
         // A thread resolves (row, column) of two rectangle positions once and loads them for all channels of the
         // chunk: sixteen loads in flight per round trip.
+        // uniform bases + 32-bit offsets: a chunk of X and the weight tensor have fewer than 2^31 elements
+        const float* xc = xn + (size_t)kc * in_plane;
+        const float* wc = w + (size_t)kc * (g.wflip ? g.m * kk : kk);
         for (int i0 = 0; i0 < rect; i0 += 512) {
             int pos[2], off[2];
             bool ok[2];
@@ -111,7 +114,7 @@ __global__ __launch_bounds__(256, (MT * PT <= 2 ? 4 : 2)) void conv_implicit_f32
             for (int u = 0; u < 2; ++u)
 #pragma unroll
                 for (int ch = 0; ch < kIgChunk; ++ch)
-                    v[u][ch] = xn[(size_t)(kc + min(ch, cl - 1)) * in_plane + off[u]];
+                    v[u][ch] = xc[(uint32_t)(min(ch, cl - 1) * in_plane + off[u])];
 #pragma unroll
             for (int u = 0; u < 2; ++u)
                 if (pos[u] < rect) {
@@ -119,28 +122,33 @@ __global__ __launch_bounds__(256, (MT * PT <= 2 ? 4 : 2)) void conv_implicit_f32
                     for (int ch = 0; ch < kIgChunk; ++ch) xs[ch * g.plane + pos[u]] = (ok[u] && ch < cl) ? v[u][ch] : 0.f;
                 }
         }
-        // weights: the chunk's cl * kh * kw values of an output channel are contiguous in W; eight loads per round trip
-        const int wtotal = MT * 32 * wrow;
-        for (int i0 = 0; i0 < wtotal; i0 += 8 * 256) {
-            float v[8];
-            int dst[8];
+        // weights: the chunk's cl * kh * kw values of an output channel are contiguous in W. A thread stays on one
+        // output channel and strides over k, so source and LDS index are a base plus k; six loads per round trip
+        {
+            constexpr int TPR = 8 / MT;                      // threads per output channel
+            const int row = (int)threadIdx.x / TPR, q = (int)threadIdx.x % TPR;
+            const bool rok = m0 + row < g.m;
+            const int klim = rok ? cl * kk : 0;              // k at and beyond it is zero-filled
+            const int sbase = (m0 + (rok ? row : 0)) * (g.wflip ? kk : g.c * kk);
+            float* wdst = ws + row * g.wpitch;
+            for (int k0 = q; k0 < wrow; k0 += 6 * TPR) {
+                float v[6];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int i = i0 + u * 256 + (int)threadIdx.x;
-                const int row = fast_div(i, wrow, inv_wrow), k = i - row * wrow;
-                const bool ok = i < wtotal && m0 + row < g.m && k < cl * kk;
-                size_t src = ((size_t)(m0 + row) * g.c + kc) * kk + k;
-                if (g.wflip) {
-                    const int ch = fast_div(k, kk, inv_kk), tap = k - ch * kk;
-                    src = ((size_t)(kc + ch) * g.m + m0 + row) * kk + (kk - 1 - tap);
+                for (int u = 0; u < 6; ++u) {
+                    const int k = k0 + u * TPR;
+                    const bool ok = k < klim;
+                    int src = sbase + k;
+                    if (g.wflip) {
+                        const int ch = fast_div(ok ? k : 0, kk, inv_kk), tap = (ok ? k : 0) - ch * kk;
+                        src = sbase + ch * g.m * kk + (kk - 1 - tap);
+                    }
+                    v[u] = wc[(uint32_t)(ok ? src : 0)];
+                    v[u] = ok ? v[u] : 0.f;
                 }
-                v[u] = w[ok ? src : 0];
-                v[u] = ok ? v[u] : 0.f;
-                dst[u] = i < wtotal ? row * g.wpitch + k : -1;
-            }
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (dst[u] >= 0) ws[dst[u]] = v[u];
+                for (int u = 0; u < 6; ++u)
+                    if (k0 + u * TPR < wrow) wdst[k0 + u * TPR] = v[u];
+            }
         }
         __syncthreads();
         for (int hy = 0; hy < g.kh; ++hy)
@@ -225,6 +233,7 @@ bool plan_implicit(const ConvGeom& g, int ids_h, int ids_w, int wflip, ImplicitP
         a.prow = (rows - 1) * g.sh + (g.kh - 1) * g.dh + 1;
         const int64_t rect = (int64_t)a.prow * a.pwid;
         if (rect > (1 << 20) || (int64_t)mt * 32 * kIgChunk * g.kh * g.kw > (1 << 20)) continue;
+        if ((int64_t)g.m * g.c * g.kh * g.kw >= (1LL << 31) || (int64_t)kIgChunk * g.h * g.w >= (1LL << 31)) continue;
         a.plane = (int)(ceil_div(rect + 32, (int64_t)64) * 64 - 32);   // >= rect, == 32 (mod 64)
         const size_t lds = ((size_t)kIgChunk * a.plane + (size_t)mt * 32 * a.wpitch + mt * 32) * sizeof(float);
         if (lds > 72 * 1024) continue;                  // two workgroups per CU
