@@ -74,8 +74,8 @@ __global__ __launch_bounds__(kFusedThreads) void expand_depthwise_kernel(const f
     const int npix = a.ih * a.w;
     const int ntiles = (npix + 31) / 32;
     const int j = lane & 31, hh = lane >> 5;
-    const size_t plane = (size_t)a.h * a.w;
-    const float* xn = x + (size_t)n * a.cin * plane + (size_t)hh * plane;
+    const int plane = a.h * a.w;
+    const float* xn = x + (size_t)n * a.cin * plane;     // uniform base; per-lane offsets fit 32 bits (checked on the host)
     float bias1[16];
 #pragma unroll
     for (int e = 0; e < 16; ++e) bias1[e] = 0.f;
@@ -87,24 +87,24 @@ __global__ __launch_bounds__(kFusedThreads) void expand_depthwise_kernel(const f
     constexpr int kWaves = kFusedThreads / 64;
     const int my_tiles = wave < ntiles ? (ntiles - wave + kWaves - 1) / kWaves : 0;
     const int steps = my_tiles * chunks;
-    auto pixel_ptr = [&](int t) -> const float* {
+    auto pixel_off = [&](int t) -> uint32_t {
         const int p = min(t * 32 + j, npix - 1);
         const int row = p / a.w;
-        return xn + (size_t)min(max(iy0 + row, 0), a.h - 1) * a.w + (p - row * a.w);
+        return (uint32_t)(hh * plane + min(max(iy0 + row, 0), a.h - 1) * a.w + (p - row * a.w));
     };
     // ring of kDepth chunks (16 input channels each) in flight per wavefront
     constexpr int kDepth = 4;
     float ring[kDepth][8];
     int it = wave, ich = 0;
-    const float* ixp = steps > 0 ? pixel_ptr(it) : xn;
+    uint32_t ixo = steps > 0 ? pixel_off(it) : 0u;
     auto issue = [&](float (&dst)[8], int k) {
         if (k >= steps) return;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) dst[s] = ixp[(size_t)(ich * 16 + 2 * s) * plane];
+        for (int s = 0; s < 8; ++s) dst[s] = xn[ixo + (uint32_t)((ich * 16 + 2 * s) * plane)];
         if (++ich == chunks) {
             ich = 0;
             it += kWaves;
-            if (k + 1 < steps) ixp = pixel_ptr(it);
+            if (k + 1 < steps) ixo = pixel_off(it);
         }
     };
 #pragma unroll
@@ -212,7 +212,7 @@ int dmlhip_conv2d_expand_depthwise_f32(const dmlhip_conv2d_desc* pw, const dmlhi
                 "conv2d_expand_depthwise: the depthwise input must be the pointwise output");
     DML_REQUIRE(pw->c % 16 == 0 && pw->m % kCB == 0, DMLHIP_ERR_UNSUPPORTED,
                 "conv2d_expand_depthwise: needs input channels %% 16 == 0 and expanded channels %% 32 == 0");
-    DML_REQUIRE(pw->h * pw->w < (1LL << 30) && pw->w <= 4096, DMLHIP_ERR_UNSUPPORTED,
+    DML_REQUIRE(pw->h * pw->w < (1LL << 30) && pw->w <= 4096 && pw->c * pw->h * pw->w < (1LL << 31), DMLHIP_ERR_UNSUPPORTED,
                 "conv2d_expand_depthwise: image too large");
     if (pw->n == 0) return 0;
     DML_REQUIRE(x && w_pw && w_dw && y, DMLHIP_ERR_NULL, "conv2d_expand_depthwise: NULL tensor pointer");
