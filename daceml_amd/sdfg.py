@@ -39,6 +39,8 @@ class Array:
         self.strides = tuple(int(s) for s in strides) if strides is not None else contiguous_strides(self.shape)
         self.view_of = view_of
         self.view_offset = int(view_offset)
+        #: a transient that holds data across calls (AllocationLifetime.Persistent in DaCe): a parameter snapshot
+        self.persistent = False
 
     @property
     def total_size(self) -> int:

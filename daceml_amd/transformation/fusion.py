@@ -66,7 +66,8 @@ def _is_op(node, name: str) -> bool:
 def _internal(sdfg: SDFG, state: SDFGState, array: str, n_consumers: int = 1) -> bool:
     """A transient that only the matched pattern reads."""
     d = sdfg.arrays[array]
-    return d.transient and d.view_of is None and len(_consumers(state, array)) == n_consumers
+    return (d.transient and not getattr(d, "persistent", False) and d.view_of is None
+            and len(_consumers(state, array)) == n_consumers)
 
 
 def _scalar_const(sdfg: SDFG, array: Optional[str]) -> Optional[float]:

@@ -413,6 +413,47 @@ def test_module_with_two_inputs_two_outputs_and_a_skipped_gradient():
     assert_close(host(a2.grad), ar2.grad.cpu().numpy(), torch.float32, "partial output gradient", rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.gpu
+def test_parameter_to_transient():
+    """The reference's own test of this transformation (tests/transformation/test_param_to_transient.py): a Linear
+    layer whose weight becomes a buffer of the compiled program. On top of it: the program works on a snapshot (a
+    later change of the nn.Parameter is not seen) and the weight is no longer an argument."""
+    from daceml_amd.transformation import parameter_to_transient
+
+    class Module(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc1 = nn.Linear(10, 3)
+
+        def forward(self, x):
+            return self.fc1(x)
+
+    torch.manual_seed(3)
+    pt_module = Module().cuda()
+    dace_module = Module().cuda()
+    dace_module.load_state_dict(pt_module.state_dict())
+    x = torch.rand(2, 10).cuda()
+    plain = DaceModule(dace_module)
+    assert torch.allclose(plain(x), pt_module(x), rtol=1e-5, atol=1e-6)
+    assert "fc1DOTweight" in plain.compiled.arglist()
+
+    wrapped = DaceModule(dace_module)
+    wrapped.append_post_onnx_hook("param_to_transient", lambda model: parameter_to_transient(model, "fc1.weight"))
+    want = pt_module(x)
+    assert torch.allclose(wrapped(x), want, rtol=1e-5, atol=1e-6)
+    assert "fc1DOTweight" not in wrapped.compiled.arglist() and "fc1.weight" not in wrapped.dace_model.inputs
+    assert "init_fc1.weight" in wrapped.post_compile_hooks
+    with torch.no_grad():
+        dace_module.fc1.weight.mul_(2.0)          # the snapshot does not follow the parameter ...
+        dace_module.fc1.bias.add_(1.0)            # ... an ordinary parameter does
+    assert torch.allclose(wrapped(x), want + 1.0, rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        again = DaceModule(dace_module)
+        again.append_post_onnx_hook("twice", lambda model: (parameter_to_transient(model, "fc1.weight"),
+                                                           parameter_to_transient(model, "fc1.weight")))
+        again(x)
+
+
 class MBConvBN(nn.Module):
     """MBConv block as efficientnet_pytorch builds it (what tests/autodiff/torch/test_efficientnet_block_backward.py
     trains): every conv without bias followed by BatchNorm, swish as x * sigmoid(x), squeeze-excite with biases."""
