@@ -26,3 +26,5 @@ class _Module(types.ModuleType):
 
 
 sys.modules[__name__].__class__ = _Module
+
+from .onnx_importer import ONNXModel  # noqa: E402,F401  (daceml/onnx/__init__.py:5)
