@@ -50,6 +50,26 @@ def build():
     f["reduce_x"] = r.standard_normal((6, 5, 8))
     f["reduce_sum_01"] = O.reduce_sum(f["reduce_x"], [0, 1], 0)
     f["reduce_mean_2"] = O.reduce_mean(f["reduce_x"], [2], 1)
+    # later additions draw after everything above, so the earlier vectors keep their values
+    x = r.standard_normal((4, 3, 5, 6)) * 2 + 1
+    sc, bi = r.uniform(0.5, 1.5, 3), r.standard_normal(3) * 0.1
+    rm, rv = r.standard_normal(3) * 0.2, r.uniform(0.5, 1.5, 3)
+    y, om, ov, sm, sv = O.batchnorm_training(x, sc, bi, rm, rv, 1e-5, 0.9)
+    dy = r.standard_normal(x.shape)
+    dx, dsc, dbi = O.batchnorm_backward(dy, x, sc, sm, sv, 1e-5)
+    f.update(bn_x=x, bn_scale=sc, bn_bias=bi, bn_mean=rm, bn_var=rv, bn_y=y, bn_out_mean=om, bn_out_var=ov,
+             bn_saved_mean=sm, bn_saved_var=sv, bn_dy=dy, bn_dx=dx, bn_dscale=dsc, bn_dbias=dbi,
+             bn_y_inference=O.batchnorm_inference(x, sc, bi, rm, rv, 1e-5))
+    dy = r.standard_normal(f["conv_y"].shape)
+    dx, dw, _ = O.conv2d_backward(f["conv_x"], f["conv_w"], dy, strides=(2, 2))
+    f.update(conv_dy=dy, conv_dx=dx, conv_dw=dw)
+    # the expand + depthwise stages of an MBConv block: 1x1 conv + swish, then 3x3 depthwise stride 2 pad 1 + swish
+    x = r.standard_normal((1, 16, 6, 7))
+    w1, b1 = r.standard_normal((32, 16, 1, 1)) * 0.35, r.standard_normal(32) * 0.1
+    w2, b2 = r.standard_normal((32, 1, 3, 3)) * 0.45, r.standard_normal(32) * 0.1
+    mid = O.swish(O.conv2d(x, w1, b1))
+    f.update(mb_x=x, mb_w1=w1, mb_b1=b1, mb_w2=w2, mb_b2=b2,
+             mb_y=O.swish(O.conv2d(mid, w2, b2, (2, 2), (1, 1, 1, 1), (1, 1), 32)))
     return f
 
 

@@ -60,9 +60,25 @@ def test_kernels_against_fixtures(dtype):
                  "matmul", atol=None if dtype == torch.float16 else 4e-6)
     assert_close(host(K.reduce(L.RSUM, d("reduce_x"), [0, 1], False, out_dtype=torch.float32)),
                  ref(lambda x: O.reduce_sum(x, [0, 1], 0), "reduce_x"), torch.float32, "reduce_sum", atol=1e-5)
+    y, om, ov, sm, sv = K.batchnorm_training(d("bn_x"), d("bn_scale"), d("bn_bias"), d("bn_mean"), d("bn_var"), 1e-5, 0.9)
+    names = ("bn_x", "bn_scale", "bn_bias", "bn_mean", "bn_var")
+    want = ref(lambda *a: O.batchnorm_training(*a, 1e-5, 0.9), *names)
+    for got, w, what in zip((y, om, ov, sm, sv), want, ("y", "running mean", "running variance", "mean", "variance")):
+        assert_close(host(got), w, dtype, "batchnorm " + what)
+    assert_close(host(K.batchnorm_inference(*[d(n) for n in names], 1e-5)),
+                 ref(lambda *a: O.batchnorm_inference(*a, 1e-5), *names), dtype, "batchnorm inference")
     if dtype == torch.float32:
         assert_close(host(K.conv2d(d("conv_x"), d("conv_w"), None, strides=(2, 2))), FIX["conv_y"], dtype, "conv C1",
                      rtol=1e-5, atol=1e-5)
+        dx, dw = K.conv2d_backward(d("conv_x"), d("conv_w"), d("conv_dy"), (2, 2))
+        assert_close(host(dx), FIX["conv_dx"], dtype, "conv C1 dx", rtol=1e-5, atol=1e-5)
+        assert_close(host(dw), FIX["conv_dw"], dtype, "conv C1 dw", rtol=1e-5, atol=2e-5)
+        dx, dsc, dbi = K.batchnorm_backward(d("bn_dy"), d("bn_x"), d("bn_scale"), d("bn_saved_mean"), d("bn_saved_var"), 1e-5)
+        for got, name in ((dx, "bn_dx"), (dsc, "bn_dscale"), (dbi, "bn_dbias")):
+            assert_close(host(got), FIX[name], dtype, name, rtol=1e-4, atol=1e-5)
+        got = K.conv2d_expand_depthwise(d("mb_x"), d("mb_w1"), d("mb_b1"), d("mb_w2"), d("mb_b2"), stride=2,
+                                        act_pw=L.ACT_SWISH, act_dw=L.ACT_SWISH)
+        assert_close(host(got), FIX["mb_y"], dtype, "expand + depthwise", rtol=1e-5, atol=4e-6)
     else:
         out, lse = K.attention(d("attn_q"), d("attn_k"), d("attn_v"), 0.125)
         want, want_lse = ref(lambda q, k, v: O.attention(q, k, v, 0.125), "attn_q", "attn_k", "attn_v")
