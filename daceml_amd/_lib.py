@@ -78,6 +78,14 @@ SIGNATURES = {
     "dmlhip_batchnorm_training_f32": (c_int, [_P] * 10 + [c_int64, c_int64, c_int64, c_float, c_float, _P, c_size_t, _P]),
     "dmlhip_batchnorm_backward_f16": (c_int, [_P] * 8 + [c_int64, c_int64, c_int64, c_float, _P, c_size_t, _P]),
     "dmlhip_batchnorm_backward_f32": (c_int, [_P] * 8 + [c_int64, c_int64, c_int64, c_float, _P, c_size_t, _P]),
+    "dmlhip_batchnorm_inference_act_f16": (c_int, [_P] * 6 + [c_int64, c_int64, c_int64, c_float, c_int, _P]),
+    "dmlhip_batchnorm_inference_act_f32": (c_int, [_P] * 6 + [c_int64, c_int64, c_int64, c_float, c_int, _P]),
+    "dmlhip_batchnorm_training_act_f16": (c_int, [_P] * 10 + [c_int64, c_int64, c_int64, c_float, c_float, c_int, _P,
+                                                              c_size_t, _P]),
+    "dmlhip_batchnorm_training_act_f32": (c_int, [_P] * 10 + [c_int64, c_int64, c_int64, c_float, c_float, c_int, _P,
+                                                              c_size_t, _P]),
+    "dmlhip_batchnorm_backward_act_f16": (c_int, [_P] * 9 + [c_int64, c_int64, c_int64, c_float, c_int, _P, c_size_t, _P]),
+    "dmlhip_batchnorm_backward_act_f32": (c_int, [_P] * 9 + [c_int64, c_int64, c_int64, c_float, c_int, _P, c_size_t, _P]),
     "dmlhip_binary_f16": (c_int, [c_int, _P, _P, _P, c_int, _I64P, _I64P, _I64P, _P]),
     "dmlhip_binary_f32": (c_int, [c_int, _P, _P, _P, c_int, _I64P, _I64P, _I64P, _P]),
     "dmlhip_unary_f16": (c_int, [c_int, _P, _P, c_int64, c_float, _P]),

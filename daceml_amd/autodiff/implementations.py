@@ -259,7 +259,8 @@ class HipLayerNormalizationBackward(BackwardImplementation):
 class HipBatchNormalizationBackward(BackwardImplementation):
     """Training-mode BatchNormalization: one BatchNormalizationGrad node reading X, scale and the statistics the
     forward node saved (CuDNNBatchNormBackward, daceml/autodiff/implementations/onnx_ops.py:1268-1510). The
-    running statistics carry no gradient."""
+    running statistics carry no gradient. A forward node with a fused activation hands the activation and its bias to
+    the gradient node, which recomputes the normalised value."""
     @staticmethod
     def backward_can_be_applied(node, state, sdfg) -> bool:
         outs = {e.src_conn for e in state.out_edges(node)}
@@ -267,9 +268,13 @@ class HipBatchNormalizationBackward(BackwardImplementation):
 
     @staticmethod
     def backward(forward_node, context, given_gradients, required_gradients):
-        g = _new(context, "BatchNormalizationGrad", forward_node.label + "_backward", epsilon=forward_node.epsilon)
+        act = getattr(forward_node, "_activation", "none")
+        g = _new(context, "BatchNormalizationGrad", forward_node.label + "_backward", epsilon=forward_node.epsilon,
+                 activation=act)
         connect_input_from_forward(forward_node, g, context, "X")
         connect_input_from_forward(forward_node, g, context, "scale")
+        if act != "none":
+            connect_input_from_forward(forward_node, g, context, "B")
         connect_output_from_forward(forward_node, g, context, "saved_mean")
         connect_output_from_forward(forward_node, g, context, "saved_var")
         req = {"X": "dX", "scale": "dscale", "B": "dB"}

@@ -7,6 +7,7 @@
 // channel's first element (shifted-data variance: no cancellation against a large mean), written as per-workgroup
 // partials; the second kernel of each pair starts by combining its channel's partials (S <= kMaxSplit of them).
 #include <initializer_list>
+#include <type_traits>
 
 #include "common.h"
 
@@ -67,6 +68,23 @@ __device__ __forceinline__ void store_piece(T* p, int64_t idx, int count, const 
     }
 }
 
+// The activation that may follow the normalisation inside the same kernel (NONE, RELU, SWISH), and its derivative
+// with respect to the normalised value z — the backward kernels recompute z from X instead of reading a stored copy.
+template <int ACT>
+__device__ __forceinline__ float bn_act(float z) {
+    if constexpr (ACT == DMLHIP_ACT_SWISH) return z * sigmoid_epilogue_f(z);
+    else if constexpr (ACT == DMLHIP_ACT_RELU) return fmaxf(z, 0.f);
+    else return z;
+}
+template <int ACT>
+__device__ __forceinline__ float bn_act_grad(float z) {
+    if constexpr (ACT == DMLHIP_ACT_SWISH) {
+        const float sg = sigmoid_epilogue_f(z);
+        return sg * (1.0f + z * (1.0f - sg));
+    } else if constexpr (ACT == DMLHIP_ACT_RELU) return z > 0.f ? 1.f : 0.f;
+    else return 1.f;
+}
+
 // partial[(c * S + s) * 2 + {0, 1}] = sum of (x - K), sum of (x - K)^2 over the workgroup's chunks
 template <typename T>
 __global__ __launch_bounds__(kThreads) void bn_stats_kernel(const T* __restrict__ x, float* __restrict__ partial,
@@ -114,7 +132,7 @@ __device__ __forceinline__ void combine_partials(const float* partial, int c, in
 
 // TRAINING: statistics from `partial`; workgroup s == 0 also writes the saved and the running statistics.
 // otherwise: statistics are the given mean / var.
-template <typename T, bool TRAINING>
+template <typename T, bool TRAINING, int ACT>
 __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const T* __restrict__ x, const T* __restrict__ scale,
                                                             const T* __restrict__ bias, const T* __restrict__ in_mean,
                                                             const T* __restrict__ in_var, const float* __restrict__ partial,
@@ -148,27 +166,36 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(const T* __restrict_
     for_each_piece<T>(g, c, s, [&](int64_t idx, int count) {
         float v[VecOf<T>::n];
         load_piece<T>(x, idx, count, v);
-        for (int j = 0; j < count; ++j) v[j] = (v[j] - mean) * a + b;   // centred first: no cancellation for large means
+        for (int j = 0; j < count; ++j) v[j] = bn_act<ACT>((v[j] - mean) * a + b);   // centred first: no cancellation for large means
         store_piece<T>(y, idx, count, v);
     });
 }
 
-// partial pairs: sum of dy, sum of dy * (x - mean)
-template <typename T>
+// partial pairs: sum of dz, sum of dz * (x - mean), with dz = dy * act'(z) the gradient at the normalised value
+template <typename T, int ACT>
 __global__ __launch_bounds__(kThreads) void bn_bwd_stats_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                                const T* __restrict__ scale, const T* __restrict__ bias,
                                                                 const T* __restrict__ saved_mean,
+                                                                const T* __restrict__ saved_var, float eps,
                                                                 float* __restrict__ partial, BnGeom g) {
     __shared__ float scratch[kThreads / kWave];
     const int c = blockIdx.x, s = blockIdx.y;
     const float mean = to_f32(saved_mean[c]);
+    float a = 0.f, b = 0.f;
+    if constexpr (ACT != DMLHIP_ACT_NONE) {
+        a = to_f32(scale[c]) * (1.0f / sqrtf(to_f32(saved_var[c]) + eps));
+        b = to_f32(bias[c]);
+    }
     float s1 = 0.f, s2 = 0.f;
     for_each_piece<T>(g, c, s, [&](int64_t idx, int count) {
         float v[VecOf<T>::n], d[VecOf<T>::n];
         load_piece<T>(x, idx, count, v);
         load_piece<T>(dy, idx, count, d);
         for (int j = 0; j < count; ++j) {
-            s1 += d[j];
-            s2 += d[j] * (v[j] - mean);
+            const float xc = v[j] - mean;
+            const float dz = d[j] * bn_act_grad<ACT>(xc * a + b);
+            s1 += dz;
+            s2 += dz * xc;
         }
     });
     s1 = block_reduce<OpSum, kThreads / kWave>(s1, scratch);
@@ -179,10 +206,10 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_stats_kernel(const T* __restr
     }
 }
 
-// dx = scale * invstd * (dy - mean(dy) - (x - mean) * invstd^2 * mean(dy * (x - mean)))
-template <typename T>
+// dx = scale * invstd * (dz - mean(dz) - (x - mean) * invstd^2 * mean(dz * (x - mean)))
+template <typename T, int ACT>
 __global__ __launch_bounds__(kThreads) void bn_bwd_apply_kernel(const T* __restrict__ dy, const T* __restrict__ x,
-                                                                const T* __restrict__ scale,
+                                                                const T* __restrict__ scale, const T* __restrict__ bias,
                                                                 const T* __restrict__ saved_mean,
                                                                 const T* __restrict__ saved_var,
                                                                 const float* __restrict__ partial, T* __restrict__ dx,
@@ -203,11 +230,16 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_apply_kernel(const T* __restr
     const float k0 = to_f32(scale[c]) * invstd;
     const float k1 = sum_dy / cnt;
     const float k2 = invstd * invstd * sum_dyxc / cnt;
+    float b = 0.f;
+    if constexpr (ACT != DMLHIP_ACT_NONE) b = to_f32(bias[c]);
     for_each_piece<T>(g, c, s, [&](int64_t idx, int count) {
         float v[VecOf<T>::n], d[VecOf<T>::n];
         load_piece<T>(x, idx, count, v);
         load_piece<T>(dy, idx, count, d);
-        for (int j = 0; j < count; ++j) v[j] = k0 * (d[j] - k1 - (v[j] - mean) * k2);
+        for (int j = 0; j < count; ++j) {
+            const float xc = v[j] - mean;
+            v[j] = k0 * (d[j] * bn_act_grad<ACT>(xc * k0 + b) - k1 - xc * k2);
+        }
         store_piece<T>(dx, idx, count, v);
     });
 }
@@ -238,22 +270,38 @@ size_t bn_workspace(int64_t n, int64_t c, int64_t hw) {
     return c > 0 ? (size_t)c * kMaxSplit * 2 * sizeof(float) : 0;
 }
 
+// runs `body(std::integral_constant<int, ACT>)` for the activation code, or reports an unsupported one
+template <typename F>
+int with_activation(const char* what, int act, F&& body) {
+    switch (act) {
+        case DMLHIP_ACT_NONE: return body(std::integral_constant<int, DMLHIP_ACT_NONE>{});
+        case DMLHIP_ACT_RELU: return body(std::integral_constant<int, DMLHIP_ACT_RELU>{});
+        case DMLHIP_ACT_SWISH: return body(std::integral_constant<int, DMLHIP_ACT_SWISH>{});
+        default:
+            set_error("%s: activation %d is not one of NONE, RELU, SWISH", what, act);
+            return DMLHIP_ERR_ENUM;
+    }
+}
+
 template <typename T>
 int bn_inference(const void* x, const void* scale, const void* bias, const void* mean, const void* var, void* y,
-                 int64_t n, int64_t c, int64_t hw, float eps, void* stream) {
+                 int64_t n, int64_t c, int64_t hw, float eps, int act, void* stream) {
     DML_REQUIRE(x && scale && bias && mean && var && y, DMLHIP_ERR_NULL, "batchnorm_inference: NULL pointer");
     BnGeom g;
     if (int e = make_geom("batchnorm_inference", n, c, hw, {x, y}, &g)) return e;
-    hipLaunchKernelGGL((bn_apply_kernel<T, false>), dim3((unsigned)c, (unsigned)g.split), kThreads, 0, (hipStream_t)stream,
-                       (const T*)x, (const T*)scale, (const T*)bias, (const T*)mean, (const T*)var, (const float*)nullptr,
-                       (T*)y, (T*)nullptr, (T*)nullptr, (T*)nullptr, (T*)nullptr, eps, 0.f, g);
-    return launch_status("batchnorm_inference");
+    return with_activation("batchnorm_inference", act, [&](auto actc) {
+        constexpr int ACT = decltype(actc)::value;
+        hipLaunchKernelGGL((bn_apply_kernel<T, false, ACT>), dim3((unsigned)c, (unsigned)g.split), kThreads, 0,
+                           (hipStream_t)stream, (const T*)x, (const T*)scale, (const T*)bias, (const T*)mean, (const T*)var,
+                           (const float*)nullptr, (T*)y, (T*)nullptr, (T*)nullptr, (T*)nullptr, (T*)nullptr, eps, 0.f, g);
+        return launch_status("batchnorm_inference");
+    });
 }
 
 template <typename T>
 int bn_training(const void* x, const void* scale, const void* bias, const void* in_mean, const void* in_var, void* y,
                 void* out_mean, void* out_var, void* saved_mean, void* saved_var, int64_t n, int64_t c, int64_t hw,
-                float eps, float momentum, void* workspace, size_t workspace_bytes, void* stream) {
+                float eps, float momentum, int act, void* workspace, size_t workspace_bytes, void* stream) {
     DML_REQUIRE(x && scale && bias && in_mean && in_var && y && out_mean && out_var && saved_mean && saved_var,
                 DMLHIP_ERR_NULL, "batchnorm_training: NULL pointer");
     BnGeom g;
@@ -263,30 +311,39 @@ int bn_training(const void* x, const void* scale, const void* bias, const void* 
     const dim3 grid((unsigned)c, (unsigned)g.split);
     hipLaunchKernelGGL((bn_stats_kernel<T>), grid, kThreads, 0, (hipStream_t)stream, (const T*)x, (float*)workspace, g);
     if (int e = launch_status("batchnorm_training(statistics)")) return e;
-    hipLaunchKernelGGL((bn_apply_kernel<T, true>), grid, kThreads, 0, (hipStream_t)stream, (const T*)x, (const T*)scale,
-                       (const T*)bias, (const T*)in_mean, (const T*)in_var, (const float*)workspace, (T*)y, (T*)out_mean,
-                       (T*)out_var, (T*)saved_mean, (T*)saved_var, eps, momentum, g);
-    return launch_status("batchnorm_training");
+    return with_activation("batchnorm_training", act, [&](auto actc) {
+        constexpr int ACT = decltype(actc)::value;
+        hipLaunchKernelGGL((bn_apply_kernel<T, true, ACT>), grid, kThreads, 0, (hipStream_t)stream, (const T*)x,
+                           (const T*)scale, (const T*)bias, (const T*)in_mean, (const T*)in_var, (const float*)workspace,
+                           (T*)y, (T*)out_mean, (T*)out_var, (T*)saved_mean, (T*)saved_var, eps, momentum, g);
+        return launch_status("batchnorm_training");
+    });
 }
 
 template <typename T>
-int bn_backward(const void* dy, const void* x, const void* scale, const void* saved_mean, const void* saved_var,
-                void* dx, float* dscale, float* dbias, int64_t n, int64_t c, int64_t hw, float eps, void* workspace,
-                size_t workspace_bytes, void* stream) {
+int bn_backward(const void* dy, const void* x, const void* scale, const void* bias, const void* saved_mean,
+                const void* saved_var, void* dx, float* dscale, float* dbias, int64_t n, int64_t c, int64_t hw, float eps,
+                int act, void* workspace, size_t workspace_bytes, void* stream) {
     DML_REQUIRE(dy && x && scale && saved_mean && saved_var, DMLHIP_ERR_NULL, "batchnorm_backward: NULL pointer");
+    DML_REQUIRE(bias || act == DMLHIP_ACT_NONE, DMLHIP_ERR_NULL,
+                "batchnorm_backward: the bias is needed to recompute the activation's input");
     DML_REQUIRE(dx || dscale || dbias, DMLHIP_ERR_NULL, "batchnorm_backward: no gradient requested");
     BnGeom g;
     if (int e = make_geom("batchnorm_backward", n, c, hw, {dy, x, dx}, &g)) return e;
     DML_REQUIRE(workspace && workspace_bytes >= bn_workspace(n, c, hw), DMLHIP_ERR_WORKSPACE,
                 "batchnorm_backward: workspace of %zu bytes needed, got %zu", bn_workspace(n, c, hw), workspace_bytes);
     const dim3 grid((unsigned)c, (unsigned)g.split);
-    hipLaunchKernelGGL((bn_bwd_stats_kernel<T>), grid, kThreads, 0, (hipStream_t)stream, (const T*)dy, (const T*)x,
-                       (const T*)saved_mean, (float*)workspace, g);
-    if (int e = launch_status("batchnorm_backward(sums)")) return e;
-    hipLaunchKernelGGL((bn_bwd_apply_kernel<T>), grid, kThreads, 0, (hipStream_t)stream, (const T*)dy, (const T*)x,
-                       (const T*)scale, (const T*)saved_mean, (const T*)saved_var, (const float*)workspace, (T*)dx, dscale,
-                       dbias, eps, g);
-    return launch_status("batchnorm_backward");
+    return with_activation("batchnorm_backward", act, [&](auto actc) {
+        constexpr int ACT = decltype(actc)::value;
+        hipLaunchKernelGGL((bn_bwd_stats_kernel<T, ACT>), grid, kThreads, 0, (hipStream_t)stream, (const T*)dy, (const T*)x,
+                           (const T*)scale, (const T*)bias, (const T*)saved_mean, (const T*)saved_var, eps,
+                           (float*)workspace, g);
+        if (int e = launch_status("batchnorm_backward(sums)")) return e;
+        hipLaunchKernelGGL((bn_bwd_apply_kernel<T, ACT>), grid, kThreads, 0, (hipStream_t)stream, (const T*)dy, (const T*)x,
+                           (const T*)scale, (const T*)bias, (const T*)saved_mean, (const T*)saved_var,
+                           (const float*)workspace, (T*)dx, dscale, dbias, eps, g);
+        return launch_status("batchnorm_backward");
+    });
 }
 
 }  // namespace
@@ -298,41 +355,49 @@ extern "C" {
 
 size_t dmlhip_batchnorm_workspace_bytes(int64_t n, int64_t c, int64_t hw) { return bn_workspace(n, c, hw); }
 
-int dmlhip_batchnorm_inference_f16(const void* x, const void* scale, const void* bias, const void* mean, const void* var,
-                                   void* y, int64_t n, int64_t c, int64_t hw, float eps, void* stream) {
-    return bn_inference<_Float16>(x, scale, bias, mean, var, y, n, c, hw, eps, stream);
-}
-int dmlhip_batchnorm_inference_f32(const void* x, const void* scale, const void* bias, const void* mean, const void* var,
-                                   void* y, int64_t n, int64_t c, int64_t hw, float eps, void* stream) {
-    return bn_inference<float>(x, scale, bias, mean, var, y, n, c, hw, eps, stream);
-}
+#define DML_BN_ENTRIES(SFX, T)                                                                                         \
+    int dmlhip_batchnorm_inference_##SFX(const void* x, const void* scale, const void* bias, const void* mean,         \
+                                         const void* var, void* y, int64_t n, int64_t c, int64_t hw, float eps,        \
+                                         void* stream) {                                                               \
+        return bn_inference<T>(x, scale, bias, mean, var, y, n, c, hw, eps, DMLHIP_ACT_NONE, stream);                  \
+    }                                                                                                                  \
+    int dmlhip_batchnorm_inference_act_##SFX(const void* x, const void* scale, const void* bias, const void* mean,     \
+                                             const void* var, void* y, int64_t n, int64_t c, int64_t hw, float eps,    \
+                                             int act, void* stream) {                                                  \
+        return bn_inference<T>(x, scale, bias, mean, var, y, n, c, hw, eps, act, stream);                              \
+    }                                                                                                                  \
+    int dmlhip_batchnorm_training_##SFX(const void* x, const void* scale, const void* bias, const void* in_mean,       \
+                                        const void* in_var, void* y, void* out_mean, void* out_var, void* saved_mean,  \
+                                        void* saved_var, int64_t n, int64_t c, int64_t hw, float eps, float momentum,  \
+                                        void* workspace, size_t workspace_bytes, void* stream) {                       \
+        return bn_training<T>(x, scale, bias, in_mean, in_var, y, out_mean, out_var, saved_mean, saved_var, n, c, hw,  \
+                              eps, momentum, DMLHIP_ACT_NONE, workspace, workspace_bytes, stream);                     \
+    }                                                                                                                  \
+    int dmlhip_batchnorm_training_act_##SFX(const void* x, const void* scale, const void* bias, const void* in_mean,   \
+                                            const void* in_var, void* y, void* out_mean, void* out_var,                \
+                                            void* saved_mean, void* saved_var, int64_t n, int64_t c, int64_t hw,       \
+                                            float eps, float momentum, int act, void* workspace,                       \
+                                            size_t workspace_bytes, void* stream) {                                    \
+        return bn_training<T>(x, scale, bias, in_mean, in_var, y, out_mean, out_var, saved_mean, saved_var, n, c, hw,  \
+                              eps, momentum, act, workspace, workspace_bytes, stream);                                 \
+    }                                                                                                                  \
+    int dmlhip_batchnorm_backward_##SFX(const void* dy, const void* x, const void* scale, const void* saved_mean,      \
+                                        const void* saved_var, void* dx, float* dscale, float* dbias, int64_t n,       \
+                                        int64_t c, int64_t hw, float eps, void* workspace, size_t workspace_bytes,     \
+                                        void* stream) {                                                                \
+        return bn_backward<T>(dy, x, scale, nullptr, saved_mean, saved_var, dx, dscale, dbias, n, c, hw, eps,          \
+                              DMLHIP_ACT_NONE, workspace, workspace_bytes, stream);                                    \
+    }                                                                                                                  \
+    int dmlhip_batchnorm_backward_act_##SFX(const void* dy, const void* x, const void* scale, const void* bias,        \
+                                            const void* saved_mean, const void* saved_var, void* dx, float* dscale,    \
+                                            float* dbias, int64_t n, int64_t c, int64_t hw, float eps, int act,        \
+                                            void* workspace, size_t workspace_bytes, void* stream) {                   \
+        return bn_backward<T>(dy, x, scale, bias, saved_mean, saved_var, dx, dscale, dbias, n, c, hw, eps, act,        \
+                              workspace, workspace_bytes, stream);                                                     \
+    }
 
-int dmlhip_batchnorm_training_f16(const void* x, const void* scale, const void* bias, const void* in_mean,
-                                  const void* in_var, void* y, void* out_mean, void* out_var, void* saved_mean,
-                                  void* saved_var, int64_t n, int64_t c, int64_t hw, float eps, float momentum,
-                                  void* workspace, size_t workspace_bytes, void* stream) {
-    return bn_training<_Float16>(x, scale, bias, in_mean, in_var, y, out_mean, out_var, saved_mean, saved_var, n, c, hw,
-                                 eps, momentum, workspace, workspace_bytes, stream);
-}
-int dmlhip_batchnorm_training_f32(const void* x, const void* scale, const void* bias, const void* in_mean,
-                                  const void* in_var, void* y, void* out_mean, void* out_var, void* saved_mean,
-                                  void* saved_var, int64_t n, int64_t c, int64_t hw, float eps, float momentum,
-                                  void* workspace, size_t workspace_bytes, void* stream) {
-    return bn_training<float>(x, scale, bias, in_mean, in_var, y, out_mean, out_var, saved_mean, saved_var, n, c, hw, eps,
-                              momentum, workspace, workspace_bytes, stream);
-}
-
-int dmlhip_batchnorm_backward_f16(const void* dy, const void* x, const void* scale, const void* saved_mean,
-                                  const void* saved_var, void* dx, float* dscale, float* dbias, int64_t n, int64_t c,
-                                  int64_t hw, float eps, void* workspace, size_t workspace_bytes, void* stream) {
-    return bn_backward<_Float16>(dy, x, scale, saved_mean, saved_var, dx, dscale, dbias, n, c, hw, eps, workspace,
-                                 workspace_bytes, stream);
-}
-int dmlhip_batchnorm_backward_f32(const void* dy, const void* x, const void* scale, const void* saved_mean,
-                                  const void* saved_var, void* dx, float* dscale, float* dbias, int64_t n, int64_t c,
-                                  int64_t hw, float eps, void* workspace, size_t workspace_bytes, void* stream) {
-    return bn_backward<float>(dy, x, scale, saved_mean, saved_var, dx, dscale, dbias, n, c, hw, eps, workspace,
-                              workspace_bytes, stream);
-}
+DML_BN_ENTRIES(f16, _Float16)
+DML_BN_ENTRIES(f32, float)
+#undef DML_BN_ENTRIES
 
 }  // extern "C"

@@ -139,43 +139,49 @@ def _bn_geometry(x):
     return n, c, hw
 
 
-def batchnorm_inference(x, scale, bias, mean, var, eps=1e-5):
-    """y = (x - mean) / sqrt(var + eps) * scale + bias over [N, C, ...] with given per-channel statistics."""
+def batchnorm_inference(x, scale, bias, mean, var, eps=1e-5, act: int = L.ACT_NONE):
+    """y = act((x - mean) / sqrt(var + eps) * scale + bias) over [N, C, ...] with given per-channel statistics."""
     _check(x, scale, bias, mean, var, dtype=x.dtype)
     x = _dense(x)
     n, c, hw = _bn_geometry(x)
     y = torch.empty_like(x)
-    L.check(_fn("batchnorm_inference", x.dtype)(_ptr(x), _ptr(_dense(scale)), _ptr(_dense(bias)), _ptr(_dense(mean)),
-                                                _ptr(_dense(var)), _ptr(y), n, c, hw, float(eps), _stream()))
+    L.check(_fn("batchnorm_inference_act", x.dtype)(_ptr(x), _ptr(_dense(scale)), _ptr(_dense(bias)), _ptr(_dense(mean)),
+                                                    _ptr(_dense(var)), _ptr(y), n, c, hw, float(eps), int(act), _stream()))
     return y
 
 
-def batchnorm_training(x, scale, bias, in_mean, in_var, eps=1e-5, momentum=0.9):
-    """Returns (y, out_mean, out_var, saved_mean, saved_var); ``momentum`` weighs the running value (ONNX)."""
+def batchnorm_training(x, scale, bias, in_mean, in_var, eps=1e-5, momentum=0.9, act: int = L.ACT_NONE):
+    """Returns (y, out_mean, out_var, saved_mean, saved_var); ``momentum`` weighs the running value (ONNX); ``act`` is
+    applied to the normalised value in the same kernel."""
     _check(x, scale, bias, in_mean, in_var, dtype=x.dtype)
     x = _dense(x)
     n, c, hw = _bn_geometry(x)
     y = torch.empty_like(x)
     stats = [torch.empty(c, dtype=x.dtype, device=x.device) for _ in range(4)]
     ws = workspace(L.load().dmlhip_batchnorm_workspace_bytes(n, c, hw), x.device)
-    L.check(_fn("batchnorm_training", x.dtype)(_ptr(x), _ptr(_dense(scale)), _ptr(_dense(bias)), _ptr(_dense(in_mean)),
-                                               _ptr(_dense(in_var)), _ptr(y), *[_ptr(t) for t in stats], n, c, hw,
-                                               float(eps), float(momentum), _ptr(ws), ws.numel(), _stream()))
+    L.check(_fn("batchnorm_training_act", x.dtype)(_ptr(x), _ptr(_dense(scale)), _ptr(_dense(bias)),
+                                                   _ptr(_dense(in_mean)), _ptr(_dense(in_var)), _ptr(y),
+                                                   *[_ptr(t) for t in stats], n, c, hw, float(eps), float(momentum),
+                                                   int(act), _ptr(ws), ws.numel(), _stream()))
     return (y, *stats)
 
 
-def batchnorm_backward(dy, x, scale, saved_mean, saved_var, eps=1e-5):
-    """Returns (dx, dscale_fp32, dbias_fp32)."""
+def batchnorm_backward(dy, x, scale, saved_mean, saved_var, eps=1e-5, act: int = L.ACT_NONE, bias=None):
+    """Returns (dx, dscale_fp32, dbias_fp32). With ``act`` the given gradient is the one of the activated output and
+    ``bias`` is needed (the normalised value is recomputed)."""
     _check(dy, x, scale, saved_mean, saved_var, dtype=x.dtype)
+    if act != L.ACT_NONE and bias is None:
+        raise ValueError("batchnorm_backward with an activation needs the bias")
     dy, x = _dense(dy), _dense(x)
     n, c, hw = _bn_geometry(x)
     dx = torch.empty_like(x)
     dscale = torch.empty(c, dtype=torch.float32, device=x.device)
     dbias = torch.empty(c, dtype=torch.float32, device=x.device)
     ws = workspace(L.load().dmlhip_batchnorm_workspace_bytes(n, c, hw), x.device)
-    L.check(_fn("batchnorm_backward", x.dtype)(_ptr(dy), _ptr(x), _ptr(_dense(scale)), _ptr(_dense(saved_mean)),
-                                               _ptr(_dense(saved_var)), _ptr(dx), _ptr(dscale), _ptr(dbias), n, c, hw,
-                                               float(eps), _ptr(ws), ws.numel(), _stream()))
+    L.check(_fn("batchnorm_backward_act", x.dtype)(_ptr(dy), _ptr(x), _ptr(_dense(scale)),
+                                                   _ptr(None if bias is None else _dense(bias)), _ptr(_dense(saved_mean)),
+                                                   _ptr(_dense(saved_var)), _ptr(dx), _ptr(dscale), _ptr(dbias), n, c, hw,
+                                                   float(eps), int(act), _ptr(ws), ws.numel(), _stream()))
     return dx, dscale, dbias
 
 

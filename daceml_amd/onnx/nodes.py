@@ -157,7 +157,9 @@ SCHEMAS = [
     # element): the reverse of a mean / sum reduction (ReverseReduce, daceml/autodiff/implementations/dace_nodes.py:13-105)
     # x_shape: the shape X is read with when its descriptor has the size-1 dims squeezed out (keepdims = 0)
     _schema("ScaledExpand", "X Scale", "Y", since=1, x_shape=None),
-    _schema("BatchNormalizationGrad", "dY X scale saved_mean saved_var", "dX? dscale? dB?", since=1, epsilon=1e-5),
+    # `activation` other than "none": dY is the gradient of activation(BatchNormalization(X)) and B is needed
+    _schema("BatchNormalizationGrad", "dY X scale saved_mean saved_var B?", "dX? dscale? dB?", since=1, epsilon=1e-5,
+            activation="none"),
     _schema("LayerNormalizationGrad", "Y_grad X scale mean inv_std_var", "X_grad scale_grad bias_grad", since=1,
             axis=-1),
     _schema("GeluGrad", "dY X", "dX", since=1),

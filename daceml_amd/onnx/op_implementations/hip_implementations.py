@@ -827,12 +827,15 @@ class HipBatchNormalization(ONNXForward):
     (img_op_implementations.py:333-412; cuDNN variant cudnn_implementations.py:444-649): biased batch variance,
     running statistics updated as ``in * momentum + saved * (1 - momentum)``. As in the reference (:392-410) the
     updated running statistics are also written back to the arrays they came from, when those are caller-owned
-    buffers."""
+    buffers. A private ``_activation`` attribute ("relu" / "swish") set by the fusion pass applies a following
+    activation in the same kernel."""
     @staticmethod
     def forward_can_be_applied(node, state, sdfg) -> bool:
         try:
             ins, outs = _descs(node, state, sdfg)
             x, y = ins["X"], outs["Y"]
+            if getattr(node, "_activation", "none") not in ("none", "relu", "swish"):
+                return False
             stats = [outs.get(k) for k in ("out_mean", "out_var", "saved_mean", "saved_var")]
             if any(s is None for s in stats) and any(s is not None for s in stats):
                 return False
@@ -847,16 +850,19 @@ class HipBatchNormalization(ONNXForward):
         n, c, hw = _bn_dims(x)
         sfx = _SFX[x.dtype]
         training = "saved_mean" in {e.src_conn for e in state.out_edges(node)}
+        act = getattr(node, "_activation", "none")
+        fused = [] if act == "none" else [I32(_ACT[act])]
+        variant = "" if act == "none" else "act_"
         if not training:
-            call = HipCall("dmlhip_batchnorm_inference_" + sfx,
+            call = HipCall("dmlhip_batchnorm_inference_" + variant + sfx,
                            [Ptr("X"), Ptr("scale"), Ptr("B"), Ptr("in_mean"), Ptr("in_var"), Ptr("Y"), I64(n), I64(c),
-                            I64(hw), F32(node.epsilon), Stream()])
+                            I64(hw), F32(node.epsilon)] + fused + [Stream()])
             return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="batchnorm")
         ws = L.load().dmlhip_batchnorm_workspace_bytes(n, c, hw)
-        calls = [HipCall("dmlhip_batchnorm_training_" + sfx,
+        calls = [HipCall("dmlhip_batchnorm_training_" + variant + sfx,
                          [Ptr("X"), Ptr("scale"), Ptr("B"), Ptr("in_mean"), Ptr("in_var"), Ptr("Y"), Ptr("out_mean"),
                           Ptr("out_var"), Ptr("saved_mean"), Ptr("saved_var"), I64(n), I64(c), I64(hw),
-                          F32(node.epsilon), F32(node.momentum), Workspace(), WorkspaceBytes(), Stream()])]
+                          F32(node.epsilon), F32(node.momentum)] + fused + [Workspace(), WorkspaceBytes(), Stream()])]
         for src, dst in (("out_mean", "in_mean"), ("out_var", "in_var")):
             arr = next(iter(state.in_edges_by_connector(node, dst))).data.data
             if not sdfg.arrays[arr].transient and arr not in sdfg.constants:
@@ -877,6 +883,10 @@ class HipBatchNormalizationGrad(ONNXForward):
             if not (_bn_ok(x, ins["scale"], ins["saved_mean"], ins["saved_var"]) and _dense(dy)
                     and dy.shape == x.shape and dy.dtype == x.dtype and outs):
                 return False
+            if node.activation not in ("none", "relu", "swish"):
+                return False
+            if node.activation != "none" and not ("B" in ins and _bn_ok(x, ins["B"])):
+                return False
             dx = outs.get("dX")
             if dx is not None and not (_dense(dx) and dx.shape == x.shape and dx.dtype == x.dtype):
                 return False
@@ -890,11 +900,13 @@ class HipBatchNormalizationGrad(ONNXForward):
         x = in_desc_with_name(node, state, sdfg, "X")
         n, c, hw = _bn_dims(x)
         ws = L.load().dmlhip_batchnorm_workspace_bytes(n, c, hw)
-        call = HipCall("dmlhip_batchnorm_backward_" + _SFX[x.dtype],
-                       [Ptr("dY"), Ptr("X"), Ptr("scale"), Ptr("saved_mean"), Ptr("saved_var"),
-                        _opt(node, state, "dX", False), _opt(node, state, "dscale", False),
-                        _opt(node, state, "dB", False), I64(n), I64(c), I64(hw), F32(node.epsilon), Workspace(),
-                        WorkspaceBytes(), Stream()])
+        fused = node.activation != "none"
+        call = HipCall("dmlhip_batchnorm_backward_" + ("act_" if fused else "") + _SFX[x.dtype],
+                       [Ptr("dY"), Ptr("X"), Ptr("scale")] + ([Ptr("B")] if fused else []) +
+                       [Ptr("saved_mean"), Ptr("saved_var"), _opt(node, state, "dX", False),
+                        _opt(node, state, "dscale", False), _opt(node, state, "dB", False), I64(n), I64(c), I64(hw),
+                        F32(node.epsilon)] + ([I32(_ACT[node.activation])] if fused else []) +
+                       [Workspace(), WorkspaceBytes(), Stream()])
         return _tasklet(node, state, [call], workspace_bytes=ws, bytes_moved=5 * _nbytes(x), kind="batchnorm_backward")
 
 

@@ -325,6 +325,40 @@ def fuse_conv_activation(sdfg: SDFG) -> int:
     return count
 
 
+def fuse_batchnorm_activation(sdfg: SDFG) -> int:
+    """BatchNormalization followed only by Swish / Relu: the activation moves into the normalisation kernels (forward
+    and, through BatchNormalizationGrad's ``activation``, backward), which saves a pass over the tensor each way. Works
+    for the inference and the training form; runs after fuse_swish."""
+    names = {"Swish": "swish", "Relu": "relu"}
+    count = 0
+    for state in sdfg.states():
+        for bn in [n for n in state.nodes() if _is_op(n, "BatchNormalization")]:
+            if getattr(bn, "_activation", "none") != "none":
+                continue
+            y = _out_array(state, bn, "Y")
+            cons = _consumers(state, y)
+            if len(cons) != 1 or not isinstance(cons[0][0], ONNXOp) or cons[0][0].schema.name not in names:
+                continue
+            if not _internal(sdfg, state, y):
+                continue
+            act = cons[0][0]
+            out = _out_array(state, act, "Y")
+            if tuple(sdfg.arrays[out].shape) != tuple(sdfg.arrays[y].shape) or sdfg.arrays[out].dtype != sdfg.arrays[y].dtype:
+                continue
+            for e in [e for e in state.out_edges(bn) if e.src_conn == "Y"]:
+                state.remove_edge(e)
+            _remove_node(state, act)
+            for n in [n for n in state.nodes() if isinstance(n, AccessNode) and n.data == y]:
+                if not state.in_edges(n) and not state.out_edges(n):
+                    state.remove_node(n)
+            state.add_edge(bn, "Y", state.add_write(out), None, sdfg.make_array_memlet(out))
+            bn._activation = names[act.schema.name]
+            count += 1
+    if count:
+        _drop_unused_arrays(sdfg)
+    return count
+
+
 def fuse_gate_into_conv(sdfg: SDFG) -> int:
     """Squeeze-excite: Mul(X[n,c,h,w], gate[n,c,1,1]) read only by a pointwise Conv becomes one GatedConv, which
     saves a full read and write of X. Forward graphs only (GatedConv has no backward implementation)."""
@@ -1081,6 +1115,7 @@ def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True,
     # a Conv with a folded activation, GatedConv and SkipLayerNormalization have no backward implementation: graphs that
     # will be differentiated keep those nodes apart
     stats["conv_activation"] = 0 if training else fuse_conv_activation(sdfg)
+    stats["batchnorm_activation"] = fuse_batchnorm_activation(sdfg)
     stats["gated_conv"] = 0 if training else fuse_gate_into_conv(sdfg)
     stats["expand_depthwise"] = 0 if training else fuse_expand_depthwise(sdfg)
     stats["matmul_to_einsum"] = lower_matmul(sdfg)

@@ -355,6 +355,33 @@ int dmlhip_batchnorm_backward_f32(const void* dy, const void* x, const void* sca
                                   const void* saved_var, void* dx, float* dscale, float* dbias, int64_t n,
                                   int64_t c, int64_t hw, float eps, void* workspace, size_t workspace_bytes,
                                   void* stream);
+/* The same three with an activation (DMLHIP_ACT_NONE, _RELU or _SWISH; anything else: DMLHIP_ERR_ENUM) applied to the
+ * normalised value inside the kernel: the exported chains BatchNormalization -> Relu and BatchNormalization -> Sigmoid,
+ * Mul (pure_implementations.py:556-560, 741-743, 86-88) without a second pass over the tensor. backward_act takes
+ * the gradient with respect to the activated output, recomputes the normalised value from x, scale, bias and the
+ * saved statistics (hence the bias argument) and returns the gradients of the fused pair. */
+int dmlhip_batchnorm_inference_act_f16(const void* x, const void* scale, const void* bias, const void* mean,
+                                       const void* var, void* y, int64_t n, int64_t c, int64_t hw, float eps, int act,
+                                       void* stream);
+int dmlhip_batchnorm_inference_act_f32(const void* x, const void* scale, const void* bias, const void* mean,
+                                       const void* var, void* y, int64_t n, int64_t c, int64_t hw, float eps, int act,
+                                       void* stream);
+int dmlhip_batchnorm_training_act_f16(const void* x, const void* scale, const void* bias, const void* in_mean,
+                                      const void* in_var, void* y, void* out_mean, void* out_var, void* saved_mean,
+                                      void* saved_var, int64_t n, int64_t c, int64_t hw, float eps, float momentum,
+                                      int act, void* workspace, size_t workspace_bytes, void* stream);
+int dmlhip_batchnorm_training_act_f32(const void* x, const void* scale, const void* bias, const void* in_mean,
+                                      const void* in_var, void* y, void* out_mean, void* out_var, void* saved_mean,
+                                      void* saved_var, int64_t n, int64_t c, int64_t hw, float eps, float momentum,
+                                      int act, void* workspace, size_t workspace_bytes, void* stream);
+int dmlhip_batchnorm_backward_act_f16(const void* dy, const void* x, const void* scale, const void* bias,
+                                      const void* saved_mean, const void* saved_var, void* dx, float* dscale,
+                                      float* dbias, int64_t n, int64_t c, int64_t hw, float eps, int act,
+                                      void* workspace, size_t workspace_bytes, void* stream);
+int dmlhip_batchnorm_backward_act_f32(const void* dy, const void* x, const void* scale, const void* bias,
+                                      const void* saved_mean, const void* saved_var, void* dx, float* dscale,
+                                      float* dbias, int64_t n, int64_t c, int64_t hw, float eps, int act,
+                                      void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -664,6 +664,44 @@ def test_einsum_grouped(eq, sa, sb, with_bias, out_dtype):
     _einsum_grouped_case(eq, sa, sb, with_bias, out_dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("act", ["swish", "relu"])
+def test_batchnorm_with_activation(dtype, act):
+    """BatchNormalization with the activation inside the kernels against the composition of the oracle's functions:
+    forward (training and inference forms) and the backward that recomputes the normalised value."""
+    from daceml_amd import _lib as L, kernels as K
+    code = {"swish": L.ACT_SWISH, "relu": L.ACT_RELU}[act]
+    fwd = {"swish": O.swish, "relu": O.relu}[act]
+    npdt = _np(dtype)
+    r = rng(150)
+    x = (r.standard_normal((5, 7, 6, 9)) * 1.5 + 0.5).astype(npdt)
+    scale, bias = r.uniform(0.5, 1.5, 7).astype(npdt), (r.standard_normal(7) * 0.3).astype(npdt)
+    mean, var = (r.standard_normal(7) * 0.2).astype(npdt), r.uniform(0.5, 1.5, 7).astype(npdt)
+    dy = r.standard_normal(x.shape).astype(npdt)
+    f64 = lambda t: t.astype(np.float64)
+    z, om, ov, sm, sv = O.batchnorm_training(f64(x), f64(scale), f64(bias), f64(mean), f64(var), 1e-5, 0.9)
+    got = K.batchnorm_training(dev(x), dev(scale), dev(bias), dev(mean), dev(var), 1e-5, 0.9, act=code)
+    for g_, w_, what in zip(got, (fwd(z), om, ov, sm, sv), ("y", "running mean", "running variance", "mean", "variance")):
+        assert_close(host(g_), w_, dtype, "batchnorm+%s %s" % (act, what))
+    assert_close(host(K.batchnorm_inference(dev(x), dev(scale), dev(bias), dev(mean), dev(var), 1e-5, act=code)),
+                 fwd(O.batchnorm_inference(f64(x), f64(scale), f64(bias), f64(mean), f64(var), 1e-5)), dtype,
+                 "batchnorm+%s inference" % act)
+    # backward: the kernels see the statistics rounded to the tensor type, as the forward kernel stored them
+    smr, svr = host(got[3]).astype(np.float64), host(got[4]).astype(np.float64)
+    zr = (f64(x) - smr.reshape(1, -1, 1, 1)) / np.sqrt(svr.reshape(1, -1, 1, 1) + 1e-5) * f64(scale).reshape(1, -1, 1, 1) \
+        + f64(bias).reshape(1, -1, 1, 1)
+    dz = O.swish_backward(f64(dy), zr) if act == "swish" else f64(dy) * (zr > 0)
+    wdx, wds, wdb = O.batchnorm_backward(dz, f64(x), f64(scale), smr, svr, 1e-5)
+    dx, ds, db = K.batchnorm_backward(dev(dy), dev(x), dev(scale), got[3], got[4], 1e-5, act=code, bias=dev(bias))
+    kw = dict(rtol=1e-4, atol=2e-5) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+    assert_close(host(dx), wdx, dtype, "batchnorm+%s dx" % act, **kw)
+    kw = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=3e-2, atol=0.3)
+    assert_close(host(ds), wds, torch.float32, "batchnorm+%s dscale" % act, **kw)
+    assert_close(host(db), wdb, torch.float32, "batchnorm+%s dbias" % act, **kw)
+    with pytest.raises(ValueError):
+        K.batchnorm_backward(dev(dy), dev(x), dev(scale), got[3], got[4], 1e-5, act=code)
+
+
 @pytest.mark.parametrize("eq,sa,sb,n,with_res,out_dtype,single", [
     ("aij,jk->aik", (2, 256, 128), (128, 192), 3, True, torch.float16, True),    # q/k/v input gradients + residual path
     ("aij,jk->aik", (2, 256, 128), (128, 192), 2, False, torch.float16, True),
