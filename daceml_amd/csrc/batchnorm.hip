@@ -1,5 +1,8 @@
 // BatchNormalization over NCHW tensors: inference, training forward (batch statistics + running-statistics update)
 // and backward. HBM-bound: training reads X twice and writes Y once, backward reads dY and X twice and writes dX.
+// A Relu or Swish that follows the normalisation can run inside the same kernels (template parameter ACT): the
+// forward applies it before the store, the backward recomputes the normalised value from X and multiplies the incoming
+// gradient by the activation's derivative, so neither pass touches the tensor more often than without it.
 //
 // A channel's data are N segments of HW contiguous elements. Segments are cut into chunks of at most kChunk
 // elements; workgroup (c, s) of a grid C x S walks the chunks s, s+S, ... of channel c, so the launch fills the
