@@ -473,6 +473,10 @@ CONV_CASES = [
     ((5, 12, 20, 24), (70, 12, 3, 3), (1, 1), (2, 2), (2, 2), 1, False),    # dilated, ragged output channels
     ((4, 20, 30, 31), (33, 20, 3, 5), (2, 1), (1, 2), (1, 1), 1, True),     # 3x5 taps, strides 2x1, pads 1x2
     ((16, 8, 112, 112), (16, 8, 3, 3), (1, 1), (1, 1), (1, 1), 1, False),   # many pixels: 256-pixel workgroups
+    # one image: the weight-gradient kernels have a single partial result and write dW directly
+    ((1, 32, 16, 16), (24, 32, 1, 1), (1, 1), (0, 0), (1, 1), 1, True),     # pointwise
+    ((1, 64, 16, 16), (128, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1, False),   # dense
+    ((1, 6, 20, 20), (6, 1, 3, 3), (1, 1), (1, 1), (1, 1), 6, True),        # depthwise
     ((2, 8, 9, 9), (4, 4, 3, 3), (1, 1), (1, 1), (1, 1), 2, True),          # grouped
     ((1, 2, 12, 12), (3, 2, 3, 3), (1, 1), (2, 2), (2, 2), 1, False),       # dilated
     ((2, 4, 8, 8), (6, 4, 1, 1), (2, 2), (0, 0), (1, 1), 1, True),          # 1x1 strided -> direct
