@@ -152,26 +152,34 @@ __global__ __launch_bounds__(kFusedThreads) void expand_depthwise_kernel(const f
         __syncthreads();
     }
 
-    // ---- phase 2: depthwise 3x3 stencil, one wavefront per (channel, output row), lanes along the output columns
-    const int pairs = kCB * a.toh;
-    for (int pr = wave; pr < pairs; pr += kWaves) {
-        const int c = pr % kCB, orow = pr / kCB;
+    // ---- phase 2: depthwise 3x3 stencil, lanes along the output columns; a wavefront takes a channel and two output
+    // rows of the strip at a time, so that two independent chains of LDS reads and activations are in flight
+    const int row_pairs = (a.toh + 1) / 2;
+    for (int pr = wave; pr < kCB * row_pairs; pr += kWaves) {
+        const int c = pr % kCB, orow = (pr / kCB) * 2;
         const int oy = oy0 + orow;
         if (oy >= a.oh) continue;
+        const bool two = orow + 1 < a.toh && oy + 1 < a.oh;
         float wv[10];
 #pragma unroll
         for (int i = 0; i < 10; ++i) wv[i] = WD[c * 10 + i];
         const float* e0 = E + (c * a.ih + orow * a.stride) * a.wp;
+        const float* e1 = e0 + (two ? a.stride * a.wp : 0);
         float* yrow = y + (((size_t)n * a.cmid + c0 + c) * a.oh + oy) * a.ow;
         for (int oc = lane; oc < a.ow; oc += 64) {
-            float s = wv[9];
+            float s0 = wv[9], s1 = wv[9];
 #pragma unroll
             for (int ky = 0; ky < 3; ++ky) {
-                const float* er = e0 + ky * a.wp + oc * a.stride;
+                const float* r0 = e0 + ky * a.wp + oc * a.stride;
+                const float* r1 = e1 + ky * a.wp + oc * a.stride;
 #pragma unroll
-                for (int kx = 0; kx < 3; ++kx) s += wv[ky * 3 + kx] * er[kx];
+                for (int kx = 0; kx < 3; ++kx) {
+                    s0 += wv[ky * 3 + kx] * r0[kx];
+                    s1 += wv[ky * 3 + kx] * r1[kx];
+                }
             }
-            yrow[oc] = act_f<ACT2>(s);
+            yrow[oc] = act_f<ACT2>(s0);
+            if (two) yrow[a.ow + oc] = act_f<ACT2>(s1);
         }
     }
 }
