@@ -247,13 +247,6 @@ struct DenseGradArgs {
     int a_groups, b_tiles;   // workgroups = a_groups * b_tiles * (image groups * pixel ranges); the first two vary fastest
 };
 
-__device__ __forceinline__ int small_div(int a, int b, float inv_b) {   // a / b for 0 <= a < 2^22
-    int q = (int)((float)a * inv_b);
-    const int r = a - q * b;
-    q += (r >= b) - (r < 0);
-    return q;
-}
-
 template <int TA>
 __global__ __launch_bounds__(256, 2) void dense_bwd_weight_kernel(const DenseGradArgs g) {
     extern __shared__ __attribute__((aligned(16))) float dg_lds[];
@@ -275,8 +268,8 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_weight_kernel(const DenseGra
 #pragma unroll
     for (int e = 0; e < RB; ++e) {
         const int j = b0 + wave + 4 * e;
-        const int ch = small_div(min(j, jn - 1), kk, inv_kk), tap = min(j, jn - 1) - ch * kk;
-        const int hy = small_div(tap, g.kw, inv_kw), hx = tap - hy * g.kw;
+        const int ch = fast_div(min(j, jn - 1), kk, inv_kk), tap = min(j, jn - 1) - ch * kk;
+        const int hy = fast_div(tap, g.kw, inv_kw), hx = tap - hy * g.kw;
         coff[e] = j < jn ? ch * in_plane : -1;
         tshift[e] = ((hy * g.dh) << 16) | (hx * g.dw);
     }
@@ -300,7 +293,7 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_weight_kernel(const DenseGra
             pa[e] = dyn[(size_t)(ok ? row : 0) * ohw];
             pa[e] = ok ? pa[e] : 0.f;
         }
-        const int oy = small_div(pc, g.ow, inv_ow), ox = pc - oy * g.ow;
+        const int oy = fast_div(pc, g.ow, inv_ow), ox = pc - oy * g.ow;
         const int by = oy * g.sh - g.ph, bx = ox * g.sw - g.pw;
         const float* xn = g.x + (size_t)img * g.c * in_plane;
 #pragma unroll

@@ -26,14 +26,6 @@ struct ImplicitArgs {
     int ids_h, ids_w, wflip;
 };
 
-// a / b for 0 <= a < 2^22 and 0 < b: the float quotient is within one of the result, the remainder says which way
-__device__ __forceinline__ int fast_div(int a, int b, float inv_b) {
-    int q = (int)((float)a * inv_b);
-    const int r = a - q * b;
-    q += (r >= b) - (r < 0);
-    return q;
-}
-
 // Few accumulators (MT * PT <= 2 blocks of 32 x 32) leave room for four workgroups per CU instead of two: their
 // staging phases and matrix phases overlap each other.
 template <int MT, int PT>
