@@ -175,6 +175,24 @@ def secondary_workload(name, device, steps, warmup, verbose):
                 "w": dev(rng.uniform(0, 1, (16, 3, 3, 3)).astype(np.float32)),
                 "y": torch.empty((5, 16, 4, 4), dtype=torch.float32, device=device)}
         what, dtype = "single Conv fp32 X[5,3,10,10] W[16,3,3,3] stride 2 (BASELINE.json configs[0]; launch latency)", "f32"
+    elif name == "conv_dense_train":
+        # not a BASELINE.json configuration: a ResNet-sized dense 3x3 convolution with its data and weight gradients,
+        # the shape the implicit-GEMM kernels are quoted on
+        from daceml_amd.autodiff import add_backward_pass
+        g = graphs.GraphBuilder("conv_dense_train", torch.float32)
+        xin = g.input("x", (32, 64, 56, 56))
+        g.input("w", (64, 64, 3, 3))
+        g.output(g.node("Conv", {"X": xin, "W": "w"}, {"Y": (32, 64, 56, 56)}, label="conv", kernel_shape=[3, 3],
+                        pads=[1, 1, 1, 1])["Y"], "y")
+        sdfg = g.sdfg
+        add_backward_pass(sdfg, g.state, ["y"], ["x", "w"])
+        args = {"x": dev(rng.standard_normal((32, 64, 56, 56)).astype(np.float32)),
+                "w": dev((rng.standard_normal((64, 64, 3, 3)) * np.sqrt(2.0 / 576)).astype(np.float32)),
+                "y": torch.empty((32, 64, 56, 56), dtype=torch.float32, device=device),
+                "gradient_y": dev(rng.standard_normal((32, 64, 56, 56)).astype(np.float32)),
+                "gradient_x": torch.empty((32, 64, 56, 56), dtype=torch.float32, device=device),
+                "gradient_w": torch.empty((64, 64, 3, 3), dtype=torch.float32, device=device)}
+        what, dtype = "dense Conv 3x3 fp32 X[32,64,56,56] W[64,64,3,3] pad 1, forward + data and weight gradients", "f32"
     else:
         sys.exit("unknown workload %r" % name)
     prog = CompiledSDFG(sdfg, device=device)
@@ -274,7 +292,7 @@ def module_workload(device, steps, warmup):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="bert_fwd_bwd", choices=["bert_fwd_bwd", "bert_fwd", "nodes", "mbconv", "conv", "module_bert"],
+    ap.add_argument("--workload", default="bert_fwd_bwd", choices=["bert_fwd_bwd", "bert_fwd", "nodes", "mbconv", "conv", "conv_dense_train", "module_bert"],
                     help="bert_fwd_bwd is the headline (default); the others are BASELINE.json's remaining configs")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)

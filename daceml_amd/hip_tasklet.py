@@ -85,6 +85,10 @@ class Stream:
 class HipCall:
     symbol: str
     args: List[Any]
+    #: algorithmic work of this call alone, for nodes whose calls are separate pieces of work (the two gradients of a
+    #: convolution); None: the node's figures go to its first call
+    flops: Any = None
+    bytes_moved: Any = None
 
 
 class HipTasklet(Node):

@@ -1113,15 +1113,17 @@ class HipConvGrad(ONNXForward):
         d = _conv_struct(node, x, w)
         lib = L.load()
         calls, ws = [], 0
+        work = 2 * dy.total_size * w.shape[1] * w.shape[2] * w.shape[3]     # of each of the two gradients
         if "dX" in outs:
             calls.append(HipCall("dmlhip_conv2d_backward_data_f32",
-                                 [Struct(d, "dmlhip_conv2d_desc"), Ptr("dY"), Ptr("W"), Ptr("dX"), Stream()]))
+                                 [Struct(d, "dmlhip_conv2d_desc"), Ptr("dY"), Ptr("W"), Ptr("dX"), Stream()],
+                                 flops=work, bytes_moved=_nbytes(dy, w, x)))
         if "dW" in outs:
             import ctypes
             ws = max(ws, lib.dmlhip_conv2d_backward_weight_workspace_bytes(ctypes.byref(d)))
             calls.append(HipCall("dmlhip_conv2d_backward_weight_f32",
                                  [Struct(d, "dmlhip_conv2d_desc"), Ptr("X"), Ptr("dY"), Ptr("dW"), Workspace(),
-                                  WorkspaceBytes(), Stream()]))
+                                  WorkspaceBytes(), Stream()], flops=work, bytes_moved=_nbytes(x, dy, w)))
         if "dB" in outs:
             # dB[m] = sum_{b, y, x} dY[b, m, y, x]: reduce the spatial dims into the head of the
             # workspace, then the batch dim from there

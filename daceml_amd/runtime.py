@@ -180,8 +180,9 @@ class CompiledSDFG:
                     raise TypeError("unknown HIP call argument %r" % (a, ))
             # work is attributed to the node's first call only (later calls are follow-up passes)
             first = call is calls[0]
-            self._launches.append(_Launch(fn, tuple(args), node.label, call.symbol, node.flops if first else 0,
-                                          node.bytes_moved if first else 0, node.kind, state.label))
+            flops = call.flops if call.flops is not None else (node.flops if first else 0)
+            moved = call.bytes_moved if call.bytes_moved is not None else (node.bytes_moved if first else 0)
+            self._launches.append(_Launch(fn, tuple(args), node.label, call.symbol, flops, moved, node.kind, state.label))
 
     # -- execution -----------------------------------------------------------
     def _bind_arguments(self, kwargs: Dict[str, torch.Tensor], partial: bool = False):
