@@ -57,8 +57,10 @@ template <int OP> __device__ __forceinline__ float unary_grad(float x, float p) 
 
 // ------------------------------------------------------------------ binary, dense fast paths
 // MODE 0: a and b dense and equal-shaped. MODE 1: b is a row vector of `period` elements repeated
-// along the flattened output (bias add). MODE 2: b is one scalar. SWAP evaluates op(b, a) so that
-// the same three layouts serve a broadcast first operand.
+// along the flattened output (bias add). MODE 2: b is one scalar. MODE 3: b holds one value per row of `period`
+// output elements (a per-image, per-channel factor against [N, C, H, W]; n < 2^32). MODE 4: a holds one value per row
+// and b is one scalar (a reduced tensor expanded back over its rows and scaled). SWAP evaluates op(b, a) so that
+// the same layouts serve a broadcast first operand.
 template <typename T, int OP, int MODE, bool SWAP>
 __global__ __launch_bounds__(kEwBlock) void binary_vec_kernel(const T* __restrict__ a, const T* __restrict__ b,
                                                               T* __restrict__ c, int64_t n, int64_t period) {
@@ -66,26 +68,28 @@ __global__ __launch_bounds__(kEwBlock) void binary_vec_kernel(const T* __restric
     constexpr int VN = VecOf<T>::n;
     const int64_t nvec = n / VN;
     const int64_t stride = (int64_t)gridDim.x * kEwBlock;
-    float bs = 0.f;
-    if constexpr (MODE == 2) bs = to_f32(b[0]);
+    float bs = 0.f, as = 0.f;
+    if constexpr (MODE == 2 || MODE == 4) bs = to_f32(b[0]);
     for (int64_t i = (int64_t)blockIdx.x * kEwBlock + threadIdx.x; i < nvec; i += stride) {
-        V av = reinterpret_cast<const V*>(a)[i];
-        V bv;
+        V av, bv;
+        if constexpr (MODE == 4) as = to_f32(a[(uint32_t)(i * VN) / (uint32_t)period]);
+        else av = reinterpret_cast<const V*>(a)[i];
         if constexpr (MODE == 0) bv = reinterpret_cast<const V*>(b)[i];
         if constexpr (MODE == 1) bv = reinterpret_cast<const V*>(b)[(i * VN % period) / VN];
+        if constexpr (MODE == 3) bs = to_f32(b[(uint32_t)(i * VN) / (uint32_t)period]);   // period % VN == 0: one row
         V cv;
 #pragma unroll
         for (int e = 0; e < VN; ++e) {
-            const float x = to_f32(av[e]);
-            const float y = MODE == 2 ? bs : to_f32(bv[e]);
+            const float x = MODE == 4 ? as : to_f32(av[e]);
+            const float y = (MODE == 2 || MODE == 3 || MODE == 4) ? bs : to_f32(bv[e]);
             cv[e] = from_f32<T>(SWAP ? binary_apply<OP>(y, x) : binary_apply<OP>(x, y));
         }
         reinterpret_cast<V*>(c)[i] = cv;
     }
-    // tail (n not a multiple of the vector width; only reachable for MODE 0 and 2)
+    // tail (n not a multiple of the vector width; MODE 1, 3 and 4 are launched with whole vectors only)
     for (int64_t i = nvec * VN + (int64_t)blockIdx.x * kEwBlock + threadIdx.x; i < n; i += stride) {
-        const float x = to_f32(a[i]);
-        const float y = MODE == 2 ? bs : to_f32(b[MODE == 1 ? i % period : i]);
+        const float x = to_f32(a[MODE == 4 ? i / period : i]);
+        const float y = (MODE == 2 || MODE == 4) ? bs : to_f32(b[MODE == 1 ? i % period : (MODE == 3 ? i / period : i)]);
         c[i] = from_f32<T>(SWAP ? binary_apply<OP>(y, x) : binary_apply<OP>(x, y));
     }
 }
@@ -260,6 +264,12 @@ int binary_launch(const T* a, const T* b, T* c, int64_t n, const BcastDims& d, h
     if (al && d.ndim == 2 && d.shape[1] % VN == 0) {
         if (d.sa[0] == d.shape[1] && d.sa[1] == 1 && d.sb[0] == 0 && d.sb[1] == 1) { DML_BIN(1, false, a, b, d.shape[1]); return 0; }
         if (d.sb[0] == d.shape[1] && d.sb[1] == 1 && d.sa[0] == 0 && d.sa[1] == 1) { DML_BIN(1, true, b, a, d.shape[1]); return 0; }
+        if (n < (1LL << 32)) {   // one operand dense, the other one value per row
+            if (d.sa[0] == d.shape[1] && d.sa[1] == 1 && d.sb[0] == 1 && d.sb[1] == 0) { DML_BIN(3, false, a, b, d.shape[1]); return 0; }
+            if (d.sb[0] == d.shape[1] && d.sb[1] == 1 && d.sa[0] == 1 && d.sa[1] == 0) { DML_BIN(3, true, b, a, d.shape[1]); return 0; }
+            if (d.sa[0] == 1 && d.sa[1] == 0 && d.sb[0] == 0 && d.sb[1] == 0) { DML_BIN(4, false, a, b, d.shape[1]); return 0; }
+            if (d.sb[0] == 1 && d.sb[1] == 0 && d.sa[0] == 0 && d.sa[1] == 0) { DML_BIN(4, true, b, a, d.shape[1]); return 0; }
+        }
     }
 #undef DML_BIN
     hipLaunchKernelGGL((binary_general_kernel<T, OP>), ew_grid(n), kEwBlock, 0, st, a, b, c, n, d);

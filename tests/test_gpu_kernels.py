@@ -217,7 +217,9 @@ def test_batchnorm_argument_errors():
 @pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
 @pytest.mark.parametrize("sa,sb", [((4, 8, 64), (4, 8, 64)), ((4, 8, 64), (64, )), ((64, ), (4, 8, 64)),
                                    ((4, 8, 64), (1, )), ((1, ), (5, 7)), ((4, 1, 6), (1, 5, 6)), ((3, 5), (3, 1)),
-                                   ((2, 3, 4, 5, 6), (3, 1, 5, 1)), ((1000, 33), (33, )), ((7, ), (7, ))])
+                                   ((2, 3, 4, 5, 6), (3, 1, 5, 1)), ((1000, 33), (33, )), ((7, ), (7, )),
+                                   # one value per (image, channel) against [N, C, H, W], both ways round
+                                   ((3, 5, 4, 8), (3, 5, 1, 1)), ((3, 5, 1, 1), (3, 5, 4, 8)), ((6, 40), (6, 1))])
 def test_binary(dtype, op, sa, sb):
     from daceml_amd import _lib as L, kernels as K
     a, a64 = _inputs(13, sa, dtype)
