@@ -3,8 +3,9 @@
 // go through a workspace and a fixed-order reduction, never atomics).
 //
 //   * depthwise data gradient: dX[iy, ix] = sum_{hy, hx} W[hy, hx] dY[(iy + P - hy) / S, (ix + P - hx) / S] over the taps
-//     for which the divisions are exact. A thread owns one S x S block of dX; which taps reach which of its pixels is
-//     known at compile time, so there is no divisibility test and each dY value of the small neighbourhood is loaded once.
+//     for which the divisions are exact. A thread owns S rows of four dX pixels; which taps reach which of its pixels
+//     is known at compile time, so there is no divisibility test, each dY value of the small neighbourhood is loaded
+//     once and a row's four pixels leave as one 16-byte store.
 //   * depthwise weight gradient: dW[hy, hx] = sum_{n, oy, ox} dY[n, oy, ox] X[n, oy S - P + hy, ox S - P + hx]; one
 //     workgroup per (image, channel) plane keeps K*K running sums per thread, the planes' results are summed over the
 //     images by the reduction kernel.
@@ -40,12 +41,14 @@ template <int K, int S, int P> struct DwBack {
     static constexpr int span() { return hi() - lo() + 1; }
 };
 
-template <int K, int S, int P>
+// CX adjacent cells per thread: with S * CX == 4 a thread's pixels of a row are one aligned 16-byte store, and the dY
+// columns shared by neighbouring cells are loaded once.
+template <int K, int S, int P, int CX>
 __global__ __launch_bounds__(256) void depthwise_bwd_data_kernel(const float* __restrict__ dy, const float* __restrict__ w,
                                                                  float* __restrict__ dx, int c, int h, int wd, int oh, int ow,
-                                                                 int cw, int cells, uint32_t chunks, int pairs) {
+                                                                 int cw, int cells, uint32_t chunks, int vec) {
     using G = DwBack<K, S, P>;
-    constexpr int LO = G::lo(), NB = G::span();
+    constexpr int LO = G::lo(), NB = G::span(), NBX = NB + CX - 1, PX = S * CX;
     const uint32_t plane = blockIdx.x / chunks, chunk = blockIdx.x - plane * chunks;
     const int ci = (int)(plane % (uint32_t)c);
     float wk[K * K];
@@ -57,13 +60,13 @@ __global__ __launch_bounds__(256) void depthwise_bwd_data_kernel(const float* __
     for (int rep = 0; rep < 4; ++rep) {
         const int idx = (int)chunk * 1024 + rep * 256 + (int)threadIdx.x;
         if (idx >= cells) return;
-        const int a = idx / cw, b = idx - a * cw;
-        float nb[NB][NB];
+        const int a = idx / cw, b = (idx - a * cw) * CX;     // first cell of the thread's group
+        float nb[NB][NBX];
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
             const int oy = a + LO + u;
 #pragma unroll
-            for (int v = 0; v < NB; ++v) {
+            for (int v = 0; v < NBX; ++v) {
                 const int ox = b + LO + v;
                 const bool ok = oy >= 0 && oy < oh && ox >= 0 && ox < ow;
                 nb[u][v] = ok ? gp[(size_t)(ok ? oy : 0) * ow + (ok ? ox : 0)] : 0.f;
@@ -72,28 +75,32 @@ __global__ __launch_bounds__(256) void depthwise_bwd_data_kernel(const float* __
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             const int iy = a * S + i;
-            float out[S];
+            float out[PX];
 #pragma unroll
-            for (int j = 0; j < S; ++j) {
-                float acc = 0.f;
+            for (int cx = 0; cx < CX; ++cx)
 #pragma unroll
-                for (int t = 0; t < G::taps(i); ++t)
+                for (int j = 0; j < S; ++j) {
+                    float acc = 0.f;
 #pragma unroll
-                    for (int u = 0; u < G::taps(j); ++u)
-                        acc += wk[(G::r(i) + S * t) * K + G::r(j) + S * u] * nb[G::q(i) - t - LO][G::q(j) - u - LO];
-                out[j] = acc;
-            }
+                    for (int t = 0; t < G::taps(i); ++t)
+#pragma unroll
+                        for (int u = 0; u < G::taps(j); ++u)
+                            acc += wk[(G::r(i) + S * t) * K + G::r(j) + S * u] *
+                                   nb[G::q(i) - t - LO][cx + G::q(j) - u - LO];
+                    out[cx * S + j] = acc;
+                }
             if (iy < h) {
-                if constexpr (S == 2) {
-                    // even row length and an 8-byte aligned tensor: the block's two pixels of a row go out as one store
-                    if (pairs) {
-                        *reinterpret_cast<floatx2*>(xp + (size_t)iy * wd + b * 2) = floatx2{out[0], out[1]};
+                float* row = xp + (size_t)iy * wd + b * S;
+                if constexpr (PX == 4) {
+                    // row length a multiple of 4 and a 16-byte aligned tensor: one store for the thread's four pixels
+                    if (vec) {
+                        *reinterpret_cast<floatx4*>(row) = floatx4{out[0], out[1], out[2], out[3]};
                         continue;
                     }
                 }
 #pragma unroll
-                for (int j = 0; j < S; ++j)
-                    if (b * S + j < wd) xp[(size_t)iy * wd + b * S + j] = out[j];
+                for (int j = 0; j < PX; ++j)
+                    if (b * S + j < wd) row[j] = out[j];
             }
         }
     }
@@ -426,16 +433,17 @@ bool depthwise_bwd_supported(int k, int s, int p) {
 
 int launch_depthwise_bwd_data(const float* dy, const float* w, float* dx, int n, int c, int h, int wd, int oh, int ow, int k,
                               int s, hipStream_t st) {
-    const int ch = (h + s - 1) / s, cw = (wd + s - 1) / s;
+    const int cx = 4 / s;                                         // cells per thread: four pixels of a row
+    const int ch = (h + s - 1) / s, cw = (int)ceil_div((wd + s - 1) / s, cx);
     const int64_t cells = (int64_t)ch * cw;
     const int64_t chunks = ceil_div(cells, (int64_t)1024);
     const int64_t blocks = (int64_t)n * c * chunks;
     DML_REQUIRE(cells <= (1 << 30) && blocks <= 2147483647LL, DMLHIP_ERR_SHAPE, "conv2d_backward_data: too many workgroups");
-    const int pairs = wd % 2 == 0 && ((uintptr_t)dx & 7) == 0;
+    const int vec = wd % 4 == 0 && ((uintptr_t)dx & 15) == 0;
 #define DML_DWB(K, S, P)                                                                                               \
     if (k == K && s == S) {                                                                                            \
-        hipLaunchKernelGGL((depthwise_bwd_data_kernel<K, S, P>), (unsigned)blocks, 256, 0, st, dy, w, dx, c, h, wd, oh, ow, \
-                           cw, (int)cells, (uint32_t)chunks, pairs);                                                        \
+        hipLaunchKernelGGL((depthwise_bwd_data_kernel<K, S, P, 4 / S>), (unsigned)blocks, 256, 0, st, dy, w, dx, c, h, wd, \
+                           oh, ow, cw, (int)cells, (uint32_t)chunks, vec);                                             \
         return launch_status("conv2d_backward_data(depthwise)");                                                       \
     }
     DML_DWB(3, 1, 1) DML_DWB(3, 2, 1) DML_DWB(5, 1, 2) DML_DWB(5, 2, 2)
