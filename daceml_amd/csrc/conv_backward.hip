@@ -57,8 +57,8 @@ __global__ __launch_bounds__(256) void depthwise_bwd_data_kernel(const float* __
     const float* gp = dy + (size_t)plane * oh * ow;
     float* xp = dx + (size_t)plane * h * wd;
 #pragma unroll 1
-    for (int rep = 0; rep < 4; ++rep) {
-        const int idx = (int)chunk * 1024 + rep * 256 + (int)threadIdx.x;
+    for (int rep = 0; rep < 8; ++rep) {
+        const int idx = (int)chunk * 2048 + rep * 256 + (int)threadIdx.x;
         if (idx >= cells) return;
         const int a = idx / cw, b = (idx - a * cw) * CX;     // first cell of the thread's group
         float nb[NB][NBX];
@@ -436,7 +436,7 @@ int launch_depthwise_bwd_data(const float* dy, const float* w, float* dx, int n,
     const int cx = 4 / s;                                         // cells per thread: four pixels of a row
     const int ch = (h + s - 1) / s, cw = (int)ceil_div((wd + s - 1) / s, cx);
     const int64_t cells = (int64_t)ch * cw;
-    const int64_t chunks = ceil_div(cells, (int64_t)1024);
+    const int64_t chunks = ceil_div(cells, (int64_t)2048);
     const int64_t blocks = (int64_t)n * c * chunks;
     DML_REQUIRE(cells <= (1 << 30) && blocks <= 2147483647LL, DMLHIP_ERR_SHAPE, "conv2d_backward_data: too many workgroups");
     const int vec = wd % 4 == 0 && ((uintptr_t)dx & 15) == 0;
