@@ -111,7 +111,7 @@ template <int K, int S>
 __global__ __launch_bounds__(256) void depthwise_bwd_weight_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                                    float* __restrict__ part, int h, int wd, int oh, int ow,
                                                                    int pad) {
-    __shared__ float scratch[4];
+    __shared__ float red[4][K * K];
     const size_t plane = blockIdx.x;
     const float* xp = x + plane * h * wd;
     const float* gp = dy + plane * oh * ow;
@@ -136,12 +136,18 @@ __global__ __launch_bounds__(256) void depthwise_bwd_weight_kernel(const float* 
             }
         }
     }
+    // wavefront sums first, then one exchange through LDS for all K * K values (a single barrier)
 #pragma unroll
-    for (int i = 0; i < K * K; ++i) {
-        const float s = block_reduce<OpSum, 4>(acc[i], scratch);
-        if (threadIdx.x == 0) part[plane * (K * K) + i] = s;
-        __syncthreads();
+    for (int i = 0; i < K * K; ++i) acc[i] = wave_reduce<OpSum>(acc[i]);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < K * K; ++i) red[wave][i] = acc[i];
     }
+    __syncthreads();
+    if (threadIdx.x < K * K)
+        part[plane * (K * K) + threadIdx.x] =
+            (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
 // ---------------------------------------------------------------- pointwise, weight gradient
