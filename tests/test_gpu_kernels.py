@@ -475,6 +475,8 @@ CONV_CASES = [
     ((5, 12, 20, 24), (70, 12, 3, 3), (1, 1), (2, 2), (2, 2), 1, False),    # dilated, ragged output channels
     ((4, 20, 30, 31), (33, 20, 3, 5), (2, 1), (1, 2), (1, 1), 1, True),     # 3x5 taps, strides 2x1, pads 1x2
     ((16, 8, 112, 112), (16, 8, 3, 3), (1, 1), (1, 1), (1, 1), 1, False),   # many pixels: 256-pixel workgroups
+    ((2, 37, 33, 35), (33, 37, 3, 3), (1, 1), (1, 1), (1, 1), 1, True),     # dense, every extent odd / ragged
+    ((3, 24, 31, 29), (48, 24, 5, 5), (2, 2), (2, 2), (1, 1), 1, False),    # dense 5x5 stride 2: gradient over zero-dilated dY
     # one image: the weight-gradient kernels have a single partial result and write dW directly
     ((1, 32, 16, 16), (24, 32, 1, 1), (1, 1), (0, 0), (1, 1), 1, True),     # pointwise
     ((1, 64, 16, 16), (128, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1, False),   # dense
