@@ -366,6 +366,46 @@ __global__ __launch_bounds__(256) void conv_1x1_spatial1_kernel(const T* __restr
     if (lane == 0) y[o] = from_f32<T>(apply_act(act, s + (bias ? to_f32(bias[im]) : 0.f)));
 }
 
+// Gradients of those squeeze-excite sized products. One thread per output, a short loop, coalesced along the
+// output's fast index: dX[n, c] = sum_m dY[n, m] W[m, c] and dW[m, c] = sum_n dY[n, m] X[n, c].
+__global__ __launch_bounds__(256) void conv_1x1_spatial1_bwd_data_kernel(const float* __restrict__ dy,
+                                                                         const float* __restrict__ w, float* __restrict__ dx,
+                                                                         int n, int c, int m) {
+    const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (o >= (int64_t)n * c) return;
+    const int in = (int)(o / c), ic = (int)(o % c);
+    const float* g = dy + (int64_t)in * m;
+    // four running sums: independent chains for the loads, and a shorter chain of roundings for the result
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int k = 0;
+    for (; k + 3 < m; k += 4) {
+        a0 += g[k] * w[(int64_t)k * c + ic];
+        a1 += g[k + 1] * w[(int64_t)(k + 1) * c + ic];
+        a2 += g[k + 2] * w[(int64_t)(k + 2) * c + ic];
+        a3 += g[k + 3] * w[(int64_t)(k + 3) * c + ic];
+    }
+    for (; k < m; ++k) a0 += g[k] * w[(int64_t)k * c + ic];
+    dx[o] = (a0 + a1) + (a2 + a3);
+}
+
+__global__ __launch_bounds__(256) void conv_1x1_spatial1_bwd_weight_kernel(const float* __restrict__ x,
+                                                                           const float* __restrict__ dy,
+                                                                           float* __restrict__ dw, int n, int c, int m) {
+    const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (o >= (int64_t)m * c) return;
+    const int im = (int)(o / c), ic = (int)(o % c);
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int b = 0;
+    for (; b + 3 < n; b += 4) {
+        a0 += dy[(int64_t)b * m + im] * x[(int64_t)b * c + ic];
+        a1 += dy[(int64_t)(b + 1) * m + im] * x[(int64_t)(b + 1) * c + ic];
+        a2 += dy[(int64_t)(b + 2) * m + im] * x[(int64_t)(b + 2) * c + ic];
+        a3 += dy[(int64_t)(b + 3) * m + im] * x[(int64_t)(b + 3) * c + ic];
+    }
+    for (; b < n; ++b) a0 += dy[(int64_t)b * m + im] * x[(int64_t)b * c + ic];
+    dw[o] = (a0 + a1) + (a2 + a3);
+}
+
 int launch_pointwise_f32(const float* x, const float* w, const float* bias, const float* in_scale, float* y, int n, int cin,
                          int cout, int64_t hw, int act, hipStream_t st, bool w_transposed = false) {
     int mt = (int)ceil_div(cout, 32);
@@ -562,6 +602,11 @@ int dmlhip_conv2d_backward_data_f32(const dmlhip_conv2d_desc* d, const void* dy,
     if (g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.group == 1 && g.m > 0) {
         // dX[b] (C x HW) = W^T (C x M) . dY[b] (M x HW)
         const int64_t hw = (int64_t)g.h * g.w;
+        if (hw == 1 && (int64_t)g.n * g.c <= (1 << 22)) {
+            hipLaunchKernelGGL(conv_1x1_spatial1_bwd_data_kernel, (unsigned)ceil_div((int64_t)g.n * g.c, 256), 256, 0, st,
+                               (const float*)dy, (const float*)w, (float*)dx, g.n, g.c, g.m);
+            return launch_status("conv2d_backward_data(1x1 on 1x1)");
+        }
         // many pixels: the streaming pointwise kernel with dY as its input and W read as [cin = M][cout = C]
         if (hw % 4 == 0 && hw >= 128 && g.n <= 65535 && aligned16(dy) && aligned16(dx))
             return launch_pointwise_f32((const float*)dy, (const float*)w, nullptr, nullptr, (float*)dx, g.n, g.m, g.c, hw,
@@ -588,6 +633,7 @@ int dmlhip_conv2d_backward_data_f32(const dmlhip_conv2d_desc* d, const void* dy,
 size_t dmlhip_conv2d_backward_weight_workspace_bytes(const dmlhip_conv2d_desc* d) {
     ConvGeom g;
     if (make_geom(d, &g, "conv2d_backward_weight")) return 0;
+    if (is_pointwise(g) && (int64_t)g.h * g.w == 1 && (int64_t)g.m * g.c <= (1 << 22)) return 0;   // one small kernel
     if (is_pointwise(g) && g.n >= 1) {
         // the larger of what the two paths need: per-workgroup results of the streaming kernel, or per-image
         // products of the batched GEMM (taken when the streaming kernel does not apply or an operand is unaligned)
@@ -653,6 +699,11 @@ int dmlhip_conv2d_backward_weight_f32(const dmlhip_conv2d_desc* d, const void* x
         const size_t part_bytes = (size_t)dense_parts * total * sizeof(float);
         return dmlhip_reduce_f32(DMLHIP_RSUM, part, dw, DMLHIP_F32, 1, dense_parts, total, (char*)workspace + part_bytes,
                                  workspace_bytes - part_bytes, stream);
+    }
+    if (is_pointwise(g) && red > 0 && (int64_t)g.h * g.w == 1 && total <= (1 << 22)) {
+        hipLaunchKernelGGL(conv_1x1_spatial1_bwd_weight_kernel, (unsigned)ceil_div(total, 256), 256, 0, st,
+                           (const float*)x, (const float*)dy, (float*)dw, g.n, g.c, g.m);
+        return launch_status("conv2d_backward_weight(1x1 on 1x1)");
     }
     if (is_pointwise(g) && red > 0) {
         const int64_t hw = (int64_t)g.h * g.w;
