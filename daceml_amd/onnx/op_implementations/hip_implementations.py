@@ -16,7 +16,7 @@ from ... import _lib as L
 from ... import contraction as C
 from ...hip_tasklet import (F32, I32, I64, HipCall, HipTasklet, I64Array, Null, Ptr, PtrArray, Stream, Struct,
                             USize, ViewTasklet, Workspace, WorkspaceBytes)
-from ...sdfg import (FLOAT_DTYPES, SDFG, Array, SDFGState, in_desc_with_name, out_desc_with_name)
+from ...sdfg import (FLOAT_DTYPES, SDFG, AccessNode, Array, SDFGState, in_desc_with_name, out_desc_with_name)
 from ..forward_implementation_abc import ONNXForward
 from ..nodes import ONNXOp
 from .utils import op_implementation
@@ -859,15 +859,27 @@ class HipBatchNormalization(ONNXForward):
                             I64(hw), F32(node.epsilon)] + fused + [Stream()])
             return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="batchnorm")
         ws = L.load().dmlhip_batchnorm_workspace_bytes(n, c, hw)
-        calls = [HipCall("dmlhip_batchnorm_training_" + variant + sfx,
-                         [Ptr("X"), Ptr("scale"), Ptr("B"), Ptr("in_mean"), Ptr("in_var"), Ptr("Y"), Ptr("out_mean"),
-                          Ptr("out_var"), Ptr("saved_mean"), Ptr("saved_var"), I64(n), I64(c), I64(hw),
-                          F32(node.epsilon), F32(node.momentum)] + fused + [Workspace(), WorkspaceBytes(), Stream()])]
+        # running statistics: where the updated value has no reader of its own and the array it came from is a
+        # caller-owned buffer, the kernel writes it there directly (its out_* may alias its in_*); otherwise it goes to
+        # the node's output and, for caller-owned inputs, is copied back as the reference does (:392-410)
+        out_ptr, copies = {}, []
         for src, dst in (("out_mean", "in_mean"), ("out_var", "in_var")):
-            arr = next(iter(state.in_edges_by_connector(node, dst))).data.data
-            if not sdfg.arrays[arr].transient and arr not in sdfg.constants:
-                calls.append(HipCall("dmlhip_unary_" + sfx, [I32(L.IDENTITY), Ptr(src), Ptr(dst), I64(c), F32(0.0),
-                                                             Stream()]))
+            in_arr = next(iter(state.in_edges_by_connector(node, dst))).data.data
+            out_arr = next(iter(state.out_edges_by_connector(node, src))).data.data
+            caller_owned = not sdfg.arrays[in_arr].transient and in_arr not in sdfg.constants
+            unread = (sdfg.arrays[out_arr].transient
+                      and not any(isinstance(e.src, AccessNode) and e.src.data == out_arr
+                                  for st in sdfg.states() for e in st.edges())
+                      and not any(d.view_of == out_arr for d in sdfg.arrays.values()))
+            out_ptr[src] = Ptr(dst) if (caller_owned and unread) else Ptr(src)
+            if caller_owned and not unread:
+                copies.append(HipCall("dmlhip_unary_" + sfx, [I32(L.IDENTITY), Ptr(src), Ptr(dst), I64(c), F32(0.0),
+                                                              Stream()]))
+        calls = [HipCall("dmlhip_batchnorm_training_" + variant + sfx,
+                         [Ptr("X"), Ptr("scale"), Ptr("B"), Ptr("in_mean"), Ptr("in_var"), Ptr("Y"), out_ptr["out_mean"],
+                          out_ptr["out_var"], Ptr("saved_mean"), Ptr("saved_var"), I64(n), I64(c), I64(hw),
+                          F32(node.epsilon), F32(node.momentum)] + fused + [Workspace(), WorkspaceBytes(), Stream()])]
+        calls += copies
         return _tasklet(node, state, calls, workspace_bytes=ws, bytes_moved=3 * _nbytes(x), kind="batchnorm")
 
 
