@@ -49,6 +49,54 @@ __global__ __launch_bounds__(kRedBlock) void row_reduce_kernel(const TIn* __rest
     if (row < rows && tid == 0) y[row] = from_f32<TOut>(a * scale);
 }
 
+// y[row] = sum_j a[row, j] * b[row, j]: a Mul whose only reader is a ReduceSum over the trailing axes, without the
+// product tensor (the gradient of a per-row factor such as a squeeze-excite gate)
+template <typename T, bool WAVE>
+__global__ __launch_bounds__(kRedBlock) void row_dot_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                            T* __restrict__ y, int64_t rows, int64_t r) {
+    __shared__ float scratch[kRedWaves];
+    const int64_t row = WAVE ? (int64_t)blockIdx.x * kRedWaves + threadIdx.x / kWave : (int64_t)blockIdx.x;
+    const int tid = WAVE ? (threadIdx.x & (kWave - 1)) : threadIdx.x;
+    const int nth = WAVE ? kWave : kRedBlock;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    if (row < rows) {
+        const T* ar = a + row * r;
+        const T* br = b + row * r;
+        int64_t c = tid;
+        for (; c + 3 * nth < r; c += 4 * nth) {
+            a0 += to_f32(ar[c]) * to_f32(br[c]);
+            a1 += to_f32(ar[c + nth]) * to_f32(br[c + nth]);
+            a2 += to_f32(ar[c + 2 * nth]) * to_f32(br[c + 2 * nth]);
+            a3 += to_f32(ar[c + 3 * nth]) * to_f32(br[c + 3 * nth]);
+        }
+        for (; c < r; c += nth) a0 += to_f32(ar[c]) * to_f32(br[c]);
+    }
+    float s = (a0 + a1) + (a2 + a3);
+    if constexpr (WAVE) {
+        s = wave_reduce<OpSum>(s);
+    } else {
+        s = block_reduce<OpSum, kRedWaves>(s, scratch);
+    }
+    if (row < rows && tid == 0) y[row] = from_f32<T>(s);
+}
+
+template <typename T>
+int row_dot_impl(const void* a, const void* b, void* y, int64_t rows, int64_t r, void* stream) {
+    DML_REQUIRE(rows >= 0 && r >= 0, DMLHIP_ERR_SHAPE, "row_dot: negative extent");
+    DML_REQUIRE(rows <= 2147483647LL, DMLHIP_ERR_SHAPE, "row_dot: too many rows");
+    DML_REQUIRE(r == 0 || rows <= (INT64_MAX / 16) / r, DMLHIP_ERR_SHAPE, "row_dot: size overflows");
+    if (rows == 0) return 0;
+    DML_REQUIRE(y && (r == 0 || (a && b)), DMLHIP_ERR_NULL, "row_dot: NULL tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (r <= 2048)
+        hipLaunchKernelGGL((row_dot_kernel<T, true>), (unsigned)ceil_div(rows, kRedWaves), kRedBlock, 0, st, (const T*)a,
+                           (const T*)b, (T*)y, rows, r);
+    else
+        hipLaunchKernelGGL((row_dot_kernel<T, false>), (unsigned)rows, kRedBlock, 0, st, (const T*)a, (const T*)b, (T*)y,
+                           rows, r);
+    return launch_status("row_dot");
+}
+
 // ---------------------------------------------------------------- inner > 1
 // grid: x = column tiles, y = outer, z = splits of r. V = elements per lane along inner.
 template <typename TIn, typename TOut, int OP, int V>
@@ -380,6 +428,13 @@ int dmlhip_reduce_f16(int op, const void* x, void* y, int out_dtype, int64_t out
 int dmlhip_reduce_f32(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r, int64_t inner,
                       void* workspace, size_t workspace_bytes, void* stream) {
     return reduce_impl<float>(op, x, y, out_dtype, outer, r, inner, workspace, workspace_bytes, stream);
+}
+
+int dmlhip_row_dot_f16(const void* a, const void* b, void* y, int64_t rows, int64_t cols, void* stream) {
+    return row_dot_impl<_Float16>(a, b, y, rows, cols, stream);
+}
+int dmlhip_row_dot_f32(const void* a, const void* b, void* y, int64_t rows, int64_t cols, void* stream) {
+    return row_dot_impl<float>(a, b, y, rows, cols, stream);
 }
 
 }  // extern "C"

@@ -185,6 +185,21 @@ def batchnorm_backward(dy, x, scale, saved_mean, saved_var, eps=1e-5, act: int =
     return dx, dscale, dbias
 
 
+def row_dot(a: torch.Tensor, b: torch.Tensor, keep: int) -> torch.Tensor:
+    """sum(a * b) over every axis from ``keep`` on; the result has the leading ``keep`` axes."""
+    _check(a, b, dtype=a.dtype)
+    if a.shape != b.shape:
+        raise ValueError("row_dot: operands must have one shape, got %s and %s" % (tuple(a.shape), tuple(b.shape)))
+    a, b = _dense(a), _dense(b)
+    rows = 1
+    for d in a.shape[:keep]:
+        rows *= d
+    cols = a.numel() // rows if rows else 0
+    y = torch.empty(tuple(a.shape[:keep]), dtype=a.dtype, device=a.device)
+    L.check(_fn("row_dot", a.dtype)(_ptr(a), _ptr(b), _ptr(y), rows, cols, _stream()))
+    return y
+
+
 # ----------------------------------------------------------------------------- elementwise
 def _bcast_strides(t: torch.Tensor, shape: Sequence[int]):
     nd = len(shape)

@@ -150,6 +150,9 @@ SCHEMAS = [
     # data__i over every axis but the last (the bias gradients of a backward pass)
     _schema("EinsumSum", "A* B* Residual?", "Output", since=1, equation=REQUIRED, alpha=1.0),
     _schema("MultiReduceSum", "data*", "reduced*", since=1),
+    # reduced = ReduceSum(Mul(A, B), axes) with A and B of one shape and `axes` the trailing axes: the product is not
+    # written (the gradient of a broadcast factor)
+    _schema("MulReduceSum", "A B", "reduced", since=1, axes=REQUIRED, keepdims=1),
     # backward nodes emitted by the "hip" BackwardImplementations (names follow the ONNX Runtime
     # training contrib ops)
     _schema("SoftmaxGrad", "dY Y", "dX", since=1, axis=-1),

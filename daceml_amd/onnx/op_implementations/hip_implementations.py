@@ -731,6 +731,32 @@ def _make_reduce(op_name: str, code: int, doc: str):
     return op_implementation(op=op_name, name=IMPL)(_Reduce)
 
 
+@op_implementation(op="MulReduceSum", name=IMPL)
+class HipMulReduceSum(ONNXForward):
+    """Mul (pure_implementations.py:86-88) read only by ReduceSum over the trailing axes (:294-296) as one row-wise dot
+    product: the product tensor is never written."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            a = in_desc_with_name(node, state, sdfg, "A")
+            b = in_desc_with_name(node, state, sdfg, "B")
+            y = out_desc_with_name(node, state, sdfg, "reduced")
+            geo = _reduce_geometry(a.shape, node.axes)
+            if geo is None or a.shape != b.shape or not (a.dtype in FLOAT_DTYPES and a.dtype == b.dtype == y.dtype):
+                return False
+            outer, r, inner, _ = geo
+            return inner == 1 and _dense(a, b, y) and y.total_size == outer and outer < 2 ** 31
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        a = in_desc_with_name(node, state, sdfg, "A")
+        outer, r, _, _ = _reduce_geometry(a.shape, node.axes)
+        call = HipCall("dmlhip_row_dot_" + _SFX[a.dtype], [Ptr("A"), Ptr("B"), Ptr("reduced"), I64(outer), I64(r), Stream()])
+        return _tasklet(node, state, [call], flops=2 * a.total_size, bytes_moved=2 * _nbytes(a), kind="reduce")
+
+
 HipReduceSum = _make_reduce("ReduceSum", L.RSUM, "ReduceSum (pure_implementations.py:294-296); adjacent axes.")
 HipReduceMax = _make_reduce("ReduceMax", L.RMAX, "ReduceMax (pure_implementations.py:299-301); adjacent axes.")
 HipReduceMin = _make_reduce("ReduceMin", L.RMIN, "ReduceMin (pure_implementations.py:304-306); adjacent axes.")

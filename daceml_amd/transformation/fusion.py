@@ -1089,10 +1089,47 @@ def fuse_einsum_sums(sdfg: SDFG, max_group: int = 4) -> int:
     return saved
 
 
+def fuse_mul_reduce(sdfg: SDFG) -> int:
+    """Mul of two equal-shaped arrays whose product only a ReduceSum over the trailing axes reads becomes one
+    MulReduceSum (a dot product per row): the product tensor disappears. This is what the reversal of a broadcast
+    multiplication leaves for the broadcast operand, e.g. the gradient of a squeeze-excite gate."""
+    count = 0
+    for state in sdfg.states():
+        for red in [n for n in state.nodes() if _is_op(n, "ReduceSum")]:
+            data = _in_array(state, red, "data")
+            prod = _producer(state, data)
+            if prod is None or not _is_op(prod[0], "Mul") or not _internal(sdfg, state, data):
+                continue
+            mul = prod[0]
+            a, b = _in_array(state, mul, "A"), _in_array(state, mul, "B")
+            da, db, dd = sdfg.arrays[a], sdfg.arrays[b], sdfg.arrays[data]
+            if not (tuple(da.shape) == tuple(db.shape) == tuple(dd.shape) and da.dtype == db.dtype == dd.dtype):
+                continue
+            if not (da.is_contiguous() and db.is_contiguous()):
+                continue
+            nd = len(dd.shape)
+            axes = sorted(set(range(nd) if red.axes is None else [x % nd for x in red.axes]))
+            if not axes or axes != list(range(axes[0], nd)):          # the trailing axes, all of them
+                continue
+            out = _out_array(state, red, "reduced")
+            if sdfg.arrays[out].dtype != dd.dtype:
+                continue
+            label = red.label
+            keep = red.keepdims
+            _remove_node(state, red)
+            _remove_node(state, mul)
+            _add_node(sdfg, state, "MulReduceSum", label, {"A": a, "B": b}, {"reduced": out}, axes=axes, keepdims=keep)
+            count += 1
+    if count:
+        _drop_unused_arrays(sdfg)
+    return count
+
+
 def optimize_backward(sdfg: SDFG) -> Dict[str, int]:
     """Rewrites for the state(s) autodiff added — what a ``post_autodiff_hooks`` entry of the reference's module
     wrapper would run (daceml/torch/module.py:46-365)."""
     stats = {"bias_gradients": fuse_bias_gradients(sdfg)}
+    stats["mul_reductions"] = fuse_mul_reduce(sdfg)    # before fuse_reductions: these sums stop being plain ReduceSums
     stats["reductions"] = fuse_reductions(sdfg)
     stats["einsum_sums"] = fuse_einsum_sums(sdfg)      # before grouping: a summed group needs no separate outputs
     stats["grouped_einsums"] = group_einsums(sdfg)

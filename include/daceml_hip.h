@@ -151,6 +151,12 @@ int dmlhip_reduce_f16(int op, const void* x, void* y, int out_dtype, int64_t out
                       int64_t inner, void* workspace, size_t workspace_bytes, void* stream);
 int dmlhip_reduce_f32(int op, const void* x, void* y, int out_dtype, int64_t outer, int64_t r,
                       int64_t inner, void* workspace, size_t workspace_bytes, void* stream);
+/* y[row] = sum_j a[row, j] * b[row, j] for dense [rows, cols] operands, fp32 accumulation, y in the operands' type:
+ * ONNXMul (pure_implementations.py:86-88) read only by ONNXReduceSum over the trailing axes (:294-296) — what the
+ * reversal of a broadcast multiplication emits for the broadcast operand (autodiff/backward_pass_generator.py:1284-1421
+ * with ReverseReduce, autodiff/implementations/dace_nodes.py:13-105) — without writing the product. */
+int dmlhip_row_dot_f16(const void* a, const void* b, void* y, int64_t rows, int64_t cols, void* stream);
+int dmlhip_row_dot_f32(const void* a, const void* b, void* y, int64_t rows, int64_t cols, void* stream);
 /* Several independent ReduceSum nodes over all leading axes (keepdims = 0) in one launch pair:
  * y[t][c] = sum_r x[t][r, c] for count <= DMLHIP_MULTI_MAX row-major matrices [rows[t], cols[t]].
  * This is the shape of the bias gradients DefaultEinsumBackward's callers need

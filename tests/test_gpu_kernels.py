@@ -235,6 +235,22 @@ def test_binary(dtype, op, sa, sb):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape,keep", [((3, 5, 7, 9), 2), ((4, 3000), 1), ((6, 1), 1), ((2, 3, 4), 0), ((5, 64), 2)])
+def test_row_dot(dtype, shape, keep):
+    """sum(a * b) over the trailing axes in one kernel, against the oracle's Mul followed by ReduceSum."""
+    from daceml_amd import kernels as K
+    a, a64 = _inputs(160, shape, dtype)
+    b, b64 = _inputs(161, shape, dtype)
+    want = O.reduce_sum(O.mul(a64, b64), list(range(keep, len(shape))), 0) if keep < len(shape) else O.mul(a64, b64)
+    got = K.row_dot(dev(a), dev(b), keep)
+    assert tuple(got.shape) == tuple(np.shape(want))
+    cols = int(np.prod(shape[keep:]))
+    kw = dict(rtol=1e-5, atol=1e-6 * max(1.0, np.sqrt(cols / 64.0))) if dtype == torch.float32 else \
+        dict(rtol=2e-2, atol=1e-2 * max(1.0, np.sqrt(cols / 64.0)))
+    assert_close(host(got), want, dtype, "row dot %s keep %d" % (shape, keep), **kw)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_pow(dtype):
     from daceml_amd import _lib as L, kernels as K
     a, a64 = _inputs(15, (33, 65), dtype)

@@ -430,7 +430,8 @@ def test_attention_fusion_roles_and_graph():
     assert ins == {"Q", "K", "V", "O", "LogSumExp", "dO"}
     # the six bias gradients become one node; nothing else in the state changes
     n_before = len(sdfg.states()[1].library_nodes())
-    assert fusion.optimize_backward(sdfg) == {"bias_gradients": 6, "reductions": 0, "einsum_sums": 6, "grouped_einsums": 5}
+    assert fusion.optimize_backward(sdfg) == {"bias_gradients": 6, "mul_reductions": 0, "reductions": 0, "einsum_sums": 6,
+                                             "grouped_einsums": 5}
     bnodes = sdfg.states()[1].library_nodes()
     # six bias-gradient reductions (now InputSum outputs of the weight-gradient contractions), two gradient sums and five
     # contractions fewer (q/k/v input gradients: 3 -> 1 EinsumSum that also adds the residual path; o/q/k/v weight
@@ -491,6 +492,25 @@ def test_batchnorm_activation_fusion_keeps_the_backward_pass():
     grad = [n for n in g.sdfg.states()[1].library_nodes() if n.schema.name == "BatchNormalizationGrad"]
     assert len(grad) == 1 and grad[0].activation == "swish" and "B" in grad[0].in_connectors
     assert [n.schema.name for n in g.sdfg.states()[1].library_nodes()] == ["BatchNormalizationGrad"]
+
+
+def test_mul_reduce_fusion_on_a_gate_gradient():
+    """y = x * gate[n, c, 1, 1]: the gate's gradient is ReduceSum(Mul(dy, x)) over the two trailing axes; after
+    optimize_backward it is one MulReduceSum and the product array is gone."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.transformation import fusion
+    g = graphs.GraphBuilder("gate", torch.float32)
+    x, gate = g.input("x", (2, 6, 8, 8)), g.input("gate", (2, 6, 1, 1))
+    g.output(g.node("Mul", {"A": x, "B": gate}, {"C": (2, 6, 8, 8)}, label="m")["C"], "y")
+    add_backward_pass(g.sdfg, g.state, ["y"], ["x", "gate"])
+    before = sorted(n.schema.name for n in g.sdfg.states()[1].library_nodes())
+    assert before == ["Mul", "Mul", "ReduceSum"]
+    assert fusion.optimize_backward(g.sdfg)["mul_reductions"] == 1
+    after = {n.schema.name: n for n in g.sdfg.states()[1].library_nodes()}
+    assert sorted(after) == ["Mul", "MulReduceSum"]
+    assert list(after["MulReduceSum"].axes) == [2, 3] and after["MulReduceSum"].keepdims == 1
+    assert not any(name.endswith("_full_B") for name in g.sdfg.arrays)      # the product array was dropped
 
 
 def test_pow_backward_needs_a_constant_exponent():
