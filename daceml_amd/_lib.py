@@ -100,6 +100,8 @@ SIGNATURES = {
     "dmlhip_reduce_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "dmlhip_reduce_f16": (c_int, [c_int, _P, _P, c_int, c_int64, c_int64, c_int64, _P, c_size_t, _P]),
     "dmlhip_reduce_f32": (c_int, [c_int, _P, _P, c_int, c_int64, c_int64, c_int64, _P, c_size_t, _P]),
+    "dmlhip_row_affine_f16": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, _P]),
+    "dmlhip_row_affine_f32": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, _P]),
     "dmlhip_row_dot_f16": (c_int, [_P, _P, _P, c_int64, c_int64, _P]),
     "dmlhip_row_dot_f32": (c_int, [_P, _P, _P, c_int64, c_int64, _P]),
     "dmlhip_transpose_f16": (c_int, [_P, _P, c_int, _I64P, _I64P, _P]),

@@ -94,6 +94,50 @@ __global__ __launch_bounds__(kEwBlock) void binary_vec_kernel(const T* __restric
     }
 }
 
+// y[r, j] = a[r, j] * s[r] + t[r] * scale[0]: a dense tensor times one factor per row plus one (scaled) value per row
+// expanded over the row — the two gradient contributions that meet at the input of a squeeze-excite block (through
+// the gate multiplication and through the average pool), without their two intermediate tensors and the Sum pass.
+template <typename T>
+__global__ __launch_bounds__(kEwBlock) void row_affine_kernel(const T* __restrict__ a, const T* __restrict__ s,
+                                                              const T* __restrict__ t, const T* __restrict__ scale,
+                                                              T* __restrict__ y, int64_t rows, int64_t cols, int vec) {
+    using V = typename VecOf<T>::type;
+    constexpr int VN = VecOf<T>::n;
+    const float k = scale ? to_f32(scale[0]) : 1.0f;
+    const int64_t n = rows * cols;
+    const int64_t stride = (int64_t)gridDim.x * kEwBlock;
+    if (vec) {   // whole vectors inside one row, n < 2^32
+        const int64_t nvec = n / VN;
+        for (int64_t i = (int64_t)blockIdx.x * kEwBlock + threadIdx.x; i < nvec; i += stride) {
+            const uint32_t row = (uint32_t)(i * VN) / (uint32_t)cols;
+            const float sv = to_f32(s[row]), tv = to_f32(t[row]) * k;
+            V av = reinterpret_cast<const V*>(a)[i], yv;
+#pragma unroll
+            for (int e = 0; e < VN; ++e) yv[e] = from_f32<T>(to_f32(av[e]) * sv + tv);
+            reinterpret_cast<V*>(y)[i] = yv;
+        }
+    } else {
+        for (int64_t i = (int64_t)blockIdx.x * kEwBlock + threadIdx.x; i < n; i += stride) {
+            const int64_t row = i / cols;
+            y[i] = from_f32<T>(to_f32(a[i]) * to_f32(s[row]) + to_f32(t[row]) * k);
+        }
+    }
+}
+
+template <typename T>
+int row_affine_impl(const void* a, const void* s, const void* t, const void* scale, void* y, int64_t rows, int64_t cols,
+                    void* stream) {
+    DML_REQUIRE(rows >= 0 && cols >= 0, DMLHIP_ERR_SHAPE, "row_affine: negative extent");
+    DML_REQUIRE(cols == 0 || rows <= (INT64_MAX / 16) / cols, DMLHIP_ERR_SHAPE, "row_affine: size overflows");
+    const int64_t n = rows * cols;
+    if (n == 0) return 0;
+    DML_REQUIRE(a && s && t && y, DMLHIP_ERR_NULL, "row_affine: NULL tensor pointer");
+    const int vec = aligned16(a) && aligned16(y) && cols % VecOf<T>::n == 0 && n < (1LL << 32);
+    hipLaunchKernelGGL((row_affine_kernel<T>), ew_grid(ceil_div(n, vec ? VecOf<T>::n : 1)), kEwBlock, 0, (hipStream_t)stream,
+                       (const T*)a, (const T*)s, (const T*)t, (const T*)scale, (T*)y, rows, cols, vec);
+    return launch_status("row_affine");
+}
+
 struct BcastDims {
     int ndim;
     int64_t shape[DMLHIP_MAX_DIMS];
@@ -413,6 +457,14 @@ int dmlhip_bias_gelu_f16(const void* x, const void* bias, void* y, void* pre_out
 int dmlhip_bias_gelu_f32(const void* x, const void* bias, void* y, void* pre_out, int64_t rows, int64_t cols,
                          void* stream) {
     return bias_gelu_impl<float>(x, bias, y, pre_out, rows, cols, stream);
+}
+int dmlhip_row_affine_f16(const void* a, const void* s, const void* t, const void* scale, void* y, int64_t rows,
+                          int64_t cols, void* stream) {
+    return row_affine_impl<_Float16>(a, s, t, scale, y, rows, cols, stream);
+}
+int dmlhip_row_affine_f32(const void* a, const void* s, const void* t, const void* scale, void* y, int64_t rows,
+                          int64_t cols, void* stream) {
+    return row_affine_impl<float>(a, s, t, scale, y, rows, cols, stream);
 }
 int dmlhip_cast(int src_dtype, int dst_dtype, const void* x, void* y, int64_t n, void* stream) {
     DML_REQUIRE((src_dtype == DMLHIP_F16 || src_dtype == DMLHIP_F32) &&

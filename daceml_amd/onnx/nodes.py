@@ -153,6 +153,9 @@ SCHEMAS = [
     # reduced = ReduceSum(Mul(A, B), axes) with A and B of one shape and `axes` the trailing axes: the product is not
     # written (the gradient of a broadcast factor)
     _schema("MulReduceSum", "A B", "reduced", since=1, axes=REQUIRED, keepdims=1),
+    # Y = A * S + T * Scale with S and T holding one value per row of A (A's shape with trailing 1s) and Scale one
+    # element: Sum(Mul(A, S), ScaledExpand(T, Scale)) in one pass
+    _schema("RowAffine", "A S T Scale?", "Y", since=1),
     # backward nodes emitted by the "hip" BackwardImplementations (names follow the ONNX Runtime
     # training contrib ops)
     _schema("SoftmaxGrad", "dY Y", "dX", since=1, axis=-1),

@@ -731,6 +731,47 @@ def _make_reduce(op_name: str, code: int, doc: str):
     return op_implementation(op=op_name, name=IMPL)(_Reduce)
 
 
+def _row_split(full, per_row):
+    """(rows, cols) when `per_row` is `full` with its trailing axes collapsed to 1, else None."""
+    full, per_row = tuple(full), tuple(per_row)
+    if len(full) != len(per_row):
+        return None
+    k = len(full)
+    while k > 0 and per_row[k - 1] == 1:
+        k -= 1
+    if per_row[:k] != full[:k]:
+        return None
+    return _prod(full[:k]), _prod(full[k:])
+
+
+@op_implementation(op="RowAffine", name=IMPL)
+class HipRowAffine(ONNXForward):
+    """Sum (pure_implementations.py:584-646) of Mul(A, per-row S) (:86-88) and a per-row T expanded over the rows and
+    scaled (ReverseReduce, autodiff/implementations/dace_nodes.py:13-105) in one pass over A."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            a, s_, t, y = ins["A"], ins["S"], ins["T"], outs["Y"]
+            if not (_float_ok(a, s_, t, y) and a.dtype == s_.dtype == t.dtype == y.dtype and _dense(a, s_, t, y)):
+                return False
+            if "Scale" in ins and not (ins["Scale"].total_size == 1 and ins["Scale"].dtype == a.dtype):
+                return False
+            split = _row_split(a.shape, s_.shape)
+            return split is not None and split == _row_split(a.shape, t.shape) and tuple(y.shape) == tuple(a.shape)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        ins, outs = _descs(node, state, sdfg)
+        a = ins["A"]
+        rows, cols = _row_split(a.shape, ins["S"].shape)
+        call = HipCall("dmlhip_row_affine_" + _SFX[a.dtype], [Ptr("A"), Ptr("S"), Ptr("T"), _opt(node, state, "Scale"),
+                                                             Ptr("Y"), I64(rows), I64(cols), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(a), kind="elementwise")
+
+
 @op_implementation(op="MulReduceSum", name=IMPL)
 class HipMulReduceSum(ONNXForward):
     """Mul (pure_implementations.py:86-88) read only by ReduceSum over the trailing axes (:294-296) as one row-wise dot

@@ -1125,11 +1125,69 @@ def fuse_mul_reduce(sdfg: SDFG) -> int:
     return count
 
 
+def _per_row_of(full, per_row) -> bool:
+    """`per_row` is `full` with a (non-empty) run of trailing axes collapsed to 1."""
+    full, per_row = tuple(full), tuple(per_row)
+    if len(full) != len(per_row) or full == per_row:
+        return False
+    k = len(full)
+    while k > 0 and per_row[k - 1] == 1:
+        k -= 1
+    return per_row[:k] == full[:k]
+
+
+def fuse_row_affine(sdfg: SDFG) -> int:
+    """A gradient-accumulation Sum of exactly Mul(A, S) and ScaledExpand(T, Scale), with S and T holding one value per
+    row of A, becomes one RowAffine node: the two summands are never written. This is the meeting point of the two
+    gradient paths of a squeeze-excite block (through the gate multiplication and through the average pool)."""
+    count = 0
+    for state in sdfg.states():
+        for add in [n for n in state.nodes() if _is_op(n, "Sum")]:
+            ins = [e.data.data for e in state.in_edges(add)]
+            if len(ins) != 2:
+                continue
+            prods = [_producer(state, a) for a in ins]
+            if any(p is None for p in prods) or not all(_internal(sdfg, state, a) for a in ins):
+                continue
+            kinds = [p[0].schema.name if isinstance(p[0], ONNXOp) else "" for p in prods]
+            if sorted(kinds) != ["Mul", "ScaledExpand"]:
+                continue
+            mul = prods[kinds.index("Mul")][0]
+            exp = prods[kinds.index("ScaledExpand")][0]
+            out = _out_array(state, add, "sum")
+            oshape = tuple(sdfg.arrays[out].shape)
+            ma, mb = _in_array(state, mul, "A"), _in_array(state, mul, "B")
+            if tuple(sdfg.arrays[ma].shape) == oshape and _per_row_of(oshape, sdfg.arrays[mb].shape):
+                dense, factor = ma, mb
+            elif tuple(sdfg.arrays[mb].shape) == oshape and _per_row_of(oshape, sdfg.arrays[ma].shape):
+                dense, factor = mb, ma
+            else:
+                continue
+            t = _in_array(state, exp, "X")
+            kept = tuple(exp.x_shape) if exp.x_shape is not None else tuple(sdfg.arrays[t].shape)
+            if kept != tuple(sdfg.arrays[factor].shape) or not all(
+                    sdfg.arrays[x].is_contiguous() for x in (dense, factor, t)):
+                continue
+            if len({sdfg.arrays[x].dtype for x in (dense, factor, t, out)}) != 1:
+                continue
+            new_ins = {"A": dense, "S": factor, "T": t, "Scale": _in_array(state, exp, "Scale")}
+            label = add.label
+            _remove_node(state, add)
+            _remove_node(state, mul)
+            _remove_node(state, exp)
+            _add_node(sdfg, state, "RowAffine", label, new_ins, {"Y": out})
+            count += 1
+    if count:
+        _drop_unused_arrays(sdfg)
+    return count
+
+
 def optimize_backward(sdfg: SDFG) -> Dict[str, int]:
     """Rewrites for the state(s) autodiff added — what a ``post_autodiff_hooks`` entry of the reference's module
     wrapper would run (daceml/torch/module.py:46-365)."""
     stats = {"bias_gradients": fuse_bias_gradients(sdfg)}
     stats["mul_reductions"] = fuse_mul_reduce(sdfg)    # before fuse_reductions: these sums stop being plain ReduceSums
+    stats["row_affine"] = fuse_row_affine(sdfg)
     stats["reductions"] = fuse_reductions(sdfg)
     stats["einsum_sums"] = fuse_einsum_sums(sdfg)      # before grouping: a summed group needs no separate outputs
     stats["grouped_einsums"] = group_einsums(sdfg)

@@ -130,6 +130,15 @@ int dmlhip_unary_backward_f32(int op, const void* x, const void* dy, void* dx, i
 int dmlhip_sum_f16(const void* const* inputs, int n_inputs, void* out, int64_t n, void* stream);
 int dmlhip_sum_f32(const void* const* inputs, int n_inputs, void* out, int64_t n, void* stream);
 
+/* y[r, j] = a[r, j] * s[r] + t[r] * scale[0] over dense [rows, cols] (scale may be NULL = 1): ONNXSum
+ * (pure_implementations.py:584-646) of an ONNXMul with a per-row factor (:86-88) and a per-row value broadcast back over
+ * the row (ReverseReduce, autodiff/implementations/dace_nodes.py:13-105) — the gradient accumulation at the input of a
+ * squeeze-excite block — in one pass. */
+int dmlhip_row_affine_f16(const void* a, const void* s, const void* t, const void* scale, void* y, int64_t rows,
+                          int64_t cols, void* stream);
+int dmlhip_row_affine_f32(const void* a, const void* s, const void* t, const void* scale, void* y, int64_t rows,
+                          int64_t cols, void* stream);
+
 /* Add(bias[cols]) followed by the GELU chain, fused; bias may be NULL.
  * pre_out (nullable) receives x+bias, which the backward needs. */
 int dmlhip_bias_gelu_f16(const void* x, const void* bias, void* y, void* pre_out, int64_t rows,

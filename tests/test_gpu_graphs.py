@@ -255,6 +255,37 @@ def test_unfused_layernorm_and_gelu_chains_backward(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_squeeze_excite_gradient_meeting_point(dtype):
+    """y = x * mean_hw(x): the gradient of x arrives through the multiplication and through the average pool. After
+    optimize_backward the backward state is two kernels — the gate's gradient as a row-wise dot product and the sum of
+    both paths as one RowAffine — checked against autograd."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.transformation import fusion
+    g = graphs.GraphBuilder("se_meeting_point", dtype)
+    x = g.input("x", (3, 5, 6, 8))
+    gate = g.node("GlobalAveragePool", {"X": x}, {"Y": (3, 5, 1, 1)}, label="pool")["Y"]
+    g.output(g.node("Mul", {"A": x, "B": gate}, {"C": (3, 5, 6, 8)}, label="scale")["C"], "y")
+    assert add_backward_pass(g.sdfg, g.state, ["y"], ["x"]) == {"x": "gradient_x"}
+    stats = fusion.optimize_backward(g.sdfg)
+    assert stats["mul_reductions"] == 1 and stats["row_affine"] == 1
+    assert sorted(n.schema.name for n in g.sdfg.states()[1].library_nodes()) == ["MulReduceSum", "RowAffine"]
+    prog = _compile(g.sdfg)
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    xv = rng(31).standard_normal((3, 5, 6, 8)).astype(npdt)
+    dyv = rng(32).standard_normal((3, 5, 6, 8)).astype(npdt)
+    out = {"y": torch.empty((3, 5, 6, 8), dtype=dtype, device="cuda"),
+           "gradient_x": torch.empty((3, 5, 6, 8), dtype=dtype, device="cuda")}
+    prog(x=dev(xv), gradient_y=dev(dyv), **out)
+    tx = torch.tensor(xv.astype(np.float64), requires_grad=True)
+    ty = tx * tx.mean((2, 3), keepdim=True)
+    ty.backward(torch.tensor(dyv.astype(np.float64)))
+    kw = dict(rtol=1e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    assert_close(host(out["y"]), ty.detach().numpy(), dtype, "forward", **kw)
+    assert_close(host(out["gradient_x"]), tx.grad.numpy(), dtype, "gradient of x", **kw)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_reduce_and_transpose_backward(dtype):
     """ReduceMean (keepdims 1), ReduceSum (keepdims 0) and Transpose reversed with ScaledExpand / Transpose nodes,
     against autograd: y = transpose(x - mean(x, -1, keepdim)) * sum(x, (0, 1))."""

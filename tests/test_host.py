@@ -430,8 +430,8 @@ def test_attention_fusion_roles_and_graph():
     assert ins == {"Q", "K", "V", "O", "LogSumExp", "dO"}
     # the six bias gradients become one node; nothing else in the state changes
     n_before = len(sdfg.states()[1].library_nodes())
-    assert fusion.optimize_backward(sdfg) == {"bias_gradients": 6, "mul_reductions": 0, "reductions": 0, "einsum_sums": 6,
-                                             "grouped_einsums": 5}
+    assert fusion.optimize_backward(sdfg) == {"bias_gradients": 6, "mul_reductions": 0, "row_affine": 0, "reductions": 0,
+                                             "einsum_sums": 6, "grouped_einsums": 5}
     bnodes = sdfg.states()[1].library_nodes()
     # six bias-gradient reductions (now InputSum outputs of the weight-gradient contractions), two gradient sums and five
     # contractions fewer (q/k/v input gradients: 3 -> 1 EinsumSum that also adds the residual path; o/q/k/v weight
