@@ -37,31 +37,59 @@ def build_program(device):
     from daceml_amd.autodiff import add_backward_pass
     from daceml_amd.runtime import CompiledSDFG
     from daceml_amd.transformation import fusion
-    from oracle import bert_layer as OB  # parameter names / init only
 
     sdfg = graphs.bert_encoder_layer(B, S, H, HEADS, FFN, torch.float16, eps=1e-12)
     fusion.auto_optimize(sdfg, training=True)
-    add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + OB.PARAM_NAMES,
-                      grad_dtypes={n: torch.float32 for n in OB.PARAM_NAMES})
+    add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + graphs.BERT_PARAM_NAMES,
+                      grad_dtypes={n: torch.float32 for n in graphs.BERT_PARAM_NAMES})
     fusion.optimize_backward(sdfg)
-    return CompiledSDFG(sdfg, device=device), OB
+    return CompiledSDFG(sdfg, device=device)
 
 
-def synthetic_inputs(OB, device):
+def synthetic_inputs(device):
     """Seeded synthetic data of the config's shape: x, dy ~ N(0,1); weights N(0, 0.02), biases 0, LN 1/0."""
     import numpy as np
     import torch
-    p = OB.init_params(H, FFN, 1234 + 4, np.float32)
+    from daceml_amd import graphs
+    p = graphs.bert_init_params(H, FFN, 1234 + 4)
     rng = np.random.default_rng(1234 + 5)
     x = rng.standard_normal((B, S, H)).astype(np.float16)
     dy = rng.standard_normal((B, S, H)).astype(np.float16)
     args = {"x": torch.from_numpy(x).to(device), "gradient_y": torch.from_numpy(dy).to(device),
             "y": torch.empty((B, S, H), dtype=torch.float16, device=device),
             "gradient_x": torch.empty((B, S, H), dtype=torch.float16, device=device)}
-    for n in OB.PARAM_NAMES:
+    for n in graphs.BERT_PARAM_NAMES:
         args[n] = torch.from_numpy(p[n].astype(np.float16)).to(device)
         args["gradient_" + n] = torch.empty(p[n].shape, dtype=torch.float32, device=device)
     return args, x, dy, p
+
+
+def check_against_oracle(args, x, dy, p):
+    """Untimed: the outputs of one step at the bench's own shape against the fp64 CPU oracle (checker only), at the
+    tolerance the fp16 path is held to (rtol 2e-2 / atol 1e-2; fp32 master gradients: atol max(1e-2, 2 % of their scale))."""
+    import numpy as np
+    from oracle import bert_layer as OB
+    x64 = x.astype(np.float64)
+    p64 = {k: v.astype(np.float16).astype(np.float64) for k, v in p.items()}
+    y, saved = OB.forward(x64, p64, HEADS, eps=1e-12, keep=True)
+    g = OB.backward(x64, p64, HEADS, dy.astype(np.float64), saved, eps=1e-12)
+    del saved
+    worst, ok, n_checked = {}, True, 0
+    for name, want, scaled in [("y", y, False), ("gradient_x", g["x"], False)] + \
+            [("gradient_" + n, g[n], True) for n in OB.PARAM_NAMES]:
+        got = args[name].float().cpu().numpy().astype(np.float64)
+        atol = max(1e-2, 2e-2 * float(np.abs(want).max())) if scaled else 1e-2
+        err = np.abs(got - want)
+        excess = err - (atol + 2e-2 * np.abs(want))
+        worst[name] = float(err.max())
+        ok = ok and bool((excess <= 0).all()) and bool(np.isfinite(got).all())
+        n_checked += got.size
+    return {"checked": ok, "max_abs_error": {"y": worst["y"], "gradient_x": worst["gradient_x"],
+                                             "parameter_gradients": max(v for k, v in worst.items()
+                                                                        if k not in ("y", "gradient_x"))},
+            "elements_checked": n_checked,
+            "check": "y, gradient_x and all 16 parameter gradients of the first (untimed) step vs the fp64 oracle, "
+                     "rtol 2e-2 / atol 1e-2 (parameter gradients: atol max(1e-2, 2e-2 x their max))"}
 
 
 def kernel_breakdown(prog, reps=10):
@@ -76,10 +104,11 @@ def kernel_breakdown(prog, reps=10):
     return [(l, ms / reps) for l, ms in acc]
 
 
-def cpu_baseline(OB, x, dy, p, budget_s=25.0):
+def cpu_baseline(x, dy, p, budget_s=25.0):
     """The oracle's forward+backward (fp32 NumPy, BLAS contractions) on the full workload, repeated within
     a time budget."""
     import numpy as np
+    from oracle import bert_layer as OB
     x32 = x.astype(np.float32)
     dy32 = dy.astype(np.float32)
     p32 = {k: v.astype(np.float32) for k, v in p.items()}
@@ -98,6 +127,8 @@ def cpu_baseline(OB, x, dy, p, budget_s=25.0):
     except Exception:
         cores = os.cpu_count() or 1
     return {"value": round(min(times) * 1e3, 2), "unit": "ms/iter", "cores": int(cores), "kind": "port",
+            "cores_note": "threads of the BLAS behind np.matmul (the contractions); every other NumPy statement "
+                          "(LayerNorm, GELU, softmax pieces) runs on one core",
             "sample": "full workload (B=8, S=512), %d fwd+bwd repetitions of the NumPy restatement of the pure "
                       "expansions in fp32, best of them" % len(times)}
 
@@ -126,11 +157,10 @@ def secondary_workload(name, device, steps, warmup, verbose):
     rng = np.random.default_rng(1234)
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
     if name == "bert_fwd":
-        from oracle import bert_layer as OB
         sdfg = graphs.bert_encoder_layer(B, S, H, HEADS, FFN, torch.float16, eps=1e-12)
         fusion.auto_optimize(sdfg)
-        p = OB.init_params(H, FFN, 1234 + 2, np.float32)
-        args = {n: dev(p[n].astype(np.float16)) for n in OB.PARAM_NAMES}
+        p = graphs.bert_init_params(H, FFN, 1234 + 2)
+        args = {n: dev(p[n].astype(np.float16)) for n in graphs.BERT_PARAM_NAMES}
         args["x"] = dev(rng.standard_normal((B, S, H)).astype(np.float16))
         args["y"] = torch.empty((B, S, H), dtype=torch.float16, device=device)
         what, dtype = "BERT-large encoder layer forward, B=8 S=512, fp16 (BASELINE.json configs[2])", "f16"
@@ -298,6 +328,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true", help="skip the untimed comparison with the CPU oracle")
     ap.add_argument("--verbose", action="store_true", help="per-launch table on stderr")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region, launch a plain 128 MiB -> 128 MiB copy kernel three times: under "
@@ -317,17 +348,29 @@ def main():
     if a.workload != "bert_fwd_bwd":
         return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose)
 
-    prog, OB = build_program(device)
-    args, x, dy, p = synthetic_inputs(OB, device)
+    prog = build_program(device)
+    args, x, dy, p = synthetic_inputs(device)
     prog(**args)  # binds pointers, first run
+    torch.cuda.synchronize()
+    checked = None if a.no_check else check_against_oracle(args, x, dy, p)
     for _ in range(a.warmup):
         prog.launch()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(a.steps):
+    for i in range(a.steps):
+        marks[i].record()
         prog.launch()
+    marks[a.steps].record()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / a.steps * 1e3
+    # per-step statistics as the reference's profiler reports them (event_profiler.py:87-143): HIP events between
+    # the steps of the timed region
+    import statistics
+    per_step = [marks[i].elapsed_time(marks[i + 1]) for i in range(a.steps)]
+    step_stats = {"min": round(min(per_step), 4), "median": round(statistics.median(per_step), 4),
+                  "mean": round(statistics.fmean(per_step), 4), "max": round(max(per_step), 4),
+                  "stdev": round(statistics.pstdev(per_step), 4)}
 
     if a.calibrate_copy:
         from daceml_amd import _lib as L, kernels as K
@@ -381,9 +424,12 @@ def main():
         "attention_nodes": attn,
         "hbm_nodes": hbm,
         "sum_of_kernel_ms": round(sum(t for _, t in rows), 4),
+        "step_ms": step_stats,
     }
+    if checked is not None:
+        out.update(checked)
     if not a.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(OB, x, dy, p)
+        out["cpu_baseline"] = cpu_baseline(x, dy, p)
     print(json.dumps(out))
 
 

@@ -111,7 +111,24 @@ class BackwardPassGenerator:
                 if r in self._active_arrays and self._differentiable_input(n, e.dst_conn):
                     self._expected[r] = self._expected.get(r, 0) + 1
 
-        ready: Dict[str, str] = {a: self.array_grad_map[a] for a in self.given_gradients}
+        # an output that other nodes of the subgraph also read: the caller's gradient is ONE contribution; the
+        # consumers' contributions are summed with it into a transient of its own (never into the caller's
+        # buffer), and the producer's reverse node waits for that sum
+        ready: Dict[str, str] = {}
+        for name in self.given_gradients:
+            r = _root(sdfg, name)
+            if self._expected.get(r, 0) == 0:
+                ready[r] = self.array_grad_map[name]
+                continue
+            if r != name:
+                raise AutoDiffException("output %r is a view of %r, which other nodes read" % (name, r))
+            self._expected[r] += 1
+            self._contrib[r] = [self.array_grad_map[name]]
+            total, i = "gradient_%s_total" % name, 0
+            while total in sdfg.arrays:
+                i += 1
+                total = "gradient_%s_total_%d" % (name, i)
+            self.array_grad_map[r] = total
         for n in reversed(nodes):
             self._reverse_node(n, ready)
         result = {}

@@ -130,6 +130,27 @@ BERT_PARAMS = [
 ]
 
 
+#: the arrays `bert_encoder_layer` takes besides ``x``
+BERT_PARAM_NAMES = [short + suffix for _, short in BERT_PARAMS for suffix in ("_w", "_b")] + \
+    ["ln1_g", "ln1_b", "ln2_g", "ln2_b"]
+
+
+def bert_init_params(hidden: int, ffn: int, seed: int, bias_std: float = 0.0):
+    """Synthetic parameters of one layer as fp32 NumPy arrays: weights N(0, 0.02), biases zero (or N(0, bias_std)),
+    LayerNorm gamma 1 / beta 0. Deterministic in `seed`."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    p = {}
+    for _, short in BERT_PARAMS:
+        o, i = {"ffn1": (ffn, hidden), "ffn2": (hidden, ffn)}.get(short, (hidden, hidden))
+        p[short + "_w"] = (rng.standard_normal((o, i)) * 0.02).astype(np.float32)
+        p[short + "_b"] = (rng.standard_normal(o) * bias_std).astype(np.float32)
+    for ln in ("ln1", "ln2"):
+        p[ln + "_g"] = np.ones(hidden, np.float32)
+        p[ln + "_b"] = np.zeros(hidden, np.float32)
+    return p
+
+
 def bert_encoder_layer(batch: int, seq: int, hidden: int, heads: int, ffn: int, dtype=torch.float16,
                        eps: float = 1e-12) -> SDFG:
     """One post-LN BERT encoder layer (HuggingFace ``BertLayer``; no mask, no dropout), decomposed as the

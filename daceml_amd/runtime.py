@@ -221,6 +221,41 @@ class CompiledSDFG:
         alive until the launches that use them have been enqueued."""
         self._bind_arguments(tensors, partial=True)
 
+    def forwarded_transients(self, forward_states: Sequence[str], backward_states: Sequence[str]) -> List[str]:
+        """Transient buffers that the forward states write and the backward states touch: the values a pending
+        backward call depends on (what the reference's dispatcher turns into extra forward outputs and saves on the
+        autograd context, daceml/autodiff/torch.py:56-104, ctypes_module.py:150-156)."""
+        def root(name):
+            while self.sdfg.arrays[name].view_of is not None:
+                name = self.sdfg.arrays[name].view_of
+            return name
+
+        written, touched = set(), set()
+        for state in self.sdfg.states():
+            for e in state.edges():
+                r = root(e.data.data)
+                if state.label in forward_states and isinstance(e.dst, AccessNode):
+                    written.add(r)
+                if state.label in backward_states:
+                    touched.add(r)
+        return [n for n in self.buffers if n in written and n in touched and self.sdfg.arrays[n].transient and
+                n not in self.sdfg.constants]
+
+    def rebind_transients(self, tensors: Dict[str, torch.Tensor], release: bool = False):
+        """Point transient arrays at caller-provided buffers (same shape and dtype, dense). With ``release`` the
+        buffers this object allocated for them are dropped."""
+        for name, t in tensors.items():
+            desc = self.sdfg.arrays[name]
+            if not desc.transient or desc.view_of is not None or name in self.sdfg.constants:
+                raise ValueError("%r is not a transient buffer of this SDFG" % name)
+            if t.dtype != desc.dtype or tuple(t.shape) != desc.shape or not t.is_contiguous() or t.device != self.device:
+                raise ValueError("buffer for %r must be a dense %s %s tensor on %s" % (name, desc.dtype, desc.shape,
+                                                                                        self.device))
+            self._ptr[name].value = t.data_ptr()
+            if release:
+                self.buffers[name] = t
+        self._refresh()
+
     def launch(self, states: Optional[Sequence[str]] = None):
         """Enqueue every kernel (of the named states) on the current stream, with the pointers of the
         last binding."""

@@ -9,10 +9,10 @@ backward-state rewrites), expanded and bound to the kernels (``post_compile_hook
 enqueues the forward state on the current stream, and in ``backward`` enqueues the backward state and returns
 ``None`` for inputs that need no gradient.
 
-One difference in structure: forward and backward live in ONE SDFG (two states) that shares its transients, so
-``post_autodiff_hooks`` receive that SDFG for both arguments, and values the backward state reads are kept in
-SDFG-owned buffers instead of being saved on the autograd context: a module instance supports one
-forward -> backward in flight at a time (a second forward overwrites what the first one's backward would read).
+One difference in structure: forward and backward live in ONE SDFG (two states). ``post_autodiff_hooks`` receive
+that SDFG for both arguments. What a backward call reads - the tensors the forward call was bound to, the outputs,
+and the SDFG buffers the forward state fills for the backward state - is saved on the autograd context per call
+(``ctx.save_for_backward``), so inputs may be dropped or overwritten and several forward calls may be pending.
 """
 import collections
 import logging
@@ -192,7 +192,14 @@ class DaceModule(nn.Module):
         grad_of_input = [grads.get(a) for a in in_arrays]
         n_tensor = len(tensor_inputs)
 
-        def run_forward(tensors):
+        # what a backward call reads besides the gradients it is given: the tensors the forward call was bound to
+        # and the SDFG's own buffers that the forward state fills for the backward state. Both are saved on the
+        # autograd context (ctypes_module.py:150-170) - the former keep the memory behind the bound pointers alive,
+        # the latter get fresh memory per forward call, so that any number of forward calls may be pending
+        forwarded = compiled.forwarded_transients(forward_states, backward_states) if self.backward else []
+        self.forwarded_transients = list(forwarded)
+
+        def run_forward(tensors, keep=False):
             call = {}
             for name, t in zip(in_arrays, tensors):
                 if name in arglist:
@@ -204,19 +211,31 @@ class DaceModule(nn.Module):
                 call[name] = t
                 outs.append(t)
             compiled.bind(call)
+            saved = {}
+            if keep:
+                for name in forwarded:
+                    d = sdfg.arrays[name]
+                    saved[name] = torch.empty(d.shape, dtype=d.dtype, device=device)
+                compiled.rebind_transients(saved, release=True)
             compiled.launch(forward_states)
-            return tuple(outs)
+            return tuple(outs), call, saved
 
         class DifferentiableFunction(torch.autograd.Function):
             @staticmethod
             def forward(ctx, *tensors):
-                outs = run_forward(tensors)
+                outs, call, saved = run_forward(tensors, keep=True)
+                ctx.daceml_bound_names = list(call)
+                ctx.daceml_saved_names = list(saved)
+                ctx.save_for_backward(*call.values(), *saved.values())
                 ctx.mark_non_differentiable(*[o for o in outs if not o.dtype.is_floating_point])
                 return outs[0] if len(outs) == 1 else outs
 
             @staticmethod
             def backward(ctx, *grad_outputs):
-                call = {}
+                kept = ctx.saved_tensors
+                nb = len(ctx.daceml_bound_names)
+                call = dict(zip(ctx.daceml_bound_names, kept[:nb]))
+                compiled.rebind_transients(dict(zip(ctx.daceml_saved_names, kept[nb:])))
                 for name, g in zip(out_arrays, grad_outputs):
                     gname = "gradient_" + name
                     if gname not in arglist:
@@ -243,7 +262,7 @@ class DaceModule(nn.Module):
             tensors = tuple(args) + tuple(params[n] for n in param_inputs)
             if self.backward:
                 return DifferentiableFunction.apply(*tensors)
-            outs = run_forward(tensors)
+            outs = run_forward(tensors)[0]
             return outs[0] if len(outs) == 1 else outs
 
         return function

@@ -621,3 +621,32 @@ def test_backward_pass_structure():
     # everything in both states expands with the hip implementations
     from daceml_amd.runtime import expand_onnx_nodes
     assert expand_onnx_nodes(sdfg) == len(names) + 11
+
+
+def test_an_output_that_another_node_reads_keeps_its_incoming_gradient():
+    """y0 = f(x), y1 = g(y0), both outputs: the caller's gradient of y0 is one contribution and g's reverse node
+    the other; they are summed into a transient (the caller's buffer is only read), and f's reverse node reads
+    that sum (accumulation rule of backward_pass_generator.py:715-752)."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    g = graphs.GraphBuilder("chain", torch.float32)
+    x = g.input("x", (4, 8))
+    t = g.node("Sigmoid", {"X": x}, {"Y": (4, 8)}, label="t")["Y"]
+    s = g.node("Sigmoid", {"X": t}, {"Y": (4, 8)}, label="s")["Y"]
+    g.output(t, "y0")
+    g.output(s, "y1")
+    grads = add_backward_pass(g.sdfg, g.state, ["y0", "y1"], ["x"])
+    assert grads == {"x": "gradient_x"}
+    bst = g.sdfg.states()[1]
+    sums = [n for n in bst.library_nodes() if n.schema.name == "Sum"]
+    assert len(sums) == 1
+    summed = sorted(e.data.data for e in bst.in_edges(sums[0]))
+    assert "gradient_y0" in summed and len(summed) == 2
+    total = next(iter(bst.out_edges(sums[0]))).data.data
+    assert total != "gradient_y0" and g.sdfg.arrays[total].transient
+    # nothing writes the buffers the caller handed in
+    written = {e.data.data for n in bst.library_nodes() for e in bst.out_edges(n)}
+    assert not written & {"gradient_y0", "gradient_y1"}
+    # the reverse node of the first Sigmoid reads the sum
+    reads = {e.data.data for n in bst.library_nodes() if n.schema.name == "SigmoidGrad" for e in bst.in_edges(n)}
+    assert total in reads

@@ -496,3 +496,107 @@ def test_mbconv_block_training_through_the_wrapper():
     for (n, p_), (_, pr) in zip(net.named_parameters(), ref.named_parameters()):
         scale = max(float(pr.grad.abs().max()), 1.0)
         assert_close(host(p_.grad), pr.grad.cpu().numpy(), torch.float32, "gradient of " + n, rtol=1e-3, atol=1e-4 * scale)
+
+
+# ----------------------------------------------------------------------------- what a pending backward depends on
+def _small_encoder_reference(net, x64, gy64):
+    ref = copy.deepcopy(net).double()
+    xr = x64.clone().requires_grad_(True)
+    ref(xr).backward(gy64)
+    return xr.grad, {n: p_.grad for n, p_ in ref.named_parameters()}
+
+
+@pytest.mark.gpu
+def test_backward_survives_dropped_and_overwritten_inputs():
+    """The dispatcher saves what backward reads on the autograd context (daceml/torch/dispatchers/ctypes_module.py:
+    150-170): a non-contiguous input (whose dense copy nobody else owns) and an input that the caller drops and
+    whose memory is reused before ``backward()`` still give autograd's gradients."""
+    torch.manual_seed(11)
+    net = SmallEncoder().cuda()
+    w = DaceModule(copy.deepcopy(net), backward=True)
+    base = torch.randn(8, 3, 5, device="cuda")           # [feature, batch, time]: the permuted view is not dense
+    gy = torch.randn(3, 5, 8, device="cuda")
+    want_dx, want = _small_encoder_reference(net, base.permute(1, 2, 0).double(), gy.double())
+
+    leaf = base.clone().requires_grad_(True)
+    x = leaf.permute(1, 2, 0)
+    assert not x.is_contiguous()
+    y = w(x)
+    del x
+    # churn the caching allocator: same-sized blocks are handed out again and overwritten
+    junk = [torch.full((3, 5, 8), float("nan"), device="cuda") for _ in range(64)]
+    junk += [torch.full((3, 5, 16), float("nan"), device="cuda") for _ in range(64)]
+    y.backward(gy)
+    del junk
+    assert_close(host(leaf.grad.permute(1, 2, 0)), want_dx.cpu().numpy(), torch.float32, "dx", rtol=1e-4, atol=1e-5)
+    for n, p_ in w.model.named_parameters():
+        assert_close(host(p_.grad), want[n].cpu().numpy(), torch.float32, "gradient of " + n, rtol=1e-4, atol=1e-5)
+
+    # an activation of an upstream layer that only the graph owns: w(embedding(ids))
+    w2 = DaceModule(copy.deepcopy(net), backward=True)
+    emb = nn.Embedding(10, 8).cuda()
+    ids = torch.randint(0, 10, (3, 5), device="cuda")
+    y = w2(emb(ids))
+    junk = [torch.full((3, 5, 8), float("nan"), device="cuda") for _ in range(64)]
+    y.backward(gy)
+    del junk
+    _, want2 = _small_encoder_reference(net, emb(ids).detach().double(), gy.double())
+    for n, p_ in w2.model.named_parameters():
+        assert_close(host(p_.grad), want2[n].cpu().numpy(), torch.float32, "gradient of " + n + " (embedding input)",
+                     rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_two_forward_calls_pending_before_their_backward_calls():
+    """Each forward call keeps its own copies of the buffers its backward call reads, so backward calls may come
+    in any order after several forward calls (as with the reference's dispatcher)."""
+    torch.manual_seed(12)
+    net = SmallEncoder().cuda()
+    w = DaceModule(copy.deepcopy(net), backward=True)
+    assert w.function is None
+    xs = [torch.randn(3, 5, 8, device="cuda", requires_grad=True) for _ in range(2)]
+    gys = [torch.randn(3, 5, 8, device="cuda") for _ in range(2)]
+    ys = [w(x) for x in xs]
+    assert w.forwarded_transients, "the backward state reads buffers the forward state fills"
+    for i in (0, 1):                                    # first call's backward after the second call's forward
+        ys[i].backward(gys[i])
+    total = {n: torch.zeros_like(p_, dtype=torch.float64) for n, p_ in net.named_parameters()}
+    for i in (0, 1):
+        dx, grads = _small_encoder_reference(net, xs[i].detach().double(), gys[i].double())
+        assert_close(host(xs[i].grad), dx.cpu().numpy(), torch.float32, "dx of call %d" % i, rtol=1e-4, atol=1e-5)
+        for n in total:
+            total[n] += grads[n]
+    for n, p_ in w.model.named_parameters():
+        assert_close(host(p_.grad), total[n].cpu().numpy(), torch.float32, "accumulated gradient of " + n,
+                     rtol=1e-4, atol=2e-5)
+
+
+class HiddenAndPooled(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc = nn.Linear(16, 16)
+
+    def forward(self, a):
+        h = torch.sigmoid(self.fc(a))
+        return h, torch.tanh(h)
+
+
+@pytest.mark.gpu
+def test_module_returning_an_intermediate_and_a_function_of_it():
+    """An output that another node of the graph also reads receives the caller's gradient PLUS the consumer's."""
+    torch.manual_seed(13)
+    net = HiddenAndPooled().cuda()
+    ref = copy.deepcopy(net).double()
+    w = DaceModule(net, backward=True)
+    a = torch.randn(4, 16, device="cuda", requires_grad=True)
+    ar = a.detach().double().requires_grad_(True)
+    h, t = w(a)
+    hr, tr = ref(ar)
+    g0, g1 = torch.randn_like(h), torch.randn_like(t)
+    keep0 = g0.clone()
+    torch.autograd.backward([h, t], [g0, g1])
+    torch.autograd.backward([hr, tr], [g0.double(), g1.double()])
+    assert torch.equal(g0, keep0), "the caller's gradient buffer is read only"
+    assert_close(host(a.grad), ar.grad.cpu().numpy(), torch.float32, "gradient of the input", rtol=1e-4, atol=1e-5)
+    for (n, p_), (_, pr) in zip(net.named_parameters(), ref.named_parameters()):
+        assert_close(host(p_.grad), pr.grad.cpu().numpy(), torch.float32, "gradient of " + n, rtol=1e-4, atol=1e-5)
