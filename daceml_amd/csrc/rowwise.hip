@@ -4,6 +4,8 @@
 // register budget or are not 16-byte aligned take a workgroup-per-row fallback.
 #include "common.h"
 
+#include <mutex>
+
 namespace dml {
 namespace {
 
@@ -597,6 +599,41 @@ int layernorm_bwd_impl(const void* dy, const void* x, const float* mean, const f
     return launch_status("layernorm_backward(stage 2)");
 }
 
+// ------------------------------------------------------------------ scratch for callers that cannot allocate
+// A fixed-size device array that stands in for the caller's workspace in dmlhip_layernorm_backward_noalloc_f16.
+// One copy per GPU, resident until the process ends. In host code the array's name is only a handle for
+// hipGetSymbolAddress: the device address is looked up once per device and that pointer is what kernels get.
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of the current device's copy of `scratch`.
+int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        set_error("layernorm_backward_noalloc: hipGetDevice failed: %s", hipGetErrorString(e));
+        return (int)e;
+    }
+    DML_REQUIRE(dev >= 0 && dev < kMaxDevices, DMLHIP_ERR_UNSUPPORTED,
+                "layernorm_backward_noalloc: device index %d beyond the %d devices the scratch table holds", dev,
+                kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            set_error("layernorm_backward_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
 }  // namespace
 }  // namespace dml
 
@@ -641,6 +678,22 @@ int dmlhip_layernorm_backward_f32(const void* dy, const void* x, const float* me
                                   int64_t cols, void* workspace, size_t workspace_bytes, void* stream) {
     return layernorm_bwd_impl<float>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, rows, cols, workspace,
                                      workspace_bytes, stream);
+}
+size_t dmlhip_layernorm_backward_noalloc_max_bytes(void) { return kStaticScratchBytes; }
+int dmlhip_layernorm_backward_noalloc_f16(const void* dy, const void* x, const float* mean, const float* rstd,
+                                          const void* gamma, void* dx, float* dgamma, float* dbeta, int64_t rows,
+                                          int64_t cols, void* stream) {
+    if (int e = check_rows("layernorm_backward_noalloc", rows, cols)) return e;
+    const size_t need = dmlhip_layernorm_backward_workspace_bytes(rows, cols);
+    DML_REQUIRE(need <= kStaticScratchBytes, DMLHIP_ERR_WORKSPACE,
+                "layernorm_backward_noalloc: %lld x %lld needs %zu bytes of scratch, the built-in buffer holds %zu; "
+                "use dmlhip_layernorm_backward_f16 with a workspace", (long long)rows, (long long)cols, need,
+                kStaticScratchBytes);
+    void* ws = nullptr;
+    if (int e = static_scratch(&ws)) return e;
+    // every partial row that stage 2 reads is written by stage 1 of the same call: nothing has to start at zero
+    return layernorm_bwd_impl<_Float16>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, rows, cols, ws,
+                                        kStaticScratchBytes, stream);
 }
 
 }  // extern "C"

@@ -95,6 +95,20 @@ int dmlhip_layernorm_backward_f32(const void* dy, const void* x, const float* me
                                   float* dgamma, float* dbeta, int64_t rows, int64_t cols,
                                   void* workspace, size_t workspace_bytes, void* stream);
 
+/* dmlhip_layernorm_backward_f16 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the
+ * reference. Same arguments and results as dmlhip_layernorm_backward_f16 without the workspace: the
+ * per-workgroup partial sums go to a fixed device array inside the library (one copy per GPU, resident
+ * until the process ends) of dmlhip_layernorm_backward_noalloc_max_bytes() = 8 MiB. Shapes whose
+ * dmlhip_layernorm_backward_workspace_bytes(rows, cols) exceeds that are refused with
+ * DMLHIP_ERR_WORKSPACE. The call allocates and frees nothing. Every call on a GPU shares that GPU's
+ * array: calls that overlap on one GPU (different streams or threads) race; calls on one stream do not. */
+size_t dmlhip_layernorm_backward_noalloc_max_bytes(void);
+int dmlhip_layernorm_backward_noalloc_f16(const void* dy, const void* x, const float* mean,
+                                          const float* rstd, const void* gamma, void* dx,
+                                          float* dgamma, float* dbeta, int64_t rows, int64_t cols,
+                                          void* stream);
+
 /* ------------------------------------------------------------------ elementwise
  * Add/Sub/Mul/Div/Pow "pure": pure_implementations.py:39-41,76-93 (NumPy broadcasting).
  * `shape` is the broadcast output shape (ndim <= DMLHIP_MAX_DIMS); a_strides / b_strides are
