@@ -1,6 +1,6 @@
 """Build libdaceml_hip.so (gfx950 code objects + the C ABI) in-tree with hipcc.
 
-Usage: ``python -m daceml_amd.csrc.build [--force]``. The shared library is written next to
+Usage: ``python -m daceml_amd.csrc.build [--incremental]``. The shared library is written next to
 the sources so that it travels with the source tree; nothing is installed.
 """
 import concurrent.futures
@@ -55,19 +55,27 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build(force: bool = True, jobs: int = 8, sources=None) -> str:
-    """Compile every source and link the shared library. Returns the library path."""
+def _stale(src: str) -> bool:
+    """Is the object file of `src` older than the source or any header?"""
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    if not os.path.exists(obj):
+        return True
+    deps = [os.path.join(HERE, src)] + [os.path.join(HERE, f) for f in os.listdir(HERE) if f.endswith(".h")]
+    deps.append(os.path.join(HERE, "..", "..", "include", "daceml_hip.h"))
+    return os.path.getmtime(obj) < max(os.path.getmtime(d) for d in deps)
+
+
+def build(force: bool = True, jobs: int = 8) -> str:
+    """Compile every source (with force=False: only those whose object file is out of date) and link the shared
+    library from all object files. Returns the library path."""
     os.makedirs(OBJ_DIR, exist_ok=True)
-    srcs = [s for s in (sources or SOURCES) if os.path.exists(os.path.join(HERE, s))]
-    if not force and os.path.exists(LIB_PATH):
-        newest = max(os.path.getmtime(os.path.join(HERE, f)) for f in os.listdir(HERE)
-                     if f.endswith((".hip", ".cpp", ".h")))
-        header = os.path.join(HERE, "..", "..", "include", "daceml_hip.h")
-        newest = max(newest, os.path.getmtime(header))
-        if os.path.getmtime(LIB_PATH) >= newest:
-            return LIB_PATH
+    srcs = [s for s in SOURCES if os.path.exists(os.path.join(HERE, s))]
+    todo = srcs if force else [s for s in srcs if _stale(s)]
+    if not todo and os.path.exists(LIB_PATH):
+        return LIB_PATH
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(_compile, srcs))
+        list(pool.map(_compile, todo))
+    objs = [os.path.join(OBJ_DIR, os.path.splitext(s)[0] + ".o") for s in srcs]
     cmd = [hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB_PATH, *objs]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -76,5 +84,5 @@ def build(force: bool = True, jobs: int = 8, sources=None) -> str:
 
 
 if __name__ == "__main__":
-    path = build(force="--force" in sys.argv or True)
+    path = build(force="--incremental" not in sys.argv)
     print(path)
