@@ -135,11 +135,10 @@ SIGNATURES = {
     "dmlhip_attention_backward_workspace_bytes": (c_size_t, [POINTER(AttentionDesc)]),
     "dmlhip_attention_backward_f16": (c_int, [POINTER(AttentionDesc), POINTER(AttentionDesc), _P, _P, _P, _P, _P, _P, _P,
                                               _P, _P, _P, c_size_t, _P]),
-}
-
-# exported for the test-suite only (not declared in the public header)
-DEBUG_SIGNATURES = {
+    # diagnostics (switches for tests and measurements, declared at the end of the header)
+    "dmlhip_conv2d_expand_depthwise_lds_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "dmlhip_debug_force_gemm_config": (None, [c_int]),
+    "dmlhip_debug_gemm_direct_lds": (None, [c_int]),
     "dmlhip_debug_grouped_single_launches": (ctypes.c_longlong, []),
     "dmlhip_debug_force_fused_strip": (None, [c_int]),
 }
@@ -167,7 +166,7 @@ def load():
             "%s not found. Build it with `python -m daceml_amd.csrc.build` (needs hipcc); "
             "this package has no fallback compute path." % LIB_PATH)
     lib = ctypes.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in list(SIGNATURES.items()) + list(DEBUG_SIGNATURES.items()):
+    for name, (restype, argtypes) in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes

@@ -189,7 +189,7 @@ size_t fused_lds_bytes(int toh, int stride, int w, int cin) {
     return ((size_t)kCB * ih * (w + 2) + (size_t)kCB * (cin + 1) + (size_t)kCB * 10) * sizeof(float);
 }
 
-int g_fused_toh = 0;   // test hook: pin the strip height
+thread_local int g_fused_toh = 0;   // diagnostic switch (per calling thread): pin the strip height
 
 }  // namespace
 }  // namespace dml
@@ -199,6 +199,12 @@ using namespace dml;
 extern "C" {
 
 void dmlhip_debug_force_fused_strip(int toh) { g_fused_toh = toh; }
+
+size_t dmlhip_conv2d_expand_depthwise_lds_bytes(int64_t w, int64_t cin, int64_t stride) {
+    if (w <= 0 || w > 4096 || cin <= 0 || cin > (1 << 20) || (stride != 1 && stride != 2)) return 0;
+    const size_t need = fused_lds_bytes(1, (int)stride, (int)w, (int)cin);
+    return need <= 156 * 1024 ? need : 0;
+}
 
 int dmlhip_conv2d_expand_depthwise_f32(const dmlhip_conv2d_desc* pw, const dmlhip_conv2d_desc* dw, const void* x,
                                        const void* w_pw, const void* b_pw, const void* w_dw, const void* b_dw, void* y,

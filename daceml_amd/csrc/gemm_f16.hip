@@ -17,6 +17,8 @@
 // into RU chunks of eight K values, so no separate transpose kernel or HBM round trip is needed.
 #include "gemm_f16_common.h"
 
+#include <atomic>
+
 namespace dml {
 using namespace gemm16;
 namespace {
@@ -363,8 +365,10 @@ int operand_mode(const void* p, int64_t rows, int64_t k, int64_t s_row, int64_t 
     return 2;
 }
 
-int g_force_cfg = -1;  // test hook: pin the tile configuration
-int g_direct_lds = 1;  // test hook: 0 forces the register-staged loaders
+// Diagnostic switches (declared in the public header). Per calling thread, so that one thread pinning a configuration
+// does not change what other threads launch.
+thread_local int g_force_cfg = -1;  // pin the tile configuration
+thread_local int g_direct_lds = 1;  // 0 forces the register-staged loaders
 
 }  // namespace
 }  // namespace dml
@@ -373,12 +377,11 @@ using namespace dml;
 
 extern "C" {
 
-// Not part of the public header: lets the tests exercise every tile configuration.
 void dmlhip_debug_force_gemm_config(int cfg) { g_force_cfg = cfg; }
 void dmlhip_debug_gemm_direct_lds(int on) { g_direct_lds = on; }
-static long long g_grouped_single_launches = 0;
+static std::atomic<long long> g_grouped_single_launches{0};
 // Number of grouped calls that went out as ONE launch (tests check that grouping really happens).
-long long dmlhip_debug_grouped_single_launches() { return g_grouped_single_launches; }
+long long dmlhip_debug_grouped_single_launches() { return g_grouped_single_launches.load(); }
 
 struct GemmGroup {
     int count;

@@ -112,17 +112,6 @@ struct Stream<R, 1, T> {  // row-contiguous: tile [64 k][R], chunk c (8 rows) of
     }
 };
 
-#ifdef DML_GEMM_TRACE
-// Lab-only timeline: lane `slot` of one VGPR receives the low half of the shader clock; written out at the end.
-__device__ unsigned* dml_gemm_trace_buf;
-#define DML_TR(slot)                                                                                               \
-    do {                                                                                                           \
-        const int s_ = (slot);                                                                                     \
-        if (s_ < 64) { const int t_ = (int)__builtin_readcyclecounter(); trace_v = ((int)(threadIdx.x & 63) == s_) ? t_ : trace_v; } \
-    } while (0)
-#else
-#define DML_TR(slot)
-#endif
 
 // ---------------------------------------------------------------- kernel
 // KSUM: the operand pairs g.ga[i] / g.gb[i] are concatenated along K (one output, see GemmArgs::ksum). A template
@@ -140,10 +129,6 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     constexpr int LPT = BM / 32 + BN / 32;  // DMA instructions per wavefront per tile
     extern __shared__ __attribute__((aligned(16))) char lds[];
 
-#ifdef DML_GEMM_TRACE
-    int trace_v = 0;
-#endif
-    DML_TR(0);
     // All of this is wave-uniform integer arithmetic in 32 bits (the host checks total_blocks < 2^31): 64-bit
     // divisions are long software sequences, and this prologue runs before the first load can be issued.
     uint32_t bid = blockIdx.x;
@@ -250,12 +235,9 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
             if constexpr (KSUM) advance();
         }
     }
-    DML_TR(1);
     if (nk >= NSTAGE - 1) wait_vm_lgkm0<(NSTAGE - 2) * LPT>();
     else wait_vm_lgkm0<0>();
-    DML_TR(2);
     __builtin_amdgcn_s_barrier();
-    DML_TR(3);
 
     half8 af[2][TM], bf[2][TN];
     if (nk > 0) {
@@ -300,12 +282,9 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
             } else {
                 // last sub-step: its fragments are the only reads outstanding. Tile kt+1 must have
                 // landed for every wavefront before anybody reads it.
-                DML_TR(4 + 3 * kt);
                 if (fill < nk) wait_vm_lgkm0<(NSTAGE - 2) * LPT>();
                 else wait_vm_lgkm0<0>();
-                DML_TR(5 + 3 * kt);
                 __builtin_amdgcn_s_barrier();
-                DML_TR(6 + 3 * kt);
                 if (more) {
                     sa.template frags<0>((uint32_t)nxt_stage * STAGE, af[0]);
                     sb.template frags<0>((uint32_t)nxt_stage * STAGE, bf[0]);
@@ -349,7 +328,6 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     }
     wait_vm_lgkm0<0>();
     __syncthreads();
-    DML_TR(62);
 
     // ---- epilogue (see store_strip): 32 x WN strips through this wavefront's LDS region
     constexpr int PITCH = WN + 4;
@@ -389,10 +367,6 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
             }
         }
     }
-#ifdef DML_GEMM_TRACE
-    DML_TR(63);
-    if (dml_gemm_trace_buf) dml_gemm_trace_buf[((size_t)blockIdx.x * 4 + wave) * 64 + lane] = (unsigned)trace_v;
-#endif
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE, bool KSUM = false, bool ASUM = false>

@@ -28,6 +28,7 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
+from .. import _lib
 from .. import contraction as C
 from .. import onnx as donnx
 from ..onnx.nodes import ONNXOp
@@ -435,9 +436,11 @@ def fuse_expand_depthwise(sdfg: SDFG) -> int:
             acts = (getattr(pw, "_activation", "none"), getattr(dw, "_activation", "none"))
             if not pointwise or not depthwise or acts not in EXPAND_DEPTHWISE_ACTIVATIONS:
                 continue
-            # the kernel's tiling: 16 input channels per step, 32 expanded channels per workgroup, and three expanded
-            # rows of 32 channels must fit LDS
-            if xd.shape[1] % 16 or md.shape[1] % 32 or 32 * 3 * (xd.shape[3] + 2) * 4 > 140 * 1024:
+            # the kernel's tiling: 16 input channels per step, 32 expanded channels per workgroup, and the smallest
+            # row strip (three padded expanded rows of 32 channels, the 32 x (Cin + 1) weight block, the taps) must
+            # fit LDS - asked of the library, which sizes the launch with the same function
+            if xd.shape[1] % 16 or md.shape[1] % 32 or \
+                    not _lib.load().dmlhip_conv2d_expand_depthwise_lds_bytes(xd.shape[3], xd.shape[1], strides[0]):
                 continue
             ins = {"X": x, "W_pw": _in_array(state, pw, "W"), "W_dw": _in_array(state, dw, "W")}
             for conn, node in (("B_pw", pw), ("B_dw", dw)):

@@ -311,6 +311,9 @@ int dmlhip_conv2d_gated_f32(const dmlhip_conv2d_desc* d, const void* x, const vo
 int dmlhip_conv2d_expand_depthwise_f32(const dmlhip_conv2d_desc* pw, const dmlhip_conv2d_desc* dw, const void* x,
                                        const void* w_pw, const void* b_pw, const void* w_dw, const void* b_dw,
                                        void* y, void* stream);
+/* LDS bytes the smallest row strip of dmlhip_conv2d_expand_depthwise_f32 needs for images `w` wide with `cin` input
+ * channels and depthwise stride `stride`; 0 when no strip fits (the call would return DMLHIP_ERR_UNSUPPORTED). */
+size_t dmlhip_conv2d_expand_depthwise_lds_bytes(int64_t w, int64_t cin, int64_t stride);
 /* cudnnConvolutionBackwardData / BackwardFilter (autodiff/implementations/onnx_ops.py:663-703)
  * and the ATen depthwise backward (onnx_ops.py:1201-1231). dw is overwritten. The bias
  * gradient is dmlhip_reduce over [n, m, oh*ow] done by the caller (two reduce calls). */
@@ -411,6 +414,22 @@ int dmlhip_batchnorm_backward_act_f32(const void* dy, const void* x, const void*
                                       const void* saved_mean, const void* saved_var, void* dx, float* dscale,
                                       float* dbias, int64_t n, int64_t c, int64_t hw, float eps, int act,
                                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ diagnostics
+ * Switches for tests and measurements; nothing in the reference corresponds to them (its cuDNN expansion exposes
+ * `node._algorithm`, cudnn_implementations.py:131-146, for the same purpose). The two "force" switches and the
+ * loader switch are per calling thread: they change only what that thread launches afterwards, and a value of
+ * -1 / 0 / 1 respectively restores the default choice. The counter is process-wide and atomic. */
+/* Pin the tile configuration of the fp16 contraction kernels: 0 = 128x128 tile with a 4-stage ring, 1 = 256x128,
+ * 2 = 256x256, 3 = 128x128 with a 2-stage ring; -1 = chosen per problem (default). */
+void dmlhip_debug_force_gemm_config(int cfg);
+/* 0: the fp16 contractions stage their operands through registers instead of loading them straight into LDS;
+ * 1 = default. */
+void dmlhip_debug_gemm_direct_lds(int on);
+/* Number of grouped / K-concatenated / row-sum contraction calls that went out as one launch so far. */
+long long dmlhip_debug_grouped_single_launches(void);
+/* Pin the output-row strip height of dmlhip_conv2d_expand_depthwise_f32 (used if it fits LDS); 0 = default. */
+void dmlhip_debug_force_fused_strip(int toh);
 
 #ifdef __cplusplus
 }

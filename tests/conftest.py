@@ -33,3 +33,15 @@ def pytest_collection_modifyitems(config, items):
 def lib():
     from daceml_amd import _lib
     return _lib.load()
+
+
+@pytest.fixture(autouse=True)
+def _reset_diagnostic_switches():
+    """A test that pins a tile configuration and fails midway must not leave the pin set for the tests after it."""
+    yield
+    from daceml_amd import _lib
+    lib = _lib._lib
+    if lib is not None:
+        lib.dmlhip_debug_force_gemm_config(-1)
+        lib.dmlhip_debug_gemm_direct_lds(1)
+        lib.dmlhip_debug_force_fused_strip(0)

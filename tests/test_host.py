@@ -650,3 +650,21 @@ def test_an_output_that_another_node_reads_keeps_its_incoming_gradient():
     # the reverse node of the first Sigmoid reads the sum
     reads = {e.data.data for n in bst.library_nodes() if n.schema.name == "SigmoidGrad" for e in bst.in_edges(n)}
     assert total in reads
+
+
+def test_expand_depthwise_fusion_asks_the_library_whether_a_strip_fits(lib):
+    """The fusion pass fuses pointwise + depthwise only where the kernel's smallest row strip fits LDS, weight block
+    included: a wide input-channel count that the kernel would refuse at launch stays two convolutions."""
+    from daceml_amd import graphs
+    from daceml_amd.transformation import fusion
+    q = lib.dmlhip_conv2d_expand_depthwise_lds_bytes
+    # three padded rows of 32 channels + the 32 x (Cin + 1) weight block + taps and biases, in floats
+    assert q(112, 32, 2) == (32 * 3 * 114 + 32 * 33 + 320) * 4
+    assert q(112, 32, 1) == q(112, 32, 2)
+    assert q(112, 1024, 2) == 0 and q(5000, 32, 1) == 0 and q(112, 32, 3) == 0 and q(0, 32, 1) == 0
+
+    def fused(cin):
+        sdfg = graphs.mbconv_block(1, cin, 32, expand=2, cout=24, se_reduce=4, stride=2, dtype=torch.float32)
+        return fusion.auto_optimize(sdfg)["expand_depthwise"]
+    assert fused(1024) == 1      # 13 KB of rows + 131 KB of weights: fits
+    assert fused(1200) == 0      # 154 KB of weights alone: the launch would be refused
