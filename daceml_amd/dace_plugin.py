@@ -1,193 +1,391 @@
 """Registers the "hip" implementations inside a real DaCeML installation.
 
-Only meaningful where ``dace`` and ``daceml`` import (neither does in the build image, so this module
-has not been executed; it is kept small and follows the cuDNN expansion,
-daceml/onnx/op_implementations/cudnn_implementations.py:123-410, and its environment,
-daceml/onnx/environments/cudnn.py:11-70, line by line).
+Only meaningful where ``dace`` and ``daceml`` import. Neither does in the build image, so the functions that touch
+the DaCe API (``install`` and what it calls with a ``dace`` argument) have not been executed; they follow the cuDNN
+expansion (daceml/onnx/op_implementations/cudnn_implementations.py:123-410), its environment
+(daceml/onnx/environments/cudnn.py:11-70) and the cuDNN reverse node (daceml/autodiff/implementations/onnx_ops.py:
+494-760) call by call. Everything that decides WHAT is emitted - the C++ of every tasklet, the arrays and connector
+names of every nested SDFG - is computed by ``daceml_amd.lowering`` without DaCe and is covered by host-side tests
+that compile the emitted code against ``include/daceml_hip.h``.
 
 ``install()``:
-  1. defines a ``@dace.library.environment`` that adds ``include/`` and links ``libdaceml_hip.so``;
-  2. for every implementation in this package's ``ONNXForward`` registry builds a DaCeML ``ONNXForward``
-     subclass whose ``forward`` runs this package's planner on descriptors taken from the DaCe SDFG and
-     renders the resulting ``HipCall``s as the body of a C++ tasklet with pointer connectors;
-  3. registers it twice — ``@op_implementation`` (so autodiff's registry lookups see it) and
-     ``donnx.ONNX<Op>.register_implementation`` wrapped like onnx_op.py:668-697 (node classes snapshot
-     the registry at import time, so the decorator alone is not enough);
-  4. registers the ``BackwardImplementation``s the same way.
-After ``install()``, ``donnx.default_implementation = "hip"`` (or ``node.implementation = "hip"``) selects
-the kernels for existing SDFGs, the PyTorch frontend and autodiff-generated nodes.
+  1. defines a ``@dace.library.environment`` that adds ``include/`` and links ``libdaceml_hip.so``; its per-SDFG
+     state holds one workspace buffer;
+  2. for every "hip" implementation in this package's ``ONNXForward`` registry whose operator DaCeML has a node class
+     for, builds a DaCeML ``ONNXForward`` subclass: ``forward`` mirrors the node on a stand-in SDFG, runs this
+     package's expansion and returns a nested SDFG that holds one C++ tasklet with pointer connectors
+     (``empty_sdfg_for_node`` + ``add_tasklet``, cudnn_implementations.py:384-410);
+  3. registers it twice - ``@op_implementation`` (so autodiff's registry lookups see it) and
+     ``donnx.ONNX<Op>.register_implementation`` wrapped like onnx_op.py:668-697 (node classes snapshot the registry
+     at import time, so the decorator alone is not enough);
+  4. registers a DaCeML ``BackwardImplementation`` (``@autoregister_params(op=..., name="hip")``,
+     daceml/autodiff/base_abc.py:63-159) for every "hip" backward implementation of this package: its ``backward``
+     lowers this package's reverse nodes to C++ tasklets in a nested SDFG added to the backward state, named by the
+     connector contract of base_abc.py:75-108. Without this step the generator re-expands forward nodes with "pure"
+     implementations and differentiates their tasklets (backward_pass_generator.py:425-494), bypassing the kernels.
+After ``install()``, ``donnx.default_implementation = "hip"`` (or ``node.implementation = "hip"``) selects the
+kernels for existing SDFGs, the PyTorch frontend and autodiff-generated nodes; ``node.backward_implementation =
+"hip"`` (or ``ONNX<Op>.default_backward_implementation``) selects the reverse nodes.
+
+The fused node types (LayerNormalization, Gelu, FusedEinsum, FusedAttention ...) have no opset-12 class upstream, so
+they are not reached node by node. ``fuse_state`` / ``fuse_and_expand`` reach them a state at a time: the state's ONNX
+library nodes are mirrored into this package's SDFG, run through its fusion pass and expansions, and spliced back as
+ONE nested SDFG of C++ tasklets (the role ``ReplacementTransformation``, daceml/transformation/replacement.py:67-181,
+plays for single-node patterns upstream). ``fuse_and_expand`` is meant as a ``post_onnx_hook`` of the reference's
+``DaceModule`` in place of ``auto_optimize``.
 """
+import copy
 import os
 
-from . import hip_tasklet as T
-from . import _lib as L
+from . import lowering
+from .lowering import render_tasklet_code  # noqa: F401  (public: the C++ body of one expansion)
 
 _ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_LIB_DIR = os.path.join(_ROOT, "daceml_amd", "csrc")
+
+#: bytes of the per-SDFG workspace the environment allocates (every workspace query of the BERT-large and MBConv
+#: configurations is far below it; a tasklet whose expansion needs more is refused at expansion time)
+WORKSPACE_BYTES = 256 << 20
+
+ENVIRONMENT_INIT_CODE = """\
+__state->dmlhip_workspace_bytes = %dull;
+__state->dmlhip_workspace = nullptr;
+if (hipMalloc(&__state->dmlhip_workspace, __state->dmlhip_workspace_bytes) != hipSuccess)
+    throw std::runtime_error("daceml_amd: cannot allocate the kernel workspace");
+""" % WORKSPACE_BYTES
+ENVIRONMENT_FINALIZE_CODE = "if (__state->dmlhip_workspace) (void)hipFree(__state->dmlhip_workspace);\n"
+ENVIRONMENT_STATE_FIELDS = ["void* dmlhip_workspace;", "size_t dmlhip_workspace_bytes;"]
+ENVIRONMENT_HEADERS = ["daceml_hip.h", "hip/hip_runtime_api.h", "stdexcept", "string"]
 
 
-def _c_literal(arg, conn_ptr):
-    """C++ expression for one HipCall argument; `conn_ptr` maps a connector to its tasklet pointer name."""
-    if isinstance(arg, T.Ptr):
-        return "(%s + %d)" % (conn_ptr(arg.conn), arg.offset) if arg.offset else conn_ptr(arg.conn)
-    if isinstance(arg, T.Null):
-        return "nullptr"
-    if isinstance(arg, (T.I64, T.I32, T.USize)):
-        return str(int(arg.value))
-    if isinstance(arg, T.F32):
-        return "%.9ef" % arg.value
-    if isinstance(arg, T.Stream):
-        return "(void*)__dace_current_stream"
-    raise NotImplementedError(type(arg).__name__)
+def _torch_dtypes(dace):
+    import torch
+    return {dace.float16: torch.float16, dace.float32: torch.float32, dace.float64: torch.float64,
+            dace.int64: torch.int64, dace.int32: torch.int32, dace.bool: torch.bool, dace.uint8: torch.uint8}
 
 
-def render_tasklet_code(tasklet: T.HipTasklet, conn_ptr=lambda c: "_" + c):
-    """C++ body of a DaCe tasklet that performs the tasklet's HipCalls. Arrays, descriptor structs and the
-    workspace become locals / state fields declared ahead of the calls."""
-    lines, n = [], 0
-    for call in tasklet.calls:
-        args = []
-        for a in call.args:
-            if isinstance(a, T.I64Array):
-                name = "__dml_arr%d" % n
-                n += 1
-                lines.append("const int64_t %s[] = {%s};" % (name, ", ".join(str(int(v)) for v in a.values) or "0"))
-                args.append(name)
-            elif isinstance(a, T.PtrArray):
-                name = "__dml_ptrs%d" % n
-                n += 1
-                # void*[]: converts to both `const void* const*` (inputs) and `void* const*` (outputs)
-                lines.append("void* %s[] = {%s};" % (name, ", ".join("(void*)" + conn_ptr(c) for c in a.conns)))
-                args.append(name)
-            elif isinstance(a, T.Struct):
-                name = "__dml_desc%d" % n
-                n += 1
-                fields = []
-                for fname, ftype in a.value._fields_:
-                    v = getattr(a.value, fname)
-                    if hasattr(v, "__len__"):
-                        fields.append("{%s}" % ", ".join(str(x) for x in v))
-                    else:
-                        fields.append(repr(float(v)) + "f" if "float" in str(ftype) else str(int(v)))
-                lines.append("%s %s = {%s};" % (a.c_type, name, ", ".join(fields)))
-                args.append("&" + name)
-            elif isinstance(a, T.Workspace):
-                args.append("((char*)__state->dmlhip_workspace + %d)" % a.offset)
-            elif isinstance(a, T.WorkspaceBytes):
-                args.append("(__state->dmlhip_workspace_bytes - %d)" % a.offset)
-            else:
-                args.append(_c_literal(a, conn_ptr))
-        lines.append('if (int __s = %s(%s)) { fprintf(stderr, "%s: %%s\\n", dmlhip_last_error_string()); }' %
-                     (call.symbol, ", ".join(args), call.symbol))
-    return "\n".join(lines)
+def _dace_dtypes(dace):
+    return {v: k for k, v in _torch_dtypes(dace).items()}
 
 
-def install():
-    """Register everything with an importable DaCeML. Raises ImportError where dace / daceml are absent."""
-    import dace
+def make_environment(dace):
+    """Links libdaceml_hip.so (pattern: daceml/onnx/environments/cudnn.py:11-49)."""
     import dace.library
-    from dace import nodes as dnodes
+
+    @dace.library.environment
+    class DaceMLHip:
+        cmake_minimum_version = None
+        cmake_packages = []
+        cmake_variables = {}
+        cmake_includes = [os.path.join(_ROOT, "include"), "/opt/rocm/include"]
+        cmake_libraries = [os.path.join(_LIB_DIR, "libdaceml_hip.so")]
+        cmake_compile_flags = ["-D__HIP_PLATFORM_AMD__"]
+        cmake_link_flags = ["-L" + _LIB_DIR, "-Wl,-rpath," + _LIB_DIR]
+        cmake_files = []
+        state_fields = list(ENVIRONMENT_STATE_FIELDS)
+        headers = list(ENVIRONMENT_HEADERS)
+        init_code = ENVIRONMENT_INIT_CODE
+        finalize_code = ENVIRONMENT_FINALIZE_CODE
+        dependencies = []
+
+    return DaceMLHip
+
+
+# ----------------------------------------------------------------------------- DaCe -> this package
+def mirror_node(dace, our_onnx, node, state, sdfg):
+    """Rebuild `node` with this package's classes on a one-node stand-in SDFG (descriptors only). Returns
+    (our node, our state, our SDFG); arrays keep their outer names."""
+    from .sdfg import SDFG as OurSDFG
+    s = OurSDFG(node.label)
+    st = s.add_state()
+    ours = _mirror_into(dace, our_onnx, node, state, sdfg, s, st)
+    return ours, st, s
+
+
+def _mirror_into(dace, our_onnx, node, state, sdfg, s, st):
+    from .sdfg import Array as OurArray
+    to_torch = _torch_dtypes(dace)
+    cls = our_onnx.get_onnx_node(node.schema.name)
+    attrs = {a: getattr(node, a) for a in cls.schema.attributes if hasattr(node, a) and getattr(node, a) is not None}
+    ours = cls(node.label, **attrs)
+    st.add_node(ours)
+    for edges, is_input in ((state.in_edges(node), True), (state.out_edges(node), False)):
+        for e in edges:
+            name = e.data.data
+            if name not in s.arrays:
+                d = sdfg.arrays[name]
+                s.arrays[name] = OurArray([int(x) for x in d.shape], to_torch[d.dtype], transient=bool(d.transient),
+                                          strides=[int(x) for x in d.strides])
+            if is_input:
+                if e.dst_conn not in ours.in_connectors:
+                    ours.add_in_connector(e.dst_conn)
+                st.add_edge(st.add_read(name), None, ours, e.dst_conn, s.make_array_memlet(name))
+            else:
+                if e.src_conn not in ours.out_connectors:
+                    ours.add_out_connector(e.src_conn)
+                st.add_edge(ours, e.src_conn, st.add_write(name), None, s.make_array_memlet(name))
+    return ours
+
+
+# ----------------------------------------------------------------------------- this package -> DaCe
+def emit_nested_sdfg(dace, program: lowering.TaskletProgram, descriptors, environment):
+    """A ``dace.SDFG`` with one state that holds `program`'s tasklets as C++ tasklets between access nodes.
+    `descriptors` maps array names to DaCe data descriptors to copy (arrays not listed are new transients in GPU
+    global memory). Pattern: cudnn_implementations.py:384-410 (forward), onnx_ops.py:704-756 (reverse)."""
+    to_dace = _dace_dtypes(dace)
+    nsdfg = dace.SDFG(program.name + "_expansion")
+    nstate = nsdfg.add_state()
+    for name, d in program.arrays.items():
+        if name in descriptors:
+            desc = copy.deepcopy(descriptors[name])
+            desc.transient = False
+            nsdfg.add_datadesc(name, desc)
+        else:
+            nsdfg.add_array(name, list(d.shape), to_dace[d.dtype], strides=list(d.strides), transient=True,
+                            storage=dace.StorageType.GPU_Global)
+    last_write = {}   # array -> access node of its latest producer: orders the tasklets by data dependencies
+    for spec in program.tasklets:
+        ins = {"_" + c: dace.pointer(nsdfg.arrays[a].dtype) for c, a in spec.inputs.items()}
+        outs = {"_" + c: dace.pointer(nsdfg.arrays[a].dtype) for c, a in spec.outputs.items()}
+        tasklet = nstate.add_tasklet(spec.label, ins, outs, spec.code(), dace.dtypes.Language.CPP)
+        tasklet.environments = {environment.full_class_path()}
+        for conn, arr in spec.inputs.items():
+            src = last_write.get(arr) or nstate.add_read(arr)
+            nstate.add_edge(src, None, tasklet, "_" + conn, nsdfg.make_array_memlet(arr))
+        for conn, arr in spec.outputs.items():
+            dst = nstate.add_write(arr)
+            nstate.add_edge(tasklet, "_" + conn, dst, None, nsdfg.make_array_memlet(arr))
+            last_write[arr] = dst
+    return nsdfg
+
+
+def _check_workspace(program: lowering.TaskletProgram):
+    if program.workspace_bytes > WORKSPACE_BYTES:
+        raise ValueError("%s needs a workspace of %d bytes, the environment provides %d" %
+                         (program.name, program.workspace_bytes, WORKSPACE_BYTES))
+
+
+def forward_program(tasklet) -> lowering.TaskletProgram:
+    """The TaskletProgram of one forward expansion: arrays are named after the node's connectors, as
+    ``empty_sdfg_for_node`` names them (op_implementations/utils.py:105-139)."""
+    if not tasklet.calls:
+        raise ValueError("%r moves no data (a view): there is nothing to emit" % tasklet)
+    spec = lowering.TaskletSpec(tasklet.label, {c: c for c in tasklet.in_connectors},
+                                {c: c for c in tasklet.out_connectors}, list(tasklet.calls), {})
+    return lowering.TaskletProgram(tasklet.label, {}, {}, [spec], int(tasklet.workspace_bytes))
+
+
+# ----------------------------------------------------------------------------- installation
+def install():
+    """Register everything with an importable DaCeML. Raises ImportError where dace / daceml are absent. Returns
+    ``{"forward": [ops], "backward": [ops]}``."""
+    import dace
     from dace.transformation.transformation import ExpandTransformation
     import daceml.onnx as donnx
     from daceml.onnx.forward_implementation_abc import ONNXForward as RefONNXForward
     from daceml.onnx.op_implementations.utils import op_implementation as ref_op_implementation
-    from daceml.util.utils import in_desc_with_name, out_desc_with_name  # noqa: F401
+    from daceml.util.utils import in_desc_with_name, out_desc_with_name
 
     from . import onnx as our_onnx
     from .onnx.forward_implementation_abc import ONNXForward as OurONNXForward
-    from .sdfg import SDFG as OurSDFG, Array as OurArray
 
-    lib_dir = os.path.join(_ROOT, "daceml_amd", "csrc")
-
-    @dace.library.environment
-    class DaceMLHip:
-        """Links libdaceml_hip.so (pattern: daceml/onnx/environments/cudnn.py:11-49)."""
-        cmake_minimum_version = None
-        cmake_packages = []
-        cmake_variables = {}
-        cmake_includes = [os.path.join(_ROOT, "include")]
-        cmake_libraries = [os.path.join(lib_dir, "libdaceml_hip.so")]
-        cmake_compile_flags = []
-        cmake_link_flags = ["-L" + lib_dir, "-Wl,-rpath," + lib_dir]
-        cmake_files = []
-        state_fields = ["void* dmlhip_workspace;", "size_t dmlhip_workspace_bytes;"]
-        headers = ["daceml_hip.h", "cstdio"]
-        init_code = ("__state->dmlhip_workspace_bytes = 256u << 20;\n"
-                     "hipMalloc(&__state->dmlhip_workspace, __state->dmlhip_workspace_bytes);")
-        finalize_code = "hipFree(__state->dmlhip_workspace);"
-        dependencies = []
-
-    import torch
-    _to_torch = {dace.float16: torch.float16, dace.float32: torch.float32, dace.float64: torch.float64,
-                 dace.int64: torch.int64, dace.int32: torch.int32, dace.bool: torch.bool}
-
-    def mirror(node, state, sdfg):
-        """Rebuild the node with this package's classes on a one-node stand-in SDFG (descriptors only)."""
-        s = OurSDFG(node.label)
-        st = s.add_state()
-        attrs = {a: getattr(node, a) for a in our_onnx.get_onnx_node(node.schema.name).schema.attributes
-                 if hasattr(node, a)}
-        ours = our_onnx.get_onnx_node(node.schema.name)(node.label, **attrs)
-        for e in state.in_edges(node):
-            d = sdfg.arrays[e.data.data]
-            s.arrays.setdefault(e.data.data, OurArray(d.shape, _to_torch[d.dtype], strides=d.strides))
-            ours.add_in_connector(e.dst_conn)
-            st.add_edge(st.add_read(e.data.data), None, ours, e.dst_conn, s.make_array_memlet(e.data.data))
-        for e in state.out_edges(node):
-            d = sdfg.arrays[e.data.data]
-            s.arrays.setdefault(e.data.data, OurArray(d.shape, _to_torch[d.dtype], strides=d.strides))
-            ours.add_out_connector(e.src_conn)
-            st.add_edge(ours, e.src_conn, st.add_write(e.data.data), None, s.make_array_memlet(e.data.data))
-        return ours, st, s
-
-    registered = []
+    env = make_environment(dace)
+    registered = {"forward": [], "backward": []}
     for impl, args in list(OurONNXForward.extensions().items()):
         if args.get("name") != "hip" or not donnx.has_onnx_node(args["op"]):
-            continue  # fused node types (LayerNormalization, FusedEinsum ...) have no opset-12 class upstream
+            continue   # fused node types have no opset-12 class upstream: see fuse_state
         op = args["op"]
 
         def make(op=op, impl=impl):
             class HipImplementation(RefONNXForward):
-                environments = [DaceMLHip]
+                environments = [env]
 
                 @staticmethod
                 def forward_can_be_applied(node, state, sdfg) -> bool:
                     try:
-                        ours, st, s = mirror(node, state, sdfg)
-                        return impl.forward_can_be_applied(ours, st, s)
+                        ours, st, s = mirror_node(dace, our_onnx, node, state, sdfg)
+                        if not impl.forward_can_be_applied(ours, st, s):
+                            return False
+                        _check_workspace(forward_program(impl.forward(ours, st, s)))
+                        return True
                     except Exception:
                         return False
 
                 @staticmethod
                 def forward(node, state, sdfg):
-                    ours, st, s = mirror(node, state, sdfg)
-                    tasklet = impl.forward(ours, st, s)
-                    ins = {c: dace.pointer(sdfg.arrays[next(state.in_edges_by_connector(node, c)).data.data].dtype)
-                           for c in tasklet.in_connectors}
-                    outs = {c: dace.pointer(sdfg.arrays[next(state.out_edges_by_connector(node, c)).data.data].dtype)
-                            for c in tasklet.out_connectors}
-                    code = render_tasklet_code(tasklet, conn_ptr=lambda c: "_" + c)
-                    t = dnodes.Tasklet(node.label + "_hip", {"_" + k: v for k, v in ins.items()},
-                                       {"_" + k: v for k, v in outs.items()}, code, dace.dtypes.Language.CPP)
-                    t.environments = {DaceMLHip.full_class_path()}
-                    return t
+                    ours, st, s = mirror_node(dace, our_onnx, node, state, sdfg)
+                    program = forward_program(impl.forward(ours, st, s))
+                    _check_workspace(program)
+                    descs = {}
+                    for e in state.in_edges(node):
+                        descs[e.dst_conn] = in_desc_with_name(node, state, sdfg, e.dst_conn)
+                    for e in state.out_edges(node):
+                        descs[e.src_conn] = out_desc_with_name(node, state, sdfg, e.src_conn)
+                    from .sdfg import Array as OurArray
+                    to_torch = _torch_dtypes(dace)
+                    program.arrays = {c: OurArray([int(x) for x in d.shape], to_torch[d.dtype]) for c, d in descs.items()}
+                    return emit_nested_sdfg(dace, program, descs, env)
 
             HipImplementation.__name__ = "Hip" + op
             return HipImplementation
 
         cls = ref_op_implementation(op=op, name="hip")(make())
 
-        class Expansion(ExpandTransformation):
-            environments = [DaceMLHip]
-            forward_impl = cls
+        def make_expansion(cls=cls):
+            class Expansion(ExpandTransformation):
+                environments = [env]
+                forward_impl = cls
 
-            @classmethod
-            def expansion(c, node, state, sdfg, **kwargs):
-                node.validate(sdfg, state)
-                if c.forward_impl.forward_can_be_applied(node, state, sdfg):
-                    return c.forward_impl.forward(node, state, sdfg, **kwargs)
-                # keep the reference's behaviour: fall back to whatever it would have used
-                return type(node).implementations["onnxruntime"].expansion(node, state, sdfg, **kwargs)
+                @classmethod
+                def expansion(c, node, state, sdfg, **kwargs):
+                    node.validate(sdfg, state)
+                    if c.forward_impl.forward_can_be_applied(node, state, sdfg):
+                        return c.forward_impl.forward(node, state, sdfg, **kwargs)
+                    # keep the reference's behaviour: fall back to what it would have used (onnx_op.py:685-697)
+                    return type(node).implementations["onnxruntime"].expansion(node, state, sdfg, **kwargs)
 
-        getattr(donnx, "ONNX" + op).register_implementation("hip", Expansion)
-        registered.append(op)
+            return Expansion
+
+        getattr(donnx, "ONNX" + op).register_implementation("hip", make_expansion())
+        registered["forward"].append(op)
+
+    registered["backward"] = _install_backward(dace, donnx, our_onnx, env)
     return registered
+
+
+def _install_backward(dace, donnx, our_onnx, env):
+    import dace.registry
+    from daceml.autodiff.base_abc import (BackwardImplementation as RefBackwardImplementation,
+                                          BackwardResult as RefBackwardResult)
+    import daceml.autodiff.utils as butils
+
+    from .autodiff.base_abc import BackwardImplementation as OurBackwardImplementation
+
+    done = []
+    for impl, args in list(OurBackwardImplementation.extensions().items()):
+        op = args.get("op")
+        if args.get("name") != "hip" or op is None or not donnx.has_onnx_node(op):
+            continue
+
+        def make(op=op, impl=impl):
+            def lowered(forward_node, state, sdfg, given, required):
+                ours, st, s = mirror_node(dace, our_onnx, forward_node, state, sdfg)
+                if not impl.backward_can_be_applied(ours, st, s):
+                    raise ValueError("not applicable")
+                lb = lowering.lower_backward(ours, st, s, impl, given, required)
+                _check_workspace(lb.program)
+                return lb
+
+            class HipBackward(RefBackwardImplementation):
+                @staticmethod
+                def backward_can_be_applied(node, state, sdfg) -> bool:
+                    try:
+                        given = [e.src_conn for e in state.out_edges(node)]
+                        required = [e.dst_conn for e in state.in_edges(node)
+                                    if sdfg.arrays[e.data.data].dtype in (dace.float16, dace.float32)]
+                        lowered(node, state, sdfg, given, required)
+                        return True
+                    except Exception:
+                        return False
+
+                @staticmethod
+                def backward(forward_node, context, given_gradients, required_gradients):
+                    lb = lowered(forward_node, context.forward_state, context.forward_sdfg, list(given_gradients),
+                                 list(required_gradients))
+                    descs = {}
+                    for conn in lb.forward_inputs:
+                        descs[conn] = butils.forward_in_desc_with_name(forward_node, context, conn)
+                    for conn in lb.forward_outputs:
+                        descs[conn] = butils.forward_out_desc_with_name(forward_node, context, conn)
+                    for conn, name in lb.given_grad_names.items():
+                        descs[name] = butils.forward_out_desc_with_name(forward_node, context, conn)
+                    for conn, name in lb.required_grad_names.items():
+                        descs[name] = butils.forward_in_desc_with_name(forward_node, context, conn)
+                    nsdfg = emit_nested_sdfg(dace, lb.program, descs, env)
+                    inputs = set(lb.forward_inputs) | set(lb.forward_outputs) | set(lb.given_grad_names.values())
+                    outputs = set(lb.required_grad_names.values())
+                    node = context.backward_state.add_nested_sdfg(nsdfg, None, inputs, outputs)
+                    # forward inputs are connected by the generator (connectors named like the forward node's);
+                    # forward outputs have to be asked for (autodiff/utils.py:224-261)
+                    for conn in lb.forward_outputs:
+                        butils.connect_output_from_forward(forward_node, node, context, conn)
+                    # every gradient is written in full by its kernel: nothing has to be zeroed first
+                    zero_init = {name: False for name in lb.required_grad_names.values()}
+                    return node, RefBackwardResult(required_grad_names=dict(lb.required_grad_names),
+                                                   given_grad_names=dict(lb.given_grad_names), zero_init=zero_init)
+
+            HipBackward.__name__ = "Hip%sBackward" % op
+            return HipBackward
+
+        dace.registry.autoregister_params(op=op, name="hip")(make())
+        done.append(op)
+    return done
+
+
+# ----------------------------------------------------------------------------- fused states
+def mirror_state(dace, our_onnx, state, sdfg):
+    """All ONNX library nodes of `state` on a stand-in SDFG of this package. Raises ``ValueError`` if the state
+    holds anything other than ONNX library nodes this package has classes for and access nodes."""
+    from daceml.onnx.nodes.onnx_op import ONNXOp as RefONNXOp
+    from .sdfg import SDFG as OurSDFG
+    s = OurSDFG(sdfg.name + "_" + state.label)
+    st = s.add_state(state.label)
+    for node in state.nodes():
+        if isinstance(node, dace.nodes.AccessNode):
+            continue
+        if not isinstance(node, RefONNXOp) or not our_onnx.has_onnx_node(node.schema.name):
+            raise ValueError("state %s holds %r, which has no counterpart here" % (state.label, node))
+        _mirror_into(dace, our_onnx, node, state, sdfg, s, st)
+    return st, s
+
+
+def fuse_state(sdfg, state, training: bool = False, environment=None):
+    """Replace the contents of `state` (ONNX library nodes and access nodes only) by one nested SDFG of C++ tasklets:
+    the state is mirrored, fused (``transformation.fusion.auto_optimize``), expanded with the "hip" implementations
+    and lowered. Returns the nested SDFG node. Arrays that the fused state no longer touches stay in `sdfg`."""
+    import dace
+    from . import onnx as our_onnx
+    from .runtime import expand_onnx_nodes
+    from .transformation import fusion
+    env = environment or make_environment(dace)
+    st, s = mirror_state(dace, our_onnx, state, sdfg)
+    # arrays that other states or the caller see must survive fusion as they are
+    fusion.auto_optimize(s, training=training)
+    expand_onnx_nodes(s)
+    program = lowering.lower_state(s, st, name=sdfg.name + "_" + state.label + "_fused")
+    _check_workspace(program)
+    descs = {n: sdfg.arrays[n] for n in program.arguments() if n in sdfg.arrays}
+    missing = [n for n in program.arguments() if n not in descs]
+    if missing:
+        raise ValueError("the fused state reads arrays the SDFG does not have: %s" % missing)
+    nsdfg = emit_nested_sdfg(dace, program, descs, env)
+    reads = {a for t in program.tasklets for a in t.inputs.values() if a in descs}
+    writes = {a for t in program.tasklets for a in t.outputs.values() if a in descs}
+    for node in list(state.nodes()):
+        state.remove_node(node)
+    nested = state.add_nested_sdfg(nsdfg, sdfg, reads, writes)
+    for name in sorted(reads):
+        state.add_edge(state.add_read(name), None, nested, name, sdfg.make_array_memlet(name))
+    for name in sorted(writes):
+        state.add_edge(nested, name, state.add_write(name), None, sdfg.make_array_memlet(name))
+    return nested
+
+
+def fuse_and_expand(dace_module):
+    """``post_onnx_hook`` for the reference's ``DaceModule`` (daceml/torch/module.py:179-245) in place of
+    ``auto_optimize``: every state that consists of ONNX library nodes is replaced by its fused form; states that hold
+    anything else are left to the node-by-node expansions. Inference modules only: the reference differentiates AFTER
+    its post-ONNX hooks, and a state of C++ tasklets cannot be differentiated - modules built with ``backward=True``
+    keep their library nodes and use the node-by-node forward and backward registrations of ``install()``."""
+    if getattr(dace_module, "backward", False):
+        raise ValueError("fuse_and_expand is for inference modules; with backward=True use install() and "
+                         "donnx.default_implementation = 'hip'")
+    sdfg = dace_module.sdfg
+    fused = 0
+    for state in sdfg.nodes():
+        try:
+            fuse_state(sdfg, state)
+            fused += 1
+        except ValueError:
+            continue
+    return fused

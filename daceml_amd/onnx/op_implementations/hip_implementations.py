@@ -24,6 +24,7 @@ from .utils import op_implementation
 IMPL = "hip"
 _SFX = {torch.float16: "f16", torch.float32: "f32"}
 _CODE = {torch.float16: L.F16, torch.float32: L.F32}
+_ITEMSIZE = {torch.float16: 2, torch.float32: 4}
 _ACT = {"none": L.ACT_NONE, "gelu": L.ACT_GELU, "swish": L.ACT_SWISH, "sigmoid": L.ACT_SIGMOID, "relu": L.ACT_RELU}
 
 
@@ -271,8 +272,12 @@ class HipMatMul(ONNXForward):
 
 @op_implementation(op="Gemm", name=IMPL)
 class HipGemm(ONNXForward):
-    """PureGemm (pure_implementations.py:380-553): alpha*op(A)op(B) + beta*C with C a vector over the
-    last result index (how nn.Linear exports); alpha and the bias go into the GEMM epilogue."""
+    """PureGemm (pure_implementations.py:380-553): ``Y = alpha * op(A) op(B) + beta * C``, one GEMM launch with alpha
+    and C in its epilogue. C is indexed by the trailing letters of the result and its trailing dims must equal Y's
+    (:533-539): a vector over the last result index (how nn.Linear exports; ``[1, N]`` is taken as that vector too)
+    rides as the column bias, a full ``[M, N]`` matrix as the epilogue's residual operand. ``beta`` other than 0 or 1
+    costs one small extra launch: the scaled C (the reference's ``betascale`` map, :540-551) is produced first - a
+    vector into the workspace, a matrix into Y, onto which the product is then accumulated."""
     @staticmethod
     def _eq(node):
         a, b = "ik", "kj"
@@ -281,6 +286,16 @@ class HipGemm(ONNXForward):
         if node.transB == 1:
             b = b[::-1]
         return "%s,%s->ij" % (a, b)
+
+    @staticmethod
+    def _c_kind(c: Array, y: Array) -> Optional[str]:
+        """"vector" (C[n] or C[1, n]), "matrix" (C[m, n]) or None (a shape the reference's broadcast rule refuses)."""
+        n = y.shape[-1]
+        if tuple(c.shape) == tuple(y.shape) and len(y.shape) == 2 and y.shape[0] != 1:
+            return "matrix"
+        if c.total_size == n and c.shape[-1] == n:
+            return "vector"
+        return None
 
     @staticmethod
     def forward_can_be_applied(node, state, sdfg) -> bool:
@@ -293,9 +308,9 @@ class HipGemm(ONNXForward):
                 return False
             if "C" in ins and node.beta != 0:
                 c = ins["C"]
-                if node.beta != 1 or not c.is_contiguous() or c.dtype != y.dtype:
+                if not c.is_contiguous() or c.dtype != y.dtype or not y.is_contiguous():
                     return False
-                if not (c.total_size == y.shape[-1] and c.shape[-1] == y.shape[-1]):
+                if HipGemm._c_kind(c, y) is None:
                     return False
             return True
         except Exception:
@@ -304,9 +319,45 @@ class HipGemm(ONNXForward):
     @staticmethod
     def forward(node, state, sdfg):
         ins, outs = _descs(node, state, sdfg)
-        use_c = "C" in ins and node.beta != 0
-        return _einsum_tasklet(node, state, HipGemm._eq(node), "A", "B", "Y", ins["A"], ins["B"], outs["Y"],
-                               alpha=node.alpha, bias="C" if use_c else None, bias_desc=ins["C"] if use_c else None)
+        a, b, y = ins["A"], ins["B"], outs["Y"]
+        eq = HipGemm._eq(node)
+        if "C" not in ins or node.beta == 0:
+            return _einsum_tasklet(node, state, eq, "A", "B", "Y", a, b, y, alpha=node.alpha)
+        c = ins["C"]
+        kind = HipGemm._c_kind(c, y)
+        if node.beta == 1:
+            if kind == "vector":
+                return _einsum_tasklet(node, state, eq, "A", "B", "Y", a, b, y, alpha=node.alpha, bias="C", bias_desc=c)
+            return _einsum_tasklet(node, state, eq, "A", "B", "Y", a, b, y, alpha=node.alpha, residual="C")
+        # beta * C first, then the product on top of it
+        sfx = _SFX[y.dtype]
+        plan = C.plan_contraction(eq, a.shape, a.strides, b.shape, b.strides)
+        x_conn, y_conn = ("B", "A") if plan.swapped else ("A", "B")
+        if kind == "matrix":
+            scale = HipCall("dmlhip_unary_" + sfx, [I32(L.SCALE), Ptr("C"), Ptr("Y"), I64(c.total_size),
+                                                    F32(float(node.beta)), Stream()])
+            desc = _gemm_struct(plan, node.alpha, 1.0, y.dtype, y.dtype, L.ACT_NONE)
+            tail = [Ptr(x_conn), Ptr(y_conn), Ptr("Y"), Null(), Null(), Null()]
+            ws, ws_off = 0, 0
+        else:
+            scale = HipCall("dmlhip_unary_" + sfx, [I32(L.SCALE), Ptr("C"), Workspace(0), I64(c.total_size),
+                                                    F32(float(node.beta)), Stream()])
+            desc = _gemm_struct(plan, node.alpha, 0.0, y.dtype, c.dtype, L.ACT_NONE)
+            ws_off = -(-c.total_size * _ITEMSIZE[c.dtype] // 256) * 256     # the GEMM's own scratch starts past it
+            tail = [Ptr(x_conn), Ptr(y_conn), Ptr("Y"), Workspace(0), Null(), Null()]
+            ws = ws_off
+        if a.dtype == torch.float16:
+            import ctypes
+            ws += L.load().dmlhip_gemm_f16_workspace_bytes(ctypes.byref(desc))
+            gemm = HipCall("dmlhip_gemm_f16_ws", [Struct(desc, "dmlhip_gemm_desc")] + tail +
+                           [Workspace(ws_off), WorkspaceBytes(ws_off), Stream()], flops=plan.flops,
+                           bytes_moved=_nbytes(a, b, y, c))
+        else:
+            gemm = HipCall("dmlhip_gemm_f32", [Struct(desc, "dmlhip_gemm_desc")] + tail + [Stream()], flops=plan.flops,
+                           bytes_moved=_nbytes(a, b, y, c))
+        scale.flops, scale.bytes_moved = 0, 0
+        return _tasklet(node, state, [scale, gemm], workspace_bytes=ws, flops=plan.flops,
+                        bytes_moved=_nbytes(a, b, y, c), kind="gemm")
 
 
 # ----------------------------------------------------------------------------- softmax / layernorm

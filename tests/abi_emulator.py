@@ -1,0 +1,156 @@
+"""A NumPy interpreter for a few entry points of include/daceml_hip.h, written from the header's comments.
+
+TEST INFRASTRUCTURE ONLY. It lets the host-side tests check what an expansion ASKS the library to do (descriptor
+contents, operand order, workspace use, the sequence of calls) on a machine without a GPU: an expansion's
+``HipCall``s are run against NumPy arrays and the result is compared with the oracle. It says nothing about the
+kernels themselves; those are checked on the GPU against the same oracle.
+"""
+import math
+
+import numpy as np
+from numpy.lib.stride_tricks import as_strided
+
+from daceml_amd import _lib as L
+from daceml_amd import hip_tasklet as T
+
+
+def _view(buf, offset, shape, strides):
+    """Strided view (element strides) into the flat array `buf`."""
+    item = buf.itemsize
+    flat = buf.reshape(-1)
+    return as_strided(flat[offset:], shape=shape, strides=[s * item for s in strides], writeable=False)
+
+
+def _act(kind, v):
+    if kind == L.ACT_NONE:
+        return v
+    if kind == L.ACT_GELU:
+        from scipy.special import erf
+        return 0.5 * v * (1.0 + erf(v / math.sqrt(2.0)))
+    if kind == L.ACT_RELU:
+        return np.maximum(v, 0)
+    if kind == L.ACT_SIGMOID:
+        return 1 / (1 + np.exp(-v))
+    if kind == L.ACT_SWISH:
+        return v / (1 + np.exp(-v))
+    raise ValueError(kind)
+
+
+def gemm(desc, a, b, c, bias, residual, pre_out):
+    """dmlhip_gemm_*: C[b][m, n] = act(alpha * sum_k A[b][m, k] B[b][k, n] + bias) + residual + beta * C. `a`, `b`,
+    `c`, ... are flat arrays; fp32 accumulation, one rounding to C's type."""
+    m, n, k = desc.m, desc.n, desc.k
+    batch = tuple(desc.batch)
+    av = _view(a, 0, batch + (m, k), tuple(desc.a_stride_batch) + (desc.a_stride_m, desc.a_stride_k))
+    bv = _view(b, 0, batch + (k, n), tuple(desc.b_stride_batch) + (desc.b_stride_k, desc.b_stride_n))
+    acc = np.matmul(av.astype(np.float64), bv.astype(np.float64)) * float(desc.alpha)
+    if bias is not None:
+        bb = bias.reshape(-1).astype(np.float64)
+        acc = acc + (bb[:m].reshape(m, 1) if desc.bias_along_m else bb[:n].reshape(1, n))
+    cs = tuple(desc.c_stride_batch) + (desc.c_stride_m, 1)
+    out_dtype = np.float16 if desc.out_dtype == L.F16 else np.float32
+    if c.dtype != out_dtype:
+        raise TypeError("C has dtype %s, the descriptor says %s" % (c.dtype, out_dtype))
+    if pre_out is not None:
+        pv = as_strided(pre_out.reshape(-1), shape=batch + (m, n), strides=[s * pre_out.itemsize for s in cs])
+        pv[...] = acc.astype(out_dtype)
+        acc = pv.astype(np.float64)
+    acc = _act(desc.act, acc)
+    if residual is not None:
+        acc = acc + _view(residual, 0, batch + (m, n), cs).astype(np.float64)
+    cv = as_strided(c.reshape(-1), shape=batch + (m, n), strides=[s * c.itemsize for s in cs])
+    if desc.beta != 0:
+        acc = acc + float(desc.beta) * cv.astype(np.float64)
+    cv[...] = acc.astype(out_dtype)
+
+
+def unary(op, x, y, n, param):
+    xv = x.reshape(-1)[:n].astype(np.float64)
+    if op == L.SCALE:
+        r = xv * np.float32(param).astype(np.float64)
+    elif op == L.IDENTITY:
+        r = xv
+    elif op == L.RELU:
+        r = np.maximum(xv, 0)
+    else:
+        raise NotImplementedError("unary op %d" % op)
+    y.reshape(-1)[:n] = r.astype(y.dtype)
+
+
+class Emulator:
+    """Runs the calls of a HipTasklet on NumPy arrays bound to its connectors."""
+    def __init__(self, workspace_bytes):
+        self.workspace = np.zeros(max(int(workspace_bytes), 256), dtype=np.uint8)
+        self.log = []
+
+    def run(self, tasklet, arrays):
+        """`arrays`: connector -> NumPy array (inputs are read, outputs written in place)."""
+        for call in tasklet.calls:
+            args = [self._arg(a, arrays) for a in call.args]
+            self.log.append(call.symbol)
+            if call.symbol in ("dmlhip_gemm_f16_ws", "dmlhip_gemm_f32"):
+                desc, a, b, c, bias, residual, pre = args[:7]
+                want = np.float16 if call.symbol.startswith("dmlhip_gemm_f16") else np.float32
+                assert a.dtype == want and b.dtype == want, "%s called with %s operands" % (call.symbol, a.dtype)
+                if bias is not None:
+                    bias = self._typed(bias, np.float16 if desc.bias_dtype == L.F16 else np.float32)
+                gemm(desc, a, b, c, bias, residual, pre)
+            elif call.symbol in ("dmlhip_unary_f16", "dmlhip_unary_f32"):
+                op, x, y, n, param = args[:5]
+                want = np.float16 if call.symbol.endswith("f16") else np.float32
+                x = self._typed(x, want)
+                y = self._typed(y, want)
+                unary(op, x, y, n, param)
+            else:
+                raise NotImplementedError("no emulation of %s" % call.symbol)
+
+    def _typed(self, buf, dtype):
+        """Workspace pointers arrive as raw bytes: view them with the element type the call implies."""
+        if buf.dtype == np.uint8 and dtype != np.uint8:
+            return buf[:buf.size // np.dtype(dtype).itemsize * np.dtype(dtype).itemsize].view(dtype)
+        return buf
+
+    def _arg(self, a, arrays):
+        if isinstance(a, T.Ptr):
+            return arrays[a.conn].reshape(-1)[a.offset:]
+        if isinstance(a, T.Null):
+            return None
+        if isinstance(a, (T.I64, T.I32, T.USize)):
+            return int(a.value)
+        if isinstance(a, T.F32):
+            return float(a.value)
+        if isinstance(a, T.Struct):
+            return a.value
+        if isinstance(a, T.Workspace):
+            return self.workspace[a.offset:]
+        if isinstance(a, T.WorkspaceBytes):
+            return self.workspace.size - a.offset
+        if isinstance(a, T.Stream):
+            return None
+        raise NotImplementedError(type(a).__name__)
+
+
+def run_state(sdfg, state, arrays):
+    """Run an expanded state: `arrays` maps array names to NumPy arrays (inputs given, outputs and transients are
+    allocated here when missing). Views are not supported."""
+    import torch
+    np_dtype = {torch.float16: np.float16, torch.float32: np.float32, torch.int64: np.int64}
+    ws = max([int(getattr(n, "workspace_bytes", 0)) for n in state.library_nodes()] + [0])
+    em = Emulator(ws)
+    for node in state.topological_sort():
+        if not getattr(node, "calls", None):
+            continue
+        bound = {}
+        for e in list(state.in_edges(node)) + list(state.out_edges(node)):
+            name = e.data.data
+            d = sdfg.arrays[name]
+            if d.view_of is not None:
+                raise NotImplementedError("views")
+            if name not in arrays:
+                if name in sdfg.constants:
+                    arrays[name] = sdfg.constants[name].detach().cpu().numpy().astype(np_dtype[d.dtype]).reshape(d.shape)
+                else:
+                    arrays[name] = np.full(d.shape, np.nan, dtype=np_dtype[d.dtype])
+            bound[e.dst_conn if e.dst is node else e.src_conn] = arrays[name]
+        em.run(node, bound)
+    return em
