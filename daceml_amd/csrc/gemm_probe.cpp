@@ -1,0 +1,112 @@
+// One fp16 contraction through the C ABI of libdaceml_hip.so, timed with HIP events: the stand-alone program the
+// per-configuration counter runs of the GEMM kernels are taken with (and a minimal example of calling the library
+// from C++ without Python).
+//
+//   gemm_probe M N K a-layout b-layout config iterations [check]
+//     a-layout: k = A stored [m][k] (K-contiguous), r = A stored [k][m]
+//     b-layout: k = B stored [n][k] (K-contiguous), r = B stored [k][n]
+//     config:   tile configuration for dmlhip_debug_force_gemm_config (-1 = the library's own choice)
+//     check:    compare 2000 sampled outputs with a double-precision dot product on the host
+//
+// Build (from the repository root):
+//   hipcc -O2 --offload-arch=gfx950 daceml_amd/csrc/gemm_probe.cpp -o daceml_amd/csrc/gemm_probe \
+//         -Ldaceml_amd/csrc -ldaceml_hip -Wl,-rpath,'$ORIGIN'
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "../../include/daceml_hip.h"
+
+#define PROBE_CHECK(x)                                                                    \
+    do {                                                                                  \
+        hipError_t e_ = (x);                                                              \
+        if (e_ != hipSuccess) {                                                           \
+            std::printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__);    \
+            std::exit(1);                                                                 \
+        }                                                                                 \
+    } while (0)
+
+int main(int argc, char** argv) {
+    if (argc < 8) {
+        std::printf("usage: gemm_probe M N K a-layout(k|r) b-layout(k|r) config iterations [check]\n");
+        return 1;
+    }
+    const long M = std::atol(argv[1]), N = std::atol(argv[2]), K = std::atol(argv[3]);
+    const char al = argv[4][0], bl = argv[5][0];
+    const int cfg = std::atoi(argv[6]), iters = std::atoi(argv[7]);
+    const bool check = argc > 8;
+    if (M <= 0 || N <= 0 || K <= 0 || iters <= 0 || (al != 'k' && al != 'r') || (bl != 'k' && bl != 'r')) {
+        std::printf("bad arguments\n");
+        return 1;
+    }
+    std::vector<_Float16> ha((size_t)M * K), hb((size_t)N * K);
+    std::mt19937 rng(1);
+    std::normal_distribution<float> nd(0.f, 1.f);
+    for (auto& v : ha) v = (_Float16)nd(rng);
+    for (auto& v : hb) v = (_Float16)(nd(rng) * 0.05f);
+    _Float16 *a, *b, *c;
+    PROBE_CHECK(hipMalloc(&a, ha.size() * 2));
+    PROBE_CHECK(hipMalloc(&b, hb.size() * 2));
+    PROBE_CHECK(hipMalloc(&c, (size_t)M * N * 2));
+    PROBE_CHECK(hipMemcpy(a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+    PROBE_CHECK(hipMemcpy(b, hb.data(), hb.size() * 2, hipMemcpyHostToDevice));
+    dmlhip_gemm_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.m = M; d.n = N; d.k = K;
+    d.batch[0] = d.batch[1] = d.batch[2] = 1;
+    if (al == 'k') { d.a_stride_m = K; d.a_stride_k = 1; } else { d.a_stride_m = 1; d.a_stride_k = M; }
+    if (bl == 'k') { d.b_stride_n = K; d.b_stride_k = 1; } else { d.b_stride_n = 1; d.b_stride_k = N; }
+    d.c_stride_m = N;
+    d.alpha = 1.f;
+    d.out_dtype = DMLHIP_F16;
+    d.bias_dtype = DMLHIP_F16;
+    dmlhip_debug_force_gemm_config(cfg);
+    hipStream_t st;
+    PROBE_CHECK(hipStreamCreate(&st));
+    for (int i = 0; i < 3; ++i) {
+        if (int e = dmlhip_gemm_f16(&d, a, b, c, nullptr, nullptr, nullptr, st)) {
+            std::printf("dmlhip_gemm_f16 returned %d: %s\n", e, dmlhip_last_error_string());
+            return 1;
+        }
+    }
+    PROBE_CHECK(hipStreamSynchronize(st));
+    hipEvent_t e0, e1;
+    PROBE_CHECK(hipEventCreate(&e0));
+    PROBE_CHECK(hipEventCreate(&e1));
+    PROBE_CHECK(hipEventRecord(e0, st));
+    for (int i = 0; i < iters; ++i) dmlhip_gemm_f16(&d, a, b, c, nullptr, nullptr, nullptr, st);
+    PROBE_CHECK(hipEventRecord(e1, st));
+    PROBE_CHECK(hipStreamSynchronize(st));
+    float ms = 0.f;
+    PROBE_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    const double us = ms * 1e3 / iters;
+    std::printf("M=%ld N=%ld K=%ld %c%c config %d: %.2f us per launch, %.1f TFLOP/s\n", M, N, K, al, bl, cfg, us,
+                2.0 * M * N * K / us / 1e6);
+    if (check) {
+        std::vector<_Float16> hc((size_t)M * N);
+        PROBE_CHECK(hipMemcpy(hc.data(), c, hc.size() * 2, hipMemcpyDeviceToHost));
+        double worst = 0;
+        int bad = 0;
+        for (int t = 0; t < 2000; ++t) {
+            long m = rng() % M, n = rng() % N;
+            if (t < 8) { m = (t & 1) ? M - 1 : 0; n = (t & 2) ? N - 1 : 0; }
+            double s = 0;
+            for (long k = 0; k < K; ++k) {
+                const float av = al == 'k' ? (float)ha[m * K + k] : (float)ha[k * M + m];
+                const float bv = bl == 'k' ? (float)hb[n * K + k] : (float)hb[k * N + n];
+                s += (double)av * bv;
+            }
+            const double err = std::fabs((double)(float)hc[m * N + n] - s);
+            if (err > 1e-2 + 2e-2 * std::fabs(s)) ++bad;
+            if (err > worst) worst = err;
+        }
+        std::printf("check: %d of 2000 samples beyond rtol 2e-2 / atol 1e-2, worst absolute error %.4g\n", bad, worst);
+        if (bad) return 2;
+    }
+    return 0;
+}
