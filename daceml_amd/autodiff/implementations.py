@@ -167,19 +167,53 @@ class HipFusedEinsumBackward(BackwardImplementation):
 # ----------------------------------------------------------------------------- softmax / layernorm
 @autoregister_params(op="Softmax", name=NAME)
 class HipSoftmaxBackward(BackwardImplementation):
-    """DefaultSoftmaxBackward (onnx_ops.py:237-275) as one SoftmaxGrad node; needs the forward output."""
+    """DefaultSoftmaxBackward (onnx_ops.py:237-275): ``prod = y * dy``; ``sums = ReduceSum(prod, axes=[axis],
+    keepdims=1)``; ``dx = prod - y * sums`` - the reduction runs over the single axis ``axis``, also where the forward
+    node coalesced several trailing axes. For the last axis that is one SoftmaxGrad node (one kernel, needs the forward
+    output); for any other axis the reference's own four nodes: Mul, ReduceSum, Mul, Sub."""
     @staticmethod
     def backward_can_be_applied(node, state, sdfg) -> bool:
         for e in state.in_edges_by_connector(node, "input"):
             nd = len(sdfg.arrays[e.data.data].shape)
-            return node.axis % nd == nd - 1
+            return nd >= 1 and -nd <= node.axis < nd
         return False
 
     @staticmethod
     def backward(forward_node, context, given_gradients, required_gradients):
-        sg = _new(context, "SoftmaxGrad", forward_node.label + "_backward", axis=-1)
-        connect_output_from_forward(forward_node, sg, context, "output", "Y")
-        return sg, BackwardResult(required_grad_names={"input": "dX"}, given_grad_names={"output": "dY"})
+        sdfg = context.forward_sdfg
+        out = _out_arr(context, forward_node, "output")
+        od = sdfg.arrays[out]
+        nd = len(od.shape)
+        axis = forward_node.axis % nd
+        if axis == nd - 1:
+            sg = _new(context, "SoftmaxGrad", forward_node.label + "_backward", axis=-1)
+            connect_output_from_forward(forward_node, sg, context, "output", "Y")
+            return sg, BackwardResult(required_grad_names={"input": "dX"}, given_grad_names={"output": "dY"})
+        label = forward_node.label + "_backward"
+        group = BackwardGroup(label)
+        sums_shape = tuple(1 if i == axis else e for i, e in enumerate(od.shape))
+        prod, _ = sdfg.add_transient(label + "_prod", od.shape, od.dtype)
+        sums, _ = sdfg.add_transient(label + "_sums", sums_shape, od.dtype)
+        scaled, _ = sdfg.add_transient(label + "_scaled", od.shape, od.dtype)
+        mul1 = _new(context, "Mul", label + "_mul_dy")
+        _read(context, out, mul1, "A")
+        mul1.add_in_connector("B")
+        group.map_input("output_grad", mul1, "B")
+        _write(context, mul1, "C", prod)
+        red = _new(context, "ReduceSum", label + "_sum", axes=[axis], keepdims=1)
+        _read(context, prod, red, "data")
+        _write(context, red, "reduced", sums)
+        mul2 = _new(context, "Mul", label + "_mul_sums")
+        _read(context, out, mul2, "A")
+        _read(context, sums, mul2, "B")
+        _write(context, mul2, "C", scaled)
+        sub = _new(context, "Sub", label + "_sub")
+        _read(context, prod, sub, "A")
+        _read(context, scaled, sub, "B")
+        sub.add_out_connector("C")
+        group.map_output("input_grad", sub, "C")
+        return group, BackwardResult(required_grad_names={"input": "input_grad"},
+                                     given_grad_names={"output": "output_grad"})
 
 
 @autoregister_params(op="FusedAttention", name=NAME)

@@ -747,6 +747,31 @@ def _reduce_geometry(shape, axes):
     return _prod(shape[:axes[0]]), _prod(shape[axes[0]:axes[-1] + 1]), _prod(shape[axes[-1] + 1:]), axes
 
 
+def _reduce_passes(shape, axes):
+    """The reduction as a sequence of passes over adjacent axes: [(outer, r, inner)], innermost run of reduced axes
+    first (each pass sees the tensor with the runs already reduced collapsed to 1). One pass when the axes are
+    adjacent. Sum / Max / Min compose exactly; Mean composes because every pass averages groups of one size."""
+    nd = len(shape)
+    axes = sorted(set(range(nd) if axes is None else [a % nd for a in axes]))
+    if not axes:
+        return None
+    runs, cur = [], [axes[0]]
+    for a in axes[1:]:
+        if a == cur[-1] + 1:
+            cur.append(a)
+        else:
+            runs.append(cur)
+            cur = [a]
+    runs.append(cur)
+    shape = list(shape)
+    passes = []
+    for run in reversed(runs):
+        passes.append((_prod(shape[:run[0]]), _prod(shape[run[0]:run[-1] + 1]), _prod(shape[run[-1] + 1:])))
+        for a in run:
+            shape[a] = 1
+    return passes
+
+
 def _make_reduce(op_name: str, code: int, doc: str):
     class _Reduce(ONNXForward):
         @staticmethod
@@ -754,14 +779,15 @@ def _make_reduce(op_name: str, code: int, doc: str):
             try:
                 x = in_desc_with_name(node, state, sdfg, "data")
                 y = out_desc_with_name(node, state, sdfg, "reduced")
-                geo = _reduce_geometry(x.shape, node.axes)
-                if geo is None or not (x.dtype in FLOAT_DTYPES and y.dtype in FLOAT_DTYPES and _dense(x, y)):
+                passes = _reduce_passes(x.shape, node.axes)
+                if passes is None or not (x.dtype in FLOAT_DTYPES and y.dtype in FLOAT_DTYPES and _dense(x, y)):
                     return False
-                outer, r, inner, _ = geo
-                if inner > 1 and outer > 65535:
-                    return False
-                if r == 0 and code != L.RSUM:
-                    return False
+                for outer, r, inner in passes:
+                    if inner > 1 and outer > 65535:
+                        return False
+                    if r == 0 and code != L.RSUM:
+                        return False
+                outer, r, inner = passes[-1]
                 return y.total_size == outer * inner
             except Exception:
                 return False
@@ -770,12 +796,34 @@ def _make_reduce(op_name: str, code: int, doc: str):
         def forward(node, state, sdfg):
             x = in_desc_with_name(node, state, sdfg, "data")
             y = out_desc_with_name(node, state, sdfg, "reduced")
-            outer, r, inner, _ = _reduce_geometry(x.shape, node.axes)
-            ws = L.load().dmlhip_reduce_workspace_bytes(outer, r, inner)
-            call = HipCall("dmlhip_reduce_" + _SFX[x.dtype],
-                           [I32(code), Ptr("data"), Ptr("reduced"), I32(_CODE[y.dtype]), I64(outer), I64(r), I64(inner),
-                            Workspace(), WorkspaceBytes(), Stream()])
-            return _tasklet(node, state, [call], workspace_bytes=ws, bytes_moved=_nbytes(x, y), kind="reduce")
+            passes = _reduce_passes(x.shape, node.axes)
+            lib = L.load()
+            if len(passes) == 1:
+                outer, r, inner = passes[0]
+                ws = lib.dmlhip_reduce_workspace_bytes(outer, r, inner)
+                call = HipCall("dmlhip_reduce_" + _SFX[x.dtype],
+                               [I32(code), Ptr("data"), Ptr("reduced"), I32(_CODE[y.dtype]), I64(outer), I64(r),
+                                I64(inner), Workspace(), WorkspaceBytes(), Stream()])
+                return _tasklet(node, state, [call], workspace_bytes=ws, bytes_moved=_nbytes(x, y), kind="reduce")
+            # reduced axes that are not adjacent: one pass per run of adjacent axes, innermost run first; results
+            # between the passes are fp32 and live in two alternating regions at the head of the workspace, each
+            # pass's own scratch behind them
+            align = lambda n: -(-n // 256) * 256  # noqa: E731
+            region = align(max(o * i for o, _, i in passes[:-1]) * 4)
+            scratch = max(lib.dmlhip_reduce_workspace_bytes(o, r, i) for o, r, i in passes)
+            calls = []
+            for k, (outer, r, inner) in enumerate(passes):
+                first, last = k == 0, k == len(passes) - 1
+                src = Ptr("data") if first else Workspace(((k - 1) % 2) * region)
+                dst = Ptr("reduced") if last else Workspace((k % 2) * region)
+                sfx = _SFX[x.dtype] if first else "f32"
+                out_code = _CODE[y.dtype] if last else L.F32
+                calls.append(HipCall("dmlhip_reduce_" + sfx,
+                                     [I32(code), src, dst, I32(out_code), I64(outer), I64(r), I64(inner),
+                                      Workspace(2 * region), WorkspaceBytes(2 * region), Stream()],
+                                     bytes_moved=_nbytes(x, y) if first else 0, flops=0))
+            return _tasklet(node, state, calls, workspace_bytes=2 * region + scratch, bytes_moved=_nbytes(x, y),
+                            kind="reduce")
 
     _Reduce.__name__ = "Hip" + op_name
     _Reduce.__doc__ = doc
@@ -849,10 +897,10 @@ class HipMulReduceSum(ONNXForward):
         return _tasklet(node, state, [call], flops=2 * a.total_size, bytes_moved=2 * _nbytes(a), kind="reduce")
 
 
-HipReduceSum = _make_reduce("ReduceSum", L.RSUM, "ReduceSum (pure_implementations.py:294-296); adjacent axes.")
-HipReduceMax = _make_reduce("ReduceMax", L.RMAX, "ReduceMax (pure_implementations.py:299-301); adjacent axes.")
-HipReduceMin = _make_reduce("ReduceMin", L.RMIN, "ReduceMin (pure_implementations.py:304-306); adjacent axes.")
-HipReduceMean = _make_reduce("ReduceMean", L.RMEAN, "ReduceMean (pure_implementations.py:101-103); adjacent axes.")
+HipReduceSum = _make_reduce("ReduceSum", L.RSUM, "ReduceSum (pure_implementations.py:294-296).")
+HipReduceMax = _make_reduce("ReduceMax", L.RMAX, "ReduceMax (pure_implementations.py:299-301).")
+HipReduceMin = _make_reduce("ReduceMin", L.RMIN, "ReduceMin (pure_implementations.py:304-306).")
+HipReduceMean = _make_reduce("ReduceMean", L.RMEAN, "ReduceMean (pure_implementations.py:101-103).")
 
 
 @op_implementation(op="GlobalAveragePool", name=IMPL)

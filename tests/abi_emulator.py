@@ -77,6 +77,27 @@ def unary(op, x, y, n, param):
     y.reshape(-1)[:n] = r.astype(y.dtype)
 
 
+def binary(op, a, b, c, ndim, shape, a_strides, b_strides):
+    """dmlhip_binary_*: NumPy broadcasting expressed as per-dimension element strides (0 = broadcast); c is dense."""
+    shape = tuple(int(x) for x in shape[:ndim])
+    av = _view(a, 0, shape, [int(x) for x in a_strides[:ndim]]).astype(np.float64)
+    bv = _view(b, 0, shape, [int(x) for x in b_strides[:ndim]]).astype(np.float64)
+    r = {L.ADD: np.add, L.SUB: np.subtract, L.MUL: np.multiply, L.DIV: np.divide, L.POW: np.power}[op](av, bv)
+    n = int(np.prod(shape)) if shape else 1
+    c.reshape(-1)[:n] = r.reshape(-1).astype(c.dtype)
+
+
+def reduce(op, x, y, out_dtype, outer, r, inner):
+    """dmlhip_reduce_*: x viewed as [outer, r, inner] -> y [outer, inner]."""
+    xv = x.reshape(-1)[:outer * r * inner].astype(np.float64).reshape(outer, r, inner)
+    f = {L.RSUM: np.sum, L.RMAX: np.max, L.RMIN: np.min, L.RMEAN: np.mean}[op]
+    res = f(xv, axis=1) if r > 0 else np.zeros((outer, inner))
+    want = np.float16 if out_dtype == L.F16 else np.float32
+    if y.dtype != want:
+        raise TypeError("reduce output is %s, out_dtype says %s" % (y.dtype, want))
+    y.reshape(-1)[:outer * inner] = res.reshape(-1).astype(want)
+
+
 class Emulator:
     """Runs the calls of a HipTasklet on NumPy arrays bound to its connectors."""
     def __init__(self, workspace_bytes):
@@ -101,6 +122,20 @@ class Emulator:
                 x = self._typed(x, want)
                 y = self._typed(y, want)
                 unary(op, x, y, n, param)
+            elif call.symbol in ("dmlhip_binary_f16", "dmlhip_binary_f32"):
+                op, a, b, c, ndim, shape, sa, sb = args[:8]
+                binary(op, a, b, c, ndim, shape, sa, sb)
+            elif call.symbol in ("dmlhip_reduce_f16", "dmlhip_reduce_f32"):
+                op, x, y, out_dtype, outer, r, inner = args[:7]
+                x = self._typed(x, np.float16 if call.symbol.endswith("f16") else np.float32)
+                y = self._typed(y, np.float16 if out_dtype == L.F16 else np.float32)
+                reduce(op, x, y, out_dtype, outer, r, inner)
+            elif call.symbol in ("dmlhip_softmax_backward_f16", "dmlhip_softmax_backward_f32"):
+                yv, dy, dx, rows, cols = args[:5]
+                y64 = yv.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+                d64 = dy.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+                p = y64 * d64
+                dx.reshape(-1)[:rows * cols] = (p - y64 * p.sum(-1, keepdims=True)).reshape(-1).astype(dx.dtype)
             else:
                 raise NotImplementedError("no emulation of %s" % call.symbol)
 
@@ -119,6 +154,8 @@ class Emulator:
             return int(a.value)
         if isinstance(a, T.F32):
             return float(a.value)
+        if isinstance(a, T.I64Array):
+            return tuple(a.values)
         if isinstance(a, T.Struct):
             return a.value
         if isinstance(a, T.Workspace):
