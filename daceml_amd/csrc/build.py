@@ -22,6 +22,7 @@ SOURCES = [
     "transpose.hip",
     "gemm_f16.hip",
     "gemm_f16_pipe.hip",
+    "gemm_f16_pipe_ilv.hip",
     "gemm_f32.hip",
     "conv.hip",
     "conv_fused.hip", "conv_backward.hip", "conv_implicit.hip",

@@ -1,0 +1,21 @@
+// The interleaved-loop configurations of the pipelined fp16 GEMM kernel (gemm_f16_pipe.h), a translation unit of their
+// own so that they compile beside the others.
+#include "gemm_f16_pipe.h"
+
+namespace dml {
+namespace gemm16 {
+
+int launch_pipelined_ilv(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, const void* bias, const void* residual,
+                         void* pre, int ak, int bk, int cfg, long long batch, hipStream_t st) {
+    switch (cfg) {
+        case 4: return launch_tile<256, 256, 128, 128, 2, false, false, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+        case 5: return launch_tile<128, 128, 64, 64, 4, false, false, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+        case 6: return launch_tile<256, 128, 128, 64, 3, false, false, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+        default:
+            set_error("gemm_f16: %d is not an interleaved-loop configuration", cfg);
+            return DMLHIP_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace gemm16
+}  // namespace dml
