@@ -4,6 +4,12 @@
 // Fragment reads are inline assembly so that the compiler neither guesses at aliasing between them
 // and the in-flight global->LDS transfers (it would wait for *all* transfers before a transpose
 // read) nor places the waits: the kernels wait explicitly on the lgkmcnt / vmcnt counters.
+//
+// The price: the compiler takes a read's destination registers to be written when the instruction issues, not when
+// the data arrives. Every value returned by lds_read_* must therefore be consumed, after a wait that covers it, on
+// every path that issued the read. A result left unused has no live range, its registers go to the next value the
+// compiler needs (a global address, say), and the LDS data lands on top of that value later. tests/test_isa_hazards.py
+// checks the compiled kernels for this.
 #pragma once
 
 #include "common.h"
