@@ -346,6 +346,37 @@ def test_bert_layer_matches_huggingface_bertlayer():
     np.testing.assert_allclose(OB.forward(x, p, heads, eps=cfg.layer_norm_eps), out.numpy(), rtol=1e-9, atol=1e-11)
 
 
+@pytest.mark.parametrize("b,s,h,heads,ffn", [(2, 12, 32, 4, 64), (1, 77, 96, 3, 200), (3, 130, 64, 1, 48)])
+def test_cpp_loop_nests_match_the_numpy_statements(b, s, h, heads, ffn):
+    """oracle/bert_layer_loops.cpp (fp32 C++ / OpenMP loops, the CPU baseline that bench.py times) against
+    oracle/bert_layer.py in fp64: output and all 17 gradients. The sizes leave ragged edges in every blocked loop (rows
+    not a multiple of 4, columns not of 16, K not of 256) and cross one block boundary in each dimension."""
+    import shutil
+    if shutil.which("g++") is None:
+        pytest.skip("no g++")
+    from oracle import bert_layer_loops as OL
+    p = OB.init_params(h, ffn, 5, np.float64, bias_std=0.1)
+    r = rng(45)
+    for n in ("q_w", "k_w", "v_w", "o_w", "ffn1_w", "ffn2_w"):
+        p[n] = p[n] * 8  # weights large enough that attention is far from uniform
+    p["ln1_g"], p["ln2_g"] = r.uniform(0.5, 1.5, h), r.uniform(0.5, 1.5, h)
+    p["ln1_b"], p["ln2_b"] = r.standard_normal(h) * 0.1, r.standard_normal(h) * 0.1
+    x, dy = r.standard_normal((b, s, h)), r.standard_normal((b, s, h))
+    y, saved = OB.forward(x, p, heads, eps=1e-5, keep=True)
+    want = OB.backward(x, p, heads, dy, saved, eps=1e-5)
+    y32, got = OL.forward_backward(x, p, heads, dy, eps=1e-5)
+    assert y32.dtype == np.float32
+    np.testing.assert_allclose(y32, y, rtol=1e-4, atol=1e-5)
+    for n in ["x"] + OB.PARAM_NAMES:
+        scale = max(1.0, float(np.abs(want[n]).max()))
+        np.testing.assert_allclose(got[n], want[n], rtol=1e-4, atol=2e-5 * scale, err_msg=n)
+    # forward only (no dy): same output, no gradients
+    y_only, none = OL.forward_backward(x, p, heads, eps=1e-5)
+    assert none is None and np.array_equal(y_only, y32)
+    with pytest.raises(ValueError):
+        OL.forward_backward(x, p, heads + 1 if h % (heads + 1) else h + 1, dy)
+
+
 def test_batchnorm_matches_torch_running_stats_and_autograd():
     """Training form against F.batch_norm(training=True): output, saved statistics, autograd gradients; the running
     variance through torch's own update rule (torch blends the UNBIASED variance with weight 1 - momentum_onnx;
