@@ -266,7 +266,6 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
 
     int cur_stage = 0;
     if constexpr (ILV) {
-        static_assert(!ASUM, "the interleaved loop carries no row sums");
         constexpr int NM = TM * TN;                   // MFMAs per K sub-step
         constexpr int NU = TM + TN;                   // fragments to fetch per K sub-step
         // fragments requested after one MFMA: all of them within the first half of the sub-step's MFMAs, so that the
@@ -280,11 +279,14 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
         constexpr int NA = BM / 32;
         static_assert(LPT <= DSLOTS, "more transfers than MFMA slots to put them behind");
         // One K step. FILL: the ring is still being refilled (every step but the last NSTAGE-1), so the transfers are
-        // issued unconditionally and a next tile always exists; the tail steps are a second copy of the body without
-        // them - no per-slot branches in either.
+        // issued unconditionally. MORE: another step follows, whose first fragments are requested during this step's
+        // last sub-step. Three copies of the body (filling; draining; the very last step) and no per-slot branches in
+        // any of them.
         int kt = 0;
-        auto step = [&](auto fill_c) {
+        auto step = [&](auto fill_c, auto more_c) {
             constexpr bool FILL = decltype(fill_c)::value;
+            constexpr bool MORE = decltype(more_c)::value;
+            static_assert(MORE || !FILL, "a step that refills the ring is never the last");
             const uint32_t cur_off = (uint32_t)cur_stage * STAGE;
             const int nxt_stage = cur_stage + 1 == NSTAGE ? 0 : cur_stage + 1;
             const uint32_t nxt_off = (uint32_t)nxt_stage * STAGE;
@@ -294,7 +296,6 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
             const _Float16* const fill_b = KSUM ? fb : B;
             const int fill_k = (KSUM ? fk : kt + NSTAGE - 1) * BK;
             if constexpr (KSUM && FILL) advance();
-            const bool more = FILL || kt + 1 < nk;
             static_for<0, BK / 16>([&](auto kc) {
                 constexpr int kk = decltype(kc)::value;
                 constexpr int nb = (kk + 1) & 1;
@@ -318,11 +319,9 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
                         if constexpr (!last) {
                             if constexpr (u < TM) sa.template frag_one<kk + 1, u>(cur_off, af[nb][u]);
                             else sb.template frag_one<kk + 1, u - TM>(cur_off, bf[nb][u - TM]);
-                        } else {
-                            if (more) {
-                                if constexpr (u < TM) sa.template frag_one<0, u>(nxt_off, af[nb][u]);
-                                else sb.template frag_one<0, u - TM>(nxt_off, bf[nb][u - TM]);
-                            }
+                        } else if constexpr (MORE) {
+                            if constexpr (u < TM) sa.template frag_one<0, u>(nxt_off, af[nb][u]);
+                            else sb.template frag_one<0, u - TM>(nxt_off, bf[nb][u - TM]);
                         }
                     });
                     if constexpr (FILL && kk < DSUB) {
@@ -336,11 +335,31 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 });
+                if constexpr (ASUM) {
+                    // as in the plain loop below: the two wavefronts that share these A rows take alternate sub-steps
+                    // (the fragments of this sub-step stay untouched until the reads of sub-step kk + 2 are issued)
+                    if (asum_parity == (kk & 1)) {
+                        const half2v one2 = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+                        for (int i = 0; i < TM; ++i) {
+                            const half8 f = af[kk & 1][i];
+#pragma unroll
+                            for (int e = 0; e < 8; e += 2) {
+                                const half2v p = {f[e], f[e + 1]};
+                                acc_sum[i] = __builtin_amdgcn_fdot2(p, one2, acc_sum[i], false);
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             });
             cur_stage = nxt_stage;
         };
-        for (; kt + NSTAGE - 1 < nk; ++kt) step(std::true_type{});
-        for (; kt < nk; ++kt) step(std::false_type{});
+        for (; kt + NSTAGE - 1 < nk; ++kt) step(std::true_type{}, std::true_type{});
+        if constexpr (NSTAGE > 2) {
+            for (; kt + 1 < nk; ++kt) step(std::false_type{}, std::true_type{});
+        }
+        step(std::false_type{}, std::false_type{});  // kt == nk - 1 (the host passes k >= one K step)
     } else {
         for (int kt = 0; kt < nk; ++kt) {
             const uint32_t cur_off = (uint32_t)cur_stage * STAGE;
