@@ -135,6 +135,9 @@ SIGNATURES = {
     "dmlhip_attention_backward_workspace_bytes": (c_size_t, [POINTER(AttentionDesc)]),
     "dmlhip_attention_backward_f16": (c_int, [POINTER(AttentionDesc), POINTER(AttentionDesc), _P, _P, _P, _P, _P, _P, _P,
                                               _P, _P, _P, c_size_t, _P]),
+    "dmlhip_attention_masked_f16": (c_int, [POINTER(AttentionDesc), _P, _P, _P, _P, _I64P, _P, _P, _P]),
+    "dmlhip_attention_masked_backward_f16": (c_int, [POINTER(AttentionDesc), POINTER(AttentionDesc), _P, _P, _P, _P, _I64P,
+                                                     _P, _P, _P, _P, _P, _P, _P, c_size_t, _P]),
     # diagnostics (switches for tests and measurements, declared at the end of the header)
     "dmlhip_conv2d_expand_depthwise_lds_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "dmlhip_debug_force_gemm_config": (None, [c_int]),

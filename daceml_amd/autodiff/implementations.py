@@ -219,7 +219,8 @@ class HipSoftmaxBackward(BackwardImplementation):
 @autoregister_params(op="FusedAttention", name=NAME)
 class HipFusedAttentionBackward(BackwardImplementation):
     """One FusedAttentionGrad node; the forward node is made to emit its log-sum-exp rows, which replace the
-    probability matrix that DefaultSoftmaxBackward (onnx_ops.py:237-275) would forward."""
+    probability matrix that DefaultSoftmaxBackward (onnx_ops.py:237-275) would forward. An additive mask is a
+    constant of the node: it is forwarded to the gradient node and gets no gradient of its own."""
     @staticmethod
     def backward_can_be_applied(node, state, sdfg) -> bool:
         return True
@@ -234,7 +235,10 @@ class HipFusedAttentionBackward(BackwardImplementation):
         g = _new(context, "FusedAttentionGrad", forward_node.label + "_backward", scale=forward_node.scale,
                  q_perm=forward_node.q_perm, k_perm=forward_node.k_perm, v_perm=forward_node.v_perm,
                  o_perm=forward_node.o_perm)
-        for conn in ("Q", "K", "V"):
+        if "Mask" in required_gradients:
+            raise AutoDiffException("%s: no gradient is produced for the attention mask" % forward_node.label)
+        has_mask = any(e.dst_conn == "Mask" for e in context.forward_state.in_edges(forward_node))
+        for conn in ("Q", "K", "V") + (("Mask", ) if has_mask else ()):
             connect_input_from_forward(forward_node, g, context, conn)
         connect_output_from_forward(forward_node, g, context, "Output", "O")
         _read(context, lse, g, "LogSumExp")

@@ -1,9 +1,11 @@
 // Fused scaled-dot-product attention for fp16 tensors with head dimension 64:
-//     O = softmax(scale * Q K^T) V          (no mask, no dropout; softmax over the key axis)
+//     O = softmax(scale * Q K^T [+ mask]) V          (no dropout; softmax over the key axis)
 // without materialising the [Sq, Sk] score matrix in HBM, and its backward pass. It replaces the chain
-// Einsum(Q,K) -> Mul/Div(scale) -> Softmax(axis=-1) -> Einsum(P,V) of the reference
-// (daceml/onnx/op_implementations/pure_implementations.py:219-252, 309-319) and, in backward, the nodes
-// emitted by daceml/autodiff/implementations/onnx_ops.py:25-138 and :237-275 for that chain.
+// Einsum(Q,K) -> Mul/Div(scale) [-> Add(mask)] -> Softmax(axis=-1) -> Einsum(P,V) of the reference
+// (daceml/onnx/op_implementations/pure_implementations.py:219-252, 34-36, 309-319) and, in backward, the nodes
+// emitted by daceml/autodiff/implementations/onnx_ops.py:25-138 and :237-275 for that chain. The optional additive
+// mask is one fp16 row of seq_k values per (batch0, batch1), the same for every query (the padding mask of a BERT
+// encoder, [batch, 1, 1, keys]); the kernels without it are separate instantiations.
 //
 // Work decomposition (forward): a workgroup of four wavefronts owns 128 query rows of one (batch, head);
 // each wavefront owns 32 of them. K and V stream through a three-stage LDS ring in tiles of 64 keys
@@ -28,6 +30,7 @@ namespace dml {
 namespace {
 
 constexpr int kAttnThreads = 256;
+constexpr float kLog2eF = 1.44269504088896340736f;
 constexpr int kTileBytes = 64 * 128;  // one [64][64] fp16 tile
 
 struct AttnArgs {
@@ -37,6 +40,13 @@ struct AttnArgs {
     int64_t dqs[3], dks[3], dvs[3], dos[3];   // gradient tensors (backward only)
     float scale, scale_log2;
 };
+
+// the additive mask: row (b0, b1) starts at mask + b0 * ms[0] + b1 * ms[1] (a stride of 0 broadcasts), keys contiguous
+struct AttnArgsMasked : AttnArgs {
+    const _Float16* mask;
+    int64_t ms[2];
+};
+template <bool MASK> using AttnArgsFor = std::conditional_t<MASK, AttnArgsMasked, AttnArgs>;
 
 template <int I, int N, typename F>
 __device__ __forceinline__ void static_for_attn(F&& f) {
@@ -99,6 +109,22 @@ __device__ __forceinline__ float other_half(float v) {
 __device__ __forceinline__ float cross_half_max(float v) { return fmaxf(v, other_half(v)); }
 __device__ __forceinline__ float cross_half_sum(float v) { return v + other_half(v); }
 
+// The mask values of the 32 keys a lane holds of key tile j in the forward and dQ kernels, as loaded:
+// mk[blk * 4 + g][e] belongs to key 64*j + 32*blk + 8*g + 4*h + e. Whole tiles are read eight bytes at a time (the host
+// checks the alignment); the last, partial tile element by element with the index clamped to the row.
+__device__ __forceinline__ void load_mask_tile(const _Float16* row, int j, int h, int seq_k, half4v (&mk)[8]) {
+    const int base = j * 64 + h * 4;
+    if ((j + 1) * 64 <= seq_k) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) mk[i] = *reinterpret_cast<const half4v*>(row + base + (i >> 2) * 32 + (i & 3) * 8);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) mk[i][e] = row[min(base + (i >> 2) * 32 + (i & 3) * 8 + e, seq_k - 1)];
+    }
+}
+
 __device__ __forceinline__ void decode_block(const AttnArgs& a, int tiles, long long& bid, int& b0, int& b1, int& tile) {
     // XCD-aware: consecutive tiles of one (batch, head) share K/V (or Q/dO) and should share an L2
     const long long total = a.total_blocks;
@@ -138,11 +164,13 @@ __device__ __forceinline__ void store_rows_t(const floatx16 (&acc)[2], float mul
 // ---------------------------------------------------------------- forward
 constexpr int kFwdStages = 3;
 
+template <bool MASK>
 __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _Float16* __restrict__ q_ptr,
                                                                         const _Float16* __restrict__ k_ptr,
                                                                         const _Float16* __restrict__ v_ptr,
                                                                         _Float16* __restrict__ o_ptr,
-                                                                        float* __restrict__ lse_ptr, const AttnArgs a) {
+                                                                        float* __restrict__ lse_ptr,
+                                                                        const AttnArgsFor<MASK> a) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     constexpr int STAGE = 2 * kTileBytes;
     long long bid = blockIdx.x;
@@ -156,6 +184,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
     const _Float16* Q = q_ptr + b0 * a.qs[0] + b1 * a.qs[1];
     const _Float16* K = k_ptr + b0 * a.ks[0] + b1 * a.ks[1];
     const _Float16* V = v_ptr + b0 * a.vs[0] + b1 * a.vs[1];
+    const _Float16* mask_row = nullptr;
+    if constexpr (MASK) mask_row = a.mask + b0 * a.ms[0] + b1 * a.ms[1];
 
     // Q fragments (B operand of S^T = K Q^T): lane -> query row lane%32, head elements 16*st + 8*h .. +7
     half8 qf[4];
@@ -194,6 +224,9 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
         if (j + 1 < nk) wait_vm_lgkm0<4>();
         else wait_vm_lgkm0<0>();
         __builtin_amdgcn_s_barrier();
+        // ahead of the refill below, so that waiting for these loads does not wait for the transfers issued after them
+        half4v mk[MASK ? 8 : 1];
+        if constexpr (MASK) load_mask_tile(mask_row, j, h, a.seq_k, mk);
         // every wavefront has finished tile j-1: its stage takes tile j+2
         if (j + kFwdStages - 1 < nk) {
             const int fs = stage == 0 ? kFwdStages - 1 : stage - 1;
@@ -243,6 +276,14 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
         // shift of the exponent's argument are one fused multiply-add per score)
         float mt = -INFINITY;
         const bool ragged = (j + 1) * 64 > a.seq_k;
+        if constexpr (MASK) {
+            // the mask shifts every score by its own amount: scale and shift first, then the maximum
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    sacc[blk][e] = __builtin_fmaf(sacc[blk][e], a.scale_log2, (float)mk[blk * 4 + (e >> 2)][e & 3] * kLog2eF);
+        }
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
@@ -254,8 +295,10 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
                 mt = fmaxf(mt, sacc[blk][e]);
             }
         mt = cross_half_max(mt);
-        const float m_new = fmaxf(m_run, mt * a.scale_log2);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        const float m_new = fmaxf(m_run, MASK ? mt : mt * a.scale_log2);
+        // a mask may hold -inf for every key seen so far: keep the exponents' arguments free of (-inf) - (-inf)
+        const float m_use = MASK && m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
         m_run = m_new;
         float psum = 0.f;
         half8 pf[4];
@@ -263,7 +306,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], a.scale_log2, -m_new));
+                const float p = MASK ? __builtin_amdgcn_exp2f(sacc[blk][e] - m_use)
+                                     : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], a.scale_log2, -m_new));
                 psum += p;
                 pf[blk * 2 + (e >> 3)][e & 7] = (_Float16)p;
             }
@@ -323,10 +367,11 @@ __device__ __forceinline__ half8 tr_pair(uint32_t lo_addr, uint32_t hi_addr) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+template <bool MASK>
 __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
     const _Float16* __restrict__ q_ptr, const _Float16* __restrict__ k_ptr, const _Float16* __restrict__ v_ptr,
     const _Float16* __restrict__ o_ptr, const float* __restrict__ lse_ptr, const _Float16* __restrict__ do_ptr,
-    _Float16* __restrict__ dq_ptr, float* __restrict__ dvec_ptr, const AttnArgs a) {
+    _Float16* __restrict__ dq_ptr, float* __restrict__ dvec_ptr, const AttnArgsFor<MASK> a) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     constexpr int STAGE = 2 * kTileBytes;
     long long bid = blockIdx.x;
@@ -341,6 +386,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
 
     const _Float16* K = k_ptr + b0 * a.ks[0] + b1 * a.ks[1];
     const _Float16* V = v_ptr + b0 * a.vs[0] + b1 * a.vs[1];
+    const _Float16* mask_row = nullptr;
+    if constexpr (MASK) mask_row = a.mask + b0 * a.ms[0] + b1 * a.ms[1];
 
     half8 qf[4], dof[4];
     float dsum = 0.f;
@@ -386,6 +433,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
         if (j + 1 < nk) wait_vm_lgkm0<4>();
         else wait_vm_lgkm0<0>();
         __builtin_amdgcn_s_barrier();
+        half4v mk[MASK ? 8 : 1];   // ahead of the refill, as in the forward kernel
+        if constexpr (MASK) load_mask_tile(mask_row, j, h, a.seq_k, mk);
         if (j + kBwdStages - 1 < nk) {
             const int fs = stage == 0 ? kBwdStages - 1 : stage - 1;
             dma.issue(K, a.ks[2], (j + kBwdStages - 1) * 64, kmax, lds + fs * STAGE, wave);
@@ -433,7 +482,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                float p = __builtin_amdgcn_exp2f(sacc[blk][e] * a.scale_log2 - lse2);
+                float p;
+                if constexpr (MASK)
+                    p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], a.scale_log2,
+                                                              (float)mk[blk * 4 + (e >> 2)][e & 3] * kLog2eF) - lse2);
+                else
+                    p = __builtin_amdgcn_exp2f(sacc[blk][e] * a.scale_log2 - lse2);
                 if (ragged) {
                     const int key = j * 64 + blk * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
                     if (key >= a.seq_k) p = 0.f;
@@ -453,10 +507,11 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
     store_rows_t(dqacc, a.scale, lds + wave * 4096, dq_ptr + b0 * a.dqs[0] + b1 * a.dqs[1], a.dqs[2], q0, a.seq_q, lane);
 }
 
+template <bool MASK>
 __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dkv_kernel(
     const _Float16* __restrict__ q_ptr, const _Float16* __restrict__ k_ptr, const _Float16* __restrict__ v_ptr,
     const float* __restrict__ lse_ptr, const float* __restrict__ dvec_ptr, const _Float16* __restrict__ do_ptr,
-    _Float16* __restrict__ dk_ptr, _Float16* __restrict__ dv_ptr, const AttnArgs a) {
+    _Float16* __restrict__ dk_ptr, _Float16* __restrict__ dv_ptr, const AttnArgsFor<MASK> a) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     constexpr int STAGE = 2 * kTileBytes + 512;  // Q tile, dO tile, 64 lse, 64 D
     long long bid = blockIdx.x;
@@ -473,6 +528,10 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dkv_kernel(
     const _Float16* G = do_ptr + b0 * a.dos[0] + b1 * a.dos[1];
     const float* LSE = lse_ptr + bh * a.seq_q;
     const float* DV = dvec_ptr + bh * a.seq_q;
+
+    // this lane's key row carries one mask value, whatever the query
+    float mask2 = 0.f;
+    if constexpr (MASK) mask2 = (float)a.mask[b0 * a.ms[0] + b1 * a.ms[1] + krow] * kLog2eF;
 
     // K and V fragments of this lane's key row (B operands)
     half8 kfr[4], vfr[4];
@@ -558,7 +617,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dkv_kernel(
             half8 pf[2], dsf[2];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                float p = __builtin_amdgcn_exp2f(sacc[e] * a.scale_log2 - lv[e >> 2][e & 3] * kLog2e);
+                float p = MASK ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[e], a.scale_log2, mask2) - lv[e >> 2][e & 3] * kLog2e)
+                               : __builtin_amdgcn_exp2f(sacc[e] * a.scale_log2 - lv[e >> 2][e & 3] * kLog2e);
                 if (ragged) {
                     const int qi = j * 64 + qb * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
                     if (qi >= a.seq_q) p = 0.f;
@@ -616,6 +676,87 @@ int fill_args(const dmlhip_attention_desc* d, const dmlhip_attention_desc* g, At
     return 0;
 }
 
+// `m` = the arguments with the mask row pointer and strides added (checked here)
+int fill_mask(const AttnArgs& a, const void* mask, const int64_t* ms, AttnArgsMasked& m, const char* what) {
+    DML_REQUIRE(reinterpret_cast<uintptr_t>(mask) % 8 == 0, DMLHIP_ERR_ALIGN, "%s: the mask must be 8-byte aligned", what);
+    DML_REQUIRE(ms[0] >= 0 && ms[1] >= 0 && ms[0] % 4 == 0 && ms[1] % 4 == 0, DMLHIP_ERR_ALIGN,
+                "%s: mask strides must be non-negative multiples of 4 elements (0 = broadcast)", what);
+    static_cast<AttnArgs&>(m) = a;
+    m.mask = static_cast<const _Float16*>(mask);
+    m.ms[0] = ms[0];
+    m.ms[1] = ms[1];
+    return 0;
+}
+
+int attention_forward(const dmlhip_attention_desc* d, const void* q, const void* k, const void* v, const void* mask,
+                      const int64_t* ms, void* o, void* lse, void* stream, const char* what) {
+    AttnArgs a = {};
+    if (int e = fill_args(d, nullptr, a, what)) return e;
+    const long long bh = (long long)d->batch[0] * d->batch[1];
+    if (bh == 0 || d->seq_q == 0) return 0;
+    DML_REQUIRE(q && k && v && o, DMLHIP_ERR_NULL, "%s: NULL tensor pointer", what);
+    DML_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o), DMLHIP_ERR_ALIGN,
+                "%s: tensors must be 16-byte aligned", what);
+    a.total_blocks = bh * a.q_tiles;
+    DML_REQUIRE(a.total_blocks <= 2147483647LL, DMLHIP_ERR_SHAPE, "%s: too many workgroups", what);
+    if (mask) {
+        AttnArgsMasked m;
+        if (int e = fill_mask(a, mask, ms, m, what)) return e;
+        hipLaunchKernelGGL(attention_fwd_kernel<true>, (unsigned)a.total_blocks, kAttnThreads, kFwdStages * 2 * kTileBytes,
+                           (hipStream_t)stream, (const _Float16*)q, (const _Float16*)k, (const _Float16*)v, (_Float16*)o,
+                           (float*)lse, m);
+    } else {
+        hipLaunchKernelGGL(attention_fwd_kernel<false>, (unsigned)a.total_blocks, kAttnThreads, kFwdStages * 2 * kTileBytes,
+                           (hipStream_t)stream, (const _Float16*)q, (const _Float16*)k, (const _Float16*)v, (_Float16*)o,
+                           (float*)lse, a);
+    }
+    return launch_status(what);
+}
+
+int attention_backward(const dmlhip_attention_desc* d, const dmlhip_attention_desc* grad, const void* q, const void* k,
+                       const void* v, const void* mask, const int64_t* ms, const void* o, const void* lse, const void* d_o,
+                       void* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream, const char* what) {
+    AttnArgs a = {};
+    DML_REQUIRE(grad, DMLHIP_ERR_NULL, "%s: NULL gradient descriptor", what);
+    if (int e = fill_args(d, grad, a, what)) return e;
+    const long long bh = (long long)d->batch[0] * d->batch[1];
+    if (bh == 0 || (d->seq_q == 0 && d->seq_k == 0)) return 0;
+    DML_REQUIRE(d->seq_q > 0, DMLHIP_ERR_SHAPE, "%s: no query rows but %lld key rows", what, (long long)d->seq_k);
+    DML_REQUIRE(q && k && v && o && lse && d_o && dq && dk && dv, DMLHIP_ERR_NULL, "%s: NULL tensor pointer", what);
+    DML_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) && aligned16(d_o) && aligned16(dq) &&
+                    aligned16(dk) && aligned16(dv),
+                DMLHIP_ERR_ALIGN, "%s: tensors must be 16-byte aligned", what);
+    const size_t need = dmlhip_attention_backward_workspace_bytes(d);
+    DML_REQUIRE(workspace && workspace_bytes >= need, DMLHIP_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given",
+                what, need, workspace_bytes);
+    AttnArgsMasked m;
+    if (mask)
+        if (int e = fill_mask(a, mask, ms, m, what)) return e;
+    hipStream_t st = (hipStream_t)stream;
+    const long long dq_blocks = bh * a.q_tiles, dkv_blocks = bh * ((a.seq_k + 127) / 128);
+    DML_REQUIRE(dq_blocks <= 2147483647LL && dkv_blocks <= 2147483647LL, DMLHIP_ERR_SHAPE, "%s: too many workgroups", what);
+    a.total_blocks = m.total_blocks = dq_blocks;
+    if (mask)
+        hipLaunchKernelGGL(attention_bwd_dq_kernel<true>, (unsigned)dq_blocks, kAttnThreads, kBwdStages * 2 * kTileBytes, st,
+                           (const _Float16*)q, (const _Float16*)k, (const _Float16*)v, (const _Float16*)o, (const float*)lse,
+                           (const _Float16*)d_o, (_Float16*)dq, (float*)workspace, m);
+    else
+        hipLaunchKernelGGL(attention_bwd_dq_kernel<false>, (unsigned)dq_blocks, kAttnThreads, kBwdStages * 2 * kTileBytes, st,
+                           (const _Float16*)q, (const _Float16*)k, (const _Float16*)v, (const _Float16*)o, (const float*)lse,
+                           (const _Float16*)d_o, (_Float16*)dq, (float*)workspace, a);
+    if (int e = launch_status(what)) return e;
+    a.total_blocks = m.total_blocks = dkv_blocks;
+    if (mask)
+        hipLaunchKernelGGL(attention_bwd_dkv_kernel<true>, (unsigned)dkv_blocks, kAttnThreads,
+                           kBwdStages * (2 * kTileBytes + 512), st, (const _Float16*)q, (const _Float16*)k, (const _Float16*)v,
+                           (const float*)lse, (const float*)workspace, (const _Float16*)d_o, (_Float16*)dk, (_Float16*)dv, m);
+    else
+        hipLaunchKernelGGL(attention_bwd_dkv_kernel<false>, (unsigned)dkv_blocks, kAttnThreads,
+                           kBwdStages * (2 * kTileBytes + 512), st, (const _Float16*)q, (const _Float16*)k, (const _Float16*)v,
+                           (const float*)lse, (const float*)workspace, (const _Float16*)d_o, (_Float16*)dk, (_Float16*)dv, a);
+    return launch_status(what);
+}
+
 }  // namespace
 }  // namespace dml
 
@@ -625,19 +766,13 @@ extern "C" {
 
 int dmlhip_attention_f16(const dmlhip_attention_desc* d, const void* q, const void* k, const void* v, void* o, void* lse,
                          void* stream) {
-    AttnArgs a = {};
-    if (int e = fill_args(d, nullptr, a, "attention")) return e;
-    const long long bh = (long long)d->batch[0] * d->batch[1];
-    if (bh == 0 || d->seq_q == 0) return 0;
-    DML_REQUIRE(q && k && v && o, DMLHIP_ERR_NULL, "attention: NULL tensor pointer");
-    DML_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o), DMLHIP_ERR_ALIGN,
-                "attention: tensors must be 16-byte aligned");
-    a.total_blocks = bh * a.q_tiles;
-    DML_REQUIRE(a.total_blocks <= 2147483647LL, DMLHIP_ERR_SHAPE, "attention: too many workgroups");
-    hipLaunchKernelGGL(attention_fwd_kernel, (unsigned)a.total_blocks, kAttnThreads, kFwdStages * 2 * kTileBytes,
-                       (hipStream_t)stream, (const _Float16*)q, (const _Float16*)k, (const _Float16*)v, (_Float16*)o,
-                       (float*)lse, a);
-    return launch_status("attention");
+    return attention_forward(d, q, k, v, nullptr, nullptr, o, lse, stream, "attention");
+}
+
+int dmlhip_attention_masked_f16(const dmlhip_attention_desc* d, const void* q, const void* k, const void* v,
+                                const void* mask, const int64_t* mask_stride, void* o, void* lse, void* stream) {
+    DML_REQUIRE(mask && mask_stride, DMLHIP_ERR_NULL, "attention_masked: NULL mask or mask strides");
+    return attention_forward(d, q, k, v, mask, mask_stride, o, lse, stream, "attention_masked");
 }
 
 size_t dmlhip_attention_backward_workspace_bytes(const dmlhip_attention_desc* d) {
@@ -648,33 +783,17 @@ size_t dmlhip_attention_backward_workspace_bytes(const dmlhip_attention_desc* d)
 int dmlhip_attention_backward_f16(const dmlhip_attention_desc* d, const dmlhip_attention_desc* grad, const void* q,
                                   const void* k, const void* v, const void* o, const void* lse, const void* d_o, void* dq,
                                   void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream) {
-    AttnArgs a = {};
-    DML_REQUIRE(grad, DMLHIP_ERR_NULL, "attention_backward: NULL gradient descriptor");
-    if (int e = fill_args(d, grad, a, "attention_backward")) return e;
-    const long long bh = (long long)d->batch[0] * d->batch[1];
-    if (bh == 0 || (d->seq_q == 0 && d->seq_k == 0)) return 0;
-    DML_REQUIRE(d->seq_q > 0, DMLHIP_ERR_SHAPE, "attention_backward: no query rows but %lld key rows",
-                (long long)d->seq_k);
-    DML_REQUIRE(q && k && v && o && lse && d_o && dq && dk && dv, DMLHIP_ERR_NULL, "attention_backward: NULL tensor pointer");
-    DML_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) && aligned16(d_o) && aligned16(dq) &&
-                    aligned16(dk) && aligned16(dv),
-                DMLHIP_ERR_ALIGN, "attention_backward: tensors must be 16-byte aligned");
-    const size_t need = dmlhip_attention_backward_workspace_bytes(d);
-    DML_REQUIRE(workspace && workspace_bytes >= need, DMLHIP_ERR_WORKSPACE,
-                "attention_backward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-    hipStream_t st = (hipStream_t)stream;
-    a.total_blocks = bh * a.q_tiles;
-    DML_REQUIRE(a.total_blocks <= 2147483647LL, DMLHIP_ERR_SHAPE, "attention_backward: too many workgroups");
-    hipLaunchKernelGGL(attention_bwd_dq_kernel, (unsigned)a.total_blocks, kAttnThreads, kBwdStages * 2 * kTileBytes, st,
-                       (const _Float16*)q, (const _Float16*)k, (const _Float16*)v, (const _Float16*)o, (const float*)lse,
-                       (const _Float16*)d_o, (_Float16*)dq, (float*)workspace, a);
-    if (int e = launch_status("attention_backward(dq)")) return e;
-    a.total_blocks = bh * ((a.seq_k + 127) / 128);
-    DML_REQUIRE(a.total_blocks <= 2147483647LL, DMLHIP_ERR_SHAPE, "attention_backward: too many workgroups");
-    hipLaunchKernelGGL(attention_bwd_dkv_kernel, (unsigned)a.total_blocks, kAttnThreads,
-                       kBwdStages * (2 * kTileBytes + 512), st, (const _Float16*)q, (const _Float16*)k, (const _Float16*)v,
-                       (const float*)lse, (const float*)workspace, (const _Float16*)d_o, (_Float16*)dk, (_Float16*)dv, a);
-    return launch_status("attention_backward(dk, dv)");
+    return attention_backward(d, grad, q, k, v, nullptr, nullptr, o, lse, d_o, dq, dk, dv, workspace, workspace_bytes,
+                              stream, "attention_backward");
+}
+
+int dmlhip_attention_masked_backward_f16(const dmlhip_attention_desc* d, const dmlhip_attention_desc* grad, const void* q,
+                                         const void* k, const void* v, const void* mask, const int64_t* mask_stride,
+                                         const void* o, const void* lse, const void* d_o, void* dq, void* dk, void* dv,
+                                         void* workspace, size_t workspace_bytes, void* stream) {
+    DML_REQUIRE(mask && mask_stride, DMLHIP_ERR_NULL, "attention_masked_backward: NULL mask or mask strides");
+    return attention_backward(d, grad, q, k, v, mask, mask_stride, o, lse, d_o, dq, dk, dv, workspace, workspace_bytes,
+                              stream, "attention_masked_backward");
 }
 
 }  // extern "C"

@@ -523,8 +523,19 @@ def _attn_desc(q, k, v, o, scale):
     return d
 
 
-def attention(q, k, v, scale, out=None, need_lse=True):
-    """softmax(scale * q k^T) v for [b0, b1, seq, 64] fp16 views (any batch / sequence strides). Returns (out, lse)."""
+def _attn_mask_strides(mask, q, k):
+    """Element strides over (batch0, batch1) of an additive mask broadcastable to [b0, b1, seq_q, seq_k] that does
+    not depend on the query: a [.., 1, seq_k] view with contiguous keys; size-1 batch dimensions broadcast."""
+    if mask.dtype != torch.float16 or mask.dim() != 4 or mask.shape[2] != 1 or mask.shape[3] != k.shape[2] or \
+            (mask.shape[3] > 1 and mask.stride(3) != 1) or any(mask.shape[i] not in (1, q.shape[i]) for i in (0, 1)):
+        raise ValueError("attention: the mask must be an fp16 [b0 | 1, b1 | 1, 1, seq_k] view with contiguous keys, got %s"
+                         % (tuple(mask.shape), ))
+    return (ctypes.c_int64 * 2)(*[0 if mask.shape[i] == 1 else int(mask.stride(i)) for i in (0, 1)])
+
+
+def attention(q, k, v, scale, out=None, need_lse=True, mask=None):
+    """softmax(scale * q k^T [+ mask]) v for [b0, b1, seq, 64] fp16 views (any batch / sequence strides); `mask` is
+    an additive [b0 | 1, b1 | 1, 1, seq_k] fp16 tensor. Returns (out, lse)."""
     _check(q, k, v, dtype=torch.float16)
     if k.shape[:2] != q.shape[:2] or v.shape[:3] != k.shape[:3] or k.shape[3] != q.shape[3] or v.shape[3] != q.shape[3]:
         raise ValueError("attention: incompatible shapes %s %s %s" % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
@@ -532,11 +543,16 @@ def attention(q, k, v, scale, out=None, need_lse=True):
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     lse = torch.empty(q.shape[:3], dtype=torch.float32, device=q.device) if need_lse else None
     d = _attn_desc(q, k, v, out, scale)
-    L.check(L.load().dmlhip_attention_f16(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _stream()))
+    if mask is None:
+        L.check(L.load().dmlhip_attention_f16(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _stream()))
+    else:
+        _check(mask, dtype=torch.float16)
+        L.check(L.load().dmlhip_attention_masked_f16(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(mask),
+                                                     _attn_mask_strides(mask, q, k), _ptr(out), _ptr(lse), _stream()))
     return out, lse
 
 
-def attention_backward(q, k, v, out, lse, dout, scale):
+def attention_backward(q, k, v, out, lse, dout, scale, mask=None):
     """Gradients (dq, dk, dv) of :func:`attention`; dense outputs."""
     _check(q, k, v, out, dout, dtype=torch.float16)
     dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), \
@@ -546,9 +562,16 @@ def attention_backward(q, k, v, out, lse, dout, scale):
     lib = L.load()
     need = lib.dmlhip_attention_backward_workspace_bytes(ctypes.byref(d))
     ws = workspace(need, q.device)
-    L.check(lib.dmlhip_attention_backward_f16(ctypes.byref(d), ctypes.byref(g), _ptr(q), _ptr(k), _ptr(v), _ptr(out),
-                                              _ptr(lse), _ptr(dout), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(),
-                                              _stream()))
+    if mask is None:
+        L.check(lib.dmlhip_attention_backward_f16(ctypes.byref(d), ctypes.byref(g), _ptr(q), _ptr(k), _ptr(v), _ptr(out),
+                                                  _ptr(lse), _ptr(dout), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(),
+                                                  _stream()))
+    else:
+        _check(mask, dtype=torch.float16)
+        L.check(lib.dmlhip_attention_masked_backward_f16(ctypes.byref(d), ctypes.byref(g), _ptr(q), _ptr(k), _ptr(v),
+                                                         _ptr(mask), _attn_mask_strides(mask, q, k), _ptr(out), _ptr(lse),
+                                                         _ptr(dout), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(),
+                                                         _stream()))
     return dq, dk, dv
 
 

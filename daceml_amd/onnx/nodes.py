@@ -133,9 +133,11 @@ SCHEMAS = [
             alpha=1.0, activation="none", accumulate=0),
     # Einsum(Q,K) [* scale] -> Softmax(last axis) -> Einsum(P,V) as one node (the scores never reach memory).
     # *_perm: which dimension of that tensor is (batch0, batch1, sequence, head); -1 for an absent batch dim.
-    _schema("FusedAttention", "Q K V", "Output LogSumExp?", since=1, scale=1.0, q_perm=REQUIRED, k_perm=REQUIRED,
+    # Mask: added to the scaled scores before the Softmax; broadcasts against [batch.., queries, keys] by the
+    # right-aligned rule of Add and must not vary with the query.
+    _schema("FusedAttention", "Q K V Mask?", "Output LogSumExp?", since=1, scale=1.0, q_perm=REQUIRED, k_perm=REQUIRED,
             v_perm=REQUIRED, o_perm=REQUIRED),
-    _schema("FusedAttentionGrad", "Q K V O LogSumExp dO", "dQ dK dV", since=1, scale=1.0, q_perm=REQUIRED,
+    _schema("FusedAttentionGrad", "Q K V O LogSumExp dO Mask?", "dQ dK dV", since=1, scale=1.0, q_perm=REQUIRED,
             k_perm=REQUIRED, v_perm=REQUIRED, o_perm=REQUIRED),
     # Conv 1x1 whose input is first multiplied by a per-image, per-channel factor Gate [n, c, 1, 1] (squeeze-excite)
     _schema("GatedConv", "X Gate W B?", "Y", since=1, auto_pad="NOTSET", dilations=None, group=1, kernel_shape=None,

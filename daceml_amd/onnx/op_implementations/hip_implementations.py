@@ -8,7 +8,7 @@ library behind an expansion — these play). ``forward_can_be_applied`` never ra
 what the kernels cover returns False.
 """
 import math
-from typing import List, Optional, Sequence
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -1350,6 +1350,29 @@ def _attn_ok(node, descs_perms) -> bool:
     return ext(k, kp, 2) == ext(v, vp, 2) and ext(q, qp, 2) == ext(o, op_, 2) and ext(k, kp, 2) > 0
 
 
+def attention_mask_strides(mask: Array, q: Array, k: Array, q_perm, k_perm) -> Optional[Tuple[int, int]]:
+    """Element strides of an additive mask over (batch0, batch1), or None when the kernels cannot take it. The mask
+    broadcasts against the scores [batch.., queries, keys] by Add's right-aligned rule (pure_implementations.py:34-36
+    is NumPy's); the kernels want fp16, one contiguous row of keys per batch entry and no dependence on the query."""
+    ext = [1 if q_perm[i] < 0 else q.shape[q_perm[i]] for i in (0, 1)] + [q.shape[q_perm[2]], k.shape[k_perm[2]]]
+    nd = 2 + sum(1 for i in (0, 1) if q_perm[i] >= 0)
+    if mask.dtype != torch.float16 or len(mask.shape) > nd:
+        return None
+    shape = [1] * (4 - len(mask.shape)) + list(mask.shape)
+    strides = [0] * (4 - len(mask.shape)) + list(mask.strides)
+    if shape[3] != ext[3] or (shape[3] > 1 and strides[3] != 1) or (shape[2] != 1 and ext[2] != 1):
+        return None
+    out = []
+    for i in (0, 1):
+        if shape[i] == 1:
+            out.append(0)
+        elif shape[i] == ext[i] and strides[i] % 4 == 0:
+            out.append(int(strides[i]))
+        else:
+            return None
+    return out[0], out[1]
+
+
 @op_implementation(op="FusedAttention", name=IMPL)
 class HipFusedAttention(ONNXForward):
     """softmax(scale * Q K^T) V in one kernel: the composition of PureEinsum (pure_implementations.py:219-252),
@@ -1366,6 +1389,8 @@ class HipFusedAttention(ONNXForward):
             ins, outs = _descs(node, state, sdfg)
             if not _attn_ok(node, HipFusedAttention._pairs(node, ins, outs)):
                 return False
+            if "Mask" in ins and attention_mask_strides(ins["Mask"], ins["Q"], ins["K"], node.q_perm, node.k_perm) is None:
+                return False
             lse = outs.get("LogSumExp")
             return lse is None or (lse.dtype == torch.float32 and lse.is_contiguous())
         except Exception:
@@ -1376,8 +1401,14 @@ class HipFusedAttention(ONNXForward):
         ins, outs = _descs(node, state, sdfg)
         pairs = HipFusedAttention._pairs(node, ins, outs)
         d = _attn_struct(pairs, ins["Q"], ins["K"], node.scale, node.q_perm, node.k_perm)
-        call = HipCall("dmlhip_attention_f16", [Struct(d, "dmlhip_attention_desc"), Ptr("Q"), Ptr("K"), Ptr("V"),
-                                                Ptr("Output"), _opt(node, state, "LogSumExp", False), Stream()])
+        if "Mask" in ins:
+            ms = attention_mask_strides(ins["Mask"], ins["Q"], ins["K"], node.q_perm, node.k_perm)
+            call = HipCall("dmlhip_attention_masked_f16",
+                           [Struct(d, "dmlhip_attention_desc"), Ptr("Q"), Ptr("K"), Ptr("V"), Ptr("Mask"), I64Array(ms),
+                            Ptr("Output"), _opt(node, state, "LogSumExp", False), Stream()])
+        else:
+            call = HipCall("dmlhip_attention_f16", [Struct(d, "dmlhip_attention_desc"), Ptr("Q"), Ptr("K"), Ptr("V"),
+                                                    Ptr("Output"), _opt(node, state, "LogSumExp", False), Stream()])
         bh = d.batch[0] * d.batch[1]
         return _tasklet(node, state, [call], flops=4 * bh * d.seq_q * d.seq_k * 64,
                         bytes_moved=_nbytes(ins["Q"], ins["K"], ins["V"], outs["Output"]), kind="attention")
@@ -1400,6 +1431,8 @@ class HipFusedAttentionGrad(ONNXForward):
             ins, outs = _descs(node, state, sdfg)
             fwd, grad = HipFusedAttentionGrad._pairs(node, ins, outs)
             lse = ins["LogSumExp"]
+            if "Mask" in ins and attention_mask_strides(ins["Mask"], ins["Q"], ins["K"], node.q_perm, node.k_perm) is None:
+                return False
             return _attn_ok(node, fwd) and _attn_ok(node, grad) and lse.dtype == torch.float32 and lse.is_contiguous()
         except Exception:
             return False
@@ -1412,10 +1445,17 @@ class HipFusedAttentionGrad(ONNXForward):
         d = _attn_struct(fwd, ins["Q"], ins["K"], node.scale, node.q_perm, node.k_perm)
         g = _attn_struct(grad, ins["Q"], ins["K"], node.scale, node.q_perm, node.k_perm)
         ws = L.load().dmlhip_attention_backward_workspace_bytes(ctypes.byref(d))
-        call = HipCall("dmlhip_attention_backward_f16",
-                       [Struct(d, "dmlhip_attention_desc"), Struct(g, "dmlhip_attention_desc"), Ptr("Q"), Ptr("K"),
-                        Ptr("V"), Ptr("O"), Ptr("LogSumExp"), Ptr("dO"), Ptr("dQ"), Ptr("dK"), Ptr("dV"), Workspace(),
-                        WorkspaceBytes(), Stream()])
+        if "Mask" in ins:
+            ms = attention_mask_strides(ins["Mask"], ins["Q"], ins["K"], node.q_perm, node.k_perm)
+            call = HipCall("dmlhip_attention_masked_backward_f16",
+                           [Struct(d, "dmlhip_attention_desc"), Struct(g, "dmlhip_attention_desc"), Ptr("Q"), Ptr("K"),
+                            Ptr("V"), Ptr("Mask"), I64Array(ms), Ptr("O"), Ptr("LogSumExp"), Ptr("dO"), Ptr("dQ"), Ptr("dK"),
+                            Ptr("dV"), Workspace(), WorkspaceBytes(), Stream()])
+        else:
+            call = HipCall("dmlhip_attention_backward_f16",
+                           [Struct(d, "dmlhip_attention_desc"), Struct(g, "dmlhip_attention_desc"), Ptr("Q"), Ptr("K"),
+                            Ptr("V"), Ptr("O"), Ptr("LogSumExp"), Ptr("dO"), Ptr("dQ"), Ptr("dK"), Ptr("dV"), Workspace(),
+                            WorkspaceBytes(), Stream()])
         bh = d.batch[0] * d.batch[1]
         return _tasklet(node, state, [call], workspace_bytes=ws, flops=8 * bh * d.seq_q * d.seq_k * 64,  # four contractions; the recomputed scores are not counted
                        

@@ -775,8 +775,10 @@ def _attention_roles(eq_scores: str, eq_context: str):
 
 
 def fuse_attention(sdfg: SDFG) -> int:
-    """Einsum(Q, K) with an optional folded scale -> Softmax over the keys -> Einsum(P, V) becomes one
-    FusedAttention node when neither the scores nor the probabilities are read by anything else."""
+    """Einsum(Q, K) with an optional folded scale [-> Add(mask)] -> Softmax over the keys -> Einsum(P, V) becomes one
+    FusedAttention node when neither the scores nor the probabilities are read by anything else. The mask (the
+    padding mask of a BERT encoder, [batch, 1, 1, keys]) becomes an input of the node when the kernels can take it:
+    fp16, constant along the queries; otherwise the chain stays as it is."""
     count = 0
     for state in sdfg.states():
         for sm in [n for n in state.nodes() if _is_op(n, "Softmax")]:
@@ -789,11 +791,29 @@ def fuse_attention(sdfg: SDFG) -> int:
             if prod is None or len(cons) != 1 or cons[0][1] != "Inputs__0":
                 continue
             es, ctx = prod[0], cons[0][0]
+            add, mask = None, None
+            if _is_op(es, "Add"):
+                # scores + mask in either operand order; the scores are the operand a contraction produces and nobody
+                # else reads, the mask is whatever the other operand is
+                add = es
+                for sc, mc in (("A", "B"), ("B", "A")):
+                    sarr = _in_array(state, add, sc)
+                    p2 = _producer(state, sarr)
+                    if p2 is not None and (_is_op(p2[0], "Einsum") or _is_op(p2[0], "FusedEinsum")) \
+                            and _internal(sdfg, state, sarr) and tuple(sdfg.arrays[sarr].shape) == tuple(sdfg.arrays[x].shape):
+                        es, mask = p2[0], _in_array(state, add, mc)
+                        break
+                if mask is None:
+                    continue
             if not (_is_op(es, "Einsum") or _is_op(es, "FusedEinsum")) or not _is_op(ctx, "Einsum"):
                 continue
             scale = 1.0
             if _is_op(es, "FusedEinsum"):
                 conns = {e.dst_conn for e in state.in_edges(es)} | {e.src_conn for e in state.out_edges(es)}
+                if "Bias" in conns and mask is None:
+                    # a mask of a single batch entry is a vector over the keys: the bias-folding pass has taken it
+                    mask = _in_array(state, es, "Bias")
+                    conns.discard("Bias")
                 if conns - {"Inputs__0", "Inputs__1", "Output"} or es.activation != "none" or es.accumulate:
                     continue
                 scale = float(es.alpha)
@@ -811,13 +831,22 @@ def fuse_attention(sdfg: SDFG) -> int:
                 if d.dtype != torch.float16 or d.shape[pm[3]] != 64 or d.strides[pm[3]] != 1 \
                         or any(d.strides[i] % 8 for i in pm[:3] if i >= 0):
                     ok = False
+            if mask is not None:
+                from ..onnx.op_implementations.hip_implementations import attention_mask_strides
+                if attention_mask_strides(sdfg.arrays[mask], sdfg.arrays[qa], sdfg.arrays[ka], q_perm, k_perm) is None:
+                    ok = False
             if not ok:
                 continue
             label = ctx.label + "_attention"
             _remove_node(state, es)
+            if add is not None:
+                _remove_node(state, add)
             _remove_node(state, sm)
             _remove_node(state, ctx)
-            _add_node(sdfg, state, "FusedAttention", label, {"Q": qa, "K": ka, "V": va}, {"Output": oa}, scale=scale,
+            ins = {"Q": qa, "K": ka, "V": va}
+            if mask is not None:
+                ins["Mask"] = mask
+            _add_node(sdfg, state, "FusedAttention", label, ins, {"Output": oa}, scale=scale,
                       q_perm=q_perm, k_perm=k_perm, v_perm=v_perm, o_perm=o_perm)
             count += 1
     if count:

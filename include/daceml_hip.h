@@ -330,7 +330,8 @@ int dmlhip_conv2d_backward_weight_f32(const dmlhip_conv2d_desc* d, const void* x
  * Einsum / MatMul(Q, K) (pure_implementations.py:111-252), the scalar Mul / Div (:76-93),
  * Softmax(axis=-1) (:309-319) and Einsum(P, V); the backward entry point replaces the nodes
  * DefaultEinsumBackward and DefaultSoftmaxBackward emit for that chain
- * (autodiff/implementations/onnx_ops.py:25-138, 237-275). No mask, no dropout.
+ * (autodiff/implementations/onnx_ops.py:25-138, 237-275). No dropout; the *_masked_* entry
+ * points below add a mask row to the scaled scores first.
  * Tensors are [batch0, batch1, seq, head_dim] views: element strides for batch0, batch1 and
  * seq are given per tensor (multiples of 8), head_dim is contiguous and must be 64.
  * lse (optional in forward, required by backward): fp32 [batch0, batch1, seq_q] dense,
@@ -351,6 +352,23 @@ int dmlhip_attention_backward_f16(const dmlhip_attention_desc* d,
                                   const void* k, const void* v, const void* o, const void* lse,
                                   const void* d_o, void* dq, void* dk, void* dv,
                                   void* workspace, size_t workspace_bytes, void* stream);
+/* The same with an additive mask between the scaling and the softmax - the elementwise Add of
+ * pure_implementations.py:34-36 as the exporter places it in a BERT encoder (scores + mask, mask
+ * [batch, 1, 1, keys]): O = softmax(scale * Q K^T + mask, over keys) V. mask: fp16, one row of seq_k
+ * contiguous values per (batch0, batch1), the same for every query; row (b0, b1) starts at
+ * mask + b0 * mask_stride[0] + b1 * mask_stride[1] elements (0 = broadcast over that dimension;
+ * multiples of 4; mask 8-byte aligned). Values may be -inf; a query row whose keys are all at -inf
+ * yields NaN, as the reference's Softmax does. The backward treats the mask as a constant (no gradient
+ * for it) and must be given the mask the forward call was given. */
+int dmlhip_attention_masked_f16(const dmlhip_attention_desc* d, const void* q, const void* k,
+                                const void* v, const void* mask, const int64_t* mask_stride, void* o,
+                                void* lse, void* stream);
+int dmlhip_attention_masked_backward_f16(const dmlhip_attention_desc* d,
+                                         const dmlhip_attention_desc* grad, const void* q,
+                                         const void* k, const void* v, const void* mask,
+                                         const int64_t* mask_stride, const void* o, const void* lse,
+                                         const void* d_o, void* dq, void* dk, void* dv,
+                                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- BatchNormalization (NCHW) ------------------------------------------------------------------
  * Replaces PureBatchNormalization (daceml/onnx/op_implementations/img_op_implementations.py:333-412) and

@@ -171,13 +171,17 @@ def softmax_backward(output, output_grad, axis):
     return prod - input_grad
 
 
-def attention(q, k, v, scale):
+def attention(q, k, v, scale, mask=None):
     """The attention sub-graph as the reference expands it, node by node: Einsum(Q, K)
-    (pure_implementations.py:219-252), the scalar Mul (:86-88), Softmax(axis=-1) (:309-319) and Einsum(P, V).
-    q [..., Sq, d], k [..., Sk, d], v [..., Sk, dv] with identical leading dims. Returns (out, lse) with
-    lse = log(sum_j exp(scale * q.k_j)) per query row (what a fused kernel keeps instead of P)."""
+    (pure_implementations.py:219-252), the scalar Mul (:86-88), with ``mask`` the elementwise Add (:34-36) of a
+    tensor broadcastable to the scores (a BERT encoder's padding mask is [batch, 1, 1, Sk]), Softmax(axis=-1)
+    (:309-319) and Einsum(P, V). q [..., Sq, d], k [..., Sk, d], v [..., Sk, dv] with identical leading dims. Returns
+    (out, lse) with lse = log(sum_j exp(scale * q.k_j + mask_j)) per query row (what a fused kernel keeps instead of
+    P)."""
     lead = "abcdefgh"[:q.ndim - 2]
     scores = mul(einsum("%sik,%sjk->%sij" % (lead, lead, lead), q, k), np.asarray(scale, dtype=q.dtype))
+    if mask is not None:
+        scores = add(scores, mask)
     probs = softmax(scores, axis=scores.ndim - 1)
     out = einsum("%sij,%sjk->%sik" % (lead, lead, lead), probs, v)
     m = np.max(scores, axis=-1, keepdims=True)
@@ -185,15 +189,18 @@ def attention(q, k, v, scale):
     return out, lse
 
 
-def attention_backward(q, k, v, scale, out_grad):
+def attention_backward(q, k, v, scale, out_grad, mask=None):
     """Backward of :func:`attention` as autodiff emits it: DefaultEinsumBackward for both contractions
     (autodiff/implementations/onnx_ops.py:25-138), DefaultSoftmaxBackward (:237-275), and the scalar Mul
-    reversed (d/dx (x*c) = c). Returns (dq, dk, dv)."""
+    reversed (d/dx (x*c) = c); the Add of a constant mask passes the gradient through. Returns (dq, dk, dv)."""
     lead = "abcdefgh"[:q.ndim - 2]
     eq_s = "%sik,%sjk->%sij" % (lead, lead, lead)
     eq_o = "%sij,%sjk->%sik" % (lead, lead, lead)
     c = np.asarray(scale, dtype=q.dtype)
-    probs = softmax(mul(einsum(eq_s, q, k), c), axis=q.ndim - 1)
+    scores = mul(einsum(eq_s, q, k), c)
+    if mask is not None:
+        scores = add(scores, mask)
+    probs = softmax(scores, axis=q.ndim - 1)
     dprobs = einsum_backward(eq_o, [probs, v], out_grad, 0)
     dv = einsum_backward(eq_o, [probs, v], out_grad, 1)
     dscores = mul(softmax_backward(probs, dprobs, q.ndim - 1), c)

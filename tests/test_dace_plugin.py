@@ -137,6 +137,12 @@ def _sample_sdfgs():
     g.output(g.layer_norm(h, "gamma", "beta", 1e-5, "ln"), "y")
     assert fusion.auto_optimize(g.sdfg)["skip_layernorm"] == 1
     out.append(("skip_layernorm", g.sdfg))
+    # attention with an additive mask, forward and reverse
+    from tests.test_zx_attention_mask import _chain
+    g = _chain((2, 1, 1, 48))
+    assert fusion.auto_optimize(g.sdfg)["attention"] == 1
+    add_backward_pass(g.sdfg, g.state, ["o"], ["q", "k", "v"])
+    out.append(("masked_attention_train", g.sdfg))
     return out
 
 

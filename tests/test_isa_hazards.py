@@ -59,7 +59,7 @@ _Z6kernelv:
 
 def test_fused_attention_kernels(tmp_path):
     count, found = isa_hazards.check_file(_assembly(os.path.join(ROOT, "daceml_amd", "csrc", "attention.hip"), tmp_path))
-    assert count == 3, "forward, dQ and dK/dV kernels"
+    assert count == 6, "forward, dQ and dK/dV kernels, each with and without a mask"
     assert not found, _report(found)
 
 

@@ -217,6 +217,40 @@ def test_attention_matches_torch_sdpa_and_autograd():
     np.testing.assert_array_equal(dq0, 0.0)
 
 
+def test_masked_attention_matches_torch_sdpa_and_autograd():
+    """The additive mask: against scaled_dot_product_attention(attn_mask=...) and its autograd in fp64 for a padding
+    mask [batch, 1, 1, keys] and a full [batch, heads, queries, keys] bias; -inf entries give exactly zero
+    probability, a mask constant along the keys changes nothing, and the masked keys receive no gradient."""
+    q = rng(94).standard_normal((2, 3, 7, 8))
+    k = rng(95).standard_normal((2, 3, 5, 8))
+    v = rng(96).standard_normal((2, 3, 5, 8))
+    do = rng(97).standard_normal((2, 3, 7, 8))
+    scale = 0.41
+    pad = np.zeros((2, 1, 1, 5))
+    pad[1, 0, 0, 3:] = -10000.0
+    full = rng(98).standard_normal((2, 3, 7, 5))
+    for mask in (pad, full):
+        out, lse = O.attention(q, k, v, scale, mask)
+        tq, tk, tv = (torch.tensor(t, requires_grad=True) for t in (q, k, v))
+        ref = F.scaled_dot_product_attention(tq, tk, tv, attn_mask=torch.tensor(mask), scale=scale)
+        np.testing.assert_allclose(out, ref.detach().numpy(), rtol=1e-12, atol=1e-12)
+        ref.backward(torch.tensor(do))
+        for got, want in zip(O.attention_backward(q, k, v, scale, do, mask), (tq.grad, tk.grad, tv.grad)):
+            np.testing.assert_allclose(got, want.numpy(), rtol=1e-11, atol=1e-12)
+        s = scale * np.einsum("d,jd->j", q[1, 2, 4], k[1, 2]) + np.broadcast_to(mask, (2, 3, 7, 5))[1, 2, 4]
+        np.testing.assert_allclose(lse[1, 2, 4], math.log(np.exp(s).sum()), rtol=1e-12)
+    # -inf: the masked keys drop out exactly - same result as attention over the first three keys alone
+    hard = np.zeros((2, 1, 1, 5))
+    hard[:, 0, 0, 3:] = -np.inf
+    np.testing.assert_allclose(O.attention(q, k, v, scale, hard)[0], O.attention(q, k[:, :, :3], v[:, :, :3], scale)[0],
+                               rtol=1e-13)
+    dq, dk, dv = O.attention_backward(q, k, v, scale, do, hard)
+    assert np.all(dk[:, :, 3:] == 0) and np.all(dv[:, :, 3:] == 0)
+    # a shift common to all keys of a row cancels in the softmax
+    shift = rng(99).standard_normal((2, 3, 7, 1))
+    np.testing.assert_allclose(O.attention(q, k, v, scale, shift)[0], O.attention(q, k, v, scale)[0], rtol=1e-12)
+
+
 def test_gemm_attributes():
     a, b, c = rng(26).standard_normal((4, 5)), rng(27).standard_normal((6, 5)), rng(28).standard_normal(6)
     np.testing.assert_allclose(O.gemm(a, b, c, alpha=0.5, beta=2.0, transB=1), 0.5 * a @ b.T + 2.0 * c, rtol=1e-12)
