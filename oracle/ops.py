@@ -365,6 +365,56 @@ def einsum(equation: str, *inputs):
     return np.einsum(equation, *inputs)
 
 
+def einsum_f32_sequential(equation: str, a, b):
+    """The same contraction evaluated the way the compiled pure expansion does in single precision: one fp32
+    accumulator per output element, the contracted indices walked in row-major order, one rounded product and one
+    rounded addition per term (the write-conflict-resolution sum of the map that ``create_einsum_sdfg`` builds for
+    pure_implementations.py:219-252). It measures what fp32 summation alone costs against the fp64 value, which is
+    what an fp32 kernel with some other summation order can be held to. Two operands, no repeated letters."""
+    (ta, tb), to = parse_einsum(equation)
+    a32, b32 = np.asarray(a, dtype=np.float32), np.asarray(b, dtype=np.float32)
+    contracted = [l for l in ta if l in tb and l not in to]
+    ext = {l: a32.shape[ta.index(l)] for l in contracted}
+    keep_a = "".join(l for l in ta if l not in contracted)
+    keep_b = "".join(l for l in tb if l not in contracted)
+    step = "%s,%s->%s" % (keep_a, keep_b, to)
+    out_shape = tuple((a32.shape[ta.index(l)] if l in ta else b32.shape[tb.index(l)]) for l in to)
+    acc = np.zeros(out_shape, dtype=np.float32)
+    for idx in np.ndindex(*[ext[l] for l in contracted]):
+        pick = dict(zip(contracted, idx))
+        sa = a32[tuple(pick.get(l, slice(None)) for l in ta)]
+        sb = b32[tuple(pick.get(l, slice(None)) for l in tb)]
+        acc += np.einsum(step, sa, sb)      # no contraction left: one fp32 product per element, then one fp32 add
+    return acc
+
+
+def conv2d_f32_sequential(X, W, B=None, strides=(1, 1), pads=(0, 0, 0, 0), dilations=(1, 1), group=1):
+    """conv2d() in single precision in the order of PureConv2D's loop nest (img_op_implementations.py:265-288,
+    314-328): the accumulator starts from the bias (or zero) and takes the products of (c, hy, hx) in that order, each
+    product and each addition rounded to fp32."""
+    X32, W32 = np.asarray(X, dtype=np.float32), np.asarray(W, dtype=np.float32)
+    n, c, h, w = X32.shape
+    m, cg, kh, kw = W32.shape
+    pt, pl, pb, pr = pads
+    sy, sx = strides
+    dy, dx = dilations
+    oh = conv_out_size(h, kh, sy, pt + pb, dy)
+    ow = conv_out_size(w, kw, sx, pl + pr, dx)
+    Xp = np.zeros((n, c, h + pt + pb, w + pl + pr), dtype=np.float32)
+    Xp[:, :, pt:pt + h, pl:pl + w] = X32
+    Y = np.zeros((n, m, oh, ow), dtype=np.float32)
+    if B is not None:
+        Y += np.asarray(B, dtype=np.float32).reshape(1, m, 1, 1)
+    mg = m // group
+    for g in range(group):
+        for cc in range(cg):
+            for hy in range(kh):
+                for hx in range(kw):
+                    patch = Xp[:, g * cg + cc, hy * dy:hy * dy + (oh - 1) * sy + 1:sy, hx * dx:hx * dx + (ow - 1) * sx + 1:sx]
+                    Y[:, g * mg:(g + 1) * mg] += W32[g * mg:(g + 1) * mg, cc, hy, hx].reshape(1, mg, 1, 1) * patch[:, None]
+    return Y
+
+
 def matmul(A, B):
     """PureMatMul: pure_implementations.py:111-216 (refuses 1-D operands, lowers to ONNXEinsum)."""
     if A.ndim == 1 or B.ndim == 1:

@@ -251,6 +251,61 @@ def test_masked_attention_matches_torch_sdpa_and_autograd():
     np.testing.assert_allclose(O.attention(q, k, v, scale, shift)[0], O.attention(q, k, v, scale)[0], rtol=1e-12)
 
 
+def _bound_use(got, want, rtol, atol):
+    """Largest |error| as a fraction of the bound atol + rtol * |want|."""
+    return float((np.abs(got - want) / (atol + rtol * np.abs(want))).max())
+
+
+def test_sequential_fp32_evaluations_agree_with_the_definitions():
+    a, b = rng(100).standard_normal((2, 5, 7)), rng(101).standard_normal((7, 4))
+    np.testing.assert_allclose(O.einsum_f32_sequential("aik,kj->aij", a, b), O.einsum("aik,kj->aij", a, b), rtol=1e-5, atol=2e-6)
+    a, b = rng(102).standard_normal((2, 6, 5)), rng(103).standard_normal((2, 6, 3))
+    np.testing.assert_allclose(O.einsum_f32_sequential("aij,aik->jk", a, b), O.einsum("aij,aik->jk", a, b), rtol=1e-5, atol=2e-6)
+    x, w, c = rng(104).standard_normal((2, 6, 9, 8)), rng(105).standard_normal((4, 3, 3, 2)), rng(106).standard_normal(4)
+    args = ((2, 1), (1, 0, 1, 0), (1, 2), 2)
+    np.testing.assert_allclose(O.conv2d_f32_sequential(x, w, c, *args), O.conv2d(x, w, c, *args), rtol=1e-5, atol=5e-6)
+    # exact on integers: the order of summation is the only thing the fp32 evaluation changes
+    ai, bi = rng(107).integers(-8, 8, (3, 40)).astype(np.float64), rng(108).integers(-8, 8, (40, 5)).astype(np.float64)
+    np.testing.assert_array_equal(O.einsum_f32_sequential("ik,kj->ij", ai, bi), ai @ bi)
+
+
+def test_fp32_bounds_of_the_gpu_tests_are_what_fp32_summation_costs():
+    """The GPU tests hold fp32 contractions and convolutions to rtol 1e-5 / atol 1e-6, the absolute part widened with
+    the number of terms K (contractions: sqrt(K / 64), convolutions on all-positive data: K / 64). Evidence that the
+    widening is the cost of fp32 summation and not slack: the reference's own evaluation order in fp32 (one
+    accumulator, terms in index order) on the very inputs of those tests
+    (a) stays inside the widened bound in every case, using up to 85 % of it, and
+    (b) breaks the un-widened bound on the long sums - 272 and 1000 terms in the contractions, the 147-term 7x7
+        convolution - so no summation order of comparable quality could be asked to meet it there."""
+    from tests import test_gpu_kernels as TK
+    widened, plain = {}, {}
+    for eq, sa, sb in TK.GEMM_CASES:
+        a = (rng(80).standard_normal(sa) * 0.25).astype(np.float32)
+        b = (rng(81).standard_normal(sb) * 0.25).astype(np.float32)
+        want = O.einsum(eq, a.astype(np.float64), b.astype(np.float64))
+        (ta, tb), to = eq.split("->")[0].split(","), eq.split("->")[1]
+        k = int(np.prod([s_ for l, s_ in zip(ta, sa) if l in tb and l not in to] or [1]))
+        seq = O.einsum_f32_sequential(eq, a, b)
+        widened[("einsum", eq, k)] = _bound_use(seq, want, 1e-5, 1e-6 * max(1.0, np.sqrt(k / 64.0)))
+        plain[("einsum", eq, k)] = _bound_use(seq, want, 1e-5, 1e-6)
+    for xs, ws, st, pd, dl, grp, has_bias in TK.CONV_CASES:
+        x = rng(90).uniform(0, 1, xs).astype(np.float32)
+        w = (rng(91).uniform(0, 1, ws) / np.sqrt(np.prod(ws[1:]))).astype(np.float32)
+        c = rng(92).standard_normal(ws[0]).astype(np.float32) if has_bias else None
+        pads = (pd[0], pd[1], pd[0], pd[1])
+        want = O.conv2d(x.astype(np.float64), w.astype(np.float64), None if c is None else c.astype(np.float64), st, pads, dl, grp)
+        seq = O.conv2d_f32_sequential(x, w, c, st, pads, dl, grp)
+        k = ws[1] * ws[2] * ws[3]
+        widened[("conv", ws, k)] = _bound_use(seq, want, 1e-5, 1e-6 * max(1.0, k / 64.0))
+        plain[("conv", ws, k)] = _bound_use(seq, want, 1e-5, 1e-6)
+    assert max(widened.values()) < 1.0, sorted(widened.items(), key=lambda kv: -kv[1])[:3]
+    assert max(widened.values()) > 0.5, "the widened bounds would be slack"
+    over = {key for key, v in plain.items() if v > 1.0}
+    assert {key[2] for key in over} >= {272, 1000, 147}, over
+    # up to 64 terms nothing is widened, and nothing needs to be
+    assert all(v < 1.0 for key, v in plain.items() if key[2] <= 64)
+
+
 def test_gemm_attributes():
     a, b, c = rng(26).standard_normal((4, 5)), rng(27).standard_normal((6, 5)), rng(28).standard_normal(6)
     np.testing.assert_allclose(O.gemm(a, b, c, alpha=0.5, beta=2.0, transB=1), 0.5 * a @ b.T + 2.0 * c, rtol=1e-12)
