@@ -267,11 +267,50 @@ def secondary_workload(name, device, steps, warmup, verbose):
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     roof["traffic"] = None
     roof["kernel"] = top.label
-    print(json.dumps({"metric": what + " ms/iter at 1 GPU", "value": round(ms, 4), "unit": "ms/iter", "n_gpus": 1,
-                      "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
-                      "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-                      "config": {"workload": what, "launches_per_step": len(prog.launches)}, "roofline": roof,
-                      "launches": launches}))
+    line = {"metric": what + " ms/iter at 1 GPU", "value": round(ms, 4), "unit": "ms/iter", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
+            "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+            "config": {"workload": what, "launches_per_step": len(prog.launches)}, "roofline": roof,
+            "launches": launches}
+    if name == "nodes":
+        line["layernorm_cold"] = layernorm_cold(device, rng, max(2, min(steps, 6)))
+    print(json.dumps(line))
+
+
+def layernorm_cold(device, rng, rounds, buffers=40):
+    """The LayerNorm of the `nodes` workload with input and output rotating over `buffers` distinct pairs: 40 pairs
+    of [8,512,1024] fp16 are 671 MB, so by the time a pair comes round again it has left the 256 MB last-level cache
+    and the launch reads from HBM. (The `launches` entry of the same node re-uses one pair, which stays in cache.)"""
+    import numpy as np
+    import torch
+    from daceml_amd import graphs
+    from daceml_amd.runtime import CompiledSDFG
+    from daceml_amd.transformation import fusion
+    g = graphs.GraphBuilder("layernorm_cold", torch.float16)
+    xin = g.input("x", (8, 512, 1024))
+    g.input("gamma", (1024, ))
+    g.input("beta", (1024, ))
+    g.output(g.layer_norm(xin, "gamma", "beta", 1e-5, "ln"), "y")
+    fusion.auto_optimize(g.sdfg)
+    prog = CompiledSDFG(g.sdfg, device=device)
+    gamma = torch.from_numpy(rng.uniform(0.5, 1.5, 1024).astype(np.float16)).to(device)
+    beta = torch.from_numpy((rng.standard_normal(1024) * 0.1).astype(np.float16)).to(device)
+    xs = [torch.randn((8, 512, 1024), dtype=torch.float16, device=device) for _ in range(buffers)]
+    ys = [torch.empty((8, 512, 1024), dtype=torch.float16, device=device) for _ in range(buffers)]
+    prog(x=xs[0], gamma=gamma, beta=beta, y=ys[0])
+    times = []
+    for r in range(rounds + 1):
+        for i in range(buffers):
+            prog.bind({"x": xs[i], "y": ys[i]})
+            t = sum(ms for _, ms in prog.launch_timed())
+            if r > 0:   # the first round is the warm-up of everything but the data
+                times.append(t)
+    us = float(np.mean(times)) * 1e3
+    nbytes = sum(l.bytes_moved or 0 for l in prog.launches)
+    gbs = nbytes / (us * 1e-6) / 1e9
+    return {"us": round(us, 2), "min_us": round(float(np.min(times)) * 1e3, 2), "GB/s": round(gbs, 1),
+            "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": int(nbytes), "buffers": buffers, "launches": len(prog.launches),
+            "samples": len(times)}
 
 
 def module_workload(device, steps, warmup):
