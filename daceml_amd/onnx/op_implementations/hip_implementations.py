@@ -1090,31 +1090,60 @@ class HipBatchNormalizationGrad(ONNXForward):
 
 # ----------------------------------------------------------------------------- convolution
 def _conv_struct(node, x: Array, w: Array, act=L.ACT_NONE) -> Optional[L.Conv2dDesc]:
-    """Attribute handling of CudnnConvolution (cudnn_implementations.py:148-275): 2-D, symmetric pads,
-    auto_pad NOTSET, any stride / dilation / group."""
-    if len(x.shape) != 4 or len(w.shape) != 4 or node.auto_pad != "NOTSET":
+    """Attribute handling of CudnnConvolution (cudnn_implementations.py:148-275): 1-D and 2-D, symmetric pads,
+    auto_pad NOTSET, any stride / dilation / group. A 1-D convolution over [N, C, L] is the 2-D one over [N, C, 1, L]
+    with a 1 x k filter (the reference hands cuDNN [N, C, L, 1] and a k x 1 filter, :243-250; the dense tensors are
+    the same bytes either way, and a row of L contiguous elements is what these kernels stream)."""
+    nsp = len(x.shape) - 2
+    if nsp not in (1, 2) or len(w.shape) != len(x.shape) or node.auto_pad != "NOTSET":
         return None
-    strides = list(node.strides) if node.strides is not None else [1, 1]
-    dil = list(node.dilations) if node.dilations is not None else [1, 1]
-    pads = list(node.pads) if node.pads is not None else [0, 0, 0, 0]
-    if len(strides) != 2 or len(dil) != 2 or len(pads) != 4:
+    strides = list(node.strides) if node.strides is not None else [1] * nsp
+    dil = list(node.dilations) if node.dilations is not None else [1] * nsp
+    pads = list(node.pads) if node.pads is not None else [0] * (2 * nsp)
+    if len(strides) != nsp or len(dil) != nsp or len(pads) != 2 * nsp:
         return None
-    if pads[0] != pads[2] or pads[1] != pads[3]:
+    if any(pads[i] != pads[nsp + i] for i in range(nsp)):
         return None
     if node.kernel_shape is not None and list(node.kernel_shape) != list(w.shape[2:]):
         return None
     group = int(node.group)
     if group < 1 or x.shape[1] != w.shape[1] * group or w.shape[0] % group:
         return None
+    if nsp == 1:
+        strides, dil, pads = [1] + strides, [1] + dil, [0, pads[0], 0, pads[1]]
     d = L.Conv2dDesc()
-    d.n, d.c, d.h, d.w = x.shape
-    d.m, d.kh, d.kw = w.shape[0], w.shape[2], w.shape[3]
+    d.n, d.c = x.shape[0], x.shape[1]
+    d.h, d.w = (1, x.shape[2]) if nsp == 1 else x.shape[2:]
+    d.m = w.shape[0]
+    d.kh, d.kw = (1, w.shape[2]) if nsp == 1 else w.shape[2:]
     d.stride_h, d.stride_w = strides
     d.pad_h, d.pad_w = pads[0], pads[1]
     d.dil_h, d.dil_w = dil
     d.group = group
     d.act = act
     return d
+
+
+def _tensor_layout(desc: Array) -> Optional[str]:
+    """"NCHW", "NHWC" or None for a 3-D / 4-D tensor whose shape is in ONNX order [N, C, spatial..]: the test of
+    ``_get_tensor_layout`` (cudnn_implementations.py:20-66) - the strides are those of the dense tensor, or those of
+    a dense channels-last tensor viewed in ONNX order. Where the two coincide (one channel, or one pixel) it is NCHW."""
+    shape, strides = tuple(desc.shape), tuple(desc.strides)
+    if len(shape) not in (3, 4):
+        return None
+    if desc.is_contiguous():
+        return "NCHW"
+    last = shape[:1] + shape[2:] + shape[1:2]                # the channels-last shape
+    dense = [_prod(last[i + 1:]) for i in range(len(last))]  # and its dense strides
+    as_onnx = tuple(dense[:1] + dense[-1:] + dense[1:-1])
+    relevant = [i for i in range(len(shape)) if shape[i] > 1]
+    return "NHWC" if all(strides[i] == as_onnx[i] for i in relevant) else None
+
+
+def _conv_out_shape(d: L.Conv2dDesc, x: Array):
+    """Shape of Y for the descriptor `_conv_struct` made from X (three dimensions for a 1-D convolution)."""
+    oh, ow = _conv_out_hw(d)
+    return (d.n, d.m, ow) if len(x.shape) == 3 else (d.n, d.m, oh, ow)
 
 
 def _conv_out_hw(d: L.Conv2dDesc):
@@ -1136,7 +1165,7 @@ class HipConv(ONNXForward):
         try:
             ins, outs = _descs(node, state, sdfg)
             x, w, y = ins["X"], ins["W"], outs["Y"]
-            if not (_float_ok(x, w, y) and _dense(x, w, y)):
+            if not (_float_ok(x, w, y) and _dense(w)) or _tensor_layout(x) is None or _tensor_layout(y) is None:
                 return False
             if "B" in ins and not (ins["B"].dtype == x.dtype and ins["B"].is_contiguous()
                                    and ins["B"].total_size == w.shape[0]):
@@ -1144,20 +1173,41 @@ class HipConv(ONNXForward):
             d = _conv_struct(node, x, w)
             if d is None:
                 return False
-            oh, ow = _conv_out_hw(d)
-            return tuple(y.shape) == (x.shape[0], w.shape[0], oh, ow)
+            return tuple(y.shape) == _conv_out_shape(d, x)
         except Exception:
             return False
 
     @staticmethod
     def forward(node, state, sdfg):
+        """One call for dense NCHW tensors. A channels-last X or Y (ONNX-order shape, NHWC strides: what
+        CudnnConvolution passes to cuDNN as CUDNN_TENSOR_NHWC, cudnn_implementations.py:69-110) is brought into the
+        kernels' layout by a transpose into the workspace before, respectively out of it after, the convolution."""
         ins, outs = _descs(node, state, sdfg)
         x, w, y = ins["X"], ins["W"], outs["Y"]
         d = _conv_struct(node, x, w, _ACT[getattr(node, "_activation", "none")])
-        call = HipCall("dmlhip_conv2d_" + _SFX[x.dtype],
-                       [Struct(d, "dmlhip_conv2d_desc"), Ptr("X"), Ptr("W"), _opt(node, state, "B"), Ptr("Y"), Stream()])
-        flops = 2 * y.total_size * (w.shape[1] * w.shape[2] * w.shape[3])
-        return _tasklet(node, state, [call], flops=flops, bytes_moved=_nbytes(x, w, y), kind="conv")
+        sfx = _SFX[x.dtype]
+        calls, ws = [], 0
+        x_arg, y_arg = Ptr("X"), Ptr("Y")
+        if _tensor_layout(x) == "NHWC":
+            last = tuple(x.shape[:1]) + tuple(x.shape[2:]) + tuple(x.shape[1:2])
+            back = (0, len(last) - 1) + tuple(range(1, len(last) - 1))
+            calls.append(HipCall("dmlhip_transpose_" + sfx, [Ptr("X"), Workspace(0), I32(len(last)), I64Array(last),
+                                                             I64Array(back), Stream()], flops=0, bytes_moved=2 * _nbytes(x)))
+            x_arg = Workspace(0)
+            ws = (_nbytes(x) + 255) // 256 * 256
+        y_nhwc = _tensor_layout(y) == "NHWC"
+        if y_nhwc:
+            y_arg = Workspace(ws)
+        flops = 2 * y.total_size * int(math.prod(w.shape[1:]))
+        calls.append(HipCall("dmlhip_conv2d_" + sfx, [Struct(d, "dmlhip_conv2d_desc"), x_arg, Ptr("W"), _opt(node, state, "B"),
+                                                      y_arg, Stream()], flops=flops, bytes_moved=_nbytes(x, w, y)))
+        if y_nhwc:
+            nd = len(y.shape)
+            calls.append(HipCall("dmlhip_transpose_" + sfx, [Workspace(ws), Ptr("Y"), I32(nd), I64Array(tuple(y.shape)),
+                                                             I64Array((0, ) + tuple(range(2, nd)) + (1, )), Stream()],
+                                 flops=0, bytes_moved=2 * _nbytes(y)))
+            ws += (_nbytes(y) + 255) // 256 * 256
+        return _tasklet(node, state, calls, workspace_bytes=ws, flops=flops, bytes_moved=_nbytes(x, w, y), kind="conv")
 
 
 @op_implementation(op="GatedConv", name=IMPL)
@@ -1271,8 +1321,7 @@ class HipConvGrad(ONNXForward):
             d = _conv_struct(node, x, w)
             if d is None:
                 return False
-            oh, ow = _conv_out_hw(d)
-            if tuple(dy.shape) != (x.shape[0], w.shape[0], oh, ow):
+            if tuple(dy.shape) != _conv_out_shape(d, x):
                 return False
             for name, ref in (("dX", x), ("dW", w)):
                 if name in outs and not (outs[name].shape == ref.shape and outs[name].is_contiguous()
@@ -1291,7 +1340,7 @@ class HipConvGrad(ONNXForward):
         d = _conv_struct(node, x, w)
         lib = L.load()
         calls, ws = [], 0
-        work = 2 * dy.total_size * w.shape[1] * w.shape[2] * w.shape[3]     # of each of the two gradients
+        work = 2 * dy.total_size * int(math.prod(w.shape[1:]))     # of each of the two gradients
         if "dX" in outs:
             calls.append(HipCall("dmlhip_conv2d_backward_data_f32",
                                  [Struct(d, "dmlhip_conv2d_desc"), Ptr("dY"), Ptr("W"), Ptr("dX"), Stream()],
@@ -1306,7 +1355,7 @@ class HipConvGrad(ONNXForward):
             # dB[m] = sum_{b, y, x} dY[b, m, y, x]: reduce the spatial dims into the head of the
             # workspace, then the batch dim from there
             n, m = dy.shape[0], dy.shape[1]
-            hw = dy.shape[2] * dy.shape[3]
+            hw = int(math.prod(dy.shape[2:]))
             part = (n * m * 4 + 255) // 256 * 256
             ws = max(ws, part + lib.dmlhip_reduce_workspace_bytes(1, n, m))
             calls.append(HipCall("dmlhip_reduce_f32", [I32(L.RSUM), Ptr("dY"), Workspace(), I32(L.F32), I64(n * m),

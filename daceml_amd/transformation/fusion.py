@@ -373,7 +373,8 @@ def fuse_gate_into_conv(sdfg: SDFG) -> int:
             mul = prod[0]
             a, b = _in_array(state, mul, "A"), _in_array(state, mul, "B")
             xd = sdfg.arrays[xa]
-            if len(xd.shape) != 4 or xd.dtype != torch.float32:
+            if len(xd.shape) != 4 or xd.dtype != torch.float32 or not xd.is_contiguous() \
+                    or not sdfg.arrays[_out_array(state, conv, "Y")].is_contiguous():
                 continue
             gate_shape = (xd.shape[0], xd.shape[1], 1, 1)
             if tuple(sdfg.arrays[b].shape) == gate_shape and tuple(sdfg.arrays[a].shape) == tuple(xd.shape):
@@ -423,7 +424,8 @@ def fuse_expand_depthwise(sdfg: SDFG) -> int:
             x = _in_array(state, pw, "X")
             xd, md = sdfg.arrays[x], sdfg.arrays[mid]
             w1, w2 = sdfg.arrays[_in_array(state, pw, "W")], sdfg.arrays[_in_array(state, dw, "W")]
-            if len(xd.shape) != 4 or any(d.dtype != torch.float32 for d in (xd, md, w1, w2)):
+            if len(xd.shape) != 4 or any(d.dtype != torch.float32 for d in (xd, md, w1, w2)) or not xd.is_contiguous() \
+                    or not sdfg.arrays[_out_array(state, dw, "Y")].is_contiguous():
                 continue
             pointwise = (tuple(w1.shape[2:]) == (1, 1) and pw.group == 1 and pw.auto_pad == "NOTSET"
                          and all(v == 1 for v in (pw.strides or [1, 1])) and not any(pw.pads or [0])

@@ -98,6 +98,44 @@ def reduce(op, x, y, out_dtype, outer, r, inner):
     y.reshape(-1)[:outer * inner] = res.reshape(-1).astype(want)
 
 
+def _conv_views(desc, x, w):
+    import torch
+    cg = desc.c // desc.group
+    xt = torch.from_numpy(x.reshape(-1)[:desc.n * desc.c * desc.h * desc.w].astype(np.float64)).reshape(desc.n, desc.c, desc.h, desc.w)
+    wt = torch.from_numpy(w.reshape(-1)[:desc.m * cg * desc.kh * desc.kw].astype(np.float64)).reshape(desc.m, cg, desc.kh, desc.kw)
+    kw = dict(stride=(desc.stride_h, desc.stride_w), padding=(desc.pad_h, desc.pad_w), dilation=(desc.dil_h, desc.dil_w),
+              groups=desc.group)
+    return xt, wt, kw
+
+
+def conv2d(desc, x, w, bias, y):
+    """dmlhip_conv2d_*: dense NCHW / OIHW cross-correlation described by dmlhip_conv2d_desc, then the activation."""
+    import torch
+    xt, wt, kw = _conv_views(desc, x, w)
+    bt = None if bias is None else torch.from_numpy(bias.reshape(-1)[:desc.m].astype(np.float64))
+    out = _act(desc.act, torch.nn.functional.conv2d(xt, wt, bt, **kw).numpy())
+    y.reshape(-1)[:out.size] = out.reshape(-1).astype(y.dtype)
+
+
+def conv2d_backward(desc, which, x_or_dy, other, out):
+    """dmlhip_conv2d_backward_data_f32 (dY, W -> dX) / dmlhip_conv2d_backward_weight_f32 (X, dY -> dW)."""
+    import torch
+    cg = desc.c // desc.group
+    kw = dict(stride=(desc.stride_h, desc.stride_w), padding=(desc.pad_h, desc.pad_w), dilation=(desc.dil_h, desc.dil_w),
+              groups=desc.group)
+    eh, ew = (desc.kh - 1) * desc.dil_h + 1, (desc.kw - 1) * desc.dil_w + 1
+    oh = (desc.h + 2 * desc.pad_h - eh) // desc.stride_h + 1
+    ow = (desc.w + 2 * desc.pad_w - ew) // desc.stride_w + 1
+    f64 = lambda a, shape: torch.from_numpy(a.reshape(-1)[:int(np.prod(shape))].astype(np.float64)).reshape(shape)  # noqa: E731
+    if which == "data":
+        dy, w = f64(x_or_dy, (desc.n, desc.m, oh, ow)), f64(other, (desc.m, cg, desc.kh, desc.kw))
+        res = torch.nn.grad.conv2d_input((desc.n, desc.c, desc.h, desc.w), w, dy, **kw)
+    else:
+        x, dy = f64(x_or_dy, (desc.n, desc.c, desc.h, desc.w)), f64(other, (desc.n, desc.m, oh, ow))
+        res = torch.nn.grad.conv2d_weight(x, (desc.m, cg, desc.kh, desc.kw), dy, **kw)
+    out.reshape(-1)[:res.numel()] = res.numpy().reshape(-1).astype(out.dtype)
+
+
 class Emulator:
     """Runs the calls of a HipTasklet on NumPy arrays bound to its connectors."""
     def __init__(self, workspace_bytes):
@@ -130,6 +168,23 @@ class Emulator:
                 x = self._typed(x, np.float16 if call.symbol.endswith("f16") else np.float32)
                 y = self._typed(y, np.float16 if out_dtype == L.F16 else np.float32)
                 reduce(op, x, y, out_dtype, outer, r, inner)
+            elif call.symbol in ("dmlhip_transpose_f16", "dmlhip_transpose_f32"):
+                x, y, ndim, shape, perm = args[:5]
+                dt = np.float16 if call.symbol.endswith("f16") else np.float32
+                x, y = self._typed(x, dt), self._typed(y, dt)
+                shape, perm = tuple(shape[:ndim]), tuple(perm[:ndim])
+                n = int(np.prod(shape))
+                y.reshape(-1)[:n] = np.transpose(x.reshape(-1)[:n].reshape(shape), perm).reshape(-1)
+            elif call.symbol in ("dmlhip_conv2d_f16", "dmlhip_conv2d_f32"):
+                desc, x, w, bias, y = args[:5]
+                dt = np.float16 if call.symbol.endswith("f16") else np.float32
+                conv2d(desc, self._typed(x, dt), w, bias, self._typed(y, dt))
+            elif call.symbol == "dmlhip_conv2d_backward_data_f32":
+                desc, dy, w, dx = args[:4]
+                conv2d_backward(desc, "data", dy, w, dx)
+            elif call.symbol == "dmlhip_conv2d_backward_weight_f32":
+                desc, x, dy, dw = args[:4]
+                conv2d_backward(desc, "weight", x, dy, dw)
             elif call.symbol in ("dmlhip_softmax_backward_f16", "dmlhip_softmax_backward_f32"):
                 yv, dy, dx, rows, cols = args[:5]
                 y64 = yv.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
