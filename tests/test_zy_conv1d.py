@@ -2,8 +2,9 @@
 lowered to the 2-D kernels as [N, C, 1, L] with a 1 x k filter. Oracle: ``oracle.ops.conv2d`` on the same reshaping,
 itself checked here against ``torch.nn.functional.conv1d``.
 
-The host-side tests interpret the emitted calls with tests/abi_emulator.py. The GPU tests are SKIPPED for now: rows of
-height one with 1 x k filters and unequal strides are shapes the 2-D kernels have not been run with."""
+The host-side tests interpret the emitted calls with tests/abi_emulator.py; the GPU tests run small problems (direct
+kernel and contraction kernels) and one long sequence that is large enough for the implicit-GEMM kernel - SKIPPED for
+now, because that kernel has not been run with a single output row."""
 import numpy as np
 import pytest
 import torch
@@ -125,11 +126,12 @@ def test_shapes_that_are_not_a_1d_or_2d_convolution_are_refused():
         g.state.library_nodes()[0].expand(g.sdfg, g.state)
 
 
-@pytest.mark.skip(reason="1-D convolutions on the 2-D kernels (rows of height one, 1 x k filters) have not been run on hardware yet")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("case", CASES)
 def test_conv1d_on_gpu(case, dtype):
+    """These sizes are served by the direct kernel (one thread per output element, every tap bounds-checked) and, for
+    the 1 x 1 filter, by the contraction kernels."""
     from daceml_amd.runtime import CompiledSDFG
     n, c, l, m, k, stride, pad, dil, group, bias = case
     x, w, b, want = _data(*case, dtype=np.float16 if dtype == torch.float16 else np.float32)
@@ -142,3 +144,16 @@ def test_conv1d_on_gpu(case, dtype):
     prog(**args)
     tol = dict(rtol=1e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=2e-2, atol=1e-2)
     assert_close(host(y), want, dtype, "conv1d %s" % (case, ), **tol)
+
+
+@pytest.mark.skip(reason="the implicit-GEMM convolution kernel has not been run with a single output row yet")
+@pytest.mark.gpu
+def test_long_conv1d_on_gpu():
+    from daceml_amd.runtime import CompiledSDFG
+    case = (4, 32, 4096, 64, 5, 1, 2, 1, 1, True)
+    x, w, b, want = _data(*case)
+    g = _graph(torch.float32, *case, out_l=want.shape[2])
+    prog = CompiledSDFG(g.sdfg)
+    y = torch.full(want.shape, float("nan"), dtype=torch.float32, device="cuda")
+    prog(x=dev(x), w=dev(w), b=dev(b), y=y)
+    assert_close(host(y), want, torch.float32, "conv1d %s" % (case, ), rtol=1e-5, atol=1e-6 * (32 * 5) / 64)
