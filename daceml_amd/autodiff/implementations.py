@@ -78,11 +78,15 @@ def _new(ctx, op: str, label: str, **attrs):
 
 # ----------------------------------------------------------------------------- contractions
 def _einsum_backward(forward_node, ctx: BackwardContext, given, required, eq: str, alpha: float, act: str,
-                     bias_conn: Optional[str], residual_conn: Optional[str]):
+                     bias_conn: Optional[str], residual_conn: Optional[str],
+                     conns: Tuple[str, str, str] = ("Inputs__0", "Inputs__1", "Output"), group: Optional[BackwardGroup] = None,
+                     skip: Tuple[str, ...] = ()):
+    """`conns`: the forward node's connectors for the two operands and the result (MatMul and Gemm call them A, B, Y);
+    `skip`: required connectors the caller differentiates itself, into `group`."""
     sdfg = ctx.forward_sdfg
-    out = _out_arr(ctx, forward_node, "Output")
+    out = _out_arr(ctx, forward_node, conns[2])
     od = sdfg.arrays[out]
-    group = BackwardGroup(forward_node.label + "_backward")
+    group = group or BackwardGroup(forward_node.label + "_backward")
     req, passthrough = {}, {}
     grad_src: Optional[Tuple[Node, str]] = None   # producer of d(pre-activation) when an activation is undone
     dpre_arr = None
@@ -104,12 +108,14 @@ def _einsum_backward(forward_node, ctx: BackwardContext, given, required, eq: st
             group.map_input("Output_grad", node, conn)
 
     for conn in required:
-        if conn in ("Inputs__0", "Inputs__1"):
-            idx = int(conn[-1])
+        if conn in skip:
+            continue
+        if conn in conns[:2]:
+            idx = conns.index(conn)
             others, rev_eq = C.reverse_equation(eq, idx)
             es = _new(ctx, "FusedEinsum", "%s_grad_%d" % (forward_node.label, idx), equation=rev_eq, alpha=alpha)
             feed_dout(es, "Inputs__0")
-            connect_input_from_forward(forward_node, es, ctx, "Inputs__%d" % others[0], "Inputs__1")
+            connect_input_from_forward(forward_node, es, ctx, conns[others[0]], "Inputs__1")
             group.map_output(conn + "_grad", es, "Output")
             req[conn] = conn + "_grad"
         elif conn == bias_conn:
@@ -124,8 +130,85 @@ def _einsum_backward(forward_node, ctx: BackwardContext, given, required, eq: st
             passthrough[conn] = "Output"
         else:
             raise AutoDiffException("unexpected input connector %r" % conn)
-    return group, BackwardResult(required_grad_names=req, given_grad_names={"Output": "Output_grad"},
+    return group, BackwardResult(required_grad_names=req, given_grad_names={conns[2]: "Output_grad"},
                                  passthrough=passthrough)
+
+
+@autoregister_params(op="MatMul", name=NAME)
+class HipMatMulBackward(BackwardImplementation):
+    """The reference has no reverse node for MatMul: its generator expands the node with "pure" first
+    (backward_pass_generator.py:425-494), which makes it the Einsum of pure_implementations.py:132-191, and
+    differentiates that with DefaultEinsumBackward. Same here, without rewriting the forward node."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ranks = [len(sdfg.arrays[next(iter(state.in_edges_by_connector(node, c))).data.data].shape) for c in ("A", "B")]
+            return min(ranks) >= 2
+        except StopIteration:
+            return False
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        sdfg = context.forward_sdfg
+        ra, rb = (len(sdfg.arrays[_in_arr(context, forward_node, c)].shape) for c in ("A", "B"))
+        return _einsum_backward(forward_node, context, given_gradients, required_gradients, C.matmul_equation(ra, rb), 1.0,
+                                "none", None, None, conns=("A", "B", "Y"))
+
+
+@autoregister_params(op="Gemm", name=NAME)
+class HipGemmBackward(BackwardImplementation):
+    """Y = alpha op(A) op(B) + beta C (PureGemm, pure_implementations.py:380-553): A and B as for the Einsum PureGemm
+    builds, with alpha folded into the two new contractions; C receives beta times the incoming gradient, summed over
+    the rows where C is a vector broadcast over them (the Add's reversal plus ReverseReduce, dace_nodes.py:13-105)."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            a = sdfg.arrays[next(iter(state.in_edges_by_connector(node, "A"))).data.data]
+            b = sdfg.arrays[next(iter(state.in_edges_by_connector(node, "B"))).data.data]
+            return len(a.shape) == 2 and len(b.shape) == 2
+        except StopIteration:
+            return False
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        sdfg = context.forward_sdfg
+        node = forward_node
+        eq = "%s,%s->ij" % ("ki" if node.transA else "ik", "jk" if node.transB else "kj")
+        group = BackwardGroup(node.label + "_backward")
+        _, result = _einsum_backward(node, context, given_gradients, required_gradients, eq, float(node.alpha), "none", None,
+                                     None, conns=("A", "B", "Y"), group=group, skip=("C", ))
+        if "C" in required_gradients:
+            beta = float(node.beta)
+            yd = sdfg.arrays[_out_arr(context, node, "Y")]
+            cd = sdfg.arrays[_in_arr(context, node, "C")]
+            full = tuple(cd.shape) == tuple(yd.shape)
+            if full and beta == 1.0:
+                result.passthrough["C"] = "Y"
+                return group, result
+            src = None       # (node, connector) that produces the unscaled gradient; None: the incoming gradient itself
+            if not full:
+                if tuple(cd.shape) not in ((yd.shape[1], ), (1, yd.shape[1])):
+                    raise AutoDiffException("%s: C of shape %s is not a row vector of Y %s" % (node.label, cd.shape, yd.shape))
+                rs = _new(context, "ReduceSum", node.label + "_c_grad", axes=[0], keepdims=1 if len(cd.shape) == 2 else 0)
+                rs.add_in_connector("data")
+                group.map_input("Output_grad", rs, "data")
+                rs.add_out_connector("reduced")
+                src = (rs, "reduced")
+            if beta != 1.0:
+                mul = _new(context, "Mul", node.label + "_c_grad_scale")
+                mul.add_in_connector("A")
+                if src is None:
+                    group.map_input("Output_grad", mul, "A")
+                else:
+                    tmp, _ = sdfg.add_transient(node.label + "_c_grad_unscaled", cd.shape, cd.dtype)
+                    _write(context, src[0], src[1], tmp)
+                    _read(context, tmp, mul, "A")
+                _read(context, _scalar_constant(context, node.label + "_backward_beta", beta, cd.dtype), mul, "B")
+                mul.add_out_connector("C")
+                src = (mul, "C")
+            group.map_output("C_grad", src[0], src[1])
+            result.required_grad_names["C"] = "C_grad"
+        return group, result
 
 
 @autoregister_params(op="Einsum", name=NAME)
@@ -653,6 +736,18 @@ class HipTransposeBackward(BackwardImplementation):
         g.add_in_connector("data")
         g.add_out_connector("transposed")
         return g, BackwardResult(required_grad_names={"data": "transposed"}, given_grad_names={"transposed": "data"})
+
+
+@autoregister_params(op="Reshape", name=NAME)
+class HipReshapeBackward(BackwardImplementation):
+    """The gradient of a Reshape (pure_implementations.py:571-573, a copy into the new shape) is the incoming gradient
+    copied back into the shape of the input: one more Reshape node."""
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        g = _new(context, "Reshape", forward_node.label + "_backward")
+        g.add_in_connector("data")
+        g.add_out_connector("reshaped")
+        return g, BackwardResult(required_grad_names={"data": "reshaped"}, given_grad_names={"reshaped": "data"})
 
 
 @autoregister_params(op="GlobalAveragePool", name=NAME)

@@ -36,14 +36,19 @@ def _act(kind, v):
     raise ValueError(kind)
 
 
-def gemm(desc, a, b, c, bias, residual, pre_out):
-    """dmlhip_gemm_*: C[b][m, n] = act(alpha * sum_k A[b][m, k] B[b][k, n] + bias) + residual + beta * C. `a`, `b`,
-    `c`, ... are flat arrays; fp32 accumulation, one rounding to C's type."""
+def _gemm_products(desc, a, b):
+    """alpha * sum_k A[b][m, k] B[b][k, n] in fp64, shape batch + (m, n)."""
     m, n, k = desc.m, desc.n, desc.k
     batch = tuple(desc.batch)
     av = _view(a, 0, batch + (m, k), tuple(desc.a_stride_batch) + (desc.a_stride_m, desc.a_stride_k))
     bv = _view(b, 0, batch + (k, n), tuple(desc.b_stride_batch) + (desc.b_stride_k, desc.b_stride_n))
-    acc = np.matmul(av.astype(np.float64), bv.astype(np.float64)) * float(desc.alpha)
+    return np.matmul(av.astype(np.float64), bv.astype(np.float64)) * float(desc.alpha)
+
+
+def _gemm_finish(desc, acc, c, bias, residual, pre_out):
+    """The epilogue: + bias, (pre_out), activation, + residual, + beta * C, one rounding to C's type."""
+    m, n = desc.m, desc.n
+    batch = tuple(desc.batch)
     if bias is not None:
         bb = bias.reshape(-1).astype(np.float64)
         acc = acc + (bb[:m].reshape(m, 1) if desc.bias_along_m else bb[:n].reshape(1, n))
@@ -64,17 +69,125 @@ def gemm(desc, a, b, c, bias, residual, pre_out):
     cv[...] = acc.astype(out_dtype)
 
 
+def gemm(desc, a, b, c, bias, residual, pre_out):
+    """dmlhip_gemm_*: C[b][m, n] = act(alpha * sum_k A[b][m, k] B[b][k, n] + bias) + residual + beta * C. `a`, `b`,
+    `c`, ... are flat arrays; fp32 accumulation, one rounding to C's type."""
+    _gemm_finish(desc, _gemm_products(desc, a, b), c, bias, residual, pre_out)
+
+
+def _unary_value(op, xv, param):
+    from scipy.special import erf
+    sig = lambda v: 1 / (1 + np.exp(-v))  # noqa: E731
+    return {L.ERF: lambda: erf(xv), L.SQRT: lambda: np.sqrt(xv), L.EXP: lambda: np.exp(xv), L.LOG: lambda: np.log(xv),
+            L.TANH: lambda: np.tanh(xv), L.RELU: lambda: np.maximum(xv, 0), L.SIGMOID: lambda: sig(xv),
+            L.RECIPROCAL: lambda: 1 / xv, L.GELU: lambda: 0.5 * xv * (1 + erf(xv / math.sqrt(2.0))),
+            L.SWISH: lambda: xv * sig(xv), L.SCALE: lambda: xv * np.float32(param).astype(np.float64),
+            L.IDENTITY: lambda: xv}[op]()
+
+
+def _unary_derivative(op, xv, param):
+    from scipy.special import erf
+    sig = 1 / (1 + np.exp(-xv))
+    return {L.ERF: lambda: 2 / math.sqrt(math.pi) * np.exp(-xv * xv), L.SQRT: lambda: 0.5 / np.sqrt(xv),
+            L.EXP: lambda: np.exp(xv), L.LOG: lambda: 1 / xv, L.TANH: lambda: 1 - np.tanh(xv)**2,
+            L.RELU: lambda: (xv > 0).astype(np.float64), L.SIGMOID: lambda: sig * (1 - sig),
+            L.RECIPROCAL: lambda: -1 / (xv * xv),
+            L.GELU: lambda: 0.5 * (1 + erf(xv / math.sqrt(2.0))) + xv * np.exp(-0.5 * xv * xv) / math.sqrt(2 * math.pi),
+            L.SWISH: lambda: sig * (1 + xv * (1 - sig)), L.SCALE: lambda: np.full_like(xv, np.float32(param)),
+            L.IDENTITY: lambda: np.ones_like(xv)}[op]()
+
+
 def unary(op, x, y, n, param):
-    xv = x.reshape(-1)[:n].astype(np.float64)
-    if op == L.SCALE:
-        r = xv * np.float32(param).astype(np.float64)
-    elif op == L.IDENTITY:
-        r = xv
-    elif op == L.RELU:
-        r = np.maximum(xv, 0)
-    else:
-        raise NotImplementedError("unary op %d" % op)
-    y.reshape(-1)[:n] = r.astype(y.dtype)
+    y.reshape(-1)[:n] = _unary_value(op, x.reshape(-1)[:n].astype(np.float64), param).astype(y.dtype)
+
+
+def unary_backward(op, x, dy, dx, n, param):
+    """dmlhip_unary_backward_*: dx = dy * f'(x), x the forward input."""
+    xv, dv = x.reshape(-1)[:n].astype(np.float64), dy.reshape(-1)[:n].astype(np.float64)
+    dx.reshape(-1)[:n] = (dv * _unary_derivative(op, xv, param)).astype(dx.dtype)
+
+
+def layernorm(x, residual, gamma, beta, y, sum_out, mean, rstd, rows, cols, eps):
+    s = x.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+    if residual is not None:
+        s = s + residual.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+        if sum_out is not None:
+            sum_out.reshape(-1)[:rows * cols] = s.reshape(-1).astype(sum_out.dtype)
+            s = sum_out.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)   # the kernel normalises what it stores
+    elif sum_out is not None:
+        sum_out.reshape(-1)[:rows * cols] = s.reshape(-1).astype(sum_out.dtype)
+    mu = s.mean(-1, keepdims=True)
+    var = ((s - mu)**2).mean(-1, keepdims=True)
+    rs = 1 / np.sqrt(var + np.float32(eps).astype(np.float64))
+    out = (s - mu) * rs * gamma.reshape(-1)[:cols].astype(np.float64) + beta.reshape(-1)[:cols].astype(np.float64)
+    y.reshape(-1)[:rows * cols] = out.reshape(-1).astype(y.dtype)
+    if mean is not None:
+        mean.reshape(-1)[:rows] = mu.reshape(-1).astype(np.float32)
+    if rstd is not None:
+        rstd.reshape(-1)[:rows] = rs.reshape(-1).astype(np.float32)
+
+
+def layernorm_backward(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, rows, cols):
+    d = dy.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+    xv = x.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+    mu = mean.reshape(-1)[:rows].astype(np.float64).reshape(rows, 1)
+    rs = rstd.reshape(-1)[:rows].astype(np.float64).reshape(rows, 1)
+    xhat = (xv - mu) * rs
+    if dgamma is not None:
+        dgamma.reshape(-1)[:cols] = (d * xhat).sum(0).astype(np.float32)
+    if dbeta is not None:
+        dbeta.reshape(-1)[:cols] = d.sum(0).astype(np.float32)
+    g = d * gamma.reshape(-1)[:cols].astype(np.float64)
+    res = (g - g.mean(-1, keepdims=True) - xhat * (g * xhat).mean(-1, keepdims=True)) * rs
+    dx.reshape(-1)[:rows * cols] = res.reshape(-1).astype(dx.dtype)
+
+
+def _attn_view(desc, buf, strides, seq):
+    shape = (int(desc.batch[0]), int(desc.batch[1]), int(seq), int(desc.head_dim))
+    return _view(buf, 0, shape, [int(strides[0]), int(strides[1]), int(strides[2]), 1])
+
+
+def _attn_probs(desc, q, k, mask, mask_stride):
+    qv = _attn_view(desc, q, desc.q_stride, desc.seq_q).astype(np.float64)
+    kv = _attn_view(desc, k, desc.k_stride, desc.seq_k).astype(np.float64)
+    scores = np.einsum("abqd,abkd->abqk", qv, kv) * np.float32(desc.scale).astype(np.float64)
+    if mask is not None:
+        mv = _view(mask, 0, (int(desc.batch[0]), int(desc.batch[1]), int(desc.seq_k)),
+                   [int(mask_stride[0]), int(mask_stride[1]), 1]).astype(np.float64)
+        scores = scores + mv[:, :, None, :]
+    m = scores.max(-1, keepdims=True)
+    e = np.exp(scores - m)
+    return e / e.sum(-1, keepdims=True), (m + np.log(e.sum(-1, keepdims=True)))[..., 0]
+
+
+def _strided_store(buf, desc, strides, seq, value):
+    shape = value.shape
+    out = as_strided(buf.reshape(-1), shape=shape, strides=[int(s) * buf.itemsize for s in list(strides)[:3]] + [buf.itemsize])
+    out[...] = value.astype(buf.dtype)
+    del desc, seq
+
+
+def attention(desc, q, k, v, o, lse, mask=None, mask_stride=None):
+    """dmlhip_attention(_masked)_f16: softmax(scale q k^T [+ mask]) v on [batch0, batch1, seq, head] views."""
+    p, l = _attn_probs(desc, q, k, mask, mask_stride)
+    vv = _attn_view(desc, v, desc.v_stride, desc.seq_k).astype(np.float64)
+    _strided_store(o, desc, desc.o_stride, desc.seq_q, np.einsum("abqk,abkd->abqd", p, vv))
+    if lse is not None:
+        lse.reshape(-1)[:l.size] = l.reshape(-1).astype(np.float32)
+
+
+def attention_backward(desc, grad, q, k, v, o, lse, d_o, dq, dk, dv, mask=None, mask_stride=None):
+    p, _ = _attn_probs(desc, q, k, mask, mask_stride)
+    qv = _attn_view(desc, q, desc.q_stride, desc.seq_q).astype(np.float64)
+    kv = _attn_view(desc, k, desc.k_stride, desc.seq_k).astype(np.float64)
+    vv = _attn_view(desc, v, desc.v_stride, desc.seq_k).astype(np.float64)
+    g = _attn_view(desc, d_o, grad.o_stride, desc.seq_q).astype(np.float64)
+    dp = np.einsum("abqd,abkd->abqk", g, vv)
+    ds = p * (dp - (dp * p).sum(-1, keepdims=True)) * np.float32(desc.scale).astype(np.float64)
+    _strided_store(dv, desc, grad.v_stride, desc.seq_k, np.einsum("abqk,abqd->abkd", p, g))
+    _strided_store(dq, desc, grad.q_stride, desc.seq_q, np.einsum("abqk,abkd->abqd", ds, kv))
+    _strided_store(dk, desc, grad.k_stride, desc.seq_k, np.einsum("abqk,abqd->abkd", ds, qv))
+    del o, lse
 
 
 def binary(op, a, b, c, ndim, shape, a_strides, b_strides):
@@ -160,6 +273,50 @@ class Emulator:
                 x = self._typed(x, want)
                 y = self._typed(y, want)
                 unary(op, x, y, n, param)
+            elif call.symbol in ("dmlhip_unary_backward_f16", "dmlhip_unary_backward_f32"):
+                op, x, dy, dx, n, param = args[:6]
+                unary_backward(op, x, dy, dx, n, param)
+            elif call.symbol in ("dmlhip_sum_f16", "dmlhip_sum_f32"):
+                inputs, count, out, n = args[:4]
+                assert len(inputs) == count
+                out.reshape(-1)[:n] = sum(i.reshape(-1)[:n].astype(np.float64) for i in inputs).astype(out.dtype)
+            elif call.symbol in ("dmlhip_softmax_f16", "dmlhip_softmax_f32"):
+                x, y, rows, cols = args[:4]
+                xv = x.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+                e = np.exp(xv - xv.max(-1, keepdims=True))
+                y.reshape(-1)[:rows * cols] = (e / e.sum(-1, keepdims=True)).reshape(-1).astype(y.dtype)
+            elif call.symbol in ("dmlhip_layernorm_f16", "dmlhip_layernorm_f32"):
+                layernorm(*args[:11])
+            elif call.symbol in ("dmlhip_layernorm_backward_f16", "dmlhip_layernorm_backward_f32"):
+                layernorm_backward(*args[:10])
+            elif call.symbol == "dmlhip_attention_f16":
+                attention(*args[:6])
+            elif call.symbol == "dmlhip_attention_masked_f16":
+                desc, q, k, v, mask, ms, o, lse = args[:8]
+                attention(desc, q, k, v, o, lse, mask, ms)
+            elif call.symbol == "dmlhip_attention_backward_f16":
+                attention_backward(*args[:11])
+            elif call.symbol == "dmlhip_attention_masked_backward_f16":
+                desc, grad, q, k, v, mask, ms, o, lse, d_o, dq, dk, dv = args[:13]
+                attention_backward(desc, grad, q, k, v, o, lse, d_o, dq, dk, dv, mask, ms)
+            elif call.symbol == "dmlhip_gemm_f16_grouped":
+                desc, groups, a, b, c, bias = args[:6]
+                for i in range(groups):
+                    bi = None if bias is None else self._typed(bias[i], np.float16 if desc.bias_dtype == L.F16 else np.float32)
+                    gemm(desc, a[i], b[i], c[i], bi, None, None)
+            elif call.symbol == "dmlhip_gemm_f16_grouped_asum":
+                desc, groups, a, b, c, asum, asum_dtype = args[:7]
+                for i in range(groups):
+                    gemm(desc, a[i], b[i], c[i], None, None, None)
+                    av = _view(a[i], 0, (desc.m, desc.k), (desc.a_stride_m, desc.a_stride_k)).astype(np.float64)
+                    asum[i].reshape(-1)[:desc.m] = av.sum(1).astype(np.float16 if asum_dtype == L.F16 else np.float32)
+            elif call.symbol == "dmlhip_gemm_f16_ksum":
+                desc, groups, a, b, c, bias, residual = args[:7]
+                # the kernel keeps the sum of the products in its accumulators: one rounding at the end
+                total = sum(_gemm_products(desc, a[i], b[i]) for i in range(groups))
+                if bias is not None:
+                    bias = self._typed(bias, np.float16 if desc.bias_dtype == L.F16 else np.float32)
+                _gemm_finish(desc, total, c, bias, residual, None)
             elif call.symbol in ("dmlhip_binary_f16", "dmlhip_binary_f32"):
                 op, a, b, c, ndim, shape, sa, sb = args[:8]
                 binary(op, a, b, c, ndim, shape, sa, sb)
@@ -211,6 +368,8 @@ class Emulator:
             return float(a.value)
         if isinstance(a, T.I64Array):
             return tuple(a.values)
+        if isinstance(a, T.PtrArray):
+            return [arrays[c].reshape(-1) for c in a.conns]
         if isinstance(a, T.Struct):
             return a.value
         if isinstance(a, T.Workspace):
@@ -222,27 +381,40 @@ class Emulator:
         raise NotImplementedError(type(a).__name__)
 
 
+def _memory(sdfg, arrays, name, np_dtype):
+    """The flat memory an array name stands for: its own allocation, or for a view the base's memory from the view's
+    offset on (descriptors carry the view's strides)."""
+    d = sdfg.arrays[name]
+    if d.view_of is not None:
+        return _memory(sdfg, arrays, d.view_of, np_dtype).reshape(-1)[d.view_offset:]
+    if name not in arrays:
+        if name in sdfg.constants:
+            arrays[name] = sdfg.constants[name].detach().cpu().numpy().astype(np_dtype[d.dtype]).reshape(d.shape)
+        else:
+            arrays[name] = np.full(d.shape, np.nan, dtype=np_dtype[d.dtype])
+    return arrays[name]
+
+
 def run_state(sdfg, state, arrays):
     """Run an expanded state: `arrays` maps array names to NumPy arrays (inputs given, outputs and transients are
-    allocated here when missing). Views are not supported."""
+    allocated here when missing)."""
     import torch
     np_dtype = {torch.float16: np.float16, torch.float32: np.float32, torch.int64: np.int64}
-    ws = max([int(getattr(n, "workspace_bytes", 0)) for n in state.library_nodes()] + [0])
+    ws = max([int(getattr(n, "workspace_bytes", 0)) for n in state.nodes()] + [0])
     em = Emulator(ws)
     for node in state.topological_sort():
         if not getattr(node, "calls", None):
             continue
         bound = {}
         for e in list(state.in_edges(node)) + list(state.out_edges(node)):
-            name = e.data.data
-            d = sdfg.arrays[name]
-            if d.view_of is not None:
-                raise NotImplementedError("views")
-            if name not in arrays:
-                if name in sdfg.constants:
-                    arrays[name] = sdfg.constants[name].detach().cpu().numpy().astype(np_dtype[d.dtype]).reshape(d.shape)
-                else:
-                    arrays[name] = np.full(d.shape, np.nan, dtype=np_dtype[d.dtype])
-            bound[e.dst_conn if e.dst is node else e.src_conn] = arrays[name]
+            bound[e.dst_conn if e.dst is node else e.src_conn] = _memory(sdfg, arrays, e.data.data, np_dtype)
         em.run(node, bound)
     return em
+
+
+def run_sdfg(sdfg, arrays):
+    """Every state in order (forward, then backward). Returns the list of calls made."""
+    log = []
+    for st in sdfg.states():
+        log += run_state(sdfg, st, arrays).log
+    return log

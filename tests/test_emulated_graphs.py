@@ -1,0 +1,133 @@
+"""Whole graphs without a GPU: the BERT encoder layer - as the exporter emits it, and after the fusion passes - is
+differentiated, expanded, and the calls its tasklets make are interpreted by tests/abi_emulator.py on NumPy arrays.
+Compared with the oracle, this checks everything on the host side of the C ABI for the headline workload: the fusion
+passes, the reverse nodes and gradient accumulation of the autodiff generator, the views that replace Transpose /
+Reshape nodes, every descriptor, operand order, pointer table and workspace offset. (The kernels behind the ABI are
+checked against the same oracle in tests/test_gpu_graphs.py.)"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bert_layer as OB
+from tests.abi_emulator import run_sdfg
+from tests.util import assert_close, rng
+
+B, S, H, HEADS, FFN = 2, 64, 128, 2, 256
+
+
+def _inputs(dtype, seed=1234):
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    p = OB.init_params(H, FFN, seed, np.float32, bias_std=0.02)
+    r = rng(seed + 1)
+    p["ln1_g"], p["ln2_g"] = r.uniform(0.5, 1.5, H).astype(np.float32), r.uniform(0.5, 1.5, H).astype(np.float32)
+    p["ln1_b"], p["ln2_b"] = (r.standard_normal(H) * 0.1).astype(np.float32), (r.standard_normal(H) * 0.1).astype(np.float32)
+    x = r.standard_normal((B, S, H)).astype(npdt)
+    dy = rng(77).standard_normal((B, S, H)).astype(npdt)
+    return x, dy, {k: v.astype(npdt) for k, v in p.items()}
+
+
+def _oracle(x, dy, p):
+    x64, p64 = x.astype(np.float64), {k: v.astype(np.float64) for k, v in p.items()}
+    y, saved = OB.forward(x64, p64, HEADS, eps=1e-5, keep=True)
+    return y, OB.backward(x64, p64, HEADS, dy.astype(np.float64), saved, eps=1e-5)
+
+
+def _check(arrays, x, dy, p, dtype, grads=True):
+    y, want = _oracle(x, dy, p)
+    f16 = dtype == torch.float16
+    assert_close(arrays["y"], y, dtype, "y", **({} if f16 else dict(rtol=1e-4, atol=2e-5)))
+    if not grads:
+        return
+    assert_close(arrays["gradient_x"], want["x"], dtype, "dx", **({} if f16 else dict(rtol=1e-4, atol=2e-5)))
+    for n in OB.PARAM_NAMES:
+        scale = float(np.abs(want[n]).max())
+        tol = dict(rtol=2e-2, atol=2e-2 * scale + 1e-3) if f16 else dict(rtol=1e-4, atol=1e-5 * max(scale, 1.0))
+        assert_close(arrays["gradient_" + n], want[n], dtype, "d" + n, **tol)
+
+
+@pytest.mark.parametrize("dtype,attention", [(torch.float16, True), (torch.float16, False), (torch.float32, False)])
+def test_fused_bert_layer_forward_and_backward(dtype, attention):
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.transformation import fusion
+    x, dy, p = _inputs(dtype)
+    sdfg = graphs.bert_encoder_layer(B, S, H, HEADS, FFN, dtype, eps=1e-5)
+    fusion.auto_optimize(sdfg, training=True, attention=attention, gelu_epilogue=not attention)
+    add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + OB.PARAM_NAMES,
+                      grad_dtypes={n: torch.float32 for n in OB.PARAM_NAMES})
+    if attention:
+        fusion.optimize_backward(sdfg)
+    expand_onnx_nodes(sdfg)
+    arrays = {"x": x.copy(), "gradient_y": dy.copy(), **{k: v.copy() for k, v in p.items()}}
+    log = run_sdfg(sdfg, arrays)
+    if attention:
+        assert sorted(set(log)) == ["dmlhip_attention_backward_f16", "dmlhip_attention_f16", "dmlhip_gemm_f16_grouped",
+                                    "dmlhip_gemm_f16_grouped_asum", "dmlhip_gemm_f16_ksum", "dmlhip_gemm_f16_ws",
+                                    "dmlhip_layernorm_backward_f16", "dmlhip_layernorm_f16", "dmlhip_unary_backward_f16",
+                                    "dmlhip_unary_f16"]
+        assert len(log) == 19       # the launch count of the benchmarked step
+    _check(arrays, x, dy, p, dtype)
+    # inputs are read-only
+    assert np.array_equal(arrays["x"], x) and all(np.array_equal(arrays[k], v) for k, v in p.items())
+
+
+def test_exporter_form_bert_layer_differentiates_without_any_fusion():
+    """The graph exactly as imported (MatMul, Reshape, Transpose, the nine-node LayerNorm and five-node GELU chains):
+    every node has a reverse implementation, among them MatMul (the reference expands it to an Einsum first,
+    backward_pass_generator.py:425-494) and Reshape."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.runtime import expand_onnx_nodes
+    dtype = torch.float32
+    x, dy, p = _inputs(dtype)
+    sdfg = graphs.bert_encoder_layer(B, S, H, HEADS, FFN, dtype, eps=1e-5)
+    names = {n.schema.name for n in sdfg.states()[0].library_nodes()}
+    assert {"MatMul", "Reshape", "Transpose", "ReduceMean", "Pow", "Sqrt", "Erf", "Softmax"} <= names
+    grads = add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + OB.PARAM_NAMES)
+    assert set(grads) == {"x"} | set(OB.PARAM_NAMES)
+    expand_onnx_nodes(sdfg)
+    arrays = {"x": x.copy(), "gradient_y": dy.copy(), **{k: v.copy() for k, v in p.items()}}
+    run_sdfg(sdfg, arrays)
+    _check(arrays, x, dy, p, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_inference_graph(dtype):
+    from daceml_amd import graphs
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.transformation import fusion
+    x, dy, p = _inputs(dtype)
+    sdfg = graphs.bert_encoder_layer(B, S, H, HEADS, FFN, dtype, eps=1e-5)
+    fusion.auto_optimize(sdfg)
+    expand_onnx_nodes(sdfg)
+    arrays = {"x": x.copy(), **{k: v.copy() for k, v in p.items()}}
+    run_sdfg(sdfg, arrays)
+    _check(arrays, x, dy, p, dtype, grads=False)
+
+
+def test_masked_attention_graph_forward_and_backward():
+    """The chain with the additive mask through fusion, autodiff and the masked entry points."""
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.transformation import fusion
+    from oracle import ops as O
+    from tests.test_zx_attention_mask import _chain
+    b, h, sq, sk = 2, 3, 40, 48
+    g = _chain((b, 1, 1, sk), b=b, h=h, sq=sq, sk=sk)
+    assert fusion.auto_optimize(g.sdfg)["attention"] == 1
+    add_backward_pass(g.sdfg, g.state, ["o"], ["q", "k", "v"])
+    expand_onnx_nodes(g.sdfg)
+    r = rng(5)
+    q, k, v = (r.standard_normal((b, h, n, 64)).astype(np.float16) for n in (sq, sk, sk))
+    do = r.standard_normal((b, h, sq, 64)).astype(np.float16)
+    mask = np.zeros((b, 1, 1, sk), np.float16)
+    mask[1, :, :, 30:] = -10000.0
+    arrays = {"q": q.copy(), "k": k.copy(), "v": v.copy(), "mask": mask.copy(), "gradient_o": do.copy()}
+    log = run_sdfg(g.sdfg, arrays)
+    assert log == ["dmlhip_attention_masked_f16", "dmlhip_attention_masked_backward_f16"]
+    f64 = lambda t: t.astype(np.float64)  # noqa: E731
+    want, _ = O.attention(f64(q), f64(k), f64(v), 0.125, f64(mask))
+    assert_close(arrays["o"], want, torch.float16, "masked attention (emulated)")
+    for name, w in zip(("q", "k", "v"), O.attention_backward(f64(q), f64(k), f64(v), 0.125, f64(do), f64(mask))):
+        assert_close(arrays["gradient_" + name], w, torch.float16, "d" + name, atol=1e-2 * max(1.0, float(np.abs(w).max())))

@@ -91,6 +91,72 @@ def test_gemm_refuses_what_the_reference_refuses():
         O.gemm(np.zeros((M, K)), np.zeros((K, N)), np.zeros((M, 1)))
 
 
+def _gemm_gradients(a, b, c, dy, ta, tb, alpha, beta, ckind):
+    """Autograd in fp64 on the definition Y = alpha op(A) op(B) + beta C."""
+    ta_, tb_ = (torch.tensor(t.astype(np.float64), requires_grad=True) for t in (a, b))
+    tc = None if c is None else torch.tensor(c.astype(np.float64), requires_grad=True)
+    y = alpha * ((ta_.T if ta else ta_) @ (tb_.T if tb else tb_))
+    if tc is not None:
+        y = y + beta * tc
+    y.backward(torch.tensor(dy.astype(np.float64)))
+    return ta_.grad.numpy(), tb_.grad.numpy(), None if tc is None or beta == 0 else tc.grad.numpy()
+
+
+BACKWARD_CASES = [c for c in CASES if c[:2] in ((0, 0), (1, 1), (0, 1))]
+
+
+def _backward_graph(dtype, ta, tb, alpha, beta, ckind):
+    from daceml_amd.autodiff import add_backward_pass
+    g, a, b, c, want = _case(dtype, ta, tb, alpha, beta, ckind)
+    wrt = ["a", "b"] + (["c"] if c is not None and beta != 0 else [])
+    grads = add_backward_pass(g.sdfg, g.state, ["y"], wrt)
+    assert grads == {n: "gradient_" + n for n in wrt}
+    dy = rng(9).standard_normal((M, N)).astype(a.dtype)
+    return g, a, b, c, dy, wrt
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("ta,tb,alpha,beta,ckind", BACKWARD_CASES)
+def test_gemm_reverse_node_lowers_correctly(dtype, ta, tb, alpha, beta, ckind):
+    """Gemm has a reverse implementation of its own (A and B as for the Einsum PureGemm builds, C = beta times the
+    incoming gradient, summed over the rows for a vector): checked against autograd through the emulated calls."""
+    from daceml_amd.runtime import expand_onnx_nodes
+    from tests.abi_emulator import run_sdfg
+    g, a, b, c, dy, wrt = _backward_graph(dtype, ta, tb, alpha, beta, ckind)
+    expand_onnx_nodes(g.sdfg)
+    arrays = {"a": a.copy(), "b": b.copy(), "gradient_y": dy.copy()}
+    if c is not None:
+        arrays["c"] = c.copy()
+    run_sdfg(g.sdfg, arrays)
+    wa, wb, wc = _gemm_gradients(a, b, c, dy, ta, tb, alpha, beta, ckind)
+    tol = dict(rtol=2e-2, atol=2e-2) if dtype == torch.float16 else dict(rtol=1e-5, atol=2e-6)
+    assert_close(arrays["gradient_a"], wa, dtype, "dA %s" % ((ta, tb, alpha, beta, ckind), ), **tol)
+    assert_close(arrays["gradient_b"], wb, dtype, "dB", **tol)
+    if "c" in wrt:
+        assert arrays["gradient_c"].shape == c.shape
+        assert_close(arrays["gradient_c"], wc, dtype, "dC", **(tol if dtype == torch.float32 else dict(rtol=2e-2, atol=5e-2)))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("ta,tb,alpha,beta,ckind", BACKWARD_CASES[::3])
+def test_gemm_backward_on_gpu(dtype, ta, tb, alpha, beta, ckind):
+    from daceml_amd.runtime import CompiledSDFG
+    g, a, b, c, dy, wrt = _backward_graph(dtype, ta, tb, alpha, beta, ckind)
+    prog = CompiledSDFG(g.sdfg)
+    args = {"a": dev(a), "b": dev(b), "y": torch.empty((M, N), dtype=dtype, device="cuda"), "gradient_y": dev(dy)}
+    if c is not None:
+        args["c"] = dev(c)
+    outs = {n: torch.full(tuple(g.sdfg.arrays["gradient_" + n].shape), float("nan"), dtype=dtype, device="cuda") for n in wrt}
+    prog(**args, **{"gradient_" + n: t for n, t in outs.items()})
+    wa, wb, wc = _gemm_gradients(a, b, c, dy, ta, tb, alpha, beta, ckind)
+    tol = dict(rtol=2e-2, atol=2e-2) if dtype == torch.float16 else dict(rtol=1e-5, atol=2e-6)
+    assert_close(host(outs["a"]), wa, dtype, "dA %s" % ((ta, tb, alpha, beta, ckind), ), **tol)
+    assert_close(host(outs["b"]), wb, dtype, "dB", **tol)
+    if "c" in wrt:
+        assert_close(host(outs["c"]), wc, dtype, "dC", **(tol if dtype == torch.float32 else dict(rtol=2e-2, atol=5e-2)))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("ta,tb,alpha,beta,ckind", CASES)
