@@ -431,8 +431,8 @@ def test_install_registers_forward_and_backward_implementations(monkeypatch):
     registered = dace_plugin.install()
     assert sorted(registered["forward"]) == sorted(["Softmax", "Einsum", "MatMul", "Gemm", "Add", "Mul", "Conv",
                                                     "Transpose", "Relu", "ReduceSum"])
-    assert sorted(registered["backward"]) == sorted(["Softmax", "Einsum", "Add", "Mul", "Conv", "Transpose", "Relu",
-                                                     "ReduceSum"])
+    assert sorted(registered["backward"]) == sorted(["Softmax", "Einsum", "MatMul", "Gemm", "Add", "Mul", "Conv",
+                                                     "Transpose", "Relu", "ReduceSum"])
     # both registrations of the forward side (registry and node class)
     assert set(rec.forward_registry) == set(registered["forward"])
     assert all("hip" in rec.node_implementations[op] for op in registered["forward"])
