@@ -336,6 +336,29 @@ class Emulator:
                 desc, x, w, bias, y = args[:5]
                 dt = np.float16 if call.symbol.endswith("f16") else np.float32
                 conv2d(desc, self._typed(x, dt), w, bias, self._typed(y, dt))
+            elif call.symbol == "dmlhip_conv2d_gated_f32":
+                desc, x, gate, w, bias, y = args[:6]
+                n = desc.n * desc.c * desc.h * desc.w
+                gated = (x.reshape(-1)[:n].astype(np.float64).reshape(desc.n, desc.c, desc.h * desc.w) *
+                         gate.reshape(-1)[:desc.n * desc.c].astype(np.float64).reshape(desc.n, desc.c, 1))
+                conv2d(desc, gated.reshape(-1), w, bias, y)
+            elif call.symbol == "dmlhip_conv2d_expand_depthwise_f32":
+                pw, dw, x, w_pw, b_pw, w_dw, b_dw, y = args[:8]
+                mid = np.empty(pw.n * pw.m * pw.h * pw.w, dtype=np.float64)   # the expanded tensor is never rounded to memory
+                conv2d(pw, x, w_pw, b_pw, mid)
+                conv2d(dw, mid, w_dw, b_dw, y)
+            elif call.symbol in ("dmlhip_row_dot_f16", "dmlhip_row_dot_f32"):
+                a, b, y, rows, cols = args[:5]
+                av = a.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+                bv = b.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+                y.reshape(-1)[:rows] = (av * bv).sum(1).astype(y.dtype)
+            elif call.symbol in ("dmlhip_row_affine_f16", "dmlhip_row_affine_f32"):
+                a, sc, t, scale, y, rows, cols = args[:7]
+                av = a.reshape(-1)[:rows * cols].astype(np.float64).reshape(rows, cols)
+                f = 1.0 if scale is None else float(scale.reshape(-1)[0])
+                res = av * sc.reshape(-1)[:rows].astype(np.float64).reshape(rows, 1) + \
+                    t.reshape(-1)[:rows].astype(np.float64).reshape(rows, 1) * f
+                y.reshape(-1)[:rows * cols] = res.reshape(-1).astype(y.dtype)
             elif call.symbol == "dmlhip_conv2d_backward_data_f32":
                 desc, dy, w, dx = args[:4]
                 conv2d_backward(desc, "data", dy, w, dx)

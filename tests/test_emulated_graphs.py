@@ -131,3 +131,79 @@ def test_masked_attention_graph_forward_and_backward():
     assert_close(arrays["o"], want, torch.float16, "masked attention (emulated)")
     for name, w in zip(("q", "k", "v"), O.attention_backward(f64(q), f64(k), f64(v), 0.125, f64(do), f64(mask))):
         assert_close(arrays["gradient_" + name], w, torch.float16, "d" + name, atol=1e-2 * max(1.0, float(np.abs(w).max())))
+
+
+# ----------------------------------------------------------------------------- MBConv block
+def _mbconv(seed=4, b=3, cin=16, hw=28, cout=24):
+    from daceml_amd import graphs
+    r = rng(seed)
+    sdfg = graphs.mbconv_block(b, cin, hw, expand=6, cout=cout, se_reduce=4, stride=2, dtype=torch.float32)
+    x = r.standard_normal((b, cin, hw, hw)).astype(np.float32)
+    params = {}
+    for name, desc in sdfg.arglist().items():
+        if name in ("x", "y"):
+            continue
+        if name.endswith("_w"):
+            fan_in = int(np.prod(desc.shape[1:]))
+            params[name] = (r.standard_normal(desc.shape) * np.sqrt(2.0 / fan_in)).astype(np.float32)
+        else:
+            params[name] = (r.standard_normal(desc.shape) * 0.1).astype(np.float32)
+    return sdfg, x, params
+
+
+def _mbconv_reference(x, p, dy=None):
+    """The block in torch, fp64 (its structure: expand 1x1 + swish, depthwise 3x3 stride 2 + swish, squeeze-excite,
+    project 1x1), with autograd for the gradients."""
+    import torch.nn.functional as F
+    t = {k: torch.tensor(v.astype(np.float64), requires_grad=True) for k, v in p.items()}
+    xt = torch.tensor(x.astype(np.float64), requires_grad=True)
+    sw = lambda v: v * torch.sigmoid(v)  # noqa: E731
+    h = sw(F.conv2d(xt, t["expand_w"], t["expand_b"]))
+    h = sw(F.conv2d(h, t["dw_w"], t["dw_b"], stride=2, padding=1, groups=h.shape[1]))
+    g = h.mean((2, 3), keepdim=True)
+    g = torch.sigmoid(F.conv2d(sw(F.conv2d(g, t["se1_w"], t["se1_b"])), t["se2_w"], t["se2_b"]))
+    y = F.conv2d(h * g, t["proj_w"], t["proj_b"])
+    grads = None
+    if dy is not None:
+        y.backward(torch.tensor(dy.astype(np.float64)))
+        grads = {"x": xt.grad.numpy(), **{k: v.grad.numpy() for k, v in t.items()}}
+    return y.detach().numpy(), grads
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_mbconv_block_forward(fused):
+    import copy
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.transformation import fusion
+    sdfg, x, p = _mbconv(cin=16, hw=28)
+    want, _ = _mbconv_reference(x, p)
+    if fused:
+        stats = fusion.auto_optimize(sdfg)
+        assert stats["gated_conv"] == 1 and stats["expand_depthwise"] == 1
+    expand_onnx_nodes(sdfg)
+    arrays = {"x": x.copy(), **copy.deepcopy(p)}
+    log = run_sdfg(sdfg, arrays)
+    if fused:
+        assert "dmlhip_conv2d_expand_depthwise_f32" in log and "dmlhip_conv2d_gated_f32" in log
+    assert_close(arrays["y"], want, torch.float32, "mbconv forward fused=%s" % fused, rtol=1e-4, atol=1e-5)
+
+
+def test_mbconv_block_training_step():
+    import copy
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.transformation import fusion
+    sdfg, x, p = _mbconv(cin=16, hw=28)
+    fusion.auto_optimize(sdfg, training=True)
+    wrt = ["x"] + sorted(p)
+    grads = add_backward_pass(sdfg, sdfg.states()[0], ["y"], wrt)
+    fusion.optimize_backward(sdfg)
+    expand_onnx_nodes(sdfg)
+    dy = rng(6).standard_normal(tuple(sdfg.arrays["y"].shape)).astype(np.float32)
+    arrays = {"x": x.copy(), "gradient_y": dy.copy(), **copy.deepcopy(p)}
+    run_sdfg(sdfg, arrays)
+    want_y, want = _mbconv_reference(x, p, dy)
+    assert_close(arrays["y"], want_y, torch.float32, "mbconv training forward", rtol=1e-4, atol=1e-5)
+    for n in wrt:
+        scale = max(1.0, float(np.abs(want[n]).max()))
+        assert_close(arrays[grads[n]], want[n], torch.float32, "mbconv d" + n, rtol=1e-4, atol=1e-5 * scale)
