@@ -384,6 +384,10 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region, launch a plain 128 MiB -> 128 MiB copy kernel three times: under "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its counters give the scale of those counters")
+    ap.add_argument("--gemm-config", type=int, default=-1,
+                    help="pin the tile configuration of the fp16 contraction kernel for the whole run (the library's "
+                         "diagnostic switch; -1 = the library's own choice). For comparing configurations, not for the "
+                         "reported figure: the JSON line carries the value in config.gemm_config")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures the single-GPU path only: this build uses one GPU (no collectives, no sharding); "
@@ -393,6 +397,9 @@ def main():
         sys.exit("bench.py needs a GPU")
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
+    if a.gemm_config >= 0:
+        from daceml_amd import _lib
+        _lib.load().dmlhip_debug_force_gemm_config(a.gemm_config)
 
     if a.workload == "module_bert":
         return module_workload(device, a.steps, a.warmup)
@@ -464,7 +471,8 @@ def main():
         "dtype": "f16 (fp32 accumulate, fp32 master gradients)", "data": "synthetic",
         "config": {"workload": "BERT-large encoder layer forward + autodiff backward, B=8 S=512 hidden=1024 heads=16 "
                                "ffn=4096, fp16 (BASELINE.json configs[4])",
-                   "launches_per_step": len(prog.launches)},
+                   "launches_per_step": len(prog.launches),
+                   **({"gemm_config": a.gemm_config} if a.gemm_config >= 0 else {})},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_FP16_TFLOPS, 4),
                      "traffic": GEMM_TRAFFIC_BYTES_PER_STEP["fetched"] + GEMM_TRAFFIC_BYTES_PER_STEP["written"],
