@@ -142,6 +142,63 @@ def layernorm_backward(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, rows, cols):
     dx.reshape(-1)[:rows * cols] = res.reshape(-1).astype(dx.dtype)
 
 
+def _bn_tensor(buf, n, c, hw):
+    return buf.reshape(-1)[:n * c * hw].astype(np.float64).reshape(n, c, hw)
+
+
+def _bn_vec(buf, c):
+    return buf.reshape(-1)[:c].astype(np.float64).reshape(1, c, 1)
+
+
+def _act_derivative(kind, z):
+    if kind == L.ACT_NONE:
+        return np.ones_like(z)
+    if kind == L.ACT_RELU:
+        return (z > 0).astype(np.float64)
+    if kind == L.ACT_SWISH:
+        sg = 1 / (1 + np.exp(-z))
+        return sg * (1 + z * (1 - sg))
+    raise ValueError(kind)
+
+
+def batchnorm_inference(x, scale, bias, mean, var, y, n, c, hw, eps, act=L.ACT_NONE):
+    z = (_bn_tensor(x, n, c, hw) - _bn_vec(mean, c)) / np.sqrt(_bn_vec(var, c) + np.float32(eps).astype(np.float64)) * \
+        _bn_vec(scale, c) + _bn_vec(bias, c)
+    y.reshape(-1)[:n * c * hw] = _act(act, z).reshape(-1).astype(y.dtype)
+
+
+def batchnorm_training(x, scale, bias, in_mean, in_var, y, out_mean, out_var, saved_mean, saved_var, n, c, hw, eps, momentum,
+                       act=L.ACT_NONE):
+    xv = _bn_tensor(x, n, c, hw)
+    mu = xv.mean((0, 2), keepdims=True)
+    var = ((xv - mu)**2).mean((0, 2), keepdims=True)
+    mom = np.float32(momentum).astype(np.float64)
+    new_mean = _bn_vec(in_mean, c) * mom + mu * (1 - mom)      # before the outputs are written: out_* may alias in_*
+    new_var = _bn_vec(in_var, c) * mom + var * (1 - mom)
+    z = (xv - mu) / np.sqrt(var + np.float32(eps).astype(np.float64)) * _bn_vec(scale, c) + _bn_vec(bias, c)
+    y.reshape(-1)[:n * c * hw] = _act(act, z).reshape(-1).astype(y.dtype)
+    for buf, val in ((out_mean, new_mean), (out_var, new_var), (saved_mean, mu), (saved_var, var)):
+        if buf is not None:
+            buf.reshape(-1)[:c] = val.reshape(-1).astype(buf.dtype)
+
+
+def batchnorm_backward(dy, x, scale, bias, saved_mean, saved_var, dx, dscale, dbias, n, c, hw, eps, act=L.ACT_NONE):
+    xv, d = _bn_tensor(x, n, c, hw), _bn_tensor(dy, n, c, hw)
+    mu, var = _bn_vec(saved_mean, c), _bn_vec(saved_var, c)
+    rs = 1 / np.sqrt(var + np.float32(eps).astype(np.float64))
+    xhat = (xv - mu) * rs
+    if act != L.ACT_NONE:
+        d = d * _act_derivative(act, xhat * _bn_vec(scale, c) + _bn_vec(bias, c))
+    if dscale is not None:
+        dscale.reshape(-1)[:c] = (d * xhat).sum((0, 2)).astype(np.float32)
+    if dbias is not None:
+        dbias.reshape(-1)[:c] = d.sum((0, 2)).astype(np.float32)
+    if dx is not None:
+        g = d * _bn_vec(scale, c)
+        res = (g - g.mean((0, 2), keepdims=True) - xhat * (g * xhat).mean((0, 2), keepdims=True)) * rs
+        dx.reshape(-1)[:n * c * hw] = res.reshape(-1).astype(dx.dtype)
+
+
 def _attn_view(desc, buf, strides, seq):
     shape = (int(desc.batch[0]), int(desc.batch[1]), int(seq), int(desc.head_dim))
     return _view(buf, 0, shape, [int(strides[0]), int(strides[1]), int(strides[2]), 1])
@@ -336,6 +393,19 @@ class Emulator:
                 desc, x, w, bias, y = args[:5]
                 dt = np.float16 if call.symbol.endswith("f16") else np.float32
                 conv2d(desc, self._typed(x, dt), w, bias, self._typed(y, dt))
+            elif call.symbol.startswith("dmlhip_batchnorm_inference"):
+                x, scale, bias, mean, var, y, n, c, hw, eps = args[:10]
+                batchnorm_inference(x, scale, bias, mean, var, y, n, c, hw, eps, args[10] if "_act_" in call.symbol else L.ACT_NONE)
+            elif call.symbol.startswith("dmlhip_batchnorm_training"):
+                batchnorm_training(*args[:15], args[15] if "_act_" in call.symbol else L.ACT_NONE)
+            elif call.symbol.startswith("dmlhip_batchnorm_backward"):
+                if "_act_" in call.symbol:
+                    dy, x, scale, bias, sm, sv, dx, ds, db, n, c, hw, eps, act = args[:14]
+                else:
+                    dy, x, scale, sm, sv, dx, ds, db, n, c, hw, eps = args[:12]
+                    bias, act = None, L.ACT_NONE
+                batchnorm_backward(dy, x, scale, bias, sm, sv, dx, self._typed(ds, np.float32) if ds is not None else None,
+                                   self._typed(db, np.float32) if db is not None else None, n, c, hw, eps, act)
             elif call.symbol == "dmlhip_conv2d_gated_f32":
                 desc, x, gate, w, bias, y = args[:6]
                 n = desc.n * desc.c * desc.h * desc.w

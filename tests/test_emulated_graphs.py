@@ -207,3 +207,62 @@ def test_mbconv_block_training_step():
     for n in wrt:
         scale = max(1.0, float(np.abs(want[n]).max()))
         assert_close(arrays[grads[n]], want[n], torch.float32, "mbconv d" + n, rtol=1e-4, atol=1e-5 * scale)
+
+
+# ----------------------------------------------------------------------------- an exported module in training mode
+def test_conv_batchnorm_relu_module_training_step():
+    """torch.nn.Conv2d -> BatchNorm2d -> ReLU in training mode through the exporter, the importer, the fusion passes
+    (the ReLU moves into the normalisation kernels) and the autodiff generator, interpreted on the CPU: output, input
+    and parameter gradients against autograd in fp64, and the running statistics the forward call leaves behind."""
+    import copy
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.onnx.onnx_importer import clean_onnx_name
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.torch import DaceModule
+    from daceml_amd.transformation import fusion
+    torch.manual_seed(11)
+    net = torch.nn.Sequential(torch.nn.Conv2d(3, 8, 3, padding=1), torch.nn.BatchNorm2d(8), torch.nn.ReLU())
+    with torch.no_grad():
+        net[1].weight.uniform_(0.5, 1.5)
+        net[1].bias.normal_(0, 0.2)
+        net[1].running_mean.normal_(0, 0.3)
+        net[1].running_var.uniform_(0.5, 2.0)
+    ref = copy.deepcopy(net).double().train()
+    x = torch.randn(4, 3, 10, 10)
+    wrapped = DaceModule(copy.deepcopy(net).train(), training=True, backward=True)
+    model = wrapped._import((x, ))
+    sdfg, state = model.sdfg, model.state
+    names = [n.schema.name for n in state.library_nodes()]
+    assert names == ["Conv", "BatchNormalization"] and state.library_nodes()[1]._activation == "relu"
+    fusion.lower_matmul(sdfg)
+    params = dict(net.named_parameters())
+    wrt = [clean_onnx_name(n) for n in model.inputs if n == model.inputs[0] or n in params]
+    grads = add_backward_pass(sdfg, state, list(model.outputs), wrt)
+    fusion.optimize_backward(sdfg)
+    expand_onnx_nodes(sdfg)
+    state_dict = {**params, **dict(net.named_buffers())}
+    arrays = {clean_onnx_name(model.inputs[0]): x.numpy().copy()}
+    for n in model.inputs[1:]:
+        arrays[clean_onnx_name(n)] = state_dict[n].detach().numpy().copy()
+    dy = torch.randn(4, 8, 10, 10)
+    arrays["gradient_" + model.outputs[0]] = dy.numpy().copy()
+    log = run_sdfg(sdfg, arrays)
+    assert any(s_.startswith("dmlhip_batchnorm_training_act") for s_ in log)
+    assert any(s_.startswith("dmlhip_batchnorm_backward_act") for s_ in log)
+    xr = x.double().requires_grad_(True)
+    want = ref(xr)
+    want.backward(dy.double())
+    assert_close(arrays[model.outputs[0]], want.detach().numpy(), torch.float32, "training forward", rtol=1e-4, atol=1e-5)
+    assert_close(arrays[grads[clean_onnx_name(model.inputs[0])]], xr.grad.numpy(), torch.float32, "dx", rtol=1e-4, atol=1e-5)
+    for n, pr in ref.named_parameters():
+        scale = max(1.0, float(pr.grad.abs().max()))
+        assert_close(arrays[grads[clean_onnx_name(n)]], pr.grad.numpy(), torch.float32, "gradient of " + n, rtol=1e-4,
+                     atol=1e-5 * scale)
+    # running statistics: torch blends the unbiased batch variance, the reference (and the kernels) the biased one
+    # (img_op_implementations.py:373-390); the mean follows the same rule in both
+    assert_close(arrays[clean_onnx_name("1.running_mean")], ref[1].running_mean.numpy(), torch.float32, "running mean",
+                 rtol=1e-4, atol=1e-6)
+    count = 4 * 10 * 10
+    biased = (ref[1].running_var.numpy() - 0.9 * net[1].running_var.numpy()) / 0.1 * (count - 1) / count
+    assert_close(arrays[clean_onnx_name("1.running_var")], 0.9 * net[1].running_var.numpy() + 0.1 * biased, torch.float32,
+                 "running variance", rtol=1e-4, atol=1e-6)
