@@ -511,3 +511,24 @@ def run_sdfg(sdfg, arrays):
     for st in sdfg.states():
         log += run_state(sdfg, st, arrays).log
     return log
+
+
+def run_program(program, arrays):
+    """Run a lowered TaskletProgram (daceml_amd/lowering.py): `arrays` maps the program's array names to NumPy arrays
+    (arguments given; transients, constants and missing outputs are allocated here). Connectors address their array
+    from the element offset the lowering recorded for them."""
+    import torch
+    np_dtype = {torch.float16: np.float16, torch.float32: np.float32, torch.int64: np.int64}
+    for name, d in program.arrays.items():
+        if name not in arrays:
+            if name in program.constants:
+                arrays[name] = program.constants[name].detach().cpu().numpy().astype(np_dtype[d.dtype]).reshape(d.shape)
+            else:
+                arrays[name] = np.full(d.shape, np.nan, dtype=np_dtype[d.dtype])
+    em = Emulator(program.workspace_bytes)
+    for spec in program.tasklets:
+        bound = {}
+        for conn, arr in list(spec.inputs.items()) + list(spec.outputs.items()):
+            bound[conn] = arrays[arr].reshape(-1)[spec.offsets.get(conn, 0):]
+        em.run(spec, bound)
+    return em

@@ -9,6 +9,7 @@ import subprocess
 import sys
 import types
 
+import numpy as np
 import pytest
 import torch
 
@@ -270,6 +271,100 @@ def test_reverse_nodes_lower_to_stand_alone_programs(tmp_path):
     with pytest.raises(NotApplicable):
         lowering.lower_backward(node, g.state, g.sdfg, find_backward_implementation(g.sdfg, g.state, node), ["Y"],
                                 ["X", "Scale", "B"])
+
+
+def test_stand_alone_reverse_programs_compute_what_the_in_graph_reverse_computes():
+    """The reverse of a node lowered on its own (what DaCeML's generator would call through the registered
+    BackwardImplementation, with arrays named after connectors) against the reverse the library's own generator builds
+    inside the graph for the same node - both interpreted by tests/abi_emulator.py on the same values. The in-graph
+    form is checked against the oracle by tests/test_emulated_graphs.py; this checks the plumbing around it: connector
+    naming, copies for passed-through gradients, view offsets, constants."""
+    from daceml_amd.runtime import expand_onnx_nodes
+    from tests.abi_emulator import run_program, run_sdfg
+    np_dtype = {torch.float16: np.float16, torch.float32: np.float32}
+    samples = [graphs.bert_encoder_layer(2, 16, 64, 2, 128, torch.float32),
+               graphs.mbconv_block(2, 16, 16, expand=2, cout=8, se_reduce=4, stride=2, dtype=torch.float32),
+               _unary_graph(torch.float32, differentiable=True)]
+    compared = set()
+    for base in samples:
+        count = len([x for x in base.states()[0].topological_sort() if isinstance(x, ONNXOp)])
+        for i in range(count):
+            sdfg = copy.deepcopy(base)
+            st = sdfg.states()[0]
+            node = [x for x in st.topological_sort() if isinstance(x, ONNXOp)][i]
+            impl = find_backward_implementation(sdfg, st, node)
+            given = [e.src_conn for e in st.out_edges(node)]
+            required = [e.dst_conn for e in st.in_edges(node)
+                        if e.data.data not in sdfg.constants and sdfg.arrays[e.data.data].dtype.is_floating_point]
+            in_arr = {e.dst_conn: e.data.data for e in st.in_edges(node)}
+            out_arr = {e.src_conn: e.data.data for e in st.out_edges(node)}
+            if len(set(in_arr.values())) != len(in_arr):
+                continue      # the same array on two connectors: the in-graph form sums the two gradients
+            lb = lowering.lower_backward(node, st, sdfg, impl, given, required)
+
+            # the same node alone in a graph of its own, reversed by the generator
+            ref = copy.deepcopy(base)
+            rst = ref.states()[0]
+            rnode = [x for x in rst.topological_sort() if isinstance(x, ONNXOp)][i]
+            for other in [x for x in rst.nodes() if isinstance(x, ONNXOp) and x is not rnode]:
+                fusion._remove_node(rst, other)
+            for name in list(in_arr.values()) + list(out_arr.values()):
+                ref.arrays[name].transient = False
+            grads = add_backward_pass(ref, rst, [out_arr[c] for c in given], [in_arr[c] for c in required])
+            expand_onnx_nodes(ref)
+            r = np.random.default_rng(100 + i)
+            arrays = {}
+            for c, name in in_arr.items():
+                d = ref.arrays[name]
+                if name not in ref.constants:
+                    arrays[name] = r.uniform(0.5, 1.5, d.shape).astype(np_dtype[d.dtype])
+            for c in given:
+                d = ref.arrays[out_arr[c]]
+                arrays["gradient_" + out_arr[c]] = r.standard_normal(d.shape).astype(np_dtype[d.dtype])
+            run_sdfg(ref, arrays)
+
+            mine = {}
+            for c in lb.forward_inputs:
+                mine[c] = arrays[in_arr[c]].copy()
+            for c in lb.forward_outputs:
+                mine[c] = arrays[out_arr[c]].copy()
+            for c, name in lb.given_grad_names.items():
+                mine[name] = arrays["gradient_" + out_arr[c]].copy()
+            run_program(lb.program, mine)
+            for c in required:
+                got, want = mine[lb.required_grad_names[c]], arrays[grads[in_arr[c]]]
+                assert got.shape == want.shape, (node, c)
+                np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-7, err_msg="%s input %s" % (node, c))
+            compared.add(node.schema.name)
+    assert {"MatMul", "Softmax", "Add", "Sub", "Mul", "Div", "Pow", "Sqrt", "Erf", "ReduceMean", "Transpose", "Reshape",
+            "Conv", "Sigmoid", "GlobalAveragePool", "Tanh", "Relu", "Exp", "Log", "Reciprocal"} <= compared, compared
+
+
+def test_lowered_states_compute_what_the_runtime_computes():
+    """A fused training graph (views in place of Transpose / Reshape nodes, grouped and K-concatenated contractions,
+    fused attention) lowered state by state to TaskletPrograms - what is emitted as C++ - and interpreted, against
+    the same expanded graph interpreted in the runtime's order: identical bits in every output."""
+    from daceml_amd.runtime import expand_onnx_nodes
+    from tests.abi_emulator import run_program, run_sdfg
+    sdfg = graphs.bert_encoder_layer(2, 64, 128, 2, 256, torch.float16)
+    fusion.auto_optimize(sdfg, training=True)
+    add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + graphs.BERT_PARAM_NAMES,
+                      grad_dtypes={n: torch.float32 for n in graphs.BERT_PARAM_NAMES})
+    fusion.optimize_backward(sdfg)
+    expand_onnx_nodes(sdfg)
+    assert any(d.view_of is not None for d in sdfg.arrays.values())
+    r = np.random.default_rng(3)
+    p = graphs.bert_init_params(128, 256, 5, bias_std=0.02)
+    base = {n: p[n].astype(np.float16) for n in graphs.BERT_PARAM_NAMES}
+    base["x"] = r.standard_normal((2, 64, 128)).astype(np.float16)
+    base["gradient_y"] = r.standard_normal((2, 64, 128)).astype(np.float16)
+    ref = {k: v.copy() for k, v in base.items()}
+    run_sdfg(sdfg, ref)
+    got = {k: v.copy() for k, v in base.items()}
+    for st in sdfg.states():
+        run_program(lowering.lower_state(sdfg, st), got)
+    for name in ["y", "gradient_x"] + ["gradient_" + n for n in graphs.BERT_PARAM_NAMES]:
+        assert np.array_equal(got[name], ref[name]), name
 
 
 def test_emitted_program_runs_the_calls_in_dependency_order():
