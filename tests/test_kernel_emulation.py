@@ -1,0 +1,256 @@
+"""The hand-scheduled kernels run on the CPU, lane by lane.
+
+tests/kernel_emulation/ compiles a kernel's own source for the host: every lane is a fibre, lanes meet at matrix
+instructions, LDS transpose reads, permutes and barriers, and global -> LDS transfers land either when they issue or
+only when the issuing lane waits for them (emu.h says what each extreme exposes). A result that is right under both,
+for several wavefront orders, means the tile ring, the waits and the barriers of the K loop are in the right places,
+fragments are read from the right stage, and the tail of the loop is handled - for every tile configuration, operand
+layout and K length tried. Needs the ROCm clang as a host compiler (the kernels use its vector extensions), no GPU.
+It checks the logic of the source, not the machine code: that is what the GPU tests and tests/isa_hazards.py are for."""
+import ctypes
+import os
+import shutil
+import subprocess
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EMU = os.path.join(ROOT, "tests", "kernel_emulation")
+CSRC = os.path.join(ROOT, "daceml_amd", "csrc")
+
+
+def _clang():
+    for c in ("/opt/rocm/lib/llvm/bin/clang++", shutil.which("amdclang++"), shutil.which("clang++")):
+        if c and os.path.exists(c):
+            return c
+    pytest.skip("no clang++ to compile the kernels for the host")
+
+
+def _stage_sources(tmp, files):
+    """Copies of the kernel sources with lds_ops.h swapped for its host stand-in, laid out like the repository (the
+    headers include ../../include/daceml_hip.h)."""
+    dst = os.path.join(tmp, "daceml_amd", "csrc")
+    os.makedirs(dst, exist_ok=True)
+    os.makedirs(os.path.join(tmp, "include"), exist_ok=True)
+    shutil.copy(os.path.join(ROOT, "include", "daceml_hip.h"), os.path.join(tmp, "include"))
+    for f in files:
+        text = open(os.path.join(CSRC, f)).read().replace('#include "lds_ops.h"', '#include "lds_ops_emu.h"')
+        # an LDS pointer cast to its address space is the byte offset inside LDS on the GPU; here LDS is host memory
+        text = text.replace("(uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds", "lds_addr(lds)")
+        # the one LDS read that is written as inline assembly outside lds_ops.h
+        text = text.replace('asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr));', "memcpy(&v, emu::g_lds + addr, 16);")
+        open(os.path.join(dst, f if not f.endswith(".hip") else f[:-4] + "_emu.h"), "w").write(text)
+    shutil.copy(os.path.join(EMU, "lds_ops_emu.h"), dst)
+    return dst
+
+
+def _build(tmp, name, harness, files, mutate=None):
+    """`mutate`: {file: function(text) -> text} applied to the staged copies (to show that a defect is detected)."""
+    src_dir = _stage_sources(tmp, files)
+    for f, fn in (mutate or {}).items():
+        path = os.path.join(src_dir, f)
+        text = open(path).read()
+        changed = fn(text)
+        assert changed != text, "the mutation of %s did not apply" % f
+        open(path, "w").write(changed)
+    out = os.path.join(tmp, name + ".so")
+    cmd = [_clang(), "-std=c++17", "-O1", "-fPIC", "-shared", "-x", "c++", "-Wno-everything", "-I", os.path.join(EMU, "shim"),
+           "-I", EMU, "-I", src_dir, os.path.join(EMU, harness), os.path.join(EMU, "emu.cpp"), "-o", out]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-6000:]
+    return ctypes.CDLL(out)
+
+
+@pytest.fixture(scope="module")
+def gemm_lib(tmp_path_factory):
+    lib = _build(str(tmp_path_factory.mktemp("emu_gemm")), "emu_gemm", "gemm_harness.cpp",
+                 ["common.h", "gemm_f16_common.h", "gemm_f16_pipe.h"])
+    lib.emu_gemm.restype = ctypes.c_int
+    return lib
+
+
+def _operand(r, rows, k, kind):
+    """(memory image, logical [rows, k] matrix in fp64)."""
+    x = (r.standard_normal((rows, k)) * 0.5).astype(np.float16)
+    return (np.ascontiguousarray(x.T) if kind else x), x.astype(np.float64)
+
+
+def _run_gemm(lib, cfg, variant, akind, bkind, m, n, k, pairs, seed, late):
+    r = np.random.default_rng(1000 * cfg + 10 * variant + akind * 2 + bkind + k)
+    a = [_operand(r, m, k, akind) for _ in range(pairs)]
+    b = [_operand(r, n, k, bkind) for _ in range(pairs)]
+    c = np.full((m, n), np.nan, dtype=np.float32)
+    asum = np.full(m, np.nan, dtype=np.float32)
+    pa = (ctypes.c_void_p * pairs)(*[x[0].ctypes.data for x in a])
+    pb = (ctypes.c_void_p * pairs)(*[x[0].ctypes.data for x in b])
+    status = lib.emu_gemm(cfg, variant, akind, bkind, m, n, k, pairs, pa, pb, c.ctypes.data_as(ctypes.c_void_p),
+                          asum.ctypes.data_as(ctypes.c_void_p), seed, late)
+    assert status == 0, "status %d (1 = the lanes deadlocked)" % status
+    want = sum(x[1] @ y[1].T for x, y in zip(a, b))
+    what = "cfg %d variant %d layouts %d%d %dx%dx%d seed %d %s" % (cfg, variant, akind, bkind, m, n, k, seed,
+                                                                  "late" if late else "early")
+    np.testing.assert_allclose(c, want, rtol=1e-5, atol=1e-4, err_msg=what)
+    if variant == 2:
+        np.testing.assert_allclose(asum, a[0][1].sum(1), rtol=1e-5, atol=1e-4, err_msg=what + " (row sums)")
+
+
+LAYOUTS = [(0, 0), (0, 1), (1, 0), (1, 1)]
+
+
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3])
+def test_the_emulation_reproduces_the_kernels_that_run_on_hardware(gemm_lib, cfg):
+    """The tile configurations the library uses (validated on the GPU): if the model of the matrix instruction, the
+    transpose read or the transfers were wrong, these would fail first."""
+    for akind, bkind in LAYOUTS:
+        for k, late in ((64, 0), (320, 1)):
+            _run_gemm(gemm_lib, cfg, 0, akind, bkind, 256, 256, k, 1, seed=1, late=late)
+    _run_gemm(gemm_lib, cfg, 0, 0, 1, 200, 136, 192, 1, seed=2, late=1)      # rows and columns short of a tile
+
+
+@pytest.mark.parametrize("cfg", [4, 5, 6])
+@pytest.mark.parametrize("late", [0, 1])
+def test_interleaved_k_loop(gemm_lib, cfg, late):
+    """Configurations 4 - 6: every operand layout, K from one step to more than twice the ring's depth (the loop has
+    a filling part, a draining part and a last step), two wavefront orders, ragged edges."""
+    for akind, bkind in LAYOUTS:
+        for k in (64, 128, 192, 256, 576):
+            _run_gemm(gemm_lib, cfg, 0, akind, bkind, 256, 256, k, 1, seed=3, late=late)
+    for seed in (4, 5):
+        _run_gemm(gemm_lib, cfg, 0, 0, 0, 256, 256, 384, 1, seed=seed, late=late)
+    _run_gemm(gemm_lib, cfg, 0, 1, 0, 200, 136, 320, 1, seed=6, late=late)
+    _run_gemm(gemm_lib, cfg, 0, 0, 1, 520, 264, 128, 1, seed=7, late=late)    # several tiles, the last ones ragged
+
+
+@pytest.mark.parametrize("cfg", [0, 3, 5])
+def test_operand_pairs_and_row_sums(gemm_lib, cfg):
+    """The K-concatenated and row-sum forms, plain loop (0, 3) and interleaved loop (5)."""
+    for late in (0, 1):
+        for akind, bkind in LAYOUTS:
+            _run_gemm(gemm_lib, cfg, 1, akind, bkind, 128, 256, 128, 3, seed=8, late=late)
+        _run_gemm(gemm_lib, cfg, 1, 0, 0, 128, 128, 64, 4, seed=9, late=late)     # one step per pair
+        _run_gemm(gemm_lib, cfg, 1, 1, 1, 200, 136, 192, 2, seed=10, late=late)
+        for bkind in (0, 1):
+            _run_gemm(gemm_lib, cfg, 2, 1, bkind, 256, 256, 320, 1, seed=11, late=late)
+        _run_gemm(gemm_lib, cfg, 2, 1, 1, 200, 136, 64, 1, seed=12, late=late)
+
+
+def _fails(fn):
+    try:
+        fn()
+    except AssertionError:
+        return True
+    return False
+
+
+def test_a_wait_that_lets_one_tile_too_many_stay_in_flight_is_detected(tmp_path):
+    """The check has teeth: with the interleaved loop's wait loosened by one tile, transfers that land late are read
+    before they arrive (wrong under LATE, still right when they land at issue)."""
+    def loosen(text):
+        return text.replace("if constexpr (FILL) wait_vm_lgkm0<(NSTAGE - 2) * LPT>();",
+                            "if constexpr (FILL) wait_vm_lgkm0<(NSTAGE - 1) * LPT>();")
+    lib = _build(str(tmp_path), "emu_gemm", "gemm_harness.cpp", ["common.h", "gemm_f16_common.h", "gemm_f16_pipe.h"],
+                 mutate={"gemm_f16_pipe.h": loosen})
+    lib.emu_gemm.restype = ctypes.c_int
+    for cfg in (4, 5, 6):
+        assert _fails(lambda: _run_gemm(lib, cfg, 0, 0, 0, 256, 256, 576, 1, seed=3, late=1)), cfg
+        _run_gemm(lib, cfg, 0, 0, 0, 256, 256, 576, 1, seed=3, late=0)
+
+
+def test_a_missing_barrier_is_detected(tmp_path):
+    """Without the barrier of the last sub-step a wavefront that runs ahead refills a tile the others still read (or
+    reads one they have not finished waiting for)."""
+    def drop(text):
+        i = text.index("if constexpr (FILL) wait_vm_lgkm0<(NSTAGE - 2) * LPT>();")
+        j = text.index("__builtin_amdgcn_s_barrier();", i)
+        return text[:j] + text[j + len("__builtin_amdgcn_s_barrier();"):]
+    lib = _build(str(tmp_path), "emu_gemm", "gemm_harness.cpp", ["common.h", "gemm_f16_common.h", "gemm_f16_pipe.h"],
+                 mutate={"gemm_f16_pipe.h": drop})
+    lib.emu_gemm.restype = ctypes.c_int
+    for cfg in (4, 5, 6):
+        assert _fails(lambda: _run_gemm(lib, cfg, 0, 0, 0, 256, 256, 576, 1, seed=3, late=0)), cfg
+
+
+def test_a_mask_that_one_kernel_ignores_is_detected(tmp_path):
+    def ignore(text):
+        return text.replace("if constexpr (MASK) mask2 = (float)a.mask[b0 * a.ms[0] + b1 * a.ms[1] + krow] * kLog2eF;",
+                            "if constexpr (MASK) mask2 = 0.f * (float)a.mask[0];")
+    lib = _build(str(tmp_path), "emu_attention", "attention_harness.cpp", ["common.h", "attention.hip"],
+                 mutate={"attention_emu.h": ignore})
+    lib.emu_attention.restype = ctypes.c_int
+    assert _fails(lambda: _attention_case(lib, 2, 2, 128, 128, "pad", seed=4, late=0))
+    _attention_case(lib, 2, 2, 128, 128, None, seed=4, late=0)
+
+
+# ----------------------------------------------------------------------------- fused attention
+@pytest.fixture(scope="module")
+def attention_lib(tmp_path_factory):
+    lib = _build(str(tmp_path_factory.mktemp("emu_attention")), "emu_attention", "attention_harness.cpp",
+                 ["common.h", "attention.hip"])
+    lib.emu_attention.restype = ctypes.c_int
+    return lib
+
+
+def _attention_case(lib, b0, b1, sq, sk, mask_kind, seed, late):
+    from daceml_amd import _lib as L
+    from oracle import ops as O
+    r = np.random.default_rng(50 + sq + sk)
+    q, k, v, do = (r.standard_normal((b0, b1, s_, 64)).astype(np.float16) for s_ in (sq, sk, sk, sq))
+    mask, m64, ms = None, None, None
+    if mask_kind:
+        per_head = "h" in mask_kind
+        pitch = (sk + 3) // 4 * 4
+        mem = np.zeros((b0, b1 if per_head else 1, 1, pitch), np.float16)
+        if "pad" in mask_kind:
+            for b in range(b0):
+                mem[b, :, :, max(1, sk - 5 - 9 * b):sk] = -10000.0
+        elif "inf" in mask_kind:
+            mem[..., sk // 2:sk] = -np.inf
+        else:
+            mem[..., :sk] = (r.standard_normal(mem[..., :sk].shape) * 2).astype(np.float16)
+        mask, m64 = mem, mem[..., :sk].astype(np.float64)
+        ms = (ctypes.c_int64 * 2)(mem.shape[1] * pitch if b0 > 1 else 0, pitch if per_head and b1 > 1 else 0)
+    d = L.AttentionDesc()
+    d.batch[0], d.batch[1], d.seq_q, d.seq_k, d.head_dim, d.scale = b0, b1, sq, sk, 64, 0.125
+    for name, s_ in (("q_stride", sq), ("k_stride", sk), ("v_stride", sk), ("o_stride", sq)):
+        st = getattr(d, name)
+        st[0], st[1], st[2] = b1 * s_ * 64, s_ * 64, 64
+    out = np.full(q.shape, np.nan, np.float16)
+    lse = np.full((b0, b1, sq), np.nan, np.float32)
+    dq, dk, dv = (np.full(t.shape, np.nan, np.float16) for t in (q, k, v))
+    dvec = np.full((b0, b1, sq), np.nan, np.float32)
+    ptr = lambda a: None if a is None else a.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
+    for which in (0, 1, 2):
+        status = lib.emu_attention(which, ctypes.byref(d), ptr(q), ptr(k), ptr(v), ptr(out), ptr(lse), ptr(do), ptr(dq),
+                                   ptr(dk), ptr(dv), ptr(dvec), ptr(mask), ms, seed, late)
+        assert status == 0, "kernel %d: status %d" % (which, status)
+    f64 = lambda t: t.astype(np.float64)  # noqa: E731
+    want, want_lse = O.attention(f64(q), f64(k), f64(v), 0.125, m64)
+    what = "%s mask=%s seed %d %s" % ((b0, b1, sq, sk), mask_kind, seed, "late" if late else "early")
+    np.testing.assert_allclose(out.astype(np.float64), want, rtol=2e-2, atol=1e-2, err_msg=what)
+    np.testing.assert_allclose(lse, want_lse, rtol=1e-3, atol=1e-3, err_msg=what + " (lse)")
+    # the backward kernels read the forward output as the forward kernel rounded it
+    for name, got, w in zip(("dq", "dk", "dv"), (dq, dk, dv), O.attention_backward(f64(q), f64(k), f64(v), 0.125, f64(do), m64)):
+        np.testing.assert_allclose(got.astype(np.float64), w, rtol=2e-2, atol=1e-2 * max(1.0, float(np.abs(w).max())),
+                                   err_msg="%s %s" % (name, what))
+    if mask_kind == "inf":
+        assert not dk[:, :, sk // 2:].any() and not dv[:, :, sk // 2:].any()
+
+
+@pytest.mark.parametrize("late", [0, 1])
+def test_attention_kernels_without_a_mask(attention_lib, late):
+    """The instantiations that run on hardware: the model must reproduce them before it says anything about the
+    masked ones."""
+    _attention_case(attention_lib, 1, 2, 128, 128, None, seed=1, late=late)
+    _attention_case(attention_lib, 1, 1, 100, 77, None, seed=2, late=late)
+    _attention_case(attention_lib, 1, 1, 64, 321, None, seed=3, late=late)
+
+
+@pytest.mark.parametrize("late", [0, 1])
+@pytest.mark.parametrize("mask_kind", ["pad", "bias", "h-bias", "inf"])
+def test_attention_kernels_with_an_additive_mask(attention_lib, mask_kind, late):
+    """Forward, dQ and dK / dV kernels with the mask: whole and ragged key tiles (the last tile reads the mask element
+    by element), a mask shared by the heads or one per head, large negative and -inf entries."""
+    _attention_case(attention_lib, 2, 2, 128, 128, mask_kind, seed=4, late=late)
+    _attention_case(attention_lib, 2, 1, 100, 77, mask_kind, seed=5, late=late)
+    _attention_case(attention_lib, 1, 2, 40, 200, mask_kind, seed=6, late=late)
