@@ -439,10 +439,10 @@ int dmlhip_batchnorm_backward_act_f32(const void* dy, const void* x, const void*
  * loader switch are per calling thread: they change only what that thread launches afterwards, and a value of
  * -1 / 0 / 1 respectively restores the default choice. The counter is process-wide and atomic. */
 /* Pin the tile configuration of the fp16 contraction kernels: 0 = 128x128 tile with a 4-stage ring, 1 = 256x128,
- * 2 = 256x256, 3 = 128x128 with a 2-stage ring; -1 = chosen per problem (default). 4, 5, 6 = the tiles of 2, 0, 1
+ * 2 = 256x256, 3 = 128x128 with a 2-stage ring; -1 = chosen per problem (default). 4, 5, 6, 7 = the tiles of 2, 0, 1, 3
  * with the interleaved K loop (fragment reads and global->LDS transfers issued one at a time between the MFMAs):
  * never chosen by the library, not yet measured or validated on hardware. Products with row sums or K-concatenated
- * operand pairs exist on the 128x128 tile only: 5 runs them with the interleaved loop, 4 and 6 leave them on the
+ * operand pairs exist on the 128x128 tile only: 5 and 7 run them with the interleaved loop, 4 and 6 leave them on the
  * plain one. */
 void dmlhip_debug_force_gemm_config(int cfg);
 /* 0: the fp16 contractions stage their operands through registers instead of loading them straight into LDS;

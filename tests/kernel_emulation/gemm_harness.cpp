@@ -61,6 +61,7 @@ emu::kernel_fn pick_cfg(int cfg, int ak, int bk, int* bm, int* bn) {
         case 0: return pick<128, 128, 64, 64, 4, KSUM, ASUM, false>(ak, bk);
         case 3: return pick<128, 128, 64, 64, 2, KSUM, ASUM, false>(ak, bk);
         case 5: return pick<128, 128, 64, 64, 4, KSUM, ASUM, true>(ak, bk);
+        case 7: return pick<128, 128, 64, 64, 2, KSUM, ASUM, true>(ak, bk);
         default: return nullptr;
     }
 }

@@ -108,10 +108,10 @@ def test_the_emulation_reproduces_the_kernels_that_run_on_hardware(gemm_lib, cfg
     _run_gemm(gemm_lib, cfg, 0, 0, 1, 200, 136, 192, 1, seed=2, late=1)      # rows and columns short of a tile
 
 
-@pytest.mark.parametrize("cfg", [4, 5, 6])
+@pytest.mark.parametrize("cfg", [4, 5, 6, 7])
 @pytest.mark.parametrize("late", [0, 1])
 def test_interleaved_k_loop(gemm_lib, cfg, late):
-    """Configurations 4 - 6: every operand layout, K from one step to more than twice the ring's depth (the loop has
+    """Configurations 4 - 7: every operand layout, K from one step to more than twice the ring's depth (the loop has
     a filling part, a draining part and a last step), two wavefront orders, ragged edges."""
     for akind, bkind in LAYOUTS:
         for k in (64, 128, 192, 256, 576):
@@ -122,9 +122,9 @@ def test_interleaved_k_loop(gemm_lib, cfg, late):
     _run_gemm(gemm_lib, cfg, 0, 0, 1, 520, 264, 128, 1, seed=7, late=late)    # several tiles, the last ones ragged
 
 
-@pytest.mark.parametrize("cfg", [0, 3, 5])
+@pytest.mark.parametrize("cfg", [0, 3, 5, 7])
 def test_operand_pairs_and_row_sums(gemm_lib, cfg):
-    """The K-concatenated and row-sum forms, plain loop (0, 3) and interleaved loop (5)."""
+    """The K-concatenated and row-sum forms, plain loop (0, 3) and interleaved loop (5, 7)."""
     for late in (0, 1):
         for akind, bkind in LAYOUTS:
             _run_gemm(gemm_lib, cfg, 1, akind, bkind, 128, 256, 128, 3, seed=8, late=late)
@@ -152,7 +152,7 @@ def test_a_wait_that_lets_one_tile_too_many_stay_in_flight_is_detected(tmp_path)
     lib = _build(str(tmp_path), "emu_gemm", "gemm_harness.cpp", ["common.h", "gemm_f16_common.h", "gemm_f16_pipe.h"],
                  mutate={"gemm_f16_pipe.h": loosen})
     lib.emu_gemm.restype = ctypes.c_int
-    for cfg in (4, 5, 6):
+    for cfg in (4, 5, 6, 7):
         assert _fails(lambda: _run_gemm(lib, cfg, 0, 0, 0, 256, 256, 576, 1, seed=3, late=1)), cfg
         _run_gemm(lib, cfg, 0, 0, 0, 256, 256, 576, 1, seed=3, late=0)
 

@@ -1,5 +1,5 @@
-"""The interleaved-K-loop configurations of the pipelined fp16 GEMM kernel (4: 256 x 256 tile, 5: 128 x 128, 6:
-256 x 128; reachable only through ``dmlhip_debug_force_gemm_config``) on the cases the chosen configurations are
+"""The interleaved-K-loop configurations of the pipelined fp16 GEMM kernel (4: 256 x 256 tile, 5: 128 x 128 with a four-stage ring, 6:
+256 x 128, 7: 128 x 128 with two stages; reachable only through ``dmlhip_debug_force_gemm_config``) on the cases the chosen configurations are
 tested with, plus products with enough K steps to run the ring's steady state, its tail and every operand layout.
 
 SKIPPED: these configurations were written without access to a GPU and have not run on hardware; the library never
@@ -13,10 +13,10 @@ from tests import test_gpu_kernels as TK
 from tests.util import assert_close, dev, host
 
 pytestmark = [pytest.mark.gpu,
-              pytest.mark.skip(reason="interleaved GEMM configurations 4-6 have not been run on hardware yet")]
+              pytest.mark.skip(reason="interleaved GEMM configurations 4-7 have not been run on hardware yet")]
 
 
-@pytest.mark.parametrize("cfg", [4, 5, 6])
+@pytest.mark.parametrize("cfg", [4, 5, 6, 7])
 @pytest.mark.parametrize("eq,sa,sb", TK.GEMM_CASES)
 def test_einsum_f16_interleaved(cfg, eq, sa, sb):
     TK.test_einsum_f16(cfg, eq, sa, sb)
@@ -36,7 +36,7 @@ LONG_K_CASES = [
 ]
 
 
-@pytest.mark.parametrize("cfg", [4, 5, 6])
+@pytest.mark.parametrize("cfg", [4, 5, 6, 7])
 @pytest.mark.parametrize("eq,sa,sb", LONG_K_CASES)
 def test_long_products_interleaved(cfg, eq, sa, sb):
     from daceml_amd import kernels as K
@@ -56,7 +56,7 @@ def test_long_products_interleaved(cfg, eq, sa, sb):
     assert torch.equal(got, base)
 
 
-@pytest.mark.parametrize("cfg", [4, 5, 6])
+@pytest.mark.parametrize("cfg", [4, 5, 6, 7])
 def test_epilogues_interleaved(cfg):
     TK._set_cfg(cfg)
     TK.test_gemm_f16_epilogue()
@@ -65,19 +65,24 @@ def test_epilogues_interleaved(cfg):
 
 
 def test_grouped_summed_and_row_sum_products_interleaved():
-    """Configuration 5 also carries the K-concatenated and the row-sum forms."""
+    """Configurations 5 and 7 also carry the K-concatenated and the row-sum forms."""
+    for cfg in (5, 7):
+        _grouped_forms(cfg)
+
+
+def _grouped_forms(cfg):
     for case in [("aik,jk->aij", (2, 256, 128), (192, 128), True, torch.float16),
                  ("aij,jk->aik", (2, 128, 192), (192, 256), False, torch.float16),
                  ("aij,aik->jk", (2, 256, 128), (2, 256, 64), False, torch.float32)]:
-        TK._set_cfg(5)
+        TK._set_cfg(cfg)
         TK._einsum_grouped_case(*case)
     for case in [("aij,jk->aik", (2, 256, 128), (128, 192), 3, True, torch.float16, True),
                  ("aik,jk->aij", (2, 128, 256), (128, 256), 4, True, torch.float16, True),
                  ("aij,aik->jk", (2, 256, 128), (2, 256, 64), 3, False, torch.float32, True)]:
-        TK._set_cfg(5)
+        TK._set_cfg(cfg)
         TK.test_einsum_sum(*case)
     for case in [((2, 256, 128), (2, 256, 64), 1, torch.float32, True), ((2, 256, 256), (2, 256, 128), 3, torch.float32, True),
                  ((4, 128, 384), (4, 128, 192), 4, torch.float16, True), ((2, 256, 200), (2, 256, 72), 2, torch.float32, True)]:
-        TK._set_cfg(5)
+        TK._set_cfg(cfg)
         TK.test_einsum_grouped_asum(*case)
     TK._set_cfg(-1)
