@@ -38,31 +38,45 @@ void entry(void* p) {
 template <int BM, int BN, int WM, int WN, int NSTAGE, bool KSUM, bool ASUM, bool ILV>
 emu::kernel_fn pick(int ak, int bk) {
     if (ak == 0 && bk == 0) return entry<BM, BN, WM, WN, 0, 0, NSTAGE, KSUM, ASUM, ILV>;
+#ifdef EMU_MINIMAL   // the builds that show a planted defect being found need one layout of the interleaved loop only
+    return nullptr;
+#else
     if (ak == 0 && bk == 1) return entry<BM, BN, WM, WN, 0, 1, NSTAGE, KSUM, ASUM, ILV>;
     if (ak == 1 && bk == 0) return entry<BM, BN, WM, WN, 1, 0, NSTAGE, KSUM, ASUM, ILV>;
     return entry<BM, BN, WM, WN, 1, 1, NSTAGE, KSUM, ASUM, ILV>;
+#endif
 }
 
 template <bool KSUM, bool ASUM>
 emu::kernel_fn pick_cfg(int cfg, int ak, int bk, int* bm, int* bn) {
     *bm = *bn = 128;
+#ifdef EMU_MINIMAL
+    if constexpr (KSUM || ASUM) return nullptr;
+    else
+#endif
+    {
     if constexpr (!KSUM && !ASUM) {
         if (cfg == 1 || cfg == 6) { *bm = 256; }
         if (cfg == 2 || cfg == 4) { *bm = 256; *bn = 256; }
         switch (cfg) {
+#ifndef EMU_MINIMAL
             case 1: return pick<256, 128, 128, 64, 3, false, false, false>(ak, bk);
             case 2: return pick<256, 256, 128, 128, 2, false, false, false>(ak, bk);
+#endif
             case 4: return pick<256, 256, 128, 128, 2, false, false, true>(ak, bk);
             case 6: return pick<256, 128, 128, 64, 3, false, false, true>(ak, bk);
             default: break;
         }
     }
     switch (cfg) {
+#ifndef EMU_MINIMAL
         case 0: return pick<128, 128, 64, 64, 4, KSUM, ASUM, false>(ak, bk);
         case 3: return pick<128, 128, 64, 64, 2, KSUM, ASUM, false>(ak, bk);
+#endif
         case 5: return pick<128, 128, 64, 64, 4, KSUM, ASUM, true>(ak, bk);
         case 7: return pick<128, 128, 64, 64, 2, KSUM, ASUM, true>(ak, bk);
         default: return nullptr;
+    }
     }
 }
 
