@@ -121,6 +121,24 @@ def test_interleaved_k_loop(gemm_lib, cfg, late):
     _run_gemm(gemm_lib, cfg, 0, 0, 1, 520, 264, 128, 1, seed=7, late=late)    # several tiles, the last ones ragged
 
 
+def test_every_configuration_adds_in_the_same_order(gemm_lib):
+    """Each accumulator receives the same matrix instructions in the same order whatever the tile shape, ring depth
+    or loop form: the fp32 results of all eight configurations are identical (which the GPU tests of the interleaved
+    configurations assert against the default configuration)."""
+    def run(cfg, akind, bkind):
+        r = np.random.default_rng(7)
+        a, b = _operand(r, 256, 576, akind), _operand(r, 256, 576, bkind)
+        c = np.full((256, 256), np.nan, dtype=np.float32)
+        pa, pb = (ctypes.c_void_p * 1)(a[0].ctypes.data), (ctypes.c_void_p * 1)(b[0].ctypes.data)
+        assert gemm_lib.emu_gemm(cfg, 0, akind, bkind, 256, 256, 576, 1, pa, pb, c.ctypes.data_as(ctypes.c_void_p), None, 1,
+                                 1) == 0
+        return c
+    for akind, bkind in ((0, 0), (1, 0)):
+        base = run(0, akind, bkind)
+        for cfg in range(1, 8):
+            assert np.array_equal(run(cfg, akind, bkind), base), (cfg, akind, bkind)
+
+
 @pytest.mark.parametrize("cfg", [0, 3, 5, 7])
 def test_operand_pairs_and_row_sums(gemm_lib, cfg):
     """The K-concatenated and row-sum forms, plain loop (0, 3) and interleaved loop (5, 7)."""
