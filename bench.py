@@ -146,19 +146,21 @@ def cpu_baseline(x, dy, p, budget_s=25.0):
 
 
 # ----------------------------------------------------------------------------- the other configurations
-def _time_program(prog, steps, warmup):
+def _time_program(prog, steps, warmup, graph=False):
+    """ms per step; with `graph` the step's launches are replayed from a HIP graph captured once."""
     import torch
+    step = prog.capture().replay if graph else prog.launch
     for _ in range(warmup):
-        prog.launch()
+        step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        prog.launch()
+        step()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) / steps * 1e3
 
 
-def secondary_workload(name, device, steps, warmup, verbose):
+def secondary_workload(name, device, steps, warmup, verbose, graph=False):
     """BASELINE.json configs[0..3]: parity-test cases that are also worth a measured line. Same JSON keys as the
     headline; `roofline` is that of the launch that takes the most time."""
     import numpy as np
@@ -239,7 +241,7 @@ def secondary_workload(name, device, steps, warmup, verbose):
         sys.exit("unknown workload %r" % name)
     prog = CompiledSDFG(sdfg, device=device)
     prog(**args)
-    ms = _time_program(prog, steps, warmup)
+    ms = _time_program(prog, steps, warmup, graph)
     rows = kernel_breakdown(prog)
     launches = []
     for l, t in rows:
@@ -270,8 +272,8 @@ def secondary_workload(name, device, steps, warmup, verbose):
     line = {"metric": what + " ms/iter at 1 GPU", "value": round(ms, 4), "unit": "ms/iter", "n_gpus": 1,
             "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
             "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-            "config": {"workload": what, "launches_per_step": len(prog.launches)}, "roofline": roof,
-            "launches": launches}
+            "config": {"workload": what, "launches_per_step": len(prog.launches), "hip_graph": bool(graph)},
+            "roofline": roof, "launches": launches}
     if name == "nodes":
         line["layernorm_cold"] = layernorm_cold(device, rng, max(2, min(steps, 6)))
     print(json.dumps(line))
@@ -384,6 +386,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region, launch a plain 128 MiB -> 128 MiB copy kernel three times: under "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its counters give the scale of those counters")
+    ap.add_argument("--graph", action="store_true",
+                    help="secondary workloads: replay the step from a HIP graph captured once instead of launching "
+                         "kernel by kernel (what a step of a few short kernels is bound by)")
     ap.add_argument("--gemm-config", type=int, default=-1,
                     help="pin the tile configuration of the fp16 contraction kernel for the whole run (the library's "
                          "diagnostic switch; -1 = the library's own choice). For comparing configurations, not for the "
@@ -404,7 +409,7 @@ def main():
     if a.workload == "module_bert":
         return module_workload(device, a.steps, a.warmup)
     if a.workload != "bert_fwd_bwd":
-        return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose)
+        return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose, a.graph)
 
     prog = build_program(device)
     args, x, dy, p = synthetic_inputs(device)

@@ -68,6 +68,18 @@ class _Launch:
         self.flops, self.bytes_moved, self.kind, self.state = flops, bytes_moved, kind, state
 
 
+class CapturedLaunches:
+    """A HIP graph of a CompiledSDFG's launches under one binding (``CompiledSDFG.capture``)."""
+    def __init__(self, program: "CompiledSDFG", graph, binding: int):
+        self.program, self.graph, self.binding = program, graph, binding
+
+    def replay(self):
+        """Enqueue the recorded launches on the current stream."""
+        if self.program._binding != self.binding:
+            raise RuntimeError("the program has been bound to other tensors since this graph was captured; capture again")
+        self.graph.replay()
+
+
 class CompiledSDFG:
     """An expanded SDFG bound to device buffers; call it with the non-transient arrays by name."""
     def __init__(self, sdfg: SDFG, device: Optional[torch.device] = None, expand: bool = True):
@@ -83,6 +95,7 @@ class CompiledSDFG:
         self._derived = []                    # (c_void_p, base name, byte offset)
         self._ptr_arrays = []                 # (ctypes array, [(slot, name)])
         self._stream = ctypes.c_void_p(0)
+        self._binding = 0                     # bumped whenever a pointer may have changed
         self.buffers: Dict[str, torch.Tensor] = {}
         self._allocate()
         self._launches: List[_Launch] = []
@@ -116,7 +129,9 @@ class CompiledSDFG:
         for name, t in self.buffers.items():
             self._ptr[name].value = t.data_ptr()
 
-    def _refresh(self):
+    def _refresh(self, changed: bool = True):
+        if changed:
+            self._binding += 1
         for obj, base, off in self._derived:
             obj.value = (self._ptr[base].value or 0) + off
         for arr, slots in self._ptr_arrays:
@@ -186,6 +201,7 @@ class CompiledSDFG:
 
     # -- execution -----------------------------------------------------------
     def _bind_arguments(self, kwargs: Dict[str, torch.Tensor], partial: bool = False):
+        changed = False
         for name, desc in self.sdfg.arrays.items():
             if desc.transient or name in self.sdfg.constants or desc.view_of is not None:
                 continue
@@ -201,11 +217,13 @@ class CompiledSDFG:
                                                                              tuple(t.shape)))
             if tuple(t.stride()) != desc.strides and t.numel() > 1:
                 raise ValueError("argument %r must have strides %s (pass a contiguous tensor)" % (name, desc.strides))
+            if self._ptr[name].value != t.data_ptr():
+                changed = True
             self._ptr[name].value = t.data_ptr()
         extra = set(kwargs) - set(self.sdfg.arrays)
         if extra:
             raise TypeError("unknown argument(s) %s" % sorted(extra))
-        self._refresh()
+        self._refresh(changed)
 
     def arglist(self) -> Dict[str, Array]:
         return {k: v for k, v in self.sdfg.arrays.items()
@@ -266,6 +284,24 @@ class CompiledSDFG:
             status = l.fn(*l.args)
             if status != 0:
                 raise L.HipKernelError(status, "%s (%s): %s" % (l.label, l.symbol, L.last_error()))
+
+    def capture(self, states: Optional[Sequence[str]] = None, warmup: int = 2) -> "CapturedLaunches":
+        """The launches (of the named states) with the pointers of the current binding, recorded once into a HIP graph:
+        ``replay()`` then costs one graph launch instead of one host call per kernel, which is what a step of a few
+        short kernels is bound by. The library allocates nothing, copies nothing and clears nothing on the host side
+        of a call, so every entry point can be recorded. The graph holds raw pointers: it belongs to the binding it
+        was captured under and refuses to replay after ``bind`` / ``__call__`` / ``rebind_transients`` changed it."""
+        current = torch.cuda.current_stream(self.device)
+        side = torch.cuda.Stream(self.device)
+        side.wait_stream(current)
+        with torch.cuda.stream(side):
+            for _ in range(max(warmup, 1)):   # first launches set kernel attributes (large LDS) outside the capture
+                self.launch(states)
+        current.wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            self.launch(states)
+        return CapturedLaunches(self, graph, self._binding)
 
     def launch_timed(self):
         """Like launch(), with a HIP event pair around every kernel; returns [(launch, ms)]."""
