@@ -160,7 +160,7 @@ def _time_program(prog, steps, warmup, graph=False):
     return (time.perf_counter() - t0) / steps * 1e3
 
 
-def secondary_workload(name, device, steps, warmup, verbose, graph=False):
+def secondary_workload(name, device, steps, warmup, verbose, graph=False, fused_rolling=""):
     """BASELINE.json configs[0..3]: parity-test cases that are also worth a measured line. Same JSON keys as the
     headline; `roofline` is that of the launch that takes the most time."""
     import numpy as np
@@ -272,7 +272,8 @@ def secondary_workload(name, device, steps, warmup, verbose, graph=False):
     line = {"metric": what + " ms/iter at 1 GPU", "value": round(ms, 4), "unit": "ms/iter", "n_gpus": 1,
             "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
             "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-            "config": {"workload": what, "launches_per_step": len(prog.launches), "hip_graph": bool(graph)},
+            "config": {"workload": what, "launches_per_step": len(prog.launches), "hip_graph": bool(graph),
+                       **({"fused_rolling": fused_rolling} if fused_rolling else {})},
             "roofline": roof, "launches": launches}
     if name == "nodes":
         line["layernorm_cold"] = layernorm_cold(device, rng, max(2, min(steps, 6)))
@@ -393,6 +394,10 @@ def main():
                     help="pin the tile configuration of the fp16 contraction kernel for the whole run (the library's "
                          "diagnostic switch; -1 = the library's own choice). For comparing configurations, not for the "
                          "reported figure: the JSON line carries the value in config.gemm_config")
+    ap.add_argument("--fused-rolling", default="",
+                    help="ROWS,WAVES: run the fused expand + depthwise convolution with its rolling-window kernel (the "
+                         "library's diagnostic switch; ROWS -1 = as many as fit). For comparing kernels, not for the "
+                         "reported figure: the JSON line carries the value in config.fused_rolling")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures the single-GPU path only: this build uses one GPU (no collectives, no sharding); "
@@ -405,11 +410,15 @@ def main():
     if a.gemm_config >= 0:
         from daceml_amd import _lib
         _lib.load().dmlhip_debug_force_gemm_config(a.gemm_config)
+    if a.fused_rolling:
+        from daceml_amd import _lib
+        rows, waves = (int(v) for v in a.fused_rolling.split(","))
+        _lib.load().dmlhip_debug_fused_rolling(rows, waves)
 
     if a.workload == "module_bert":
         return module_workload(device, a.steps, a.warmup)
     if a.workload != "bert_fwd_bwd":
-        return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose, a.graph)
+        return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose, a.graph, a.fused_rolling)
 
     prog = build_program(device)
     args, x, dy, p = synthetic_inputs(device)

@@ -144,6 +144,7 @@ SIGNATURES = {
     "dmlhip_debug_gemm_direct_lds": (None, [c_int]),
     "dmlhip_debug_grouped_single_launches": (ctypes.c_longlong, []),
     "dmlhip_debug_force_fused_strip": (None, [c_int]),
+    "dmlhip_debug_fused_rolling": (None, [c_int, c_int]),
 }
 
 _lib = None

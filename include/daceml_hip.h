@@ -452,6 +452,12 @@ void dmlhip_debug_gemm_direct_lds(int on);
 long long dmlhip_debug_grouped_single_launches(void);
 /* Pin the output-row strip height of dmlhip_conv2d_expand_depthwise_f32 (used if it fits LDS); 0 = default. */
 void dmlhip_debug_force_fused_strip(int toh);
+/* dmlhip_conv2d_expand_depthwise_f32 with a rolling window instead of strips: a workgroup walks down a segment of output
+ * rows with the expanded rows in a ring in LDS, half of its wavefronts expanding the next rows while the other half runs
+ * the stencil. rows: 0 = strips (default), -1 = as many output rows per batch as fit LDS, > 0 = at most that many;
+ * waves: 8 or 16 wavefronts per workgroup. Never chosen by the library, not yet measured or validated on hardware;
+ * shapes whose rows do not fit LDS keep the strips. Per calling thread. */
+void dmlhip_debug_fused_rolling(int rows, int waves);
 
 #ifdef __cplusplus
 }

@@ -45,3 +45,4 @@ def _reset_diagnostic_switches():
         lib.dmlhip_debug_force_gemm_config(-1)
         lib.dmlhip_debug_gemm_direct_lds(1)
         lib.dmlhip_debug_force_fused_strip(0)
+        lib.dmlhip_debug_fused_rolling(0, 8)

@@ -66,6 +66,21 @@ inline f16v mfma_32x32x16_f16(h8 a, h8 b, f16v c) {
     return d;
 }
 
+// D = C + A B, 32 x 32 x 2 in fp32: lane l holds A[l % 32][l / 32] and B[l / 32][l % 32]; C / D as above.
+inline f16v mfma_32x32x2_f32(float a, float b, f16v c) {
+    struct Ops { float a, b; } mine = {a, b};
+    const Ops* all = static_cast<const Ops*>(wave_exchange(&mine, sizeof(mine)));
+    const int lane = thread_idx().x & 63, col = lane & 31;
+    f16v d = c;
+    for (int e = 0; e < 16; ++e) {
+        const int row = 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+        float acc = 0.f;
+        for (int k = 0; k < 2; ++k) acc += all[row + 32 * k].a * all[col + 32 * k].b;
+        d[e] = c[e] + acc;
+    }
+    return d;
+}
+
 inline int ds_bpermute(int byte_index, int value) {
     const int* all = static_cast<const int*>(wave_exchange(&value, sizeof(value)));
     return all[(byte_index >> 2) & 63];
@@ -108,6 +123,7 @@ typedef emu_dim3 dim3;
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
 #define __builtin_amdgcn_readfirstlane(x) (x)
 #define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) emu::mfma_32x32x16_f16(a, b, c)
+#define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) emu::mfma_32x32x2_f32(a, b, c)
 #define __builtin_amdgcn_ds_bpermute(i, v) emu::ds_bpermute(i, v)
 #define __builtin_amdgcn_ballot_w64(p) emu::ballot(p)
 #define __builtin_amdgcn_readlane(v, l) emu::readlane(v, l)
@@ -119,13 +135,18 @@ typedef emu_dim3 dim3;
 /* global -> LDS transfer of `size` bytes per lane: lane l's piece lands at the LDS pointer + size * l */
 #define __builtin_amdgcn_global_load_lds(g, l, size, offset, aux) \
     emu::dma_issue((const void*)(g), (uint32_t)((const char*)(l) - emu::g_lds) + (size) * (threadIdx.x & 63), size)
+inline uint32_t __umulhi(uint32_t a, uint32_t b) { return (uint32_t)(((uint64_t)a * b) >> 32); }
+inline uint32_t __float_as_uint(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+inline float __uint_as_float(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
 using std::max;
 using std::min;
 
 // host-side names the launch helpers in the kernel headers mention (never called here)
 typedef void* hipStream_t;
 typedef int hipError_t;
-enum { hipSuccess = 0, hipFuncAttributeMaxDynamicSharedMemorySize = 0 };
+enum { hipSuccess = 0, hipFuncAttributeMaxDynamicSharedMemorySize = 0, hipDeviceAttributeMultiprocessorCount = 0 };
+inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+inline hipError_t hipDeviceGetAttribute(int* v, int, int) { *v = 256; return hipSuccess; }
 inline hipError_t hipFuncSetAttribute(const void*, int, int) { return hipSuccess; }
 inline const char* hipGetErrorString(hipError_t) { return ""; }
 #define hipLaunchKernelGGL(...) ((void)0)

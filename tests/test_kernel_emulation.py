@@ -271,3 +271,114 @@ def test_attention_kernels_with_an_additive_mask(attention_lib, mask_kind, late)
     _attention_case(attention_lib, 2, 2, 128, 128, mask_kind, seed=4, late=late)
     _attention_case(attention_lib, 2, 1, 100, 77, mask_kind, seed=5, late=late)
     _attention_case(attention_lib, 1, 2, 40, 200, mask_kind, seed=6, late=late)
+
+
+# ----------------------------------------------------------------------------- fused pointwise + depthwise convolution
+def _conv_fused_lib(tmp, mutate=None):
+    lib = _build(tmp, "emu_conv_fused", "conv_fused_harness.cpp", ["common.h", "conv_geom.h", "conv_fused.hip"], mutate)
+    lib.emu_expand_depthwise.restype = ctypes.c_int
+    return lib
+
+
+@pytest.fixture(scope="module")
+def conv_fused_lib(tmp_path_factory):
+    return _conv_fused_lib(str(tmp_path_factory.mktemp("emu_conv_fused")))
+
+
+def _expand_depthwise_problem(n, cin, cmid, h, w, stride, acts, bias):
+    from oracle import ops as O
+    r = np.random.default_rng(140)
+    x = r.standard_normal((n, cin, h, w)).astype(np.float32)
+    w1 = (r.standard_normal((cmid, cin, 1, 1)) * np.sqrt(2.0 / cin)).astype(np.float32)
+    w2 = (r.standard_normal((cmid, 1, 3, 3)) * np.sqrt(2.0 / 9)).astype(np.float32)
+    b1 = (r.standard_normal(cmid) * 0.1).astype(np.float32) if bias else None
+    b2 = (r.standard_normal(cmid) * 0.1).astype(np.float32) if bias else None
+    f1, f2 = {0: (lambda t: t, lambda t: t), 1: (O.swish, O.swish), 2: (lambda t: np.maximum(t, 0.0), lambda t: t)}[acts]
+    f64 = lambda t: None if t is None else t.astype(np.float64)  # noqa: E731
+    mid = f1(O.conv2d(f64(x), f64(w1), f64(b1)))
+    want = f2(O.conv2d(mid, f64(w2), f64(b2), (stride, stride), (1, 1, 1, 1), (1, 1), cmid))
+    return (x, w1, b1, w2, b2), want
+
+
+def _run_expand_depthwise(lib, mode, rows, waves, cus, acts, shape, operands, want, seed):
+    y = np.full(want.shape, np.nan, np.float32)
+    geometry = (ctypes.c_int * 4)()
+    ptr = lambda a: None if a is None else a.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
+    status = lib.emu_expand_depthwise(mode, rows, waves, cus, acts, *shape, *[ptr(t) for t in operands], ptr(y), seed,
+                                      geometry)
+    what = "%s mode %d rows %d waves %d cus %d seed %d geometry %s" % (shape, mode, rows, waves, cus, seed, list(geometry))
+    assert status == 0, "status %d: %s" % (status, what)
+    np.testing.assert_allclose(y, want, rtol=1e-5, atol=4e-6, err_msg=what)
+    return y, list(geometry)
+
+
+# n, cin, cmid, h, w, stride | activations (0 none/none, 1 swish/swish, 2 relu/none), biases
+EXPAND_DEPTHWISE_SHAPES = [
+    ((2, 16, 32, 9, 11, 2), 1, True),        # odd sizes, stride 2, the last batch is short
+    ((3, 32, 64, 14, 14, 1), 0, True),
+    ((1, 48, 32, 7, 5, 1), 2, False),        # three input-channel steps, rows narrower than a tile of pixels
+    ((2, 32, 64, 5, 70, 2), 0, True),        # rows wider than a wavefront
+    ((1, 16, 32, 1, 1, 1), 1, True),         # a single pixel: every neighbour is padding, divisions by a width of 1
+    ((1, 32, 64, 40, 40, 1), 2, False),
+    ((1, 32, 32, 112, 112, 2), 1, True),     # the rows of the benchmarked MBConv block, one image, one channel block
+    ((1, 16, 32, 37, 130, 1), 1, True),
+]
+
+
+@pytest.mark.parametrize("shape,acts,bias", EXPAND_DEPTHWISE_SHAPES)
+def test_expand_depthwise_rolling_window(conv_fused_lib, shape, acts, bias):
+    """The strip kernel (which runs on hardware: the model has to reproduce it) and the rolling-window kernel on the
+    same problems: every batch height, 8 and 16 wavefronts, segmentations from one segment per image to one per batch
+    (driven by the number of compute units the workgroups are spread over), several wavefront orders. The rolling
+    kernel adds in the strip kernel's order, so the two agree bit for bit."""
+    operands, want = _expand_depthwise_problem(*shape, acts, bias)
+    ref, _ = _run_expand_depthwise(conv_fused_lib, 0, 2, 8, 256, acts, shape, operands, want, seed=1)
+    seen = set()
+    for rows, waves, cus, seed in [(0, 8, 256, 1), (1, 8, 1, 2), (2, 16, 3, 3), (4, 8, 2, 4), (2, 8, 7, 5), (0, 16, 1, 6)]:
+        got, geometry = _run_expand_depthwise(conv_fused_lib, 1, rows, waves, cus, acts, shape, operands, want, seed)
+        assert np.array_equal(got, ref), "rolling window differs from the strips: rows %d waves %d" % (rows, waves)
+        seen.add(tuple(geometry))
+    if shape[3] >= 14:
+        assert len({g[3] for g in seen}) > 1 and len({g[0] for g in seen}) > 1, "one geometry only: %s" % seen
+
+
+def test_rolling_window_geometry_of_the_benchmarked_block(conv_fused_lib):
+    """[96,32,112,112] -> 192 channels, stride 2, on 256 compute units: two output rows per batch in a ring of nine
+    expanded rows (137 KB of LDS), four segments of 14 output rows per image: 2304 workgroups, nine per compute unit."""
+    shape = (1, 32, 32, 112, 112, 2)
+    operands, want = _expand_depthwise_problem(*shape, 1, True)
+    # one image and one channel block of the block's 96 x 6: the same rows, spread as if over 256 / (96 * 6) of a chip
+    _, geometry = _run_expand_depthwise(conv_fused_lib, 1, 0, 8, 256, 1, shape, operands, want, seed=7)
+    assert geometry[:2] == [2, 9]
+
+
+def test_a_ring_one_row_short_is_detected(tmp_path):
+    """Teeth: with one row less in the ring, the rows a batch adds land on a row the running stencil still reads."""
+    def shrink(text):
+        return text.replace("a.ring = 2 * r * stride + 3 - stride;", "a.ring = 2 * r * stride + 2 - stride;")
+    lib = _conv_fused_lib(str(tmp_path), {"conv_fused_emu.h": shrink})
+    shape = (1, 16, 32, 24, 20, 1)
+    operands, want = _expand_depthwise_problem(*shape, 0, True)
+    failures = 0
+    for seed in range(1, 7):
+        try:
+            _run_expand_depthwise(lib, 1, 2, 8, 1, 0, shape, operands, want, seed)
+        except AssertionError:
+            failures += 1
+    assert failures, "no wavefront order exposed the short ring"
+
+
+def test_a_missing_barrier_between_batches_is_detected(tmp_path):
+    def drop(text):
+        marker = "            consume(oy0, oy1, wave, WAVES);\n        }\n        __syncthreads();"
+        return text.replace(marker, "            consume(oy0, oy1, wave, WAVES);\n        }")
+    lib = _conv_fused_lib(str(tmp_path), {"conv_fused_emu.h": drop})
+    shape = (1, 16, 32, 24, 20, 1)
+    operands, want = _expand_depthwise_problem(*shape, 0, True)
+    failures = 0
+    for seed in range(1, 7):
+        try:
+            _run_expand_depthwise(lib, 1, 2, 8, 1, 0, shape, operands, want, seed)
+        except AssertionError:
+            failures += 1
+    assert failures, "no wavefront order exposed the missing barrier"
