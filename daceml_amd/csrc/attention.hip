@@ -284,16 +284,22 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
                 for (int e = 0; e < 16; ++e)
                     sacc[blk][e] = __builtin_fmaf(sacc[blk][e], a.scale_log2, (float)mk[blk * 4 + (e >> 2)][e & 3] * kLog2eF);
         }
+        if (ragged) {
+            // a branch of its own (the empty statement keeps the compiler from turning it into 32 compare-and-select
+            // pairs that every tile would pay for): only a last, partial tile has keys to take out
+            asm volatile("");
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
+            for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                if (ragged) {
+                for (int e = 0; e < 16; ++e) {
                     const int key = j * 64 + blk * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
                     if (key >= a.seq_k) sacc[blk][e] = -INFINITY;
                 }
-                mt = fmaxf(mt, sacc[blk][e]);
-            }
+        }
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mt = fmaxf(mt, sacc[blk][e]);
         mt = cross_half_max(mt);
         const float m_new = fmaxf(m_run, MASK ? mt : mt * a.scale_log2);
         // a mask may hold -inf for every key seen so far: keep the exponents' arguments free of (-inf) - (-inf)
@@ -478,22 +484,31 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
         }
         const bool ragged = (j + 1) * 64 > a.seq_k;
         half8 dsf[4];
+        float p[2][16];
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                float p;
                 if constexpr (MASK)
-                    p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], a.scale_log2,
-                                                              (float)mk[blk * 4 + (e >> 2)][e & 3] * kLog2eF) - lse2);
+                    p[blk][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], a.scale_log2,
+                                                                      (float)mk[blk * 4 + (e >> 2)][e & 3] * kLog2eF) - lse2);
                 else
-                    p = __builtin_amdgcn_exp2f(sacc[blk][e] * a.scale_log2 - lse2);
-                if (ragged) {
-                    const int key = j * 64 + blk * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-                    if (key >= a.seq_k) p = 0.f;
-                }
-                dsf[blk * 2 + (e >> 3)][e & 7] = (_Float16)(p * (pacc[blk][e] - dvec));
+                    p[blk][e] = __builtin_amdgcn_exp2f(sacc[blk][e] * a.scale_log2 - lse2);
             }
+        if (ragged) {
+            asm volatile("");   // a real branch: see the forward kernel
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = j * 64 + blk * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
+                    if (key >= a.seq_k) p[blk][e] = 0.f;
+                }
+        }
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) dsf[blk * 2 + (e >> 3)][e & 7] = (_Float16)(p[blk][e] * (pacc[blk][e] - dvec));
         wait_lgkm<0>();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -615,16 +630,23 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dkv_kernel(
                 qtf[blk][1] = tr_pair<(2 * qb + 1) * 2048>(qt + fr.trread[blk][0], qt + fr.trread[blk][1]);
             }
             half8 pf[2], dsf[2];
+            float p[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                p[e] = MASK ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[e], a.scale_log2, mask2) - lv[e >> 2][e & 3] * kLog2e)
+                            : __builtin_amdgcn_exp2f(sacc[e] * a.scale_log2 - lv[e >> 2][e & 3] * kLog2e);
+            if (ragged) {
+                asm volatile("");   // a real branch: see the forward kernel
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int qi = j * 64 + qb * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
+                    if (qi >= a.seq_q) p[e] = 0.f;
+                }
+            }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                float p = MASK ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[e], a.scale_log2, mask2) - lv[e >> 2][e & 3] * kLog2e)
-                               : __builtin_amdgcn_exp2f(sacc[e] * a.scale_log2 - lv[e >> 2][e & 3] * kLog2e);
-                if (ragged) {
-                    const int qi = j * 64 + qb * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-                    if (qi >= a.seq_q) p = 0.f;
-                }
-                pf[e >> 3][e & 7] = (_Float16)p;
-                dsf[e >> 3][e & 7] = (_Float16)(p * (pacc[e] - dvv[e >> 2][e & 3]));
+                pf[e >> 3][e & 7] = (_Float16)p[e];
+                dsf[e >> 3][e & 7] = (_Float16)(p[e] * (pacc[e] - dvv[e >> 2][e & 3]));
             }
             wait_lgkm<0>();
             __builtin_amdgcn_sched_barrier(0);
