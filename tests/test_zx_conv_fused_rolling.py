@@ -3,17 +3,17 @@
 where it must agree with the strip kernel bit for bit (both add in the same order).
 
 SKIPPED: the kernel was written without access to a GPU and has not run on hardware (its source runs lane by lane
-on the CPU in tests/test_kernel_emulation.py); the library never selects it. The skip goes once it has passed here."""
+on the CPU in tests/test_kernel_emulation.py); the library never selects it. The skip goes once it has passed here (DACEML_RUN_UNVALIDATED=1 runs it)."""
 import numpy as np
 import pytest
 import torch
 
 from oracle import ops as O
 from tests import test_gpu_kernels as TK
-from tests.util import assert_close, dev, host
+from tests.util import assert_close, dev, host, not_yet_on_hardware
 
 pytestmark = [pytest.mark.gpu,
-              pytest.mark.skip(reason="the rolling-window expand + depthwise kernel has not been run on hardware yet")]
+              not_yet_on_hardware("the rolling-window expand + depthwise kernel has not been run on hardware yet")]
 
 
 @pytest.mark.parametrize("waves", [8, 16])

@@ -3,17 +3,17 @@
 tested with, plus products with enough K steps to run the ring's steady state, its tail and every operand layout.
 
 SKIPPED: these configurations were written without access to a GPU and have not run on hardware; the library never
-selects them. The skip goes once they have passed here."""
+selects them. The skip goes once they have passed here (DACEML_RUN_UNVALIDATED=1 runs them)."""
 import numpy as np
 import pytest
 import torch
 
 from oracle import ops as O
 from tests import test_gpu_kernels as TK
-from tests.util import assert_close, dev, host
+from tests.util import assert_close, dev, host, not_yet_on_hardware
 
 pytestmark = [pytest.mark.gpu,
-              pytest.mark.skip(reason="interleaved GEMM configurations 4-7 have not been run on hardware yet")]
+              not_yet_on_hardware("interleaved GEMM configurations 4-7 have not been run on hardware yet")]
 
 
 @pytest.mark.parametrize("cfg", [4, 5, 6, 7])
