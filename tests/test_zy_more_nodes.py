@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from oracle import ops as O
-from tests.util import assert_close, dev, host, rng
+from tests.util import assert_close, dev, first_run_on_hardware, host, rng
 
 REDUCE_CASES = [((4, 6, 8), [0, 2]), ((3, 5, 7, 9), [0, 2]), ((3, 5, 7, 9), [1, 3]), ((2, 3, 4, 5, 6), [0, 2, 4]),
                 ((6, 1, 5, 4), [0, 3]), ((4, 6, 8), [0, 1])]
@@ -60,6 +60,7 @@ def test_reduce_over_separate_axes_lowers_to_passes(dtype, name, shape, axes, ke
     assert np.array_equal(arrays["x"], x)
 
 
+@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("name", ["sum", "mean", "max", "min"])
@@ -119,6 +120,7 @@ def test_softmax_reverse_node_for_any_axis_lowers_correctly(dtype, shape, axis):
     assert_close(arrays["gradient_x"], want, dtype, "emulated softmax backward %s axis %d" % (shape, axis), **tol)
 
 
+@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("shape,axis", SOFTMAX_CASES)
