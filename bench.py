@@ -31,7 +31,7 @@ METRIC = "BERT-large encoder layer fp16 fwd+bwd ms/iter at 1 GPU; % MFMA & HBM r
 B, S, H, HEADS, FFN = 8, 512, 1024, 16, 4096
 
 
-def build_program(device):
+def build_program(device, gelu_epilogue=False):
     import torch
     from daceml_amd import graphs
     from daceml_amd.autodiff import add_backward_pass
@@ -39,7 +39,7 @@ def build_program(device):
     from daceml_amd.transformation import fusion
 
     sdfg = graphs.bert_encoder_layer(B, S, H, HEADS, FFN, torch.float16, eps=1e-12)
-    fusion.auto_optimize(sdfg, training=True)
+    fusion.auto_optimize(sdfg, training=True, gelu_epilogue=gelu_epilogue)
     add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + graphs.BERT_PARAM_NAMES,
                       grad_dtypes={n: torch.float32 for n in graphs.BERT_PARAM_NAMES})
     fusion.optimize_backward(sdfg)
@@ -394,6 +394,10 @@ def main():
                     help="pin the tile configuration of the fp16 contraction kernel for the whole run (the library's "
                          "diagnostic switch; -1 = the library's own choice). For comparing configurations, not for the "
                          "reported figure: the JSON line carries the value in config.gemm_config")
+    ap.add_argument("--gelu-epilogue", action="store_true",
+                    help="fold the Gelu of the feed-forward block into the epilogue of the contraction before it (off in "
+                         "the reported configuration: measured slower with one workgroup per compute unit); recorded in "
+                         "config.gelu_epilogue")
     ap.add_argument("--fused-rolling", default="",
                     help="ROWS,WAVES: run the fused expand + depthwise convolution with its rolling-window kernel (the "
                          "library's diagnostic switch; ROWS -1 = as many as fit). For comparing kernels, not for the "
@@ -420,7 +424,7 @@ def main():
     if a.workload != "bert_fwd_bwd":
         return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose, a.graph, a.fused_rolling)
 
-    prog = build_program(device)
+    prog = build_program(device, a.gelu_epilogue)
     args, x, dy, p = synthetic_inputs(device)
     prog(**args)  # binds pointers, first run
     torch.cuda.synchronize()
@@ -486,7 +490,8 @@ def main():
         "config": {"workload": "BERT-large encoder layer forward + autodiff backward, B=8 S=512 hidden=1024 heads=16 "
                                "ffn=4096, fp16 (BASELINE.json configs[4])",
                    "launches_per_step": len(prog.launches),
-                   **({"gemm_config": a.gemm_config} if a.gemm_config >= 0 else {})},
+                   **({"gemm_config": a.gemm_config} if a.gemm_config >= 0 else {}),
+                   **({"gelu_epilogue": True} if a.gelu_epilogue else {})},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_FP16_TFLOPS, 4),
                      "traffic": GEMM_TRAFFIC_BYTES_PER_STEP["fetched"] + GEMM_TRAFFIC_BYTES_PER_STEP["written"],
