@@ -236,7 +236,7 @@ __device__ __forceinline__ void store_strip(const GemmArgs& g, void* c_ptr, void
 // 4 = row-contiguous. Returns DMLHIP_ERR_UNSUPPORTED when no instantiation fits.
 int launch_pipelined(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, const void* bias, const void* residual,
                      void* pre, int amode, int bmode, int cfg, long long batch, hipStream_t st);
-// Configurations 4 - 7 (the interleaved K loop on the tiles of 2, 0, 1 and 3); ak / bk: 0 = K-contiguous, 1 = row-contiguous.
+// Configurations 4 - 7 and 9 (the interleaved K loop on the tiles of 2, 0, 1, 3 and 8); ak / bk: 0 = K-contiguous, 1 = row-contiguous.
 int launch_pipelined_ilv(GemmArgs& g, const _Float16* a, const _Float16* b, void* c, const void* bias, const void* residual,
                          void* pre, int ak, int bk, int cfg, long long batch, hipStream_t st);
 

@@ -72,10 +72,15 @@ struct Stream<R, 0, T> {  // K-contiguous: tile [R][64 k], chunk c of row r at s
 };
 
 template <int R, int T>
-struct Stream<R, 1, T> {  // row-contiguous: tile [64 k][R], chunk c (8 rows) of K row k at slot c ^ ((k & 3) << 2)
+struct Stream<R, 1, T> {  // row-contiguous: tile [64 k][R], chunk c (8 rows) of K row k at slot c ^ shift(k)
     static constexpr int N = R / 32;
     static constexpr int P = R * 2;    // bytes per K row of the tile
     static constexpr int READS = 2 * T;
+    // A transpose read touches four consecutive K rows, 32 bytes of each. With 256-byte K rows (R = 128) they would
+    // all start in the same bank: K row k is shifted by 64 (k % 4) bytes. With 128-byte K rows (R = 64) rows k and
+    // k + 2 collide: shifted by 64 ((k / 2) % 2) bytes. Both depend on k % 4 only, so the reads' immediate offsets
+    // (multiples of four K rows) leave the shift alone.
+    static_assert(R == 64 || R % 128 == 0, "K rows of 128 bytes or of a multiple of 256");
     int off[N];
     uint32_t faddr[T];                 // per 32-row block: address of this lane's first transpose read (stage 0)
     __device__ __forceinline__ void init(int64_t, int64_t s_k, int row0, int rows, int wave, int lane, int wrow0,
@@ -84,7 +89,9 @@ struct Stream<R, 1, T> {  // row-contiguous: tile [64 k][R], chunk c (8 rows) of
         for (int i = 0; i < N; ++i) {
             const int o = (i * 4 + wave) * 1024 + lane * 16;
             const int kl = o / P, pos = (o % P) >> 4;
-            const int cidx = pos ^ ((kl & 3) << 2);
+            int cidx;
+            if constexpr (R == 64) cidx = pos ^ (((kl >> 1) & 1) << 2);
+            else cidx = pos ^ ((kl & 3) << 2);
             off[i] = (int)(kl * s_k) + min(row0 + cidx * 8, rows - 8);
         }
         // transpose read: the 16 lanes of group G = l/16 jointly read K rows kq..kq+3 of 16 tile rows; lane
@@ -95,7 +102,8 @@ struct Stream<R, 1, T> {  // row-contiguous: tile [64 k][R], chunk c (8 rows) of
 #pragma unroll
         for (int i = 0; i < T; ++i) {
             const int row = wrow0 + i * 32 + (grp & 1) * 16 + 4 * (s & 3);
-            faddr[i] = tile0 + kq * P + (((row >> 3) ^ ((kq & 3) << 2)) << 4) + (row & 7) * 2;
+            if constexpr (R == 64) faddr[i] = tile0 + kq * P + (((row >> 3) ^ (((kq >> 1) & 1) << 2)) << 4) + (row & 7) * 2;
+            else faddr[i] = tile0 + kq * P + (((row >> 3) ^ ((kq & 3) << 2)) << 4) + (row & 7) * 2;
         }
     }
     __device__ __forceinline__ void issue(const _Float16* base, int64_t s_k, int k0, char* tile, int wave) const {

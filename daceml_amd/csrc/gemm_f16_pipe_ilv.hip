@@ -29,6 +29,7 @@ int launch_pipelined_ilv(GemmArgs& g, const _Float16* a, const _Float16* b, void
         case 4: return launch_tile<256, 256, 128, 128, 2, false, false, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
         case 5: return launch_tile<128, 128, 64, 64, 4, false, false, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
         case 6: return launch_tile<256, 128, 128, 64, 3, false, false, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
+        case 9: return launch_tile<128, 64, 64, 32, 3, false, false, true>(g, a, b, c, bias, residual, pre, ak, bk, batch, st);
         default:
             set_error("gemm_f16: %d is not an interleaved-loop configuration", cfg);
             return DMLHIP_ERR_UNSUPPORTED;

@@ -441,9 +441,10 @@ int dmlhip_batchnorm_backward_act_f32(const void* dy, const void* x, const void*
 /* Pin the tile configuration of the fp16 contraction kernels: 0 = 128x128 tile with a 4-stage ring, 1 = 256x128,
  * 2 = 256x256, 3 = 128x128 with a 2-stage ring; -1 = chosen per problem (default). 4, 5, 6, 7 = the tiles of 2, 0, 1, 3
  * with the interleaved K loop (fragment reads and global->LDS transfers issued one at a time between the MFMAs):
- * never chosen by the library, not yet measured or validated on hardware. Products with row sums or K-concatenated
- * operand pairs exist on the 128x128 tile only: 5 and 7 run them with the interleaved loop, 4 and 6 leave them on the
- * plain one. */
+ * never chosen by the library, not yet measured or validated on hardware. 8 = 128x64 tile with a 3-stage ring (twice
+ * the workgroups, two per compute unit, for products that give each compute unit a single 128x128 tile), 9 = the same
+ * with the interleaved loop: likewise. Products with row sums or K-concatenated operand pairs exist on the 128x128 tile
+ * only: 5 and 7 run them with the interleaved loop, 4, 6, 8 and 9 leave them on the plain one. */
 void dmlhip_debug_force_gemm_config(int cfg);
 /* 0: the fp16 contractions stage their operands through registers instead of loading them straight into LDS;
  * 1 = default. */

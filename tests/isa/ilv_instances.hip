@@ -15,7 +15,7 @@ namespace gemm16 {
 const void* isa_check_kernels[] = {
     ILV_KERNELS(256, 256, 128, 128, 2, false, false), ILV_KERNELS(128, 128, 64, 64, 4, false, false),
     ILV_KERNELS(256, 128, 128, 64, 3, false, false),
-    ILV_KERNELS(128, 128, 64, 64, 2, false, false),
+    ILV_KERNELS(128, 128, 64, 64, 2, false, false), ILV_KERNELS(128, 64, 64, 32, 3, false, false),
     ILV_KERNELS(128, 128, 64, 64, 4, true, false),   // K-concatenated operand pairs
     ILV_KERNELS(128, 128, 64, 64, 4, false, true)};  // row sums of A alongside
 

@@ -58,6 +58,7 @@ emu::kernel_fn pick_cfg(int cfg, int ak, int bk, int* bm, int* bn) {
     if constexpr (!KSUM && !ASUM) {
         if (cfg == 1 || cfg == 6) { *bm = 256; }
         if (cfg == 2 || cfg == 4) { *bm = 256; *bn = 256; }
+        if (cfg == 8 || cfg == 9) { *bn = 64; }
         switch (cfg) {
 #ifndef EMU_MINIMAL
             case 1: return pick<256, 128, 128, 64, 3, false, false, false>(ak, bk);
@@ -65,6 +66,10 @@ emu::kernel_fn pick_cfg(int cfg, int ak, int bk, int* bm, int* bn) {
 #endif
             case 4: return pick<256, 256, 128, 128, 2, false, false, true>(ak, bk);
             case 6: return pick<256, 128, 128, 64, 3, false, false, true>(ak, bk);
+#ifndef EMU_MINIMAL
+            case 8: return pick<128, 64, 64, 32, 3, false, false, false>(ak, bk);
+            case 9: return pick<128, 64, 64, 32, 3, false, false, true>(ak, bk);
+#endif
             default: break;
         }
     }

@@ -65,5 +65,5 @@ def test_fused_attention_kernels(tmp_path):
 
 def test_interleaved_gemm_loop(tmp_path):
     count, found = isa_hazards.check_file(_assembly(os.path.join(ROOT, "tests", "isa", "ilv_instances.hip"), tmp_path))
-    assert count == 24, "four tile configurations, operand pairs and row sums x four operand-layout pairs"
+    assert count == 28, "five tile configurations, operand pairs and row sums x four operand-layout pairs"
     assert not found, _report(found)

@@ -108,10 +108,11 @@ def test_the_emulation_reproduces_the_kernels_that_run_on_hardware(gemm_lib, cfg
     _run_gemm(gemm_lib, cfg, 0, 0, 1, 200, 136, 192, 1, seed=2, late=1)      # rows and columns short of a tile
 
 
-@pytest.mark.parametrize("cfg", [4, 5, 6, 7])
+@pytest.mark.parametrize("cfg", [4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("late", [0, 1])
 def test_interleaved_k_loop(gemm_lib, cfg, late):
-    """Configurations 4 - 7: every operand layout, K from one step to more than twice the ring's depth (the loop has
+    """Configurations 4 - 7 and 9 (and 8: the plain loop on the 128 x 64 tile, whose row-contiguous operand has its own
+    LDS layout, new as well): every operand layout, K from one step to more than twice the ring's depth (the loop has
     a filling part, a draining part and a last step), two wavefront orders, ragged edges."""
     for akind, bkind in LAYOUTS:
         for k in (64, 128, 192, 256, 576) if akind == bkind else (64, 192, 320):
@@ -123,7 +124,7 @@ def test_interleaved_k_loop(gemm_lib, cfg, late):
 
 def test_every_configuration_adds_in_the_same_order(gemm_lib):
     """Each accumulator receives the same matrix instructions in the same order whatever the tile shape, ring depth
-    or loop form: the fp32 results of all eight configurations are identical (which the GPU tests of the interleaved
+    or loop form: the fp32 results of all ten configurations are identical (which the GPU tests of the interleaved
     configurations assert against the default configuration)."""
     def run(cfg, akind, bkind):
         r = np.random.default_rng(7)
@@ -135,7 +136,7 @@ def test_every_configuration_adds_in_the_same_order(gemm_lib):
         return c
     for akind, bkind in ((0, 0), (1, 0)):
         base = run(0, akind, bkind)
-        for cfg in range(1, 8):
+        for cfg in range(1, 10):
             assert np.array_equal(run(cfg, akind, bkind), base), (cfg, akind, bkind)
 
 

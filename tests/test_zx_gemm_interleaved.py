@@ -1,5 +1,5 @@
 """The interleaved-K-loop configurations of the pipelined fp16 GEMM kernel (4: 256 x 256 tile, 5: 128 x 128 with a four-stage ring, 6:
-256 x 128, 7: 128 x 128 with two stages; reachable only through ``dmlhip_debug_force_gemm_config``) on the cases the chosen configurations are
+256 x 128, 7: 128 x 128 with two stages, 9: 128 x 64 - and 8, the plain loop on that new tile; reachable only through ``dmlhip_debug_force_gemm_config``) on the cases the chosen configurations are
 tested with, plus products with enough K steps to run the ring's steady state, its tail and every operand layout.
 
 SKIPPED: these configurations were written without access to a GPU and have not run on hardware; the library never
@@ -16,7 +16,7 @@ pytestmark = [pytest.mark.gpu,
               not_yet_on_hardware("interleaved GEMM configurations 4-7 have not been run on hardware yet")]
 
 
-@pytest.mark.parametrize("cfg", [4, 5, 6, 7])
+@pytest.mark.parametrize("cfg", [4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("eq,sa,sb", TK.GEMM_CASES)
 def test_einsum_f16_interleaved(cfg, eq, sa, sb):
     TK.test_einsum_f16(cfg, eq, sa, sb)
@@ -36,7 +36,7 @@ LONG_K_CASES = [
 ]
 
 
-@pytest.mark.parametrize("cfg", [4, 5, 6, 7])
+@pytest.mark.parametrize("cfg", [4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("eq,sa,sb", LONG_K_CASES)
 def test_long_products_interleaved(cfg, eq, sa, sb):
     from daceml_amd import kernels as K
@@ -56,7 +56,7 @@ def test_long_products_interleaved(cfg, eq, sa, sb):
     assert torch.equal(got, base)
 
 
-@pytest.mark.parametrize("cfg", [4, 5, 6, 7])
+@pytest.mark.parametrize("cfg", [4, 5, 6, 7, 8, 9])
 def test_epilogues_interleaved(cfg):
     TK._set_cfg(cfg)
     TK.test_gemm_f16_epilogue()
