@@ -307,6 +307,10 @@ class ONNXModel:
             for s, e, a, st in zip(starts, ends, axes, steps):
                 idx[a] = slice(s, e, st)
             r = v[0][tuple(idx)]
+        elif op == "Reshape":
+            r = v[0].reshape([int(d) for d in v[1].tolist()])
+        elif op == "Transpose":
+            r = np.transpose(v[0], attrs.get("perm"))
         elif op == "ConstantOfShape":
             fill = attrs.get("value")
             fill = np.zeros((), np.float32) if fill is None else np.asarray(fill).reshape(())
@@ -393,6 +397,26 @@ class ONNXModel:
             return [(x[0], w[0]) + tuple(out)], [dt], ins, attrs
         if op == "GlobalAveragePool":
             return [tuple(shp[0][:2]) + (1, ) * (len(shp[0]) - 2)], [dt], ins, attrs
+        if op == "Pad":
+            # opset 11+: pads and the fill value are inputs; they become attributes, and have to be known now
+            mode = attrs.get("mode", "constant")
+            mode = mode.decode() if isinstance(mode, bytes) else str(mode)
+            pads = attrs.get("pads")
+            if pads is None:
+                if len(ins) < 2 or ins[1] not in self._known:
+                    raise UnsupportedModel("Pad node %r: the pads must be known at import time" % node.name)
+                pads = np.asarray(self._known[ins[1]]).reshape(-1).tolist()
+            value = float(attrs.get("value", 0.0))
+            if len(ins) > 2 and ins[2]:
+                if ins[2] not in self._known:
+                    raise UnsupportedModel("Pad node %r: the fill value must be known at import time" % node.name)
+                value = float(np.asarray(self._known[ins[2]]).reshape(-1)[0])
+            pads = [int(p) for p in pads]
+            rank = len(shp[0])
+            if len(pads) != 2 * rank or any(p < 0 for p in pads):
+                raise UnsupportedModel("Pad node %r: pads %s on a tensor of rank %d" % (node.name, pads, rank))
+            out = tuple(d + pads[i] + pads[rank + i] for i, d in enumerate(shp[0]))
+            return [out], [dt], ins[:1], {"mode": mode, "pads": pads, "value": value}
         if op == "LayerNormalization":
             return [shp[0]], [dt], ins, attrs
         if op == "BatchNormalization":

@@ -20,6 +20,7 @@ expansions it replaces (that composition is the oracle of the fused kernels).
     fuse_attention           Einsum(Q,K)[*scale], Softmax, Einsum(P,V)    -> FusedAttention
     fuse_reductions          independent ReduceSum(leading axes) nodes    -> MultiReduceSum (one launch pair)
     group_einsums            independent, identically shaped FusedEinsums -> GroupedEinsum (one launch)
+    fuse_pad_into_conv       Pad (zeros, spatial axes), Conv              -> Conv(pads)
     fuse_conv_activation     Conv, Swish | Sigmoid | Relu                 -> Conv(_activation)
     fuse_gate_into_conv      Mul(X, gate[n,c,1,1]), Conv 1x1              -> GatedConv (inference graphs)
 """
@@ -294,6 +295,46 @@ def fuse_swish(sdfg: SDFG) -> int:
             _add_node(sdfg, state, "Swish", sig.label.replace("_sigmoid", "") + "_fused", {"X": x}, {"Y": out})
             count += 1
     _drop_unused_arrays(sdfg)
+    return count
+
+
+def fuse_pad_into_conv(sdfg: SDFG) -> int:
+    """A Pad with zeros along the spatial axes, read only by a Conv, becomes that Conv's padding (PadConvFusion,
+    daceml/transformation/pad_conv_fusion.py:27-104: constant mode, fill value 0, nothing padded on the batch and
+    channel axes, the padded tensor has no other reader). One condition more than the reference: the padding that
+    results has to be the same before and after each spatial axis, which is what the convolution kernels take; a Pad
+    that does not fold stays in the graph and its expansion says that there is no implementation."""
+    count = 0
+    for state in sdfg.states():
+        for conv in [n for n in state.nodes() if _is_op(n, "Conv")]:
+            xa = _in_array(state, conv, "X")
+            prod = _producer(state, xa)
+            if prod is None or not _is_op(prod[0], "Pad") or not _internal(sdfg, state, xa):
+                continue
+            pad = prod[0]
+            rank = len(sdfg.arrays[xa].shape)
+            nsp = rank - 2
+            pads = [int(p) for p in pad.pads]
+            if pad.mode != "constant" or float(pad.value) != 0.0 or rank not in (3, 4) or len(pads) != 2 * rank:
+                continue
+            if any(pads[i] or pads[rank + i] for i in (0, 1)) or conv.auto_pad != "NOTSET":
+                continue
+            have = [int(p) for p in (conv.pads or [0] * (2 * nsp))]
+            begin = [have[i] + pads[2 + i] for i in range(nsp)]
+            end = [have[nsp + i] + pads[rank + 2 + i] for i in range(nsp)]
+            if begin != end:
+                continue
+            src = _in_array(state, pad, "data")
+            for e in list(state.in_edges_by_connector(conv, "X")):
+                state.remove_edge(e)
+                if isinstance(e.src, AccessNode) and not state.in_edges(e.src) and not state.out_edges(e.src):
+                    state.remove_node(e.src)
+            _remove_node(state, pad)
+            state.add_edge(state.add_read(src), None, conv, "X", sdfg.make_array_memlet(src))
+            conv.pads = begin + end
+            count += 1
+    if count:
+        _drop_unused_arrays(sdfg)
     return count
 
 
@@ -1241,6 +1282,7 @@ def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True,
     stats["gelu"] = fuse_gelu(sdfg)
     stats["layernorm"] = fuse_layernorm(sdfg)
     stats["swish"] = fuse_swish(sdfg)
+    stats["pad_into_conv"] = fuse_pad_into_conv(sdfg)
     # a Conv with a folded activation, GatedConv and SkipLayerNormalization have no backward implementation: graphs that
     # will be differentiated keep those nodes apart
     stats["conv_activation"] = 0 if training else fuse_conv_activation(sdfg)

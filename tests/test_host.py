@@ -368,7 +368,7 @@ def test_fusion_pipeline_on_bert_layer():
     before = [n.schema.name for n in st.library_nodes()]
     assert before.count("MatMul") == 8 and before.count("Erf") == 1 and before.count("ReduceMean") == 4
     stats = fusion.auto_optimize(sdfg, training=True, gelu_epilogue=True)
-    assert stats == {"gelu": 1, "layernorm": 2, "swish": 0, "conv_activation": 0, "batchnorm_activation": 0, "gated_conv": 0, "expand_depthwise": 0,
+    assert stats == {"gelu": 1, "layernorm": 2, "swish": 0, "pad_into_conv": 0, "conv_activation": 0, "batchnorm_activation": 0, "gated_conv": 0, "expand_depthwise": 0,
                      "matmul_to_einsum": 8,
                      "views": 15, "epilogues": 7, "skip_layernorm": 0, "attention": 0,   # head dim 32: not fused
                      "grouped_einsums": 0}                                               # training: after autodiff

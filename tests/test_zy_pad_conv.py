@@ -1,0 +1,121 @@
+"""A Pad with zeros in front of a Conv becomes the Conv's padding (PadConvFusion, pad_conv_fusion.py:13-104): the way
+``nn.ZeroPad2d`` / ``F.pad`` + ``nn.Conv2d`` leave the exporter. Host-side tests only: what remains after the rewrite
+is an ordinary Conv node, whose kernels have their own GPU tests; the calls it lowers to are interpreted on the CPU
+by tests/abi_emulator.py and compared with PyTorch in double precision."""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import assert_close
+
+
+def _import(net, x):
+    from daceml_amd.torch import DaceModule
+    return DaceModule(net)._import((x, ))
+
+
+def _run_emulated(model, net, x):
+    from daceml_amd.onnx.onnx_importer import clean_onnx_name
+    from daceml_amd.runtime import expand_onnx_nodes
+    from tests.abi_emulator import run_state
+    st = model.sdfg.states()[0]
+    expand_onnx_nodes(model.sdfg)
+    values = [x.numpy().copy()] + [p.detach().numpy().copy() for p in net.parameters()]
+    arrays = dict(zip([clean_onnx_name(n) for n in model.inputs], values))
+    em = run_state(model.sdfg, st, arrays)
+    return em, arrays[model.outputs[0]]
+
+
+@pytest.mark.parametrize("padding", [1, (2, 2, 1, 1)])
+def test_exported_zero_pad_and_conv_become_one_conv(padding):
+    """ZeroPad2d takes (left, right, top, bottom); the exporter computes the ONNX pads through a chain of shape
+    arithmetic that the importer evaluates at import time."""
+    torch.manual_seed(3)
+    net = torch.nn.Sequential(torch.nn.ZeroPad2d(padding), torch.nn.Conv2d(4, 6, 3, stride=2))
+    x = torch.randn(2, 4, 11, 12)
+    model = _import(net, x)
+    nodes = model.sdfg.states()[0].library_nodes()
+    assert [n.schema.name for n in nodes] == ["Conv"]
+    assert nodes[0].pads == ([1, 1, 1, 1] if padding == 1 else [1, 2, 1, 2])       # top, left, bottom, right
+    em, got = _run_emulated(model, net, x)
+    assert em.log == ["dmlhip_conv2d_f32"]
+    assert_close(got, net.double()(x.double()).detach().numpy(), torch.float32, "pad + conv", rtol=1e-5, atol=2e-6)
+
+
+def test_padding_adds_to_the_padding_the_conv_has():
+    torch.manual_seed(4)
+    net = torch.nn.Sequential(torch.nn.ZeroPad2d(1), torch.nn.Conv2d(3, 5, 5, padding=1))
+    x = torch.randn(1, 3, 8, 8)
+    model = _import(net, x)
+    nodes = model.sdfg.states()[0].library_nodes()
+    assert [n.schema.name for n in nodes] == ["Conv"] and nodes[0].pads == [2, 2, 2, 2]
+    _, got = _run_emulated(model, net, x)
+    assert_close(got, net.double()(x.double()).detach().numpy(), torch.float32, "pad + padded conv", rtol=1e-5, atol=2e-6)
+
+
+def test_exported_pad_and_conv1d():
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv = torch.nn.Conv1d(4, 6, 3)
+
+        def forward(self, x):
+            return self.conv(torch.nn.functional.pad(x, (2, 2)))
+
+    torch.manual_seed(5)
+    net, x = Net(), torch.randn(2, 4, 30)
+    model = _import(net, x)
+    nodes = model.sdfg.states()[0].library_nodes()
+    assert [n.schema.name for n in nodes] == ["Conv"] and nodes[0].pads == [2, 2]
+    _, got = _run_emulated(model, net, x)
+    assert_close(got, net.double()(x.double()).detach().numpy(), torch.float32, "pad + conv1d", rtol=1e-5, atol=2e-6)
+
+
+def test_padding_that_differs_before_and_after_an_axis_stays_a_pad_node():
+    """TensorFlow-style "same" padding of a strided convolution pads one side only: the convolution kernels take one
+    padding per axis, so the Pad stays, and expanding it names what is missing."""
+    import daceml_amd.onnx as donnx
+    from daceml_amd.runtime import expand_onnx_nodes
+    net = torch.nn.Sequential(torch.nn.ZeroPad2d((0, 1, 0, 1)), torch.nn.Conv2d(4, 6, 3, stride=2))
+    model = _import(net, torch.randn(1, 4, 8, 8))
+    nodes = model.sdfg.states()[0].library_nodes()
+    assert sorted(n.schema.name for n in nodes) == ["Conv", "Pad"]
+    pad = [n for n in nodes if n.schema.name == "Pad"][0]
+    assert pad.pads == [0, 0, 0, 0, 0, 0, 1, 1] and pad.mode == "constant" and pad.value == 0.0
+    with pytest.raises(donnx.NotApplicable, match="Pad"):
+        expand_onnx_nodes(model.sdfg)
+
+
+def _pad_conv_graph(pads, value=0.0, mode="constant", second_reader=False, conv_pads=None):
+    from daceml_amd import graphs
+    g = graphs.GraphBuilder("pad_conv", torch.float32)
+    x = g.input("x", (1, 2, 6, 6))
+    shape = tuple(d + pads[i] + pads[4 + i] for i, d in enumerate((1, 2, 6, 6)))
+    p = g.node("Pad", {"data": x}, {"output": shape}, label="pad", pads=list(pads), value=value, mode=mode)["output"]
+    cp = conv_pads or [0, 0, 0, 0]
+    out = (1, 3, shape[2] + cp[0] + cp[2] - 2, shape[3] + cp[1] + cp[3] - 2)
+    y = g.node("Conv", {"X": p, "W": g.input("w", (3, shape[1], 3, 3))}, {"Y": out}, label="conv", kernel_shape=[3, 3],
+               pads=cp)["Y"]
+    g.output(y, "y")
+    if second_reader:
+        g.output(g.node("Relu", {"X": p}, {"Y": shape}, label="relu")["Y"], "z")
+    return g
+
+
+def test_what_the_rewrite_refuses():
+    from daceml_amd.transformation import fusion
+    assert fusion.fuse_pad_into_conv(_pad_conv_graph([0, 0, 1, 2, 0, 0, 1, 2]).sdfg) == 1
+    for kwargs in (dict(pads=[0, 0, 1, 1, 0, 0, 1, 1], value=1.0),                 # not zeros
+                   dict(pads=[0, 0, 1, 1, 0, 0, 1, 1], mode="reflect"),
+                   dict(pads=[0, 1, 1, 1, 0, 0, 1, 1]),                            # pads the channel axis
+                   dict(pads=[1, 0, 1, 1, 0, 0, 1, 1]),                            # pads the batch axis
+                   dict(pads=[0, 0, 1, 1, 0, 0, 1, 1], second_reader=True),        # the padded tensor is read elsewhere
+                   dict(pads=[0, 0, 1, 1, 0, 0, 2, 1]),                            # top 1, bottom 2
+                   dict(pads=[0, 0, 1, 1, 0, 0, 1, 1], conv_pads=[0, 0, 1, 0])):   # symmetric Pad, lopsided Conv
+        g = _pad_conv_graph(**kwargs)
+        assert fusion.fuse_pad_into_conv(g.sdfg) == 0, kwargs
+        assert sorted(n.schema.name for n in g.state.library_nodes())[:2] == ["Conv", "Pad"]
+    # a lopsided Pad that completes a lopsided Conv folds
+    g = _pad_conv_graph(pads=[0, 0, 0, 1, 0, 0, 1, 0], conv_pads=[1, 0, 0, 1])
+    assert fusion.fuse_pad_into_conv(g.sdfg) == 1
+    assert g.state.library_nodes()[0].pads == [1, 1, 1, 1]
