@@ -750,6 +750,23 @@ class HipReshapeBackward(BackwardImplementation):
         return g, BackwardResult(required_grad_names={"data": "reshaped"}, given_grad_names={"reshaped": "data"})
 
 
+@autoregister_params(op="Pad", name=NAME)
+class HipPadBackward(BackwardImplementation):
+    """The gradient of a constant Pad is the incoming gradient without the padded border: one more Pad node with the
+    amounts negated (and where the forward node cropped, zeros come back in)."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        return node.mode == "constant"
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        g = _new(context, "Pad", forward_node.label + "_backward", pads=[-int(p) for p in forward_node.pads], value=0.0,
+                 mode="constant")
+        g.add_in_connector("data")
+        g.add_out_connector("output")
+        return g, BackwardResult(required_grad_names={"data": "output"}, given_grad_names={"output": "data"})
+
+
 @autoregister_params(op="GlobalAveragePool", name=NAME)
 class HipGlobalAveragePoolBackward(BackwardImplementation):
     """Y = mean of X over the spatial dims (img_op_implementations.py:415-417): dX = dY / (H*W), broadcast back over

@@ -20,6 +20,7 @@ SOURCES = [
     "elementwise.hip",
     "reduce.hip",
     "transpose.hip",
+    "pad.hip",
     "gemm_f16.hip",
     "gemm_f16_pipe.hip",
     "gemm_f16_pipe_ilv.hip",

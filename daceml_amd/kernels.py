@@ -343,6 +343,24 @@ def transpose(x: torch.Tensor, perm: Optional[Sequence[int]] = None) -> torch.Te
     return y
 
 
+def pad(x: torch.Tensor, pads: Sequence[int], value: float = 0.0) -> torch.Tensor:
+    """ONNX Pad in constant mode: ``pads`` lists the amounts in front of every axis, then those behind (negative
+    amounts crop)."""
+    _check(x)
+    x = _dense(x)
+    nd = x.dim()
+    if nd > L.MAX_DIMS:
+        raise NotImplementedError("more than %d dims" % L.MAX_DIMS)
+    pads = [int(p) for p in pads]
+    if len(pads) != 2 * nd:
+        raise ValueError("pads must hold %d amounts, got %d" % (2 * nd, len(pads)))
+    begin, end = pads[:nd], pads[nd:]
+    y = torch.empty([d + b + e for d, b, e in zip(x.shape, begin, end)], dtype=x.dtype, device=x.device)
+    L.check(_fn("pad_constant", x.dtype)(_ptr(x), _ptr(y), nd, L.i64_array(x.shape), L.i64_array(begin), L.i64_array(end),
+                                         float(value), _stream()))
+    return y
+
+
 # ----------------------------------------------------------------------------- contraction
 def gemm(desc: "L.GemmDesc", a, b, c, bias=None, residual=None, pre_out=None):
     """Raw strided-batched GEMM; `desc` fully describes operand layout."""

@@ -116,9 +116,9 @@ SCHEMAS = [
             strides=None),
     _schema("GlobalAveragePool", "X", "Y"),
     # Pad in its attribute form: the importer turns the `pads` / `constant_value` inputs of opset 11+ into these when
-    # they are known at import time. It has no implementation of its own (the reference has none either and runs a
-    # stand-alone Pad in onnxruntime): fusion.fuse_pad_into_conv folds it into the Conv that reads it, as
-    # PadConvFusion does (daceml/transformation/pad_conv_fusion.py:13-104)
+    # they are known at import time. fusion.fuse_pad_into_conv folds it into the Conv that reads it, as PadConvFusion
+    # does (daceml/transformation/pad_conv_fusion.py:13-104); what does not fold runs on the constant-pad kernel (the
+    # reference has no expansion for Pad and leaves a stand-alone one to onnxruntime)
     _schema("Pad", "data", "output", since=2, mode="constant", pads=REQUIRED, value=0.0),
     # "mean" / "var" name both inputs and outputs in ONNX; the connectors carry the in_ / out_ prefixes of the
     # reference (tests/test_shared_input_output.py)

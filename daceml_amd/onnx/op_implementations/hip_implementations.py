@@ -955,6 +955,36 @@ class HipTranspose(ONNXForward):
         return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="transpose")
 
 
+@op_implementation(op="Pad", name=IMPL)
+class HipPad(ONNXForward):
+    """Pad with a constant (the node's attribute form: the importer has turned the ``pads`` / ``constant_value``
+    inputs into attributes). Negative amounts crop, which is how the node's own reverse is expressed. The reference
+    has no expansion for Pad; in front of a Conv the fusion pass removes it (fuse_pad_into_conv)."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            x = in_desc_with_name(node, state, sdfg, "data")
+            y = out_desc_with_name(node, state, sdfg, "output")
+            nd = len(x.shape)
+            pads = [int(p) for p in node.pads]
+            return (node.mode == "constant" and _float_ok(x, y) and _dense(x, y) and nd <= L.MAX_DIMS
+                    and len(pads) == 2 * nd
+                    and tuple(y.shape) == tuple(d + pads[i] + pads[nd + i] for i, d in enumerate(x.shape)))
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "data")
+        y = out_desc_with_name(node, state, sdfg, "output")
+        nd = len(x.shape)
+        pads = [int(p) for p in node.pads]
+        call = HipCall("dmlhip_pad_constant_" + _SFX[x.dtype],
+                       [Ptr("data"), Ptr("output"), I32(nd), I64Array(tuple(x.shape)), I64Array(tuple(pads[:nd])),
+                        I64Array(tuple(pads[nd:])), F32(float(node.value)), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=_nbytes(x) + _nbytes(y), kind="elementwise")
+
+
 @op_implementation(op="Reshape", name=IMPL)
 class HipReshape(ONNXForward):
     """Reshape (pure_implementations.py:571-573): a dense copy into the output descriptor."""

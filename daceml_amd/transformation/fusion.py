@@ -303,7 +303,7 @@ def fuse_pad_into_conv(sdfg: SDFG) -> int:
     daceml/transformation/pad_conv_fusion.py:27-104: constant mode, fill value 0, nothing padded on the batch and
     channel axes, the padded tensor has no other reader). One condition more than the reference: the padding that
     results has to be the same before and after each spatial axis, which is what the convolution kernels take; a Pad
-    that does not fold stays in the graph and its expansion says that there is no implementation."""
+    that does not fold stays in the graph and runs on the constant-pad kernel."""
     count = 0
     for state in sdfg.states():
         for conv in [n for n in state.nodes() if _is_op(n, "Conv")]:

@@ -203,6 +203,17 @@ int dmlhip_transpose_f16(const void* x, void* y, int ndim, const int64_t* shape,
 int dmlhip_transpose_f32(const void* x, void* y, int ndim, const int64_t* shape,
                          const int64_t* perm, void* stream);
 
+/* ------------------------------------------------------------------ Pad
+ * ONNX Pad, mode "constant", with the amounts and the fill value known when the node is lowered. The reference has no
+ * expansion for it (a stand-alone Pad runs in onnxruntime; PadConvFusion, transformation/pad_conv_fusion.py:13-104,
+ * folds the common case into the Conv's padding, and so does this library's fusion pass). `shape` is x's shape,
+ * ndim <= DMLHIP_MAX_DIMS; y has shape[k] + begin[k] + end[k] elements along axis k; negative amounts crop (the
+ * gradient of a Pad is the Pad with the amounts negated). */
+int dmlhip_pad_constant_f16(const void* x, void* y, int ndim, const int64_t* shape, const int64_t* begin,
+                            const int64_t* end, float value, void* stream);
+int dmlhip_pad_constant_f32(const void* x, void* y, int ndim, const int64_t* shape, const int64_t* begin,
+                            const int64_t* end, float value, void* stream);
+
 /* ------------------------------------------------------------------ contractions
  * PureEinsum / PureMatMul / PureGemm: pure_implementations.py:111-252,380-553, which the
  * reference lowers to cuBLAS (strided-batched) GEMM through DaCe. One strided, batched GEMM:

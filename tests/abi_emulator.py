@@ -389,6 +389,16 @@ class Emulator:
                 shape, perm = tuple(shape[:ndim]), tuple(perm[:ndim])
                 n = int(np.prod(shape))
                 y.reshape(-1)[:n] = np.transpose(x.reshape(-1)[:n].reshape(shape), perm).reshape(-1)
+            elif call.symbol in ("dmlhip_pad_constant_f16", "dmlhip_pad_constant_f32"):
+                x, y, ndim, shape, begin, end, value = args[:7]
+                dt = np.float16 if call.symbol.endswith("f16") else np.float32
+                x, y = self._typed(x, dt), self._typed(y, dt)
+                shape, begin, end = (tuple(int(v) for v in t[:ndim]) for t in (shape, begin, end))
+                src = x.reshape(-1)[:int(np.prod(shape))].reshape(shape)
+                # negative amounts crop first, positive ones pad afterwards
+                src = src[tuple(slice(max(-b, 0), d - max(-e, 0)) for d, b, e in zip(shape, begin, end))]
+                out = np.pad(src, [(max(b, 0), max(e, 0)) for b, e in zip(begin, end)], constant_values=dt(value))
+                y.reshape(-1)[:out.size] = out.reshape(-1)
             elif call.symbol in ("dmlhip_conv2d_f16", "dmlhip_conv2d_f32"):
                 desc, x, w, bias, y = args[:5]
                 dt = np.float16 if call.symbol.endswith("f16") else np.float32

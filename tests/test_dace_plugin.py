@@ -144,6 +144,15 @@ def _sample_sdfgs():
     assert fusion.auto_optimize(g.sdfg)["attention"] == 1
     add_backward_pass(g.sdfg, g.state, ["o"], ["q", "k", "v"])
     out.append(("masked_attention_train", g.sdfg))
+    # a Pad that does not fold into the Conv behind it (one-sided), forward and reverse
+    g = graphs.GraphBuilder("pad_conv_train", torch.float32)
+    p = g.node("Pad", {"data": g.input("x", (2, 3, 6, 6))}, {"output": (2, 3, 7, 8)}, label="pad",
+               pads=[0, 0, 0, 2, 0, 0, 1, 0])["output"]
+    g.output(g.node("Conv", {"X": p, "W": g.input("w", (4, 3, 3, 3))}, {"Y": (2, 4, 5, 6)}, label="conv",
+                    kernel_shape=[3, 3])["Y"], "y")
+    assert fusion.auto_optimize(g.sdfg, training=True)["pad_into_conv"] == 0
+    add_backward_pass(g.sdfg, g.state, ["y"], ["x", "w"])
+    out.append(("pad_conv_train", g.sdfg))
     return out
 
 

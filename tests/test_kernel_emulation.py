@@ -383,3 +383,42 @@ def test_a_missing_barrier_between_batches_is_detected(tmp_path):
         except AssertionError:
             failures += 1
     assert failures, "no wavefront order exposed the missing barrier"
+
+
+# ----------------------------------------------------------------------------- constant pad
+@pytest.fixture(scope="module")
+def pad_lib(tmp_path_factory):
+    lib = _build(str(tmp_path_factory.mktemp("emu_pad")), "emu_pad", "pad_harness.cpp", ["common.h", "pad.hip"])
+    lib.emu_pad.restype = ctypes.c_int
+    return lib
+
+
+@pytest.mark.parametrize("shape,pads,value", [
+    ((2, 3, 5, 7), (0, 0, 1, 2, 0, 0, 3, 0), 0.0),           # spatial axes, lopsided
+    ((2, 3, 5, 7), (1, 2, 0, 0, 0, 1, 0, 0), -1.5),          # batch and channel axes, a fill value
+    ((4, 9), (-1, 2, 0, -3), 7.0),                           # cropping and padding mixed
+    ((3, 4, 6), (0, -1, -2, 0, -1, -1), 0.0),                # cropping only: the reverse of a pad
+    ((300, 41), (2, 1, 3, 0), 0.25),                         # more than one workgroup
+    ((5, ), (0, 0), 0.0),                                    # nothing to do
+    ((2, 2, 2, 2, 2, 3), (1, 0, 0, 1, 0, 0, 0, 1, 0, 0, 1, 2), 1.0)])   # six axes
+def test_constant_pad_kernel(pad_lib, shape, pads, value):
+    """The kernel's index arithmetic, through its own host function (which also builds the launch geometry)."""
+    r = np.random.default_rng(len(shape) * 10 + len(pads))
+    x = r.standard_normal(shape).astype(np.float32)
+    nd = len(shape)
+    begin, end = pads[:nd], pads[nd:]
+    crop = x[tuple(slice(max(-b, 0), d - max(-e, 0)) for d, b, e in zip(shape, begin, end))]
+    want = np.pad(crop, [(max(b, 0), max(e, 0)) for b, e in zip(begin, end)], constant_values=np.float32(value))
+    y = np.full(want.shape, np.nan, np.float32)
+    i64 = lambda t: (ctypes.c_int64 * len(t))(*t)  # noqa: E731
+    status = pad_lib.emu_pad(x.ctypes.data_as(ctypes.c_void_p), y.ctypes.data_as(ctypes.c_void_p), nd, i64(shape),
+                             i64(begin), i64(end), ctypes.c_float(value), 1)
+    assert status == 0
+    assert np.array_equal(y, want)
+
+
+def test_constant_pad_refuses_a_crop_larger_than_the_axis(pad_lib):
+    x = np.zeros((4, 4), np.float32)
+    i64 = lambda t: (ctypes.c_int64 * len(t))(*t)  # noqa: E731
+    assert pad_lib.emu_pad(x.ctypes.data_as(ctypes.c_void_p), x.ctypes.data_as(ctypes.c_void_p), 2, i64((4, 4)),
+                           i64((-3, 0)), i64((-2, 0)), ctypes.c_float(0.0), 1) < 0

@@ -1,12 +1,14 @@
 """A Pad with zeros in front of a Conv becomes the Conv's padding (PadConvFusion, pad_conv_fusion.py:13-104): the way
-``nn.ZeroPad2d`` / ``F.pad`` + ``nn.Conv2d`` leave the exporter. Host-side tests only: what remains after the rewrite
-is an ordinary Conv node, whose kernels have their own GPU tests; the calls it lowers to are interpreted on the CPU
-by tests/abi_emulator.py and compared with PyTorch in double precision."""
+``nn.ZeroPad2d`` / ``F.pad`` + ``nn.Conv2d`` leave the exporter. What remains after the rewrite is an ordinary Conv
+node, whose kernels have their own GPU tests. A Pad that does not fold (the padding differs between the two sides of
+an axis, a fill value, other axes) runs on a kernel of its own; its reverse is a Pad with negated amounts. The calls
+are interpreted on the CPU by tests/abi_emulator.py and compared with NumPy / PyTorch in double precision; the pad
+kernel's GPU test is SKIPPED until it has run on hardware (DACEML_RUN_UNVALIDATED=1 runs it)."""
 import numpy as np
 import pytest
 import torch
 
-from tests.util import assert_close
+from tests.util import assert_close, dev, host, not_yet_on_hardware
 
 
 def _import(net, x):
@@ -73,17 +75,69 @@ def test_exported_pad_and_conv1d():
 
 def test_padding_that_differs_before_and_after_an_axis_stays_a_pad_node():
     """TensorFlow-style "same" padding of a strided convolution pads one side only: the convolution kernels take one
-    padding per axis, so the Pad stays, and expanding it names what is missing."""
-    import daceml_amd.onnx as donnx
-    from daceml_amd.runtime import expand_onnx_nodes
+    padding per axis, so the Pad stays and runs as a kernel of its own in front of the unpadded Conv."""
+    torch.manual_seed(6)
     net = torch.nn.Sequential(torch.nn.ZeroPad2d((0, 1, 0, 1)), torch.nn.Conv2d(4, 6, 3, stride=2))
-    model = _import(net, torch.randn(1, 4, 8, 8))
+    x = torch.randn(1, 4, 8, 8)
+    model = _import(net, x)
     nodes = model.sdfg.states()[0].library_nodes()
     assert sorted(n.schema.name for n in nodes) == ["Conv", "Pad"]
     pad = [n for n in nodes if n.schema.name == "Pad"][0]
     assert pad.pads == [0, 0, 0, 0, 0, 0, 1, 1] and pad.mode == "constant" and pad.value == 0.0
-    with pytest.raises(donnx.NotApplicable, match="Pad"):
-        expand_onnx_nodes(model.sdfg)
+    em, got = _run_emulated(model, net, x)
+    assert em.log == ["dmlhip_pad_constant_f32", "dmlhip_conv2d_f32"]
+    assert_close(got, net.double()(x.double()).detach().numpy(), torch.float32, "lopsided pad, conv", rtol=1e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("shape,pads,value", [((2, 3, 5, 6), [0, 0, 1, 2, 0, 0, 0, 3], 0.0),
+                                              ((4, 7), [1, 0, 2, 2], -2.5),
+                                              ((3, 8, 5), [0, -2, 1, 0, -1, 0], 0.0)])
+def test_pad_node_lowers_to_the_pad_entry_point(dtype, shape, pads, value):
+    from daceml_amd import graphs
+    from daceml_amd.runtime import expand_onnx_nodes
+    from tests.abi_emulator import run_state
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    nd = len(shape)
+    out = tuple(d + pads[i] + pads[nd + i] for i, d in enumerate(shape))
+    g = graphs.GraphBuilder("pad", dtype)
+    y = g.node("Pad", {"data": g.input("x", shape)}, {"output": out}, label="pad", pads=pads, value=value)["output"]
+    g.output(y, "y")
+    expand_onnx_nodes(g.sdfg)
+    x = np.random.default_rng(8).standard_normal(shape).astype(npdt)
+    arrays = {"x": x.copy(), "y": np.full(out, np.nan, npdt)}
+    em = run_state(g.sdfg, g.state, arrays)
+    assert em.log == ["dmlhip_pad_constant_" + ("f16" if dtype == torch.float16 else "f32")]
+    crop = x[tuple(slice(max(-pads[i], 0), d - max(-pads[nd + i], 0)) for i, d in enumerate(shape))]
+    want = np.pad(crop, [(max(pads[i], 0), max(pads[nd + i], 0)) for i in range(nd)], constant_values=npdt(value))
+    assert np.array_equal(arrays["y"], want)
+
+
+def test_pad_is_differentiated_by_cropping():
+    """Pad -> Conv with a lopsided padding, differentiated: the Pad's reverse node is a Pad with negated amounts, and
+    the input gradient equals autograd's."""
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.runtime import expand_onnx_nodes
+    from tests.abi_emulator import run_sdfg
+    g = graphs.GraphBuilder("pad_conv_train", torch.float32)
+    p = g.node("Pad", {"data": g.input("x", (2, 3, 6, 6))}, {"output": (2, 3, 7, 8)}, label="pad",
+               pads=[0, 0, 0, 2, 0, 0, 1, 0])["output"]
+    y = g.node("Conv", {"X": p, "W": g.input("w", (4, 3, 3, 3))}, {"Y": (2, 4, 5, 6)}, label="conv", kernel_shape=[3, 3])["Y"]
+    g.output(y, "y")
+    add_backward_pass(g.sdfg, g.state, ["y"], ["x", "w"])
+    back = [n for st in g.sdfg.states() for n in st.library_nodes() if n.label == "pad_backward"]
+    assert len(back) == 1 and back[0].schema.name == "Pad" and back[0].pads == [0, 0, 0, -2, 0, 0, -1, 0]
+    expand_onnx_nodes(g.sdfg)
+    r = np.random.default_rng(9)
+    x, w = r.standard_normal((2, 3, 6, 6)).astype(np.float32), (r.standard_normal((4, 3, 3, 3)) * 0.2).astype(np.float32)
+    dy = r.standard_normal((2, 4, 5, 6)).astype(np.float32)
+    arrays = {"x": x.copy(), "w": w.copy(), "gradient_y": dy.copy()}
+    run_sdfg(g.sdfg, arrays)
+    xt, wt = torch.tensor(x, dtype=torch.float64, requires_grad=True), torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    torch.nn.functional.conv2d(torch.nn.functional.pad(xt, (2, 0, 0, 1)), wt).backward(torch.tensor(dy, dtype=torch.float64))
+    assert_close(arrays["gradient_x"], xt.grad.numpy(), torch.float32, "dx through pad", rtol=1e-5, atol=2e-6)
+    assert_close(arrays["gradient_w"], wt.grad.numpy(), torch.float32, "dw behind pad", rtol=1e-5, atol=1e-5)
 
 
 def _pad_conv_graph(pads, value=0.0, mode="constant", second_reader=False, conv_pads=None):
@@ -119,3 +173,19 @@ def test_what_the_rewrite_refuses():
     g = _pad_conv_graph(pads=[0, 0, 0, 1, 0, 0, 1, 0], conv_pads=[1, 0, 0, 1])
     assert fusion.fuse_pad_into_conv(g.sdfg) == 1
     assert g.state.library_nodes()[0].pads == [1, 1, 1, 1]
+
+
+@pytest.mark.gpu
+@not_yet_on_hardware("the constant-pad kernel has not been run on hardware yet")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("shape,pads,value", [((2, 3, 5, 6), [0, 0, 1, 2, 0, 0, 0, 3], 0.0), ((4, 7), [1, 0, 2, 2], -2.5),
+                                              ((3, 8, 5), [0, -2, 1, 0, -1, 0], 0.0),
+                                              ((96, 32, 112, 112), [0, 0, 0, 0, 0, 0, 1, 1], 0.0)])
+def test_pad_on_gpu(dtype, shape, pads, value):
+    from daceml_amd import kernels as K
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    nd = len(shape)
+    x = np.random.default_rng(10).standard_normal(shape).astype(npdt)
+    crop = x[tuple(slice(max(-pads[i], 0), d - max(-pads[nd + i], 0)) for i, d in enumerate(shape))]
+    want = np.pad(crop, [(max(pads[i], 0), max(pads[nd + i], 0)) for i in range(nd)], constant_values=npdt(value))
+    assert np.array_equal(host(K.pad(dev(x), pads, value)), want)
