@@ -181,8 +181,26 @@ class BackwardPassGenerator:
             gconn = result.required_grad_names.get(conn)
             if gconn is None:
                 raise AutoDiffException("%r: the reverse node computes no gradient for input %r" % (node, conn))
-            target = self._contribution_array(root, in_arr)
             src, sconn = self._source(rev, gconn)
+            begin = self._slice_of_root(root, in_arr)
+            if begin is not None:
+                # the node read a slice of `root`: its gradient is the gradient of the slice with zeros around it -
+                # a Pad from a buffer shaped like the slice into a contribution shaped like the root
+                fd, rd = sdfg.arrays[in_arr], sdfg.arrays[root]
+                part, _ = sdfg.add_transient("%s_slice_%d" % (self.array_grad_name(root), len(self._contrib.get(root, []))),
+                                             fd.shape, self.grad_dtype(root))
+                bst.add_edge(src, sconn, bst.add_write(part), None, sdfg.make_array_memlet(part))
+                target = self._contribution_array(root, root)
+                end = [r - b - d for r, b, d in zip(rd.shape, begin, fd.shape)]
+                pad = donnx.get_onnx_node("Pad")("scatter_" + part, pads=list(begin) + end, value=0.0, mode="constant")
+                bst.add_node(pad)
+                pad.add_in_connector("data")
+                pad.add_out_connector("output")
+                bst.add_edge(bst.add_read(part), None, pad, "data", sdfg.make_array_memlet(part))
+                bst.add_edge(pad, "output", bst.add_write(target), None, sdfg.make_array_memlet(target))
+                self._register(root, target, ready)
+                continue
+            target = self._contribution_array(root, in_arr)
             bst.add_edge(src, sconn, bst.add_write(target), None, sdfg.make_array_memlet(target))
             self._register(root, _root(sdfg, target) if sdfg.arrays[target].view_of else target, ready)
 
@@ -195,6 +213,23 @@ class BackwardPassGenerator:
         if isinstance(rev, BackwardGroup):
             return rev.outputs[conn]
         return rev, conn
+
+    def _slice_of_root(self, root: str, array: str) -> Optional[List[int]]:
+        """Where `array` starts along each axis of `root` when it is a rectangular part of it (a view with the root's
+        own strides that covers fewer elements); None when it is the root or a view of all of it."""
+        fd, rd = self.sdfg.arrays[array], self.sdfg.arrays[root]
+        if array == root or fd.view_of is None or fd.total_size == rd.total_size:
+            return None
+        if len(fd.shape) != len(rd.shape) or tuple(fd.strides) != tuple(rd.strides) or not rd.is_contiguous():
+            raise AutoDiffException("%r is a part of %r that is not a rectangular slice with unit steps: no gradient"
+                                    % (array, root))
+        begin, rest = [], fd.view_offset
+        for stride in rd.strides:
+            begin.append(rest // stride if stride else 0)
+            rest -= begin[-1] * stride if stride else 0
+        if rest or any(b + d > r for b, d, r in zip(begin, fd.shape, rd.shape)):
+            raise AutoDiffException("%r does not lie inside %r as a rectangle" % (array, root))
+        return begin
 
     # -- gradient buffers --------------------------------------------------------
     def _view_like(self, grad_array: str, forward_array: str) -> str:

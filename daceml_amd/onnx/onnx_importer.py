@@ -212,6 +212,9 @@ class ONNXModel:
             return
         if self._fold(op, node, ins, attrs):
             return
+        if op == "Slice":
+            self._import_slice(node, ins, attrs)
+            return
         if op in ("Dropout", ) and (not self.training or float(attrs.get("ratio", 0.5)) == 0.0):
             self._alias[node.output[0]] = ins[0]     # identity outside training; a mask output is never read
             return
@@ -264,6 +267,40 @@ class ONNXModel:
                         op_node.add_out_connector(conn)
                     self.state.add_edge(op_node, conn, self._access_node(clean, True), None,
                                         self.sdfg.make_array_memlet(clean))
+
+    def _import_slice(self, node, ins: List[str], attrs):
+        """A Slice of run-time data whose bounds are known now (the exporter slices the packed q / k / v projection
+        weight of ``nn.MultiheadAttention`` this way) becomes a view of its input: same buffer, an offset, strides
+        multiplied by the steps. No node, no copy; whether a reader can take the strides is that reader's business."""
+        known = lambda i: len(ins) > i and ins[i] and ins[i] in self._known  # noqa: E731
+        if "starts" in attrs:                                  # opset < 10: attributes
+            starts, ends = list(attrs["starts"]), list(attrs["ends"])
+            axes = list(attrs["axes"]) if "axes" in attrs else list(range(len(starts)))
+            steps = [1] * len(starts)
+        else:
+            if not (known(1) and known(2)) or (len(ins) > 3 and ins[3] and not known(3)) or \
+                    (len(ins) > 4 and ins[4] and not known(4)):
+                raise UnsupportedModel("Slice node %r: the bounds must be known at import time" % node.name)
+            starts = np.asarray(self._known[ins[1]]).reshape(-1).tolist()
+            ends = np.asarray(self._known[ins[2]]).reshape(-1).tolist()
+            axes = np.asarray(self._known[ins[3]]).reshape(-1).tolist() if known(3) else list(range(len(starts)))
+            steps = np.asarray(self._known[ins[4]]).reshape(-1).tolist() if known(4) else [1] * len(starts)
+        d = self._desc(ins[0])
+        shape, strides, offset = list(d.shape), list(d.strides), 0
+        for start, end, axis, step in zip(starts, ends, axes, steps):
+            axis = int(axis) % len(shape)
+            if int(step) <= 0:
+                raise UnsupportedModel("Slice node %r: step %d is not supported" % (node.name, step))
+            # clamping rule of the ONNX specification for positive steps
+            n = shape[axis]
+            lo, hi = int(start), int(end)
+            lo = min(max(lo + n if lo < 0 else lo, 0), n)
+            hi = min(max(hi + n if hi < 0 else hi, 0), n)
+            offset += lo * strides[axis]
+            shape[axis] = max(0, -(-(hi - lo) // int(step)))
+            strides[axis] *= int(step)
+        self.sdfg.add_view(clean_onnx_name(node.output[0]), clean_onnx_name(self._resolve(ins[0])), tuple(shape),
+                           tuple(strides), offset, find_new_name=False)
 
     # ------------------------------------------------------------------ import-time evaluation
     def _fold(self, op: str, node, ins: List[str], attrs) -> bool:
