@@ -299,6 +299,52 @@ class HipSoftmaxBackward(BackwardImplementation):
                                      given_grad_names={"output": "output_grad"})
 
 
+@autoregister_params(op="LogSoftmax", name=NAME)
+class HipLogSoftmaxBackward(BackwardImplementation):
+    """DefaultLogSoftmaxBackward (onnx_ops.py:338-373): ``dx = dy - exp(y) * ReduceSum(dy, axes=[axis], keepdims=1)``
+    as the reference's own nodes - Exp, ReduceSum, Mul, Sub - with the sum over every axis the forward node made one
+    row of (from ``axis`` on)."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        for e in state.in_edges_by_connector(node, "input"):
+            nd = len(sdfg.arrays[e.data.data].shape)
+            return nd >= 1 and -nd <= node.axis < nd
+        return False
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        sdfg = context.forward_sdfg
+        out = _out_arr(context, forward_node, "output")
+        od = sdfg.arrays[out]
+        nd = len(od.shape)
+        axis = forward_node.axis % nd
+        label = forward_node.label + "_backward"
+        group = BackwardGroup(label)
+        sums_shape = tuple(1 if i >= axis else e for i, e in enumerate(od.shape))
+        probs, _ = sdfg.add_transient(label + "_exp", od.shape, od.dtype)
+        sums, _ = sdfg.add_transient(label + "_sums", sums_shape, od.dtype)
+        scaled, _ = sdfg.add_transient(label + "_scaled", od.shape, od.dtype)
+        ex = _new(context, "Exp", label + "_exp")
+        _read(context, out, ex, "input")
+        _write(context, ex, "output", probs)
+        red = _new(context, "ReduceSum", label + "_sum", axes=list(range(axis, nd)), keepdims=1)
+        red.add_in_connector("data")
+        group.map_input("output_grad", red, "data")
+        _write(context, red, "reduced", sums)
+        mul = _new(context, "Mul", label + "_mul")
+        _read(context, probs, mul, "A")
+        _read(context, sums, mul, "B")
+        _write(context, mul, "C", scaled)
+        sub = _new(context, "Sub", label + "_sub")
+        sub.add_in_connector("A")
+        group.map_input("output_grad", sub, "A")
+        _read(context, scaled, sub, "B")
+        sub.add_out_connector("C")
+        group.map_output("input_grad", sub, "C")
+        return group, BackwardResult(required_grad_names={"input": "input_grad"},
+                                     given_grad_names={"output": "output_grad"})
+
+
 @autoregister_params(op="FusedAttention", name=NAME)
 class HipFusedAttentionBackward(BackwardImplementation):
     """One FusedAttentionGrad node; the forward node is made to emit its log-sum-exp rows, which replace the

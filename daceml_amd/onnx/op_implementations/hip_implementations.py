@@ -386,6 +386,50 @@ class HipSoftmax(ONNXForward):
         return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x), kind="softmax")
 
 
+@op_implementation(op="LogSoftmax", name=IMPL)
+class HipLogSoftmax(ONNXForward):
+    """LogSoftmax (pure_implementations.py:649-656), opset-12 semantics like Softmax: everything from ``axis`` on is
+    one row. The pure expansion's six statements as six calls on the reduction and elementwise kernels - row maximum,
+    ``x - max``, ``exp``, row sum, ``log``, subtraction - with the temporaries in the workspace: the logarithm is
+    taken of the row sum, never of a probability, so large negative inputs keep their finite values (a
+    ``log(softmax(x))`` would turn everything below the smallest normal into ``-inf``, in fp16 everything below
+    about -16)."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        return HipSoftmax.forward_can_be_applied(node, state, sdfg)
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "input")
+        axis = node.axis % len(x.shape)
+        rows, cols = _prod(x.shape[:axis]), _prod(x.shape[axis:])
+        sfx, code = _SFX[x.dtype], _CODE[x.dtype]
+        item = 2 if x.dtype == torch.float16 else 4
+        align = lambda n: -(-n // 256) * 256  # noqa: E731
+        # workspace: row maxima | x - max | row sums | their logarithms | scratch of the reductions
+        o_max, o_sub = 0, align(rows * item)
+        o_sum = o_sub + align(rows * cols * item)
+        o_log = o_sum + align(rows * item)
+        o_scr = o_log + align(rows * item)
+        scratch = L.load().dmlhip_reduce_workspace_bytes(rows, cols, 1)
+        full, per_row = (rows, cols), (cols, 1)
+        reduce = lambda op, src, dst: HipCall(  # noqa: E731
+            "dmlhip_reduce_" + sfx, [I32(op), src, dst, I32(code), I64(rows), I64(cols), I64(1), Workspace(o_scr),
+                                     WorkspaceBytes(o_scr), Stream()], flops=0, bytes_moved=0)
+        sub = lambda a, b, c: HipCall(  # noqa: E731
+            "dmlhip_binary_" + sfx, [I32(L.SUB), a, b, c, I32(2), I64Array(full), I64Array(per_row), I64Array((1, 0)),
+                                     Stream()], flops=0, bytes_moved=0)
+        unary = lambda op, src, dst, n: HipCall(  # noqa: E731
+            "dmlhip_unary_" + sfx, [I32(op), src, dst, I64(n), F32(0.0), Stream()], flops=0, bytes_moved=0)
+        calls = [reduce(L.RMAX, Ptr("input"), Workspace(o_max)),
+                 sub(Ptr("input"), Workspace(o_max), Workspace(o_sub)),
+                 unary(L.EXP, Workspace(o_sub), Ptr("output"), rows * cols),       # the output doubles as a temporary
+                 reduce(L.RSUM, Ptr("output"), Workspace(o_sum)),
+                 unary(L.LOG, Workspace(o_sum), Workspace(o_log), rows),
+                 sub(Workspace(o_sub), Workspace(o_log), Ptr("output"))]
+        return _tasklet(node, state, calls, workspace_bytes=o_scr + scratch, bytes_moved=8 * _nbytes(x), kind="softmax")
+
+
 @op_implementation(op="SoftmaxGrad", name=IMPL)
 class HipSoftmaxGrad(ONNXForward):
     """The node DefaultSoftmaxBackward builds from ONNXMul / ONNXReduceSum / a subtraction map

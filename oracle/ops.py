@@ -171,6 +171,29 @@ def softmax_backward(output, output_grad, axis):
     return prod - input_grad
 
 
+def log_softmax(input, axis=1):
+    """LogSoftmax (opset-12 semantics, the axes from ``axis`` on are one row): pure_implementations.py:649-656,
+    statement by statement - the logarithm is taken of the row sum."""
+    red = tuple(range(input.ndim))[axis:]
+    keepdims = axis != 0
+    maximum = np.maximum.reduce(input, axis=red, keepdims=keepdims)
+    max_sub = input - maximum
+    exponent = np.exp(max_sub)
+    total = np.add.reduce(exponent, axis=red, keepdims=keepdims)
+    log_sum = np.log(total)
+    return max_sub - log_sum
+
+
+def log_softmax_backward(output, output_grad, axis):
+    """DefaultLogSoftmaxBackward: autodiff/implementations/onnx_ops.py:338-373.
+
+    ``exp_output = Exp(y); sums = ReduceSum(dy, axes=[axis], keepdims=1); dx = dy - exp_output * sums``.
+    """
+    exp_output = np.exp(output)
+    sums = reduce_sum(output_grad, axes=[axis], keepdims=1)
+    return output_grad - exp_output * sums
+
+
 def attention(q, k, v, scale, mask=None):
     """The attention sub-graph as the reference expands it, node by node: Einsum(Q, K)
     (pure_implementations.py:219-252), the scalar Mul (:86-88), with ``mask`` the elementwise Add (:34-36) of a

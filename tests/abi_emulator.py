@@ -376,7 +376,8 @@ class Emulator:
                 _gemm_finish(desc, total, c, bias, residual, None)
             elif call.symbol in ("dmlhip_binary_f16", "dmlhip_binary_f32"):
                 op, a, b, c, ndim, shape, sa, sb = args[:8]
-                binary(op, a, b, c, ndim, shape, sa, sb)
+                dt = np.float16 if call.symbol.endswith("f16") else np.float32
+                binary(op, self._typed(a, dt), self._typed(b, dt), self._typed(c, dt), ndim, shape, sa, sb)
             elif call.symbol in ("dmlhip_reduce_f16", "dmlhip_reduce_f32"):
                 op, x, y, out_dtype, outer, r, inner = args[:7]
                 x = self._typed(x, np.float16 if call.symbol.endswith("f16") else np.float32)

@@ -153,6 +153,12 @@ def _sample_sdfgs():
     assert fusion.auto_optimize(g.sdfg, training=True)["pad_into_conv"] == 0
     add_backward_pass(g.sdfg, g.state, ["y"], ["x", "w"])
     out.append(("pad_conv_train", g.sdfg))
+    for dtype, tag in ((torch.float16, "f16"), (torch.float32, "f32")):
+        g = graphs.GraphBuilder("log_softmax_" + tag, dtype)
+        g.output(g.node("LogSoftmax", {"input": g.input("x", (6, 4, 10))}, {"output": (6, 4, 10)}, label="lsm", axis=1)["output"],
+                 "y")
+        add_backward_pass(g.sdfg, g.state, ["y"], ["x"])
+        out.append(("log_softmax_train_" + tag, g.sdfg))
     return out
 
 

@@ -62,6 +62,33 @@ def test_softmax_backward_matches_autograd():
     assert np.abs(O.softmax_backward(y.detach().numpy(), dy.numpy(), 2).sum(-1)).max() < 1e-12
 
 
+def test_log_softmax_matches_torch_scipy_and_keeps_small_probabilities():
+    from scipy.special import log_softmax as scipy_log_softmax
+    x = rng(40).standard_normal((3, 4, 9)) * 3
+    np.testing.assert_allclose(O.log_softmax(x, 2), F.log_softmax(torch.tensor(x), dim=-1).numpy(), rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(O.log_softmax(x, 2), scipy_log_softmax(x, axis=-1), rtol=1e-12, atol=1e-13)
+    # opset-12 coalescing: axis=1 on a 3-D tensor makes axes 1 and 2 one row
+    np.testing.assert_allclose(O.log_softmax(x, 1), scipy_log_softmax(x.reshape(3, -1), axis=1).reshape(x.shape), rtol=1e-12,
+                               atol=1e-13)
+    np.testing.assert_allclose(np.exp(O.log_softmax(x, 1)).reshape(3, -1).sum(1), 1.0, rtol=1e-12)
+    # a probability far below the smallest double still has its logarithm (log(softmax(x)) would give -inf)
+    big = np.array([[0.0, -800.0, -2000.0]])
+    np.testing.assert_allclose(O.log_softmax(big, 1), [[0.0, -800.0, -2000.0]], atol=1e-12)
+    assert np.isinf(np.log(O.softmax(big, 1))).any()
+    # what distinguishes it from Softmax: log of the Softmax where that is representable
+    np.testing.assert_allclose(O.log_softmax(x, 2), np.log(O.softmax(x, 2)), rtol=1e-12, atol=1e-13)
+
+
+def test_log_softmax_backward_matches_autograd():
+    x = torch.tensor(rng(41).standard_normal((3, 4, 9)), requires_grad=True)
+    dy = torch.tensor(rng(42).standard_normal((3, 4, 9)))
+    y = F.log_softmax(x, dim=-1)
+    y.backward(dy)
+    got = O.log_softmax_backward(y.detach().numpy(), dy.numpy(), 2)
+    np.testing.assert_allclose(got, x.grad.numpy(), rtol=1e-10, atol=1e-12)
+    assert np.abs(got.sum(-1)).max() < 1e-12        # a shift of a row changes nothing: gradients sum to zero
+
+
 # ----------------------------------------------------------------------------- layernorm / gelu
 def test_layernorm_chain_matches_torch_and_two_pass_loop():
     x = rng(5).standard_normal((3, 5, 16))

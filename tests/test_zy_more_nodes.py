@@ -137,3 +137,105 @@ def test_softmax_backward_for_any_axis_on_gpu(dtype, shape, axis):
     # the reverse node reads the forward output as the kernel rounded it
     want = O.softmax_backward(host(y).astype(np.float64), dy.astype(np.float64), axis % len(shape))
     assert_close(host(dx), want, dtype, "softmax backward %s axis %d" % (shape, axis), **tol)
+
+
+# ----------------------------------------------------------------------------- LogSoftmax
+LOG_SOFTMAX_CASES = [((8, 10), 1), ((3, 4, 33), -1), ((2, 3, 4, 5), 1), ((6, 40), 0), ((2, 300), 1)]
+
+
+def _log_softmax_graph(dtype, shape, axis, backward):
+    from daceml_amd import graphs
+    from daceml_amd.autodiff import add_backward_pass
+    g = graphs.GraphBuilder("log_softmax", dtype)
+    y = g.node("LogSoftmax", {"input": g.input("x", shape)}, {"output": shape}, label="lsm", axis=axis)["output"]
+    g.output(y, "y")
+    if backward:
+        add_backward_pass(g.sdfg, g.state, ["y"], ["x"])
+    return g
+
+
+def _log_softmax_data(dtype, shape):
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    r = rng(47)
+    x = (r.standard_normal(shape) * 4).astype(npdt)
+    x.reshape(-1)[::7] -= 30          # probabilities that fp16 cannot hold: their logarithms still have to come out
+    return x, r.standard_normal(shape).astype(npdt)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,axis", LOG_SOFTMAX_CASES)
+def test_log_softmax_lowers_to_the_reference_statements(dtype, shape, axis):
+    """Six calls in the pure expansion's order (pure_implementations.py:649-656); the reverse is the reference's
+    Exp / ReduceSum / Mul / Sub (onnx_ops.py:338-373) over all the axes of a row."""
+    from tests.abi_emulator import run_sdfg
+    from daceml_amd.runtime import expand_onnx_nodes
+    g = _log_softmax_graph(dtype, shape, axis, backward=True)
+    assert sorted(n.schema.name for n in g.sdfg.states()[1].library_nodes()) == ["Exp", "Mul", "ReduceSum", "Sub"]
+    expand_onnx_nodes(g.sdfg)
+    x, dy = _log_softmax_data(dtype, shape)
+    arrays = {"x": x.copy(), "gradient_y": dy.copy()}
+    log = run_sdfg(g.sdfg, arrays)
+    sfx = "f16" if dtype == torch.float16 else "f32"
+    assert log[:6] == ["dmlhip_%s_%s" % (k, sfx) for k in ("reduce", "binary", "unary", "reduce", "unary", "binary")]
+    ax = axis % len(shape)
+    want = O.log_softmax(x.astype(np.float64), ax)
+    assert np.isfinite(arrays["y"]).all()
+    tol = dict(rtol=2e-2, atol=2e-2) if dtype == torch.float16 else dict(rtol=1e-5, atol=2e-6)
+    assert_close(arrays["y"], want, dtype, "emulated LogSoftmax %s axis %d" % (shape, axis), **tol)
+    # the reverse reads the forward output as the kernels rounded it; the sum runs over the whole row
+    y = arrays["y"].astype(np.float64)
+    dy64 = dy.astype(np.float64)
+    want_dx = dy64 - np.exp(y) * dy64.sum(axis=tuple(range(ax, len(shape))), keepdims=True)
+    assert_close(arrays["gradient_x"], want_dx, dtype, "emulated LogSoftmax reverse %s axis %d" % (shape, axis),
+                 **(dict(rtol=2e-2, atol=3e-2) if dtype == torch.float16 else dict(rtol=1e-5, atol=1e-5)))
+    if ax == len(shape) - 1:
+        np.testing.assert_allclose(want_dx, O.log_softmax_backward(y, dy64, ax), rtol=1e-12, atol=1e-12)
+
+
+def test_exported_log_softmax_head():
+    """A classifier head as LeNet ends (tests/torch/test_lenet.py of the reference): Linear, LogSoftmax."""
+    from daceml_amd.onnx.onnx_importer import clean_onnx_name
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.torch import DaceModule
+    from tests.abi_emulator import run_state
+
+    class Head(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = torch.nn.Linear(84, 10)
+
+        def forward(self, x):
+            return torch.nn.functional.log_softmax(self.fc(x), dim=1)
+
+    torch.manual_seed(8)
+    net, x = Head(), torch.randn(8, 84)
+    model = DaceModule(net)._import((x, ))
+    st = model.sdfg.states()[0]
+    assert "LogSoftmax" in [n.schema.name for n in st.library_nodes()]
+    expand_onnx_nodes(model.sdfg)
+    names = [clean_onnx_name(n) for n in model.inputs]
+    arrays = dict(zip(names, [x.numpy().copy()] + [p.detach().numpy().copy() for p in net.parameters()]))
+    run_state(model.sdfg, st, arrays)
+    assert_close(arrays[model.outputs[0]], net.double()(x.double()).detach().numpy(), torch.float32, "Linear + LogSoftmax",
+                 rtol=1e-5, atol=2e-6)
+
+
+@first_run_on_hardware("written without access to a GPU: first run on hardware")
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,axis", LOG_SOFTMAX_CASES)
+def test_log_softmax_on_gpu(dtype, shape, axis):
+    from daceml_amd.runtime import CompiledSDFG
+    g = _log_softmax_graph(dtype, shape, axis, backward=True)
+    x, dy = _log_softmax_data(dtype, shape)
+    prog = CompiledSDFG(g.sdfg)
+    y = torch.full(shape, float("nan"), dtype=dtype, device="cuda")
+    dx = torch.full(shape, float("nan"), dtype=dtype, device="cuda")
+    prog(x=dev(x), y=y, gradient_y=dev(dy), gradient_x=dx)
+    ax = axis % len(shape)
+    tol = dict(rtol=2e-2, atol=2e-2) if dtype == torch.float16 else dict(rtol=1e-5, atol=2e-6)
+    assert_close(host(y), O.log_softmax(x.astype(np.float64), ax), dtype, "LogSoftmax %s axis %d" % (shape, axis), **tol)
+    y64, dy64 = host(y).astype(np.float64), dy.astype(np.float64)
+    want_dx = dy64 - np.exp(y64) * dy64.sum(axis=tuple(range(ax, len(shape))), keepdims=True)
+    assert_close(host(dx), want_dx, dtype, "LogSoftmax reverse %s axis %d" % (shape, axis),
+                 **(dict(rtol=2e-2, atol=3e-2) if dtype == torch.float16 else dict(rtol=1e-5, atol=1e-5)))
