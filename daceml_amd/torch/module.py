@@ -24,6 +24,7 @@ from torch import nn
 from ..autodiff import add_backward_pass
 from ..onnx.onnx_importer import ONNXModel, clean_onnx_name
 from ..runtime import CompiledSDFG
+from ..sdfg import AccessNode
 from ..transformation import fusion
 from .export import export_onnx
 
@@ -49,12 +50,14 @@ class DaceModule(nn.Module):
     :param backward: build the backward pass, so that the result takes part in autograd.
     :param inputs_to_skip: ONNX input names that need no gradient.
     :param auto_optimize: run the fusion pipeline (and the backward-state rewrites).
+    :param debug_transients: every intermediate tensor of the graph becomes an output, returned after the module's own
+        (daceml/torch/module.py:129-143); the fusion passes then leave those tensors in place.
     :param sdfg_name: name of the SDFG (defaults to the module's class name).
     """
     def __init__(self, module: nn.Module, dummy_inputs: Optional[Tuple[torch.Tensor, ...]] = None,
                  cuda: Optional[bool] = None, training: bool = False, backward: bool = False,
                  inputs_to_skip: Optional[List[str]] = None, auto_optimize: bool = True,
-                 sdfg_name: Optional[str] = None):
+                 sdfg_name: Optional[str] = None, debug_transients: bool = False):
         super().__init__()
         if cuda is False:
             raise ValueError("the HIP implementations run on a GPU; cuda=False is not available")
@@ -77,6 +80,23 @@ class DaceModule(nn.Module):
         self.post_autodiff_hooks: "collections.OrderedDict[str, Callable]" = collections.OrderedDict()
         #: run after the kernels are bound; called with the CompiledSDFG
         self.post_compile_hooks: "collections.OrderedDict[str, Callable]" = collections.OrderedDict()
+
+        self.debug_transients = debug_transients
+        if self.debug_transients:
+            def transients_outputs(dace_module):
+                # as the reference does it: in node order, everything transient except the statistics side outputs
+                sdfg = dace_module.sdfg
+                for state in sdfg.states():
+                    for node in state.nodes():
+                        if not isinstance(node, AccessNode):
+                            continue
+                        desc = sdfg.arrays[node.data]
+                        if desc.transient and desc.view_of is None and node.data not in dace_module.dace_model.outputs \
+                                and "mean" not in node.data and "std" not in node.data:
+                            dace_module.dace_model.outputs.append(node.data)
+                            desc.transient = False
+
+            self.prepend_post_onnx_hook("make_transients_outputs", transients_outputs)
 
         if self.auto_optimize:
             def optimize_forward(dace_module):
@@ -275,14 +295,14 @@ class DaceModule(nn.Module):
 
 
 def dace_module(moduleclass=None, dummy_inputs=None, cuda=None, training=False, backward=False,
-                inputs_to_skip=None, auto_optimize=True, sdfg_name=None):
+                inputs_to_skip=None, auto_optimize=True, sdfg_name=None, debug_transients=False):
     """Class decorator: instances of the decorated ``nn.Module`` class are created wrapped in a ``DaceModule``
     (daceml/torch/module.py:399-441)."""
     def wrap(cls):
         def make(*args, **kwargs):
             return DaceModule(cls(*args, **kwargs), dummy_inputs=dummy_inputs, cuda=cuda, training=training,
                               backward=backward, inputs_to_skip=inputs_to_skip, auto_optimize=auto_optimize,
-                              sdfg_name=sdfg_name)
+                              sdfg_name=sdfg_name, debug_transients=debug_transients)
         make.__name__ = cls.__name__
         make.__doc__ = cls.__doc__
         return make
