@@ -50,6 +50,9 @@ class DaceModule(nn.Module):
     :param backward: build the backward pass, so that the result takes part in autograd.
     :param inputs_to_skip: ONNX input names that need no gradient.
     :param auto_optimize: run the fusion pipeline (and the backward-state rewrites).
+    :param onnx_simplify, simplify, compile_torch_extension: accepted so that code written for the reference's wrapper
+        constructs this one unchanged; they select tools this path does not have (onnx-simplifier, DaCe's simplification
+        pass, the generated C++ dispatcher in place of the ctypes one) and change nothing here.
     :param debug_transients: every intermediate tensor of the graph becomes an output, returned after the module's own
         (daceml/torch/module.py:129-143); the fusion passes then leave those tensors in place.
     :param sdfg_name: name of the SDFG (defaults to the module's class name).
@@ -57,7 +60,8 @@ class DaceModule(nn.Module):
     def __init__(self, module: nn.Module, dummy_inputs: Optional[Tuple[torch.Tensor, ...]] = None,
                  cuda: Optional[bool] = None, training: bool = False, backward: bool = False,
                  inputs_to_skip: Optional[List[str]] = None, auto_optimize: bool = True,
-                 sdfg_name: Optional[str] = None, debug_transients: bool = False):
+                 sdfg_name: Optional[str] = None, debug_transients: bool = False, onnx_simplify: bool = True,
+                 simplify: bool = True, compile_torch_extension: bool = True):
         super().__init__()
         if cuda is False:
             raise ValueError("the HIP implementations run on a GPU; cuda=False is not available")
@@ -295,7 +299,8 @@ class DaceModule(nn.Module):
 
 
 def dace_module(moduleclass=None, dummy_inputs=None, cuda=None, training=False, backward=False,
-                inputs_to_skip=None, auto_optimize=True, sdfg_name=None, debug_transients=False):
+                inputs_to_skip=None, onnx_simplify=True, simplify=True, auto_optimize=True, sdfg_name=None,
+                compile_torch_extension=True, debug_transients=False):
     """Class decorator: instances of the decorated ``nn.Module`` class are created wrapped in a ``DaceModule``
     (daceml/torch/module.py:399-441)."""
     def wrap(cls):
