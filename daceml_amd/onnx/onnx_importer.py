@@ -123,7 +123,18 @@ class ONNXModel:
             if clean not in self.sdfg.arrays or not self.sdfg.arrays[clean].transient:
                 raise UnsupportedModel("output %r is not produced by a node of the graph" % out.name)
             new = "__return" if len(graph.output) == 1 else "__return_%d" % i
-            self._rename_array(clean, new)
+            desc = self.sdfg.arrays[clean]
+            if desc.view_of is not None:
+                # an output that is a part of another array (a Slice): the caller's buffer gets a copy of it
+                self.sdfg.add_array(new, tuple(desc.shape), desc.dtype, transient=True)
+                copy = donnx.get_onnx_node("Identity")("copy_%s" % new)
+                self.state.add_node(copy)
+                copy.add_in_connector("input")
+                copy.add_out_connector("output")
+                self.state.add_edge(self._access_node(clean, False), None, copy, "input", self.sdfg.make_array_memlet(clean))
+                self.state.add_edge(copy, "output", self._access_node(new, True), None, self.sdfg.make_array_memlet(new))
+            else:
+                self._rename_array(clean, new)
             self.sdfg.arrays[new].transient = False
             self.outputs.append(new)
         self._drop_unreferenced()
