@@ -44,6 +44,31 @@ def test_exported_zero_pad_and_conv_become_one_conv(padding):
     assert_close(got, net.double()(x.double()).detach().numpy(), torch.float32, "pad + conv", rtol=1e-5, atol=2e-6)
 
 
+def test_the_reference_test_module():
+    """tests/transformation/test_pad_conv_fusion.py of the reference: ``F.pad(x, [2, 2])`` (the last axis only) in
+    front of ``Conv2d(3, 6, 3)`` on a [4, 3, 24, 24] input - one rewrite, same output."""
+    class Module(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv = torch.nn.Conv2d(3, 6, kernel_size=(3, 3))
+
+        def forward(self, x):
+            return self.conv(torch.nn.functional.pad(x, [2, 2]))
+
+    from daceml_amd.torch import DaceModule
+    from daceml_amd.transformation import fusion
+    torch.manual_seed(11)
+    net, x = Module(), torch.rand(4, 3, 24, 24)
+    model = DaceModule(net, auto_optimize=False)._import((x, ))
+    assert sorted(n.schema.name for n in model.sdfg.states()[0].library_nodes()) == ["Conv", "Pad"]
+    assert fusion.fuse_pad_into_conv(model.sdfg) == 1
+    nodes = model.sdfg.states()[0].library_nodes()
+    assert [n.schema.name for n in nodes] == ["Conv"] and nodes[0].pads == [0, 2, 0, 2]
+    _, got = _run_emulated(model, net, x)
+    assert_close(got, net.double()(x.double()).detach().numpy(), torch.float32, "reference pad + conv module", rtol=1e-5,
+                 atol=2e-6)
+
+
 def test_padding_adds_to_the_padding_the_conv_has():
     torch.manual_seed(4)
     net = torch.nn.Sequential(torch.nn.ZeroPad2d(1), torch.nn.Conv2d(3, 5, 5, padding=1))
