@@ -1,0 +1,185 @@
+"""The modules of the reference's own autodiff test (tests/autodiff/torch/test_pytorch.py:76-262), differentiated here
+the way its ``run_pytorch_module`` does (:13-73): the module's output is reduced with ``sum()`` or ``max()``, and the
+gradient that reaches the input is compared with PyTorch's.
+
+On the CPU the whole pipeline runs - export, import, the training form of the fusion pipeline, the backward pass, the
+backward rewrites, expansion - and the calls of both states are interpreted by tests/abi_emulator.py; the gradient of
+the reduction (ones, or a one at the maximum) is what the caller's autograd would hand over. On the GPU the same
+modules run through ``DaceModule(backward=True)`` with the reference's tolerances; those tests compose kernels that run
+on hardware, in shapes nothing else uses: a first run."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from tests.util import first_run_on_hardware
+
+
+class Simple(nn.Module):
+    def forward(self, x):
+        return torch.log(torch.sqrt(x))
+
+
+class Repeated(nn.Module):
+    def forward(self, x):
+        return torch.sqrt(torch.sqrt(x))
+
+
+class Softmax(nn.Module):
+    def forward(self, x):
+        return F.softmax(x, dim=1)
+
+
+class ReshapeOnPath(nn.Module):
+    def forward(self, x):
+        reshaped = torch.reshape(x + 1, [3, 3])
+        return torch.log(reshaped) + torch.reshape(torch.tensor([[3, 2, 1]], device=reshaped.device), [3])
+
+
+class WeightsLN(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc1 = nn.Linear(784, 120)
+        self.fc2 = nn.Linear(120, 32)
+        self.ln = nn.LayerNorm(32)
+        self.fc3 = nn.Linear(32, 10)
+
+    def forward(self, x):
+        x = F.relu(self.fc1(x))
+        x = F.relu(self.fc2(x))
+        return self.fc3(self.ln(x))
+
+
+class LN(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.ln = nn.LayerNorm(3)
+
+    def forward(self, x):
+        return self.ln(x)
+
+
+class Weights(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc1 = nn.Linear(784, 120)
+        self.fc2 = nn.Linear(120, 32)
+        self.fc3 = nn.Linear(32, 10)
+
+    def forward(self, x):
+        return self.fc3(F.relu(self.fc2(F.relu(self.fc1(x)))))
+
+
+class NestedSum(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc1 = nn.Parameter(torch.rand(10, 10))
+
+    def forward(self, x):
+        return x * 2 + x @ self.fc1
+
+
+class TransAdd(nn.Module):
+    def forward(self, x):
+        return torch.transpose((x + 1).reshape(4, 4), 1, 0)
+
+
+class BatchedMatmul(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc1 = nn.Parameter(torch.ones([10, 5, 3]))
+
+    def forward(self, x):
+        return self.fc1 @ x
+
+
+class ScalarForwarding(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.factor = nn.Parameter(torch.ones(()))
+
+    def forward(self, x):
+        return self.factor * x
+
+
+class ScalarBuffer(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.register_buffer("factor", torch.tensor(2))
+
+    def forward(self, x):
+        return self.factor * x
+
+
+class BroadcastedMul(nn.Module):
+    def forward(self, x):
+        return x * x.sum(axis=0)
+
+
+CASES = [("simple", Simple, {}), ("repeated", Repeated, {}), ("softmax", Softmax, dict(use_max=True)),
+         ("reshape_on_memlet_path", ReshapeOnPath, dict(shape=(9, ))), ("weights_ln", WeightsLN, dict(shape=(4, 784))),
+         ("layernorm", LN, dict(shape=(1, 3), use_max=True)), ("weights", Weights, dict(shape=(4, 784))),
+         ("nested_gradient_summation", NestedSum, dict(shape=(4, 10))), ("trans_add", TransAdd, dict(shape=(16, ))),
+         ("batched_matmul", BatchedMatmul, {}), ("scalar_forwarding", ScalarForwarding, {}),
+         ("scalar_buffer", ScalarBuffer, {}), ("simple_broadcasted_mul", BroadcastedMul, {})]
+
+
+def _emulated_input_gradient(module, shape=(3, 5), use_max=False):
+    from daceml_amd.autodiff import add_backward_pass
+    from daceml_amd.onnx.onnx_importer import clean_onnx_name
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.torch import DaceModule
+    from daceml_amd.transformation import fusion
+    from tests.abi_emulator import run_sdfg
+    torch.manual_seed(0)
+    x = torch.rand(*shape, dtype=torch.float32)
+    xt = x.clone().requires_grad_(True)
+    out = module(xt)
+    (out.max() if use_max else out.sum()).backward()
+    model = DaceModule(module, backward=True, auto_optimize=False)._import((x, ))
+    sdfg, st = model.sdfg, model.sdfg.states()[0]
+    fusion.auto_optimize(sdfg, training=True)
+    names = [clean_onnx_name(n) for n in model.inputs]
+    add_backward_pass(sdfg, st, list(model.outputs), names[:1])
+    fusion.optimize_backward(sdfg)
+    expand_onnx_nodes(sdfg)
+    tensors = dict(module.named_parameters())
+    tensors.update(dict(module.named_buffers()))
+    arrays = {names[0]: x.numpy().copy()}
+    for n in model.inputs[1:]:
+        arrays[clean_onnx_name(n)] = tensors[n].detach().numpy().copy()
+    g = torch.zeros_like(out)
+    if use_max:
+        g.view(-1)[out.argmax()] = 1.0
+    else:
+        g[...] = 1.0
+    arrays["gradient_" + model.outputs[0]] = g.numpy().copy()
+    run_sdfg(sdfg, arrays)
+    return arrays["gradient_" + names[0]], xt.grad.numpy()
+
+
+@pytest.mark.parametrize("name", [c[0] for c in CASES])
+def test_reference_autodiff_module_lowers_correctly(name):
+    _, make, kwargs = next(c for c in CASES if c[0] == name)
+    got, want = _emulated_input_gradient(make(), **kwargs)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+@first_run_on_hardware("written without access to a GPU: first run on hardware")
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", [c[0] for c in CASES])
+def test_reference_autodiff_module_on_gpu(name):
+    from daceml_amd.torch import DaceModule
+    _, make, kwargs = next(c for c in CASES if c[0] == name)
+    torch.manual_seed(0)
+    module = make().cuda()
+    shape, use_max = kwargs.get("shape", (3, 5)), kwargs.get("use_max", False)
+    value = torch.rand(*shape, dtype=torch.float32).cuda()
+    pytorch_input = value.clone().requires_grad_(True)
+    out = module(pytorch_input)
+    (out.max() if use_max else out.sum()).backward()
+    dace_input = value.clone().requires_grad_(True)
+    out = DaceModule(module, backward=True)(dace_input)
+    (out.max() if use_max else out.sum()).backward()
+    torch.testing.assert_close(dace_input.grad, pytorch_input.grad, rtol=1e-4, atol=1e-3)   # the reference's tolerances
