@@ -383,6 +383,14 @@ class Emulator:
                 x = self._typed(x, np.float16 if call.symbol.endswith("f16") else np.float32)
                 y = self._typed(y, np.float16 if out_dtype == L.F16 else np.float32)
                 reduce(op, x, y, out_dtype, outer, r, inner)
+            elif call.symbol in ("dmlhip_reduce_sum_multi_f16", "dmlhip_reduce_sum_multi_f32"):
+                count, xs, ys, out_dtype, rows, cols = args[:6]
+                assert len(xs) == len(ys) == count <= L.MULTI_MAX if hasattr(L, "MULTI_MAX") else len(xs) == len(ys) == count
+                want = np.float16 if out_dtype == L.F16 else np.float32
+                for x, y, r, c in zip(xs, ys, rows[:count], cols[:count]):
+                    if y.dtype != want:
+                        raise TypeError("multi reduce output is %s, out_dtype says %s" % (y.dtype, want))
+                    y.reshape(-1)[:c] = x.reshape(-1)[:r * c].astype(np.float64).reshape(r, c).sum(0).astype(want)
             elif call.symbol in ("dmlhip_transpose_f16", "dmlhip_transpose_f32"):
                 x, y, ndim, shape, perm = args[:5]
                 dt = np.float16 if call.symbol.endswith("f16") else np.float32
