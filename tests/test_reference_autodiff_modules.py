@@ -243,3 +243,46 @@ def test_reference_conv2d_model_on_gpu():
     torch_output.backward(dy)
     torch.testing.assert_close(dace_output, torch_output, rtol=1e-5, atol=1e-6)
     torch.testing.assert_close(dace_inputs.grad, torch_inputs.grad, rtol=1e-5, atol=1e-6)
+
+
+# ----------------------------------------------------------------------------- tests/torch/test_img_op_implementations.py
+def _emulated_forward(net, x, training):
+    from daceml_amd.onnx.onnx_importer import clean_onnx_name
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.torch import DaceModule
+    from tests.abi_emulator import run_state
+    model = DaceModule(net, training=training)._import((x, ))
+    st = model.sdfg.states()[0]
+    expand_onnx_nodes(model.sdfg)
+    tensors = dict(net.named_parameters())
+    tensors.update(dict(net.named_buffers()))
+    arrays = {clean_onnx_name(model.inputs[0]): x.numpy().copy()}
+    for n in model.inputs[1:]:
+        arrays[clean_onnx_name(n)] = tensors[n].detach().numpy().copy()
+    run_state(model.sdfg, st, arrays)
+    return model, arrays
+
+
+def test_reference_batchnorm_module_lowers_correctly():
+    """test_bn (:9-29): ``BatchNorm2d(64)`` in training mode on [1, 64, 60, 60] - output and both running statistics."""
+    from daceml_amd.onnx.onnx_importer import clean_onnx_name
+    torch.manual_seed(0)
+    x = torch.rand(1, 64, 60, 60)
+    pt_model, dace_model = nn.BatchNorm2d(64), nn.BatchNorm2d(64)
+    dace_model.load_state_dict(pt_model.state_dict())
+    model, arrays = _emulated_forward(dace_model, x, training=True)
+    want = pt_model(x)
+    np.testing.assert_allclose(arrays[model.outputs[0]], want.detach().numpy(), rtol=1e-4, atol=1e-5)
+    # the running statistics come back either in place or as further outputs, depending on what reads them
+    written = {n: a for n, a in arrays.items() if a.shape == (64, )}
+    assert any(np.allclose(a, pt_model.running_mean.numpy(), rtol=1e-4, atol=1e-6) for a in written.values())
+    assert any(np.allclose(a, pt_model.running_var.numpy(), rtol=1e-4, atol=1e-6) for a in written.values())
+    assert clean_onnx_name("running_mean") in arrays
+
+
+def test_reference_global_average_pool_module_lowers_correctly():
+    """test_global_avg_pool (:32-42): ``AdaptiveAvgPool2d(1)`` on [1, 64, 60, 60]."""
+    torch.manual_seed(0)
+    x = torch.rand(1, 64, 60, 60)
+    model, arrays = _emulated_forward(nn.AdaptiveAvgPool2d(1), x, training=True)
+    np.testing.assert_allclose(arrays[model.outputs[0]], nn.AdaptiveAvgPool2d(1)(x).numpy(), rtol=1e-5, atol=1e-6)
