@@ -108,6 +108,10 @@ SIGNATURES = {
     "dmlhip_row_dot_f32": (c_int, [_P, _P, _P, c_int64, c_int64, _P]),
     "dmlhip_transpose_f16": (c_int, [_P, _P, c_int, _I64P, _I64P, _P]),
     "dmlhip_transpose_f32": (c_int, [_P, _P, c_int, _I64P, _I64P, _P]),
+    "dmlhip_maxpool2d_f16": (c_int, [_P, _P] + [c_int64] * 7 + [_P]),
+    "dmlhip_maxpool2d_f32": (c_int, [_P, _P] + [c_int64] * 7 + [_P]),
+    "dmlhip_maxpool2d_backward_f16": (c_int, [_P, _P, _P] + [c_int64] * 7 + [_P]),
+    "dmlhip_maxpool2d_backward_f32": (c_int, [_P, _P, _P] + [c_int64] * 7 + [_P]),
     "dmlhip_pad_constant_f16": (c_int, [_P, _P, c_int, _I64P, _I64P, _I64P, c_float, _P]),
     "dmlhip_pad_constant_f32": (c_int, [_P, _P, c_int, _I64P, _I64P, _I64P, c_float, _P]),
     "dmlhip_gemm_f16": (c_int, [POINTER(GemmDesc), _P, _P, _P, _P, _P, _P, _P]),

@@ -813,6 +813,23 @@ class HipPadBackward(BackwardImplementation):
         return g, BackwardResult(required_grad_names={"data": "output"}, given_grad_names={"output": "data"})
 
 
+@autoregister_params(op="MaxPool", name=NAME)
+class HipMaxPoolBackward(BackwardImplementation):
+    """DefaultMaxPoolBackward (onnx_ops.py:284-335): one MaxPoolGrad node, which reads the forward input."""
+    @staticmethod
+    def backward_can_be_applied(node, state, sdfg) -> bool:
+        return not any(e.src_conn == "Indices" for e in state.out_edges(node))
+
+    @staticmethod
+    def backward(forward_node, context, given_gradients, required_gradients):
+        g = _new(context, "MaxPoolGrad", forward_node.label + "_backward", kernel_shape=list(forward_node.kernel_shape),
+                 strides=None if forward_node.strides is None else list(forward_node.strides))
+        _read(context, _in_arr(context, forward_node, "X"), g, "X")
+        g.add_in_connector("dY")
+        g.add_out_connector("dX")
+        return g, BackwardResult(required_grad_names={"X": "dX"}, given_grad_names={"Y": "dY"})
+
+
 @autoregister_params(op="GlobalAveragePool", name=NAME)
 class HipGlobalAveragePoolBackward(BackwardImplementation):
     """Y = mean of X over the spatial dims (img_op_implementations.py:415-417): dX = dY / (H*W), broadcast back over

@@ -21,6 +21,7 @@ SOURCES = [
     "reduce.hip",
     "transpose.hip",
     "pad.hip",
+    "pool.hip",
     "gemm_f16.hip",
     "gemm_f16_pipe.hip",
     "gemm_f16_pipe_ilv.hip",

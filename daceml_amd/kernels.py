@@ -343,6 +343,38 @@ def transpose(x: torch.Tensor, perm: Optional[Sequence[int]] = None) -> torch.Te
     return y
 
 
+def _pool_geometry(x, kernel, stride):
+    if x.dim() != 4:
+        raise ValueError("max_pool2d takes [N, C, H, W] tensors")
+    kh, kw = kernel
+    sh, sw = stride
+    n, c, h, w = x.shape
+    oh = (h - kh) // sh + 1 if h >= kh else 0
+    ow = (w - kw) // sw + 1 if w >= kw else 0
+    return n * c, h, w, kh, kw, sh, sw, oh, ow
+
+
+def max_pool2d(x: torch.Tensor, kernel: Sequence[int], stride: Sequence[int]) -> torch.Tensor:
+    """MaxPool without padding or dilation (floor output extents)."""
+    _check(x)
+    x = _dense(x)
+    planes, h, w, kh, kw, sh, sw, oh, ow = _pool_geometry(x, kernel, stride)
+    y = torch.empty((x.shape[0], x.shape[1], oh, ow), dtype=x.dtype, device=x.device)
+    L.check(_fn("maxpool2d", x.dtype)(_ptr(x), _ptr(y), planes, h, w, kh, kw, sh, sw, _stream()))
+    return y
+
+
+def max_pool2d_backward(x: torch.Tensor, dy: torch.Tensor, kernel: Sequence[int], stride: Sequence[int]) -> torch.Tensor:
+    _check(x, dy)
+    x, dy = _dense(x), _dense(dy)
+    planes, h, w, kh, kw, sh, sw, oh, ow = _pool_geometry(x, kernel, stride)
+    if tuple(dy.shape) != (x.shape[0], x.shape[1], oh, ow):
+        raise ValueError("gradient of shape %s for an output of shape %s" % (tuple(dy.shape), (x.shape[0], x.shape[1], oh, ow)))
+    dx = torch.empty_like(x)
+    L.check(_fn("maxpool2d_backward", x.dtype)(_ptr(x), _ptr(dy), _ptr(dx), planes, h, w, kh, kw, sh, sw, _stream()))
+    return dx
+
+
 def pad(x: torch.Tensor, pads: Sequence[int], value: float = 0.0) -> torch.Tensor:
     """ONNX Pad in constant mode: ``pads`` lists the amounts in front of every axis, then those behind (negative
     amounts crop)."""

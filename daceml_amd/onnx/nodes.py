@@ -115,6 +115,10 @@ SCHEMAS = [
     _schema("Conv", "X W B?", "Y", auto_pad="NOTSET", dilations=None, group=1, kernel_shape=None, pads=None,
             strides=None),
     _schema("GlobalAveragePool", "X", "Y"),
+    _schema("MaxPool", "X", "Y Indices?", auto_pad="NOTSET", ceil_mode=0, dilations=None, kernel_shape=REQUIRED, pads=None,
+            storage_order=0, strides=None),
+    # reverse of MaxPool: the reference's DefaultMaxPoolBackward reads the forward input and the output gradient
+    _schema("MaxPoolGrad", "X dY", "dX", since=1, kernel_shape=REQUIRED, strides=None),
     # Pad in its attribute form: the importer turns the `pads` / `constant_value` inputs of opset 11+ into these when
     # they are known at import time. fusion.fuse_pad_into_conv folds it into the Conv that reads it, as PadConvFusion
     # does (daceml/transformation/pad_conv_fusion.py:13-104); what does not fold runs on the constant-pad kernel (the

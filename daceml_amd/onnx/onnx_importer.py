@@ -445,6 +445,20 @@ class ONNXModel:
             return [(x[0], w[0]) + tuple(out)], [dt], ins, attrs
         if op == "GlobalAveragePool":
             return [tuple(shp[0][:2]) + (1, ) * (len(shp[0]) - 2)], [dt], ins, attrs
+        if op == "MaxPool":
+            x = shp[0]
+            nsp = len(x) - 2
+            k = list(attrs["kernel_shape"])
+            strides = list(attrs.get("strides") or [1] * nsp)
+            pads = list(attrs.get("pads") or [0] * (2 * nsp))
+            dil = list(attrs.get("dilations") or [1] * nsp)
+            if attrs.get("auto_pad", "NOTSET") != "NOTSET":
+                raise UnsupportedModel("MaxPool node %r: auto_pad %r is not supported" % (node.name, attrs["auto_pad"]))
+            out = []
+            for i in range(nsp):
+                span = x[2 + i] + pads[i] + pads[nsp + i] - ((k[i] - 1) * dil[i] + 1)
+                out.append((-(-span // strides[i]) if int(attrs.get("ceil_mode", 0)) else span // strides[i]) + 1)
+            return [tuple(x[:2]) + tuple(out)], [dt], ins, attrs
         if op == "Pad":
             # opset 11+: pads and the fill value are inputs; they become attributes, and have to be known now
             mode = attrs.get("mode", "constant")

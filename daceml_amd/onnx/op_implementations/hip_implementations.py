@@ -969,6 +969,74 @@ class HipGlobalAveragePool(ONNXForward):
         return _tasklet(node, state, [call], bytes_moved=_nbytes(x), kind="reduce")
 
 
+def _pool_geometry(node, x: Array):
+    """(kh, kw, sh, sw, oh, ow) of a MaxPool / MaxPoolGrad node over [N, C, H, W]."""
+    kh, kw = (int(v) for v in node.kernel_shape)
+    sh, sw = (int(v) for v in (node.strides or [1, 1]))
+    h, w = x.shape[2], x.shape[3]
+    return kh, kw, sh, sw, ((h - kh) // sh + 1 if h >= kh else 0), ((w - kw) // sw + 1 if w >= kw else 0)
+
+
+@op_implementation(op="MaxPool", name=IMPL)
+class HipMaxPool(ONNXForward):
+    """PureMaxPool2D (img_op_implementations.py:28-161), with its conditions: two spatial axes, no padding, no dilation,
+    no ``Indices`` output, ``ceil_mode`` and ``storage_order`` 0."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            x = in_desc_with_name(node, state, sdfg, "X")
+            y = out_desc_with_name(node, state, sdfg, "Y")
+            if _has_out(node, state, "Indices") or len(x.shape) != 4 or not (_float_ok(x, y) and _dense(x, y)):
+                return False
+            if node.auto_pad != "NOTSET" or node.ceil_mode != 0 or node.storage_order != 0:
+                return False
+            if len(node.kernel_shape) != 2 or (node.strides is not None and len(node.strides) != 2):
+                return False
+            if any(p != 0 for p in (node.pads or [])) or any(d != 1 for d in (node.dilations or [])):
+                return False
+            kh, kw, sh, sw, oh, ow = _pool_geometry(node, x)
+            return min(kh, kw, sh, sw) >= 1 and tuple(y.shape) == (x.shape[0], x.shape[1], oh, ow)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "X")
+        y = out_desc_with_name(node, state, sdfg, "Y")
+        kh, kw, sh, sw, _, _ = _pool_geometry(node, x)
+        call = HipCall("dmlhip_maxpool2d_" + _SFX[x.dtype],
+                       [Ptr("X"), Ptr("Y"), I64(x.shape[0] * x.shape[1]), I64(x.shape[2]), I64(x.shape[3]), I64(kh), I64(kw),
+                        I64(sh), I64(sw), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=_nbytes(x, y), kind="pool")
+
+
+@op_implementation(op="MaxPoolGrad", name=IMPL)
+class HipMaxPoolGrad(ONNXForward):
+    """DefaultMaxPoolBackward (autodiff/implementations/onnx_ops.py:284-335) as one kernel: the gradient of each window
+    goes to the first position of the window that holds its maximum."""
+    @staticmethod
+    def forward_can_be_applied(node, state, sdfg) -> bool:
+        try:
+            ins, outs = _descs(node, state, sdfg)
+            x, dy, dx = ins["X"], ins["dY"], outs["dX"]
+            if len(x.shape) != 4 or not (_float_ok(x, dy, dx) and _dense(x, dy, dx)) or x.shape != dx.shape:
+                return False
+            kh, kw, sh, sw, oh, ow = _pool_geometry(node, x)
+            return min(kh, kw, sh, sw) >= 1 and tuple(dy.shape) == (x.shape[0], x.shape[1], oh, ow)
+        except Exception:
+            return False
+
+    @staticmethod
+    def forward(node, state, sdfg):
+        x = in_desc_with_name(node, state, sdfg, "X")
+        dy = in_desc_with_name(node, state, sdfg, "dY")
+        kh, kw, sh, sw, _, _ = _pool_geometry(node, x)
+        call = HipCall("dmlhip_maxpool2d_backward_" + _SFX[x.dtype],
+                       [Ptr("X"), Ptr("dY"), Ptr("dX"), I64(x.shape[0] * x.shape[1]), I64(x.shape[2]), I64(x.shape[3]),
+                        I64(kh), I64(kw), I64(sh), I64(sw), Stream()])
+        return _tasklet(node, state, [call], bytes_moved=2 * _nbytes(x) + _nbytes(dy), kind="pool")
+
+
 # ----------------------------------------------------------------------------- data movement
 @op_implementation(op="Transpose", name=IMPL)
 class HipTranspose(ONNXForward):

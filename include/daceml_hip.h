@@ -203,6 +203,21 @@ int dmlhip_transpose_f16(const void* x, void* y, int ndim, const int64_t* shape,
 int dmlhip_transpose_f32(const void* x, void* y, int ndim, const int64_t* shape,
                          const int64_t* perm, void* stream);
 
+/* ------------------------------------------------------------------ MaxPool
+ * PureMaxPool2D (img_op_implementations.py:28-161): x is `planes` = batch * channels images of h x w, the window
+ * kh x kw moves by sh, sw; no padding, no dilation, output extents (h - kh) / sh + 1 and (w - kw) / sw + 1 rounded
+ * down. The backward entry point is DefaultMaxPoolBackward (autodiff/implementations/onnx_ops.py:284-335): dx receives
+ * the gradient of every window at the first position (row by row) that holds the window's maximum, zero elsewhere;
+ * it needs x, not the forward output. */
+int dmlhip_maxpool2d_f16(const void* x, void* y, int64_t planes, int64_t h, int64_t w, int64_t kh, int64_t kw,
+                         int64_t sh, int64_t sw, void* stream);
+int dmlhip_maxpool2d_f32(const void* x, void* y, int64_t planes, int64_t h, int64_t w, int64_t kh, int64_t kw,
+                         int64_t sh, int64_t sw, void* stream);
+int dmlhip_maxpool2d_backward_f16(const void* x, const void* dy, void* dx, int64_t planes, int64_t h, int64_t w,
+                                  int64_t kh, int64_t kw, int64_t sh, int64_t sw, void* stream);
+int dmlhip_maxpool2d_backward_f32(const void* x, const void* dy, void* dx, int64_t planes, int64_t h, int64_t w,
+                                  int64_t kh, int64_t kw, int64_t sh, int64_t sw, void* stream);
+
 /* ------------------------------------------------------------------ Pad
  * ONNX Pad, mode "constant", with the amounts and the fill value known when the node is lowered. The reference has no
  * expansion for it (a stand-alone Pad runs in onnxruntime; PadConvFusion, transformation/pad_conv_fusion.py:13-104,

@@ -138,6 +138,44 @@ def reduce_mean(data, axes=None, keepdims=1):
     return np.mean(data, axis=_norm_axes(axes, data.ndim), keepdims=bool(keepdims))
 
 
+def maxpool2d(X, kernel_shape, strides=None):
+    """MaxPool "pure": img_op_implementations.py:28-161 - two spatial axes, no padding, no dilation, output extents
+    rounded down; Y starts at the smallest value and takes the maximum over ``X[b, c, out*stride + h]`` (:19-21,
+    :141-143)."""
+    kh, kw = kernel_shape
+    sh, sw = strides if strides is not None else (1, 1)
+    n, c, h, w = X.shape
+    oh, ow = (h - kh) // sh + 1, (w - kw) // sw + 1
+    Y = np.full((n, c, oh, ow), -np.inf, dtype=X.dtype)
+    for hy in range(kh):
+        for hx in range(kw):
+            Y = np.maximum(Y, X[:, :, hy:hy + (oh - 1) * sh + 1:sh, hx:hx + (ow - 1) * sw + 1:sw])
+    return Y
+
+
+def maxpool2d_backward(X, Y_grad, kernel_shape, strides):
+    """DefaultMaxPoolBackward: autodiff/implementations/onnx_ops.py:284-335. Per output element the window is scanned
+    row by row with a strict comparison ("deterministic argmax"), and the gradient goes to the first maximum. Windows
+    that overlap add up here (as in PyTorch); the reference's tasklet assigns, which agrees wherever windows do not
+    overlap - every case its own tests run."""
+    kh, kw = kernel_shape
+    sh, sw = strides
+    n, c, oh, ow = Y_grad.shape
+    X_grad = np.zeros_like(X)
+    for b in range(n):
+        for ch in range(c):
+            for ti in range(oh):
+                for tj in range(ow):
+                    win = X[b, ch, sh * ti:sh * ti + kh, sw * tj:sw * tj + kw]
+                    best, bi, bj = win[0, 0], 0, 0
+                    for i in range(kh):
+                        for j in range(kw):
+                            if win[i, j] > best:
+                                best, bi, bj = win[i, j], i, j
+                    X_grad[b, ch, sh * ti + bi, sw * tj + bj] += Y_grad[b, ch, ti, tj]
+    return X_grad
+
+
 def global_average_pool(X):
     """GlobalAveragePool "pure": img_op_implementations.py:415-417; output keeps 1x1 spatial dims."""
     return np.mean(X, axis=(2, 3), keepdims=True)

@@ -398,6 +398,23 @@ class Emulator:
                 shape, perm = tuple(shape[:ndim]), tuple(perm[:ndim])
                 n = int(np.prod(shape))
                 y.reshape(-1)[:n] = np.transpose(x.reshape(-1)[:n].reshape(shape), perm).reshape(-1)
+            elif call.symbol in ("dmlhip_maxpool2d_f16", "dmlhip_maxpool2d_f32", "dmlhip_maxpool2d_backward_f16",
+                                 "dmlhip_maxpool2d_backward_f32"):
+                import torch
+                backward = "backward" in call.symbol
+                x, a1 = args[0], args[1]
+                planes, h, w, kh, kw, sh, sw = args[3:10] if backward else args[2:9]
+                xt = torch.from_numpy(x.reshape(-1)[:planes * h * w].astype(np.float64).reshape(1, planes, h, w))
+                oh, ow = ((h - kh) // sh + 1 if h >= kh else 0), ((w - kw) // sw + 1 if w >= kw else 0)
+                if not backward:
+                    out = torch.nn.functional.max_pool2d(xt, (kh, kw), (sh, sw)).numpy()
+                    a1.reshape(-1)[:out.size] = out.reshape(-1).astype(a1.dtype)
+                else:
+                    dx = args[2]
+                    xt.requires_grad_(True)
+                    g = torch.from_numpy(a1.reshape(-1)[:planes * oh * ow].astype(np.float64).reshape(1, planes, oh, ow))
+                    torch.nn.functional.max_pool2d(xt, (kh, kw), (sh, sw)).backward(g)
+                    dx.reshape(-1)[:planes * h * w] = xt.grad.numpy().reshape(-1).astype(dx.dtype)
             elif call.symbol in ("dmlhip_pad_constant_f16", "dmlhip_pad_constant_f32"):
                 x, y, ndim, shape, begin, end, value = args[:7]
                 dt = np.float16 if call.symbol.endswith("f16") else np.float32

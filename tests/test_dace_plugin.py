@@ -159,6 +159,11 @@ def _sample_sdfgs():
                  "y")
         add_backward_pass(g.sdfg, g.state, ["y"], ["x"])
         out.append(("log_softmax_train_" + tag, g.sdfg))
+        g = graphs.GraphBuilder("maxpool_" + tag, dtype)
+        g.output(g.node("MaxPool", {"X": g.input("x", (2, 3, 9, 8))}, {"Y": (2, 3, 4, 3)}, label="pool", kernel_shape=[3, 3],
+                        strides=[2, 2])["Y"], "y")
+        add_backward_pass(g.sdfg, g.state, ["y"], ["x"])
+        out.append(("maxpool_train_" + tag, g.sdfg))
     return out
 
 

@@ -422,3 +422,38 @@ def test_constant_pad_refuses_a_crop_larger_than_the_axis(pad_lib):
     i64 = lambda t: (ctypes.c_int64 * len(t))(*t)  # noqa: E731
     assert pad_lib.emu_pad(x.ctypes.data_as(ctypes.c_void_p), x.ctypes.data_as(ctypes.c_void_p), 2, i64((4, 4)),
                            i64((-3, 0)), i64((-2, 0)), ctypes.c_float(0.0), 1) < 0
+
+
+# ----------------------------------------------------------------------------- MaxPool
+@pytest.fixture(scope="module")
+def pool_lib(tmp_path_factory):
+    lib = _build(str(tmp_path_factory.mktemp("emu_pool")), "emu_pool", "pool_harness.cpp", ["common.h", "pool.hip"])
+    lib.emu_maxpool.restype = ctypes.c_int
+    lib.emu_maxpool.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int64] * 7 + [ctypes.c_uint]
+    return lib
+
+
+@pytest.mark.parametrize("shape,kernel,stride", [((2, 6, 28, 28), (2, 2), (2, 2)),     # the pools of the reference's LeNet
+                                                 ((2, 3, 13, 13), (2, 2), (2, 2)),     # a last row and column left over
+                                                 ((1, 2, 9, 7), (3, 3), (2, 2)),       # overlapping windows
+                                                 ((2, 1, 7, 10), (3, 2), (1, 3)),      # gaps between windows
+                                                 ((1, 1, 5, 5), (5, 5), (1, 1)),       # one window
+                                                 ((1, 2, 4, 4), (1, 1), (1, 1))])      # the identity
+def test_maxpool_kernels(pool_lib, shape, kernel, stride):
+    """Forward and backward kernels through their host functions against PyTorch (which also sends the gradient to the
+    first maximum of a window); quantised inputs make equal maxima common."""
+    import torch
+    r = np.random.default_rng(sum(shape))
+    x = np.round(r.standard_normal(shape) * 2).astype(np.float32)
+    n, c, h, w = shape
+    xt = torch.tensor(x.astype(np.float64), requires_grad=True)
+    want = torch.nn.functional.max_pool2d(xt, kernel, stride)
+    dy = r.standard_normal(tuple(want.shape)).astype(np.float32)
+    want.backward(torch.tensor(dy.astype(np.float64)))
+    y = np.full(tuple(want.shape), np.nan, np.float32)
+    dx = np.full(shape, np.nan, np.float32)
+    ptr = lambda a: a.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
+    assert pool_lib.emu_maxpool(ptr(x), None, ptr(y), n * c, h, w, *kernel, *stride, 1) == 0
+    assert np.array_equal(y, want.detach().numpy().astype(np.float32))
+    assert pool_lib.emu_maxpool(ptr(x), ptr(dy), ptr(dx), n * c, h, w, *kernel, *stride, 2) == 0
+    np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-6, atol=1e-6)

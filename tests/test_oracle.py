@@ -62,6 +62,26 @@ def test_softmax_backward_matches_autograd():
     assert np.abs(O.softmax_backward(y.detach().numpy(), dy.numpy(), 2).sum(-1)).max() < 1e-12
 
 
+@pytest.mark.parametrize("shape,kernel,stride", [((2, 3, 8, 8), (2, 2), (2, 2)), ((1, 2, 9, 7), (3, 3), (2, 2)),
+                                                 ((2, 1, 7, 10), (3, 2), (1, 3)), ((1, 1, 5, 5), (5, 5), (1, 1))])
+def test_maxpool_matches_torch_and_autograd(shape, kernel, stride):
+    x = rng(50).standard_normal(shape)
+    want = F.max_pool2d(torch.tensor(x), kernel, stride)
+    np.testing.assert_array_equal(O.maxpool2d(x, kernel, stride), want.numpy())
+    dy = rng(51).standard_normal(tuple(want.shape))
+    xt = torch.tensor(x, requires_grad=True)
+    F.max_pool2d(xt, kernel, stride).backward(torch.tensor(dy))
+    np.testing.assert_allclose(O.maxpool2d_backward(x, dy, kernel, stride), xt.grad.numpy(), rtol=1e-14, atol=1e-14)
+
+
+def test_maxpool_gradient_goes_to_the_first_of_equal_maxima():
+    x = np.zeros((1, 1, 2, 4))
+    x[0, 0] = [[1.0, 5.0, 5.0, 2.0], [5.0, 0.0, 7.0, 7.0]]
+    dx = O.maxpool2d_backward(x, np.array([[[[1.0, 10.0]]]]), (2, 2), (2, 2))
+    np.testing.assert_array_equal(dx[0, 0], [[0.0, 1.0, 0.0, 0.0], [0.0, 0.0, 10.0, 0.0]])
+    assert dx.sum() == 11.0                       # every output's gradient lands exactly once
+
+
 def test_log_softmax_matches_torch_scipy_and_keeps_small_probabilities():
     from scipy.special import log_softmax as scipy_log_softmax
     x = rng(40).standard_normal((3, 4, 9)) * 3
