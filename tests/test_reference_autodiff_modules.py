@@ -286,3 +286,45 @@ def test_reference_global_average_pool_module_lowers_correctly():
     x = torch.rand(1, 64, 60, 60)
     model, arrays = _emulated_forward(nn.AdaptiveAvgPool2d(1), x, training=True)
     np.testing.assert_allclose(arrays[model.outputs[0]], nn.AdaptiveAvgPool2d(1)(x).numpy(), rtol=1e-5, atol=1e-6)
+
+
+# ----------------------------------------------------------------------------- tests/torch/test_reshape.py, test_multi_output.py
+def test_reference_reshape_module_lowers_correctly():
+    """test_reshape_module (:20-35): ``x.reshape([5, 5])`` of a [25] input, without the fusion pipeline."""
+    from daceml_amd.torch import DaceModule
+
+    class Model(nn.Module):
+        def forward(self, x):
+            return x.reshape([5, 5])
+
+    from daceml_amd.onnx.onnx_importer import clean_onnx_name
+    from daceml_amd.runtime import expand_onnx_nodes
+    from tests.abi_emulator import run_state
+    x = torch.rand([25])
+    model = DaceModule(Model(), auto_optimize=False, dummy_inputs=None)._import((x, ))
+    st = model.sdfg.states()[0]
+    expand_onnx_nodes(model.sdfg)
+    arrays = {clean_onnx_name(model.inputs[0]): x.numpy().copy()}
+    run_state(model.sdfg, st, arrays)
+    np.testing.assert_array_equal(arrays[model.outputs[0]], x.numpy().reshape(5, 5))
+
+
+def test_reference_two_input_two_output_module_lowers_correctly():
+    """tests/torch/test_multi_output.py (:11-37): ``(x + y, x * y)`` style modules with several inputs and outputs."""
+    from daceml_amd.onnx.onnx_importer import clean_onnx_name
+    from daceml_amd.runtime import expand_onnx_nodes
+    from daceml_amd.torch import DaceModule
+    from tests.abi_emulator import run_state
+
+    class Model(nn.Module):
+        def forward(self, x, y):
+            return x + y, x * y
+
+    x, y = torch.rand(5, 10), torch.rand(5, 10)
+    model = DaceModule(Model())._import((x, y))
+    st = model.sdfg.states()[0]
+    expand_onnx_nodes(model.sdfg)
+    arrays = dict(zip([clean_onnx_name(n) for n in model.inputs], [x.numpy().copy(), y.numpy().copy()]))
+    run_state(model.sdfg, st, arrays)
+    np.testing.assert_allclose(arrays[model.outputs[0]], (x + y).numpy(), rtol=1e-6)
+    np.testing.assert_allclose(arrays[model.outputs[1]], (x * y).numpy(), rtol=1e-6)
