@@ -250,10 +250,12 @@ class HipFusedEinsumBackward(BackwardImplementation):
 # ----------------------------------------------------------------------------- softmax / layernorm
 @autoregister_params(op="Softmax", name=NAME)
 class HipSoftmaxBackward(BackwardImplementation):
-    """DefaultSoftmaxBackward (onnx_ops.py:237-275): ``prod = y * dy``; ``sums = ReduceSum(prod, axes=[axis],
-    keepdims=1)``; ``dx = prod - y * sums`` - the reduction runs over the single axis ``axis``, also where the forward
-    node coalesced several trailing axes. For the last axis that is one SoftmaxGrad node (one kernel, needs the forward
-    output); for any other axis the reference's own four nodes: Mul, ReduceSum, Mul, Sub."""
+    """DefaultSoftmaxBackward (onnx_ops.py:237-275): ``prod = y * dy``; ``sums = ReduceSum(prod, keepdims=1)``;
+    ``dx = prod - y * sums``. For the last axis that is one SoftmaxGrad node (one kernel, needs the forward output); for
+    any other axis the reference's own four nodes: Mul, ReduceSum, Mul, Sub. The sum runs over every axis the forward
+    node made one row of (``axis`` and all behind it), as in the LogSoftmax reverse below: the reference sums over
+    ``axes=[axis]`` alone, which is the same thing when the axes behind have extent 1 and otherwise is not the
+    derivative of its own (coalescing) forward."""
     @staticmethod
     def backward_can_be_applied(node, state, sdfg) -> bool:
         for e in state.in_edges_by_connector(node, "input"):
@@ -274,7 +276,7 @@ class HipSoftmaxBackward(BackwardImplementation):
             return sg, BackwardResult(required_grad_names={"input": "dX"}, given_grad_names={"output": "dY"})
         label = forward_node.label + "_backward"
         group = BackwardGroup(label)
-        sums_shape = tuple(1 if i == axis else e for i, e in enumerate(od.shape))
+        sums_shape = tuple(1 if i >= axis else e for i, e in enumerate(od.shape))
         prod, _ = sdfg.add_transient(label + "_prod", od.shape, od.dtype)
         sums, _ = sdfg.add_transient(label + "_sums", sums_shape, od.dtype)
         scaled, _ = sdfg.add_transient(label + "_scaled", od.shape, od.dtype)
@@ -283,7 +285,7 @@ class HipSoftmaxBackward(BackwardImplementation):
         mul1.add_in_connector("B")
         group.map_input("output_grad", mul1, "B")
         _write(context, mul1, "C", prod)
-        red = _new(context, "ReduceSum", label + "_sum", axes=[axis], keepdims=1)
+        red = _new(context, "ReduceSum", label + "_sum", axes=list(range(axis, nd)), keepdims=1)
         _read(context, prod, red, "data")
         _write(context, red, "reduced", sums)
         mul2 = _new(context, "Mul", label + "_mul_sums")

@@ -86,23 +86,6 @@ def build(force: bool = True, jobs: int = 8) -> str:
     return LIB_PATH
 
 
-PROBE_PATH = os.path.join(HERE, "gemm_probe")
-
-
-def build_probe() -> str:
-    """Compile gemm_probe.cpp (one contraction through the C ABI, for timing and counter runs) against the built
-    library. Returns the path of the executable."""
-    if not os.path.exists(LIB_PATH):
-        raise RuntimeError("build %s first" % LIB_NAME)
-    cmd = [hipcc(), "-O2", "--offload-arch=gfx950", os.path.join(HERE, "gemm_probe.cpp"), "-o", PROBE_PATH, "-L" + HERE,
-           "-ldaceml_hip", "-Wl,-rpath,$ORIGIN", "-Wno-unused-result"]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError("compiling gemm_probe.cpp failed:\n%s" % res.stderr[-4000:])
-    return PROBE_PATH
-
-
 if __name__ == "__main__":
     path = build(force="--incremental" not in sys.argv)
     print(path)
-    print(build_probe())

@@ -473,11 +473,29 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
         epilogue_kind(g, bias, residual, pre_out) != EPI_GENERAL_ACT) {
         if (cfg < 0) {
             auto blocks = [&](int bm, int bn) { return (long long)ceil_div(d->m, bm) * ceil_div(d->n, bn) * batch; };
-            // measured on MI355X inside the BERT layer: with more than one 128x128 tile per CU, two resident
-            // workgroups with two LDS stages each beat one workgroup with a deeper ring and the 256-wide
-            // tiles (whose epilogue, one workgroup per CU, overlaps with nothing)
-            if (blocks(128, 128) > 256) cfg = 3;
-            else cfg = 0;
+            const bool extra = grp || asum;   // operand pairs / row sums: the 128 x 128 tile only
+            const long long t256 = blocks(256, 256), t128 = blocks(128, 128);
+            const long long slots256 = ceil_div(t256, (long long)kCus) * kCus;
+            if (d->k < 512) {
+                // a handful of K steps (the batched products of an unfused attention): bound by the epilogue, where two
+                // resident workgroups per compute unit overlap one's stores with the other's loads
+                cfg = t128 > kCus ? 3 : 0;
+            } else if (!extra && t256 * 10 >= slots256 * 9) {
+                // Measured on MI355X, alone and inside the BERT layer (4096 x 4096 x 1024: 39 us against 45 - 54 us for
+                // every 128-wide tile; 8192^3: 1176 TFLOP/s): the 256 x 256 tile halves the bytes each compute unit
+                // pulls through L2 and LDS per MFMA, and the interleaved loop keeps its single wavefront per SIMD
+                // issuing MFMAs while transfers and fragment reads are in flight. Only when its tiles fill (nearly) every
+                // round of compute units: 192 tiles on 256 units lose more than the tile gains.
+                cfg = 4;
+            } else if (!extra && t128 <= kCus / 2) {
+                // few tiles and a long K (1024 x 1024 x 4096: 24 us against 29 - 38 us): the 128 x 64 tile doubles the
+                // workgroups, two of them per compute unit
+                cfg = 9;
+            } else {
+                // one 128 x 128 tile per compute unit, four LDS stages, interleaved loop: 5 - 20 % faster than the plain
+                // loop on every product of the layer with 4096 x 1024 or 1024 x 4096 outputs
+                cfg = 5;
+            }
         }
         return launch_pipelined(g, (const _Float16*)a, (const _Float16*)b, c, bias, residual, pre_out, amode == 1 ? 4 : 3,
                                 bmode == 1 ? 4 : 3, cfg, batch, st);

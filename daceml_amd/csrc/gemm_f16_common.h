@@ -13,6 +13,7 @@ constexpr int kThreads = 256;
 constexpr int BK = 64;         // K elements per step
 constexpr int kRowBytes = BK * 2;
 constexpr int kXcds = 8;
+constexpr int kCus = 256;   // compute units of an MI355X: what a "round" of workgroups means in the tile choice
 
 struct GemmArgs {
     int m, n, k;

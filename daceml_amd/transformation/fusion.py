@@ -301,8 +301,9 @@ def fuse_swish(sdfg: SDFG) -> int:
 def fuse_pad_into_conv(sdfg: SDFG) -> int:
     """A Pad with zeros along the spatial axes, read only by a Conv, becomes that Conv's padding (PadConvFusion,
     daceml/transformation/pad_conv_fusion.py:27-104: constant mode, fill value 0, nothing padded on the batch and
-    channel axes, the padded tensor has no other reader). One condition more than the reference: the padding that
-    results has to be the same before and after each spatial axis, which is what the convolution kernels take; a Pad
+    channel axes, the padded tensor has no other reader). Two conditions more than the reference: no entry of the
+    Pad is negative (a crop followed by a padded convolution is a different function), and the padding that results has
+    to be the same before and after each spatial axis, which is what the convolution kernels take; a Pad
     that does not fold stays in the graph and runs on the constant-pad kernel."""
     count = 0
     for state in sdfg.states():
@@ -318,6 +319,8 @@ def fuse_pad_into_conv(sdfg: SDFG) -> int:
             if pad.mode != "constant" or float(pad.value) != 0.0 or rank not in (3, 4) or len(pads) != 2 * rank:
                 continue
             if any(pads[i] or pads[rank + i] for i in (0, 1)) or conv.auto_pad != "NOTSET":
+                continue
+            if any(p < 0 for p in pads):   # a cropping Pad is not a padding of the convolution
                 continue
             have = [int(p) for p in (conv.pads or [0] * (2 * nsp))]
             begin = [have[i] + pads[2 + i] for i in range(nsp)]

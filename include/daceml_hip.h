@@ -102,7 +102,9 @@ int dmlhip_layernorm_backward_f32(const void* dy, const void* x, const float* me
  * until the process ends) of dmlhip_layernorm_backward_noalloc_max_bytes() = 8 MiB. Shapes whose
  * dmlhip_layernorm_backward_workspace_bytes(rows, cols) exceeds that are refused with
  * DMLHIP_ERR_WORKSPACE. The call allocates and frees nothing. Every call on a GPU shares that GPU's
- * array: calls that overlap on one GPU (different streams or threads) race; calls on one stream do not. */
+ * array: calls that overlap on one GPU (different streams or threads) race; calls on one stream do not.
+ * The first call on a device looks up the array's device address (hipGetSymbolAddress): make one ordinary
+ * call on each device before the first call under stream capture there. */
 size_t dmlhip_layernorm_backward_noalloc_max_bytes(void);
 int dmlhip_layernorm_backward_noalloc_f16(const void* dy, const void* x, const float* mean,
                                           const float* rstd, const void* gamma, void* dx,

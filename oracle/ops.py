@@ -209,6 +209,18 @@ def softmax_backward(output, output_grad, axis):
     return prod - input_grad
 
 
+def softmax_backward_rows(output, output_grad, axis):
+    """The derivative of ``softmax`` above as it is computed (opset-12: everything from ``axis`` on is one row):
+    ``dx = y*dy - y * sum_{axes >= axis}(y*dy)``. DefaultSoftmaxBackward sums over the single axis ``axis``, which is this
+    function when the axes behind ``axis`` have extent 1 (always the case for the last axis) and is not the derivative of
+    the reference's own forward otherwise; the build's reverse node follows this function. Pinned against autograd of
+    the flattened-row softmax in tests/test_oracle.py."""
+    axis = axis % output.ndim
+    prod = mul(output, output_grad)
+    sums = reduce_sum(prod, axes=list(range(axis, output.ndim)), keepdims=1)
+    return prod - mul(output, sums)
+
+
 def log_softmax(input, axis=1):
     """LogSoftmax (opset-12 semantics, the axes from ``axis`` on are one row): pure_implementations.py:649-656,
     statement by statement - the logarithm is taken of the row sum."""

@@ -1,16 +1,16 @@
-// One fp16 contraction through the C ABI of libdaceml_hip.so, timed with HIP events: the stand-alone program the
-// per-configuration counter runs of the GEMM kernels are taken with (and a minimal example of calling the library
-// from C++ without Python).
+// One fp16 contraction through the C ABI of libdaceml_hip.so from a C++ program (no Python, no torch): includes the
+// public header, links against the library, runs the product, times it with HIP events and, with `check`, compares
+// sampled outputs with a double-precision dot product on the host. tests/test_cabi_from_cpp.py builds it on the CPU
+// (the header and the exported symbols are usable from C++) and runs it with `check` on a GPU; the per-configuration
+// counter runs of the GEMM kernels are taken with it too.
 //
-//   gemm_probe M N K a-layout b-layout config iterations [check]
+//   gemm_from_cpp M N K a-layout b-layout config iterations [check]
 //     a-layout: k = A stored [m][k] (K-contiguous), r = A stored [k][m]
 //     b-layout: k = B stored [n][k] (K-contiguous), r = B stored [k][n]
 //     config:   tile configuration for dmlhip_debug_force_gemm_config (-1 = the library's own choice)
 //     check:    compare 2000 sampled outputs with a double-precision dot product on the host
 //
-// Build (from the repository root):
-//   hipcc -O2 --offload-arch=gfx950 daceml_amd/csrc/gemm_probe.cpp -o daceml_amd/csrc/gemm_probe \
-//         -Ldaceml_amd/csrc -ldaceml_hip -Wl,-rpath,'$ORIGIN'
+// Build: python tests/cabi/build.py
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -20,7 +20,7 @@
 #include <random>
 #include <vector>
 
-#include "../../include/daceml_hip.h"
+#include "daceml_hip.h"
 
 #define PROBE_CHECK(x)                                                                    \
     do {                                                                                  \
@@ -33,7 +33,7 @@
 
 int main(int argc, char** argv) {
     if (argc < 8) {
-        std::printf("usage: gemm_probe M N K a-layout(k|r) b-layout(k|r) config iterations [check]\n");
+        std::printf("usage: gemm_from_cpp M N K a-layout(k|r) b-layout(k|r) config iterations [check]\n");
         return 1;
     }
     const long M = std::atol(argv[1]), N = std::atol(argv[2]), K = std::atol(argv[3]);

@@ -62,6 +62,24 @@ def test_softmax_backward_matches_autograd():
     assert np.abs(O.softmax_backward(y.detach().numpy(), dy.numpy(), 2).sum(-1)).max() < 1e-12
 
 
+@pytest.mark.parametrize("shape,axis", [((3, 4, 9), 1), ((3, 5, 7, 9), 2), ((3, 5, 7, 9), 0), ((5, 33), 0), ((4, 6, 16), -1)])
+def test_softmax_backward_rows_is_the_derivative_of_the_coalescing_forward(shape, axis):
+    ax = axis % len(shape)
+    lead = int(np.prod(shape[:ax], dtype=np.int64))
+    x = torch.tensor(rng(5).standard_normal(shape), requires_grad=True)
+    dy = torch.tensor(rng(6).standard_normal(shape))
+    y = F.softmax(x.reshape(lead, -1), dim=1).reshape(shape)     # what O.softmax computes (checked above)
+    np.testing.assert_allclose(O.softmax(x.detach().numpy(), axis), y.detach().numpy(), rtol=1e-12, atol=1e-14)
+    y.backward(dy)
+    got = O.softmax_backward_rows(y.detach().numpy(), dy.numpy(), axis)
+    np.testing.assert_allclose(got, x.grad.numpy(), rtol=1e-10, atol=1e-12)
+    single = O.softmax_backward(y.detach().numpy(), dy.numpy(), ax)
+    if int(np.prod(shape[ax + 1:], dtype=np.int64)) == 1:
+        np.testing.assert_allclose(single, got, rtol=1e-12, atol=1e-14)   # the reference's single-axis sum is the same
+    else:
+        assert not np.allclose(single, x.grad.numpy(), rtol=1e-3, atol=1e-9)   # ... and is not the derivative otherwise
+
+
 @pytest.mark.parametrize("shape,kernel,stride", [((2, 3, 8, 8), (2, 2), (2, 2)), ((1, 2, 9, 7), (3, 3), (2, 2)),
                                                  ((2, 1, 7, 10), (3, 2), (1, 3)), ((1, 1, 5, 5), (5, 5), (1, 1))])
 def test_maxpool_matches_torch_and_autograd(shape, kernel, stride):

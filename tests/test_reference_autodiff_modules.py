@@ -13,7 +13,6 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
-from tests.util import first_run_on_hardware
 
 
 class Simple(nn.Module):
@@ -166,7 +165,6 @@ def test_reference_autodiff_module_lowers_correctly(name):
     np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", [c[0] for c in CASES])
 def test_reference_autodiff_module_on_gpu(name):
@@ -229,7 +227,6 @@ def test_reference_conv2d_model_lowers_correctly():
     np.testing.assert_allclose(arrays["gradient_" + names[0]], xt.grad.numpy(), rtol=1e-5, atol=1e-6)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 def test_reference_conv2d_model_on_gpu():
     from daceml_amd.torch import DaceModule

@@ -8,7 +8,6 @@ import numpy as np
 import pytest
 import torch
 
-from tests.util import first_run_on_hardware
 
 FIXTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_slice.onnx")
 
@@ -36,7 +35,6 @@ def test_reference_slice_model_on_the_emulator():
     assert arrays["__return"][0] == 3.0                          # starts [0], ends [1], axes [0]
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 def test_reference_slice_model_on_gpu():
     out = _model()(data=torch.ones(2).cuda())

@@ -11,7 +11,7 @@ import pytest
 import torch
 from torch import nn, optim
 
-from tests.util import assert_close, first_run_on_hardware
+from tests.util import assert_close
 
 
 def _mnist():
@@ -87,7 +87,6 @@ def test_training_step_lowers_correctly(name):
                      atol=1e-5 * max(1.0, float(np.abs(w).max())))
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["mnist", "bert"])
 def test_training_step_on_gpu(name):

@@ -1,19 +1,16 @@
-"""The interleaved-K-loop configurations of the pipelined fp16 GEMM kernel (4: 256 x 256 tile, 5: 128 x 128 with a four-stage ring, 6:
-256 x 128, 7: 128 x 128 with two stages, 9: 128 x 64 - and 8, the plain loop on that new tile; reachable only through ``dmlhip_debug_force_gemm_config``) on the cases the chosen configurations are
-tested with, plus products with enough K steps to run the ring's steady state, its tail and every operand layout.
-
-SKIPPED: these configurations were written without access to a GPU and have not run on hardware; the library never
-selects them. The skip goes once they have passed here (DACEML_RUN_UNVALIDATED=1 runs them)."""
+"""The interleaved-K-loop configurations of the pipelined fp16 GEMM kernel (4: 256 x 256 tile, 5: 128 x 128 with a
+four-stage ring, 6: 256 x 128, 7: 128 x 128 with two stages, 9: 128 x 64 - and 8, the plain loop on that tile), each
+pinned through ``dmlhip_debug_force_gemm_config`` (the library chooses 4, 5 and 9 by itself for products with at least
+eight K steps) on the cases the other configurations are tested with, plus products with enough K steps to run the ring's steady state, its tail and every operand layout."""
 import numpy as np
 import pytest
 import torch
 
 from oracle import ops as O
 from tests import test_gpu_kernels as TK
-from tests.util import assert_close, dev, host, not_yet_on_hardware
+from tests.util import assert_close, dev, host
 
-pytestmark = [pytest.mark.gpu,
-              not_yet_on_hardware("interleaved GEMM configurations 4-7 have not been run on hardware yet")]
+pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("cfg", [4, 5, 6, 7, 8, 9])

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from oracle import ops as O
-from tests.util import assert_close, dev, first_run_on_hardware, host, not_yet_on_hardware, rng
+from tests.util import assert_close, dev, host, not_yet_on_hardware, rng
 
 # n, c, l, m, k, stride, pad, dilation, group, bias
 CASES = [(2, 3, 40, 8, 3, 1, 1, 1, 1, True), (3, 4, 33, 6, 5, 2, 2, 1, 2, False), (1, 8, 100, 8, 3, 1, 2, 2, 8, True),
@@ -126,7 +126,6 @@ def test_shapes_that_are_not_a_1d_or_2d_convolution_are_refused():
         g.state.library_nodes()[0].expand(g.sdfg, g.state)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("case", CASES)

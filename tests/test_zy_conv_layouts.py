@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from oracle import ops as O
-from tests.util import assert_close, dev, first_run_on_hardware, host, rng
+from tests.util import assert_close, dev, host, rng
 
 # n, c, h, w, m, k, stride, pad, group, x channels-last, y channels-last
 CASES = [(2, 8, 12, 14, 16, 3, 1, 1, 1, True, True), (2, 8, 12, 14, 16, 3, 2, 1, 1, True, False),
@@ -86,7 +86,6 @@ def test_layout_detection_follows_the_reference():
         g.state.library_nodes()[0].expand(g.sdfg, g.state)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("case", CASES)

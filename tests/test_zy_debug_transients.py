@@ -4,7 +4,6 @@ import numpy as np
 import pytest
 import torch
 
-from tests.util import first_run_on_hardware
 
 
 def _module():
@@ -45,7 +44,6 @@ def test_exposed_tensors_keep_the_fusion_passes_away():
     assert len(exposed.sdfg.states()[0].library_nodes()) == 5 and len(exposed.outputs) == 5
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 def test_debug_transients_on_gpu():
     module = _module()

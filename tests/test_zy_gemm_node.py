@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import ops as O
-from tests.util import assert_close, dev, first_run_on_hardware, host, rng
+from tests.util import assert_close, dev, host, rng
 
 M, N, K = 24, 40, 64
 
@@ -137,7 +137,6 @@ def test_gemm_reverse_node_lowers_correctly(dtype, ta, tb, alpha, beta, ckind):
         assert_close(arrays["gradient_c"], wc, dtype, "dC", **(tol if dtype == torch.float32 else dict(rtol=2e-2, atol=5e-2)))
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("ta,tb,alpha,beta,ckind", BACKWARD_CASES[::3])
@@ -158,7 +157,6 @@ def test_gemm_backward_on_gpu(dtype, ta, tb, alpha, beta, ckind):
         assert_close(host(outs["c"]), wc, dtype, "dC", **(tol if dtype == torch.float32 else dict(rtol=2e-2, atol=5e-2)))
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("ta,tb,alpha,beta,ckind", CASES)
@@ -211,7 +209,6 @@ def test_exported_gemm_nodes_keep_their_attributes_and_lower_correctly():
     assert_close(arrays[model.outputs[0]], want, torch.float32, "addmm through Gemm nodes (emulated)", rtol=1e-5, atol=2e-6)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 def test_gemm_node_through_the_module_wrapper():
     from daceml_amd.torch import DaceModule

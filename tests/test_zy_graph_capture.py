@@ -1,14 +1,14 @@
 """``CompiledSDFG.capture``: the launches of a program recorded into a HIP graph and replayed.
 
-SKIPPED until it has run on hardware once (DACEML_RUN_UNVALIDATED=1 runs it). Each replay is followed by eager work and a synchronisation and compared
+Each replay is followed by eager work and a synchronisation and compared
 with the eager result on fresh inputs written into the same buffers (a graph holds pointers, not values)."""
 import numpy as np
 import pytest
 import torch
 
-from tests.util import dev, not_yet_on_hardware, rng
+from tests.util import dev, rng
 
-pytestmark = [pytest.mark.gpu, not_yet_on_hardware("graph capture of the launches has not been run on hardware yet")]
+pytestmark = pytest.mark.gpu
 
 
 def _program(dtype, attention):

@@ -1,7 +1,7 @@
 """Node forms outside the measured configurations: Reduce* over axes that are not adjacent
 (pure_implementations.py:101-103,294-306 take any ``axes``) and the Softmax reverse node for an axis other than the
-last (DefaultSoftmaxBackward, daceml/autodiff/implementations/onnx_ops.py:237-275, reduces over the single axis
-``axis``). Both are compositions of kernels that exist: several reduction passes, and the reference's own Mul /
+last (DefaultSoftmaxBackward, daceml/autodiff/implementations/onnx_ops.py:237-275; summed over every axis the forward
+made one row of, see oracle.ops.softmax_backward_rows). Both are compositions of kernels that exist: several reduction passes, and the reference's own Mul /
 ReduceSum / Mul / Sub.
 
 As in test_zy_gemm_node.py each case runs twice: on a GPU through the kernels, and without a GPU with the emitted
@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from oracle import ops as O
-from tests.util import assert_close, dev, first_run_on_hardware, host, rng
+from tests.util import assert_close, dev, host, rng
 
 REDUCE_CASES = [((4, 6, 8), [0, 2]), ((3, 5, 7, 9), [0, 2]), ((3, 5, 7, 9), [1, 3]), ((2, 3, 4, 5, 6), [0, 2, 4]),
                 ((6, 1, 5, 4), [0, 3]), ((4, 6, 8), [0, 1])]
@@ -60,7 +60,6 @@ def test_reduce_over_separate_axes_lowers_to_passes(dtype, name, shape, axes, ke
     assert np.array_equal(arrays["x"], x)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("name", ["sum", "mean", "max", "min"])
@@ -115,12 +114,11 @@ def test_softmax_reverse_node_for_any_axis_lowers_correctly(dtype, shape, axis):
     expand_onnx_nodes(g.sdfg)
     arrays = {"y": y.copy(), "gradient_y": dy.copy()}
     run_state(g.sdfg, bst, arrays)
-    want = O.softmax_backward(y.astype(np.float64), dy.astype(np.float64), axis % len(shape))
+    want = O.softmax_backward_rows(y.astype(np.float64), dy.astype(np.float64), axis % len(shape))
     tol = dict(rtol=2e-2, atol=1e-2) if dtype == torch.float16 else dict(rtol=1e-5, atol=1e-6)
     assert_close(arrays["gradient_x"], want, dtype, "emulated softmax backward %s axis %d" % (shape, axis), **tol)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("shape,axis", SOFTMAX_CASES)
@@ -135,7 +133,7 @@ def test_softmax_backward_for_any_axis_on_gpu(dtype, shape, axis):
     tol = dict(rtol=2e-2, atol=1e-2) if dtype == torch.float16 else dict(rtol=1e-5, atol=1e-6)
     assert_close(host(y), y64, dtype, "softmax %s axis %d" % (shape, axis), **tol)
     # the reverse node reads the forward output as the kernel rounded it
-    want = O.softmax_backward(host(y).astype(np.float64), dy.astype(np.float64), axis % len(shape))
+    want = O.softmax_backward_rows(host(y).astype(np.float64), dy.astype(np.float64), axis % len(shape))
     assert_close(host(dx), want, dtype, "softmax backward %s axis %d" % (shape, axis), **tol)
 
 
@@ -220,7 +218,6 @@ def test_exported_log_softmax_head():
                  rtol=1e-5, atol=2e-6)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("shape,axis", LOG_SOFTMAX_CASES)

@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.util import assert_close, first_run_on_hardware, not_yet_on_hardware
+from tests.util import assert_close, not_yet_on_hardware
 
 
 def _reference(pt, tensors, grads=None):
@@ -123,7 +123,6 @@ def _gpu_case():
     return torch.nn.MultiheadAttention(n, heads, bias=False), (q, k, v)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 def test_multihead_attention_forward_on_gpu():
     from daceml_amd.torch import DaceModule

@@ -7,7 +7,6 @@ import pytest
 import torch
 from torch import nn
 
-from tests.util import first_run_on_hardware
 
 
 class TwoOutputs(nn.Module):
@@ -48,7 +47,6 @@ def test_a_skipped_input_has_no_gradient_in_the_backward_graph():
     np.testing.assert_allclose(arrays["gradient_" + names[1]], net.fc1.grad.numpy(), rtol=1e-5, atol=1e-6)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 def test_skip_input_grads_on_gpu():
     from daceml_amd.torch import DaceModule
@@ -65,7 +63,6 @@ def test_skip_input_grads_on_gpu():
     torch.testing.assert_close(wrapped.model.fc1.grad, pt_module.fc1.grad)
 
 
-@first_run_on_hardware("written without access to a GPU: first run on hardware")
 @pytest.mark.gpu
 def test_backward_called_per_output_on_gpu():
     """test_multi_output_ad.py:8-48: each output's ``backward`` in turn; the input gradient accumulates."""

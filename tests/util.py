@@ -49,11 +49,3 @@ def not_yet_on_hardware(reason):
     import os
     import pytest
     return pytest.mark.skipif(os.environ.get("DACEML_RUN_UNVALIDATED") != "1", reason=reason)
-
-
-def first_run_on_hardware(reason):
-    """Marker for GPU tests that were written without access to a GPU and drive kernels that do run on hardware, in
-    combinations no earlier test covers: they run, but a failure is reported as expected (xfail, not strict) so that
-    it does not stop a run with -x before the tests behind it; a pass shows as XPASS. Goes once the test has passed."""
-    import pytest
-    return pytest.mark.xfail(strict=False, reason=reason)
