@@ -367,7 +367,8 @@ class HipFusedAttentionBackward(BackwardImplementation):
                  q_perm=forward_node.q_perm, k_perm=forward_node.k_perm, v_perm=forward_node.v_perm,
                  o_perm=forward_node.o_perm)
         if "Mask" in required_gradients:
-            raise AutoDiffException("%s: no gradient is produced for the attention mask" % forward_node.label)
+            raise AutoDiffException("%s: no gradient is produced for the attention mask (list the mask in the wrapper's "
+                                    "inputs_to_skip, or keep the attention block unfused)" % forward_node.label)
         has_mask = any(e.dst_conn == "Mask" for e in context.forward_state.in_edges(forward_node))
         for conn in ("Q", "K", "V") + (("Mask", ) if has_mask else ()):
             connect_input_from_forward(forward_node, g, context, conn)

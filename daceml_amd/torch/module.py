@@ -163,6 +163,23 @@ class DaceModule(nn.Module):
             hook(self)
         return self.dace_model
 
+    def _inputs_that_need_gradients(self, model: ONNXModel) -> List[str]:
+        """Every tensor input that is not skipped and every parameter that requires a gradient (module.py:333-346 of
+        the reference), as far as the graph reads them - directly or through views (the slices of a packed weight)."""
+        sdfg, state, params = model.sdfg, model.state, self._exported_parameters
+        tensor_inputs = [n for n in model.inputs if n not in params]
+        param_inputs = [n for n in model.inputs if n in params]
+        buffers = {n for n, _ in self.model.named_buffers()}
+        required = [n for n in tensor_inputs if n not in self.inputs_to_skip and
+                    sdfg.arrays[clean_onnx_name(n)].dtype.is_floating_point]
+        required += [n for n in param_inputs if n not in buffers and params[n].requires_grad]
+        used = {e.data.data for e in state.edges()}
+        for n in list(used):
+            while sdfg.arrays[n].view_of is not None:
+                n = sdfg.arrays[n].view_of
+                used.add(n)
+        return [n for n in required if clean_onnx_name(n) in used]
+
     def _initialize_sdfg(self, dummy_inputs: Sequence[torch.Tensor]):
         device = next((t.device for t in dummy_inputs if t.is_cuda), None)
         if device is None:
@@ -187,12 +204,7 @@ class DaceModule(nn.Module):
             fusion.lower_matmul(sdfg)
             # gradients for every input that is not a buffer or skipped, and every parameter that requires one
             # (module.py:333-346)
-            buffers = {n for n, _ in self.model.named_buffers()}
-            required = [n for n in tensor_inputs if n not in self.inputs_to_skip and
-                        sdfg.arrays[clean_onnx_name(n)].dtype.is_floating_point]
-            required += [n for n in param_inputs if n not in buffers and params[n].requires_grad]
-            used = {e.data.data for e in state.edges()}
-            required = [n for n in required if clean_onnx_name(n) in used]
+            required = self._inputs_that_need_gradients(model)
             # parameter gradients are accumulated and stored in fp32 also for fp16 parameters (the reductions over
             # the batch run in fp32 anyway); autograd receives them cast to the parameter's type
             master = {clean_onnx_name(n): torch.float32 for n in required

@@ -1,19 +1,16 @@
 """The rolling-window form of the fused pointwise + depthwise convolution (reachable only through
 ``dmlhip_debug_fused_rolling``) on the problems the strip kernel is tested with, and on the benchmarked MBConv shape,
 where it must agree with the strip kernel bit for bit (both add in the same order).
-
-SKIPPED: the kernel was written without access to a GPU and has not run on hardware (its source runs lane by lane
-on the CPU in tests/test_kernel_emulation.py); the library never selects it. The skip goes once it has passed here (DACEML_RUN_UNVALIDATED=1 runs it)."""
+"""
 import numpy as np
 import pytest
 import torch
 
 from oracle import ops as O
 from tests import test_gpu_kernels as TK
-from tests.util import assert_close, dev, host, not_yet_on_hardware
+from tests.util import assert_close, dev, host
 
-pytestmark = [pytest.mark.gpu,
-              not_yet_on_hardware("the rolling-window expand + depthwise kernel has not been run on hardware yet")]
+pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("waves", [8, 16])

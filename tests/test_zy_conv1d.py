@@ -3,14 +3,14 @@ lowered to the 2-D kernels as [N, C, 1, L] with a 1 x k filter. Oracle: ``oracle
 itself checked here against ``torch.nn.functional.conv1d``.
 
 The host-side tests interpret the emitted calls with tests/abi_emulator.py; the GPU tests run small problems (direct
-kernel and contraction kernels) and one long sequence that is large enough for the implicit-GEMM kernel - SKIPPED for
-now, because that kernel has not been run with a single output row (DACEML_RUN_UNVALIDATED=1 runs it)."""
+kernel and contraction kernels) and one long sequence that is large enough for the implicit-GEMM kernel, which then
+runs with a single output row."""
 import numpy as np
 import pytest
 import torch
 
 from oracle import ops as O
-from tests.util import assert_close, dev, host, not_yet_on_hardware, rng
+from tests.util import assert_close, dev, host, rng
 
 # n, c, l, m, k, stride, pad, dilation, group, bias
 CASES = [(2, 3, 40, 8, 3, 1, 1, 1, 1, True), (3, 4, 33, 6, 5, 2, 2, 1, 2, False), (1, 8, 100, 8, 3, 1, 2, 2, 8, True),
@@ -146,7 +146,6 @@ def test_conv1d_on_gpu(case, dtype):
     assert_close(host(y), want, dtype, "conv1d %s" % (case, ), **tol)
 
 
-@not_yet_on_hardware("the implicit-GEMM convolution kernel has not been run with a single output row yet")
 @pytest.mark.gpu
 def test_long_conv1d_on_gpu():
     from daceml_amd.runtime import CompiledSDFG

@@ -1,8 +1,8 @@
 """MaxPool (PureMaxPool2D, img_op_implementations.py:28-161; DefaultMaxPoolBackward, onnx_ops.py:284-335) and the network
 of the reference's tests/torch/test_lenet.py, which needs it: Conv, Relu, MaxPool twice, three Linear layers, LogSoftmax.
 
-Host side: lowering and the emitted calls interpreted by tests/abi_emulator.py against the oracle / PyTorch. The pool
-kernels have not run on hardware: their GPU tests are SKIPPED until they have (DACEML_RUN_UNVALIDATED=1 runs them)."""
+Host side: lowering and the emitted calls interpreted by tests/abi_emulator.py against the oracle / PyTorch; the GPU
+tests run the pool kernels and the network on them."""
 import numpy as np
 import pytest
 import torch
@@ -10,7 +10,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from oracle import ops as O
-from tests.util import assert_close, dev, host, not_yet_on_hardware
+from tests.util import assert_close, dev, host
 
 CASES = [((2, 3, 8, 8), [2, 2], [2, 2]), ((1, 2, 9, 7), [3, 3], [2, 2]), ((2, 1, 7, 10), [3, 2], [1, 3]),
          ((1, 4, 13, 13), [2, 2], [2, 2])]
@@ -124,7 +124,6 @@ def test_lenet_forward_and_training_step_lower_correctly():
                      atol=1e-6 * max(1.0, float(np.abs(w).max()) * 10))
 
 
-@not_yet_on_hardware("the MaxPool kernels have not been run on hardware yet")
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("shape,kernel,strides", CASES + [((64, 16, 112, 112), [2, 2], [2, 2])])
@@ -141,7 +140,6 @@ def test_maxpool_on_gpu(dtype, shape, kernel, strides):
                                **(dict(rtol=2e-2, atol=1e-2) if dtype == torch.float16 else dict(rtol=1e-6, atol=1e-6)))
 
 
-@not_yet_on_hardware("the MaxPool kernels have not been run on hardware yet")
 @pytest.mark.gpu
 def test_lenet_on_gpu():
     from daceml_amd.torch import DaceModule

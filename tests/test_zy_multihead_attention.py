@@ -4,16 +4,15 @@ q / k / v projection weight, both outputs: the attention result and the head-ave
 The exporter slices the packed weight three times; the importer turns a Slice with known bounds into a view of its
 input (no node, no copy), and the backward pass pads the gradient of each slice back into a contribution shaped like
 the packed weight. Host side: the graph is lowered and its calls are interpreted on the CPU by tests/abi_emulator.py,
-against PyTorch in double precision. The GPU test of the forward pass composes kernels that run on hardware (with
-operand pointers offset into the packed weight, which is new) and is a first run; the training test also needs the
-constant-pad kernel, which has not run yet, and is SKIPPED until then (DACEML_RUN_UNVALIDATED=1 runs it)."""
+against PyTorch in double precision. The GPU tests run the forward pass (operand pointers offset into the packed
+weight) and a training step (which also runs the constant-pad kernel) at the shapes of the reference's test."""
 from collections import Counter
 
 import numpy as np
 import pytest
 import torch
 
-from tests.util import assert_close, not_yet_on_hardware
+from tests.util import assert_close
 
 
 def _reference(pt, tensors, grads=None):
@@ -87,6 +86,16 @@ def test_multihead_attention_training_step_lowers_correctly():
                      atol=2e-6 * max(1.0, float(np.abs(w).max())))
 
 
+def test_the_wrapper_asks_for_the_gradient_of_a_weight_that_is_read_through_views_only():
+    from daceml_amd.torch import DaceModule
+    torch.manual_seed(5)
+    n, heads, s, b = 128, 2, 24, 2
+    q, k, v = (torch.randn(s, b, n) for _ in range(3))
+    dm = DaceModule(torch.nn.MultiheadAttention(n, heads, bias=False), backward=True)
+    need = dm._inputs_that_need_gradients(dm._import((q, k, v)))
+    assert {"in_proj_weight", "out_proj.weight"} <= set(need) and len(need) == 5, need
+
+
 def test_slices_of_run_time_data_become_views():
     """Bounds as the ONNX specification clamps them, negative indices, several axes, steps."""
     from daceml_amd.torch import DaceModule
@@ -133,7 +142,6 @@ def test_multihead_attention_forward_on_gpu():
         assert_close(o.cpu().numpy(), w, torch.float32, "output %d" % i, rtol=1e-4, atol=2e-5)
 
 
-@not_yet_on_hardware("the constant-pad kernel in the backward pass has not been run on hardware yet")
 @pytest.mark.gpu
 def test_multihead_attention_training_on_gpu():
     from daceml_amd.torch import DaceModule

@@ -3,12 +3,12 @@
 node, whose kernels have their own GPU tests. A Pad that does not fold (the padding differs between the two sides of
 an axis, a fill value, other axes) runs on a kernel of its own; its reverse is a Pad with negated amounts. The calls
 are interpreted on the CPU by tests/abi_emulator.py and compared with NumPy / PyTorch in double precision; the pad
-kernel's GPU test is SKIPPED until it has run on hardware (DACEML_RUN_UNVALIDATED=1 runs it)."""
+kernel has a GPU test of its own."""
 import numpy as np
 import pytest
 import torch
 
-from tests.util import assert_close, dev, host, not_yet_on_hardware
+from tests.util import assert_close, dev, host
 
 
 def _import(net, x):
@@ -201,7 +201,6 @@ def test_what_the_rewrite_refuses():
 
 
 @pytest.mark.gpu
-@not_yet_on_hardware("the constant-pad kernel has not been run on hardware yet")
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("shape,pads,value", [((2, 3, 5, 6), [0, 0, 1, 2, 0, 0, 0, 3], 0.0), ((4, 7), [1, 0, 2, 2], -2.5),
                                               ((3, 8, 5), [0, -2, 1, 0, -1, 0], 0.0),

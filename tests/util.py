@@ -40,12 +40,3 @@ def assert_close(got, want, dtype, what="", rtol=None, atol=None):
         i = np.unravel_index(np.argmax(err - bound), err.shape)
         raise AssertionError("%s: %d / %d elements out of tolerance (rtol=%g atol=%g); worst at %s: got %r want %r"
                              % (what, bad.sum(), bad.size, rtol, atol, i, got[i], want[i]))
-
-
-def not_yet_on_hardware(reason):
-    """Marker for GPU tests of code that was written without access to a GPU: skipped in an ordinary run (a kernel
-    that has never run must not be able to take the other tests down with it), run when DACEML_RUN_UNVALIDATED=1 -
-    the first thing to do with them on a machine that has a GPU, one file at a time."""
-    import os
-    import pytest
-    return pytest.mark.skipif(os.environ.get("DACEML_RUN_UNVALIDATED") != "1", reason=reason)
