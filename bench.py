@@ -276,44 +276,76 @@ def secondary_workload(name, device, steps, warmup, verbose, graph=False, fused_
                        **({"fused_rolling": fused_rolling} if fused_rolling else {})},
             "roofline": roof, "launches": launches}
     if name == "nodes":
-        line["layernorm_cold"] = layernorm_cold(device, rng, max(2, min(steps, 6)))
+        line["stream_timing"] = stream_timing(device, max(3, min(steps, 10)))
     print(json.dumps(line))
 
 
-def layernorm_cold(device, rng, rounds, buffers=40):
-    """The LayerNorm of the `nodes` workload with input and output rotating over `buffers` distinct pairs: 40 pairs
-    of [8,512,1024] fp16 are 671 MB, so by the time a pair comes round again it has left the 256 MB last-level cache
-    and the launch reads from HBM. (The `launches` entry of the same node re-uses one pair, which stays in cache.)"""
+def stream_timing(device, rounds):
+    """The two `nodes` kernels and a plain copy of the same bytes (the library's identity kernel: 128-bit loads and
+    stores, the bandwidth a one-pass kernel of that size can be held against), each timed as a stream of 40 launches
+    replayed from a HIP graph between one pair of events - no host call between the launches, so a kernel of a few
+    microseconds is not timed waiting for its own submission, as it is with an event pair around a single launch. The
+    figure per launch includes the gap to the next launch on the stream. `cached`: the launches rotate over few tensor
+    pairs that stay in the 256 MB last-level cache; `cold`: over enough pairs (LayerNorm: 40 x 16.8 MB = 671 MB) that
+    a pair has left it by the time it comes round again and the launch reads from HBM."""
     import numpy as np
     import torch
     from daceml_amd import graphs
     from daceml_amd.runtime import CompiledSDFG
     from daceml_amd.transformation import fusion
-    g = graphs.GraphBuilder("layernorm_cold", torch.float16)
-    xin = g.input("x", (8, 512, 1024))
-    g.input("gamma", (1024, ))
-    g.input("beta", (1024, ))
-    g.output(g.layer_norm(xin, "gamma", "beta", 1e-5, "ln"), "y")
-    fusion.auto_optimize(g.sdfg)
-    prog = CompiledSDFG(g.sdfg, device=device)
+    launches = 40
+    rng = np.random.default_rng(99)
     gamma = torch.from_numpy(rng.uniform(0.5, 1.5, 1024).astype(np.float16)).to(device)
     beta = torch.from_numpy((rng.standard_normal(1024) * 0.1).astype(np.float16)).to(device)
-    xs = [torch.randn((8, 512, 1024), dtype=torch.float16, device=device) for _ in range(buffers)]
-    ys = [torch.empty((8, 512, 1024), dtype=torch.float16, device=device) for _ in range(buffers)]
-    prog(x=xs[0], gamma=gamma, beta=beta, y=ys[0])
-    times = []
-    for r in range(rounds + 1):
-        for i in range(buffers):
-            prog.bind({"x": xs[i], "y": ys[i]})
-            t = sum(ms for _, ms in prog.launch_timed())
-            if r > 0:   # the first round is the warm-up of everything but the data
-                times.append(t)
-    us = float(np.mean(times)) * 1e3
-    nbytes = sum(l.bytes_moved or 0 for l in prog.launches)
-    gbs = nbytes / (us * 1e-6) / 1e9
-    return {"us": round(us, 2), "min_us": round(float(np.min(times)) * 1e3, 2), "GB/s": round(gbs, 1),
-            "frac": round(gbs / PEAK_HBM_GBS, 4), "bytes": int(nbytes), "buffers": buffers, "launches": len(prog.launches),
-            "samples": len(times)}
+
+    def run(kind, shape, pairs):
+        g = graphs.GraphBuilder("stream_" + kind, torch.float16)
+        if kind == "layernorm":
+            g.input("gamma", (1024, ))
+            g.input("beta", (1024, ))
+        for i in range(launches):
+            xin = g.input("x%d" % i, shape)
+            if kind == "layernorm":
+                out = g.layer_norm(xin, "gamma", "beta", 1e-5, "ln%d" % i)
+            elif kind == "softmax":
+                out = g.node("Softmax", {"input": xin}, {"output": shape}, label="sm%d" % i, axis=-1)["output"]
+            else:
+                out = g.node("Identity", {"input": xin}, {"output": shape}, label="copy%d" % i)["output"]
+            g.output(out, "y%d" % i)
+        fusion.auto_optimize(g.sdfg)
+        prog = CompiledSDFG(g.sdfg, device=device)
+        assert len(prog.launches) == launches, [l.symbol for l in prog.launches]
+        xs = [torch.randn(shape, dtype=torch.float16, device=device) for _ in range(pairs)]
+        ys = [torch.empty(shape, dtype=torch.float16, device=device) for _ in range(pairs)]
+        args = {"x%d" % i: xs[i % pairs] for i in range(launches)}
+        args.update({"y%d" % i: ys[i % pairs] for i in range(launches)})
+        if kind == "layernorm":
+            args.update(gamma=gamma, beta=beta)
+        prog(**args)
+        cap = prog.capture()
+        cap.replay()
+        times = []
+        for _ in range(rounds):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            cap.replay()
+            e.record()
+            torch.cuda.synchronize(device)
+            times.append(s.elapsed_time(e) * 1e3 / launches)
+        us = float(np.median(times))
+        nbytes = 4 * int(np.prod(shape))
+        gbs = nbytes / (us * 1e-6) / 1e9
+        del cap, prog, xs, ys
+        torch.cuda.empty_cache()
+        return {"us": round(us, 2), "min_us": round(float(np.min(times)), 2), "bytes": nbytes, "GB/s": round(gbs, 1),
+                "frac": round(gbs / PEAK_HBM_GBS, 4), "pairs": pairs}
+
+    ln, sm = (8, 512, 1024), (8, 16, 512, 512)
+    return {"launches_per_replay": launches, "replays": rounds,
+            "layernorm": {"cached": run("layernorm", ln, 4), "cold": run("layernorm", ln, 40)},
+            "copy_of_layernorm_bytes": {"cached": run("copy", ln, 4), "cold": run("copy", ln, 40)},
+            "softmax": {"one_pair": run("softmax", sm, 1), "cold": run("softmax", sm, 5)},
+            "copy_of_softmax_bytes": {"one_pair": run("copy", sm, 1), "cold": run("copy", sm, 5)}}
 
 
 def module_workload(device, steps, warmup):

@@ -214,13 +214,19 @@ inline size_t rolling_lds_bytes(int r, int stride, int w, int cin) {
     return ((size_t)kCB * ring * (w + 2) + (size_t)kCB * (cin + 1) + (size_t)kCB * 10) * sizeof(float);
 }
 
-// Geometry of a launch: `rows` output rows per batch (0: the most that fit), workgroups spread over `cus` compute
-// units. Returns false when not even one row per batch fits LDS.
+// Geometry of a launch: at most `rows` output rows per batch (-1: the most that fit, 0: the library's choice), workgroups
+// spread over `cus` compute units. Returns false when not even one row per batch fits LDS.
 inline bool fill_rolling(int n, int cin, int cmid, int h, int w, int stride, int rows, int cus, RollArgs& a) {
     a.n = n; a.cin = cin; a.cmid = cmid; a.h = h; a.w = w; a.stride = stride;
     a.oh = (h + 2 - 3) / stride + 1;
     a.ow = (w + 2 - 3) / stride + 1;
     int r = 0;
+    // the library's own choice (rows == 0): the most rows whose ring leaves room for a second workgroup on the compute
+    // unit (measured on the MBConv block [96,32,112,112] -> 192 channels, stride 2: 352 us with one row per batch and two
+    // workgroups of 8 wavefronts, 402 us with two rows and one workgroup, 508 us for the strips)
+    if (rows == 0)
+        for (int cand : {8, 4, 2, 1})
+            if (!r && rolling_lds_bytes(cand, stride, w, cin) <= 78 * 1024) r = cand;
     for (int cand : {8, 4, 2, 1})
         if (!r && (rows <= 0 || cand <= rows) && rolling_lds_bytes(cand, stride, w, cin) <= 156 * 1024) r = cand;
     if (!r) return false;
@@ -439,8 +445,9 @@ size_t fused_lds_bytes(int toh, int stride, int w, int cin) {
 }
 
 thread_local int g_fused_toh = 0;   // diagnostic switch (per calling thread): pin the strip height
-thread_local int g_rolling_rows = 0;    // diagnostic switch (per calling thread): 0 = strips, -1 = rolling window with the
-thread_local int g_rolling_waves = 8;   // most rows per batch that fit, > 0 = at most that many; wavefronts per workgroup
+thread_local int g_rolling_rows = 0;    // diagnostic switch (per calling thread): 0 = the library's choice, -1 = rolling window
+thread_local int g_rolling_waves = 8;   // with the most rows per batch that fit, > 0 = at most that many, -2 = strips;
+                                        // wavefronts per workgroup
 
 int compute_units() {
     static int cached[64] = {};
@@ -527,7 +534,8 @@ int dmlhip_conv2d_expand_depthwise_f32(const dmlhip_conv2d_desc* pw, const dmlhi
     const int stride = (int)dw->stride_h;
     hipStream_t st = (hipStream_t)stream;
     RollArgs ra;
-    if (g_rolling_rows != 0 && fill_rolling((int)pw->n, (int)pw->c, (int)pw->m, (int)pw->h, (int)pw->w, stride,
+    // a pinned strip height asks for the strip kernel
+    if (g_rolling_rows != -2 && g_fused_toh <= 0 && fill_rolling((int)pw->n, (int)pw->c, (int)pw->m, (int)pw->h, (int)pw->w, stride,
                                             g_rolling_rows, compute_units(), ra)) {
 #define DML_ROLLING_CASE(A1, A2)                                                                                     \
     if (pw->act == A1 && dw->act == A2)                                                                              \

@@ -369,6 +369,7 @@ int operand_mode(const void* p, int64_t rows, int64_t k, int64_t s_row, int64_t 
 // does not change what other threads launch.
 thread_local int g_force_cfg = -1;  // pin the tile configuration
 thread_local int g_direct_lds = 1;  // 0 forces the register-staged loaders
+thread_local unsigned long long* g_trace = nullptr;  // per-workgroup clock readings of the pipelined kernel
 
 }  // namespace
 }  // namespace dml
@@ -379,6 +380,7 @@ extern "C" {
 
 void dmlhip_debug_force_gemm_config(int cfg) { g_force_cfg = cfg; }
 void dmlhip_debug_gemm_direct_lds(int on) { g_direct_lds = on; }
+void dmlhip_debug_gemm_trace(void* buffer) { g_trace = (unsigned long long*)buffer; }
 static std::atomic<long long> g_grouped_single_launches{0};
 // Number of grouped calls that went out as ONE launch (tests check that grouping really happens).
 long long dmlhip_debug_grouped_single_launches() { return g_grouped_single_launches.load(); }
@@ -423,6 +425,7 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
     GemmArgs g;
     g.groups = 0;
     g.ksum = 0;
+    g.trace = g_trace;
     g.asum = !grp && asum ? asum[0] : nullptr;
     g.asum_f32 = asum_f32;
     for (int i = 0; i < DMLHIP_GROUP_MAX; ++i) g.gasum[i] = grp && asum && i < grp->count ? asum[i] : nullptr;

@@ -33,6 +33,9 @@ struct GemmArgs {
     void* asum;
     void* gasum[DMLHIP_GROUP_MAX];
     int asum_f32;
+    // diagnostic (dmlhip_debug_gemm_trace): when set, every workgroup stores four readings of the 100 MHz wall clock -
+    // start, first tile in LDS, end of the K loop, end of the epilogue - at trace[4 * workgroup]
+    unsigned long long* trace;
     const _Float16* ga[DMLHIP_GROUP_MAX];
     const _Float16* gb[DMLHIP_GROUP_MAX];
     void* gc[DMLHIP_GROUP_MAX];

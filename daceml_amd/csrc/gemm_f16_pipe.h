@@ -158,6 +158,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
 
     // All of this is wave-uniform integer arithmetic in 32 bits (the host checks total_blocks < 2^31): 64-bit
     // divisions are long software sequences, and this prologue runs before the first load can be issued.
+    if (g.trace && threadIdx.x == 0) g.trace[4 * (size_t)blockIdx.x] = wall_clock64();
     uint32_t bid = blockIdx.x;
     {
         const uint32_t total = (uint32_t)g.total_blocks;
@@ -265,6 +266,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     if (nk >= NSTAGE - 1) wait_vm_lgkm0<(NSTAGE - 2) * LPT>();
     else wait_vm_lgkm0<0>();
     __builtin_amdgcn_s_barrier();
+    if (g.trace && threadIdx.x == 0) g.trace[4 * (size_t)blockIdx.x + 1] = wall_clock64();
 
     half8 af[2][TM], bf[2][TN];
     if (nk > 0) {
@@ -452,6 +454,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
     }
     wait_vm_lgkm0<0>();
     __syncthreads();
+    if (g.trace && threadIdx.x == 0) g.trace[4 * (size_t)blockIdx.x + 2] = wall_clock64();
 
     // ---- epilogue (see store_strip): 32 x WN strips through this wavefront's LDS region
     constexpr int PITCH = WN + 4;
@@ -467,6 +470,10 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
         else store_strip<_Float16, WN, EPI>(g, c_ptr, pre_ptr, res_ptr, bias_ptr, bias_n, strip, mb, nb, coff, lane);
         __builtin_amdgcn_wave_barrier();
     });
+    if (g.trace && threadIdx.x == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's stores have been accepted
+        g.trace[4 * (size_t)blockIdx.x + 3] = wall_clock64();
+    }
     if constexpr (ASUM) {
         // lanes l and l + 32 hold the two k halves of row l; wavefront wn = 1 hands its share over through LDS
         __syncthreads();   // the epilogue strips in LDS are done with

@@ -189,6 +189,19 @@ __global__ __launch_bounds__(kRowBlock) void layernorm_wave_kernel(
     const V* rr = res ? reinterpret_cast<const V*>(res + row * cols) : nullptr;
     float v[VPL][VN];
     float s = 0.f;
+    // gamma and beta are requested together with the row, not after the two reductions: their latency (they come from
+    // L2 for all but the first rows) then runs under the row's
+    const V* gv = reinterpret_cast<const V*>(gamma);
+    const V* bv = reinterpret_cast<const V*>(beta);
+    V gvec[VPL], bvec[VPL];
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+        const int vi = lane + j * kWave;
+        if (vi < nvec) {
+            gvec[j] = gv[vi];
+            bvec[j] = bv[vi];
+        }
+    }
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
         const int vi = lane + j * kWave;
@@ -232,14 +245,13 @@ __global__ __launch_bounds__(kRowBlock) void layernorm_wave_kernel(
         if (mean) mean[row] = mu;
         if (rstd) rstd[row] = inv;
     }
-    const V* gv = reinterpret_cast<const V*>(gamma);
-    const V* bv = reinterpret_cast<const V*>(beta);
     V* yr = reinterpret_cast<V*>(y + row * cols);
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
         const int vi = lane + j * kWave;
         if (vi < nvec) {
-            V g = gv[vi], b = bv[vi], t;
+            const V g = gvec[j], b = bvec[j];
+            V t;
 #pragma unroll
             for (int e = 0; e < VN; ++e) t[e] = from_f32<T>(v[j][e] * inv * to_f32(g[e]) + to_f32(b[e]));
             yr[vi] = t;

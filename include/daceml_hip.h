@@ -477,15 +477,22 @@ void dmlhip_debug_force_gemm_config(int cfg);
 /* 0: the fp16 contractions stage their operands through registers instead of loading them straight into LDS;
  * 1 = default. */
 void dmlhip_debug_gemm_direct_lds(int on);
+/* Per-workgroup timing of the pipelined fp16 contraction kernel: with a device buffer of 4 x 8 bytes per workgroup of
+ * the next launches set here, every workgroup stores four readings of the 100 MHz wall clock (start, first tile in
+ * LDS, end of the K loop, end of the epilogue) at buffer[4 * workgroup]; NULL (default) switches it off. The caller
+ * sizes the buffer for the largest grid it launches. Per calling thread. */
+void dmlhip_debug_gemm_trace(void* buffer);
 /* Number of grouped / K-concatenated / row-sum contraction calls that went out as one launch so far. */
 long long dmlhip_debug_grouped_single_launches(void);
-/* Pin the output-row strip height of dmlhip_conv2d_expand_depthwise_f32 (used if it fits LDS); 0 = default. */
+/* Run dmlhip_conv2d_expand_depthwise_f32 on its strip kernel with this output-row strip height (used if it fits LDS);
+ * 0 = default (the library's choice of kernel and geometry). */
 void dmlhip_debug_force_fused_strip(int toh);
 /* dmlhip_conv2d_expand_depthwise_f32 with a rolling window instead of strips: a workgroup walks down a segment of output
  * rows with the expanded rows in a ring in LDS, half of its wavefronts expanding the next rows while the other half runs
- * the stencil. rows: 0 = strips (default), -1 = as many output rows per batch as fit LDS, > 0 = at most that many;
- * waves: 8 or 16 wavefronts per workgroup. Never chosen by the library, not yet measured or validated on hardware;
- * shapes whose rows do not fit LDS keep the strips. Per calling thread. */
+ * the stencil. This is what the library runs; the switch pins its geometry. rows: 0 = the library's choice (default: the
+ * most output rows per batch whose ring lets two workgroups share a compute unit's LDS, else the most that fit), -1 = as
+ * many output rows per batch as fit LDS, > 0 = at most that many, -2 = the strip kernel; waves: 8 or 16 wavefronts per
+ * workgroup. Shapes of which not one row fits LDS run on the strips. Per calling thread. */
 void dmlhip_debug_fused_rolling(int rows, int waves);
 
 #ifdef __cplusplus

@@ -4,15 +4,19 @@
 // (the header and the exported symbols are usable from C++) and runs it with `check` on a GPU; the per-configuration
 // counter runs of the GEMM kernels are taken with it too.
 //
-//   gemm_from_cpp M N K a-layout b-layout config iterations [check]
+//   gemm_from_cpp M N K a-layout b-layout config iterations [check|trace]
 //     a-layout: k = A stored [m][k] (K-contiguous), r = A stored [k][m]
 //     b-layout: k = B stored [n][k] (K-contiguous), r = B stored [k][n]
 //     config:   tile configuration for dmlhip_debug_force_gemm_config (-1 = the library's own choice)
 //     check:    compare 2000 sampled outputs with a double-precision dot product on the host
+//     trace:    one more launch with dmlhip_debug_gemm_trace: where the workgroups' time goes (microseconds after the
+//               first workgroup started; median and maximum over workgroups of: start, first tile in LDS, end of the K
+//               loop, end of the epilogue)
 //
 // Build: python tests/cabi/build.py
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -33,13 +37,14 @@
 
 int main(int argc, char** argv) {
     if (argc < 8) {
-        std::printf("usage: gemm_from_cpp M N K a-layout(k|r) b-layout(k|r) config iterations [check]\n");
+        std::printf("usage: gemm_from_cpp M N K a-layout(k|r) b-layout(k|r) config iterations [check|trace]\n");
         return 1;
     }
     const long M = std::atol(argv[1]), N = std::atol(argv[2]), K = std::atol(argv[3]);
     const char al = argv[4][0], bl = argv[5][0];
     const int cfg = std::atoi(argv[6]), iters = std::atoi(argv[7]);
-    const bool check = argc > 8;
+    const bool check = argc > 8 && std::strcmp(argv[8], "check") == 0;
+    const bool trace = argc > 8 && std::strcmp(argv[8], "trace") == 0;
     if (M <= 0 || N <= 0 || K <= 0 || iters <= 0 || (al != 'k' && al != 'r') || (bl != 'k' && bl != 'r')) {
         std::printf("bad arguments\n");
         return 1;
@@ -87,6 +92,33 @@ int main(int argc, char** argv) {
     const double us = ms * 1e3 / iters;
     std::printf("M=%ld N=%ld K=%ld %c%c config %d: %.2f us per launch, %.1f TFLOP/s\n", M, N, K, al, bl, cfg, us,
                 2.0 * M * N * K / us / 1e6);
+    if (trace) {
+        const size_t slots = 4 * ((size_t)((M + 63) / 64) * ((N + 63) / 64) + 8);   // no tile is smaller than 64 x 64
+        unsigned long long* buf;
+        PROBE_CHECK(hipMalloc(&buf, slots * 8));
+        PROBE_CHECK(hipMemset(buf, 0, slots * 8));
+        dmlhip_debug_gemm_trace(buf);
+        dmlhip_gemm_f16(&d, a, b, c, nullptr, nullptr, nullptr, st);
+        PROBE_CHECK(hipStreamSynchronize(st));
+        dmlhip_debug_gemm_trace(nullptr);
+        std::vector<unsigned long long> h(slots);
+        PROBE_CHECK(hipMemcpy(h.data(), buf, slots * 8, hipMemcpyDeviceToHost));
+        std::vector<double> ph[4];
+        unsigned long long t0 = ~0ULL;
+        for (size_t w = 0; w * 4 < slots; ++w)
+            if (h[4 * w] && h[4 * w] < t0) t0 = h[4 * w];
+        for (size_t w = 0; w * 4 < slots; ++w)
+            if (h[4 * w])
+                for (int i = 0; i < 4; ++i) ph[i].push_back((double)(h[4 * w + i] - t0) * 0.01);   // 100 MHz -> us
+        const char* names[4] = {"start", "first tile in LDS", "end of the K loop", "end of the epilogue"};
+        std::printf("trace: %zu workgroups\n", ph[0].size());
+        for (int i = 0; i < 4; ++i) {
+            std::sort(ph[i].begin(), ph[i].end());
+            const size_t n = ph[i].size();
+            std::printf("  %-20s min %6.2f  p10 %6.2f  median %6.2f  p90 %6.2f  max %6.2f us\n", names[i], ph[i][0],
+                        ph[i][n / 10], ph[i][n / 2], ph[i][n * 9 / 10], ph[i][n - 1]);
+        }
+    }
     if (check) {
         std::vector<_Float16> hc((size_t)M * N);
         PROBE_CHECK(hipMemcpy(hc.data(), c, hc.size() * 2, hipMemcpyDeviceToHost));

@@ -46,3 +46,4 @@ def _reset_diagnostic_switches():
         lib.dmlhip_debug_gemm_direct_lds(1)
         lib.dmlhip_debug_force_fused_strip(0)
         lib.dmlhip_debug_fused_rolling(0, 8)
+        lib.dmlhip_debug_gemm_trace(None)

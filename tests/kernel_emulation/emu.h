@@ -135,6 +135,7 @@ typedef emu_dim3 dim3;
 /* global -> LDS transfer of `size` bytes per lane: lane l's piece lands at the LDS pointer + size * l */
 #define __builtin_amdgcn_global_load_lds(g, l, size, offset, aux) \
     emu::dma_issue((const void*)(g), (uint32_t)((const char*)(l) - emu::g_lds) + (size) * (threadIdx.x & 63), size)
+inline unsigned long long wall_clock64() { return 0; }
 inline uint32_t __umulhi(uint32_t a, uint32_t b) { return (uint32_t)(((uint64_t)a * b) >> 32); }
 inline uint32_t __float_as_uint(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
 inline float __uint_as_float(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }

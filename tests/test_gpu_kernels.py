@@ -552,8 +552,9 @@ EXPAND_DEPTHWISE_CASES = [
 
 @pytest.mark.parametrize("n,cin,cmid,h,w,stride,acts,has_bias", EXPAND_DEPTHWISE_CASES)
 def test_conv2d_expand_depthwise(n, cin, cmid, h, w, stride, acts, has_bias):
-    """The fused pointwise + depthwise kernel against the composition of the two oracle convolutions, at the strip
-    height the library picks and at pinned ones (strips of 1 and 4 output rows recompute different halo rows)."""
+    """The fused pointwise + depthwise convolution against the composition of the two oracle convolutions: the kernel
+    the library picks (0) and the strip kernel at pinned heights (strips of 1 and 4 output rows recompute different
+    halo rows)."""
     from daceml_amd import _lib as L, kernels as K
     code = {"none": L.ACT_NONE, "swish": L.ACT_SWISH, "relu": L.ACT_RELU}
     fn = {"none": lambda t: t, "swish": O.swish, "relu": lambda t: np.maximum(t, 0.0)}

@@ -1,5 +1,5 @@
-"""The rolling-window form of the fused pointwise + depthwise convolution (reachable only through
-``dmlhip_debug_fused_rolling``) on the problems the strip kernel is tested with, and on the benchmarked MBConv shape,
+"""The rolling-window form of the fused pointwise + depthwise convolution (what the library runs; its geometry pinned
+through ``dmlhip_debug_fused_rolling``) on the problems the strip kernel is tested with, and on the benchmarked MBConv shape,
 where it must agree with the strip kernel bit for bit (both add in the same order).
 """
 import numpy as np
@@ -32,9 +32,10 @@ def test_conv2d_expand_depthwise_rolling(n, cin, cmid, h, w, stride, acts, has_b
     run = lambda: K.conv2d_expand_depthwise(dev(x), dev(w1), None if b1 is None else dev(b1), dev(w2),  # noqa: E731
                                             None if b2 is None else dev(b2), stride=stride, act_pw=code[acts[0]],
                                             act_dw=code[acts[1]])
+    lib.dmlhip_debug_fused_rolling(-2, 8)
     strips = host(run())
     try:
-        for rows in (-1, 1, 2):
+        for rows in (0, -1, 1, 2):
             lib.dmlhip_debug_fused_rolling(rows, waves)
             got = host(run())
             assert_close(got, want, torch.float32, "rolling window, rows %d" % rows, rtol=1e-5, atol=4e-6)
@@ -56,12 +57,15 @@ def test_rolling_window_on_the_benchmarked_block(waves):
     b2 = (torch.randn(192, generator=g) * 0.1).cuda()
     lib = L.load()
     run = lambda: K.conv2d_expand_depthwise(x, w1, b1, w2, b2, stride=2, act_pw=L.ACT_SWISH, act_dw=L.ACT_SWISH)  # noqa: E731
+    lib.dmlhip_debug_fused_rolling(-2, 8)
     strips = run()
     try:
         lib.dmlhip_debug_fused_rolling(-1, waves)
         got = run()
+        lib.dmlhip_debug_fused_rolling(0, waves)
+        chosen = run()
         torch.cuda.synchronize()
     finally:
         lib.dmlhip_debug_fused_rolling(0, 8)
     assert got.shape == strips.shape == (96, 192, 56, 56)
-    assert torch.equal(got, strips)
+    assert torch.equal(got, strips) and torch.equal(chosen, strips)
