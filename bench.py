@@ -93,7 +93,9 @@ def check_against_oracle(args, x, dy, p):
 
 
 def kernel_breakdown(prog, reps=10):
-    """HIP-event duration of every launch (events on the stream the kernels run on), averaged."""
+    """HIP-event duration of every launch, averaged over `reps` passes: one event on the launch stream between
+    consecutive launches, so a launch's time is the kernel plus its dispatch on the stream and the times of a pass
+    add up to the pass."""
     acc = None
     for _ in range(reps):
         rows = prog.launch_timed()

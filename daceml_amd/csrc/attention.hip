@@ -360,14 +360,14 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
 constexpr int kBwdStages = 3;
 constexpr float kLog2e = 1.44269504088896340736f;
 
-__device__ __forceinline__ floatx4 lds_read_f32x4(uint32_t addr) {
+[[nodiscard]] __device__ __forceinline__ floatx4 lds_read_f32x4(uint32_t addr) {
     floatx4 v;
     asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr));
     return v;
 }
 
 template <int OFF>
-__device__ __forceinline__ half8 tr_pair(uint32_t lo_addr, uint32_t hi_addr) {
+[[nodiscard]] __device__ __forceinline__ half8 tr_pair(uint32_t lo_addr, uint32_t hi_addr) {
     const half4v lo = lds_read_tr16_b64<OFF>(lo_addr);
     const half4v hi = lds_read_tr16_b64<OFF>(hi_addr);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);

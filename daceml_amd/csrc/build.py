@@ -36,6 +36,8 @@ SOURCES = [
 COMMON_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
     "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
+    # the LDS readers of lds_ops.h are [[nodiscard]]: dropping the value of one is an error, not a warning
+    "-Werror=unused-result",
 ]
 
 

@@ -471,7 +471,7 @@ __global__ __launch_bounds__(kThreads) void gemm_f16_pipe_kernel(const _Float16*
         __builtin_amdgcn_wave_barrier();
     });
     if (g.trace && threadIdx.x == 0) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's stores have been accepted
+        wait_vm_lgkm0<0>();   // this wavefront's stores have been accepted
         g.trace[4 * (size_t)blockIdx.x + 3] = wall_clock64();
     }
     if constexpr (ASUM) {

@@ -8,8 +8,9 @@
 // The price: the compiler takes a read's destination registers to be written when the instruction issues, not when
 // the data arrives. Every value returned by lds_read_* must therefore be consumed, after a wait that covers it, on
 // every path that issued the read. A result left unused has no live range, its registers go to the next value the
-// compiler needs (a global address, say), and the LDS data lands on top of that value later. tests/test_isa_hazards.py
-// checks the compiled kernels for this.
+// compiler needs (a global address, say), and the LDS data lands on top of that value later. The readers are
+// [[nodiscard]] and the library is built with -Werror=unused-result, so a call whose value is dropped does not compile;
+// tests/test_isa_hazards.py checks the compiled kernels for values that are assigned and then never read.
 #pragma once
 
 #include "common.h"
@@ -30,7 +31,7 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 }
 
 template <int OFFSET>
-__device__ __forceinline__ half8 lds_read_b128(uint32_t addr) {
+[[nodiscard]] __device__ __forceinline__ half8 lds_read_b128(uint32_t addr) {
     half8 v;
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
     return v;
@@ -40,7 +41,7 @@ __device__ __forceinline__ half8 lds_read_b128(uint32_t addr) {
 // elements of row s/4 (columns 4*(s%4)..+3 of the group's 16 columns); lane j receives column j of
 // the four rows. A lane thus gets four consecutive K values of "its" column, the MFMA operand layout.
 template <int OFFSET>
-__device__ __forceinline__ half4v lds_read_tr16_b64(uint32_t addr) {
+[[nodiscard]] __device__ __forceinline__ half4v lds_read_tr16_b64(uint32_t addr) {
     half4v v;
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
     return v;

@@ -545,7 +545,7 @@ class HipLayerNormalizationGrad(ONNXForward):
                 return False
             for name in ("scale_grad", "bias_grad"):
                 d = outs[name]
-                if not (d.dtype == torch.float32 and d.is_contiguous() and d.total_size == h):
+                if not (d.dtype in (torch.float32, x.dtype) and d.is_contiguous() and d.total_size == h):
                     return False
             return (_ln_common(x, ins["scale"], None, node.axis) and _stat_ok(ins["mean"], rows)
                     and _stat_ok(ins["inv_std_var"], rows))
@@ -557,11 +557,25 @@ class HipLayerNormalizationGrad(ONNXForward):
         x = in_desc_with_name(node, state, sdfg, "X")
         rows, cols = _prod(x.shape[:-1]), x.shape[-1]
         ws = L.load().dmlhip_layernorm_backward_workspace_bytes(rows, cols)
+        # The kernel sums the scale / shift gradients in fp32 and writes them as fp32. Where the graph wants them in
+        # the tensor dtype (a caller without fp32 master gradients: the reference gives a gradient the dtype of its
+        # forward array), they land behind the kernel's own workspace and are cast from there.
+        grads, casts, end = {}, [], (ws + 255) // 256 * 256
+        for name in ("scale_grad", "bias_grad"):
+            d = out_desc_with_name(node, state, sdfg, name)
+            if d.dtype == torch.float32:
+                grads[name] = Ptr(name)
+            else:
+                grads[name] = Workspace(end)
+                casts.append(HipCall("dmlhip_cast", [I32(_CODE[torch.float32]), I32(_CODE[d.dtype]), Workspace(end),
+                                                     Ptr(name), I64(cols), Stream()], flops=0, bytes_moved=0))
+                end += (cols * 4 + 255) // 256 * 256
         call = HipCall("dmlhip_layernorm_backward_" + _SFX[x.dtype],
                        [Ptr("Y_grad"), Ptr("X"), Ptr("mean"), Ptr("inv_std_var"), Ptr("scale"), Ptr("X_grad"),
-                        Ptr("scale_grad"), Ptr("bias_grad"), I64(rows), I64(cols), Workspace(), WorkspaceBytes(),
+                        grads["scale_grad"], grads["bias_grad"], I64(rows), I64(cols), Workspace(), WorkspaceBytes(),
                         Stream()])
-        return _tasklet(node, state, [call], workspace_bytes=ws, bytes_moved=3 * _nbytes(x), kind="layernorm_backward")
+        return _tasklet(node, state, [call] + casts, workspace_bytes=end, bytes_moved=3 * _nbytes(x),
+                        kind="layernorm_backward")
 
 
 # ----------------------------------------------------------------------------- elementwise

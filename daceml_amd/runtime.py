@@ -304,19 +304,22 @@ class CompiledSDFG:
         return CapturedLaunches(self, graph, self._binding)
 
     def launch_timed(self):
-        """Like launch(), with a HIP event pair around every kernel; returns [(launch, ms)]."""
+        """Like launch(), with one HIP event on the launch stream before the first kernel and one after every kernel;
+        returns [(launch, ms)] where a launch's time runs from the event before it to the event after it - the kernel
+        and its dispatch on the stream. The times add up to the time of the whole sequence between the first and the
+        last event."""
         self._stream.value = torch.cuda.current_stream(self.device).cuda_stream
-        events = []
+        marks = [torch.cuda.Event(enable_timing=True)]
+        marks[0].record()
         for l in self._launches:
-            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s.record()
             status = l.fn(*l.args)
+            e = torch.cuda.Event(enable_timing=True)
             e.record()
+            marks.append(e)
             if status != 0:
                 raise L.HipKernelError(status, "%s (%s): %s" % (l.label, l.symbol, L.last_error()))
-            events.append((l, s, e))
         torch.cuda.synchronize(self.device)
-        return [(l, s.elapsed_time(e)) for l, s, e in events]
+        return [(l, marks[i].elapsed_time(marks[i + 1])) for i, l in enumerate(self._launches)]
 
     @property
     def launches(self) -> Sequence[_Launch]:

@@ -584,9 +584,10 @@ def _reshape_to_view(sdfg: SDFG, state: SDFGState, reshape) -> bool:
     return True
 
 
-def fold_views(sdfg: SDFG) -> int:
+def fold_views(sdfg: SDFG, reshapes: bool = True) -> int:
     """Fold Transposes next to two-operand Einsums into the equation's letters, and Reshapes of dense
-    arrays into views, so that head split / merge and weight transposes cost no kernel and no HBM pass."""
+    arrays into views, so that head split / merge and weight transposes cost no kernel and no HBM pass.
+    ``reshapes=False`` leaves the Reshape nodes alone (no aliasing descriptors are created)."""
     count = 0
     for state in sdfg.states():
         changed = True
@@ -629,7 +630,7 @@ def fold_views(sdfg: SDFG) -> int:
                         count += 1
                         changed = True
                         break
-                    if _is_op(pnode, "Reshape") and _reshape_to_view(sdfg, state, pnode):
+                    if reshapes and _is_op(pnode, "Reshape") and _reshape_to_view(sdfg, state, pnode):
                         count += 1
                         changed = True
                         break
@@ -658,7 +659,8 @@ def fold_views(sdfg: SDFG) -> int:
                         count += 1
                         changed = True
                         break
-                if len(cons) == 1 and _is_op(cons[0][0], "Reshape") and _reshape_to_view(sdfg, state, cons[0][0]):
+                if reshapes and len(cons) == 1 and _is_op(cons[0][0], "Reshape") and \
+                        _reshape_to_view(sdfg, state, cons[0][0]):
                     count += 1
                     changed = True
                     break
@@ -1273,7 +1275,7 @@ def optimize_backward(sdfg: SDFG) -> Dict[str, int]:
 
 
 def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True,
-                  gelu_epilogue: bool = False) -> Dict[str, int]:
+                  gelu_epilogue: bool = False, views: bool = True) -> Dict[str, int]:
     """The pass pipeline, in dependency order (cf. daceml.util.utils.auto_optimize,
     daceml/util/utils.py:205-235). Returns how often each rewrite fired.
 
@@ -1293,7 +1295,9 @@ def auto_optimize(sdfg: SDFG, training: bool = False, attention: bool = True,
     stats["gated_conv"] = 0 if training else fuse_gate_into_conv(sdfg)
     stats["expand_depthwise"] = 0 if training else fuse_expand_depthwise(sdfg)
     stats["matmul_to_einsum"] = lower_matmul(sdfg)
-    stats["views"] = fold_views(sdfg)
+    # views=False folds Transposes into the equations of the contractions next to them but keeps Reshape nodes: for
+    # callers that hand the graph to a host with a view mechanism of its own (daceml_amd.dace_plugin.fuse_library_nodes)
+    stats["views"] = fold_views(sdfg, reshapes=views)
     stats["epilogues"] = fuse_epilogues(sdfg, keep_preactivation=training, activation_in_epilogue=gelu_epilogue)
     stats["skip_layernorm"] = 0 if training else fuse_skip_layernorm(sdfg)
     stats["attention"] = fuse_attention(sdfg) if attention else 0

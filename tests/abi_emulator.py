@@ -345,7 +345,13 @@ class Emulator:
             elif call.symbol in ("dmlhip_layernorm_f16", "dmlhip_layernorm_f32"):
                 layernorm(*args[:11])
             elif call.symbol in ("dmlhip_layernorm_backward_f16", "dmlhip_layernorm_backward_f32"):
-                layernorm_backward(*args[:10])
+                a = list(args[:10])
+                a[6], a[7] = self._typed(a[6], np.float32), self._typed(a[7], np.float32)   # fp32, possibly in the workspace
+                layernorm_backward(*a)
+            elif call.symbol == "dmlhip_cast":
+                kinds = {L.F16: np.float16, L.F32: np.float32}
+                src, dst, n = self._typed(args[2], kinds[args[0]]), self._typed(args[3], kinds[args[1]]), args[4]
+                dst.reshape(-1)[:n] = src.reshape(-1)[:n].astype(kinds[args[1]])
             elif call.symbol == "dmlhip_attention_f16":
                 attention(*args[:6])
             elif call.symbol == "dmlhip_attention_masked_f16":

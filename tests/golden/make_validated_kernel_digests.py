@@ -1,5 +1,6 @@
-"""Writes tests/golden/validated_kernel_digests.json: one SHA-256 per kernel of tests/isa/validated_instances.hip and
-of the strip kernels of daceml_amd/csrc/conv_fused.hip, over the kernel's instructions as the compiler emits them
+"""Writes tests/golden/validated_kernel_digests.json: one SHA-256 per kernel of tests/isa/validated_instances.hip, of
+the fused expand + depthwise kernels of daceml_amd/csrc/conv_fused.hip and of the attention kernels of
+daceml_amd/csrc/attention.hip, over the kernel's instructions as the compiler emits them
 (comments and block-label numbers removed).
 
 Run it on a tree whose kernels have just passed the GPU tests - the digests are a record of what was validated on

@@ -407,7 +407,9 @@ def test_emitted_program_runs_the_calls_in_dependency_order():
 # ----------------------------------------------------------------------------- install() against stand-ins
 class _Recorder:
     """Stand-ins for the few DaCe / DaCeML entry points install() touches. They record what they are given."""
-    def __init__(self):
+    def __init__(self, upstream=("Softmax", "Einsum", "MatMul", "Gemm", "Add", "Mul", "Conv", "Transpose", "Relu",
+                                 "ReduceSum")):
+        self.upstream = upstream
         self.forward_registry = {}
         self.node_implementations = {}
         self.backward_registry = {}
@@ -436,13 +438,13 @@ class _Recorder:
                 return self.add_node(n)
 
         class FakeSDFG(S.SDFG):
+            def add_array(self, name, shape, dtype, transient=False, strides=None, storage=None, find_new_name=False):
+                return super().add_array(name, shape, dtype, transient=transient, strides=strides)
+
             def add_state(self, label=None):
                 st = FakeState(label or "state_%d" % len(self._states), self)
                 self._states.append(st)
                 return st
-
-            def add_array(self, name, shape, dtype, transient=False, strides=None, storage=None, find_new_name=False):
-                return super().add_array(name, shape, dtype, transient=transient, strides=strides)
 
             def nodes(self):
                 return self.states()
@@ -454,8 +456,20 @@ class _Recorder:
         dace.pointer = lambda t: ("pointer", t)
         dace.StorageType = types.SimpleNamespace(GPU_Global="GPU_Global")
         dace.dtypes = types.SimpleNamespace(Language=types.SimpleNamespace(CPP="CPP"))
-        dace.nodes = types.SimpleNamespace(AccessNode=S.AccessNode)
+        class LibraryNode(S.Node):
+            def __init__(self, name, inputs=(), outputs=()):
+                super().__init__(name)
+                for c in inputs:
+                    self.add_in_connector(c)
+                for c in outputs:
+                    self.add_out_connector(c)
+        dace.nodes = types.SimpleNamespace(AccessNode=S.AccessNode, LibraryNode=LibraryNode)
+        properties = types.ModuleType("dace.properties")
+        properties.Property = lambda dtype=None, default=None, desc="": default
+        dace.properties = properties
         library = types.ModuleType("dace.library")
+        library.node = lambda cls: cls
+        library.expansion = lambda cls: cls
 
         def environment(cls):
             cls.full_class_path = classmethod(lambda c: "daceml_amd.dace_plugin." + c.__name__)
@@ -466,7 +480,7 @@ class _Recorder:
 
         def autoregister_params(**params):
             def dec(cls):
-                rec.backward_registry[params["op"]] = (cls, params)
+                rec.backward_registry[params.get("op") or params["node_type"]] = (cls, params)
                 return cls
             return dec
         registry.autoregister_params = autoregister_params
@@ -480,16 +494,17 @@ class _Recorder:
         import daceml_amd.onnx as our
         daceml = types.ModuleType("daceml")
         donnx = types.ModuleType("daceml.onnx")
-        upstream = {"Softmax", "Einsum", "MatMul", "Gemm", "Add", "Mul", "Conv", "Transpose", "Relu", "ReduceSum"}
+        upstream = set(rec.upstream)
         donnx.has_onnx_node = lambda name: name in upstream
 
         def node_class(op):
-            class Cls:
+            class Cls(our.get_onnx_node(op)):       # instantiable like DaCeML's: ONNX<Op>(label, **attributes)
                 implementations = {}
 
                 @classmethod
                 def register_implementation(cls, name, expansion):
                     rec.node_implementations.setdefault(op, {})[name] = expansion
+            Cls.__name__ = "ONNX" + op
             return Cls
         for op in upstream:
             setattr(donnx, "ONNX" + op, node_class(op))
@@ -528,7 +543,8 @@ class _Recorder:
                                                                                           ctx.forward_sdfg, conn)
         rec.forwarded = []
         butils.connect_output_from_forward = lambda fwd, bwd, ctx, conn: rec.forwarded.append((fwd.label, conn))
-        return {"dace": dace, "dace.library": library, "dace.registry": registry, "dace.transformation": transformation,
+        return {"dace": dace, "dace.library": library, "dace.registry": registry, "dace.properties": properties,
+                "dace.transformation": transformation,
                 "dace.transformation.transformation": tt, "daceml": daceml, "daceml.onnx": donnx,
                 "daceml.onnx.forward_implementation_abc": fia, "daceml.onnx.op_implementations": opi,
                 "daceml.onnx.op_implementations.utils": opu, "daceml.util": util, "daceml.util.utils": uu,
@@ -597,3 +613,76 @@ def test_install_registers_forward_and_backward_implementations(monkeypatch):
     st.add_edge(st.add_read("strided"), None, bad, "input", s.make_array_memlet("strided"))
     st.add_edge(bad, "output", st.add_write("out2"), None, s.make_array_memlet("out2"))
     assert rec.forward_registry["Softmax"][0].forward_can_be_applied(bad, st, s) is False
+
+
+def test_training_graphs_reach_the_fused_kernels_as_library_nodes(monkeypatch):
+    """What a ``post_onnx_hook`` of the reference's ``DaceModule(backward=True)`` does with ``fuse_for_training``: the
+    decomposed BERT encoder layer is rewritten into fused nodes that are still LIBRARY nodes - DaCeML's own classes
+    where it has one, one generic class otherwise - and each of them is given its "hip" reverse by the registry
+    lookup the reference's backward-pass generator performs (find_backward_implementation, base_abc.py:114-159)."""
+    from daceml_amd import dace_plugin, graphs
+    opset12 = ("Softmax", "Einsum", "MatMul", "Gemm", "Add", "Sub", "Mul", "Div", "Pow", "Sqrt", "Erf", "ReduceMean",
+               "Transpose", "Reshape", "Relu", "ReduceSum", "Identity", "Conv")
+    rec = _Recorder(upstream=opset12)
+    mods, FakeSDFG = rec.modules()
+    for name, mod in mods.items():
+        monkeypatch.setitem(sys.modules, name, mod)
+    monkeypatch.setattr(dace_plugin, "_FUSED_NODE_CLASS", {})
+    dace_plugin.install()
+
+    # the reference's graph after import: opset-12 nodes only, on the stand-in "DaCe" classes
+    sdfg = graphs.bert_encoder_layer(2, 64, 128, 2, 256, torch.float16, eps=1e-12)
+    state = sdfg.states()[0]
+    assert {n.schema.name for n in state.library_nodes()} <= set(opset12)
+    n_before = len(state.library_nodes())
+    sdfg.__class__ = FakeSDFG
+    state.__class__ = type(FakeSDFG("x").add_state())
+    # the reference's importer keeps the values of initialisers in ONNXModel.weights
+    module = types.SimpleNamespace(sdfg=sdfg, backward=True,
+                                   dace_model=types.SimpleNamespace(weights=dict(sdfg.constants)))
+    assert dace_plugin.fuse_for_training(module) == 1
+
+    fused_cls = dace_plugin.make_fused_node_class(mods["dace"])
+    nodes = [n for n in state.nodes() if not isinstance(n, mods["dace"].nodes.AccessNode)]
+    assert len(nodes) < n_before
+    kinds = {}
+    for n in nodes:
+        if isinstance(n, fused_cls):
+            kinds.setdefault(n.hip_kind, []).append(n)
+        else:
+            assert n.schema.name in opset12 and type(n).__name__ == "ONNX" + n.schema.name
+    assert len(kinds["LayerNormalization"]) == 2 and len(kinds["FusedAttention"]) == 1 and "FusedEinsum" in kinds
+    assert any(k in kinds for k in ("Gelu", "BiasGelu")) and "Softmax" not in {getattr(n, "schema", None) and
+                                                                                 n.schema.name for n in nodes}
+    # created with the outputs their reverse nodes will ask for
+    ln = kinds["LayerNormalization"][0]
+    assert {"Mean", "InvStdDev"} <= set(ln.out_connectors)
+    assert "LogSumExp" in kinds["FusedAttention"][0].out_connectors
+    # ... and the rewritten state still computes the layer: its forward expansions lower to the kernels' entry points
+    expand = fused_cls.implementations["hip"].expansion
+    assert "dmlhip_layernorm_f16" in expand(ln, state, sdfg).states()[0].library_nodes()[0].code
+    att = kinds["FusedAttention"][0]
+    assert "dmlhip_attention_f16" in expand(att, state, sdfg).states()[0].library_nodes()[0].code
+
+    # the generator's lookup: by node class for the fused nodes
+    cls, params = rec.backward_registry[fused_cls]
+    assert params == {"node_type": fused_cls, "name": "hip"}
+    bst = sdfg.add_state("backward")
+    ctx = types.SimpleNamespace(forward_sdfg=sdfg, forward_state=state, backward_sdfg=sdfg, backward_state=bst,
+                                backward_generator=None)
+    expected = {"LayerNormalization": "dmlhip_layernorm_backward_f16", "FusedAttention": "dmlhip_attention_backward_f16",
+                "Gelu": "dmlhip_unary_backward_f16", "BiasGelu": "dmlhip_", "FusedEinsum": "dmlhip_gemm_f16"}
+    for kind, members in kinds.items():
+        node = members[0]
+        assert cls.backward_can_be_applied(node, state, sdfg), kind
+        given = [e.src_conn for e in state.out_edges(node) if e.src_conn in ("Y", "Output", "output")]
+        required = [e.dst_conn for e in state.in_edges(node) if e.dst_conn not in ("Mask", )]
+        rec.forwarded.clear()
+        rev, result = cls.backward(node, ctx, given, required)
+        code = "\n".join(t.code for t in rev.sdfg.states()[0].library_nodes())
+        assert expected[kind] in code, (kind, code[:300])
+        assert set(result.required_grad_names) == set(required)
+        if kind == "LayerNormalization":    # the statistics come from the forward node, not from a recomputation
+            assert {c for _, c in rec.forwarded} >= {"Mean", "InvStdDev"}
+        if kind == "FusedAttention":
+            assert {c for _, c in rec.forwarded} >= {"Output", "LogSumExp"}

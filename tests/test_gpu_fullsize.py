@@ -151,11 +151,21 @@ def test_mbconv_block_config_shape():
         se = O.global_average_pool(t)
         se = O.swish(O.conv2d(se, f["se1_w"], f["se1_b"]))
         se = O.sigmoid(O.conv2d(se, f["se2_w"], f["se2_b"]))
-        want = O.conv2d(O.mul(t, se), f["proj_w"], f["proj_b"])
-        # five chained fp32 nodes (K = 32, 9, 3136-element mean, 192): 1e-5 relative with the absolute floor the
-        # block test at reduced size uses (the reference's own tolerance for this block is 1e-3,
-        # tests/torch/test_efficientnet_block.py:50-54)
-        assert_close(got[img:img + 1], want, torch.float32, "mbconv image %d" % img, rtol=1e-5, atol=5e-6)
+        gated = O.mul(t, se)
+        want = O.conv2d(gated, f["proj_w"], f["proj_b"])
+        # north_star's rtol 1e-5 / atol 1e-6 plus what fp32 arithmetic costs an output that is a cancelling sum of
+        # K = 192 products t_k (u = 2^-24 per rounding, errors taken as independent): each t_k carries n = 5 roundings
+        # (four fp32 nodes before the last convolution and the product itself), standard deviation n u |t_k| / sqrt 3;
+        # the k-th addition rounds a partial sum of size ~ sqrt(k) rms(t), together u |t|_2 sqrt(K / 2). Four standard
+        # deviations of the sum of both (measured: the worst of 150 528 outputs per image reaches 0.4 of it). The reference's own
+        # tolerance for this block is 1e-3 (tests/torch/test_efficientnet_block.py:50-54).
+        l2 = np.sqrt(O.conv2d(gated ** 2, f["proj_w"] ** 2, None))
+        bound = 1e-6 + 1e-5 * np.abs(want) + 4 * 2.0 ** -24 * np.sqrt(25 / 3 + 192 / 2) * l2
+        err = np.abs(got[img:img + 1].astype(np.float64) - want)
+        worst = float((err / bound).max())
+        assert worst < 1.0, "mbconv image %d: error reaches %.2f of the derived bound" % (img, worst)
+        print("mbconv image %d: worst error %.3g, %.2f of the derived bound (median bound %.3g)"
+              % (img, float(err.max()), worst, float(np.median(bound))))
 
 
 def test_conv_config_shape():

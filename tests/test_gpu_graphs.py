@@ -315,3 +315,4 @@ def test_reduce_and_transpose_backward(dtype):
     kw = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=3e-2, atol=0.15)
     assert_close(host(out["y"]), ty.detach().numpy(), dtype, "forward", **kw)
     assert_close(host(out["gradient_x"]), tx.grad.numpy(), dtype, "gradient of x", **kw)
+

@@ -67,3 +67,23 @@ def test_interleaved_gemm_loop(tmp_path):
     count, found = isa_hazards.check_file(_assembly(os.path.join(ROOT, "tests", "isa", "ilv_instances.hip"), tmp_path))
     assert count == 28, "five tile configurations, operand pairs and row sums x four operand-layout pairs"
     assert not found, _report(found)
+
+
+def test_dropping_the_value_of_an_lds_read_does_not_compile(tmp_path):
+    """The readers of lds_ops.h are [[nodiscard]] and the library's flags turn the warning into an error: the pattern
+    behind the register race (a read issued, its value never used) is rejected by the compiler."""
+    from daceml_amd.csrc import build as B
+    if not (shutil.which("hipcc") or os.path.exists("/opt/rocm/bin/hipcc")):
+        pytest.skip("no hipcc")
+    header = os.path.join(ROOT, "daceml_amd", "csrc", "lds_ops.h")
+    body = {"dropped": "dml::lds_read_b128<0>(0u); dml::lds_read_tr16_b64<0>(0u); o[0] = 1.f;",
+            "used": "const dml::half8 v = dml::lds_read_b128<0>(0u); dml::wait_lgkm<0>(); o[0] = (float)v[0];"}
+    results = {}
+    for name, text in body.items():
+        src = tmp_path / (name + ".hip")
+        src.write_text('#include "%s"\n__global__ void k(float* o) { %s }\n' % (header, text))
+        cmd = [B.hipcc(), *B.COMMON_FLAGS, "-x", "hip", "--offload-device-only", "-c", str(src), "-o",
+               str(tmp_path / (name + ".o"))]
+        results[name] = subprocess.run(cmd, capture_output=True, text=True)
+    assert results["used"].returncode == 0, results["used"].stderr[-2000:]
+    assert results["dropped"].returncode != 0 and "nodiscard" in results["dropped"].stderr

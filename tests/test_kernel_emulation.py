@@ -344,12 +344,15 @@ def test_expand_depthwise_rolling_window(conv_fused_lib, shape, acts, bias):
 
 
 def test_rolling_window_geometry_of_the_benchmarked_block(conv_fused_lib):
-    """[96,32,112,112] -> 192 channels, stride 2, on 256 compute units: two output rows per batch in a ring of nine
-    expanded rows (137 KB of LDS), four segments of 14 output rows per image: 2304 workgroups, nine per compute unit."""
+    """[96,32,112,112] -> 192 channels, stride 2, on 256 compute units. The library's choice (rows 0): one output row
+    per batch in a ring of five expanded rows (73 KB of LDS, so two workgroups share a compute unit); the most rows
+    that fit (rows -1): two per batch in a ring of nine (137 KB)."""
     shape = (1, 32, 32, 112, 112, 2)
     operands, want = _expand_depthwise_problem(*shape, 1, True)
     # one image and one channel block of the block's 96 x 6: the same rows, spread as if over 256 / (96 * 6) of a chip
     _, geometry = _run_expand_depthwise(conv_fused_lib, 1, 0, 8, 256, 1, shape, operands, want, seed=7)
+    assert geometry[:2] == [1, 5]
+    _, geometry = _run_expand_depthwise(conv_fused_lib, 1, -1, 8, 256, 1, shape, operands, want, seed=7)
     assert geometry[:2] == [2, 9]
 
 

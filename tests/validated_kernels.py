@@ -13,9 +13,11 @@ import subprocess
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SOURCES = [os.path.join(ROOT, "tests", "isa", "validated_instances.hip"),
-           os.path.join(ROOT, "daceml_amd", "csrc", "conv_fused.hip")]
-#: kernels of SOURCES that are recorded (the rolling-window kernels of conv_fused.hip have not run on hardware)
-RECORDED = re.compile(r"gemm_f16_pipe_kernel|expand_depthwise_kernel")
+           os.path.join(ROOT, "daceml_amd", "csrc", "conv_fused.hip"),
+           os.path.join(ROOT, "daceml_amd", "csrc", "attention.hip")]
+#: kernels of SOURCES that are recorded
+RECORDED = re.compile(r"gemm_f16_pipe_kernel|expand_depthwise_kernel|expand_depthwise_rolling_kernel|attention_fwd_kernel|"
+                      r"attention_bwd_dq_kernel|attention_bwd_dkv_kernel")
 
 
 def have_hipcc():
