@@ -24,8 +24,11 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # Bytes that cross the L2 <-> fabric boundary for the 11 GEMM launches of one step: rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE (one run each, of `bench.py --steps 3 --warmup 2 --no-cpu-baseline --calibrate-copy`), each
 # scaled by what the same counter reads for the 128 MiB copy kernel of --calibrate-copy (FETCH_SIZE x 2.000,
-# WRITE_SIZE x 1.000). Measured, not computed here: it goes stale when the GEMM tiling changes.
-GEMM_TRAFFIC_BYTES_PER_STEP = {"fetched": 866.6e6, "written": 184.6e6}
+# WRITE_SIZE x 1.000). Measured, not computed here: it goes stale when the GEMM tiling changes, so the tile selection
+# it was measured with is part of the value and is compared with the library's at run time.
+GEMM_TRAFFIC_BYTES_PER_STEP = {"fetched": 828.7e6, "written": 184.6e6,
+                               "measured_with": "tile configurations 4 (256x256) / 5 (128x128, four stages) / 9 chosen by "
+                                                "the library, interleaved K loop; profiles/bert_layer_fwd_bwd_hbm_traffic.md"}
 
 METRIC = "BERT-large encoder layer fp16 fwd+bwd ms/iter at 1 GPU; % MFMA & HBM roofline"
 B, S, H, HEADS, FFN = 8, 512, 1024, 16, 4096
@@ -534,7 +537,10 @@ def main():
                      "frac": round(tflops / PEAK_FP16_TFLOPS, 4),
                      "traffic": GEMM_TRAFFIC_BYTES_PER_STEP["fetched"] + GEMM_TRAFFIC_BYTES_PER_STEP["written"],
                      "traffic_note": "bytes per step over the same launches (rocprofv3 FETCH_SIZE + WRITE_SIZE, "
-                                     "calibrated on a copy kernel); algorithmic bytes of those launches: %d" % gemm_bytes,
+                                     "calibrated on a copy kernel; a constant measured with: %s%s); algorithmic bytes "
+                                     "of those launches: %d" % (GEMM_TRAFFIC_BYTES_PER_STEP["measured_with"],
+                                                                "; THIS RUN PINS ANOTHER CONFIGURATION" if a.gemm_config >= 0
+                                                                else "", gemm_bytes),
                      "kernel": "gemm_f16_pipe_kernel (all %d contraction launches of a step)" % n_gemm,
                      "flops_per_step": gemm_flops, "ms_per_step": round(gemm_ms, 4)},
         "attention_nodes": attn,
