@@ -191,8 +191,16 @@ __device__ __forceinline__ void store_strip(const GemmArgs& g, void* c_ptr, void
                 }
             }
             if constexpr (ACT) {
+                // the activation is chosen once per store, not once per element: with the five-way choice inside the
+                // unrolled element loop the epilogue grows to tens of thousands of instructions and runs out of the
+                // instruction cache
+                if (g.act == DMLHIP_ACT_GELU) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] = apply_act_half(g.act, v[e]);
+                    for (int e = 0; e < 8; ++e) v[e] = gelu_half_f(v[e]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] = apply_act_half(g.act, v[e]);
+                }
             }
             if constexpr (GENERAL) {
                 if (R) {
