@@ -151,6 +151,7 @@ SIGNATURES = {
     "dmlhip_debug_grouped_single_launches": (ctypes.c_longlong, []),
     "dmlhip_debug_force_fused_strip": (None, [c_int]),
     "dmlhip_debug_fused_rolling": (None, [c_int, c_int]),
+    "dmlhip_debug_attention_trace": (None, [c_void_p]),
     "dmlhip_debug_gemm_trace": (None, [c_void_p]),
 }
 

@@ -39,6 +39,7 @@ struct AttnArgs {
     int64_t qs[3], ks[3], vs[3], os[3];       // element strides: batch0, batch1, sequence (head dim stride 1)
     int64_t dqs[3], dks[3], dvs[3], dos[3];   // gradient tensors (backward only)
     float scale, scale_log2;
+    unsigned long long* trace;                // diagnostic: 16 readings of the 100 MHz clock per workgroup, or NULL
 };
 
 // the additive mask: row (b0, b1) starts at mask + b0 * ms[0] + b1 * ms[1] (a stride of 0 broadcasts), keys contiguous
@@ -54,6 +55,11 @@ __device__ __forceinline__ void static_for_attn(F&& f) {
         f(std::integral_constant<int, I>{});
         static_for_attn<I + 1, N>(f);
     }
+}
+
+// slot 0: start; 1: first tile in LDS; 2 + j: end of key tile j (j < 12); 15: end of the kernel
+__device__ __forceinline__ void trace_stamp(const AttnArgs& a, int slot) {
+    if (a.trace && threadIdx.x == 0) a.trace[16 * (size_t)blockIdx.x + slot] = wall_clock64();
 }
 
 __device__ __forceinline__ int swz_rt(int r) { return ((r >> 2) & 3) | (((r >> 1) & 1) << 2); }
@@ -109,6 +115,14 @@ __device__ __forceinline__ float other_half(float v) {
 __device__ __forceinline__ float cross_half_max(float v) { return fmaxf(v, other_half(v)); }
 __device__ __forceinline__ float cross_half_sum(float v) { return v + other_half(v); }
 
+// Two transpose reads (rows 0..3 and 8..11 of a 16-row step, say) joined into one MFMA operand.
+template <int OFF>
+[[nodiscard]] __device__ __forceinline__ half8 tr_pair(uint32_t lo_addr, uint32_t hi_addr) {
+    const half4v lo = lds_read_tr16_b64<OFF>(lo_addr);
+    const half4v hi = lds_read_tr16_b64<OFF>(hi_addr);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 // The mask values of the 32 keys a lane holds of key tile j in the forward and dQ kernels, as loaded:
 // mk[blk * 4 + g][e] belongs to key 64*j + 32*blk + 8*g + 4*h + e. Whole tiles are read eight bytes at a time (the host
 // checks the alignment); the last, partial tile element by element with the index clamped to the row.
@@ -126,15 +140,19 @@ __device__ __forceinline__ void load_mask_tile(const _Float16* row, int j, int h
 }
 
 __device__ __forceinline__ void decode_block(const AttnArgs& a, int tiles, long long& bid, int& b0, int& b1, int& tile) {
-    // XCD-aware: consecutive tiles of one (batch, head) share K/V (or Q/dO) and should share an L2
-    const long long total = a.total_blocks;
-    const long long xcd = bid % 8, idx = bid / 8;
-    const long long base = total / 8, rem = total % 8;
-    bid = xcd * base + (xcd < rem ? xcd : rem) + idx;
-    tile = (int)(bid % tiles);
-    const long long bh = bid / tiles;
-    b1 = (int)(bh % a.batch1);
-    b0 = (int)(bh / a.batch1);
+    // XCD-aware: consecutive tiles of one (batch, head) share K/V (or Q/dO) and should share an L2. 32-bit arithmetic
+    // (the host checks total_blocks < 2^31): 64-bit divisions are long software sequences, and nothing can be requested
+    // from memory before this is done.
+    const uint32_t total = (uint32_t)a.total_blocks, b = (uint32_t)bid;
+    const uint32_t xcd = b % 8u, idx = b / 8u;
+    const uint32_t base = total / 8u, rem = total % 8u;
+    const uint32_t id = xcd * base + (xcd < rem ? xcd : rem) + idx;
+    const uint32_t bh = id / (uint32_t)tiles;
+    tile = (int)(id - bh * (uint32_t)tiles);
+    const uint32_t hi = bh / (uint32_t)a.batch1;
+    b1 = (int)(bh - hi * (uint32_t)a.batch1);
+    b0 = (int)hi;
+    bid = id;
 }
 
 // One [32 q] x [64 d] fp16 result per wavefront, held transposed (acc[blk][e]: d = 32*blk + 8*(e/4) + 4*(lane/32)
@@ -173,6 +191,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
                                                                         const AttnArgsFor<MASK> a) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     constexpr int STAGE = 2 * kTileBytes;
+    trace_stamp(a, 0);
     long long bid = blockIdx.x;
     int b0, b1, qt;
     decode_block(a, a.q_tiles, bid, b0, b1, qt);
@@ -224,6 +243,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
         if (j + 1 < nk) wait_vm_lgkm0<4>();
         else wait_vm_lgkm0<0>();
         __builtin_amdgcn_s_barrier();
+        if (j == 0) trace_stamp(a, 1);
         // ahead of the refill below, so that waiting for these loads does not wait for the transfers issued after them
         half4v mk[MASK ? 8 : 1];
         if constexpr (MASK) load_mask_tile(mask_row, j, h, a.seq_k, mk);
@@ -335,6 +355,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
             oacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[1][s], pf[s], oacc[1], 0, 0, 0);
         }
         stage = stage + 1 == kFwdStages ? 0 : stage + 1;
+        if (j < 12) trace_stamp(a, 2 + j);
     }
 
     const float l_tot = cross_half_sum(l_run);
@@ -344,6 +365,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_fwd_kernel(const _F
             (m_run + __builtin_amdgcn_logf(l_tot)) * 0.69314718055994530942f;
     __syncthreads();  // all fragment reads of the last tiles are done: the ring becomes staging space
     store_rows_t(oacc, inv, lds + wave * 4096, o_ptr + b0 * a.os[0] + b1 * a.os[1], a.os[2], q0, a.seq_q, lane);
+    trace_stamp(a, 15);
 }
 
 
@@ -366,13 +388,6 @@ constexpr float kLog2e = 1.44269504088896340736f;
     return v;
 }
 
-template <int OFF>
-[[nodiscard]] __device__ __forceinline__ half8 tr_pair(uint32_t lo_addr, uint32_t hi_addr) {
-    const half4v lo = lds_read_tr16_b64<OFF>(lo_addr);
-    const half4v hi = lds_read_tr16_b64<OFF>(hi_addr);
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
 template <bool MASK>
 __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
     const _Float16* __restrict__ q_ptr, const _Float16* __restrict__ k_ptr, const _Float16* __restrict__ v_ptr,
@@ -380,6 +395,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
     _Float16* __restrict__ dq_ptr, float* __restrict__ dvec_ptr, const AttnArgsFor<MASK> a) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     constexpr int STAGE = 2 * kTileBytes;
+    trace_stamp(a, 0);
     long long bid = blockIdx.x;
     int b0, b1, qt;
     decode_block(a, a.q_tiles, bid, b0, b1, qt);
@@ -394,6 +410,22 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
     const _Float16* V = v_ptr + b0 * a.vs[0] + b1 * a.vs[1];
     const _Float16* mask_row = nullptr;
     if constexpr (MASK) mask_row = a.mask + b0 * a.ms[0] + b1 * a.ms[1];
+
+    // the first two K / V tiles are requested before anything else: the row loads below (and the row dots that wait for
+    // them) then run while the tiles are on their way, instead of ahead of them
+    TileDma dma;
+    dma.init(wave, lane);
+    TileFrags fr;
+    fr.init(lane);
+    const uint32_t lds0 = lds_addr(lds);
+    const int nk = a.k_tiles;
+    const int kmax = a.seq_k - 1;
+#pragma unroll
+    for (int s = 0; s < kBwdStages - 1; ++s)
+        if (s < nk) {
+            dma.issue(K, a.ks[2], s * 64, kmax, lds + s * STAGE, wave);
+            dma.issue(V, a.vs[2], s * 64, kmax, lds + s * STAGE + kTileBytes, wave);
+        }
 
     half8 qf[4], dof[4];
     float dsum = 0.f;
@@ -414,20 +446,6 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
     if (lane < 32 && q0 + lane < a.seq_q) dvec_ptr[bh * a.seq_q + q0 + lane] = dvec;
     const float lse2 = lse_ptr[bh * a.seq_q + qrow] * kLog2e;
 
-    TileDma dma;
-    dma.init(wave, lane);
-    TileFrags fr;
-    fr.init(lane);
-    const uint32_t lds0 = lds_addr(lds);
-    const int nk = a.k_tiles;
-    const int kmax = a.seq_k - 1;
-#pragma unroll
-    for (int s = 0; s < kBwdStages - 1; ++s)
-        if (s < nk) {
-            dma.issue(K, a.ks[2], s * 64, kmax, lds + s * STAGE, wave);
-            dma.issue(V, a.vs[2], s * 64, kmax, lds + s * STAGE + kTileBytes, wave);
-        }
-
     floatx16 dqacc[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -439,6 +457,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
         if (j + 1 < nk) wait_vm_lgkm0<4>();
         else wait_vm_lgkm0<0>();
         __builtin_amdgcn_s_barrier();
+        if (j == 0) trace_stamp(a, 1);
         half4v mk[MASK ? 8 : 1];   // ahead of the refill, as in the forward kernel
         if constexpr (MASK) load_mask_tile(mask_row, j, h, a.seq_k, mk);
         if (j + kBwdStages - 1 < nk) {
@@ -482,33 +501,33 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
             ktf[blk][2] = tr_pair<2 * 2048>(kt + fr.trread[blk][0], kt + fr.trread[blk][1]);
             ktf[blk][3] = tr_pair<3 * 2048>(kt + fr.trread[blk][0], kt + fr.trread[blk][1]);
         }
-        const bool ragged = (j + 1) * 64 > a.seq_k;
-        half8 dsf[4];
-        float p[2][16];
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                if constexpr (MASK)
-                    p[blk][e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], a.scale_log2,
-                                                                      (float)mk[blk * 4 + (e >> 2)][e & 3] * kLog2eF) - lse2);
-                else
-                    p[blk][e] = __builtin_amdgcn_exp2f(sacc[blk][e] * a.scale_log2 - lse2);
-            }
-        if (ragged) {
-            asm volatile("");   // a real branch: see the forward kernel
+        // only a last, partial tile has keys to take out: their scores become -inf in a branch of its own, ahead of the
+        // exponentials (the empty statement keeps the compiler from turning the branch into 32 compare-and-select
+        // pairs that every tile would pay for)
+        if ((j + 1) * 64 > a.seq_k) {
+            asm volatile("");
 #pragma unroll
             for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int key = j * 64 + blk * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-                    if (key >= a.seq_k) p[blk][e] = 0.f;
+                    if (key >= a.seq_k) sacc[blk][e] = -INFINITY;
                 }
         }
+        // dS^T = P^T * (dP^T - D), P^T recomputed from the scores
+        half8 dsf[4];
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) dsf[blk * 2 + (e >> 3)][e & 7] = (_Float16)(p[blk][e] * (pacc[blk][e] - dvec));
+            for (int e = 0; e < 16; ++e) {
+                float p;
+                if constexpr (MASK)
+                    p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], a.scale_log2,
+                                                              (float)mk[blk * 4 + (e >> 2)][e & 3] * kLog2eF) - lse2);
+                else
+                    p = __builtin_amdgcn_exp2f(sacc[blk][e] * a.scale_log2 - lse2);
+                dsf[blk * 2 + (e >> 3)][e & 7] = (_Float16)(p * (pacc[blk][e] - dvec));
+            }
         wait_lgkm<0>();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -517,9 +536,11 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dq_kernel(
             dqacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ktf[1][s], dsf[s], dqacc[1], 0, 0, 0);
         }
         stage = stage + 1 == kBwdStages ? 0 : stage + 1;
+        if (j < 12) trace_stamp(a, 2 + j);
     }
     __syncthreads();
     store_rows_t(dqacc, a.scale, lds + wave * 4096, dq_ptr + b0 * a.dqs[0] + b1 * a.dqs[1], a.dqs[2], q0, a.seq_q, lane);
+    trace_stamp(a, 15);
 }
 
 template <bool MASK>
@@ -529,6 +550,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dkv_kernel(
     _Float16* __restrict__ dk_ptr, _Float16* __restrict__ dv_ptr, const AttnArgsFor<MASK> a) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     constexpr int STAGE = 2 * kTileBytes + 512;  // Q tile, dO tile, 64 lse, 64 D
+    trace_stamp(a, 0);
     long long bid = blockIdx.x;
     int b0, b1, ktile;
     decode_block(a, (a.seq_k + 127) / 128, bid, b0, b1, ktile);
@@ -592,9 +614,17 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dkv_kernel(
         if (j + 1 < nq) wait_vm_lgkm0<5>();
         else wait_vm_lgkm0<0>();
         __builtin_amdgcn_s_barrier();
+        if (j == 0) trace_stamp(a, 1);
         if (j + kBwdStages - 1 < nq) issue_tile(j + kBwdStages - 1, stage == 0 ? kBwdStages - 1 : stage - 1);
         const uint32_t qt = lds0 + stage * STAGE, gt = qt + kTileBytes, lt = gt + kTileBytes, dt = lt + 256;
-        const bool ragged = (j + 1) * 64 > a.seq_q;
+        // Only a last, partial tile has query rows to take out (the transfers re-read the last row for them). Their
+        // log-sum-exp becomes +inf here, which makes their probabilities, and with them their dS, exactly zero: the
+        // arithmetic below carries no test.
+        if ((j + 1) * 64 > a.seq_q) {
+            if (wave == 0 && j * 64 + lane >= a.seq_q)
+                reinterpret_cast<float*>(lds + stage * STAGE + 2 * kTileBytes)[lane] = INFINITY;
+            __syncthreads();
+        }
 
         static_for_attn<0, 2>([&](auto qbc) {
             constexpr int qb = decltype(qbc)::value;
@@ -630,23 +660,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dkv_kernel(
                 qtf[blk][1] = tr_pair<(2 * qb + 1) * 2048>(qt + fr.trread[blk][0], qt + fr.trread[blk][1]);
             }
             half8 pf[2], dsf[2];
-            float p[16];
-#pragma unroll
-            for (int e = 0; e < 16; ++e)
-                p[e] = MASK ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[e], a.scale_log2, mask2) - lv[e >> 2][e & 3] * kLog2e)
-                            : __builtin_amdgcn_exp2f(sacc[e] * a.scale_log2 - lv[e >> 2][e & 3] * kLog2e);
-            if (ragged) {
-                asm volatile("");   // a real branch: see the forward kernel
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int qi = j * 64 + qb * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-                    if (qi >= a.seq_q) p[e] = 0.f;
-                }
-            }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                pf[e >> 3][e & 7] = (_Float16)p[e];
-                dsf[e >> 3][e & 7] = (_Float16)(p[e] * (pacc[e] - dvv[e >> 2][e & 3]));
+                const float p = MASK ? __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[e], a.scale_log2, mask2) - lv[e >> 2][e & 3] * kLog2e)
+                                     : __builtin_amdgcn_exp2f(sacc[e] * a.scale_log2 - lv[e >> 2][e & 3] * kLog2e);
+                pf[e >> 3][e & 7] = (_Float16)p;
+                dsf[e >> 3][e & 7] = (_Float16)(p * (pacc[e] - dvv[e >> 2][e & 3]));
             }
             wait_lgkm<0>();
             __builtin_amdgcn_sched_barrier(0);
@@ -659,13 +678,17 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attention_bwd_dkv_kernel(
             }
         });
         stage = stage + 1 == kBwdStages ? 0 : stage + 1;
+        if (j < 12) trace_stamp(a, 2 + j);
     }
     __syncthreads();
     store_rows_t(dkacc, a.scale, lds + wave * 4096, dk_ptr + b0 * a.dks[0] + b1 * a.dks[1], a.dks[2], k0, a.seq_k, lane);
     store_rows_t(dvacc, 1.0f, lds + wave * 4096, dv_ptr + b0 * a.dvs[0] + b1 * a.dvs[1], a.dvs[2], k0, a.seq_k, lane);
+    trace_stamp(a, 15);
 }
 
 // ---------------------------------------------------------------- host side
+thread_local unsigned long long* g_attn_trace = nullptr;   // per-workgroup clock readings (diagnostic)
+
 int fill_args(const dmlhip_attention_desc* d, const dmlhip_attention_desc* g, AttnArgs& a, const char* what) {
     DML_REQUIRE(d, DMLHIP_ERR_NULL, "%s: NULL descriptor", what);
     DML_REQUIRE(d->head_dim == 64, DMLHIP_ERR_UNSUPPORTED, "%s: head_dim %lld (only 64 is implemented)", what,
@@ -695,6 +718,7 @@ int fill_args(const dmlhip_attention_desc* d, const dmlhip_attention_desc* g, At
     DML_REQUIRE(d->scale > 0.f, DMLHIP_ERR_SHAPE, "%s: the scale must be positive, got %g", what, (double)d->scale);
     a.scale = d->scale;
     a.scale_log2 = d->scale * 1.44269504088896340736f;
+    a.trace = g_attn_trace;
     return 0;
 }
 
@@ -768,6 +792,7 @@ int attention_backward(const dmlhip_attention_desc* d, const dmlhip_attention_de
                            (const _Float16*)d_o, (_Float16*)dq, (float*)workspace, a);
     if (int e = launch_status(what)) return e;
     a.total_blocks = m.total_blocks = dkv_blocks;
+    if (a.trace) a.trace = m.trace = a.trace + 16 * dq_blocks;   // the second kernel's readings follow the first's
     if (mask)
         hipLaunchKernelGGL(attention_bwd_dkv_kernel<true>, (unsigned)dkv_blocks, kAttnThreads,
                            kBwdStages * (2 * kTileBytes + 512), st, (const _Float16*)q, (const _Float16*)k, (const _Float16*)v,
@@ -785,6 +810,8 @@ int attention_backward(const dmlhip_attention_desc* d, const dmlhip_attention_de
 using namespace dml;
 
 extern "C" {
+
+void dmlhip_debug_attention_trace(void* buffer) { g_attn_trace = (unsigned long long*)buffer; }
 
 int dmlhip_attention_f16(const dmlhip_attention_desc* d, const void* q, const void* k, const void* v, void* o, void* lse,
                          void* stream) {

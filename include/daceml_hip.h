@@ -494,6 +494,12 @@ void dmlhip_debug_force_fused_strip(int toh);
  * many output rows per batch as fit LDS, > 0 = at most that many, -2 = the strip kernel; waves: 8 or 16 wavefronts per
  * workgroup. Shapes of which not one row fits LDS run on the strips. Per calling thread. */
 void dmlhip_debug_fused_rolling(int rows, int waves);
+/* Where the attention workgroups' time goes: with a non-NULL buffer (device memory, 16 x 8 bytes per workgroup) thread 0
+ * of every workgroup stores readings of the 100 MHz wall clock: [0] start, [1] first tile in LDS, [2 + j] end of tile j
+ * (j < 12), [15] end. A forward call has batch0 x batch1 x ceil(seq_q / 128) workgroups; a backward call writes the
+ * readings of its first kernel (dQ, as many workgroups as forward) and behind them those of the second (dK / dV:
+ * batch0 x batch1 x ceil(seq_k / 128) workgroups). NULL (default) = off. Per calling thread. */
+void dmlhip_debug_attention_trace(void* buffer);
 
 #ifdef __cplusplus
 }

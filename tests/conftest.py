@@ -47,3 +47,4 @@ def _reset_diagnostic_switches():
         lib.dmlhip_debug_force_fused_strip(0)
         lib.dmlhip_debug_fused_rolling(0, 8)
         lib.dmlhip_debug_gemm_trace(None)
+        lib.dmlhip_debug_attention_trace(None)
