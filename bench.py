@@ -165,6 +165,48 @@ def _time_program(prog, steps, warmup, graph=False):
     return (time.perf_counter() - t0) / steps * 1e3
 
 
+def attention_trace(device):
+    """Where the fused-attention workgroups' time goes on the benchmarked shape ([8, 16, 512, 64] as head-split views of
+    [8, 512, 1024]): the library's per-workgroup clock readings (``dmlhip_debug_attention_trace``, 100 MHz wall clock),
+    printed as microseconds after the first workgroup of each kernel started. A diagnostic, not a benchmark line."""
+    import numpy as np
+    import torch
+    from daceml_amd import _lib, kernels as K
+    lib = _lib.load()
+    mk = lambda: torch.randn(B, S, HEADS, H // HEADS, device=device).half().permute(0, 2, 1, 3)  # noqa: E731
+    q, k, v, do = mk(), mk(), mk(), mk()
+    scale = 1.0 / float(np.sqrt(H // HEADS))
+    out, lse = K.attention(q, k, v, scale)
+    for _ in range(5):
+        K.attention(q, k, v, scale, out=out)
+        K.attention_backward(q, k, v, out, lse, do, scale)
+    wgs = B * HEADS * S // 128
+    readings = torch.zeros(2 * wgs * 16, dtype=torch.int64, device=device)
+
+    def report(name, t):
+        us = (t.astype(np.float64) - t[:, 0].min()) / 100.0
+        per_tile = np.median(np.diff(us[:, 2:2 + S // 64], axis=1), axis=0)
+        print("%-16s start %.2f (max %.2f) | first tile in LDS %.2f (max %.2f) | first tile done %.2f | further tiles %s | "
+              "end %.2f (max %.2f); workgroups of the first / second launch round end at %.2f / %.2f"
+              % (name, np.median(us[:, 0]), us[:, 0].max(), np.median(us[:, 1]), us[:, 1].max(), np.median(us[:, 2]),
+                 " ".join("%.2f" % x for x in per_tile), np.median(us[:, 15]), us[:, 15].max(),
+                 np.median(us[:256, 15]), np.median(us[256:, 15])))
+
+    lib.dmlhip_debug_attention_trace(readings.data_ptr())
+    try:
+        K.attention(q, k, v, scale, out=out)
+        torch.cuda.synchronize()
+        report("forward", readings.cpu().numpy()[:wgs * 16].reshape(wgs, 16))
+        readings.zero_()
+        K.attention_backward(q, k, v, out, lse, do, scale)
+        torch.cuda.synchronize()
+    finally:
+        lib.dmlhip_debug_attention_trace(None)
+    t = readings.cpu().numpy().reshape(2 * wgs, 16)
+    report("backward, dQ", t[:wgs])
+    report("backward, dK/dV", t[wgs:])
+
+
 def secondary_workload(name, device, steps, warmup, verbose, graph=False, fused_rolling=""):
     """BASELINE.json configs[0..3]: parity-test cases that are also worth a measured line. Same JSON keys as the
     headline; `roofline` is that of the launch that takes the most time."""
@@ -440,6 +482,9 @@ def main():
                     help="ROWS,WAVES: run the fused expand + depthwise convolution with its rolling-window kernel (the "
                          "library's diagnostic switch; ROWS -1 = as many as fit). For comparing kernels, not for the "
                          "reported figure: the JSON line carries the value in config.fused_rolling")
+    ap.add_argument("--attention-trace", action="store_true",
+                    help="print where the fused-attention workgroups' time goes on the benchmarked shape (the library's "
+                         "per-workgroup clock trace) and exit: a diagnostic, no JSON line")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures the single-GPU path only: this build uses one GPU (no collectives, no sharding); "
@@ -457,6 +502,8 @@ def main():
         rows, waves = (int(v) for v in a.fused_rolling.split(","))
         _lib.load().dmlhip_debug_fused_rolling(rows, waves)
 
+    if a.attention_trace:
+        return attention_trace(device)
     if a.workload == "module_bert":
         return module_workload(device, a.steps, a.warmup)
     if a.workload != "bert_fwd_bwd":

@@ -1,6 +1,7 @@
-"""Compile tests/cabi/gemm_from_cpp.cpp against the public header and the built library.
+"""Compile tests/cabi/gemm_from_cpp.cpp against the public header and the built library, and the stand-alone measurement
+program tests/cabi/simd_issue_probe.hip (no library: what one SIMD does with MFMA / vector / LDS instruction mixes).
 
-Usage: ``python tests/cabi/build.py``. The executable is written next to the source (git-ignored)."""
+Usage: ``python tests/cabi/build.py``. The executables are written next to the sources (git-ignored)."""
 import os
 import subprocess
 import sys
@@ -23,6 +24,17 @@ def build() -> str:
     return EXE
 
 
+def build_probe() -> str:
+    exe = os.path.join(HERE, "simd_issue_probe")
+    cmd = ["hipcc", "-O3", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-Wno-unused-command-line-argument", os.path.join(HERE, "simd_issue_probe.hip"), "-o", exe]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("compiling simd_issue_probe.hip failed:\n%s" % res.stderr[-4000:])
+    return exe
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_probe())
     sys.exit(0)

@@ -28,3 +28,8 @@ def test_product_from_cpp(shape, layouts):
                          timeout=100)
     assert res.returncode == 0, res.stdout + res.stderr
     assert "check: 0 of 2000" in res.stdout
+
+
+def test_the_measurement_program_compiles():
+    """tests/cabi/simd_issue_probe.hip (instruction-issue measurements quoted in the design notes) keeps building."""
+    assert os.path.exists(B.build_probe())
