@@ -163,25 +163,32 @@ __device__ __forceinline__ float sigmoid_epilogue_f(float x) {
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * x));
 }
 
-// GELU for fp16 tensors: erf by Abramowitz-Stegun 7.1.26 (absolute error < 1.5e-7, far below the
-// half-precision rounding of the result) on the hardware exp2 / reciprocal. Not used on fp32 paths.
-__device__ __forceinline__ float gelu_half_f(float x) {
-    const float z = fabsf(x) * 0.70710678118654752440f;
-    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
-    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
-    const float e = 1.0f - poly * __builtin_amdgcn_exp2f(-z * z * 1.44269504088896340736f);
-    return 0.5f * x * (1.0f + copysignf(e, x));
+// GELU and its derivative for fp16 tensors (not used on fp32 paths). With cdf the standard normal distribution function,
+//     tail(x) = cdf(-|x|) = erfc(|x| / sqrt 2) / 2 = q(t) exp(-x^2 / 2),   t = 1 / (1 + 0.3275911 |x| / sqrt 2)
+// by Abramowitz-Stegun 7.1.26 with halved coefficients (absolute error < 0.8e-7, far below the half-precision rounding
+// of the results) on the hardware reciprocal and exp2, and
+//     x cdf(x)          = max(x, 0) - |x| tail(x)                      (no cancellation for negative x)
+//     cdf(x) + x pdf(x) = (x > 0 ? 1 - tail : tail) + x exp(-x^2 / 2) / sqrt(2 pi)
+// Both kernels are bound by vector-instruction issue, so the forms are chosen for the fewest instructions: 12 and 15
+// besides the conversions, two of them (reciprocal, exp2) at half rate.
+__device__ __forceinline__ float gelu_tail_half_f(float x, float& ex) {
+    const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(fabsf(x), 0.3275911f * 0.70710678118654752440f, 1.0f));
+    const float q = t * (0.127414796f + t * (-0.142248368f + t * (0.7107068705f + t * (-0.7265760135f + t * 0.5307027145f))));
+    ex = __builtin_amdgcn_exp2f((x * -0.72134752044448170368f) * x);   // exp(-x^2 / 2)
+    return q * ex;
 }
 
-// Derivative of the exact GELU for fp16 tensors, cdf(x) + x * pdf(x), with the same erf approximation and the
-// hardware exp2 (the result is rounded to 11 bits; the library erff + expf make the kernel compute bound).
+__device__ __forceinline__ float gelu_half_f(float x) {
+    float ex;
+    const float tail = gelu_tail_half_f(x, ex);
+    return __builtin_fmaf(-fabsf(x), tail, fmaxf(x, 0.f));
+}
+
 __device__ __forceinline__ float gelu_grad_half_f(float x) {
-    const float z = fabsf(x) * 0.70710678118654752440f;
-    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
-    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
-    const float ex = __builtin_amdgcn_exp2f(-z * z * 1.44269504088896340736f);  // exp(-x^2 / 2)
-    const float cdf = 0.5f * (1.0f + copysignf(1.0f - poly * ex, x));
-    return cdf + x * 0.39894228040143267794f * ex;
+    float ex;
+    const float tail = gelu_tail_half_f(x, ex);
+    const float cdf = x > 0.f ? 1.0f - tail : tail;
+    return __builtin_fmaf(x * 0.39894228040143267794f, ex, cdf);
 }
 
 __device__ __forceinline__ float apply_act_half(int act, float v) {
