@@ -54,18 +54,23 @@ int main(int argc, char** argv) {
     std::normal_distribution<float> nd(0.f, 1.f);
     for (auto& v : ha) v = (_Float16)nd(rng);
     for (auto& v : hb) v = (_Float16)(nd(rng) * 0.05f);
+    // GEMM_PITCH_PAD=<elements> in the environment: the operands' rows are that much longer than their contents (what a
+    // pitch that is not a power of two does to the time of a launch)
+    const long pad = std::getenv("GEMM_PITCH_PAD") ? std::atol(std::getenv("GEMM_PITCH_PAD")) : 0;
+    const long a_rows = al == 'k' ? M : K, a_cols = al == 'k' ? K : M, b_rows = bl == 'k' ? N : K, b_cols = bl == 'k' ? K : N;
+    const long a_pitch = a_cols + pad, b_pitch = b_cols + pad;
     _Float16 *a, *b, *c;
-    PROBE_CHECK(hipMalloc(&a, ha.size() * 2));
-    PROBE_CHECK(hipMalloc(&b, hb.size() * 2));
+    PROBE_CHECK(hipMalloc(&a, (size_t)a_rows * a_pitch * 2));
+    PROBE_CHECK(hipMalloc(&b, (size_t)b_rows * b_pitch * 2));
     PROBE_CHECK(hipMalloc(&c, (size_t)M * N * 2));
-    PROBE_CHECK(hipMemcpy(a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
-    PROBE_CHECK(hipMemcpy(b, hb.data(), hb.size() * 2, hipMemcpyHostToDevice));
+    PROBE_CHECK(hipMemcpy2D(a, a_pitch * 2, ha.data(), a_cols * 2, a_cols * 2, a_rows, hipMemcpyHostToDevice));
+    PROBE_CHECK(hipMemcpy2D(b, b_pitch * 2, hb.data(), b_cols * 2, b_cols * 2, b_rows, hipMemcpyHostToDevice));
     dmlhip_gemm_desc d;
     std::memset(&d, 0, sizeof d);
     d.m = M; d.n = N; d.k = K;
     d.batch[0] = d.batch[1] = d.batch[2] = 1;
-    if (al == 'k') { d.a_stride_m = K; d.a_stride_k = 1; } else { d.a_stride_m = 1; d.a_stride_k = M; }
-    if (bl == 'k') { d.b_stride_n = K; d.b_stride_k = 1; } else { d.b_stride_n = 1; d.b_stride_k = N; }
+    if (al == 'k') { d.a_stride_m = a_pitch; d.a_stride_k = 1; } else { d.a_stride_m = 1; d.a_stride_k = a_pitch; }
+    if (bl == 'k') { d.b_stride_n = b_pitch; d.b_stride_k = 1; } else { d.b_stride_n = 1; d.b_stride_k = b_pitch; }
     d.c_stride_m = N;
     d.alpha = 1.f;
     d.out_dtype = DMLHIP_F16;
