@@ -5,6 +5,7 @@ kernel wrapper raises, there is no eager / CPU fallback.
 """
 import ctypes
 import os
+import sys
 from ctypes import (POINTER, Structure, c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -177,6 +178,13 @@ def load():
         raise HipLibraryMissing(
             "%s not found. Build it with `python -m daceml_amd.csrc.build` (needs hipcc); "
             "this package has no fallback compute path." % LIB_PATH)
+    # A process that uses PyTorch must have PyTorch's HIP runtime loaded before this library, so that both bind to the
+    # same one: loaded the other way round, launches on torch's streams fail with "no ROCm-capable device is detected".
+    if "torch" not in sys.modules:
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
     lib = ctypes.CDLL(LIB_PATH)
     for name, (restype, argtypes) in SIGNATURES.items():
         fn = getattr(lib, name)

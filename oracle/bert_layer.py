@@ -71,23 +71,45 @@ def forward(x: np.ndarray, p: Dict[str, np.ndarray], heads: int, eps: float = 1e
 
 
 def backward(x: np.ndarray, p: Dict[str, np.ndarray], heads: int, dy: np.ndarray, saved: Dict[str, np.ndarray],
-             eps: float = 1e-12) -> Dict[str, np.ndarray]:
-    """Gradients w.r.t. x and every parameter (keys ``x`` and PARAM_NAMES)."""
+             eps: float = 1e-12, term_scales: bool = False) -> Dict[str, np.ndarray]:
+    """Gradients w.r.t. x and every parameter (keys ``x`` and PARAM_NAMES).
+
+    With ``term_scales`` the result also holds, under ``"terms:" + name`` for every parameter, the root of the sum of
+    squares of the terms that gradient element adds up over the batch x sequence rows (``sqrt(sum_a (dout[a, j]
+    inp[a, k])^2)`` for a weight): what a test needs to say how far a sum of rounded terms may be from the exact one.
+    The gradients that leave the attention products (dq, dk, dv) are themselves sums over 512 keys or queries that
+    cancel to a fraction of their terms; where they enter a parameter gradient they count with the root-sum-square of
+    their own terms instead of their value. Not part of the reference's arithmetic."""
     bsz, seq, hidden = x.shape
     d = hidden // heads
     g: Dict[str, np.ndarray] = {}
 
-    def linear_bwd(dout, inp, w, name):
+    def linear_bwd(dout, inp, w, name, dout_scale=None):
         m = dout.reshape(-1, dout.shape[-1])
-        g[name + "_w"] = np.matmul(m.T, inp.reshape(-1, inp.shape[-1]))      # 'aij,aik->jk'
+        i2 = inp.reshape(-1, inp.shape[-1])
+        g[name + "_w"] = np.matmul(m.T, i2)                                   # 'aij,aik->jk'
         g[name + "_b"] = m.sum(axis=0)
+        if term_scales:
+            m2 = m * m if dout_scale is None else np.maximum(m * m, dout_scale.reshape(m.shape) ** 2)
+            g["terms:" + name + "_w"] = np.sqrt(np.matmul(m2.T, i2 * i2))
+            g["terms:" + name + "_b"] = np.sqrt(m2.sum(axis=0))
         return np.matmul(dout, w)                                             # 'aij,jk->aik'
 
+    def layernorm_terms(dout, inp, name):
+        if term_scales:
+            m = dout.reshape(-1, dout.shape[-1])
+            i2 = inp.reshape(-1, inp.shape[-1])
+            xhat = (i2 - i2.mean(axis=1, keepdims=True)) / np.sqrt(i2.var(axis=1, keepdims=True) + eps)
+            g["terms:" + name + "_g"] = np.sqrt(((m * xhat) ** 2).sum(axis=0))
+            g["terms:" + name + "_b"] = np.sqrt((m * m).sum(axis=0))
+
     dres2, g["ln2_g"], g["ln2_b"] = O.layernorm_backward(dy, saved["res2"], p["ln2_g"], eps)
+    layernorm_terms(dy, saved["res2"], "ln2")
     dact = linear_bwd(dres2, saved["act"], p["ffn2_w"], "ffn2")
     dpre = O.gelu_backward(dact, saved["pre"])
     dh1 = O.sum_variadic(dres2, linear_bwd(dpre, saved["h1"], p["ffn1_w"], "ffn1"))
     dres1, g["ln1_g"], g["ln1_b"] = O.layernorm_backward(dh1, saved["res1"], p["ln1_g"], eps)
+    layernorm_terms(dh1, saved["res1"], "ln1")
     dctx2 = linear_bwd(dres1, saved["ctx2"], p["o_w"], "o")
     dctx = O.transpose(dctx2.reshape(bsz, seq, heads, d), [0, 2, 1, 3])
     dprobs = np.matmul(dctx, O.transpose(saved["v"], [0, 1, 3, 2]))
@@ -100,8 +122,18 @@ def backward(x: np.ndarray, p: Dict[str, np.ndarray], heads: int, dy: np.ndarray
     def merge(t):
         return O.transpose(t, [0, 2, 1, 3]).reshape(bsz, seq, hidden)
 
-    dx_q = linear_bwd(merge(dq), x, p["q_w"], "q")
-    dx_k = linear_bwd(merge(dk), x, p["k_w"], "k")
-    dx_v = linear_bwd(merge(dv), x, p["v_w"], "v")
+    sq = sk = sv = None
+    if term_scales:   # root-sum-squares of the terms of dq, dk, dv
+        ds2, pr2 = dscores * dscores, saved["probs"] * saved["probs"]
+        sq = merge(np.sqrt(np.matmul(ds2, saved["k"] ** 2)))
+        sk = merge(np.sqrt(np.matmul(O.transpose(ds2, [0, 1, 3, 2]), saved["q"] ** 2)))
+        sv = merge(np.sqrt(np.matmul(O.transpose(pr2, [0, 1, 3, 2]), dctx * dctx)))
+    dx_q = linear_bwd(merge(dq), x, p["q_w"], "q", sq)
+    dx_k = linear_bwd(merge(dk), x, p["k_w"], "k", sk)
+    dx_v = linear_bwd(merge(dv), x, p["v_w"], "v", sv)
+    if term_scales:
+        # the rows of the probabilities sum to one, so the value bias's gradient is the column sum of dctx itself: the
+        # rounding of one dctx element reaches every dv element of its column, and the sum over them collects it whole
+        g["terms:v_b"] = np.maximum(g["terms:v_b"], np.sqrt((dctx2 * dctx2).reshape(-1, hidden).sum(axis=0)))
     g["x"] = O.sum_variadic(dres1, dx_v, dx_q, dx_k)
     return g

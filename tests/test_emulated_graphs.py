@@ -29,7 +29,7 @@ def _inputs(dtype, seed=1234):
 def _oracle(x, dy, p):
     x64, p64 = x.astype(np.float64), {k: v.astype(np.float64) for k, v in p.items()}
     y, saved = OB.forward(x64, p64, HEADS, eps=1e-5, keep=True)
-    return y, OB.backward(x64, p64, HEADS, dy.astype(np.float64), saved, eps=1e-5)
+    return y, OB.backward(x64, p64, HEADS, dy.astype(np.float64), saved, eps=1e-5, term_scales=True)
 
 
 def _check(arrays, x, dy, p, dtype, grads=True):
@@ -41,7 +41,9 @@ def _check(arrays, x, dy, p, dtype, grads=True):
     assert_close(arrays["gradient_x"], want["x"], dtype, "dx", **({} if f16 else dict(rtol=1e-4, atol=2e-5)))
     for n in OB.PARAM_NAMES:
         scale = float(np.abs(want[n]).max())
-        tol = dict(rtol=2e-2, atol=2e-2 * scale + 1e-3) if f16 else dict(rtol=1e-4, atol=1e-5 * max(scale, 1.0))
+        # fp16: on top of the stated tolerance, what a sum over the rows of products of fp16-stored tensors can be off by
+        tol = dict(rtol=2e-2, atol=1e-2 + 16.0 * 2.0 ** -11 * want["terms:" + n]) if f16 \
+            else dict(rtol=1e-4, atol=1e-5 * max(scale, 1.0))
         assert_close(arrays["gradient_" + n], want[n], dtype, "d" + n, **tol)
 
 

@@ -98,17 +98,20 @@ def test_bert_large_layer_forward_backward():
     x64 = x.astype(np.float64)
     p64 = {k: v.astype(np.float64) for k, v in p.items()}
     y, saved = OB.forward(x64, p64, HEADS, eps=1e-12, keep=True)
-    want = OB.backward(x64, p64, HEADS, dy.astype(np.float64), saved, eps=1e-12)
+    want = OB.backward(x64, p64, HEADS, dy.astype(np.float64), saved, eps=1e-12, term_scales=True)
     del saved
     assert_close(host(args["y"]), y, torch.float16, "y")
     assert_close(host(args["gradient_x"]), want["x"], torch.float16, "gradient_x")
     for n in graphs.BERT_PARAM_NAMES:
-        # fp32 master gradients are sums over 4096 tokens of fp16-rounded values: the absolute floor is the stated
-        # 1e-2, or 2 % of the gradient's scale where that is larger (the key bias has an exactly zero gradient -
-        # softmax is shift invariant - so what is left there is the rounding of the 4096 summed fp16 values)
-        scale = float(np.abs(want[n]).max())
+        # fp32 master gradients are sums over 4096 rows of products of tensors the fp16 path stores rounded to 11 bits
+        # (and that carry the roundings of the stages before them). On top of the stated rtol 2e-2 / atol 1e-2 an
+        # element is allowed what such a sum can be off by: 16 x 2^-11 x the root of the sum of squares of its exact
+        # terms (measured on MI355X: at most 8.3 x 2^-11 x that root over all 16 gradients, the rtol term aside).
+        # Against one absolute tolerance per tensor (2 % of its largest element: 2.4 for the FFN weights) this is
+        # 0.01 + 0.18 at their median element. The key bias has an exactly zero gradient - softmax is shift
+        # invariant - and is held to what the rounding of its 4096 summed values leaves.
         assert_close(host(args["gradient_" + n]), want[n], torch.float16, "gradient_" + n, rtol=2e-2,
-                     atol=max(1e-2, 2e-2 * scale))
+                     atol=1e-2 + 16.0 * 2.0 ** -11 * want["terms:" + n])
     # a second step on the same buffers reproduces the first bit for bit (no atomics, fixed summation orders)
     first = {k: v.clone() for k, v in args.items() if k == "y" or k.startswith("gradient_") and k != "gradient_y"}
     prog.launch()

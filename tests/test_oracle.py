@@ -575,3 +575,59 @@ def test_batchnorm_matches_torch_running_stats_and_autograd():
     np.testing.assert_allclose(y1.var(axis=(0, 2, 3)), 1.0, rtol=1e-12)
     yc = O.batchnorm_training(np.full((2, c, 3, 3), 7.0), scale, b, rm, rv, 1e-5, 0.9)[0]
     np.testing.assert_allclose(yc, np.broadcast_to(b.reshape(1, c, 1, 1), yc.shape), atol=1e-12)
+
+
+def _dres1_of(OB, x, p, dy, saved):
+    """The gradient that reaches the output projection of the attention block (steps of OB.backward, restated)."""
+    dres2, _, _ = O.layernorm_backward(dy, saved["res2"], p["ln2_g"], 1e-12)
+    dact = np.matmul(dres2, p["ffn2_w"])
+    dpre = O.gelu_backward(dact, saved["pre"])
+    dh1 = dres2 + np.matmul(dpre, p["ffn1_w"])
+    return O.layernorm_backward(dh1, saved["res1"], p["ln1_g"], 1e-12)[0]
+
+
+def test_bert_layer_term_scales_are_the_root_sum_squares_of_the_summed_terms():
+    """``backward(..., term_scales=True)``: for every parameter, the root of the sum over the batch x sequence rows of the
+    squared terms its gradient adds up, recomputed here with explicit loops over the rows (weights: dout[a, j] inp[a, k];
+    biases: dout[a, j]; LayerNorm scale: dout[a, j] xhat[a, j]). The gradients themselves must be unchanged by the flag,
+    and no sum of n terms exceeds sqrt(n) times that root (Cauchy-Schwarz)."""
+    from oracle import bert_layer as OB
+    r = np.random.default_rng(77)
+    x = r.standard_normal((2, 6, 16))
+    dy = r.standard_normal((2, 6, 16))
+    p = OB.init_params(16, 32, 5, np.float64, bias_std=0.1)
+    y, saved = OB.forward(x, p, 2, keep=True)
+    plain = OB.backward(x, p, 2, dy, saved)
+    g = OB.backward(x, p, 2, dy, saved, term_scales=True)
+    rows = 12
+    for n in OB.PARAM_NAMES:
+        assert np.array_equal(g[n], plain[n]), n
+        assert (np.abs(g[n]) <= np.sqrt(rows) * g["terms:" + n] * (1 + 1e-12) + 1e-300).all(), n
+    # dv counts with the root-sum-square of its own 6 terms per element where it enters the value projection's gradients
+    dctx = np.matmul(_dres1_of(OB, x, p, dy, saved), p["o_w"]).reshape(2, 6, 2, 8).transpose(0, 2, 1, 3)
+    sv = np.zeros((2, 2, 6, 8))
+    for q in range(6):
+        sv += (saved["probs"][:, :, q, :, None] * dctx[:, :, q, None, :]) ** 2
+    sv = np.sqrt(sv).transpose(0, 2, 1, 3).reshape(rows, 16)
+    dv = np.matmul(saved["probs"].transpose(0, 1, 3, 2), dctx).transpose(0, 2, 1, 3).reshape(rows, 16)
+    dctx_rows = dctx.transpose(0, 2, 1, 3).reshape(rows, 16)
+    np.testing.assert_allclose(g["terms:v_b"], np.maximum(np.sqrt(np.maximum(dv ** 2, sv ** 2).sum(axis=0)),
+                                                          np.sqrt((dctx_rows ** 2).sum(axis=0))), rtol=1e-10)
+    np.testing.assert_allclose(g["v_b"], dctx_rows.sum(axis=0), rtol=1e-9, atol=1e-12)   # sum_k P[q, k] = 1
+    # the output projection's weight and bias, and the second LayerNorm, term by term
+    dres2, _, _ = O.layernorm_backward(dy, saved["res2"], p["ln2_g"], 1e-12)
+    m, inp = dres2.reshape(rows, 16), saved["act"].reshape(rows, 32)
+    want_w = np.zeros((16, 32))
+    want_b = np.zeros(16)
+    for a in range(rows):
+        want_w += np.outer(m[a], inp[a]) ** 2
+        want_b += m[a] ** 2
+    np.testing.assert_allclose(g["terms:ffn2_w"], np.sqrt(want_w), rtol=1e-12)
+    np.testing.assert_allclose(g["terms:ffn2_b"], np.sqrt(want_b), rtol=1e-12)
+    res = saved["res2"].reshape(rows, 16)
+    xhat = (res - res.mean(axis=1, keepdims=True)) / np.sqrt(res.var(axis=1, keepdims=True) + 1e-12)
+    want_g = np.zeros(16)
+    for a in range(rows):
+        want_g += (dy.reshape(rows, 16)[a] * xhat[a]) ** 2
+    np.testing.assert_allclose(g["terms:ln2_g"], np.sqrt(want_g), rtol=1e-12)
+    np.testing.assert_allclose(g["terms:ln2_b"], np.sqrt((dy.reshape(rows, 16) ** 2).sum(axis=0)), rtol=1e-12)

@@ -38,8 +38,9 @@ def _layernorm_training_data():
 
 def _check_layernorm_gradients(dx, dg, db, want):
     assert_close(dx, want[0], torch.float16, "dx")
-    assert_close(dg, want[1], torch.float16, "dgamma", atol=max(1e-2, 2e-2 * float(np.abs(want[1]).max())))
-    assert_close(db, want[2], torch.float16, "dbeta", atol=max(1e-2, 2e-2 * float(np.abs(want[2]).max())))
+    # sums of 240 exact fp16 products in fp32, rounded once to fp16: the stated tolerance as it stands
+    assert_close(dg, want[1], torch.float16, "dgamma")
+    assert_close(db, want[2], torch.float16, "dbeta")
 
 
 def test_layernorm_scale_and_shift_gradients_in_fp16_lower_correctly():

@@ -54,9 +54,9 @@ def _case(lib, rows, cols, seed):
     want_dx, want_dg, want_db = O.layernorm_backward(host(dy).astype(np.float64), host(x).astype(np.float64),
                                                      host(gamma).astype(np.float64), 1e-5)
     assert_close(host(dx1), want_dx, torch.float16, "dx %d x %d" % (rows, cols))
-    scale = float(np.abs(want_dg).max())
-    assert_close(host(dg1), want_dg, torch.float16, "dgamma", atol=max(1e-2, 2e-2 * scale))
-    assert_close(host(db1), want_db, torch.float16, "dbeta", atol=max(1e-2, 2e-2 * float(np.abs(want_db).max())))
+    # fp32 sums over the rows of products of the given fp16 values: the stated tolerance as it stands
+    assert_close(host(dg1), want_dg, torch.float16, "dgamma")
+    assert_close(host(db1), want_db, torch.float16, "dbeta")
 
 
 def test_no_allocation_entry_point_matches_the_workspace_one(lib):

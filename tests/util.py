@@ -38,5 +38,6 @@ def assert_close(got, want, dtype, what="", rtol=None, atol=None):
     bad = err > bound
     if bad.any():
         i = np.unravel_index(np.argmax(err - bound), err.shape)
+        a_here = float(np.broadcast_to(np.asarray(atol, dtype=np.float64), err.shape)[i])   # atol may be per element
         raise AssertionError("%s: %d / %d elements out of tolerance (rtol=%g atol=%g); worst at %s: got %r want %r"
-                             % (what, bad.sum(), bad.size, rtol, atol, i, got[i], want[i]))
+                             % (what, bad.sum(), bad.size, rtol, a_here, i, got[i], want[i]))
