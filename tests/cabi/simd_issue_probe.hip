@@ -7,7 +7,9 @@
 //           an exponential cost;
 //   part 2: the LDS fragment reads and MFMAs of one 64-key attention tile (8 ds_read_b128 of K rows, 16
 //           ds_read_b64_tr_b16 of V^T, 8 + 8 MFMAs) without the softmax arithmetic. The reads are plain LDS loads and the
-//           transpose-read builtin: the compiler places every wait.
+//           transpose-read builtin: the compiler places every wait;
+//   part 3: the instruction mix of one K step of the 128 x 128 GEMM tile (16 MFMAs, 16 or 8 ds_read_b128, 8 or 4
+//           global -> LDS transfers per wavefront) on one wavefront per SIMD.
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -126,6 +128,47 @@ __global__ __launch_bounds__(256, 2) void tile_kernel(float* out, int iters, int
     out[blockIdx.x * 256 + threadIdx.x] = sum;
 }
 
+// ---------------------------------------------------------------- part 3
+// The per-K-step instruction mix of the 128 x 128 GEMM tile on one wavefront per SIMD: 16 MFMAs, NREADS ds_read_b128
+// (16 = four wavefronts of 64 x 64 outputs each read their A and B fragments; 8 = what a split of K across the
+// wavefronts would read) and NDMA global -> LDS transfers of 16 bytes per lane (8 = both operands through LDS) from a
+// buffer that stays in L2. Data values do not matter here; every read feeds an MFMA so that nothing is dropped.
+template <int NREADS, int NDMA, bool SHARED>
+__global__ __launch_bounds__(256) void step_kernel(float* out, const _Float16* src, int iters) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < 128 * 1024 / 4; i += 256) ((float*)lds)[i] = (float)(i & 15) * 0.001f;
+    __syncthreads();
+    floatx16 acc[4];
+    for (int t = 0; t < 4; ++t)
+        for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+    const int r = lane & 31, h = lane >> 5;
+    const char* rd = lds + (wave * 32 + r) * 128 + ((h ^ (r & 7)) << 4);
+    // SHARED: every workgroup streams through the same 256 KB, 32 KB per iteration (what a GEMM's L2 does for tiles that
+    // its workgroups share); otherwise through 256 KB of its own (64 MB in all: from the memory-side cache)
+    const _Float16* gsrc = src + (SHARED ? 0 : (size_t)blockIdx.x * (128 * 1024)) + wave * 512 + lane * 8;
+    half8 frag[16];
+    for (int i = 0; i < 16; ++i) frag[i] = *(const half8*)(rd + (i & 7) * 16);
+    for (int it = 0; it < iters; ++it) {
+        const int stage = it & 3;
+        const _Float16* g = gsrc + (size_t)(it & 7) * (16 * 1024);
+        char* dst = lds + stage * 32768 + wave * 1024;
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            acc[m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(frag[m], frag[(m + 5) & 15], acc[m & 3], 0, 0, 0);
+            if (m < NREADS) frag[m] = *(const half8*)(rd + ((stage + 1) & 3) * 32768 + m * 2048);
+            if ((m & 1) == 0 && m / 2 < NDMA)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g + (m / 2) * 2048),
+                                                 (__attribute__((address_space(3))) void*)(dst + (m / 2) * 4096), 16, 0, 0);
+        }
+        __builtin_amdgcn_s_barrier();
+    }
+    float sum = 0.f;
+    for (int t = 0; t < 4; ++t)
+        for (int e = 0; e < 16; ++e) sum += acc[t][e];
+    out[blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
 // ---------------------------------------------------------------- host
 constexpr int kIters = 2000;
 
@@ -157,6 +200,13 @@ int run_tile(const char* name, int blocks, int barrier, float* out) {
                  [&](int iters) { hipLaunchKernelGGL((tile_kernel<MODE>), blocks, 256, 64 * 1024, 0, out, iters, barrier); });
 }
 
+template <int NREADS, int NDMA, bool SHARED = true>
+int run_step(const char* name, float* out, const _Float16* src) {
+    auto kern = step_kernel<NREADS, NDMA, SHARED>;
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) != hipSuccess) return 1;
+    return timed(name, 256, "", [&](int iters) { hipLaunchKernelGGL(kern, 256, 256, 128 * 1024, 0, out, src, iters); });
+}
+
 int main() {
     float* out;
     PROBE_CHECK(hipMalloc(&out, 1024 * 256 * 4));
@@ -178,6 +228,18 @@ int main() {
             bad |= run_tile<1>("16 MFMA", blocks, barrier, out);
             bad |= run_tile<2>("24 LDS reads (+ 1 MFMA)", blocks, barrier, out);
         }
+    _Float16* src;
+    PROBE_CHECK(hipMalloc(&src, (size_t)64 << 20));
+    PROBE_CHECK(hipMemset(src, 0, (size_t)64 << 20));
+    bad |= run_step<0, 0>("step: 16 MFMA", out, src);
+    bad |= run_step<16, 0>("step: + 16 reads", out, src);
+    bad |= run_step<8, 0>("step: + 8 reads", out, src);
+    bad |= run_step<0, 8>("step: + 8 transfers", out, src);
+    bad |= run_step<16, 8>("step: + 16 reads + 8 tr.", out, src);
+    bad |= run_step<8, 8>("step: + 8 reads + 8 tr.", out, src);
+    bad |= run_step<16, 4>("step: + 16 reads + 4 tr.", out, src);
+    bad |= run_step<16, 8, false>("step: 16 r. + 8 tr., own data", out, src);
+    PROBE_CHECK(hipFree(src));
     PROBE_CHECK(hipFree(out));
     return bad;
 }
