@@ -34,7 +34,7 @@ METRIC = "BERT-large encoder layer fp16 fwd+bwd ms/iter at 1 GPU; % MFMA & HBM r
 B, S, H, HEADS, FFN = 8, 512, 1024, 16, 4096
 
 
-def build_program(device, gelu_epilogue=False):
+def build_program(device, gelu_epilogue=False, reuse_transients=True):
     import torch
     from daceml_amd import graphs
     from daceml_amd.autodiff import add_backward_pass
@@ -46,7 +46,7 @@ def build_program(device, gelu_epilogue=False):
     add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + graphs.BERT_PARAM_NAMES,
                       grad_dtypes={n: torch.float32 for n in graphs.BERT_PARAM_NAMES})
     fusion.optimize_backward(sdfg)
-    return CompiledSDFG(sdfg, device=device)
+    return CompiledSDFG(sdfg, device=device, reuse_transients=reuse_transients)
 
 
 def synthetic_inputs(device):
@@ -210,7 +210,7 @@ def attention_trace(device):
     report("backward, dK/dV", t[wgs:])
 
 
-def secondary_workload(name, device, steps, warmup, verbose, graph=False, fused_rolling=""):
+def secondary_workload(name, device, steps, warmup, verbose, graph=False, fused_rolling="", reuse_transients=True):
     """BASELINE.json configs[0..3]: parity-test cases that are also worth a measured line. Same JSON keys as the
     headline; `roofline` is that of the launch that takes the most time."""
     import numpy as np
@@ -289,7 +289,7 @@ def secondary_workload(name, device, steps, warmup, verbose, graph=False, fused_
         what, dtype = "dense Conv 3x3 fp32 X[32,64,56,56] W[64,64,3,3] pad 1, forward + data and weight gradients", "f32"
     else:
         sys.exit("unknown workload %r" % name)
-    prog = CompiledSDFG(sdfg, device=device)
+    prog = CompiledSDFG(sdfg, device=device, reuse_transients=reuse_transients)
     prog(**args)
     ms = _time_program(prog, steps, warmup, graph)
     rows = kernel_breakdown(prog)
@@ -485,6 +485,9 @@ def main():
                     help="ROWS,WAVES: run the fused expand + depthwise convolution with its rolling-window kernel (the "
                          "library's diagnostic switch; ROWS -1 = as many as fit). For comparing kernels, not for the "
                          "reported figure: the JSON line carries the value in config.fused_rolling")
+    ap.add_argument("--own-buffers", action="store_true",
+                    help="give every transient a buffer of its own instead of letting dead ones hand their memory on "
+                         "(for comparing)")
     ap.add_argument("--attention-trace", action="store_true",
                     help="print where the fused-attention workgroups' time goes on the benchmarked shape (the library's "
                          "per-workgroup clock trace) and exit: a diagnostic, no JSON line")
@@ -510,9 +513,10 @@ def main():
     if a.workload == "module_bert":
         return module_workload(device, a.steps, a.warmup)
     if a.workload != "bert_fwd_bwd":
-        return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose, a.graph, a.fused_rolling)
+        return secondary_workload(a.workload, device, a.steps, a.warmup, a.verbose, a.graph, a.fused_rolling,
+                                  reuse_transients=not a.own_buffers)
 
-    prog = build_program(device, a.gelu_epilogue)
+    prog = build_program(device, a.gelu_epilogue, reuse_transients=not a.own_buffers)
     args, x, dy, p = synthetic_inputs(device)
     prog(**args)  # binds pointers, first run
     torch.cuda.synchronize()

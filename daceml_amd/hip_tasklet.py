@@ -106,6 +106,10 @@ class HipTasklet(Node):
         self.flops = int(flops)
         self.bytes_moved = int(bytes_moved)
         self.kind = kind
+        #: {output connector: input connector}: the kernels give the right result when the output is the very buffer of
+        #: that input (same shape, type and layout); a memory planner may then let the output take over the bytes of an
+        #: input that nobody reads afterwards
+        self.in_place: dict = {}
 
 
 class ViewTasklet(Node):

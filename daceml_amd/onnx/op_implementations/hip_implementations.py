@@ -704,7 +704,9 @@ def _make_unary_grad(op_name: str, code: int, doc: str):
             x = in_desc_with_name(node, state, sdfg, "X")
             call = HipCall("dmlhip_unary_backward_" + _SFX[x.dtype],
                            [I32(code), Ptr("X"), Ptr("dY"), Ptr("dX"), I64(x.total_size), F32(0.0), Stream()])
-            return _tasklet(node, state, [call], bytes_moved=3 * _nbytes(x), kind="elementwise_backward")
+            t = _tasklet(node, state, [call], bytes_moved=3 * _nbytes(x), kind="elementwise_backward")
+            t.in_place = {"dX": "dY"}   # every thread reads its elements of dY before it writes the same elements of dX
+            return t
 
     _UnaryGrad.__name__ = "Hip" + op_name
     _UnaryGrad.__doc__ = doc

@@ -19,6 +19,7 @@ import torch
 
 from . import _lib as L
 from . import hip_tasklet as T
+from . import memory_plan
 from .onnx.nodes import ONNXOp
 from .sdfg import SDFG, AccessNode, Array, SDFGState
 
@@ -82,8 +83,17 @@ class CapturedLaunches:
 
 class CompiledSDFG:
     """An expanded SDFG bound to device buffers; call it with the non-transient arrays by name."""
-    def __init__(self, sdfg: SDFG, device: Optional[torch.device] = None, expand: bool = True):
+    def __init__(self, sdfg: SDFG, device: Optional[torch.device] = None, expand: bool = True,
+                 reuse_transients: bool = False):
+        """``reuse_transients``: transients whose lifetimes (first to last node that touches them, in launch order over
+        all states) do not overlap share memory inside one arena, a buffer that dies handing its bytes to the next
+        one that is born. The step then touches fewer distinct bytes between two uses of the same tensor, which is
+        what decides whether the second use finds it in the 256 MB last-level cache. Off by default: after a run the
+        transients of such a program no longer all hold their values (``buffers[name]`` of a dead one shows whatever
+        was written over it)."""
         self.sdfg = sdfg
+        self.reuse_transients = bool(reuse_transients)
+        self.arena_bytes = 0
         self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
         if self.device.type != "cuda":
             raise ValueError("the HIP implementations run on a GPU device; got %s" % self.device)
@@ -97,19 +107,19 @@ class CompiledSDFG:
         self._stream = ctypes.c_void_p(0)
         self._binding = 0                     # bumped whenever a pointer may have changed
         self.buffers: Dict[str, torch.Tensor] = {}
+        # [(state, node)]: the order the kernels are enqueued in
+        self._order = memory_plan.launch_order(sdfg, small_peak=self.reuse_transients)
         self._allocate()
         self._launches: List[_Launch] = []
         ws = 0
-        for state in sdfg.states():
-            for node in state.topological_sort():
-                if isinstance(node, ONNXOp):
-                    raise RuntimeError("unexpanded library node %r" % node)
-                ws = max(ws, getattr(node, "workspace_bytes", 0))
+        for state, node in self._order:
+            if isinstance(node, ONNXOp):
+                raise RuntimeError("unexpanded library node %r" % node)
+            ws = max(ws, getattr(node, "workspace_bytes", 0))
         self._ws_bytes = max(int(ws), 256)
         self._workspace = torch.empty(self._ws_bytes, dtype=torch.uint8, device=self.device)
-        for state in sdfg.states():
-            for node in state.topological_sort():
-                self._bind_node(state, node)
+        for state, node in self._order:
+            self._bind_node(state, node)
         self._refresh()
 
     # -- memory ------------------------------------------------------------
@@ -125,6 +135,17 @@ class CompiledSDFG:
                     raise ValueError("constant %r has shape %s, descriptor says %s" % (name, tuple(t.shape), desc.shape))
                 self.buffers[name] = t
             elif desc.transient:
+                self.buffers[name] = None     # placed below
+        plan = memory_plan.place_transients(self.sdfg, self._order) if self.reuse_transients else {}
+        if plan:
+            self.arena_bytes = max(off + memory_plan.nbytes(self.sdfg.arrays[name]) for name, off in plan.items())
+            self._arena = torch.empty(self.arena_bytes, dtype=torch.uint8, device=self.device)
+        for name in [n for n, t in self.buffers.items() if t is None]:
+            desc = self.sdfg.arrays[name]
+            if name in plan:
+                piece = self._arena[plan[name]:plan[name] + memory_plan.nbytes(desc)]
+                self.buffers[name] = piece.view(desc.dtype).view(desc.shape)
+            else:
                 self.buffers[name] = torch.empty(desc.shape, dtype=desc.dtype, device=self.device)
         for name, t in self.buffers.items():
             self._ptr[name].value = t.data_ptr()

@@ -215,7 +215,8 @@ class DaceModule(nn.Module):
                 hook(sdfg, sdfg)
         self.required_gradients = grads
 
-        compiled = CompiledSDFG(sdfg, device=device)
+        # transients share memory by lifetime (with debug_transients the intermediates are outputs, not transients)
+        compiled = CompiledSDFG(sdfg, device=device, reuse_transients=True)
         self.compiled = compiled
         for hook in self.post_compile_hooks.values():
             hook(compiled)

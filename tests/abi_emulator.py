@@ -555,6 +555,34 @@ def run_sdfg(sdfg, arrays):
     return log
 
 
+def run_sdfg_in_arena(sdfg, arrays):
+    """The whole SDFG as ``CompiledSDFG(reuse_transients=True)`` runs it: the nodes in the order
+    ``memory_plan.launch_order`` chooses, the transients as pieces of one arena at the offsets
+    ``memory_plan.place_transients`` gives them. The arena starts out as NaN bit patterns, so a transient read before it
+    is written, or after another one took over its bytes, shows in the results. Returns (order of node labels, plan,
+    arena bytes)."""
+    import torch
+    from daceml_amd import memory_plan
+    np_dtype = {torch.float16: np.float16, torch.float32: np.float32, torch.int64: np.int64}
+    order = memory_plan.launch_order(sdfg, small_peak=True)
+    plan = memory_plan.place_transients(sdfg, order)
+    total = max([off + memory_plan.nbytes(sdfg.arrays[n]) for n, off in plan.items()] + [0])
+    arena = np.full(total, 0xFF, dtype=np.uint8)
+    for name, off in plan.items():
+        d = sdfg.arrays[name]
+        arrays[name] = arena[off:off + memory_plan.nbytes(d)].view(np_dtype[d.dtype]).reshape(d.shape)
+    ws = max([int(getattr(n, "workspace_bytes", 0)) for _, n in order] + [0])
+    em = Emulator(ws)
+    for state, node in order:
+        if not getattr(node, "calls", None):
+            continue
+        bound = {}
+        for e in list(state.in_edges(node)) + list(state.out_edges(node)):
+            bound[e.dst_conn if e.dst is node else e.src_conn] = _memory(sdfg, arrays, e.data.data, np_dtype)
+        em.run(node, bound)
+    return [n.label for _, n in order], plan, total
+
+
 def run_program(program, arrays):
     """Run a lowered TaskletProgram (daceml_amd/lowering.py): `arrays` maps the program's array names to NumPy arrays
     (arguments given; transients, constants and missing outputs are allocated here). Connectors address their array

@@ -87,7 +87,8 @@ def test_bert_large_layer_forward_backward():
     add_backward_pass(sdfg, sdfg.states()[0], ["y"], ["x"] + graphs.BERT_PARAM_NAMES,
                       grad_dtypes={n: torch.float32 for n in graphs.BERT_PARAM_NAMES})
     fusion.optimize_backward(sdfg)
-    prog = CompiledSDFG(sdfg)
+    prog = CompiledSDFG(sdfg, reuse_transients=True)
+    assert prog.arena_bytes < 135e6     # 252 MB of transients, placed by lifetime
     args = {"x": dev(x), "gradient_y": dev(dy), "y": torch.empty((B, S, H), dtype=torch.float16, device="cuda"),
             "gradient_x": torch.empty((B, S, H), dtype=torch.float16, device="cuda")}
     for n in graphs.BERT_PARAM_NAMES:
@@ -118,6 +119,15 @@ def test_bert_large_layer_forward_backward():
     torch.cuda.synchronize()
     for k, v in first.items():
         assert torch.equal(v, args[k]), "%s differs between two identical steps" % k
+    # and so does the same graph with a buffer of its own for every transient, in the plain topological order
+    del prog
+    plain = CompiledSDFG(sdfg)
+    for k in first:
+        args[k].zero_()
+    plain(**args)
+    torch.cuda.synchronize()
+    for k, v in first.items():
+        assert torch.equal(v, args[k]), "%s differs between the arena and separate buffers" % k
 
 
 def test_mbconv_block_config_shape():

@@ -25,9 +25,9 @@ def _bert_inputs(b, s, h, ffn, dtype, seed=1234, bias_std=0.02):
     return x.astype(npdt), p
 
 
-def _compile(sdfg):
+def _compile(sdfg, reuse_transients=False):
     from daceml_amd.runtime import CompiledSDFG
-    return CompiledSDFG(sdfg)
+    return CompiledSDFG(sdfg, reuse_transients=reuse_transients)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
@@ -63,8 +63,11 @@ def test_bert_layer_forward(dtype, fused):
         assert_close(host(y), want, dtype, "bert layer forward fused=%s" % fused, rtol=1e-4, atol=2e-5)
 
 
+@pytest.mark.parametrize("reuse", [False, True], ids=["own_buffers", "arena"])
 @pytest.mark.parametrize("dtype,attention", [(torch.float16, True), (torch.float16, False), (torch.float32, False)])
-def test_bert_layer_backward(dtype, attention):
+def test_bert_layer_backward(dtype, attention, reuse):
+    """``reuse``: the transients share one arena by lifetime (and the launch order is the one chosen for a small memory
+    peak), as in the benchmarked program."""
     from daceml_amd import graphs
     from daceml_amd.autodiff import add_backward_pass
     from daceml_amd.transformation import fusion
@@ -86,7 +89,10 @@ def test_bert_layer_backward(dtype, attention):
         assert bnames == {"FusedEinsum", "SoftmaxGrad", "LayerNormalizationGrad", "GeluGrad", "ReduceSum", "Sum"}
     n_grouped = sum(n.schema.name in ("GroupedEinsum", "EinsumSum") or "InputSum" in n.out_connectors
                     for st in sdfg.states() for n in st.library_nodes())
-    prog = _compile(sdfg)   # expands the library nodes in place
+    prog = _compile(sdfg, reuse)   # expands the library nodes in place
+    if reuse:
+        own = sum(t.numel() * t.element_size() for n, t in prog.buffers.items() if sdfg.arrays[n].transient)
+        assert 0 < prog.arena_bytes < 0.7 * own
     args = {"x": dev(x), "y": torch.empty((b, s, h), dtype=dtype, device="cuda"), "gradient_y": dev(dy)}
     args.update({k: dev(v) for k, v in p.items()})
     out = {"gradient_x": torch.empty((b, s, h), dtype=dtype, device="cuda")}
