@@ -205,12 +205,10 @@ class DaceModule(nn.Module):
             # gradients for every input that is not a buffer or skipped, and every parameter that requires one
             # (module.py:333-346)
             required = self._inputs_that_need_gradients(model)
-            # parameter gradients are accumulated and stored in fp32 also for fp16 parameters (the reductions over
-            # the batch run in fp32 anyway); autograd receives them cast to the parameter's type
-            master = {clean_onnx_name(n): torch.float32 for n in required
-                      if n in params and params[n].dtype == torch.float16}
-            grads = add_backward_pass(sdfg, state, list(model.outputs), [clean_onnx_name(n) for n in required],
-                                      grad_dtypes=master)
+            # a parameter's gradient has the parameter's type, as autograd expects it: the kernels sum over the batch
+            # in fp32 and round once when they store (fp32 copies that autograd would get cast anyway cost one more
+            # launch per parameter)
+            grads = add_backward_pass(sdfg, state, list(model.outputs), [clean_onnx_name(n) for n in required])
             for hook in self.post_autodiff_hooks.values():
                 hook(sdfg, sdfg)
         self.required_gradients = grads
