@@ -165,9 +165,10 @@ __global__ __launch_bounds__(kEwBlock) void binary_general_kernel(const T* __res
 }
 
 // ------------------------------------------------------------------ unary
+// y may be the very buffer of dy (the gradient written over the gradient it was computed from: a thread reads its
+// elements before it writes them, and no other thread touches them), so these two carry no __restrict__.
 template <typename T, int OP, bool GRAD>
-__global__ __launch_bounds__(kEwBlock) void unary_kernel(const T* __restrict__ x, const T* __restrict__ dy,
-                                                         T* __restrict__ y, int64_t n, float p) {
+__global__ __launch_bounds__(kEwBlock) void unary_kernel(const T* __restrict__ x, const T* dy, T* y, int64_t n, float p) {
     using V = typename VecOf<T>::type;
     constexpr int VN = VecOf<T>::n;
     const int64_t nvec = n / VN;

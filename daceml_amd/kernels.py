@@ -242,10 +242,16 @@ def unary(op: int, x: torch.Tensor, param: float = 0.0, out: Optional[torch.Tens
     return y
 
 
-def unary_backward(op: int, x: torch.Tensor, dy: torch.Tensor, param: float = 0.0) -> torch.Tensor:
+def unary_backward(op: int, x: torch.Tensor, dy: torch.Tensor, param: float = 0.0,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out`` may be ``dy`` itself (the gradient is then written over the one it was computed from)."""
     _check(x, dy, dtype=x.dtype)
     x, dy = _dense(x), _dense(dy)
-    dx = torch.empty_like(x)
+    dx = torch.empty_like(x) if out is None else out
+    if out is not None:
+        _check(x, out, dtype=x.dtype)
+        if not out.is_contiguous():
+            raise ValueError("out must be dense")
     L.check(_fn("unary_backward", x.dtype)(op, _ptr(x), _ptr(dy), _ptr(dx), x.numel(), float(param), _stream()))
     return dx
 

@@ -136,7 +136,8 @@ int dmlhip_unary_f16(int op, const void* x, void* y, int64_t n, float param, voi
 int dmlhip_unary_f32(int op, const void* x, void* y, int64_t n, float param, void* stream);
 
 /* Backward of the unary maps above: dx = dy * f'(x), x being the forward *input* (the derivative the SymPy
- * tasklet reversal of autodiff/backward_pass_generator.py:1284-1421 writes for each of these maps). */
+ * tasklet reversal of autodiff/backward_pass_generator.py:1284-1421 writes for each of these maps). dx may be the
+ * very buffer of dy (not a shifted or partial overlap of it, and not x). */
 int dmlhip_unary_backward_f16(int op, const void* x, const void* dy, void* dx, int64_t n,
                               float param, void* stream);
 int dmlhip_unary_backward_f32(int op, const void* x, const void* dy, void* dx, int64_t n,

@@ -287,6 +287,23 @@ def test_unary_backward(dtype, name):
     f(t).backward(torch.tensor(dy64))
     got = K.unary_backward(getattr(L, name.upper()), dev(x), dev(dy))
     assert_close(host(got), t.grad.numpy(), dtype, name + " backward")
+    # written over the gradient it is computed from (what the executor's memory plan lets this node do): same bits
+    d = dev(dy)
+    assert K.unary_backward(getattr(L, name.upper()), dev(x), d, out=d) is d
+    assert torch.equal(d, got)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_unary_backward_in_place_on_a_streaming_size(dtype):
+    """16.8 M elements (the Gelu gradient of the benchmarked layer): several workgroup rounds, grid-stride loop."""
+    from daceml_amd import _lib as L, kernels as K
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(8 * 512 * 4096 + 3, device="cuda", generator=g).to(dtype)
+    dy = torch.randn(8 * 512 * 4096 + 3, device="cuda", generator=g).to(dtype)
+    want = K.unary_backward(L.GELU, x, dy)
+    d = dy.clone()
+    K.unary_backward(L.GELU, x, d, out=d)
+    assert torch.equal(d, want)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
