@@ -97,14 +97,17 @@ def lifetimes(sdfg: SDFG, order) -> Tuple[Dict[str, int], Dict[str, int]]:
     return first, last
 
 
-def place_transients(sdfg: SDFG, order, align: int = 256) -> Dict[str, int]:
+def place_transients(sdfg: SDFG, order, align: int = 256, leave_out=()) -> Dict[str, int]:
     """Byte offsets in one arena for the transients, from their lifetimes in ``order``. A node's outputs are placed
     before its inputs are released, so no kernel reads and writes the same bytes under two names - unless the node says
     it may (``in_place``: {output connector: input connector}): then an output born at the node takes over the bytes of
     that input if the input dies there, has the same size and is connected to the node once. Among the free blocks that
     fit, the one released last is taken: its lines are the ones most likely to be in cache still. Arrays that no node
-    touches are left out (the caller gives them a buffer of their own)."""
+    touches, and those named in ``leave_out``, get no place (the caller gives them a buffer of their own)."""
     first, last = lifetimes(sdfg, order)
+    for n in leave_out:
+        first.pop(n, None)
+        last.pop(n, None)
     size = {n: max((nbytes(sdfg.arrays[n]) + align - 1) // align * align, align) for n in first}
     free: List[List[int]] = []      # [offset, bytes, position of the release]
     end = 0

@@ -61,6 +61,27 @@ def _replace_node(state: SDFGState, node, new):
     state._nodes.remove(node)
 
 
+def forwarded_transients(sdfg: SDFG, forward_states: Sequence[str], backward_states: Sequence[str]) -> List[str]:
+    """Transient buffers that the forward states write and the backward states touch: the values a pending
+    backward call depends on (what the reference's dispatcher turns into extra forward outputs and saves on the
+    autograd context, daceml/autodiff/torch.py:56-104, ctypes_module.py:150-156)."""
+    def root(name):
+        while sdfg.arrays[name].view_of is not None:
+            name = sdfg.arrays[name].view_of
+        return name
+
+    written, touched = set(), set()
+    for state in sdfg.states():
+        for e in state.edges():
+            r = root(e.data.data)
+            if state.label in forward_states and isinstance(e.dst, AccessNode):
+                written.add(r)
+            if state.label in backward_states:
+                touched.add(r)
+    return [n for n, d in sdfg.arrays.items() if n in written and n in touched and d.transient and d.view_of is None
+            and n not in sdfg.constants]
+
+
 class _Launch:
     __slots__ = ("fn", "args", "label", "symbol", "flops", "bytes_moved", "kind", "state")
 
@@ -84,7 +105,7 @@ class CapturedLaunches:
 class CompiledSDFG:
     """An expanded SDFG bound to device buffers; call it with the non-transient arrays by name."""
     def __init__(self, sdfg: SDFG, device: Optional[torch.device] = None, expand: bool = True,
-                 reuse_transients: bool = False):
+                 reuse_transients: bool = False, outside_arena: Sequence[str] = ()):
         """``reuse_transients``: transients whose lifetimes (first to last node that touches them, in launch order over
         all states) do not overlap share memory inside one arena, a buffer that dies handing its bytes to the next
         one that is born. The step then touches fewer distinct bytes between two uses of the same tensor, which is
@@ -93,6 +114,9 @@ class CompiledSDFG:
         was written over it)."""
         self.sdfg = sdfg
         self.reuse_transients = bool(reuse_transients)
+        #: transients that keep a buffer of their own (a caller that rebinds them to its own memory on every call
+        #: would leave their place in the arena unused)
+        self.outside_arena = tuple(outside_arena)
         self.arena_bytes = 0
         self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
         if self.device.type != "cuda":
@@ -136,7 +160,8 @@ class CompiledSDFG:
                 self.buffers[name] = t
             elif desc.transient:
                 self.buffers[name] = None     # placed below
-        plan = memory_plan.place_transients(self.sdfg, self._order) if self.reuse_transients else {}
+        plan = memory_plan.place_transients(self.sdfg, self._order, leave_out=self.outside_arena) \
+            if self.reuse_transients else {}
         if plan:
             self.arena_bytes = max(off + memory_plan.nbytes(self.sdfg.arrays[name]) for name, off in plan.items())
             self._arena = torch.empty(self.arena_bytes, dtype=torch.uint8, device=self.device)
@@ -261,24 +286,8 @@ class CompiledSDFG:
         self._bind_arguments(tensors, partial=True)
 
     def forwarded_transients(self, forward_states: Sequence[str], backward_states: Sequence[str]) -> List[str]:
-        """Transient buffers that the forward states write and the backward states touch: the values a pending
-        backward call depends on (what the reference's dispatcher turns into extra forward outputs and saves on the
-        autograd context, daceml/autodiff/torch.py:56-104, ctypes_module.py:150-156)."""
-        def root(name):
-            while self.sdfg.arrays[name].view_of is not None:
-                name = self.sdfg.arrays[name].view_of
-            return name
-
-        written, touched = set(), set()
-        for state in self.sdfg.states():
-            for e in state.edges():
-                r = root(e.data.data)
-                if state.label in forward_states and isinstance(e.dst, AccessNode):
-                    written.add(r)
-                if state.label in backward_states:
-                    touched.add(r)
-        return [n for n in self.buffers if n in written and n in touched and self.sdfg.arrays[n].transient and
-                n not in self.sdfg.constants]
+        """See the module-level function."""
+        return forwarded_transients(self.sdfg, forward_states, backward_states)
 
     def rebind_transients(self, tensors: Dict[str, torch.Tensor], release: bool = False):
         """Point transient arrays at caller-provided buffers (same shape and dtype, dense). With ``release`` the

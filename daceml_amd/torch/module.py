@@ -23,7 +23,7 @@ from torch import nn
 
 from ..autodiff import add_backward_pass
 from ..onnx.onnx_importer import ONNXModel, clean_onnx_name
-from ..runtime import CompiledSDFG
+from ..runtime import CompiledSDFG, expand_onnx_nodes, forwarded_transients
 from ..sdfg import AccessNode
 from ..transformation import fusion
 from .export import export_onnx
@@ -213,14 +213,17 @@ class DaceModule(nn.Module):
                 hook(sdfg, sdfg)
         self.required_gradients = grads
 
-        # transients share memory by lifetime (with debug_transients the intermediates are outputs, not transients)
-        compiled = CompiledSDFG(sdfg, device=device, reuse_transients=True)
+        forward_states = [state.label]
+        backward_states = [s.label for s in sdfg.states() if s.label != state.label]
+        # transients share memory by lifetime (with debug_transients the intermediates are outputs, not transients);
+        # those a backward call reads get fresh memory on every forward call (below) and need no place of their own
+        expand_onnx_nodes(sdfg)
+        outside = forwarded_transients(sdfg, forward_states, backward_states) if self.backward else []
+        compiled = CompiledSDFG(sdfg, device=device, reuse_transients=True, outside_arena=outside)
         self.compiled = compiled
         for hook in self.post_compile_hooks.values():
             hook(compiled)
 
-        forward_states = [state.label]
-        backward_states = [s.label for s in sdfg.states() if s.label != state.label]
         in_arrays = [clean_onnx_name(n) for n in tensor_inputs + param_inputs]
         out_arrays = list(model.outputs)
         arglist = compiled.arglist()

@@ -146,3 +146,25 @@ def test_placement_of_random_lifetimes_never_overlaps():
             order = memory_plan.launch_order(sdfg, small_peak=small)
             _check_order(sdfg, order)
             _check_plan(sdfg, order, memory_plan.place_transients(sdfg, order))
+
+
+def test_transients_left_out_get_no_place_and_the_rest_packs_tighter():
+    """What DaceModule does with the buffers a backward call reads: they get fresh memory per forward call, so the arena
+    only holds the others."""
+    from daceml_amd.runtime import forwarded_transients
+    sdfg = _bert_step()
+    fwd, bwd = sdfg.states()[0].label, [s.label for s in sdfg.states()[1:]]
+    kept = forwarded_transients(sdfg, [fwd], bwd)
+    assert "gelu_mulhalf_C_43" in kept and all(sdfg.arrays[n].transient for n in kept)
+    order = memory_plan.launch_order(sdfg, small_peak=True)
+    everything = memory_plan.place_transients(sdfg, order)
+    rest = memory_plan.place_transients(sdfg, order, leave_out=kept)
+    assert set(rest) == set(everything) - set(kept) and rest
+    size = lambda plan: max(off + memory_plan.nbytes(sdfg.arrays[n]) for n, off in plan.items())  # noqa: E731
+    assert size(rest) < 0.5 * size(everything)
+    first, last = memory_plan.lifetimes(sdfg, order)
+    names = sorted(rest)
+    for i, a in enumerate(names):
+        for b in names[i + 1:]:
+            if rest[a] < rest[b] + memory_plan.nbytes(sdfg.arrays[b]) and rest[b] < rest[a] + memory_plan.nbytes(sdfg.arrays[a]):
+                assert last[a] <= first[b] or last[b] <= first[a], (a, b)
