@@ -2,7 +2,8 @@
 forward + autodiff backward through the "hip" library-node implementations, on one MI355X.
 
 Prints ONE JSON line (see the keys below). `value` is ms per forward+backward step with all inputs
-resident in HBM. `roofline` describes the dominant kernel (the fp16 MFMA GEMM): algorithmic FLOPs of
+resident in HBM: W warm-up steps, then exactly K timed steps between two synchronisations; ahead of the warm-up steps
+the program runs untimed for 40 ms so that the GPU's clock has settled under this load (`settle`). `roofline` describes the dominant kernel (the fp16 MFMA GEMM): algorithmic FLOPs of
 all contraction launches of a step divided by their summed HIP-event durations. `hbm_nodes` does the
 same against the HBM roofline for the memory-bound nodes. `cpu_baseline` is the C++ / OpenMP restatement of the
 reference's pure expansions (oracle/bert_layer_loops.cpp) timed on this host, with the NumPy + BLAS form beside it.
@@ -153,11 +154,33 @@ def cpu_baseline(x, dy, p, budget_s=25.0):
                                        "`cores` threads), every other statement on one core" % len(blas)}}
 
 
+SETTLE_MS = 40.0
+
+
+def settle(step, ms=SETTLE_MS):
+    """Untimed steps, ahead of the warm-up steps, until the GPU has been under this load for `ms` of wall time. After
+    an idle stretch (the oracle check on the CPU, a fresh process) the GPU runs its first two or three steps at boost
+    clocks, then about twenty of them 5 - 25 % slower while its power management finds the clock this load sustains; a
+    short warm-up would put that stretch into the timed region (measured: steps 5 - 24 from a cold start average
+    0.589 ms, steps 100 - 199 average 0.547 ms). Returns the number of steps run."""
+    import torch
+    n = 0
+    torch.cuda.synchronize()
+    t_end = time.perf_counter() + ms * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(5):
+            step()
+        n += 5
+        torch.cuda.synchronize()
+    return n
+
+
 # ----------------------------------------------------------------------------- the other configurations
 def _time_program(prog, steps, warmup, graph=False):
     """ms per step; with `graph` the step's launches are replayed from a HIP graph captured once."""
     import torch
     step = prog.capture().replay if graph else prog.launch
+    settle(step)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -437,6 +460,7 @@ def module_workload(device, steps, warmup):
         mod(x).backward(dy)
 
     def timed(mod):
+        settle(lambda: step(mod))
         for _ in range(warmup):
             step(mod)
         torch.cuda.synchronize()
@@ -523,6 +547,7 @@ def main():
     checked = None if a.no_check else check_against_oracle(args, x, dy, p)
     # --graph: the step replayed from a HIP graph (for comparing; the reported configuration launches kernel by kernel)
     step = prog.capture().replay if a.graph else prog.launch
+    settled = settle(step)
     for _ in range(a.warmup):
         step()
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps + 1)]
@@ -601,6 +626,10 @@ def main():
         "hbm_nodes": hbm,
         "sum_of_kernel_ms": round(sum(t for _, t in rows), 4),
         "step_ms": step_stats,
+        "untimed_steps_before_warmup": settled,
+        "untimed_steps_note": "%g ms of untimed steps ahead of the warm-up steps: after an idle stretch the GPU needs "
+                              "about twenty steps to settle on the clock this load sustains" % SETTLE_MS,
+        "transient_arena": {"bytes": prog.arena_bytes, "reuse_transients": prog.reuse_transients},
     }
     if checked is not None:
         out.update(checked)
