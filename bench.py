@@ -27,8 +27,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # scaled by what the same counter reads for the 128 MiB copy kernel of --calibrate-copy (FETCH_SIZE x 2.000,
 # WRITE_SIZE x 1.000). Measured, not computed here: it goes stale when the GEMM tiling changes, so the tile selection
 # it was measured with is part of the value and is compared with the library's at run time.
-GEMM_TRAFFIC_BYTES_PER_STEP = {"fetched": 828.7e6, "written": 184.6e6,
-                               "measured_with": "tile configurations 4 (256x256) / 5 (128x128, four stages) / 9 chosen by "
+GEMM_TRAFFIC_BYTES_PER_STEP = {"fetched": 833.6e6, "written": 184.6e6,
+                               "measured_with": "tile configurations 4 (256x256) / 5 and 7 (128x128, four / two stages) / 9 chosen by "
                                                 "the library, interleaved K loop; profiles/bert_layer_fwd_bwd_hbm_traffic.md"}
 
 METRIC = "BERT-large encoder layer fp16 fwd+bwd ms/iter at 1 GPU; % MFMA & HBM roofline"

@@ -494,6 +494,16 @@ static int run_gemm_f16(const dmlhip_gemm_desc* d, const void* a, const void* b,
                 // few tiles and a long K (1024 x 1024 x 4096: 24 us against 29 - 38 us): the 128 x 64 tile doubles the
                 // workgroups, two of them per compute unit
                 cfg = 9;
+            } else if (d->k <= 1024 && t128 >= 2 * kCus) {
+                // several rounds of short K loops (the grouped q / k / v projections: 768 tiles of 16 steps): with two
+                // LDS stages instead of four, two workgroups share a compute unit and one's epilogue and first loads
+                // overlap the other's loop - 45.3 against 46 - 49 us
+                cfg = 7;
+            } else if (!extra && d->k <= 1024 && t128 <= kCus && residual) {
+                // a short K loop whose epilogue also reads a residual tile (4096 x 1024 x 1024: 20.3 - 21.1 against
+                // 22.9 - 23.2 us): 128 x 64 tiles, two workgroups per compute unit, for the same overlap (without the
+                // residual the two tiles are level: 18.2 us)
+                cfg = 9;
             } else {
                 // one 128 x 128 tile per compute unit, four LDS stages, interleaved loop: 5 - 20 % faster than the plain
                 // loop on every product of the layer with 4096 x 1024 or 1024 x 4096 outputs
