@@ -3,6 +3,7 @@
 #pragma once
 
 #include "common.h"
+#include "lds_ops.h"
 
 #include <type_traits>
 
@@ -215,7 +216,10 @@ __device__ __forceinline__ void store_strip(const GemmArgs& g, void* c_ptr, void
             ovec ov;
 #pragma unroll
             for (int e = 0; e < 8; ++e) ov[e] = (OutT)v[e];
-            *reinterpret_cast<ovec*>(C + off) = ov;
+            // fp16 results (what the next kernel reads) go through the L2 as they are written; the fp32 ones (weight
+            // gradients, read by nobody in the step) measured no faster that way
+            if constexpr (sizeof(OutT) == 2) global_store_b128_through(C + off, ov);
+            else *reinterpret_cast<ovec*>(C + off) = ov;
         }
     } else {
         // ragged or unaligned columns: element by element (rare)

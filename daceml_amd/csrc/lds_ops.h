@@ -47,6 +47,16 @@ template <int OFFSET>
     return v;
 }
 
+// 16 bytes per lane to global memory at agent scope (sc1): the line goes through the L2 to the memory side as it is
+// written instead of staying dirty in the XCD's L2 until the kernel ends. For a result that a kernel writes in one burst
+// at its end (a GEMM tile), the write-back of up to 32 MB of dirty lines between this kernel and the next one goes
+// away. A store of more than 64 bits reads its data registers up to two wait states after it issues, and the compiler's
+// hazard recognizer, which keeps vector writes to those registers away for that long, does not look into inline assembly:
+// the two wait states are part of the statement.
+__device__ __forceinline__ void global_store_b128_through(void* p, half8 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_lgkm() {
     static_assert(N >= 0 && N <= 15, "lgkmcnt is a 4-bit counter");

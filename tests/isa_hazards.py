@@ -114,3 +114,49 @@ def check_file(path):
         if bad:
             found[name] = bad
     return count, found
+
+
+_WIDE_STORE = re.compile(r'^(global|flat|buffer|scratch)_store_(dwordx3|dwordx4|b96|b128)\b')
+_VALU_OR_LOAD = re.compile(r'^(v_|ds_read|ds_bpermute|global_load|flat_load|buffer_load|scratch_load)')
+
+
+def check_store_data(path):
+    """A second hazard of the same kind. A memory store of more than 64 bits reads its data registers up to two wait
+    states after it issues; the compiler's hazard recognizer keeps vector writes to those registers away for that long,
+    but it does not look into inline assembly. Reports, per kernel, every store of more than 64 bits that sits in an
+    inline-assembly block (between #ASMSTART and #ASMEND markers the compiler writes) and is not followed, inside the
+    block, by ``s_nop 1`` or more. Returns {kernel: [line numbers]}."""
+    found = {}
+    name, in_asm, pending = None, False, None
+    with open(path) as f:
+        for ln, line in enumerate(f, 1):
+            s = line.strip()
+            m = re.match(r'^(_Z\w+):', s)
+            if m:
+                name, in_asm, pending = m.group(1), False, None
+                continue
+            if name is None:
+                continue
+            if '#ASMSTART' in s:
+                in_asm, pending = True, None
+                continue
+            if '#ASMEND' in s:
+                if pending is not None:
+                    found.setdefault(name, []).append(pending)
+                in_asm, pending = False, None
+                continue
+            if not in_asm:
+                continue
+            code = s.split(';')[0].strip()
+            if not code:
+                continue
+            if pending is not None:
+                m = re.match(r'^s_nop\s+(\d+)', code)
+                if m and int(m.group(1)) >= 1:
+                    pending = None
+                else:
+                    found.setdefault(name, []).append(pending)
+                    pending = None
+            if _WIDE_STORE.match(code):
+                pending = ln
+    return found

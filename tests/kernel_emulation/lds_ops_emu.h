@@ -41,6 +41,8 @@ inline half4v lds_read_tr16_b64(uint32_t addr) {
     return v;
 }
 
+inline void global_store_b128_through(void* p, half8 v) { *static_cast<half8*>(p) = v; }
+
 template <int N>
 inline void wait_lgkm() {}
 

@@ -69,6 +69,22 @@ def test_interleaved_gemm_loop(tmp_path):
     assert not found, _report(found)
 
 
+def test_wide_stores_in_inline_assembly_carry_their_wait_states(tmp_path):
+    """lds_ops.h stores GEMM results with an inline-assembly ``global_store_dwordx4 ... sc1``; the two wait states the
+    compiler would have kept between such a store and the next write to its data registers are part of the statement."""
+    p = tmp_path / "k.s"
+    p.write_text("_Z1kv:\n\t;;#ASMSTART\n\tglobal_store_dwordx4 v[0:1], v[4:7], off sc1\n\t;;#ASMEND\n"
+                 "\tv_mov_b32_e32 v4, 0\n\ts_endpgm\n")
+    assert isa_hazards.check_store_data(str(p)) == {"_Z1kv": [3]}
+    p.write_text("_Z1kv:\n\t;;#ASMSTART\n\tglobal_store_dwordx4 v[0:1], v[4:7], off sc1\n\ts_nop 1\n\t;;#ASMEND\n"
+                 "\tv_mov_b32_e32 v4, 0\n\ts_endpgm\n")
+    assert isa_hazards.check_store_data(str(p)) == {}
+    asm = _assembly(os.path.join(ROOT, "tests", "isa", "ilv_instances.hip"), tmp_path)
+    text = open(asm).read()
+    assert " sc1" in text, "the GEMM epilogue stores its fp16 results through the L2"
+    assert isa_hazards.check_store_data(asm) == {}
+
+
 def test_dropping_the_value_of_an_lds_read_does_not_compile(tmp_path):
     """The readers of lds_ops.h are [[nodiscard]] and the library's flags turn the warning into an error: the pattern
     behind the register race (a read issued, its value never used) is rejected by the compiler."""
