@@ -2,6 +2,7 @@
 // bias+GELU, Cast. All are one HBM pass with 128-bit accesses on the dense fast paths; any
 // stride pattern falls back to an index-decoding kernel with the same arithmetic.
 #include "common.h"
+#include "lds_ops.h"
 
 namespace dml {
 namespace {
@@ -186,7 +187,10 @@ __global__ __launch_bounds__(kEwBlock) void unary_kernel(const T* __restrict__ x
             else if constexpr (OP == DMLHIP_GELU && sizeof(T) == 2) yv[e] = from_f32<T>(gelu_half_f(to_f32(xv[e])));
             else yv[e] = from_f32<T>(unary_apply<OP>(to_f32(xv[e]), p));
         }
-        reinterpret_cast<V*>(y)[i] = yv;
+        // fp16 results go through the L2 as they are written (see global_store_b128_through): Gelu on 32 MB 15.5 ->
+        // 14.5 us, its gradient 19.9 -> 19.0 us inside the BERT step
+        if constexpr (sizeof(T) == 2) global_store_b128_through(reinterpret_cast<V*>(y) + i, yv);
+        else reinterpret_cast<V*>(y)[i] = yv;
     }
     for (int64_t i = nvec * VN + (int64_t)blockIdx.x * kEwBlock + threadIdx.x; i < n; i += stride) {
         if constexpr (GRAD) y[i] = from_f32<T>(to_f32(dy[i]) * unary_grad<OP>(to_f32(x[i]), p));

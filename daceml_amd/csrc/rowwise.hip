@@ -3,6 +3,7 @@
 // registers, reduced with DPP lane permutes, and written once. Rows that do not fit the
 // register budget or are not 16-byte aligned take a workgroup-per-row fallback.
 #include "common.h"
+#include "lds_ops.h"
 
 #include <mutex>
 
@@ -254,7 +255,8 @@ __global__ __launch_bounds__(kRowBlock) void layernorm_wave_kernel(
             V t;
 #pragma unroll
             for (int e = 0; e < VN; ++e) t[e] = from_f32<T>(v[j][e] * inv * to_f32(g[e]) + to_f32(b[e]));
-            yr[vi] = t;
+            if constexpr (sizeof(T) == 2) global_store_b128_through(yr + vi, t);
+            else yr[vi] = t;
         }
     }
 }
@@ -373,7 +375,8 @@ __global__ __launch_bounds__(kRowBlock) void layernorm_bwd_wave_kernel(
                 V t;
 #pragma unroll
                 for (int e = 0; e < VN; ++e) t[e] = from_f32<T>((gd[j][e] - s1 - xh[j][e] * s2) * inv);
-                dr[vi] = t;
+                if constexpr (sizeof(T) == 2) global_store_b128_through(dr + vi, t);
+                else dr[vi] = t;
             }
         }
     }
