@@ -174,7 +174,7 @@ __device__ __forceinline__ void store_rows_t(const floatx16 (&acc)[2], float mul
     for (int it = 0; it < 4; ++it) {
         const int r = it * 8 + (lane >> 3), c = lane & 7;
         const half8 v = *reinterpret_cast<const half8*>(region + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
-        if (row0 + r < rows) *reinterpret_cast<half8*>(out + (int64_t)(row0 + r) * stride + c * 8) = v;
+        if (row0 + r < rows) global_store_b128_through(out + (int64_t)(row0 + r) * stride + c * 8, v);
     }
     __builtin_amdgcn_wave_barrier();
 }
