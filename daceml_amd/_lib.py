@@ -71,6 +71,8 @@ SIGNATURES = {
     "dmlhip_layernorm_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),
     "dmlhip_layernorm_backward_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "dmlhip_layernorm_backward_f16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, _P, c_size_t, _P]),
+    "dmlhip_layernorm_backward_grads_f16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int64, _P, c_size_t,
+                                                    _P]),
     "dmlhip_layernorm_backward_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, _P, c_size_t, _P]),
     "dmlhip_layernorm_backward_noalloc_max_bytes": (c_size_t, []),
     "dmlhip_layernorm_backward_noalloc_f16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, _P]),

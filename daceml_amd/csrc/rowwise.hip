@@ -404,11 +404,17 @@ __global__ __launch_bounds__(kRowBlock) void layernorm_bwd_wave_kernel(
     }
 }
 
-void launch_ln_bwd_finish(const float* part, float* dgamma, float* dbeta, int nparts, int64_t cols, hipStream_t st) {
+// dgamma / dbeta: fp32, or (grads_f16) fp16 - the fp32 column sums rounded once as they are stored
+void launch_ln_bwd_finish(const float* part, void* dgamma, void* dbeta, bool grads_f16, int nparts, int64_t cols,
+                          hipStream_t st) {
     // partial rows are [dgamma | dbeta]: one launch finishes both
     const unsigned grid = (unsigned)ceil_div(2 * cols, kWave);
-    hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, part, dgamma, nparts, 2 * cols, 2 * cols,
-                       0.f, 1.f, dbeta, cols);
+    if (grads_f16)
+        hipLaunchKernelGGL((reduce_partials_kernel<OpSum, _Float16>), grid, 1024, 0, st, part, (_Float16*)dgamma, nparts,
+                           2 * cols, 2 * cols, 0.f, 1.f, (_Float16*)dbeta, cols);
+    else
+        hipLaunchKernelGGL((reduce_partials_kernel<OpSum, float>), grid, 1024, 0, st, part, (float*)dgamma, nparts, 2 * cols,
+                           2 * cols, 0.f, 1.f, (float*)dbeta, cols);
 }
 
 // fallback: dx, workgroup per row
@@ -569,14 +575,14 @@ int ln_bwd_parts(int64_t rows) {
 
 template <typename T>
 int layernorm_bwd_impl(const void* dy, const void* x, const float* mean, const float* rstd, const void* gamma,
-                       void* dx, float* dgamma, float* dbeta, int64_t rows, int64_t cols, void* workspace,
-                       size_t workspace_bytes, void* stream) {
+                       void* dx, void* dgamma, void* dbeta, int64_t rows, int64_t cols, void* workspace,
+                       size_t workspace_bytes, void* stream, bool grads_f16 = false) {
     if (int e = check_rows("layernorm_backward", rows, cols)) return e;
     if (cols == 0) return 0;
     DML_REQUIRE(dgamma && dbeta, DMLHIP_ERR_NULL, "layernorm_backward: NULL gradient pointer");
     hipStream_t st = (hipStream_t)stream;
     if (rows == 0) {
-        launch_ln_bwd_finish(nullptr, dgamma, dbeta, 0, cols, st);
+        launch_ln_bwd_finish(nullptr, dgamma, dbeta, grads_f16, 0, cols, st);
         return launch_status("layernorm_backward");
     }
     DML_REQUIRE(dy && x && mean && rstd && gamma && dx, DMLHIP_ERR_NULL, "layernorm_backward: NULL tensor pointer");
@@ -610,7 +616,7 @@ int layernorm_bwd_impl(const void* dy, const void* x, const float* mean, const f
         hipLaunchKernelGGL((layernorm_bwd_cols_kernel<T>), grid, 256, 0, st, gp, xp, mean, rstd, part, rows, cols);
     }
     if (int e = launch_status("layernorm_backward(stage 1)")) return e;
-    launch_ln_bwd_finish(part, dgamma, dbeta, parts, cols, st);
+    launch_ln_bwd_finish(part, dgamma, dbeta, grads_f16, parts, cols, st);
     return launch_status("layernorm_backward(stage 2)");
 }
 
@@ -693,6 +699,15 @@ int dmlhip_layernorm_backward_f32(const void* dy, const void* x, const float* me
                                   int64_t cols, void* workspace, size_t workspace_bytes, void* stream) {
     return layernorm_bwd_impl<float>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, rows, cols, workspace,
                                      workspace_bytes, stream);
+}
+int dmlhip_layernorm_backward_grads_f16(const void* dy, const void* x, const float* mean, const float* rstd,
+                                        const void* gamma, void* dx, void* dgamma, void* dbeta, int grad_dtype,
+                                        int64_t rows, int64_t cols, void* workspace, size_t workspace_bytes,
+                                        void* stream) {
+    DML_REQUIRE(grad_dtype == DMLHIP_F16 || grad_dtype == DMLHIP_F32, DMLHIP_ERR_ENUM,
+                "layernorm_backward_grads: bad grad_dtype %d", grad_dtype);
+    return layernorm_bwd_impl<_Float16>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, rows, cols, workspace,
+                                        workspace_bytes, stream, grad_dtype == DMLHIP_F16);
 }
 size_t dmlhip_layernorm_backward_noalloc_max_bytes(void) { return kStaticScratchBytes; }
 int dmlhip_layernorm_backward_noalloc_f16(const void* dy, const void* x, const float* mean, const float* rstd,

@@ -557,6 +557,15 @@ class HipLayerNormalizationGrad(ONNXForward):
         x = in_desc_with_name(node, state, sdfg, "X")
         rows, cols = _prod(x.shape[:-1]), x.shape[-1]
         ws = L.load().dmlhip_layernorm_backward_workspace_bytes(rows, cols)
+        gdt = {out_desc_with_name(node, state, sdfg, n).dtype for n in ("scale_grad", "bias_grad")}
+        if x.dtype == torch.float16 and gdt == {torch.float16}:
+            # both in the tensor dtype (a caller without fp32 master gradients: the reference gives a gradient the dtype
+            # of its forward array): the entry point that rounds the fp32 column sums as it stores them
+            call = HipCall("dmlhip_layernorm_backward_grads_f16",
+                           [Ptr("Y_grad"), Ptr("X"), Ptr("mean"), Ptr("inv_std_var"), Ptr("scale"), Ptr("X_grad"),
+                            Ptr("scale_grad"), Ptr("bias_grad"), I32(_CODE[torch.float16]), I64(rows), I64(cols),
+                            Workspace(), WorkspaceBytes(), Stream()])
+            return _tasklet(node, state, [call], workspace_bytes=ws, bytes_moved=3 * _nbytes(x), kind="layernorm_backward")
         # The kernel sums the scale / shift gradients in fp32 and writes them as fp32. Where the graph wants them in
         # the tensor dtype (a caller without fp32 master gradients: the reference gives a gradient the dtype of its
         # forward array), they land behind the kernel's own workspace and are cast from there.

@@ -95,6 +95,15 @@ int dmlhip_layernorm_backward_f32(const void* dy, const void* x, const float* me
                                   float* dgamma, float* dbeta, int64_t rows, int64_t cols,
                                   void* workspace, size_t workspace_bytes, void* stream);
 
+/* dmlhip_layernorm_backward_f16 with the scale / shift gradients in the type the caller names (DMLHIP_F16 or
+ * DMLHIP_F32): under the reference a gradient has the dtype of its forward array
+ * (autodiff/backward_pass_generator.py:642-700), so an fp16 LayerNorm's scale and bias get fp16 gradients. The column
+ * sums are formed in fp32 and rounded once when they are stored. */
+int dmlhip_layernorm_backward_grads_f16(const void* dy, const void* x, const float* mean,
+                                        const float* rstd, const void* gamma, void* dx,
+                                        void* dgamma, void* dbeta, int grad_dtype, int64_t rows,
+                                        int64_t cols, void* workspace, size_t workspace_bytes, void* stream);
+
 /* dmlhip_layernorm_backward_f16 for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the
  * reference. Same arguments and results as dmlhip_layernorm_backward_f16 without the workspace: the

@@ -348,6 +348,15 @@ class Emulator:
                 a = list(args[:10])
                 a[6], a[7] = self._typed(a[6], np.float32), self._typed(a[7], np.float32)   # fp32, possibly in the workspace
                 layernorm_backward(*a)
+            elif call.symbol == "dmlhip_layernorm_backward_grads_f16":
+                kinds = {L.F16: np.float16, L.F32: np.float32}
+                a = list(args[:8]) + list(args[9:11])
+                f32 = [np.zeros(args[10], np.float32), np.zeros(args[10], np.float32)]
+                typed = [self._typed(a[6], kinds[args[8]]), self._typed(a[7], kinds[args[8]])]
+                a[6], a[7] = f32
+                layernorm_backward(*a)
+                for dst, src in zip(typed, f32):   # fp32 column sums, rounded once
+                    dst.reshape(-1)[:args[10]] = src.astype(kinds[args[8]])
             elif call.symbol == "dmlhip_cast":
                 kinds = {L.F16: np.float16, L.F32: np.float32}
                 src, dst, n = self._typed(args[2], kinds[args[0]]), self._typed(args[3], kinds[args[1]]), args[4]

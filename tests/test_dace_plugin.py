@@ -670,7 +670,8 @@ def test_training_graphs_reach_the_fused_kernels_as_library_nodes(monkeypatch):
     bst = sdfg.add_state("backward")
     ctx = types.SimpleNamespace(forward_sdfg=sdfg, forward_state=state, backward_sdfg=sdfg, backward_state=bst,
                                 backward_generator=None)
-    expected = {"LayerNormalization": "dmlhip_layernorm_backward_f16", "FusedAttention": "dmlhip_attention_backward_f16",
+    # (LayerNormalization: the scale / shift gradients have the parameters' fp16 under the reference)
+    expected = {"LayerNormalization": "dmlhip_layernorm_backward_grads_f16", "FusedAttention": "dmlhip_attention_backward_f16",
                 "Gelu": "dmlhip_unary_backward_f16", "BiasGelu": "dmlhip_", "FusedEinsum": "dmlhip_gemm_f16"}
     for kind, members in kinds.items():
         node = members[0]
